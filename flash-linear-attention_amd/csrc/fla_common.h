@@ -1,0 +1,106 @@
+// Shared device/host helpers for the gfx950 (CDNA4, wave64) kernels.
+//
+// Conventions used by every kernel in this directory
+//   * tensors are seq-first: q,k [B,T,H,K], v,o [B,T,H,V], per-head scalars [B,T,H];
+//     a packed variable-length batch is [1,T_total,H,*] plus int64 offsets[N+1].
+//   * recurrent state is fp32 [N,H,K,V].
+//   * entry points return 0, a positive hipError_t, or a negative FLA_E_* code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fla_hip.h"
+
+typedef __bf16 bf16;
+typedef _Float16 f16;
+typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef f16 f16x4 __attribute__((ext_vector_type(4)));
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define FLA_DEVICE __device__ __forceinline__
+
+#define FLA_CHECK_LAUNCH()                         \
+  do {                                             \
+    hipError_t e__ = hipGetLastError();            \
+    if (e__ != hipSuccess) return (int)e__;        \
+  } while (0)
+
+#define FLA_REQUIRE(cond, code) \
+  do {                          \
+    if (!(cond)) return (code); \
+  } while (0)
+
+static inline int64_t fla_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------------------
+// element type traits: 16-bit storage types with their 4/8-wide vectors and
+// the matching gfx950 MFMA instructions (fp32 accumulate).
+// ---------------------------------------------------------------------------
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<bf16> {
+  typedef bf16x4 v4;
+  typedef bf16x8 v8;
+  static FLA_DEVICE f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static FLA_DEVICE f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <>
+struct Elem<f16> {
+  typedef f16x4 v4;
+  typedef f16x8 v8;
+  static FLA_DEVICE f32x16 mfma32(v8 a, v8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static FLA_DEVICE f32x4 mfma16(v8 a, v8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// MFMA operand/accumulator ownership on wave64 (l = lane id):
+//   32x32x16: A lane l holds A[row = l%32][k = 8*(l/32) .. +7]
+//             B lane l holds B[k = 8*(l/32) .. +7][col = l%32]
+//             C reg r of lane l is C[row = 8*(r/4) + 4*(l/32) + r%4][col = l%32]
+//   16x16x32: A lane l holds A[row = l%16][k = 8*(l/16) .. +7]
+//             B lane l holds B[k = 8*(l/16) .. +7][col = l%16]
+//             C reg r of lane l is C[row = 4*(l/16) + r][col = l%16]
+// The contraction index may be permuted freely as long as A and B agree.
+FLA_DEVICE int c32_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+template <typename T>
+FLA_DEVICE float to_f32(T x) { return (float)x; }
+
+template <typename T>
+FLA_DEVICE T from_f32(float x) { return (T)x; }
+
+// exp(x) for x <= 0, 0 otherwise: decay factors must never amplify
+// (fla/ops/utils/exp.py:9-10).
+FLA_DEVICE float safe_exp(float x) { return x <= 0.f ? __expf(x) : 0.f; }
+
+struct SeqSpan {
+  int64_t bos;  // first token row of the sequence in the packed [B*T] row space
+  int64_t len;  // number of tokens
+};
+
+// Rows are addressed in the flattened [B*T] space; for a packed batch B == 1.
+FLA_DEVICE SeqSpan seq_span(const int64_t* offsets, int n, int64_t T) {
+  SeqSpan s;
+  if (offsets) {
+    s.bos = offsets[n];
+    s.len = offsets[n + 1] - s.bos;
+  } else {
+    s.bos = (int64_t)n * T;
+    s.len = T;
+  }
+  return s;
+}

@@ -1,0 +1,575 @@
+// Chunked GLA forward for gfx950: chunk size 64, 16-bit q/k/v, fp32 state.
+//
+//   gla_fwd_h_kernel  inter-chunk state scan.  One workgroup owns a 64(k) x 64(v)
+//                     tile of the fp32 state of one (sequence, head) in MFMA
+//                     accumulators and walks the chunks serially:
+//                       store h_c;  h <- diag(e^{G_last}) h + (k * e^{G_last-G})^T v.
+//                     The chunk-local prefix sum G of the log-gates is formed in
+//                     registers from the raw gates (no separate cumsum pass).
+//   gla_fwd_o_kernel  one workgroup per (chunk, head):
+//                       S = (s q e^{G}) (k e^{-G})^T, P = tril(S), o = (s q e^{G}) h_c + P v.
+//
+// The per-chunk states travel between the two kernels in "fragment order": the
+// scan kernel stores each wave's 32x32 accumulator tile exactly as its lanes
+// hold it (16 contiguous 16-bit values per lane), and the output kernel loads
+// those 32 bytes per lane straight into MFMA B operands (with the matching
+// permutation of the contraction index on the A side).  No LDS staging and no
+// transposition of the state on either side, and all traffic is 16-byte
+// coalesced.
+//
+// Math follows fla/ops/common/chunk_h.py:73-137 (scan), fla/ops/gla/chunk.py:29-170
+// (scores) and :320-393 (output).  Unlike the reference's 16x16 sub-block
+// scheme the scores use one reference point per chunk (exp(G) on q, exp(-G) on
+// k), which is exact in floating point as long as |G| stays below ~80 per
+// channel inside a chunk; see the range check in the host wrapper.
+#include "fla_common.h"
+#include "mfma_tiles.h"
+
+namespace {
+
+constexpr int BT = 64;        // chunk length
+constexpr int LDT = BT + 8;   // row pitch of time-contiguous LDS tiles
+
+template <typename X>
+struct Load;
+template <>
+struct Load<float> {
+  static FLA_DEVICE void x2(const float* p, float* o) {
+    f32x2 v = *(const f32x2*)p;
+    o[0] = v[0]; o[1] = v[1];
+  }
+  static FLA_DEVICE void x4(const float* p, float* o) {
+    f32x4 v = *(const f32x4*)p;
+    o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+  }
+};
+template <>
+struct Load<bf16> {
+  static FLA_DEVICE void x2(const bf16* p, float* o) {
+    typedef bf16 v2 __attribute__((ext_vector_type(2)));
+    v2 v = *(const v2*)p;
+    o[0] = (float)v[0]; o[1] = (float)v[1];
+  }
+  static FLA_DEVICE void x4(const bf16* p, float* o) {
+    bf16x4 v = *(const bf16x4*)p;
+    for (int i = 0; i < 4; ++i) o[i] = (float)v[i];
+  }
+};
+template <>
+struct Load<f16> {
+  static FLA_DEVICE void x2(const f16* p, float* o) {
+    typedef f16 v2 __attribute__((ext_vector_type(2)));
+    v2 v = *(const v2*)p;
+    o[0] = (float)v[0]; o[1] = (float)v[1];
+  }
+  static FLA_DEVICE void x4(const f16* p, float* o) {
+    f16x4 v = *(const f16x4*)p;
+    for (int i = 0; i < 4; ++i) o[i] = (float)v[i];
+  }
+};
+
+// Workgroups of one launch are dealt round-robin to the 8 XCDs by linear id.
+// Renumber so that consecutive logical ids share an XCD (and its L2).
+FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
+  if (total % 8 != 0) return id;
+  return (id % 8) * (total / 8) + id / 8;
+}
+
+struct HParams {
+  const void* k;
+  const void* v;
+  const void* g;
+  const float* h0;
+  void* h;
+  float* ht;
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int H, K, V, N;
+};
+
+// HL: 0 row-major [K,V] in T, 1 fragment order in T, 2 row-major fp32.
+template <typename T, typename GT, bool GCUM, int HL>
+__global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
+  typedef typename Elem<T>::v8 v8;
+  __shared__ __attribute__((aligned(16))) T sKt[64 * LDT];  // [k][t] decayed keys
+  __shared__ __attribute__((aligned(16))) T sVt[64 * LDT];  // [v][t]
+  __shared__ __attribute__((aligned(16))) float sPart[8 * 64];
+  __shared__ __attribute__((aligned(16))) float sDecay[64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, V = p.V;
+  const int nkt = K / 64, nvt = V / 64, ntile = nkt * nvt;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile = (int)(id % ntile);
+  const int nh = (int)(id / ntile);
+  const int n = nh / H, hh = nh % H;
+  const int kbase = (tile % nkt) * 64, vbase = (tile / nkt) * 64;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+
+  // load mapping: 8 row groups x 32 column pairs
+  const int rg = tid >> 5, c2 = (tid & 31) * 2;
+  const T* kp = (const T*)p.k + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
+  const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
+  const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + c2;
+  const int64_t kstride = (int64_t)H * K, vstride = (int64_t)H * V;
+
+  // accumulator tile of this wave: rows k = kq*32.., cols v = vq*32..
+  const int kq = wave & 1, vq = wave >> 1;
+  const int vcol = vbase + vq * 32 + (lane & 31);
+  f32x16 acc = zero16();
+  if (p.h0) {
+    const float* h0p = p.h0 + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = h0p[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
+  }
+
+  float gq[8][2], kk[8][2], vv[8][2];
+  auto load_chunk = [&](int64_t c) {
+    int64_t t0 = c * BT;
+    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int row = rg * 8 + i;
+      if (row < L) {
+        Load<GT>::x2(gp + (t0 + row) * kstride, gq[i]);
+        Load<T>::x2(kp + (t0 + row) * kstride, kk[i]);
+        Load<T>::x2(vp + (t0 + row) * vstride, vv[i]);
+      } else {
+        gq[i][0] = gq[i][1] = 0.f;
+        kk[i][0] = kk[i][1] = 0.f;
+        vv[i][0] = vv[i][1] = 0.f;
+      }
+    }
+  };
+
+  if (nchunks > 0) load_chunk(0);
+  for (int64_t c = 0; c < nchunks; ++c) {
+    int64_t t0 = c * BT;
+    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+    // ---- state entering chunk c
+    if (p.h) {
+      int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
+      if (HL == 1) {
+        T* hp = (T*)p.h + blk + (((int64_t)(kbase / 32 + kq) * (V / 32) + (vbase / 32 + vq)) * 64 + lane) * 16;
+        v8 lo, hi;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          lo[r] = (T)acc[r];
+          hi[r] = (T)acc[r + 8];
+        }
+        *(v8*)hp = lo;
+        *(v8*)(hp + 8) = hi;
+      } else if (HL == 0) {
+        T* hp = (T*)p.h + blk;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) hp[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = (T)acc[r];
+      } else {
+        float* hp = (float*)p.h + blk;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) hp[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc[r];
+      }
+    }
+    // ---- chunk-local prefix sums of the gates (or pick up the given ones)
+    float G[8][2];
+    if (!GCUM) {
+      float r0 = 0.f, r1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        r0 += gq[i][0];
+        r1 += gq[i][1];
+        G[i][0] = r0;
+        G[i][1] = r1;
+      }
+      *(f32x2*)&sPart[rg * 64 + c2] = f32x2{r0, r1};
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        G[i][0] = gq[i][0];
+        G[i][1] = gq[i][1];
+      }
+      if (((L - 1) >> 3) == rg) *(f32x2*)&sPart[c2] = f32x2{G[(L - 1) & 7][0], G[(L - 1) & 7][1]};
+    }
+    __syncthreads();  // (A) partial sums visible; previous chunk's MFMA reads of sKt/sVt are done
+    float glast0, glast1;
+    if (!GCUM) {
+      float off0 = 0.f, off1 = 0.f, tot0 = 0.f, tot1 = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        f32x2 pr = *(const f32x2*)&sPart[r * 64 + c2];
+        if (r < rg) {
+          off0 += pr[0];
+          off1 += pr[1];
+        }
+        tot0 += pr[0];
+        tot1 += pr[1];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        G[i][0] += off0;
+        G[i][1] += off1;
+      }
+      glast0 = tot0;
+      glast1 = tot1;
+    } else {
+      f32x2 pr = *(const f32x2*)&sPart[c2];
+      glast0 = pr[0];
+      glast1 = pr[1];
+    }
+    {
+      v8 ka, kb, va, vb;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        bool valid = (rg * 8 + i) < L;
+        float e0 = valid ? __expf(glast0 - G[i][0]) : 0.f;
+        float e1 = valid ? __expf(glast1 - G[i][1]) : 0.f;
+        ka[i] = (T)(kk[i][0] * e0);
+        kb[i] = (T)(kk[i][1] * e1);
+        va[i] = (T)vv[i][0];
+        vb[i] = (T)vv[i][1];
+      }
+      *(v8*)&sKt[(c2 + 0) * LDT + rg * 8] = ka;
+      *(v8*)&sKt[(c2 + 1) * LDT + rg * 8] = kb;
+      *(v8*)&sVt[(c2 + 0) * LDT + rg * 8] = va;
+      *(v8*)&sVt[(c2 + 1) * LDT + rg * 8] = vb;
+      if (rg == 0) *(f32x2*)&sDecay[c2] = f32x2{__expf(glast0), __expf(glast1)};
+    }
+    if (c + 1 < nchunks) load_chunk(c + 1);  // in flight across the barrier and the MFMAs
+    __syncthreads();  // (B) operand tiles complete
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      f32x4 d = *(const f32x4*)&sDecay[kq * 32 + 8 * a + 4 * (lane >> 5)];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc[4 * a + b] *= d[b];
+    }
+#pragma unroll
+    for (int s = 0; s < BT; s += 16)
+      acc = Elem<T>::mfma32(lds_frag32<T>(sKt, LDT, kq * 32, s, lane), lds_frag32<T>(sVt, LDT, vq * 32, s, lane), acc);
+  }
+  if (p.ht) {
+    float* htp = p.ht + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) htp[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc[r];
+  }
+}
+
+struct OParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const void* h;
+  void* o;
+  float* A;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+// One workgroup per (chunk, head).  K, V: head dims (multiples of 64).
+template <typename T, typename GT, bool GCUM, int K, int V>
+__global__ __launch_bounds__(256) void gla_fwd_o_kernel(OParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;      // q,k,g mapping
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;  // v mapping
+  constexpr int KT32 = K / 32;
+  constexpr int TV = V / 64;  // 32-wide v tiles per wave
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];  // later: P [i][j] with pitch LDT
+  __shared__ __attribute__((aligned(16))) T sVt[V * LDT];
+  __shared__ __attribute__((aligned(16))) float sPart[RG * K];
+  T* sP = sK;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H;
+  const int hh = blockIdx.y;
+  int64_t bos, len, ic, cglob;
+  if (p.offsets) {
+    int64_t n = p.indices[2 * (int64_t)blockIdx.x];
+    ic = p.indices[2 * (int64_t)blockIdx.x + 1];
+    bos = p.offsets[n];
+    len = p.offsets[n + 1] - bos;
+    cglob = blockIdx.x;
+  } else {
+    int64_t b = blockIdx.x / p.NTfix;
+    ic = blockIdx.x % p.NTfix;
+    bos = b * p.T;
+    len = p.T;
+    cglob = blockIdx.x;
+  }
+  const int64_t t0 = ic * BT;
+  const int L = (int)((len - t0) < BT ? (len - t0) : BT);
+  const int64_t row0 = bos + t0;
+
+  // ---- issue every global load up front
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  float gq[RPT][4], qq[RPT][4], kk[RPT][4];
+  {
+    const int64_t base = (row0 * H + hh) * (int64_t)K + c4;
+    const int64_t stride = (int64_t)H * K;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      if (row < L) {
+        Load<GT>::x4((const GT*)p.g + base + row * stride, gq[i]);
+        Load<T>::x4((const T*)p.q + base + row * stride, qq[i]);
+        Load<T>::x4((const T*)p.k + base + row * stride, kk[i]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gq[i][j] = qq[i][j] = kk[i][j] = 0.f;
+      }
+    }
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+  v4 vreg[RPTV];
+  {
+    const int64_t base = (row0 * H + hh) * (int64_t)V + cv4;
+    const int64_t stride = (int64_t)H * V;
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) {
+      int row = rgv * RPTV + i;
+      if (row < L) {
+        vreg[i] = *(const v4*)((const T*)p.v + base + row * stride);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) vreg[i][j] = (T)0.f;
+      }
+    }
+  }
+  // state fragments: wave (rw, cw) needs all k tiles of its TV v tiles
+  const int rw = wave >> 1, cw = wave & 1;
+  v8 hf[KT32][TV][2];
+  {
+    const T* hp = (const T*)p.h + (cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) {
+        const T* f = hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16;
+        hf[kt][tv][0] = *(const v8*)f;
+        hf[kt][tv][1] = *(const v8*)(f + 8);
+      }
+  }
+
+  // ---- gates: chunk-local prefix sum
+  float G[RPT][4];
+  if (!GCUM) {
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        run[j] += gq[i][j];
+        G[i][j] = run[j];
+      }
+    *(f32x4*)&sPart[rg * K + c4] = f32x4{run[0], run[1], run[2], run[3]};
+    __syncthreads();
+    float off[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      if (r < rg) {
+        f32x4 pr = *(const f32x4*)&sPart[r * K + c4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) off[j] += pr[j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) G[i][j] += off[j];
+  } else {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) G[i][j] = gq[i][j];
+  }
+  // ---- gated operands to LDS
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    v4 qv, kv;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      qv[j] = (T)(qq[i][j] * p.scale * __expf(G[i][j]));
+      kv[j] = (T)(kk[i][j] * __expf(-G[i][j]));
+    }
+    *(v4*)&sQ[row * LDK + c4] = qv;
+    *(v4*)&sK[row * LDK + c4] = kv;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T tmp[RPTV];
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) tmp[i] = vreg[i][j];
+    T* dst = &sVt[(cv4 + j) * LDT + rgv * RPTV];
+    if (RPTV == 4) {
+      *(v4*)dst = v4{tmp[0], tmp[1], tmp[2], tmp[3]};
+    } else {
+#pragma unroll
+      for (int i0 = 0; i0 < RPTV; i0 += 8) {
+        v8 w;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[i] = tmp[(i0 + i) < RPTV ? (i0 + i) : 0];
+        *(v8*)(dst + i0) = w;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- scores: 32x32 quadrants (0,0), (1,0), (1,1) on waves 0, 2, 3
+  const int qi = wave >> 1, qj = wave & 1;
+  f32x16 s = zero16();
+  if (qj <= qi) {
+#pragma unroll
+    for (int ks = 0; ks < K; ks += 16)
+      s = Elem<T>::mfma32(lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
+  }
+  __syncthreads();  // every wave is done reading sK before P overwrites it
+  {
+    const int j = qj * 32 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = qi * 32 + c32_row(r, lane);
+      float val = (j <= i) ? s[r] : 0.f;
+      sP[i * LDT + j] = (T)val;
+      if (p.A && i < L) p.A[((row0 + i) * H + hh) * (int64_t)BT + j] = val;
+    }
+  }
+  __syncthreads();
+
+  // ---- o = q~ h + P v
+  f32x16 acc[TV];
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+#pragma unroll
+  for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v8 a = lds_frag32_perm<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(a, hf[kt][tv][half], acc[tv]);
+    }
+  const int jend = (rw + 1) * 32;
+  for (int js = 0; js < jend; js += 16) {
+    v8 a = lds_frag32<T>(sP, LDT, rw * 32, js, lane);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
+  }
+  T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = rw * 32 + c32_row(r, lane);
+      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    }
+}
+
+template <typename T, typename GT, bool GCUM>
+int launch_h(const HParams& p, int h_dtype, int h_layout, hipStream_t st) {
+  int64_t total = (int64_t)(p.K / 64) * (p.V / 64) * p.N * p.H;
+  if (total == 0) return FLA_OK;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  dim3 grid((unsigned)total), block(256);
+  if (h_layout == FLA_H_FRAGMENT) {
+    hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 1>), grid, block, 0, st, p);
+  } else if (h_dtype == FLA_F32) {
+    hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 2>), grid, block, 0, st, p);
+  } else {
+    hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 0>), grid, block, 0, st, p);
+  }
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+template <typename T, typename GT>
+int launch_h_g(const HParams& p, int gcum, int h_dtype, int h_layout, hipStream_t st) {
+  return gcum ? launch_h<T, GT, true>(p, h_dtype, h_layout, st) : launch_h<T, GT, false>(p, h_dtype, h_layout, st);
+}
+
+template <typename T, typename GT, bool GCUM>
+int launch_o(const OParams& p, int K, int V, dim3 grid, hipStream_t st) {
+  dim3 block(256);
+#define FLA_O_CASE(KK, VV)                                                                       \
+  if (K == KK && V == VV) {                                                                      \
+    hipLaunchKernelGGL((gla_fwd_o_kernel<T, GT, GCUM, KK, VV>), grid, block, 0, st, p);          \
+    FLA_CHECK_LAUNCH();                                                                          \
+    return FLA_OK;                                                                               \
+  }
+  FLA_O_CASE(64, 64)
+  FLA_O_CASE(128, 128)
+  FLA_O_CASE(64, 128)
+  FLA_O_CASE(128, 64)
+#undef FLA_O_CASE
+  return FLA_E_UNSUPPORTED;
+}
+
+template <typename T, typename GT>
+int launch_o_g(const OParams& p, int gcum, int K, int V, dim3 grid, hipStream_t st) {
+  return gcum ? launch_o<T, GT, true>(p, K, V, grid, st) : launch_o<T, GT, false>(p, K, V, grid, st);
+}
+
+}  // namespace
+
+extern "C" int fla_chunk_gla_fwd_h(const void* k, const void* v, const void* gates, int gates_are_cumsum,
+                                   const float* h0, void* h, float* ht, const int64_t* offsets,
+                                   const int64_t* chunk_offsets, int qkv_dtype, int gate_dtype, int h_dtype,
+                                   int h_layout, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                   fla_stream_t stream) {
+  FLA_REQUIRE(k && v && gates, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 512 && V <= 512 && H <= 65535, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(chunk_offsets != nullptr && B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT, FLA_E_INVALID);
+  if (h_layout == FLA_H_FRAGMENT) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
+  else FLA_REQUIRE(h_dtype == qkv_dtype || h_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  if (gates_are_cumsum) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)h) % 16 == 0, FLA_E_ALIGNMENT);
+  HParams p{k, v, gates, h0, h, ht, offsets, chunk_offsets, T, (int)H, (int)K, (int)V, (int)N};
+  hipStream_t st = (hipStream_t)stream;
+  if (qkv_dtype == FLA_BF16) {
+    if (gate_dtype == FLA_F32) return launch_h_g<bf16, float>(p, gates_are_cumsum, h_dtype, h_layout, st);
+    if (gate_dtype == FLA_BF16) return launch_h_g<bf16, bf16>(p, 0, h_dtype, h_layout, st);
+  } else if (qkv_dtype == FLA_F16) {
+    if (gate_dtype == FLA_F32) return launch_h_g<f16, float>(p, gates_are_cumsum, h_dtype, h_layout, st);
+    if (gate_dtype == FLA_F16) return launch_h_g<f16, f16>(p, 0, h_dtype, h_layout, st);
+  }
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void* gates,
+                                   int gates_are_cumsum, const void* h, void* o, float* A_out,
+                                   const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                                   int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale,
+                                   fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && gates && h && o, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(H <= 65535, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(indices != nullptr && B == 1, FLA_E_INVALID);
+  if (gates_are_cumsum) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)h | (uintptr_t)o) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  int64_t ntfix = (T + BT - 1) / BT;
+  int64_t nblk = offsets ? NT : B * ntfix;
+  if (nblk == 0) return FLA_OK;
+  FLA_REQUIRE(nblk <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  OParams p{q, k, v, gates, h, o, A_out, offsets, indices, T, (int)H, (int)ntfix, scale};
+  dim3 grid((unsigned)nblk, (unsigned)H);
+  hipStream_t st = (hipStream_t)stream;
+  if (qkv_dtype == FLA_BF16) {
+    if (gate_dtype == FLA_F32) return launch_o_g<bf16, float>(p, gates_are_cumsum, (int)K, (int)V, grid, st);
+    if (gate_dtype == FLA_BF16) return launch_o_g<bf16, bf16>(p, 0, (int)K, (int)V, grid, st);
+  } else if (qkv_dtype == FLA_F16) {
+    if (gate_dtype == FLA_F32) return launch_o_g<f16, float>(p, gates_are_cumsum, (int)K, (int)V, grid, st);
+    if (gate_dtype == FLA_F16) return launch_o_g<f16, f16>(p, 0, (int)K, (int)V, grid, st);
+  }
+  return FLA_E_UNSUPPORTED;
+}

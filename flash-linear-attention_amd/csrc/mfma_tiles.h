@@ -1,0 +1,41 @@
+// LDS -> MFMA operand fragment loaders.  Tiles are stored with the contraction
+// index contiguous ("row-major over k") and a row pitch `ld` that is a
+// multiple of 8 elements, so every fragment is one 16-byte LDS read.
+#pragma once
+#include "fla_common.h"
+
+// 32x32x16 operand: 32 rows starting at row0, contraction slice [k0, k0+16).
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 lds_frag32(const T* tile, int ld, int row0, int k0, int lane) {
+  return *(const typename Elem<T>::v8*)(tile + (row0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5));
+}
+
+// Same slice with the contraction index permuted inside the 16-slice: slot
+// (g = lane/32, e) holds k0 + 8*(e/4) + 4*g + e%4.  This is the order in which
+// a 32x32 accumulator's registers enumerate rows, so an accumulator converted
+// to 16-bit can be fed back as the other operand without a shuffle.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 lds_frag32_perm(const T* tile, int ld, int row0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const T* p = tile + (row0 + (lane & 31)) * ld + k0 + 4 * (lane >> 5);
+  v4 lo = *(const v4*)p;
+  v4 hi = *(const v4*)(p + 8);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// 16x16x32 operand: 16 rows starting at row0, contraction slice [k0, k0+32).
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 lds_frag16(const T* tile, int ld, int row0, int k0, int lane) {
+  return *(const typename Elem<T>::v8*)(tile + (row0 + (lane & 15)) * ld + k0 + 8 * (lane >> 4));
+}
+
+FLA_DEVICE f32x16 zero16() {
+  f32x16 z;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = 0.f;
+  return z;
+}
+FLA_DEVICE f32x4 zero4() {
+  f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  return z;
+}

@@ -1,0 +1,175 @@
+"""``chunk_gla`` with the reference's signature (``fla/ops/gla/chunk.py:1409-1495``).
+
+Forward pipeline on the device (chunk size 64):
+``fla_chunk_gla_fwd_h`` (state scan, cumsum of the gates formed in-kernel)
+-> ``fla_chunk_gla_fwd_o`` (fused cumsum + gated scores + output).
+"""
+import warnings
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from ... import _backend as be
+from ...utils import VarlenPlan, check_varlen_args, contiguous, resolve_offsets
+from ..common.chunk_h import chunk_fwd_h
+from ..utils.cumsum import chunk_local_cumsum
+
+BT = 64
+_SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
+
+
+def _pad_dim(x: Optional[torch.Tensor], size: int) -> Optional[torch.Tensor]:
+    if x is None or x.shape[-1] == size:
+        return x
+    return F.pad(x, (0, size - x.shape[-1]))
+
+
+def _round64(d: int) -> int:
+    return -(-d // 64) * 64
+
+
+def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_first=True, chunk_size=64,
+                       *, k=None, gates_are_cumsum=True, A_out=None):
+    """Output kernel.  Unlike the reference (``fla/ops/gla/chunk.py:941-979``) the
+    device kernel recomputes the scores from ``q, k, g`` instead of reading ``A``,
+    so ``k`` must be given and ``h`` must be in fragment layout."""
+    if head_first or chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gla_fwd_o_gk: seq-first, chunk size 64 only")
+    if k is None:
+        raise NotImplementedError("fla_amd chunk_gla_fwd_o_gk: pass k=; scores are recomputed in the kernel")
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    NT = 0
+    if offsets is not None:
+        NT = indices.shape[0]
+    o = torch.empty_like(v)
+    be.check(be.lib().fla_chunk_gla_fwd_o(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), int(gates_are_cumsum), be.ptr(h), be.ptr(o), be.ptr(A_out),
+        be.ptr(offsets), be.ptr(indices), NT, be.dt(q), be.dt(g), B, T, H, K, V, float(scale),
+        be.stream_of(q)), "fla_chunk_gla_fwd_o")
+    return o
+
+
+def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False):
+    """Seq-first forward on 64-aligned head dims.  Returns (o, ht, A)."""
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    B, T, H, K = q.shape
+    h, ht = chunk_fwd_h(
+        k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=output_final_state,
+        offsets=None if plan is None else plan.offsets,
+        indices=None if plan is None else plan.indices,
+        head_first=False, chunk_size=BT, gates_are_cumsum=False, fragment_layout=True,
+        chunk_offsets=None if plan is None else plan.chunk_offsets)
+    A = q.new_empty(B, T, H, BT, dtype=torch.float32) if want_A else None
+    o = chunk_gla_fwd_o_gk(q, v, g, None, h, scale,
+                           offsets=None if plan is None else plan.offsets,
+                           indices=None if plan is None else plan.indices,
+                           head_first=False, chunk_size=BT, k=k, gates_are_cumsum=False, A_out=A)
+    return o, ht, A
+
+
+def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state,
+                  offsets=None, indices=None, head_first=True, chunk_size=64):
+    """Reference-shaped forward (``fla/ops/gla/chunk.py:1156-1214``) for internal
+    callers: returns ``(g_cumsum, A, h, ht, o)`` with ``h`` row-major
+    ``[B,NT,H,K,V]`` and ``A`` fp32 ``[B,T,H,64]``."""
+    if head_first:
+        raise NotImplementedError("fla_amd chunk_gla_fwd: seq-first layout only")
+    T = q.shape[1]
+    if min(chunk_size, max(16, 1 << (T - 1).bit_length())) != BT:
+        raise NotImplementedError("fla_amd chunk_gla_fwd: chunk size is fixed to 64 (needs T > 32)")
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    offs = None if plan is None else plan.offsets
+    idx = None if plan is None else plan.indices
+    if g_cumsum is None:
+        g_cumsum = chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
+    h, ht = chunk_fwd_h(k=k, v=v, g=None, gk=g_cumsum, gv=None, h0=initial_state,
+                        output_final_state=output_final_state, offsets=offs, indices=idx, head_first=False,
+                        chunk_size=BT, chunk_offsets=None if plan is None else plan.chunk_offsets)
+    hf, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g_cumsum, gv=None, h0=initial_state, output_final_state=False,
+                        offsets=offs, indices=idx, head_first=False, chunk_size=BT, fragment_layout=True,
+                        chunk_offsets=None if plan is None else plan.chunk_offsets)
+    B, _, H, _ = q.shape
+    A = q.new_empty(B, T, H, BT, dtype=torch.float32)
+    o = chunk_gla_fwd_o_gk(q, v, g_cumsum, None, hf, scale, offsets=offs, indices=idx, head_first=False,
+                           chunk_size=BT, k=k, gates_are_cumsum=True, A_out=A)
+    return g_cumsum, A, h, ht, o
+
+
+class ChunkGLAFunction(torch.autograd.Function):
+
+    @staticmethod
+    @contiguous
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, offsets, head_first):
+        be.require_gpu(q, k, v, g)
+        if head_first:
+            q, k, v, g = (x.transpose(1, 2).contiguous() for x in (q, k, v, g))
+        dtype = q.dtype
+        if dtype == torch.float32:
+            warnings.warn("fla_amd chunk_gla: fp32 q/k/v are rounded to bf16 for the MFMA kernels "
+                          "(state and gates stay fp32)", stacklevel=3)
+            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        k, v = k.to(q.dtype), v.to(q.dtype)
+        if g.dtype not in (torch.float32, q.dtype):
+            g = g.float()
+        K, V = q.shape[-1], v.shape[-1]
+        KP, VP = _round64(K), _round64(V)
+        if (KP, VP) not in _SUPPORTED_KV:
+            raise NotImplementedError(f"fla_amd chunk_gla: head dims K={K}, V={V} are outside the built tiles "
+                                      f"{sorted(_SUPPORTED_KV)} (after rounding up to multiples of 64)")
+        h0 = initial_state
+        if (KP, VP) != (K, V):
+            q, k, g = _pad_dim(q, KP), _pad_dim(k, KP), _pad_dim(g, KP)
+            v = _pad_dim(v, VP)
+            if h0 is not None:
+                h0 = F.pad(h0, (0, VP - V, 0, KP - K))
+        o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets)
+        if (KP, VP) != (K, V):
+            o = o[..., :V]
+            if ht is not None:
+                ht = ht[..., :K, :V].contiguous()
+        if dtype == torch.float32:
+            o = o.float()
+        if head_first:
+            o = o.transpose(1, 2).contiguous()
+        return o, ht
+
+    @staticmethod
+    @contiguous
+    def backward(ctx, do, dht):
+        raise NotImplementedError("fla_amd chunk_gla: the backward kernels are not built yet")
+
+
+def chunk_gla(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    scale: Optional[int] = None,
+    initial_state: torch.Tensor = None,
+    output_final_state: bool = False,
+    offsets: Optional[torch.LongTensor] = None,
+    head_first: bool = True,
+    cu_seqlens: Optional[torch.LongTensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    r"""
+    Args:
+        q, k: ``[B, H, T, K]`` if ``head_first`` else ``[B, T, H, K]``.
+        v: ``[B, H, T, V]`` / ``[B, T, H, V]``.
+        g: log forget gates applied to keys, same shape as ``k``.
+        scale: score scale, default ``K ** -0.5``.
+        initial_state: ``[N, H, K, V]`` for ``N`` sequences, or ``None``.
+        output_final_state: also return the fp32 final state ``[N, H, K, V]``.
+        offsets (synonym ``cu_seqlens``): int64 ``[N+1]`` sequence boundaries of a
+            packed batch (batch size 1, seq-first only).
+        head_first: layout switch; seq-first is the native layout.
+
+    Returns ``(o, final_state)``.
+    """
+    offsets = resolve_offsets(offsets, cu_seqlens)
+    check_varlen_args(q, offsets, head_first, initial_state)
+    if scale is None:
+        scale = q.shape[-1] ** -0.5
+    o, final_state = ChunkGLAFunction.apply(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
+    return o, final_state

@@ -1,0 +1,103 @@
+"""Boundary helpers mirroring ``fla/utils.py``: ``contiguous`` and the autocast
+shims (``fla/utils.py:10-21,88-93``), plus the host-side chunk bookkeeping.
+
+The reference caches bookkeeping results keyed on ``data_ptr``
+(``fla/utils.py:24-63``), which goes stale when a buffer is reused; here the
+``offsets`` values themselves form the key.
+"""
+import ctypes
+import functools
+from typing import Optional, Tuple
+
+import torch
+
+from . import _backend as be
+
+
+def contiguous(fn):
+    """Make every tensor argument after the first (``ctx``) contiguous."""
+    @functools.wraps(fn)
+    def wrapper(ctx, *args, **kwargs):
+        return fn(ctx,
+                  *(a.contiguous() if isinstance(a, torch.Tensor) else a for a in args),
+                  **{k: (v.contiguous() if isinstance(v, torch.Tensor) else v) for k, v in kwargs.items()})
+    return wrapper
+
+
+autocast_custom_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda")
+autocast_custom_bwd = functools.partial(torch.amp.custom_bwd, device_type="cuda")
+
+
+def _host_offsets(offsets) -> Tuple[int, ...]:
+    if isinstance(offsets, torch.Tensor):
+        return tuple(int(x) for x in offsets.detach().cpu().tolist())
+    return tuple(int(x) for x in offsets)
+
+
+@functools.lru_cache(maxsize=64)
+def _chunk_tables(offs: Tuple[int, ...], chunk_size: int):
+    n = len(offs) - 1
+    arr = (ctypes.c_int64 * (n + 1))(*offs)
+    nt = be.lib().fla_count_chunks(arr, n, chunk_size)
+    if nt < 0:
+        raise ValueError("offsets must be non-decreasing int64 positions")
+    indices = torch.empty(nt, 2, dtype=torch.int64)
+    chunk_offsets = torch.empty(n + 1, dtype=torch.int64)
+    be.check(be.lib().fla_prepare_chunk_indices(arr, n, chunk_size,
+                                                ctypes.c_void_p(indices.data_ptr()),
+                                                ctypes.c_void_p(chunk_offsets.data_ptr())),
+             "fla_prepare_chunk_indices")
+    return indices, chunk_offsets
+
+
+def prepare_chunk_indices(offsets, chunk_size: int, device=None) -> torch.Tensor:
+    """int64 ``[NT, 2]`` rows (sequence, chunk in sequence); the reference's
+    ``prepare_varlen_inputs`` (``fla/ops/gla/chunk.py:1323-1330``)."""
+    idx, _ = _chunk_tables(_host_offsets(offsets), int(chunk_size))
+    if device is None and isinstance(offsets, torch.Tensor):
+        device = offsets.device
+    return idx.to(device) if device is not None else idx.clone()
+
+
+def prepare_chunk_offsets(offsets, chunk_size: int, device=None) -> torch.Tensor:
+    """int64 ``[N+1]`` exclusive prefix sum of per-sequence chunk counts
+    (``fla/ops/common/chunk_h.py:274-279``)."""
+    _, co = _chunk_tables(_host_offsets(offsets), int(chunk_size))
+    if device is None and isinstance(offsets, torch.Tensor):
+        device = offsets.device
+    return co.to(device) if device is not None else co.clone()
+
+
+class VarlenPlan:
+    """Everything the kernels need to address a packed batch."""
+
+    def __init__(self, offsets: torch.Tensor, chunk_size: int):
+        host = _host_offsets(offsets)
+        idx, co = _chunk_tables(host, int(chunk_size))
+        dev = offsets.device
+        self.offsets = offsets.to(torch.int64).contiguous()
+        self.indices = idx.to(dev, non_blocking=True)
+        self.chunk_offsets = co.to(dev, non_blocking=True)
+        self.N = len(host) - 1
+        self.NT = idx.shape[0]
+
+
+def resolve_offsets(offsets: Optional[torch.Tensor], cu_seqlens: Optional[torch.Tensor]):
+    """``cu_seqlens`` is accepted as a synonym of ``offsets``."""
+    if offsets is not None and cu_seqlens is not None:
+        raise ValueError("pass either `offsets` or `cu_seqlens`, not both")
+    return offsets if offsets is not None else cu_seqlens
+
+
+def check_varlen_args(q, offsets, head_first, initial_state):
+    """Error behaviour of the reference entry points
+    (``fla/ops/gla/chunk.py:1483-1491`` and the identical blocks elsewhere)."""
+    if offsets is not None:
+        if q.shape[0] != 1:
+            raise ValueError(f"The batch size is expected to be 1 rather than {q.shape[0]} when using `offsets`."
+                             f"Please flatten variable-length inputs before processing.")
+        if head_first:
+            raise RuntimeError("Sequences with variable lengths are not supported for head-first mode")
+        if initial_state is not None and initial_state.shape[0] != len(offsets) - 1:
+            raise ValueError(f"The number of initial states is expected to be equal to the number of input sequences, "
+                             f"i.e., {len(offsets) - 1} rather than {initial_state.shape[0]}.")

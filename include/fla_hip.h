@@ -1,0 +1,145 @@
+/*
+ * C ABI of libfla_hip.so: hand-written gfx950 (MI355X) kernels for the chunked
+ * linear-attention hot path of flash-linear-attention (chunk_gla,
+ * chunk_gated_delta_rule, fused_recurrent_* and the sub-kernels they use).
+ *
+ * Every entry point takes plain device pointers and sizes plus the HIP stream
+ * to launch on, launches asynchronously on that stream, never synchronises
+ * and never allocates.  Return value: 0 on success, a positive hipError_t, or
+ * a negative FLA_E_* code (argument / shape not supported).
+ *
+ * Layout: seq-first.  q,k [B,T,H,K]; v,o [B,T,H,V]; per-head scalars [B,T,H];
+ * recurrent state fp32 [N,H,K,V].  Packed variable-length batches: B == 1,
+ * offsets int64 [N+1] on the device (the reference's `offsets` / newer
+ * `cu_seqlens`).  16-bit tensors are bf16 (FLA_BF16) or fp16 (FLA_F16).
+ *
+ * Each declaration cites the reference interface (path:line in
+ * flash-linear-attention) whose kernel launch it replaces.
+ */
+#ifndef FLA_HIP_H_
+#define FLA_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLA_ABI_VERSION 1
+
+enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
+
+enum fla_error {
+  FLA_OK = 0,
+  FLA_E_INVALID = -1,     /* null pointer / negative size / inconsistent arguments */
+  FLA_E_UNSUPPORTED = -2, /* shape, dtype or chunk size outside what the kernels cover */
+  FLA_E_ALIGNMENT = -3    /* pointer or row pitch not aligned for vector access */
+};
+
+typedef void* fla_stream_t; /* hipStream_t */
+
+int fla_abi_version(void);
+/* Static string for a code returned by any entry point (FLA_E_* or hipError_t). */
+const char* fla_error_string(int code);
+
+/* ------------------------------------------------------------------------
+ * Integer bookkeeping for packed batches (host arithmetic, host pointers).
+ * Replaces prepare_varlen_inputs (fla/ops/gla/chunk.py:1323-1330, inline copy
+ * at fla/ops/gated_delta_rule/chunk.py:204-207) and the chunk-offset prefix
+ * sums (fla/ops/common/chunk_h.py:274-279, chunk_delta_h.py:240-245).
+ * ---------------------------------------------------------------------- */
+/* Total number of chunks sum_n ceil(T_n / chunk_size); negative on bad input. */
+int64_t fla_count_chunks(const int64_t* offsets_host, int64_t n_seqs, int64_t chunk_size);
+/* indices_out [NT,2] = (sequence, chunk in sequence); chunk_offsets_out [N+1]
+ * = exclusive prefix sum of per-sequence chunk counts.  Either may be NULL. */
+int fla_prepare_chunk_indices(const int64_t* offsets_host, int64_t n_seqs, int64_t chunk_size,
+                              int64_t* indices_out, int64_t* chunk_offsets_out);
+
+/* ------------------------------------------------------------------------
+ * chunk_local_cumsum (fla/ops/utils/cumsum.py:389-407; scalar kernel :24-57,
+ * vector kernel :72-110).  g is [B,T,H] (S == 1) or [B,T,H,S] of g_dtype, out
+ * is fp32 of the same shape.  chunk_size is a power of two.  For packed
+ * batches pass offsets [N+1] and indices [NT,2] (device), else NULL.
+ * ---------------------------------------------------------------------- */
+int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype,
+                           int64_t B, int64_t T, int64_t H, int64_t S,
+                           int64_t chunk_size, int reverse,
+                           const int64_t* offsets, const int64_t* indices, int64_t NT,
+                           fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Token-by-token recurrence, forward (fla/ops/common/fused_recurrent.py:322-378,
+ * kernel :27-128).  Any of g [B,T,H], gk [B,T,H,K], gv [B,T,H,V] may be NULL;
+ * the gates have dtype gate_dtype, q,k,v have dtype qkv_dtype and o has dtype
+ * o_dtype.  h0 / ht are fp32 [N,H,K,V] or NULL; ht may alias h0 (state updated
+ * in place - every (n,h) tile is read before it is written by the same
+ * workgroup).  N = B, or the number of packed sequences when offsets != NULL.
+ * ---------------------------------------------------------------------- */
+int fla_fused_recurrent_fwd(const void* q, const void* k, const void* v,
+                            const void* g, const void* gk, const void* gv,
+                            void* o, const float* h0, float* ht,
+                            const int64_t* offsets,
+                            int qkv_dtype, int gate_dtype, int o_dtype,
+                            int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                            float scale, int reverse, fla_stream_t stream);
+
+/* Gated delta rule recurrence, forward
+ * (fla/ops/gated_delta_rule/fused_recurrent.py:113-167, kernel :19-110).
+ * g [B,T,H] or NULL; beta [B,T,H] (beta_per_value == 0) or [B,T,H,V]
+ * (beta_per_value == 1), NULL meaning 1.  g and beta have dtype gate_dtype. */
+int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const void* k, const void* v,
+                                             const void* g, const void* beta,
+                                             void* o, const float* h0, float* ht,
+                                             const int64_t* offsets,
+                                             int qkv_dtype, int gate_dtype, int o_dtype,
+                                             int beta_per_value,
+                                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                             int64_t N, float scale, fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Chunked GLA forward (chunk size 64).
+ *
+ * fla_chunk_gla_fwd_h: inter-chunk state scan, replaces chunk_fwd_h with gk
+ * (fla/ops/common/chunk_h.py:282-335, kernel :29-137).  gates are the raw
+ * log-gates gk [B,T,H,K] (gates_are_cumsum == 0, the chunk-local prefix sum
+ * is formed in the kernel) or their chunk-local cumsum (== 1, fp32 only).
+ * h receives the state ENTERING every chunk, [B,NT,H,K,V] (packed:
+ * [1,NT_total,H,K,V], addressed through chunk_offsets [N+1]); h_layout selects
+ *   FLA_H_ROW_MAJOR  plain [K,V] tiles of dtype h_dtype (the reference layout),
+ *   FLA_H_FRAGMENT   bf16/fp16 tiles in MFMA-fragment order, consumed only by
+ *                    fla_chunk_gla_fwd_o / fla_chunk_fwd_o (same byte size).
+ * h may be NULL when only ht is wanted.  h0, ht fp32 [N,H,K,V] or NULL.
+ *
+ * fla_chunk_gla_fwd_o: fused cumsum + intra-chunk gated scores + output,
+ * replaces chunk_gla_fwd_intra_gk + chunk_gla_fwd_o_gk
+ * (fla/ops/gla/chunk.py:840-938 kernels :29-170; :941-979 kernel :320-393).
+ * h must be FLA_H_FRAGMENT.  A_out (optional, fp32 [B,T,H,64]) receives the
+ * lower-triangular score matrix the reference saves for backward.
+ * ---------------------------------------------------------------------- */
+enum fla_h_layout { FLA_H_ROW_MAJOR = 0, FLA_H_FRAGMENT = 1 };
+
+int fla_chunk_gla_fwd_h(const void* k, const void* v, const void* gates, int gates_are_cumsum,
+                        const float* h0, void* h, float* ht,
+                        const int64_t* offsets, const int64_t* chunk_offsets,
+                        int qkv_dtype, int gate_dtype, int h_dtype, int h_layout,
+                        int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                        fla_stream_t stream);
+
+int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void* gates,
+                        int gates_are_cumsum, const void* h, void* o, float* A_out,
+                        const int64_t* offsets, const int64_t* indices, int64_t NT,
+                        int qkv_dtype, int gate_dtype,
+                        int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                        float scale, fla_stream_t stream);
+
+/* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
+ * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,
+ * mode 1: 16x16x32 tiles, mode 2: 32x32x16 with the permuted contraction order
+ * used for fragment-layout states).  M, N multiples of 32, Kd of 32. */
+int fla_selftest_mfma(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t Kd,
+                      int mode, fla_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLA_HIP_H_ */

@@ -1,0 +1,144 @@
+"""fp32 chunked forms of the two operators, exposing every intermediate.
+
+These restate the chunk algebra the kernels implement so that each kernel can
+be checked on its own:
+
+* GLA (``fla/ops/gla/chunk.py:1156-1214`` for the pipeline order;
+  ``fla/ops/common/chunk_h.py:73-137`` for "the stored state is the one
+  ENTERING the chunk" and ``G_last`` = last valid row;
+  ``fla/ops/gla/chunk.py:29-97,113-170`` for ``A``; ``:320-393`` for ``o``):
+  ``G`` = chunk-local cumsum of ``gk``;
+  ``A_ij = s * sum_k q_ik k_jk exp(G_ik - G_jk)`` for ``j <= i``;
+  ``o_i = (s q_i * exp(G_i))^T h_c + sum_{j<=i} A_ij v_j``;
+  ``h_{c+1} = diag(exp(G_last)) h_c + sum_j (k_j * exp(G_last - G_j)) v_j^T``.
+* gated delta rule (``fla/ops/gated_delta_rule/wy_fast.py:150-208`` for
+  ``Aw, Au``; ``:250-317`` for ``w, u``; ``fla/ops/common/chunk_delta_h.py:71-119``
+  for the scan; ``fla/ops/common/chunk_o.py:68-101`` for ``o``):
+  ``M = strict_lower(diag(beta) K K^T)``, ``Aw = (I + M)^-1``,
+  ``Au = (I + M * Gamma)^-1`` with ``Gamma_ij = exp(gamma_i - gamma_j)``;
+  ``w = Aw (beta * K)``, ``u = Au (beta * V)``;
+  ``v_new = u - (w * exp(gamma)) h_c``;
+  ``o = s (exp(gamma) * (Q h_c) + tril(Q K^T * Gamma) v_new)``;
+  ``h_{c+1} = exp(gamma_last) h_c + (K * exp(gamma_last - gamma))^T v_new``.
+
+No rounding to bf16 anywhere: this is the exact-arithmetic target, so kernel
+intermediates are compared with a tolerance, final outputs against the naive
+recurrences.  Chunks never straddle sequences; tail chunks are short.
+
+Test infrastructure only.
+"""
+from typing import Dict, Optional, Sequence
+
+import torch
+
+from .recurrent import _spans
+
+
+def _chunks(bos: int, eos: int, BT: int):
+    return [(s, min(s + BT, eos)) for s in range(bos, eos, BT)]
+
+
+def chunked_gla(q, k, v, gk, scale=None, initial_state=None, chunk_size=64,
+                offsets: Optional[Sequence[int]] = None,
+                dtype=torch.float32) -> Dict[str, torch.Tensor]:
+    q, k, v, gk = (x.to(dtype) for x in (q, k, v, gk))
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    BT = chunk_size
+    if scale is None:
+        scale = K ** -0.5
+    spans = _spans(B, T, offsets)
+    G = torch.zeros_like(gk)
+    A = torch.zeros(B, T, H, BT, dtype=dtype)
+    o = torch.zeros(B, T, H, V, dtype=dtype)
+    hs, finals = [], []
+    for n, (b, bos, eos) in enumerate(spans):
+        h = torch.zeros(H, K, V, dtype=dtype)
+        if initial_state is not None:
+            h = h + initial_state[n].to(dtype)
+        for s, e in _chunks(bos, eos, BT):
+            L = e - s
+            Gc = torch.cumsum(gk[b, s:e], 0)                    # [L,H,K]
+            G[b, s:e] = Gc
+            hs.append(h)
+            qc, kc, vc = q[b, s:e], k[b, s:e], v[b, s:e]
+            # A_ij = s * sum_k q_ik k_jk exp(G_ik - G_jk), j <= i
+            diff = Gc[:, None] - Gc[None, :]                    # [L,L,H,K]
+            mask = torch.tril(torch.ones(L, L, dtype=torch.bool))
+            diff = torch.where(mask[:, :, None, None], diff, torch.full_like(diff, -float('inf')))
+            Ac = scale * torch.einsum('ihk,jhk,ijhk->ihj', qc, kc, diff.exp())
+            A[b, s:e, :, :L] = Ac
+            o[b, s:e] = (torch.einsum('ihk,hkv->ihv', scale * qc * Gc.exp(), h)
+                         + torch.einsum('ihj,jhv->ihv', Ac, vc))
+            Glast = Gc[-1]                                      # [H,K]
+            kd = kc * (Glast[None] - Gc).exp()
+            h = h * Glast.exp()[:, :, None] + torch.einsum('jhk,jhv->hkv', kd, vc)
+        finals.append(h)
+    if offsets is None:
+        NT = -(-T // BT)
+        h_all = torch.stack(hs, 0).reshape(B, NT, H, K, V) if hs else torch.zeros(B, 0, H, K, V)
+    else:
+        h_all = torch.stack(hs, 0)[None]
+    return dict(g_cumsum=G, A=A, h=h_all, o=o, ht=torch.stack(finals, 0))
+
+
+def chunked_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, chunk_size=64,
+                             offsets: Optional[Sequence[int]] = None,
+                             dtype=torch.float32) -> Dict[str, torch.Tensor]:
+    q, k, v, beta = (x.to(dtype) for x in (q, k, v, beta))
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    BT = chunk_size
+    g = torch.zeros(B, T, H, dtype=dtype) if g is None else g.to(dtype)
+    if scale is None:
+        scale = K ** -0.5
+    spans = _spans(B, T, offsets)
+    gam = torch.zeros_like(g)
+    Aw = torch.zeros(B, T, H, BT, dtype=dtype)
+    Au = torch.zeros(B, T, H, BT, dtype=dtype)
+    w = torch.zeros_like(k)
+    u = torch.zeros_like(v)
+    v_new = torch.zeros_like(v)
+    o = torch.zeros_like(v)
+    hs, finals = [], []
+    for n, (b, bos, eos) in enumerate(spans):
+        h = torch.zeros(H, K, V, dtype=dtype)
+        if initial_state is not None:
+            h = h + initial_state[n].to(dtype)
+        for s, e in _chunks(bos, eos, BT):
+            L = e - s
+            gc = torch.cumsum(g[b, s:e], 0)                     # [L,H]
+            gam[b, s:e] = gc
+            qc, kc, vc, bc = q[b, s:e], k[b, s:e], v[b, s:e], beta[b, s:e]
+            kb = kc * bc[..., None]
+            vb = vc * bc[..., None]
+            eye = torch.eye(L, dtype=dtype)
+            strict = torch.tril(torch.ones(L, L, dtype=dtype), -1)
+            lower = torch.tril(torch.ones(L, L, dtype=dtype))
+            M = torch.einsum('ihk,jhk->hij', kb, kc) * strict    # [H,L,L]
+            Gam = ((gc[:, None] - gc[None, :]).permute(2, 0, 1) * lower).exp() * lower
+            aw = torch.linalg.solve_triangular(eye + M, eye.expand(H, L, L), upper=False)
+            au = torch.linalg.solve_triangular(eye + M * Gam, eye.expand(H, L, L), upper=False)
+            Aw[b, s:e, :, :L] = aw.permute(1, 0, 2)
+            Au[b, s:e, :, :L] = au.permute(1, 0, 2)
+            wc = torch.einsum('hij,jhk->ihk', aw, kb)
+            uc = torch.einsum('hij,jhv->ihv', au, vb)
+            w[b, s:e], u[b, s:e] = wc, uc
+            hs.append(h)
+            eg = gc.exp()                                       # [L,H]
+            vn = uc - torch.einsum('ihk,hkv->ihv', wc * eg[..., None], h)
+            v_new[b, s:e] = vn
+            P = torch.einsum('ihk,jhk->hij', qc, kc) * Gam       # tril by Gam's mask
+            o[b, s:e] = scale * (eg[..., None] * torch.einsum('ihk,hkv->ihv', qc, h)
+                                 + torch.einsum('hij,jhv->ihv', P, vn))
+            glast = gc[-1]                                      # [H]
+            kd = kc * (glast[None] - gc).exp()[..., None]
+            h = h * glast.exp()[:, None, None] + torch.einsum('jhk,jhv->hkv', kd, vn)
+        finals.append(h)
+    if offsets is None:
+        NT = -(-T // BT)
+        h_all = torch.stack(hs, 0).reshape(B, NT, H, K, V) if hs else torch.zeros(B, 0, H, K, V)
+    else:
+        h_all = torch.stack(hs, 0)[None]
+    return dict(g_cumsum=gam, Aw=Aw, Au=Au, w=w, u=u, h=h_all, v_new=v_new, o=o,
+                ht=torch.stack(finals, 0))

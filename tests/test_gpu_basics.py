@@ -1,0 +1,59 @@
+"""GPU: MFMA fragment self-test, chunk_local_cumsum and chunk bookkeeping on device."""
+import ctypes
+
+import pytest
+import torch
+
+from helpers import assert_close, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_mfma_fragment_layout(device, mode):
+    from fla_amd import _backend as be
+    torch.manual_seed(0)
+    M, N, Kd = 64, 96, 128
+    A = torch.randn(M, Kd, device=device).bfloat16()
+    B = torch.randn(N, Kd, device=device).bfloat16()
+    C = torch.full((M, N), float('nan'), device=device)
+    print(f"selftest mode={mode}", flush=True)
+    be.check(be.lib().fla_selftest_mfma(be.ptr(A), be.ptr(B), be.ptr(C), M, N, Kd, mode, be.stream_of(A)), "selftest")
+    torch.cuda.synchronize()
+    ref = A.float() @ B.float().t()
+    assert_close(f"mfma mode {mode}", ref, C, 1e-5)
+
+
+@pytest.mark.parametrize("shape", [(2, 300, 4, 64), (1, 150, 3, 100), (2, 1024, 2, 0), (3, 77, 5, 0), (1, 64, 2, 6)])
+@pytest.mark.parametrize("chunk", [32, 64])
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cumsum_fixed(device, shape, chunk, reverse, dtype):
+    from fla_amd.ops.utils import chunk_local_cumsum
+    from oracle.cumsum import chunk_local_cumsum as ref_cumsum
+    B, T, H, S = shape
+    gen = torch.Generator().manual_seed(1)
+    g = torch.randn((B, T, H, S) if S else (B, T, H), generator=gen).to(dtype)
+    print(f"cumsum {shape} chunk={chunk} reverse={reverse} {dtype}", flush=True)
+    out = chunk_local_cumsum(g.to(device), chunk, reverse=reverse, head_first=False)
+    assert out.dtype == torch.float32
+    ref = ref_cumsum(g, chunk, reverse=reverse)
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)
+    # head-first entry point
+    out_hf = chunk_local_cumsum(g.transpose(1, 2).contiguous().to(device), chunk, reverse=reverse, head_first=True)
+    torch.testing.assert_close(out_hf.transpose(1, 2).cpu(), ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("T,N", [(64, 2), (300, 4), (1000, 7), (2048, 4)])
+@pytest.mark.parametrize("S", [0, 100])
+@pytest.mark.parametrize("reverse", [False, True])
+def test_cumsum_varlen(device, T, N, S, reverse):
+    from fla_amd.ops.utils import chunk_local_cumsum
+    from oracle.cumsum import chunk_local_cumsum as ref_cumsum
+    gen = torch.Generator().manual_seed(2)
+    offs = random_offsets(T, N, gen, min_len=1)
+    g = torch.randn((1, T, 3, S) if S else (1, T, 3), generator=gen)
+    print(f"cumsum varlen T={T} N={N} S={S} offs={offs.tolist()}", flush=True)
+    out = chunk_local_cumsum(g.to(device), 64, reverse=reverse, offsets=offs.to(device), head_first=False)
+    ref = ref_cumsum(g, 64, reverse=reverse, offsets=offs.tolist())
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)

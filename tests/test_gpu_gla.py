@@ -1,0 +1,116 @@
+"""GPU: chunk_gla forward against the fp32 naive recurrence (tolerances of the
+north star: rel-L2 <= 1e-2 on o, <= 5e-3 on the final state, bf16 inputs)."""
+import pytest
+import torch
+
+from helpers import assert_close, gla_inputs, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+TOL_O, TOL_HT = 1e-2, 5e-3
+
+
+def _run(device, q, k, v, g, h0, offsets=None, head_first=False, scale=None):
+    from fla_amd.ops.gla import chunk_gla
+    dev = lambda x: None if x is None else x.to(device)
+    if head_first:
+        q, k, v, g = (x.transpose(1, 2).contiguous() for x in (q, k, v, g))
+    o, ht = chunk_gla(dev(q), dev(k), dev(v), dev(g), scale=scale, initial_state=dev(h0), output_final_state=True,
+                      offsets=dev(offsets), head_first=head_first)
+    torch.cuda.synchronize()
+    if head_first:
+        o = o.transpose(1, 2)
+    return o, ht
+
+
+def test_chunk_gla_config0(device):
+    """BASELINE config 0 shape (B=2, T=256, H=4, K=V=64, zero initial state), bf16 storage."""
+    from oracle.recurrent import naive_recurrent_gla
+    q, k, v, g, _ = gla_inputs(2, 256, 4, 64, 64, seed=0, h0=False)
+    print("chunk_gla config0", flush=True)
+    o, ht = _run(device, q, k, v, g, None)
+    ro, rht = naive_recurrent_gla(q, k, v, g, output_final_state=True)
+    assert o.dtype == torch.bfloat16 and ht.dtype == torch.float32
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("T", [1, 63, 64, 65, 130, 300, 1024])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
+def test_chunk_gla_shapes(device, T, K, V):
+    from oracle.recurrent import naive_recurrent_gla
+    q, k, v, g, h0 = gla_inputs(2, T, 3, K, V, seed=T + K, normalizer=16.0)
+    print(f"chunk_gla T={T} K={K} V={V}", flush=True)
+    o, ht = _run(device, q, k, v, g, h0)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("normalizer", [1.0, 16.0, 20.0])
+@pytest.mark.parametrize("gate_dtype", [torch.float32, torch.bfloat16])
+def test_chunk_gla_gates(device, normalizer, gate_dtype):
+    """Gate magnitudes of the reference sweep (tests/ops/test_gla.py:90-146) that stay
+    inside the single-reference-point range, in fp32 and in bf16 storage."""
+    from oracle.recurrent import naive_recurrent_gla
+    q, k, v, g, h0 = gla_inputs(2, 300, 4, 128, 128, seed=11, normalizer=normalizer, h0_std=1.0)
+    g = g.to(gate_dtype)
+    print(f"chunk_gla normalizer={normalizer} gates {gate_dtype}", flush=True)
+    o, ht = _run(device, q, k, v, g, h0)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+def test_chunk_gla_head_first_scale_and_odd_dims(device):
+    from oracle.recurrent import naive_recurrent_gla
+    q, k, v, g, h0 = gla_inputs(2, 200, 2, 100, 100, seed=12)
+    print("chunk_gla head-first D=100 scale=0.2", flush=True)
+    o, ht = _run(device, q, k, v, g, h0, head_first=True, scale=0.2)
+    ro, rht = naive_recurrent_gla(q, k, v, g, scale=0.2, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("T,N", [(64, 2), (300, 4), (1000, 5), (2048, 4)])
+def test_chunk_gla_varlen(device, T, N):
+    """Packed batches (tests/ops/test_gla.py:149-201): equals the per-sequence recurrence."""
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(T)
+    offs = random_offsets(T, N, gen, min_len=1)
+    q, k, v, g, h0 = gla_inputs(1, T, 4, 128, 128, seed=13, N=N, h0_std=1.0)
+    print(f"chunk_gla varlen T={T} offs={offs.tolist()}", flush=True)
+    o, ht = _run(device, q, k, v, g, h0, offsets=offs)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True, offsets=offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+def test_chunk_gla_intermediates(device):
+    """The reference-shaped internal forward: g_cumsum, A, per-chunk h against the fp32 chunked oracle."""
+    from fla_amd.ops.gla.chunk import chunk_gla_fwd
+    from oracle.chunked import chunked_gla
+    q, k, v, g, h0 = gla_inputs(2, 200, 2, 128, 128, seed=14)
+    dev = lambda x: x.to(device)
+    print("chunk_gla_fwd intermediates", flush=True)
+    gc, A, h, ht, o = chunk_gla_fwd(dev(q), dev(k), dev(v), dev(g), None, 128 ** -0.5, dev(h0), True,
+                                    head_first=False, chunk_size=64)
+    ref = chunked_gla(q, k, v, g, initial_state=h0)
+    torch.testing.assert_close(gc.cpu(), ref['g_cumsum'], rtol=1e-5, atol=1e-5)
+    assert_close("A", ref['A'], A, 1e-2)
+    assert_close("h", ref['h'], h, 5e-3)
+    assert_close("ht", ref['ht'], ht, TOL_HT)
+    assert_close("o", ref['o'], o, TOL_O)
+    assert (A.cpu().reshape(2, 200, 2, 64)[:, 0, :, 1:] == 0).all()  # strictly upper part is zero
+
+
+def test_chunk_gla_segment_chaining(device):
+    """run(T1) -> ht -> run(T2, h0=ht) equals run(T1+T2)."""
+    q, k, v, g, h0 = gla_inputs(2, 320, 2, 128, 128, seed=15)
+    print("chunk_gla chaining", flush=True)
+    o_full, ht_full = _run(device, q, k, v, g, h0)
+    cut = 192
+    o1, h1 = _run(device, q[:, :cut], k[:, :cut], v[:, :cut], g[:, :cut], h0)
+    o2, h2 = _run(device, q[:, cut:], k[:, cut:], v[:, cut:], g[:, cut:], h1.cpu())
+    assert_close("o chained", o_full.float(), torch.cat([o1, o2], 1).float(), 4e-3)
+    assert_close("ht chained", ht_full, h2, 1e-5)

@@ -1,0 +1,134 @@
+"""GPU: token-by-token recurrences (prefill and the T=1 decode step) against the
+fp32 naive recurrences of the oracle on the same seeded inputs."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import assert_close, gdr_inputs, gla_inputs, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+
+# shapes follow the reference ladder (tests/ops/test_gla.py:29-87): fp32, h0 ~ N(0,1)
+@pytest.mark.parametrize("T", [1, 7, 300])
+@pytest.mark.parametrize("D", [32, 64, 100, 128])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_recurrent_gla(device, T, D, dtype):
+    from fla_amd.ops.gla import fused_recurrent_gla
+    from oracle.recurrent import naive_recurrent_gla
+    B, H = 2, 3
+    q, k, v, g, h0 = gla_inputs(B, T, H, D, D, seed=3, dtype=dtype, normalizer=1.0, h0_std=1.0)
+    print(f"recurrent gla T={T} D={D} {dtype}", flush=True)
+    o, ht = fused_recurrent_gla(q.to(device), k.to(device), v.to(device), g.to(device), initial_state=h0.to(device),
+                                output_final_state=True, head_first=False)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+    tol = 1e-5 if dtype == torch.float32 else 5e-3
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    assert_close("o", ro, o, tol)
+    assert_close("ht", rht, ht, 1e-5)
+
+
+def test_fused_recurrent_gla_variants(device):
+    """g / gv gates, reverse, head-first, no initial state, K != V."""
+    from fla_amd.ops.common.fused_recurrent import fused_recurrent
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(4)
+    B, T, H, K, V = 2, 37, 2, 64, 128
+    q, k, v = torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, K, generator=gen), torch.randn(B, T, H, V, generator=gen)
+    gk = F.logsigmoid(torch.randn(B, T, H, K, generator=gen))
+    gv = F.logsigmoid(torch.randn(B, T, H, V, generator=gen))
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    for kwargs in [dict(g=g), dict(gv=gv), dict(gk=gk, gv=gv, g=g), dict(gk=gk, reverse=True), dict()]:
+        print(f"recurrent variants {list(kwargs)}", flush=True)
+        dev = {n: (x.to(device) if torch.is_tensor(x) else x) for n, x in kwargs.items()}
+        o, ht = fused_recurrent(q.to(device), k.to(device), v.to(device), output_final_state=True, head_first=False, **dev)
+        ro, rht = naive_recurrent_gla(q, k, v, output_final_state=True, **kwargs)
+        assert_close("o", ro, o, 1e-5)
+        assert_close("ht", rht, ht, 1e-5)
+    tr = lambda x: x.transpose(1, 2).contiguous().to(device)
+    o, ht = fused_recurrent(tr(q), tr(k), tr(v), gk=tr(gk), output_final_state=True, head_first=True)
+    ro, rht = naive_recurrent_gla(q, k, v, gk, output_final_state=True)
+    assert_close("o head-first", ro.transpose(1, 2), o, 1e-5)
+    assert_close("ht head-first", rht, ht, 1e-5)
+
+
+@pytest.mark.parametrize("T,N", [(64, 2), (300, 4), (1000, 5)])
+def test_fused_recurrent_gla_varlen(device, T, N):
+    from fla_amd.ops.gla import fused_recurrent_gla
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(5)
+    offs = random_offsets(T, N, gen)
+    q, k, v, g, h0 = gla_inputs(1, T, 2, 64, 64, seed=5, dtype=torch.float32, normalizer=1.0, N=N, h0_std=1.0)
+    print(f"recurrent gla varlen offs={offs.tolist()}", flush=True)
+    o, ht = fused_recurrent_gla(q.to(device), k.to(device), v.to(device), g.to(device), initial_state=h0.to(device),
+                                output_final_state=True, offsets=offs.to(device), head_first=False)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True, offsets=offs.tolist())
+    assert_close("o", ro, o, 1e-5)
+    assert_close("ht", rht, ht, 1e-5)
+
+
+# reference ladder: tests/ops/test_gated_delta.py:161-217 (bf16, k L2-normalised, h0 ~ N(0,1), tol 0.002)
+@pytest.mark.parametrize("T", [1, 7, 63, 300])
+@pytest.mark.parametrize("H", [2, 16])
+@pytest.mark.parametrize("D", [64, 100, 128, 200])
+def test_fused_recurrent_gated_delta_rule(device, T, H, D):
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = gdr_inputs(2, T, H, D, D, seed=6, h0_std=1.0)
+    print(f"recurrent gdr T={T} H={H} D={D}", flush=True)
+    o, ht = fused_recurrent_gated_delta_rule(q.to(device), k.to(device), v.to(device), g.to(device), beta.to(device),
+                                             initial_state=h0.to(device), output_final_state=True, head_first=False)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    assert o.dtype == q.dtype
+    assert_close("o", ro, o, 5e-3)
+    assert_close("ht", rht, ht, 2e-3)
+
+
+def test_fused_recurrent_gated_delta_rule_variants(device):
+    """fp32 inputs, per-value beta, beta=None, varlen, scale argument."""
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(7)
+    T, H, K, V, N = 200, 3, 64, 128, 3
+    q, k, v, g, beta, h0 = gdr_inputs(1, T, H, K, V, seed=7, dtype=torch.float32, N=N, h0_std=1.0)
+    offs = random_offsets(T, N, gen)
+    bv = torch.rand(1, T, H, V, generator=gen)
+    for name, b in [("scalar", beta), ("per-value", bv), ("none", None)]:
+        print(f"gdr variants beta={name}", flush=True)
+        o, ht = fused_recurrent_gated_delta_rule(q.to(device), k.to(device), v.to(device), g.to(device),
+                                                 None if b is None else b.to(device), scale=0.3,
+                                                 initial_state=h0.to(device), output_final_state=True,
+                                                 offsets=offs.to(device), head_first=False)
+        ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, b, scale=0.3, initial_state=h0,
+                                                   output_final_state=True, offsets=offs.tolist())
+        assert_close("o", ro, o, 1e-5)
+        assert_close("ht", rht, ht, 1e-5)
+
+
+@pytest.mark.parametrize("op", ["gla", "gdr"])
+def test_decode_inplace_matches_out_of_place(device, op):
+    """T=1 decode steps: the in-place state update equals the out-of-place one, and a
+    run of single steps equals one recurrent call over the whole span."""
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from fla_amd.ops.gla import fused_recurrent_gla
+    B, H, D, steps = 4, 4, 128, 5
+    if op == "gla":
+        q, k, v, g, h0 = gla_inputs(B, steps, H, D, D, seed=8, normalizer=1.0)
+        args = [x.to(device) for x in (q, k, v, g)]
+        fn = fused_recurrent_gla
+    else:
+        q, k, v, g, beta, h0 = gdr_inputs(B, steps, H, D, D, seed=8)
+        args = [x.to(device) for x in (q, k, v, g, beta)]
+        fn = fused_recurrent_gated_delta_rule
+    h0 = h0.to(device)
+    o_all, ht_all = fn(*args, initial_state=h0, output_final_state=True, head_first=False)
+    state_a = h0.clone()   # out-of-place chain
+    state_b = h0.clone()   # in-place chain
+    for t in range(steps):
+        step = [x[:, t:t + 1].contiguous() for x in args]
+        o_a, state_a = fn(*step, initial_state=state_a, output_final_state=True, head_first=False)
+        o_b, ret = fn(*step, initial_state=state_b, output_final_state=True, head_first=False, inplace_state=True)
+        assert ret.data_ptr() == state_b.data_ptr()
+        assert torch.equal(o_a, o_b) and torch.equal(state_a, state_b)
+        assert torch.equal(o_a, o_all[:, t:t + 1])
+    assert torch.equal(state_b, ht_all)
