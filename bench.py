@@ -1,0 +1,237 @@
+#!/usr/bin/env python3
+"""Benchmark of the chunked linear-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one chunk_gla forward over BASELINE config 1 (B=8, T=4096, H=16,
+K=V=128, bf16 q/k/v, fp32 log-gates and state, initial state given, final state
+returned), inputs resident in HBM.  Prints ONE JSON line:
+
+* value            tokens/s of the whole forward (B*T*steps / elapsed)
+* roofline         the dominant kernel of that forward against the HBM roofline:
+                   algorithmic bytes per launch / its average duration measured
+                   here with HIP events on the launch stream
+* cpu_baseline     the oracle's fp32 naive recurrence timed on the host cores on
+                   a bounded sample of the same workload
+* extra            the other measured rows (chunk_gated_delta_rule forward on
+                   config 2 when built, the T=1 decode steps of config 3)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "flash-linear-attention_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+MIB = 1 << 20
+
+
+def _events(n):
+    import torch
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_steps(fn, steps, warmup):
+    """Wall time of exactly `steps` calls, bracketed by synchronize on both sides."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def event_avg_us(fn, steps, warmup=3):
+    """Average device time of one call, HIP events recorded on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = _events(2 * steps)
+    for i in range(steps):
+        ev[2 * i].record()
+        fn()
+        ev[2 * i + 1].record()
+    torch.cuda.synchronize()
+    return sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(steps)) / steps * 1e3
+
+
+def gla_config1(device):
+    import torch
+    import torch.nn.functional as F
+    torch.manual_seed(0)
+    B, T, H, K, V = 8, 4096, 16, 128, 128
+    q = torch.randn(B, T, H, K, device=device).bfloat16()
+    k = torch.randn(B, T, H, K, device=device).bfloat16()
+    v = torch.randn(B, T, H, V, device=device).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, K, device=device)) / 16
+    h0 = torch.randn(B, H, K, V, device=device) * 0.1
+    return dict(B=B, T=T, H=H, K=K, V=V, q=q, k=k, v=v, g=g, h0=h0)
+
+
+def bench_gla(device, steps, warmup):
+    import torch
+    from fla_amd.ops.common.chunk_h import chunk_fwd_h
+    from fla_amd.ops.gla import chunk_gla
+    from fla_amd.ops.gla.chunk import chunk_gla_fwd_o_gk
+    c = gla_config1(device)
+    q, k, v, g, h0 = c["q"], c["k"], c["v"], c["g"], c["h0"]
+    B, T, H, K, V = c["B"], c["T"], c["H"], c["K"], c["V"]
+
+    def step():
+        return chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
+
+    elapsed = time_steps(step, steps, warmup)
+    ms = elapsed / steps * 1e3
+    tokens_per_s = B * T * steps / elapsed
+
+    # per-kernel device time, each entry point launched on its own between events
+    h_hold = {}
+
+    def run_h():
+        h_hold["h"], h_hold["ht"] = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=h0, output_final_state=True,
+                                                head_first=False, chunk_size=64, gates_are_cumsum=False,
+                                                fragment_layout=True)
+
+    run_h()
+    scale = K ** -0.5
+
+    def run_o():
+        chunk_gla_fwd_o_gk(q, v, g, None, h_hold["h"], scale, head_first=False, chunk_size=64, k=k,
+                           gates_are_cumsum=False)
+
+    n_ev = max(steps, 10)
+    us_h = event_avg_us(run_h, n_ev)
+    us_o = event_avg_us(run_o, n_ev)
+    NT = T // 64
+    qkv = B * T * H * K * 2                      # one bf16 [B,T,H,128] tensor
+    gbytes = B * T * H * K * 4                   # fp32 gates
+    hbytes = B * NT * H * K * V * 2              # bf16 per-chunk states
+    st = B * H * K * V * 4                       # one fp32 state
+    bytes_h = 2 * qkv + gbytes + hbytes + 2 * st           # k, v, g in; h, ht out; h0 in
+    bytes_o = 3 * qkv + gbytes + hbytes + qkv              # q, k, v, g, h in; o out
+    kernels = {
+        "gla_fwd_h_kernel": dict(us=us_h, bytes=bytes_h),
+        "gla_fwd_o_kernel": dict(us=us_o, bytes=bytes_o),
+    }
+    dom = max(kernels, key=lambda n: kernels[n]["us"])
+    ach = kernels[dom]["bytes"] / (kernels[dom]["us"] * 1e-6) / 1e9
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_us": round(kernels[dom]["us"], 1), "bytes_per_launch": kernels[dom]["bytes"]}
+    floor_bytes = 4 * qkv + gbytes + 2 * st      # q,k,v,o + g + h0,ht: the op's algorithmic floor
+    op = {"algorithmic_bytes": floor_bytes, "achieved_GBs": round(floor_bytes / (ms * 1e-3) / 1e9, 1),
+          "frac_of_hbm_peak": round(floor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+          "kernels_us": {n: round(kv["us"], 1) for n, kv in kernels.items()},
+          "kernels_GBs": {n: round(kv["bytes"] / (kv["us"] * 1e-6) / 1e9, 1) for n, kv in kernels.items()}}
+    return ms, tokens_per_s, roofline, op, c
+
+
+def bench_decode(device, steps=1000):
+    """BASELINE config 3: B=256, H=32, K=V=128 single-token step, state in place."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from fla_amd.ops.gla import fused_recurrent_gla
+    torch.manual_seed(0)
+    B, H, K, V = 256, 32, 128, 128
+    out = {}
+    q = torch.randn(B, 1, H, K, device=device).bfloat16()
+    kk = torch.randn(B, 1, H, K, device=device)
+    v = torch.randn(B, 1, H, V, device=device).bfloat16()
+    gk = F.logsigmoid(torch.randn(B, 1, H, K, device=device))
+    g = F.logsigmoid(torch.randn(B, 1, H, device=device))
+    beta = torch.rand(B, 1, H, device=device).sigmoid()
+    state_bytes = B * H * K * V * 4
+    small = B * H * 128 * 2
+    for name in ("gla", "gdr"):
+        S = torch.randn(B, H, K, V, device=device) * 0.1
+        if name == "gla":
+            k = kk.bfloat16()
+            fn = lambda: fused_recurrent_gla(q, k, v, gk, initial_state=S, output_final_state=True,
+                                             head_first=False, inplace_state=True)
+            nbytes = 2 * state_bytes + 4 * small + B * H * K * 4
+        else:
+            k = F.normalize(kk, dim=-1).bfloat16()
+            fn = lambda: fused_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=S,
+                                                          output_final_state=True, head_first=False,
+                                                          inplace_state=True)
+            nbytes = 2 * state_bytes + 4 * small + 2 * B * H * 4
+        elapsed = time_steps(fn, steps, 20)
+        us = elapsed / steps * 1e6
+        assert torch.isfinite(S).all()
+        out[name] = {"us_per_step": round(us, 1), "tokens_per_s": round(B / (us * 1e-6), 1),
+                     "GBs": round(nbytes / (us * 1e-6) / 1e9, 1),
+                     "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     "bytes_per_step": nbytes, "steps": steps}
+    return out
+
+
+def cpu_baseline(c, budget_s=15.0):
+    """The oracle's fp32 naive recurrence on the host cores, over as many whole
+    sequences of the same workload as fit in about `budget_s` seconds."""
+    import torch
+    from oracle.recurrent import naive_recurrent_gla
+    B = c["B"]
+    tokens, spent, used = 0, 0.0, 0
+    for b in range(B):
+        q, k, v, g, h0 = (c[n][b:b + 1].float().cpu() for n in ("q", "k", "v", "g", "h0"))
+        t0 = time.perf_counter()
+        naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+        dt = time.perf_counter() - t0
+        tokens += q.shape[1]
+        spent += dt
+        used += 1
+        if spent + dt > budget_s:
+            break
+    return {"value": round(tokens / spent, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+            "kind": "port", "seconds": round(spent, 2),
+            "sample": f"oracle naive_recurrent_gla (torch CPU fp32) on batch elements 0..{used - 1} of {B} "
+                      f"(T={c['T']}, H={c['H']}, K=V=128 each), one repetition"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build measures one GPU only (every (sequence, head) pair is independent; "
+              "nothing here uses a second GPU). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    ms, tps, roofline, op, cfg = bench_gla(device, a.steps, a.warmup)
+    extra = {"chunk_gla_fwd": op}
+    if not a.no_extra:
+        extra["decode_step"] = bench_decode(device)
+    out = {
+        "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
+        "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "chunk_gla forward, BASELINE config 1: B=8 T=4096 H=16 K=V=128, bf16 q/k/v, "
+                               "fp32 log-gates logsigmoid(N(0,1))/16, fp32 initial state, final state returned"},
+        "roofline": roofline,
+        "cpu_baseline": None if a.no_cpu_baseline else cpu_baseline(cfg),
+        "extra": extra,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

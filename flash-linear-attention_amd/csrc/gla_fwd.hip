@@ -89,13 +89,21 @@ struct HParams {
 };
 
 // HL: 0 row-major [K,V] in T, 1 fragment order in T, 2 row-major fp32.
+//
+// Only the decay multiply and four MFMAs per chunk depend on the running
+// state; loading, the prefix sum, the exponentials and the LDS staging do not.
+// The loop is therefore software-pipelined: global loads run two chunks ahead
+// in registers, the operand tiles are double-buffered in LDS, and the prefix
+// sum across the 8 row groups of a column is done with wave shuffles, so a
+// chunk costs a single workgroup barrier.
 template <typename T, typename GT, bool GCUM, int HL>
 __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
   typedef typename Elem<T>::v8 v8;
-  __shared__ __attribute__((aligned(16))) T sKt[64 * LDT];  // [k][t] decayed keys
-  __shared__ __attribute__((aligned(16))) T sVt[64 * LDT];  // [v][t]
-  __shared__ __attribute__((aligned(16))) float sPart[8 * 64];
-  __shared__ __attribute__((aligned(16))) float sDecay[64];
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  typedef GT g2 __attribute__((ext_vector_type(2)));
+  __shared__ __attribute__((aligned(16))) T sKt[2][64 * LDT];  // [k][t] decayed keys
+  __shared__ __attribute__((aligned(16))) T sVt[2][64 * LDT];  // [v][t]
+  __shared__ __attribute__((aligned(16))) float sDecay[2][64];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H, K = p.K, V = p.V;
@@ -109,8 +117,8 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
   const int64_t nchunks = (sp.len + BT - 1) / BT;
   const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
 
-  // load mapping: 8 row groups x 32 column pairs
-  const int rg = tid >> 5, c2 = (tid & 31) * 2;
+  // load mapping: a wave owns 16 columns; lane = (row group of 8 rows, column pair)
+  const int rg = lane >> 3, c2 = wave * 16 + (lane & 7) * 2;
   const T* kp = (const T*)p.k + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
   const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
   const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + c2;
@@ -126,29 +134,37 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
     for (int r = 0; r < 16; ++r) acc[r] = h0p[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
   }
 
-  float gq[8][2], kk[8][2], vv[8][2];
-  auto load_chunk = [&](int64_t c) {
+  struct Regs {
+    g2 g[8];
+    t2 k[8];
+    t2 v[8];
+  };
+  auto load_chunk = [&](int64_t c, Regs& R) {
     int64_t t0 = c * BT;
     int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       int row = rg * 8 + i;
-      if (row < L) {
-        Load<GT>::x2(gp + (t0 + row) * kstride, gq[i]);
-        Load<T>::x2(kp + (t0 + row) * kstride, kk[i]);
-        Load<T>::x2(vp + (t0 + row) * vstride, vv[i]);
+      if (c < nchunks && row < L) {
+        R.g[i] = *(const g2*)(gp + (t0 + row) * kstride);
+        R.k[i] = *(const t2*)(kp + (t0 + row) * kstride);
+        R.v[i] = *(const t2*)(vp + (t0 + row) * vstride);
       } else {
-        gq[i][0] = gq[i][1] = 0.f;
-        kk[i][0] = kk[i][1] = 0.f;
-        vv[i][0] = vv[i][1] = 0.f;
+        R.g[i] = g2{(GT)0.f, (GT)0.f};
+        R.k[i] = t2{(T)0.f, (T)0.f};
+        R.v[i] = t2{(T)0.f, (T)0.f};
       }
     }
   };
 
-  if (nchunks > 0) load_chunk(0);
+  Regs R0, R1, R2;
+  load_chunk(0, R0);
+  load_chunk(1, R1);
   for (int64_t c = 0; c < nchunks; ++c) {
+    const int buf = (int)(c & 1);
     int64_t t0 = c * BT;
     int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+    load_chunk(c + 2, R2);
     // ---- state entering chunk c
     if (p.h) {
       int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
@@ -173,50 +189,48 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
       }
     }
     // ---- chunk-local prefix sums of the gates (or pick up the given ones)
-    float G[8][2];
+    float G[8][2], glast0, glast1;
     if (!GCUM) {
       float r0 = 0.f, r1 = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        r0 += gq[i][0];
-        r1 += gq[i][1];
+        r0 += (float)R0.g[i][0];
+        r1 += (float)R0.g[i][1];
         G[i][0] = r0;
         G[i][1] = r1;
       }
-      *(f32x2*)&sPart[rg * 64 + c2] = f32x2{r0, r1};
-    } else {
+      // inclusive scan of the row-group totals across lanes 8 apart
+      float s0 = r0, s1 = r1;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        G[i][0] = gq[i][0];
-        G[i][1] = gq[i][1];
-      }
-      if (((L - 1) >> 3) == rg) *(f32x2*)&sPart[c2] = f32x2{G[(L - 1) & 7][0], G[(L - 1) & 7][1]};
-    }
-    __syncthreads();  // (A) partial sums visible; previous chunk's MFMA reads of sKt/sVt are done
-    float glast0, glast1;
-    if (!GCUM) {
-      float off0 = 0.f, off1 = 0.f, tot0 = 0.f, tot1 = 0.f;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        f32x2 pr = *(const f32x2*)&sPart[r * 64 + c2];
-        if (r < rg) {
-          off0 += pr[0];
-          off1 += pr[1];
+      for (int d = 8; d < 64; d <<= 1) {
+        float u0 = __shfl_up(s0, d, 64), u1 = __shfl_up(s1, d, 64);
+        if (lane >= d) {
+          s0 += u0;
+          s1 += u1;
         }
-        tot0 += pr[0];
-        tot1 += pr[1];
       }
+      float off0 = s0 - r0, off1 = s1 - r1;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         G[i][0] += off0;
         G[i][1] += off1;
       }
-      glast0 = tot0;
-      glast1 = tot1;
+      glast0 = __shfl(s0, 56 + (lane & 7), 64);
+      glast1 = __shfl(s1, 56 + (lane & 7), 64);
     } else {
-      f32x2 pr = *(const f32x2*)&sPart[c2];
-      glast0 = pr[0];
-      glast1 = pr[1];
+      float l0 = 0.f, l1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        G[i][0] = (float)R0.g[i][0];
+        G[i][1] = (float)R0.g[i][1];
+        if (i == ((L - 1) & 7)) {
+          l0 = G[i][0];
+          l1 = G[i][1];
+        }
+      }
+      int src = ((L - 1) >> 3) * 8 + (lane & 7);
+      glast0 = __shfl(l0, src, 64);
+      glast1 = __shfl(l1, src, 64);
     }
     {
       v8 ka, kb, va, vb;
@@ -225,28 +239,30 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
         bool valid = (rg * 8 + i) < L;
         float e0 = valid ? __expf(glast0 - G[i][0]) : 0.f;
         float e1 = valid ? __expf(glast1 - G[i][1]) : 0.f;
-        ka[i] = (T)(kk[i][0] * e0);
-        kb[i] = (T)(kk[i][1] * e1);
-        va[i] = (T)vv[i][0];
-        vb[i] = (T)vv[i][1];
+        ka[i] = (T)((float)R0.k[i][0] * e0);
+        kb[i] = (T)((float)R0.k[i][1] * e1);
+        va[i] = R0.v[i][0];
+        vb[i] = R0.v[i][1];
       }
-      *(v8*)&sKt[(c2 + 0) * LDT + rg * 8] = ka;
-      *(v8*)&sKt[(c2 + 1) * LDT + rg * 8] = kb;
-      *(v8*)&sVt[(c2 + 0) * LDT + rg * 8] = va;
-      *(v8*)&sVt[(c2 + 1) * LDT + rg * 8] = vb;
-      if (rg == 0) *(f32x2*)&sDecay[c2] = f32x2{__expf(glast0), __expf(glast1)};
+      *(v8*)&sKt[buf][(c2 + 0) * LDT + rg * 8] = ka;
+      *(v8*)&sKt[buf][(c2 + 1) * LDT + rg * 8] = kb;
+      *(v8*)&sVt[buf][(c2 + 0) * LDT + rg * 8] = va;
+      *(v8*)&sVt[buf][(c2 + 1) * LDT + rg * 8] = vb;
+      if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
     }
-    if (c + 1 < nchunks) load_chunk(c + 1);  // in flight across the barrier and the MFMAs
-    __syncthreads();  // (B) operand tiles complete
+    __syncthreads();  // tiles of chunk c complete; buffer buf^1 is free again after the next barrier
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      f32x4 d = *(const f32x4*)&sDecay[kq * 32 + 8 * a + 4 * (lane >> 5)];
+      f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];
 #pragma unroll
       for (int b = 0; b < 4; ++b) acc[4 * a + b] *= d[b];
     }
 #pragma unroll
     for (int s = 0; s < BT; s += 16)
-      acc = Elem<T>::mfma32(lds_frag32<T>(sKt, LDT, kq * 32, s, lane), lds_frag32<T>(sVt, LDT, vq * 32, s, lane), acc);
+      acc = Elem<T>::mfma32(lds_frag32<T>(sKt[buf], LDT, kq * 32, s, lane),
+                            lds_frag32<T>(sVt[buf], LDT, vq * 32, s, lane), acc);
+    R0 = R1;
+    R1 = R2;
   }
   if (p.ht) {
     float* htp = p.ht + (int64_t)nh * K * V;

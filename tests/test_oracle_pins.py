@@ -1,0 +1,268 @@
+"""CPU: pin the oracle against facts that do not come from the oracle itself -
+closed forms, special cases that reduce to library routines, brute force on
+tiny inputs, the one integer known answer the reference holds, and gradcheck."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import bookkeeping, chunked, cumsum, recurrent
+
+D = torch.float64
+
+
+def _rand(*shape, seed=0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=D)
+
+
+# ---------------------------------------------------------------- bookkeeping (integer, bit exact)
+def test_chunk_indices_known_answer():
+    # fla/ops/gla/chunk.py:1352-1355: offsets [0,100,356], chunk 64
+    idx = bookkeeping.prepare_chunk_indices([0, 100, 356], 64)
+    assert idx.dtype == np.int64
+    assert idx.tolist() == [[0, 0], [0, 1], [1, 0], [1, 1], [1, 2], [1, 3]]
+    assert bookkeeping.prepare_chunk_offsets([0, 100, 356], 64).tolist() == [0, 2, 6]
+
+
+@pytest.mark.parametrize("bt", [16, 32, 64])
+def test_chunk_indices_bruteforce(bt):
+    rng = np.random.default_rng(bt)
+    for _ in range(50):
+        lens = rng.integers(0, 400, size=rng.integers(1, 9))
+        offs = np.concatenate([[0], np.cumsum(lens)])
+        idx = bookkeeping.prepare_chunk_indices(offs, bt)
+        co = bookkeeping.prepare_chunk_offsets(offs, bt)
+        # every token position maps to exactly one (sequence, chunk) row, rows are in token order
+        expect = []
+        for n, length in enumerate(lens):
+            seen = sorted({t // bt for t in range(int(length))})
+            expect += [[n, c] for c in seen]
+        assert idx.tolist() == expect
+        assert co[-1] == len(expect) and all(co[n] == sum(1 for r in expect if r[0] < n) for n in range(len(lens)))
+
+
+@pytest.mark.parametrize("T,bt", [(1, 16), (16, 16), (17, 32), (33, 64), (64, 64), (65, 64), (4096, 64)])
+def test_gla_chunk_size_rule(T, bt):
+    assert bookkeeping.gla_chunk_size(T) == bt
+
+
+# ---------------------------------------------------------------- cumsum
+@pytest.mark.parametrize("reverse", [False, True])
+def test_cumsum_bruteforce(reverse):
+    g = _rand(1, 23, 2, 3, seed=1).float()
+    offs = [0, 5, 5, 23]
+    out = cumsum.chunk_local_cumsum(g, 4, reverse=reverse, offsets=offs)
+    for n in range(3):
+        bos, eos = offs[n], offs[n + 1]
+        for t in range(bos, eos):
+            c0 = bos + ((t - bos) // 4) * 4
+            c1 = min(c0 + 4, eos)
+            rows = range(t, c1) if reverse else range(c0, t + 1)
+            acc = torch.zeros(2, 3)
+            for r in rows:
+                acc = acc + g[0, r]
+            torch.testing.assert_close(out[0, t], acc, rtol=1e-6, atol=1e-6)
+
+
+# ---------------------------------------------------------------- GLA recurrence
+def test_gla_scalar_closed_form():
+    T = 9
+    q, k, v, g = (_rand(1, T, 1, 1, seed=s) for s in range(4))
+    g = -g.abs()
+    o, ht = recurrent.naive_recurrent_gla(q, k, v, g, scale=0.7, output_final_state=True, dtype=D)
+    G = [sum(g[0, :t + 1, 0, 0].tolist()) for t in range(T)]
+    for t in range(T):
+        want = 0.7 * q[0, t, 0, 0].item() * sum(
+            k[0, j, 0, 0].item() * v[0, j, 0, 0].item() * math.exp(G[t] - G[j]) for j in range(t + 1))
+        assert abs(o[0, t, 0, 0].item() - want) < 1e-12
+    want_h = sum(k[0, j, 0, 0].item() * v[0, j, 0, 0].item() * math.exp(G[-1] - G[j]) for j in range(T))
+    assert abs(ht[0, 0, 0, 0].item() - want_h) < 1e-12
+
+
+def test_gla_zero_gates_is_causal_linear_attention():
+    B, T, H, K, V = 2, 11, 2, 5, 3
+    q, k, v = _rand(B, T, H, K, seed=1), _rand(B, T, H, K, seed=2), _rand(B, T, H, V, seed=3)
+    o, _ = recurrent.naive_recurrent_gla(q, k, v, torch.zeros_like(k), dtype=D)
+    scores = torch.einsum('bihk,bjhk->bhij', q, k).tril() * K ** -0.5   # default scale K^-0.5 (naive.py:24)
+    want = torch.einsum('bhij,bjhv->bihv', scores, v)
+    torch.testing.assert_close(o, want, rtol=1e-12, atol=1e-12)
+
+
+def test_gla_bruteforce_all_gates_and_reverse():
+    B, T, H, K, V = 1, 6, 2, 3, 2
+    q, k, v = _rand(B, T, H, K, seed=1), _rand(B, T, H, K, seed=2), _rand(B, T, H, V, seed=3)
+    gk, gv, g = -_rand(B, T, H, K, seed=4).abs(), -_rand(B, T, H, V, seed=5).abs(), -_rand(B, T, H, seed=6).abs()
+    h0 = _rand(B, H, K, V, seed=7)
+    for reverse in (False, True):
+        o, ht = recurrent.naive_recurrent_gla(q, k, v, gk, scale=1.3, initial_state=h0, output_final_state=True,
+                                              g=g, gv=gv, reverse=reverse, dtype=D)
+        order = list(range(T))[::-1] if reverse else list(range(T))
+        for h in range(H):
+            for pos, t in enumerate(order):
+                for c in range(V):
+                    want = 0.0
+                    for a in range(K):
+                        # contribution of the initial state and of every earlier (in processing order) token
+                        dec_all = sum(gk[0, m, h, a].item() + gv[0, m, h, c].item() + g[0, m, h].item()
+                                      for m in order[:pos + 1])
+                        tot = h0[0, h, a, c].item() * math.exp(dec_all)
+                        for pj, j in enumerate(order[:pos + 1]):
+                            dec = sum(gk[0, m, h, a].item() + gv[0, m, h, c].item() + g[0, m, h].item()
+                                      for m in order[pj + 1:pos + 1])
+                            tot += k[0, j, h, a].item() * v[0, j, h, c].item() * math.exp(dec)
+                        want += 1.3 * q[0, t, h, a].item() * tot
+                    assert abs(o[0, t, h, c].item() - want) < 1e-10
+
+
+def test_gla_segment_chaining_and_varlen():
+    B, T, H, K, V = 1, 20, 2, 4, 3
+    q, k, v = _rand(B, T, H, K, seed=1), _rand(B, T, H, K, seed=2), _rand(B, T, H, V, seed=3)
+    gk = -_rand(B, T, H, K, seed=4).abs()
+    h0 = _rand(2, H, K, V, seed=5)
+    o, ht = recurrent.naive_recurrent_gla(q, k, v, gk, initial_state=h0[:1], output_final_state=True, dtype=D)
+    o1, h1 = recurrent.naive_recurrent_gla(q[:, :7], k[:, :7], v[:, :7], gk[:, :7], initial_state=h0[:1],
+                                           output_final_state=True, dtype=D)
+    o2, h2 = recurrent.naive_recurrent_gla(q[:, 7:], k[:, 7:], v[:, 7:], gk[:, 7:], initial_state=h1,
+                                           output_final_state=True, dtype=D)
+    torch.testing.assert_close(torch.cat([o1, o2], 1), o, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(h2, ht, rtol=1e-12, atol=1e-12)
+    # packed batch == per-sequence runs
+    ov, hv = recurrent.naive_recurrent_gla(q, k, v, gk, initial_state=h0, output_final_state=True,
+                                           offsets=[0, 7, 20], dtype=D)
+    oa, ha = recurrent.naive_recurrent_gla(q[:, :7], k[:, :7], v[:, :7], gk[:, :7], initial_state=h0[:1],
+                                           output_final_state=True, dtype=D)
+    ob, hb = recurrent.naive_recurrent_gla(q[:, 7:], k[:, 7:], v[:, 7:], gk[:, 7:], initial_state=h0[1:],
+                                           output_final_state=True, dtype=D)
+    torch.testing.assert_close(ov, torch.cat([oa, ob], 1), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(hv, torch.cat([ha, hb], 0), rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------- gated delta rule recurrence
+def test_gdr_beta_zero_is_pure_decay():
+    B, T, H, K, V = 1, 7, 2, 4, 3
+    q, k, v = _rand(B, T, H, K, seed=1), _rand(B, T, H, K, seed=2), _rand(B, T, H, V, seed=3)
+    g = -_rand(B, T, H, seed=4).abs()
+    h0 = _rand(B, H, K, V, seed=5)
+    o, ht = recurrent.naive_recurrent_gated_delta_rule(q, k, v, g, torch.zeros(B, T, H, dtype=D), scale=1.0,
+                                                       initial_state=h0, output_final_state=True, dtype=D)
+    dec = g.cumsum(1).exp()
+    torch.testing.assert_close(ht, h0 * dec[:, -1, :, None, None], rtol=1e-12, atol=1e-12)
+    want = torch.einsum('bthk,bhkv->bthv', q, h0) * dec[..., None]
+    torch.testing.assert_close(o, want, rtol=1e-12, atol=1e-12)
+
+
+def test_gdr_orthonormal_keys_exact_overwrite():
+    H, K, V = 2, 6, 4
+    T = K
+    Q, _ = torch.linalg.qr(_rand(H, K, K, seed=1))          # orthonormal rows per head
+    k = Q.permute(1, 0, 2)[None]                            # [1,T,H,K], k_t orthonormal across t
+    v, q = _rand(1, T, H, V, seed=2), _rand(1, T, H, K, seed=3)
+    h0 = _rand(1, H, K, V, seed=4)
+    _, S = recurrent.naive_recurrent_gated_delta_rule(q, k, v, torch.zeros(1, T, H, dtype=D),
+                                                      torch.ones(1, T, H, dtype=D), initial_state=h0,
+                                                      output_final_state=True, dtype=D)
+    read = torch.einsum('thk,hkv->thv', k[0], S[0])         # S^T k_i must return v_i for every i
+    torch.testing.assert_close(read, v[0], rtol=1e-10, atol=1e-10)
+
+
+def test_gdr_single_step_closed_form():
+    H, K, V = 3, 5, 4
+    q, k, v = _rand(1, 1, H, K, seed=1), _rand(1, 1, H, K, seed=2), _rand(1, 1, H, V, seed=3)
+    beta, g = torch.rand(1, 1, H, dtype=D), -torch.rand(1, 1, H, dtype=D)
+    o, _ = recurrent.naive_recurrent_gated_delta_rule(q, k, v, g, beta, scale=0.3, dtype=D)
+    want = 0.3 * (q * k).sum(-1, keepdim=True) * beta[..., None] * v
+    torch.testing.assert_close(o, want, rtol=1e-12, atol=1e-12)
+
+
+def test_gdr_dense_transition_matrices():
+    """S_t = (I - beta k k^T) e^{g} S_{t-1} + beta k v^T with every transition materialised."""
+    B, T, H, K, V = 1, 8, 2, 4, 3
+    q, k, v = _rand(B, T, H, K, seed=1), F.normalize(_rand(B, T, H, K, seed=2), dim=-1), _rand(B, T, H, V, seed=3)
+    g, beta = -_rand(B, T, H, seed=4).abs(), torch.rand(B, T, H, dtype=D)
+    bv = torch.rand(B, T, H, V, dtype=D)
+    h0 = _rand(B, H, K, V, seed=5)
+    for b_in in (beta, bv):
+        o, ht = recurrent.naive_recurrent_gated_delta_rule(q, k, v, g, b_in, scale=0.5, initial_state=h0,
+                                                           output_final_state=True, dtype=D)
+        for h in range(H):
+            S = h0[0, h].numpy().copy()
+            for t in range(T):
+                kk = k[0, t, h].numpy()
+                bcol = np.broadcast_to(b_in[0, t, h].numpy(), (V,))
+                Sd = math.exp(g[0, t, h].item()) * S
+                # per-value beta: column c uses its own beta
+                S = Sd - np.outer(kk, (kk @ Sd) * bcol) + np.outer(kk, v[0, t, h].numpy() * bcol)
+                np.testing.assert_allclose(o[0, t, h].numpy(), 0.5 * q[0, t, h].numpy() @ S, rtol=1e-10, atol=1e-12)
+            np.testing.assert_allclose(ht[0, h].numpy(), S, rtol=1e-10, atol=1e-12)
+
+
+# ---------------------------------------------------------------- chunked forms
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_chunked_gla_equals_recurrence(offsets):
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q, k, v = _rand(B, T, H, K, seed=1), _rand(B, T, H, K, seed=2), _rand(B, T, H, V, seed=3)
+    gk = F.logsigmoid(_rand(B, T, H, K, seed=4))
+    h0 = _rand(N, H, K, V, seed=5)
+    o, ht = recurrent.naive_recurrent_gla(q, k, v, gk, initial_state=h0, output_final_state=True, offsets=offsets,
+                                          dtype=D)
+    r = chunked.chunked_gla(q, k, v, gk, initial_state=h0, offsets=offsets, dtype=D)
+    torch.testing.assert_close(r['o'], o, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(r['ht'], ht, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(r['g_cumsum'].float(), cumsum.chunk_local_cumsum(gk, 64, offsets=offsets),
+                               rtol=1e-5, atol=1e-5)
+    # per-chunk state h[c] equals the recurrence's state after c*64 tokens of that sequence
+    if offsets is None:
+        _, h64 = recurrent.naive_recurrent_gla(q[:, :64], k[:, :64], v[:, :64], gk[:, :64], initial_state=h0,
+                                               output_final_state=True, dtype=D)
+        torch.testing.assert_close(r['h'][:, 1], h64, rtol=1e-10, atol=1e-10)
+        torch.testing.assert_close(r['h'][:, 0], h0, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_chunked_gdr_equals_recurrence(offsets):
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q, k, v = _rand(B, T, H, K, seed=1), F.normalize(_rand(B, T, H, K, seed=2), dim=-1), _rand(B, T, H, V, seed=3)
+    g, beta = F.logsigmoid(_rand(B, T, H, seed=4)), torch.rand(B, T, H, dtype=D)
+    h0 = _rand(N, H, K, V, seed=5)
+    o, ht = recurrent.naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                                       offsets=offsets, dtype=D)
+    r = chunked.chunked_gated_delta_rule(q, k, v, g, beta, initial_state=h0, offsets=offsets, dtype=D)
+    torch.testing.assert_close(r['o'], o, rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(r['ht'], ht, rtol=1e-9, atol=1e-9)
+
+
+def test_wy_inverse_identities():
+    """Aw (I + M) = I, and Au = Aw * Gamma elementwise (so one inverse suffices)."""
+    B, T, H, K, V = 1, 64, 2, 16, 8
+    q, k, v = _rand(B, T, H, K, seed=1), F.normalize(_rand(B, T, H, K, seed=2), dim=-1), _rand(B, T, H, V, seed=3)
+    g, beta = F.logsigmoid(_rand(B, T, H, seed=4)), torch.rand(B, T, H, dtype=D)
+    r = chunked.chunked_gated_delta_rule(q, k, v, g, beta, dtype=D)
+    gam = g[0].cumsum(0)
+    for h in range(H):
+        kb = k[0, :, h] * beta[0, :, h, None]
+        M = (kb @ k[0, :, h].T).tril(-1)
+        Aw, Au = r['Aw'][0, :, h], r['Au'][0, :, h]
+        torch.testing.assert_close(Aw @ (torch.eye(64, dtype=D) + M), torch.eye(64, dtype=D), rtol=1e-9, atol=1e-9)
+        Gam = (gam[:, h, None] - gam[None, :, h]).exp().tril()
+        torch.testing.assert_close(Au, Aw * Gam, rtol=1e-9, atol=1e-9)
+        torch.testing.assert_close(r['w'][0, :, h], Aw @ kb, rtol=1e-9, atol=1e-9)
+
+
+# ---------------------------------------------------------------- gradients of the oracle (autograd)
+def test_oracle_gradcheck():
+    B, T, H, K, V = 1, 5, 1, 3, 2
+    q, k, v = (_rand(B, T, H, n, seed=s).requires_grad_() for s, n in ((1, K), (2, K), (3, V)))
+    gk = (-_rand(B, T, H, K, seed=4).abs()).requires_grad_()
+    h0 = _rand(B, H, K, V, seed=5).requires_grad_()
+    f = lambda q, k, v, gk, h0: recurrent.naive_recurrent_gla(q, k, v, gk, initial_state=h0,
+                                                              output_final_state=True, dtype=D)
+    assert torch.autograd.gradcheck(f, (q, k, v, gk, h0), atol=1e-6)
+    g = (-_rand(B, T, H, seed=6).abs()).requires_grad_()
+    beta = torch.rand(B, T, H, dtype=D).requires_grad_()
+    f2 = lambda q, k, v, g, beta, h0: recurrent.naive_recurrent_gated_delta_rule(
+        q, k, v, g, beta, initial_state=h0, output_final_state=True, dtype=D)
+    assert torch.autograd.gradcheck(f2, (q, k, v, g, beta, h0), atol=1e-6)
