@@ -1,0 +1,799 @@
+// Chunked gated delta rule forward for gfx950 (chunk size 64, 16-bit q/k/v,
+// fp32 state).  gamma below is the chunk-local prefix sum of the scalar
+// per-head log-gate g (fp32, produced by fla_chunk_local_cumsum).
+//
+//   gdr_fwd_wy_kernel   one workgroup per (chunk, head):
+//                         M  = strict_lower(diag(beta) K K^T)            (MFMA)
+//                         Aw = (I + M)^-1                                (fp32, blocked)
+//                         Au = Aw * Gamma,  Gamma_ij = e^{gamma_i - gamma_j}
+//                         w  = Aw (beta K),  u = Au (beta V)             (MFMA)
+//                       The reference inverts I + M and I + M*Gamma separately
+//                       (fla/ops/gated_delta_rule/wy_fast.py:150-208); since
+//                       M*Gamma = D M D^-1 with D = diag(e^gamma), the second
+//                       inverse is D Aw D^-1 = Aw * Gamma elementwise, so one
+//                       inversion serves both.
+//   gdr_fwd_h_kernel    serial scan per (sequence, head, 32 value columns):
+//                         store h_c;  v_new = u - (w e^gamma) h_c;
+//                         h <- e^{gamma_last} h_c + (k e^{gamma_last-gamma})^T v_new
+//                       (fla/ops/common/chunk_delta_h.py:71-119).
+//   chunk_fwd_o_kernel  one workgroup per (chunk, head):
+//                         o = s (e^gamma * (q h_c) + tril(q k^T * Gamma) v_new)
+//                       (fla/ops/common/chunk_o.py:68-101).  The scalar gate is
+//                       applied to the fp32 scores / accumulators, so every
+//                       exponent is <= 0 whatever the gate magnitude.
+#include "fla_common.h"
+#include "mfma_tiles.h"
+
+namespace {
+
+constexpr int BT = 64;
+constexpr int LDT = BT + 8;  // pitch of time-contiguous 16-bit tiles
+constexpr int LDM = BT + 4;  // pitch of fp32 64x64 tiles
+
+FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
+  if (total % 8 != 0) return id;
+  return (id % 8) * (total / 8) + id / 8;
+}
+
+struct ChunkLoc {
+  int64_t row0;   // first token row of the chunk in the flattened [B*T] space
+  int L;          // valid rows
+  int64_t cglob;  // global chunk index (addresses per-chunk states)
+};
+
+FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix) {
+  ChunkLoc c;
+  int64_t bos, len, ic;
+  if (offsets) {
+    int64_t n = indices[2 * (int64_t)blockIdx.x];
+    ic = indices[2 * (int64_t)blockIdx.x + 1];
+    bos = offsets[n];
+    len = offsets[n + 1] - bos;
+  } else {
+    bos = (blockIdx.x / ntfix) * T;
+    ic = blockIdx.x % ntfix;
+    len = T;
+  }
+  c.row0 = bos + ic * BT;
+  int64_t rem = len - ic * BT;
+  c.L = (int)(rem < BT ? rem : BT);
+  c.cglob = blockIdx.x;
+  return c;
+}
+
+// C[n x n] (+)= sign * A[n x n] B[n x n], fp32 in LDS, spread over `nthr` threads.
+template <int N>
+FLA_DEVICE void lds_mm(const float* A, int lda, const float* B, int ldb, float* C, int ldc, float sign, int t,
+                       int nthr) {
+  for (int e = t; e < N * N; e += nthr) {
+    int i = e / N, j = e % N;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < N; ++k) acc += A[i * lda + k] * B[k * ldb + j];
+    C[i * ldc + j] = sign * acc;
+  }
+}
+
+struct WyParams {
+  const void* k;
+  const void* v;
+  const float* beta;
+  const float* gam;
+  void* w;
+  void* u;
+  void* Aw;
+  void* Au;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+};
+
+template <typename T, int K, int V>
+__global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int SA_ELEMS = (BT * LDK > 2 * BT * LDT) ? BT * LDK : 2 * BT * LDT;
+  constexpr int R1_BYTES = (2 * BT * LDM * 4 > V * LDT * 2) ? 2 * BT * LDM * 4 : V * LDT * 2;
+  __shared__ __attribute__((aligned(16))) T sA[SA_ELEMS];          // k row-major, later Aw | Au
+  __shared__ __attribute__((aligned(16))) T sKbT[K * LDT];         // (beta k)^T  [k][t]
+  __shared__ __attribute__((aligned(16))) char sR1[R1_BYTES];      // M, X fp32; later (beta v)^T
+  __shared__ __attribute__((aligned(16))) float sT[32 * 36];
+  __shared__ float sBeta[BT], sGam[BT];
+  T* sK = sA;
+  T* sAw = sA;
+  T* sAu = sA + BT * LDT;
+  float* sM = (float*)sR1;
+  float* sX = sM + BT * LDM;
+  T* sVbT = (T*)sR1;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, hh = blockIdx.y;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+
+  // ---- loads
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  v4 kreg[RPT];
+  float brow[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    if (row < L) {
+      kreg[i] = *(const v4*)((const T*)p.k + ((row0 + row) * H + hh) * (int64_t)K + c4);
+      brow[i] = p.beta[(row0 + row) * H + hh];
+    } else {
+      kreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      brow[i] = 0.f;
+    }
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+  v4 vreg[RPTV];
+  float bvrow[RPTV];
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) {
+    int row = rgv * RPTV + i;
+    if (row < L) {
+      vreg[i] = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + cv4);
+      bvrow[i] = p.beta[(row0 + row) * H + hh];
+    } else {
+      vreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      bvrow[i] = 0.f;
+    }
+  }
+  if (tid < BT) {
+    bool ok = tid < L;
+    sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
+    sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
+  }
+  // ---- k row-major and (beta k)^T to LDS
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) *(v4*)&sK[(rg * RPT + i) * LDK + c4] = kreg[i];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T* dst = &sKbT[(c4 + j) * LDT + rg * RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) dst[i] = (T)((float)kreg[i][j] * brow[i]);
+  }
+  __syncthreads();
+
+  // ---- S = k k^T on the lower-triangular 32x32 quadrants; M = beta_i S_ij (j < i)
+  {
+    const int qi = wave >> 1, qj = wave & 1;
+    f32x16 s = zero16();
+    if (qj <= qi) {
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 16)
+        s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
+    }
+    const int j = qj * 32 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = qi * 32 + c32_row(r, lane);
+      sM[i * LDM + j] = (j < i) ? sBeta[i] * s[r] : 0.f;
+    }
+    for (int e = tid; e < BT * LDM; e += 256) sX[e] = 0.f;
+  }
+  __syncthreads();
+
+  // ---- (I + M)^-1: 16x16 diagonal blocks by forward substitution (one lane per column)
+  if (tid < 64) {
+    const int b = tid >> 4, col = tid & 15;
+    const float* Mb = sM + (16 * b) * LDM + 16 * b;
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float s = (i == col) ? 1.f : 0.f;
+#pragma unroll
+      for (int j = 0; j < i; ++j) s -= Mb[i * LDM + j] * x[j];
+      x[i] = s;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sX[(16 * b + i) * LDM + 16 * b + col] = x[i];
+  }
+  __syncthreads();
+  // ---- 32x32 diagonal blocks: X_lo = -X_bb M_lo X_aa for the block pairs (1,0) and (3,2)
+  {
+    const int pr = tid >> 7, t = tid & 127;
+    const int a0 = 32 * pr, b0 = 32 * pr + 16;
+    lds_mm<16>(sM + b0 * LDM + a0, LDM, sX + a0 * LDM + a0, LDM, sT + pr * 256, 16, 1.f, t, 128);
+    __syncthreads();
+    lds_mm<16>(sX + b0 * LDM + b0, LDM, sT + pr * 256, 16, sX + b0 * LDM + a0, LDM, -1.f, t, 128);
+  }
+  __syncthreads();
+  // ---- 64x64: X_BA = -X_BB M_BA X_AA
+  lds_mm<32>(sM + 32 * LDM, LDM, sX, LDM, sT, 36, 1.f, tid, 256);
+  __syncthreads();
+  lds_mm<32>(sX + 32 * LDM + 32, LDM, sT, 36, sX + 32 * LDM, LDM, -1.f, tid, 256);
+  __syncthreads();
+
+  // ---- Aw, Au in 16-bit (LDS for the products, optionally global for the backward pass)
+  {
+    const int i = tid >> 2, j0 = (tid & 3) * 16;
+    const float gi = sGam[i];
+    v8 aw[2], au[2];
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj) {
+      int j = j0 + jj;
+      float x = sX[i * LDM + j];
+      float gamma = (j <= i) ? __expf(gi - sGam[j]) : 0.f;
+      aw[jj >> 3][jj & 7] = (T)x;
+      au[jj >> 3][jj & 7] = (T)(x * gamma);
+    }
+    *(v8*)&sAw[i * LDT + j0] = aw[0];
+    *(v8*)&sAw[i * LDT + j0 + 8] = aw[1];
+    *(v8*)&sAu[i * LDT + j0] = au[0];
+    *(v8*)&sAu[i * LDT + j0 + 8] = au[1];
+    if (i < L) {
+      int64_t off = ((row0 + i) * H + hh) * (int64_t)BT + j0;
+      if (p.Aw) {
+        *(v8*)((T*)p.Aw + off) = aw[0];
+        *(v8*)((T*)p.Aw + off + 8) = aw[1];
+      }
+      if (p.Au) {
+        *(v8*)((T*)p.Au + off) = au[0];
+        *(v8*)((T*)p.Au + off + 8) = au[1];
+      }
+    }
+  }
+  __syncthreads();  // X fully consumed: its storage becomes (beta v)^T
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T* dst = &sVbT[(cv4 + j) * LDT + rgv * RPTV];
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) dst[i] = (T)((float)vreg[i][j] * bvrow[i]);
+  }
+  // ---- w = Aw (beta k)
+  const int rw = wave >> 1, cw = wave & 1;
+  const int jsteps = (rw + 1) * 2;  // Aw, Au are lower triangular
+  {
+    constexpr int TK = K / 64;
+    f32x16 acc[TK];
+#pragma unroll
+    for (int t = 0; t < TK; ++t) acc[t] = zero16();
+    for (int js = 0; js < jsteps; ++js) {
+      v8 a = lds_frag32<T>(sAw, LDT, rw * 32, js * 16, lane);
+#pragma unroll
+      for (int t = 0; t < TK; ++t)
+        acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(sKbT, LDT, (cw * TK + t) * 32, js * 16, lane), acc[t]);
+    }
+    T* wp = (T*)p.w + (row0 * H + hh) * (int64_t)K;
+#pragma unroll
+    for (int t = 0; t < TK; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int i = rw * 32 + c32_row(r, lane);
+        if (i < L) wp[(int64_t)i * H * K + (cw * TK + t) * 32 + (lane & 31)] = (T)acc[t][r];
+      }
+  }
+  __syncthreads();  // (beta v)^T complete
+  {
+    constexpr int TV = V / 64;
+    f32x16 acc[TV];
+#pragma unroll
+    for (int t = 0; t < TV; ++t) acc[t] = zero16();
+    for (int js = 0; js < jsteps; ++js) {
+      v8 a = lds_frag32<T>(sAu, LDT, rw * 32, js * 16, lane);
+#pragma unroll
+      for (int t = 0; t < TV; ++t)
+        acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(sVbT, LDT, (cw * TV + t) * 32, js * 16, lane), acc[t]);
+    }
+    T* up = (T*)p.u + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+    for (int t = 0; t < TV; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int i = rw * 32 + c32_row(r, lane);
+        if (i < L) up[(int64_t)i * H * V + (cw * TV + t) * 32 + (lane & 31)] = (T)acc[t][r];
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct DHParams {
+  const void* k;
+  const void* w;
+  const void* u;
+  const float* gam;
+  const float* h0;
+  void* h;
+  void* v_new;
+  float* ht;
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int H, V, N;
+};
+
+// One workgroup: all K rows x 32 value columns of one (sequence, head) state.
+// Wave w keeps the 32x32 state tiles kt = w, w+4, ... in MFMA accumulators.
+// HL: 0 row-major [K,V] in T, 1 fragment order in T, 2 row-major fp32.
+template <typename T, int K, int HL>
+__global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  constexpr int BV = 32;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int KT32 = K / 32;
+  constexpr int NKT = (KT32 + 3) / 4;  // state tiles per wave
+  __shared__ __attribute__((aligned(16))) T sW[BT * LDK];    // w e^gamma, row-major
+  __shared__ __attribute__((aligned(16))) T sKt[K * LDT];    // (k e^{gamma_last-gamma})^T
+  __shared__ __attribute__((aligned(16))) T sUt[BV * LDT];   // u^T
+  __shared__ __attribute__((aligned(16))) T sHt[BV * LDK];   // h^T in 16-bit
+  __shared__ __attribute__((aligned(16))) T sVnT[BV * LDT];  // v_new^T
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, V = p.V;
+  const int nvt = V / BV;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vt = (int)(id % nvt);
+  const int nh = (int)(id / nvt);
+  const int n = nh / H, hh = nh % H;
+  const int vbase = vt * BV;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+
+  f32x16 acc[NKT];
+#pragma unroll
+  for (int a = 0; a < NKT; ++a) {
+    acc[a] = zero16();
+    int kt = wave + 4 * a;
+    if (p.h0 && kt < KT32) {
+      const float* h0p = p.h0 + (int64_t)nh * K * V;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
+    }
+  }
+
+  // prefetch registers: w, k as (RPT rows x 4 cols), u as (4 rows x 2 cols), gamma per row
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  const int urg = tid >> 4, uc2 = (tid & 15) * 2;
+  struct Regs {
+    v4 w[RPT];
+    v4 k[RPT];
+    float gam[RPT];
+    t2 u[4];
+    float glast;
+  };
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+  auto load_chunk = [&](int64_t c, Regs& R) {
+    int L = chunk_len(c);
+    bool live = c < nchunks;
+    int64_t rbase = sp.bos + c * BT;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      if (live && row < L) {
+        R.w[i] = *(const v4*)((const T*)p.w + ((rbase + row) * H + hh) * (int64_t)K + c4);
+        R.k[i] = *(const v4*)((const T*)p.k + ((rbase + row) * H + hh) * (int64_t)K + c4);
+        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
+      } else {
+        R.w[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.gam[i] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int row = urg * 4 + i;
+      if (live && row < L) R.u[i] = *(const t2*)((const T*)p.u + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
+      else R.u[i] = t2{(T)0.f, (T)0.f};
+    }
+    R.glast = (live && p.gam) ? p.gam[(rbase + L - 1) * H + hh] : 0.f;
+  };
+  // state-independent operand tiles of one chunk
+  auto stage_wu = [&](const Regs& R) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      float eg = __expf(R.gam[i]);
+      v4 wv;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = (T)((float)R.w[i][j] * eg);
+      *(v4*)&sW[row * LDK + c4] = wv;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      v4 uv = v4{R.u[0][j], R.u[1][j], R.u[2][j], R.u[3][j]};
+      *(v4*)&sUt[(uc2 + j) * LDT + urg * 4] = uv;
+    }
+  };
+  auto stage_k = [&](const Regs& R, int L) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      T* dst = &sKt[(c4 + j) * LDT + rg * RPT];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        bool valid = (rg * RPT + i) < L;
+        dst[i] = (T)(valid ? (float)R.k[i][j] * __expf(R.glast - R.gam[i]) : 0.f);
+      }
+    }
+  };
+  // state entering chunk c: 16-bit transpose in LDS for the MFMA, global copy for the output kernel
+  auto publish_h = [&](int64_t c) {
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+        v8 lo, hi;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          lo[r] = (T)acc[a][r];
+          hi[r] = (T)acc[a][r + 8];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4 x;
+#pragma unroll
+          for (int b = 0; b < 4; ++b) x[b] = (q < 2) ? lo[4 * q + b] : hi[4 * (q - 2) + b];
+          *(v4*)&sHt[(lane & 31) * LDK + kt * 32 + 8 * q + 4 * (lane >> 5)] = x;
+        }
+        if (p.h) {
+          int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
+          if (HL == 1) {
+            T* hp = (T*)p.h + blk + (((int64_t)kt * (V / 32) + vt) * 64 + lane) * 16;
+            *(v8*)hp = lo;
+            *(v8*)(hp + 8) = hi;
+          } else if (HL == 0) {
+            T* hp = (T*)p.h + blk;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              hp[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = (T)acc[a][r];
+          } else {
+            float* hp = (float*)p.h + blk;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              hp[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[a][r];
+          }
+        }
+      }
+    }
+  };
+
+  // Two barriers per chunk and single-buffered tiles:
+  //   phase A (after barrier 1): v_new from sW, sUt, sHt;  stage sKt of the same chunk
+  //   phase B (after barrier 2): state update from sKt, sVnT;  stage sW, sUt, sHt of the next chunk
+  // Rc holds the chunk whose tiles are staged next, Rn the one after; loads run a full
+  // iteration ahead of their use.
+  Regs Rc, Rn;
+  load_chunk(0, Rc);
+  load_chunk(1, Rn);
+  if (nchunks > 0) {
+    stage_wu(Rc);
+    publish_h(0);
+  }
+  for (int64_t c = 0; c < nchunks; ++c) {
+    const int L = chunk_len(c);
+    const int64_t rbase = sp.bos + c * BT;
+    __syncthreads();  // (1)
+    // ---- v_new = u - (w e^gamma) h : wave w owns rows 16w..16w+15, two 16-column tiles
+    {
+      f32x4 d[2] = {zero4(), zero4()};
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 32) {
+        v8 a = lds_frag16<T>(sW, LDK, wave * 16, ks, lane);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, lds_frag16<T>(sHt, LDK, j * 16, ks, lane), d[j]);
+      }
+      const int tr = wave * 16 + 4 * (lane >> 4);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        int vc = j * 16 + (lane & 15);
+        v4 uu = *(const v4*)&sUt[vc * LDT + tr];
+        v4 vn;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) vn[r] = (T)((float)uu[r] - d[j][r]);
+        *(v4*)&sVnT[vc * LDT + tr] = vn;
+        if (p.v_new) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (tr + r < L) ((T*)p.v_new)[((rbase + tr + r) * H + hh) * (int64_t)V + vbase + vc] = vn[r];
+        }
+      }
+    }
+    stage_k(Rc, L);
+    const float dec = __expf(Rc.glast);
+    Rc = Rn;
+    load_chunk(c + 2, Rn);
+    __syncthreads();  // (2)
+    // ---- h <- e^{gamma_last} h + (k e^{gamma_last-gamma})^T v_new
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][r] *= dec;
+#pragma unroll
+        for (int s = 0; s < BT; s += 16)
+          acc[a] = Elem<T>::mfma32(lds_frag32<T>(sKt, LDT, kt * 32, s, lane), lds_frag32<T>(sVnT, LDT, 0, s, lane),
+                                   acc[a]);
+      }
+    }
+    if (c + 1 < nchunks) {
+      stage_wu(Rc);
+      publish_h(c + 1);
+    }
+  }
+  if (p.ht) {
+    float* htp = p.ht + (int64_t)nh * K * V;
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) htp[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[a][r];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct DOParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const float* gam;
+  const void* h;
+  void* o;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+template <typename T, int K, int V>
+__global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int C8 = K / 8;                 // 16-byte pieces per row
+  constexpr int NP = BT * C8 / 256;          // pieces per thread
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int KT32 = K / 32, TV = V / 64;
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];  // later P
+  __shared__ __attribute__((aligned(16))) T sVt[V * LDT];
+  __shared__ float sGam[BT];
+  T* sP = sK;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, hh = blockIdx.y;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+
+  v8 qreg[NP], kreg[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c8;
+      qreg[i] = *(const v8*)((const T*)p.q + off);
+      kreg[i] = *(const v8*)((const T*)p.k + off);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qreg[i][j] = kreg[i][j] = (T)0.f;
+    }
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+  v4 vreg[RPTV];
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) {
+    int row = rgv * RPTV + i;
+    if (row < L) vreg[i] = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + cv4);
+    else vreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  }
+  if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
+  const int rw = wave >> 1, cw = wave & 1;
+  v8 hf[KT32][TV][2];
+  {
+    const T* hp = (const T*)p.h + (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) {
+        const T* f = hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16;
+        hf[kt][tv][0] = *(const v8*)f;
+        hf[kt][tv][1] = *(const v8*)(f + 8);
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sQ[row * LDK + c8] = qreg[i];
+    *(v8*)&sK[row * LDK + c8] = kreg[i];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T* dst = &sVt[(cv4 + j) * LDT + rgv * RPTV];
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) dst[i] = vreg[i][j];
+  }
+  __syncthreads();
+
+  const int qi = wave >> 1, qj = wave & 1;
+  f32x16 s = zero16();
+  if (qj <= qi) {
+#pragma unroll
+    for (int ks = 0; ks < K; ks += 16)
+      s = Elem<T>::mfma32(lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
+  }
+  __syncthreads();  // all reads of sK done before P overwrites it
+  {
+    const int j = qj * 32 + (lane & 31);
+    const float gj = sGam[j];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = qi * 32 + c32_row(r, lane);
+      float val = (j <= i) ? s[r] * p.scale * __expf(sGam[i] - gj) : 0.f;
+      sP[i * LDT + j] = (T)val;
+    }
+  }
+  __syncthreads();
+
+  f32x16 acc[TV];
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+#pragma unroll
+  for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v8 a = lds_frag32_perm<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(a, hf[kt][tv][half], acc[tv]);
+    }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float rs = p.scale * __expf(sGam[rw * 32 + c32_row(r, lane)]);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv) acc[tv][r] *= rs;
+  }
+  const int jend = (rw + 1) * 32;
+  for (int js = 0; js < jend; js += 16) {
+    v8 a = lds_frag32<T>(sP, LDT, rw * 32, js, lane);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
+  }
+  T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = rw * 32 + c32_row(r, lane);
+      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    }
+}
+
+template <typename T>
+int launch_wy(const WyParams& p, int K, int V, dim3 grid, hipStream_t st) {
+#define FLA_CASE(KK, VV)                                                                \
+  if (K == KK && V == VV) {                                                             \
+    hipLaunchKernelGGL((gdr_fwd_wy_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);      \
+    FLA_CHECK_LAUNCH();                                                                 \
+    return FLA_OK;                                                                      \
+  }
+  FLA_CASE(64, 64)
+  FLA_CASE(128, 128)
+  FLA_CASE(64, 128)
+  FLA_CASE(128, 64)
+#undef FLA_CASE
+  return FLA_E_UNSUPPORTED;
+}
+
+template <typename T>
+int launch_dh(const DHParams& p, int K, int h_dtype, int h_layout, hipStream_t st) {
+  int64_t total = (int64_t)(p.V / 32) * p.N * p.H;
+  if (total == 0) return FLA_OK;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  dim3 grid((unsigned)total), block(256);
+  int hl = (h_layout == FLA_H_FRAGMENT) ? 1 : (h_dtype == FLA_F32 ? 2 : 0);
+#define FLA_CASE(KK, HL)                                                           \
+  if (K == KK && hl == HL) {                                                       \
+    hipLaunchKernelGGL((gdr_fwd_h_kernel<T, KK, HL>), grid, block, 0, st, p);      \
+    FLA_CHECK_LAUNCH();                                                            \
+    return FLA_OK;                                                                 \
+  }
+  FLA_CASE(64, 0) FLA_CASE(64, 1) FLA_CASE(64, 2)
+  FLA_CASE(128, 0) FLA_CASE(128, 1) FLA_CASE(128, 2)
+#undef FLA_CASE
+  return FLA_E_UNSUPPORTED;
+}
+
+template <typename T>
+int launch_do(const DOParams& p, int K, int V, dim3 grid, hipStream_t st) {
+#define FLA_CASE(KK, VV)                                                                \
+  if (K == KK && V == VV) {                                                             \
+    hipLaunchKernelGGL((chunk_fwd_o_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);     \
+    FLA_CHECK_LAUNCH();                                                                 \
+    return FLA_OK;                                                                      \
+  }
+  FLA_CASE(64, 64)
+  FLA_CASE(128, 128)
+  FLA_CASE(64, 128)
+  FLA_CASE(128, 64)
+#undef FLA_CASE
+  return FLA_E_UNSUPPORTED;
+}
+
+int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B, int64_t T, int64_t H, int64_t NT,
+               dim3* grid, int* ntfix) {
+  if (offsets) FLA_REQUIRE(indices != nullptr && B == 1, FLA_E_INVALID);
+  int64_t nf = (T + BT - 1) / BT;
+  int64_t nblk = offsets ? NT : B * nf;
+  FLA_REQUIRE(nblk <= 0x7fffffffLL && H <= 65535, FLA_E_UNSUPPORTED);
+  *grid = dim3((unsigned)nblk, (unsigned)H);
+  *ntfix = (int)nf;
+  return FLA_OK;
+}
+
+}  // namespace
+
+extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum, void* w, void* u,
+                              void* Aw, void* Au, const int64_t* offsets, const int64_t* indices, int64_t NT,
+                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                              fla_stream_t stream) {
+  FLA_REQUIRE(k && v && beta && w && u, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, offsets, indices, T, (int)H, ntfix};
+  if (qkv_dtype == FLA_BF16) return launch_wy<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_wy<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, const void* u, const float* g_cumsum,
+                                                const float* h0, void* h, void* v_new, float* ht,
+                                                const int64_t* offsets, const int64_t* chunk_offsets, int qkv_dtype,
+                                                int h_dtype, int h_layout, int64_t B, int64_t T, int64_t H, int64_t K,
+                                                int64_t V, int64_t N, fla_stream_t stream) {
+  FLA_REQUIRE(k && w && u, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(V % 32 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(chunk_offsets != nullptr && B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT, FLA_E_INVALID);
+  if (h_layout == FLA_H_FRAGMENT) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
+  else FLA_REQUIRE(h_dtype == qkv_dtype || h_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)h | (uintptr_t)v_new) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  DHParams p{k, w, u, g_cumsum, h0, h, v_new, ht, offsets, chunk_offsets, T, (int)H, (int)V, (int)N};
+  if (qkv_dtype == FLA_BF16) return launch_dh<bf16>(p, (int)K, h_dtype, h_layout, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_dh<f16>(p, (int)K, h_dtype, h_layout, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_cumsum, const void* h,
+                               void* o, const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                               int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale,
+                               fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && h && o, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)h | (uintptr_t)o) % 16 == 0, FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  DOParams p{q, k, v, g_cumsum, h, o, offsets, indices, T, (int)H, ntfix, scale};
+  if (qkv_dtype == FLA_BF16) return launch_do<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_do<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}

@@ -1,5 +1,6 @@
-from .gated_delta_rule import fused_recurrent_gated_delta_rule
+from .gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
 from .gla import chunk_gla, fused_recurrent_gla
 from .utils import chunk_local_cumsum
 
-__all__ = ['chunk_gla', 'fused_recurrent_gla', 'fused_recurrent_gated_delta_rule', 'chunk_local_cumsum']
+__all__ = ['chunk_gla', 'fused_recurrent_gla', 'chunk_gated_delta_rule', 'fused_recurrent_gated_delta_rule',
+           'chunk_local_cumsum']

@@ -1,0 +1,61 @@
+"""``chunk_gated_delta_rule_fwd_h`` (``fla/ops/common/chunk_delta_h.py:248-320``),
+served by ``fla_chunk_gated_delta_rule_fwd_h``."""
+from typing import Optional, Tuple
+
+import torch
+
+from ... import _backend as be
+from ...utils import prepare_chunk_offsets
+
+BT = 64
+
+
+def chunk_gated_delta_rule_fwd_h(
+    k: torch.Tensor,
+    w: torch.Tensor,
+    u: torch.Tensor,
+    g: Optional[torch.Tensor],
+    initial_state: Optional[torch.Tensor],
+    output_final_state: bool,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+    chunk_size: int = 64,
+    *,
+    states_in_fp32: bool = False,
+    fragment_layout: bool = False,
+    chunk_offsets: Optional[torch.Tensor] = None,
+    store_v_new: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Returns ``(h, v_new, final_state)``; ``g`` is the fp32 chunk-local cumsum of
+    the log-gate ``[B,T,H]`` (or ``None``).  ``h`` is ``[B,NT,H,K,V]`` holding the
+    state entering each chunk (row-major, or MFMA-fragment order for
+    ``fla_chunk_fwd_o`` when ``fragment_layout``)."""
+    if head_first or chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd_h: seq-first, chunk size 64 only")
+    be.require_gpu(k, w, u)
+    B, T, H, K = k.shape
+    V = u.shape[-1]
+    if offsets is None:
+        N, NT = B, -(-T // BT)
+    else:
+        if chunk_offsets is None:
+            chunk_offsets = prepare_chunk_offsets(offsets, BT, device=k.device)
+        N = len(offsets) - 1
+        NT = int(indices.shape[0]) if indices is not None else int(prepare_chunk_offsets(offsets, BT)[-1])
+        offsets = offsets.to(torch.int64).contiguous()
+    h_dtype = torch.float32 if states_in_fp32 else k.dtype
+    h = k.new_empty(B, NT, H, K, V, dtype=h_dtype)
+    v_new = torch.empty_like(u) if store_v_new else None
+    ht = k.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
+    h0 = None
+    if initial_state is not None:
+        h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
+    if g is not None and g.dtype != torch.float32:
+        g = g.float()
+    be.check(be.lib().fla_chunk_gated_delta_rule_fwd_h(
+        be.ptr(k), be.ptr(w), be.ptr(u), be.ptr(g), be.ptr(h0), be.ptr(h), be.ptr(v_new), be.ptr(ht),
+        be.ptr(offsets), be.ptr(chunk_offsets), be.dt(k), be._DTYPES[h_dtype],
+        be.FLA_H_FRAGMENT if fragment_layout else be.FLA_H_ROW_MAJOR,
+        B, T, H, K, V, N, be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_h")
+    return h, v_new, ht

@@ -1,0 +1,126 @@
+"""``chunk_gated_delta_rule`` with the reference's signature
+(``fla/ops/gated_delta_rule/chunk.py:258-363``).
+
+Forward pipeline on the device (chunk size 64): ``fla_chunk_local_cumsum`` (gate)
+-> ``fla_gdr_fwd_wy`` (KK^T, block inverse, w/u) -> ``fla_chunk_gated_delta_rule_fwd_h``
+(state scan, v_new) -> ``fla_chunk_fwd_o``.
+"""
+from typing import Optional, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from ... import _backend as be
+from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
+                      resolve_offsets)
+from ..common.chunk_delta_h import chunk_gated_delta_rule_fwd_h
+from ..common.chunk_o import chunk_fwd_o
+from ..utils.cumsum import chunk_local_cumsum
+from .wy_fast import fwd_prepare_wy_repr
+
+BT = 64
+_SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
+
+
+def _round64(d: int) -> int:
+    return -(-d // 64) * 64
+
+
+def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
+                               offsets=None, indices=None, head_first=True, chunk_size=64,
+                               *, plan: Optional[VarlenPlan] = None, store_A: bool = True):
+    """Reference-shaped forward (``fla/ops/gated_delta_rule/chunk.py:20-73``): returns
+    ``(g_cumsum, o, Aw, Au, final_state)``."""
+    if head_first or chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd: seq-first, chunk size 64 only")
+    if offsets is not None and plan is None:
+        plan = VarlenPlan(offsets, BT)
+    offs = None if plan is None else plan.offsets
+    idx = None if plan is None else plan.indices
+    co = None if plan is None else plan.chunk_offsets
+    g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
+    w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
+                                       store_A=store_A)
+    h, v_new, final_state = chunk_gated_delta_rule_fwd_h(
+        k=k, w=w, u=u, g=g, initial_state=initial_state, output_final_state=output_final_state,
+        offsets=offs, indices=idx, head_first=False, chunk_size=BT, fragment_layout=True, chunk_offsets=co)
+    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False,
+                    chunk_size=BT)
+    return g, o, Aw, Au, final_state
+
+
+class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
+
+    @staticmethod
+    @contiguous
+    @autocast_custom_fwd
+    def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, offsets=None, head_first=True):
+        be.require_gpu(q, k, v, beta)
+        if head_first:
+            q, k, v = (x.transpose(1, 2).contiguous() for x in (q, k, v))
+            beta = beta.transpose(1, 2).contiguous()
+            g = None if g is None else g.transpose(1, 2).contiguous()
+        K, V = q.shape[-1], v.shape[-1]
+        KP, VP = _round64(K), _round64(V)
+        if (KP, VP) not in _SUPPORTED_KV:
+            raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: head dims K={K}, V={V} are outside the built "
+                                      f"tiles {sorted(_SUPPORTED_KV)} (after rounding up to multiples of 64)")
+        h0 = initial_state
+        if (KP, VP) != (K, V):
+            q, k = F.pad(q, (0, KP - K)), F.pad(k, (0, KP - K))
+            v = F.pad(v, (0, VP - V))
+            if h0 is not None:
+                h0 = F.pad(h0, (0, VP - V, 0, KP - K))
+        _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
+                                                    offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+        if (KP, VP) != (K, V):
+            o = o[..., :V]
+            if ht is not None:
+                ht = ht[..., :K, :V].contiguous()
+        if head_first:
+            o = o.transpose(1, 2).contiguous()
+        return o.to(q.dtype), ht
+
+    @staticmethod
+    @contiguous
+    @autocast_custom_bwd
+    def backward(ctx, do, dht):
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule: the backward kernels are not built yet")
+
+
+def chunk_gated_delta_rule(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: torch.Tensor,
+    beta: torch.Tensor,
+    scale: float = None,
+    initial_state: torch.Tensor = None,
+    output_final_state: bool = False,
+    offsets: Optional[torch.LongTensor] = None,
+    head_first: bool = True,
+    cu_seqlens: Optional[torch.LongTensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    r"""
+    Args:
+        q, k: ``[B, H, T, K]`` if ``head_first`` else ``[B, T, H, K]`` (bf16 / fp16).
+        v: ``[B, H, T, V]`` / ``[B, T, H, V]``.
+        g: per-head log decay ``[B, H, T]`` / ``[B, T, H]``.
+        beta: ``[B, H, T]`` / ``[B, T, H]``.
+        scale: default ``K ** -0.5``; must be positive.
+        initial_state: ``[N, H, K, V]`` or ``None``; output_final_state: return the fp32 final state.
+        offsets (synonym ``cu_seqlens``): int64 ``[N+1]`` boundaries of a packed batch (batch 1, seq-first).
+
+    Returns ``(o, final_state)``.
+    """
+    assert q.dtype == k.dtype == v.dtype
+    assert q.dtype != torch.float32, "ChunkDeltaRuleFunction does not support float32. Please use bfloat16."
+    assert len(beta.shape) == 3, "beta must be of shape [B, H, T] if head_first=True, or [B, T, H] if head_first=False."
+    offsets = resolve_offsets(offsets, cu_seqlens)
+    check_varlen_args(q, offsets, head_first, initial_state)
+    if scale is None:
+        scale = k.shape[-1] ** -0.5
+    else:
+        assert scale > 0, "Scale must be positive."
+    return ChunkGatedDeltaRuleFunction.apply(q, k, v, g, beta, scale, initial_state, output_final_state, offsets,
+                                             head_first)

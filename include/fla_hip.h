@@ -132,6 +132,44 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
                         int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                         float scale, fla_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Chunked gated delta rule forward (chunk size 64).  g_cumsum is the fp32
+ * chunk-local prefix sum of the per-head log-gate [B,T,H] (from
+ * fla_chunk_local_cumsum), or NULL for the un-gated delta rule; beta is fp32
+ * [B,T,H].
+ *
+ * fla_gdr_fwd_wy: WY representation, replaces fwd_prepare_wy_repr +
+ * fwd_recompute_w_u (fla/ops/gated_delta_rule/wy_fast.py:320-376 kernel
+ * :111-236; :379-426 kernel :250-317): Aw = (I + strict_lower(diag(beta) K K^T))^-1,
+ * Au = Aw * exp(g_i - g_j), w = Aw (beta K) [B,T,H,K], u = Au (beta V) [B,T,H,V].
+ * Aw, Au (optional outputs, [B,T,H,64] in the q/k/v dtype) are what the
+ * reference saves for backward.
+ *
+ * fla_chunk_gated_delta_rule_fwd_h: state scan, replaces
+ * chunk_gated_delta_rule_fwd_h (fla/ops/common/chunk_delta_h.py:248-320,
+ * kernel :27-119).  Writes the state entering every chunk to h (layout as for
+ * fla_chunk_gla_fwd_h; may be NULL), v_new [B,T,H,V] (may be NULL) and ht.
+ *
+ * fla_chunk_fwd_o: output for scalar-gated models, replaces chunk_fwd_o
+ * (fla/ops/common/chunk_o.py:444-495, kernel :23-101); h must be
+ * FLA_H_FRAGMENT; v is v_new for the delta rule.
+ * ---------------------------------------------------------------------- */
+int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum,
+                   void* w, void* u, void* Aw, void* Au,
+                   const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                   int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, fla_stream_t stream);
+
+int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, const void* u, const float* g_cumsum,
+                                     const float* h0, void* h, void* v_new, float* ht,
+                                     const int64_t* offsets, const int64_t* chunk_offsets,
+                                     int qkv_dtype, int h_dtype, int h_layout,
+                                     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                     fla_stream_t stream);
+
+int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_cumsum, const void* h, void* o,
+                    const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream);
+
 /* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
  * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,
  * mode 1: 16x16x32 tiles, mode 2: 32x32x16 with the permuted contraction order

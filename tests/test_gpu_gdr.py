@@ -1,0 +1,110 @@
+"""GPU: chunk_gated_delta_rule forward against the fp32 naive recurrence and, kernel
+by kernel, against the fp32 chunked oracle."""
+import pytest
+import torch
+
+from helpers import assert_close, gdr_inputs, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+TOL_O, TOL_HT = 1e-2, 5e-3
+
+
+def _run(device, q, k, v, g, beta, h0, offsets=None, head_first=False, scale=None):
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    dev = lambda x: None if x is None else x.to(device)
+    if head_first:
+        q, k, v = (x.transpose(1, 2).contiguous() for x in (q, k, v))
+        g, beta = g.transpose(1, 2).contiguous(), beta.transpose(1, 2).contiguous()
+    o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), scale=scale, initial_state=dev(h0),
+                                   output_final_state=True, offsets=dev(offsets), head_first=head_first)
+    torch.cuda.synchronize()
+    if head_first:
+        o = o.transpose(1, 2)
+    return o, ht
+
+
+def test_gdr_kernel_by_kernel(device):
+    """Aw, Au, w, u, per-chunk h, v_new, o and ht against the fp32 chunked oracle."""
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_h
+    from fla_amd.ops.common.chunk_o import chunk_fwd_o
+    from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_wy_repr
+    from fla_amd.ops.utils import chunk_local_cumsum
+    from oracle.chunked import chunked_gated_delta_rule
+    q, k, v, g, beta, h0 = gdr_inputs(2, 200, 2, 128, 128, seed=21)
+    ref = chunked_gated_delta_rule(q, k, v, g, beta, initial_state=h0)
+    dev = lambda x: x.to(device)
+    print("gdr kernel by kernel", flush=True)
+    gc = chunk_local_cumsum(dev(g), 64, head_first=False)
+    torch.testing.assert_close(gc.cpu(), ref['g_cumsum'], rtol=1e-5, atol=1e-5)
+    w, u, Aw, Au = fwd_prepare_wy_repr(dev(k), dev(v), dev(beta), gc, head_first=False)
+    torch.cuda.synchronize()
+    assert_close("Aw", ref['Aw'], Aw, 5e-3)
+    assert_close("Au", ref['Au'], Au, 5e-3)
+    assert_close("w", ref['w'], w, 8e-3)
+    assert_close("u", ref['u'], u, 8e-3)
+    h, v_new, ht = chunk_gated_delta_rule_fwd_h(dev(k), w, u, gc, dev(h0), True, head_first=False)
+    torch.cuda.synchronize()
+    assert_close("h", ref['h'], h, 8e-3)
+    assert_close("v_new", ref['v_new'], v_new, 1e-2)
+    assert_close("ht", ref['ht'], ht, TOL_HT)
+    hf, v_new2, _ = chunk_gated_delta_rule_fwd_h(dev(k), w, u, gc, dev(h0), False, head_first=False,
+                                                 fragment_layout=True)
+    assert torch.equal(v_new, v_new2)
+    o = chunk_fwd_o(dev(q), dev(k), v_new2, hf, gc, 128 ** -0.5, head_first=False)
+    torch.cuda.synchronize()
+    assert_close("o", ref['o'], o, TOL_O)
+
+
+# reference ladder: tests/ops/test_gated_delta.py:220-294 (T in {7,63,286,300,1000}, scale in {1, 0.1})
+@pytest.mark.parametrize("T", [1, 7, 63, 64, 65, 286, 1000])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
+def test_chunk_gdr_shapes(device, T, K, V):
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = gdr_inputs(2, T, 2, K, V, seed=T + K)
+    print(f"chunk_gdr T={T} K={K} V={V}", flush=True)
+    o, ht = _run(device, q, k, v, g, beta, h0)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    assert o.dtype == q.dtype and ht.dtype == torch.float32
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("scale", [1.0, 0.1])
+@pytest.mark.parametrize("normalizer", [0.1, 1.0, 10.0])
+def test_chunk_gdr_gates_and_scale(device, scale, normalizer):
+    """Strong and weak decays: the scalar gate is applied in fp32 with exponents <= 0."""
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = gdr_inputs(2, 300, 2, 128, 128, seed=22, h0_std=1.0, normalizer=normalizer)
+    print(f"chunk_gdr scale={scale} normalizer={normalizer}", flush=True)
+    o, ht = _run(device, q, k, v, g, beta, h0, scale=scale)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, scale=scale, initial_state=h0,
+                                               output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+def test_chunk_gdr_head_first_odd_dims_no_h0(device):
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, _ = gdr_inputs(2, 150, 3, 100, 100, seed=23, h0=False)
+    print("chunk_gdr head-first D=100", flush=True)
+    o, ht = _run(device, q, k, v, g, beta, None, head_first=True)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+# tests/ops/test_gated_delta.py:297-375
+@pytest.mark.parametrize("T,N", [(64, 2), (300, 4), (1000, 5), (2048, 4)])
+@pytest.mark.parametrize("H", [2, 16])
+def test_chunk_gdr_varlen(device, T, N, H):
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(T + H)
+    offs = random_offsets(T, N, gen, min_len=1)
+    q, k, v, g, beta, h0 = gdr_inputs(1, T, H, 128, 128, seed=24, N=N, h0_std=1.0)
+    print(f"chunk_gdr varlen T={T} H={H} offs={offs.tolist()}", flush=True)
+    o, ht = _run(device, q, k, v, g, beta, h0, offsets=offs)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
