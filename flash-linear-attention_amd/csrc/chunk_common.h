@@ -1,0 +1,86 @@
+// Helpers shared by the chunk kernels: chunk geometry, vector loads with
+// conversion to fp32, the XCD-aware workgroup renumbering.
+#pragma once
+#include "fla_common.h"
+#include "mfma_tiles.h"
+
+namespace {
+
+constexpr int BT = 64;        // chunk length
+constexpr int LDT = BT + 8;   // row pitch of time-contiguous 16-bit LDS tiles
+constexpr int LDM = BT + 4;   // row pitch of fp32 64-column LDS tiles
+
+template <typename X>
+struct Load;
+template <>
+struct Load<float> {
+  static FLA_DEVICE void x4(const float* p, float* o) {
+    f32x4 v = *(const f32x4*)p;
+    o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+  }
+};
+template <>
+struct Load<bf16> {
+  static FLA_DEVICE void x4(const bf16* p, float* o) {
+    bf16x4 v = *(const bf16x4*)p;
+    for (int i = 0; i < 4; ++i) o[i] = (float)v[i];
+  }
+};
+template <>
+struct Load<f16> {
+  static FLA_DEVICE void x4(const f16* p, float* o) {
+    f16x4 v = *(const f16x4*)p;
+    for (int i = 0; i < 4; ++i) o[i] = (float)v[i];
+  }
+};
+
+// Workgroups of one launch are dealt round-robin to the 8 XCDs by linear id.
+// Renumber so that consecutive logical ids share an XCD (and its L2).
+FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
+  if (total % 8 != 0) return id;
+  return (id % 8) * (total / 8) + id / 8;
+}
+
+struct ChunkLoc {
+  int64_t row0;   // first token row of the chunk in the flattened [B*T] space
+  int L;          // valid rows
+  int64_t cglob;  // global chunk index (addresses per-chunk states)
+};
+
+// blockIdx.x enumerates chunks: (batch, chunk) for equal lengths, rows of `indices` otherwise.
+FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix) {
+  ChunkLoc c;
+  int64_t bos, len, ic;
+  if (offsets) {
+    int64_t n = indices[2 * (int64_t)blockIdx.x];
+    ic = indices[2 * (int64_t)blockIdx.x + 1];
+    bos = offsets[n];
+    len = offsets[n + 1] - bos;
+  } else {
+    bos = (blockIdx.x / ntfix) * T;
+    ic = blockIdx.x % ntfix;
+    len = T;
+  }
+  c.row0 = bos + ic * BT;
+  int64_t rem = len - ic * BT;
+  c.L = (int)(rem < BT ? rem : BT);
+  c.cglob = blockIdx.x;
+  return c;
+}
+
+inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B, int64_t T, int64_t H, int64_t NT,
+                      dim3* grid, int* ntfix) {
+  if (offsets) FLA_REQUIRE(indices != nullptr && B == 1, FLA_E_INVALID);
+  int64_t nf = (T + BT - 1) / BT;
+  int64_t nblk = offsets ? NT : B * nf;
+  FLA_REQUIRE(nblk <= 0x7fffffffLL && H <= 65535, FLA_E_UNSUPPORTED);
+  *grid = dim3((unsigned)nblk, (unsigned)H);
+  *ntfix = (int)nf;
+  return FLA_OK;
+}
+
+// Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps
+// the operand finite in 16-bit storage.
+constexpr float kMaxInvDecayExp = 80.f;
+
+}  // namespace

@@ -1,0 +1,738 @@
+// Chunked GLA backward for gfx950 (chunk size 64, 16-bit q/k/v/do, fp32 state).
+//
+// With G the chunk-local prefix sum of the log-gates, q~ = s q e^{G},
+// k^ = k e^{G_last-G}, A = tril(q~ (k e^{-G})^T), dH_c the gradient w.r.t. the state
+// LEAVING chunk c (fla/ops/gla/chunk.py:1217-1320, fla/ops/common/chunk_h.py:156-271):
+//
+//   gla_bwd_dh_kernel    reverse state scan:  store dH_c;  dH <- diag(e^{G_last}) dH + q~^T do.
+//                        The tile is kept in both orientations ([K,V] and [V,K]) and both are
+//                        stored in MFMA-fragment order, because dv contracts dH over K and dk
+//                        over V.  Also emits sum_v h_c * dH_c per key channel (for dg) from the
+//                        recomputed forward states, and dh0.
+//   gla_bwd_dv_kernel    per (chunk, head):  dv = A^T do + k^ dH_c.
+//   gla_bwd_dqkg_kernel  per (chunk, head, 64-wide half of K):
+//                          dA = tril(do v^T)
+//                          dq = s e^{G}  * (dA (k e^{-G}) + do h_c^T)
+//                          dk = s e^{-G} * (dA^T (q e^{G})) + e^{G_last-G} * (v dH_c^T)
+//                          dg = reverse-cumsum(q*dq - k*dk) + sum_t k*dk_inter + e^{G_last} sum_v h_c*dH_c
+//                        (fla/ops/gla/chunk.py:409-567 intra, :726-837 inter incl. the dg formula
+//                        :818-823).  As in the forward, one reference point per chunk replaces
+//                        the 16x16 sub-block scheme.
+#include "chunk_common.h"
+
+namespace {
+
+struct BDhParams {
+  const void* q;
+  const void* g;
+  const void* dout;
+  const float* dht;
+  const void* hT;     // forward states, FLA_H_FRAGMENT_T
+  void* dhf;          // out: dH, FLA_H_FRAGMENT
+  void* dhtf;         // out: dH, FLA_H_FRAGMENT_T
+  float* hdh;         // out: [V/32][chunks][H][K] partial sums of h*dH over 32 value columns
+  float* dh0;         // out: fp32 [N,H,K,V] or null
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int64_t total_chunks;
+  int H, K, V, N;
+  float scale;
+};
+
+template <typename T, typename GT>
+__global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  typedef GT g2 __attribute__((ext_vector_type(2)));
+  __shared__ __attribute__((aligned(16))) T sQt[2][64 * LDT];  // [k][t] s q e^{G}
+  __shared__ __attribute__((aligned(16))) T sDt[2][64 * LDT];  // [v][t] do
+  __shared__ __attribute__((aligned(16))) float sDecay[2][64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, V = p.V;
+  const int nkt = K / 64, nvt = V / 64, ntile = nkt * nvt;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile = (int)(id % ntile);
+  const int nh = (int)(id / ntile);
+  const int n = nh / H, hh = nh % H;
+  const int kbase = (tile % nkt) * 64, vbase = (tile / nkt) * 64;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+
+  const int rg = lane >> 3, c2 = wave * 16 + (lane & 7) * 2;
+  const T* qp = (const T*)p.q + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
+  const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kbase + c2;
+  const T* dp = (const T*)p.dout + (sp.bos * H + hh) * (int64_t)V + vbase + c2;
+  const int64_t kstride = (int64_t)H * K, vstride = (int64_t)H * V;
+
+  const int kq = wave & 1, vq = wave >> 1;
+  const int kt32 = kbase / 32 + kq, vt32 = vbase / 32 + vq;
+  const int vcol = vbase + vq * 32 + (lane & 31), kcol = kbase + kq * 32 + (lane & 31);
+  f32x16 acc1 = zero16();  // rows k, cols v
+  f32x16 acc2 = zero16();  // rows v, cols k
+  if (p.dht) {
+    const float* dp0 = p.dht + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc1[r] = dp0[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
+      acc2[r] = dp0[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)];
+    }
+  }
+
+  struct Regs {
+    g2 g[8];
+    t2 q[8];
+    t2 d[8];
+    v8 h[2];
+  };
+  auto load_chunk = [&](int64_t c, Regs& R) {
+    bool live = c >= 0;
+    int64_t t0 = c * BT;
+    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int row = rg * 8 + i;
+      if (live && row < L) {
+        R.g[i] = *(const g2*)(gp + (t0 + row) * kstride);
+        R.q[i] = *(const t2*)(qp + (t0 + row) * kstride);
+        R.d[i] = *(const t2*)(dp + (t0 + row) * vstride);
+      } else {
+        R.g[i] = g2{(GT)0.f, (GT)0.f};
+        R.q[i] = t2{(T)0.f, (T)0.f};
+        R.d[i] = t2{(T)0.f, (T)0.f};
+      }
+    }
+    if (live) {
+      const T* hp = (const T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V +
+                    (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
+      R.h[0] = *(const v8*)hp;
+      R.h[1] = *(const v8*)(hp + 8);
+    }
+  };
+
+  Regs R0, R1, R2;
+  load_chunk(nchunks - 1, R0);
+  load_chunk(nchunks - 2, R1);
+  for (int64_t c = nchunks - 1; c >= 0; --c) {
+    const int buf = (int)(c & 1);
+    int64_t t0 = c * BT;
+    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+    load_chunk(c - 2, R2);
+    // ---- gradient w.r.t. the state leaving chunk c, both orientations, fragment order
+    {
+      int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
+      v8 lo, hi;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        lo[r] = (T)acc1[r];
+        hi[r] = (T)acc1[r + 8];
+      }
+      T* o1 = (T*)p.dhf + blk + (((int64_t)kt32 * (V / 32) + vt32) * 64 + lane) * 16;
+      *(v8*)o1 = lo;
+      *(v8*)(o1 + 8) = hi;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        lo[r] = (T)acc2[r];
+        hi[r] = (T)acc2[r + 8];
+      }
+      T* o2 = (T*)p.dhtf + blk + (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
+      *(v8*)o2 = lo;
+      *(v8*)(o2 + 8) = hi;
+      // sum over this wave's 32 value columns of h_c * dH_c, one key channel per lane
+      float part = 0.f;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) part += (float)R0.h[0][r] * acc2[r] + (float)R0.h[1][r] * acc2[r + 8];
+      part += __shfl_xor(part, 32, 64);
+      if (lane < 32) p.hdh[(((int64_t)vt32 * p.total_chunks + chunk0 + c) * H + hh) * K + kcol] = part;
+    }
+    // ---- chunk-local prefix sums of the gates
+    float G[8][2], glast0, glast1;
+    {
+      float r0 = 0.f, r1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        r0 += (float)R0.g[i][0];
+        r1 += (float)R0.g[i][1];
+        G[i][0] = r0;
+        G[i][1] = r1;
+      }
+      float s0 = r0, s1 = r1;
+#pragma unroll
+      for (int d = 8; d < 64; d <<= 1) {
+        float u0 = __shfl_up(s0, d, 64), u1 = __shfl_up(s1, d, 64);
+        if (lane >= d) {
+          s0 += u0;
+          s1 += u1;
+        }
+      }
+      float off0 = s0 - r0, off1 = s1 - r1;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        G[i][0] += off0;
+        G[i][1] += off1;
+      }
+      glast0 = __shfl(s0, 56 + (lane & 7), 64);
+      glast1 = __shfl(s1, 56 + (lane & 7), 64);
+    }
+    {
+      v8 qa, qb, da, db;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        bool valid = (rg * 8 + i) < L;
+        qa[i] = (T)(valid ? (float)R0.q[i][0] * p.scale * __expf(G[i][0]) : 0.f);
+        qb[i] = (T)(valid ? (float)R0.q[i][1] * p.scale * __expf(G[i][1]) : 0.f);
+        da[i] = R0.d[i][0];
+        db[i] = R0.d[i][1];
+      }
+      *(v8*)&sQt[buf][(c2 + 0) * LDT + rg * 8] = qa;
+      *(v8*)&sQt[buf][(c2 + 1) * LDT + rg * 8] = qb;
+      *(v8*)&sDt[buf][(c2 + 0) * LDT + rg * 8] = da;
+      *(v8*)&sDt[buf][(c2 + 1) * LDT + rg * 8] = db;
+      if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) acc1[4 * a + b] *= d[b];
+    }
+    {
+      const float d = sDecay[buf][kq * 32 + (lane & 31)];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[r] *= d;
+    }
+#pragma unroll
+    for (int s = 0; s < BT; s += 16) {
+      v8 fq = lds_frag32<T>(sQt[buf], LDT, kq * 32, s, lane);
+      v8 fd = lds_frag32<T>(sDt[buf], LDT, vq * 32, s, lane);
+      acc1 = Elem<T>::mfma32(fq, fd, acc1);
+      acc2 = Elem<T>::mfma32(fd, fq, acc2);
+    }
+    R0 = R1;
+    R1 = R2;
+  }
+  if (p.dh0) {
+    float* o = p.dh0 + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc1[r];
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct BDvParams {
+  const void* q;
+  const void* k;
+  const void* g;
+  const void* dout;
+  const void* dhf;
+  void* dv;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+template <typename T, typename GT, int K, int V>
+__global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int KT32 = K / 32, TV = V / 64;
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];    // s q e^{G-G_last}
+  __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];   // k e^{G_last-G}
+  __shared__ __attribute__((aligned(16))) T sDt[V * LDT];    // do^T [v][i]
+  __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];   // A^T [j][i]
+  __shared__ __attribute__((aligned(16))) float sPart[RG * K];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, hh = blockIdx.y;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  float gq[RPT][4], qq[RPT][4], kk[RPT][4];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
+      Load<GT>::x4((const GT*)p.g + off, gq[i]);
+      Load<T>::x4((const T*)p.q + off, qq[i]);
+      Load<T>::x4((const T*)p.k + off, kk[i]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gq[i][j] = qq[i][j] = kk[i][j] = 0.f;
+    }
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+  v4 dreg[RPTV];
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) {
+    int row = rgv * RPTV + i;
+    if (row < L) dreg[i] = *(const v4*)((const T*)p.dout + ((row0 + row) * H + hh) * (int64_t)V + cv4);
+    else dreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  }
+  const int rw = wave >> 1, cw = wave & 1;
+  v8 hf[KT32][TV][2];
+  {
+    const T* hp = (const T*)p.dhf + (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) {
+        const T* f = hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16;
+        hf[kt][tv][0] = *(const v8*)f;
+        hf[kt][tv][1] = *(const v8*)(f + 8);
+      }
+  }
+  // ---- prefix sums and G_last
+  float G[RPT][4], glast[4];
+  {
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        run[j] += gq[i][j];
+        G[i][j] = run[j];
+      }
+    *(f32x4*)&sPart[rg * K + c4] = f32x4{run[0], run[1], run[2], run[3]};
+    __syncthreads();
+    float off[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) glast[j] = 0.f;
+#pragma unroll
+    for (int r = 0; r < RG; ++r) {
+      f32x4 pr = *(const f32x4*)&sPart[r * K + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (r < rg) off[j] += pr[j];
+        glast[j] += pr[j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) G[i][j] += off[j];
+  }
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    v4 qv, kv;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float up = fminf(G[i][j] - glast[j], kMaxInvDecayExp);
+      qv[j] = (T)(qq[i][j] * p.scale * __expf(up));
+      kv[j] = (T)(kk[i][j] * __expf(glast[j] - G[i][j]));
+    }
+    *(v4*)&sQ[row * LDK + c4] = qv;
+    *(v4*)&sKh[row * LDK + c4] = kv;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T* dst = &sDt[(cv4 + j) * LDT + rgv * RPTV];
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) dst[i] = dreg[i][j];
+  }
+  __syncthreads();
+  // ---- A^T on the lower-triangular quadrants
+  {
+    const int qi = wave >> 1, qj = wave & 1;
+    if (qj <= qi) {
+      f32x16 s = zero16();
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 16)
+        s = Elem<T>::mfma32(lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), lds_frag32<T>(sKh, LDK, qj * 32, ks, lane), s);
+      const int j = qj * 32 + (lane & 31);
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        int i0 = qi * 32 + 8 * a + 4 * (lane >> 5);
+        v4 x;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) x[b] = (T)((j <= i0 + b) ? s[4 * a + b] : 0.f);
+        *(v4*)&sPT[j * LDT + i0] = x;
+      }
+    }
+  }
+  __syncthreads();
+  // ---- dv = A^T do + k^ dH
+  f32x16 acc[TV];
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+  for (int is = rw * 32; is < BT; is += 16) {
+    v8 a = lds_frag32<T>(sPT, LDT, rw * 32, is, lane);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), acc[tv]);
+  }
+#pragma unroll
+  for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v8 a = lds_frag32_perm<T>(sKh, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(a, hf[kt][tv][half], acc[tv]);
+    }
+  T* op = (T*)p.dv + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = rw * 32 + c32_row(r, lane);
+      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    }
+}
+
+// ---------------------------------------------------------------------------
+struct BDqkgParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const void* dout;
+  const void* hT;     // forward states, FLA_H_FRAGMENT_T
+  const void* dhtf;   // dH, FLA_H_FRAGMENT_T
+  const float* hdh;   // [V/32][chunks][H][K]
+  void* dq;
+  void* dk;
+  float* dg;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int64_t total_chunks;
+  int H, K, NTfix;
+  float scale;
+};
+
+// grid (chunks, H, K/64): one workgroup per 64-wide slice of the key dim.
+template <typename T, typename GT, int V>
+__global__ __launch_bounds__(256) void gla_bwd_dqkg_kernel(BDqkgParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDV = V + 8;
+  constexpr int C8 = V / 8, NP = BT * C8 / 256;
+  constexpr int VT32 = V / 32;
+  constexpr int ROWB = BT * LDV * 2;                       // bytes of one row-major [64][V] tile
+  constexpr int STG = BT * LDM * 4;                        // bytes of one fp32 [64][64] staging tile
+  constexpr int REG_A = ROWB > STG ? ROWB : STG;
+  constexpr int REG_C = (2 * BT * LDT * 2 > STG) ? 2 * BT * LDT * 2 : STG;
+  __shared__ __attribute__((aligned(16))) char sRA[REG_A];   // do row-major; later staging of the dq accumulators
+  __shared__ __attribute__((aligned(16))) char sRB[REG_A];   // v row-major;  later staging of the intra dk accumulators
+  __shared__ __attribute__((aligned(16))) char sRC[REG_C];   // (k e^{-G})^T | (q e^{G})^T; later staging of the inter dk acc
+  __shared__ __attribute__((aligned(16))) T sdA[BT * LDT];   // dA  [i][j]
+  __shared__ __attribute__((aligned(16))) T sdAT[BT * LDT];  // dA^T [j][i]
+  __shared__ __attribute__((aligned(16))) float sPart[16 * 64];
+  __shared__ __attribute__((aligned(16))) float sPart2[16 * 64];
+  T* sDo = (T*)sRA;
+  T* sV = (T*)sRB;
+  T* sKtT = (T*)sRC;
+  T* sQtT = sKtT + BT * LDT;
+  float* stA = (float*)sRA;
+  float* stB = (float*)sRB;
+  float* stC = (float*)sRC;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, hh = blockIdx.y;
+  const int kb = blockIdx.z * 64;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+
+  // ---- loads: q,k,g slice as 4 rows x 4 cols per lane; do, v whole rows in 16-byte pieces
+  const int rg = tid >> 4, c4 = (tid & 15) * 4;
+  float gq[4][4], qq[4][4], kk[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = rg * 4 + i;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
+      Load<GT>::x4((const GT*)p.g + off, gq[i]);
+      Load<T>::x4((const T*)p.q + off, qq[i]);
+      Load<T>::x4((const T*)p.k + off, kk[i]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gq[i][j] = qq[i][j] = kk[i][j] = 0.f;
+    }
+  }
+  v8 dreg[NP], vreg[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)V + c8;
+      dreg[i] = *(const v8*)((const T*)p.dout + off);
+      vreg[i] = *(const v8*)((const T*)p.v + off);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dreg[i][j] = vreg[i][j] = (T)0.f;
+    }
+  }
+  // operand fragments: wave (rw, cw) produces rows 32rw.., key columns kb + 32cw..
+  const int rw = wave >> 1, cw = wave & 1;
+  const int kt32 = kb / 32 + cw;
+  v8 hf[VT32][2], dhf[VT32][2];
+  {
+    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int vt = 0; vt < VT32; ++vt) {
+      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
+      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
+      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
+      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
+      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
+    }
+  }
+  // ---- prefix sums of the gates over the 16 row groups
+  float G[4][4], glast[4];
+  {
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        run[j] += gq[i][j];
+        G[i][j] = run[j];
+      }
+    *(f32x4*)&sPart[rg * 64 + c4] = f32x4{run[0], run[1], run[2], run[3]};
+    __syncthreads();
+    float off[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) glast[j] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      f32x4 pr = *(const f32x4*)&sPart[r * 64 + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (r < rg) off[j] += pr[j];
+        glast[j] += pr[j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) G[i][j] += off[j];
+  }
+  // ---- operand tiles
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sDo[row * LDV + c8] = dreg[i];
+    *(v8*)&sV[row * LDV + c8] = vreg[i];
+  }
+  float einv[4][4];  // e^{-G}, clamped
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) einv[i][j] = __expf(fminf(-G[i][j], kMaxInvDecayExp));
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v4 kt, qt;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kt[i] = (T)(kk[i][j] * einv[i][j]);
+      qt[i] = (T)(qq[i][j] * __expf(G[i][j]));
+    }
+    *(v4*)&sKtT[(c4 + j) * LDT + rg * 4] = kt;
+    *(v4*)&sQtT[(c4 + j) * LDT + rg * 4] = qt;
+  }
+  __syncthreads();
+  // ---- dA = tril(do v^T) in both orientations (each gives 8-byte LDS writes)
+  {
+    const int ib = wave >> 1, jb = wave & 1;
+    if (jb <= ib) {
+      f32x16 s1 = zero16(), s2 = zero16();
+#pragma unroll
+      for (int vs = 0; vs < V; vs += 16) {
+        v8 fd = lds_frag32<T>(sDo, LDV, ib * 32, vs, lane);
+        v8 fv = lds_frag32<T>(sV, LDV, jb * 32, vs, lane);
+        s1 = Elem<T>::mfma32(fd, fv, s1);  // rows i, cols j
+        s2 = Elem<T>::mfma32(fv, fd, s2);  // rows j, cols i
+      }
+      const int c = lane & 31;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        int r0 = 8 * a + 4 * (lane >> 5);
+        v4 x1, x2;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          int i1 = ib * 32 + r0 + b, j1 = jb * 32 + c;      // s1 element (i1, j1)
+          x1[b] = (T)((j1 <= i1) ? s1[4 * a + b] : 0.f);
+          int j2 = jb * 32 + r0 + b, i2 = ib * 32 + c;      // s2 element (j2, i2)
+          x2[b] = (T)((j2 <= i2) ? s2[4 * a + b] : 0.f);
+        }
+        *(v4*)&sdAT[(jb * 32 + c) * LDT + ib * 32 + r0] = x1;  // dA^T[j][i..i+3]
+        *(v4*)&sdA[(ib * 32 + c) * LDT + jb * 32 + r0] = x2;   // dA[i][j..j+3]
+      }
+    } else {
+      // quadrant (i block 0, j block 1) is strictly above the diagonal
+      for (int e = lane; e < 32 * 8; e += 64) {
+        int r = e >> 3, c = (e & 7) * 4;
+        *(v4*)&sdA[r * LDT + 32 + c] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        *(v4*)&sdAT[(32 + r) * LDT + c] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      }
+    }
+  }
+  __syncthreads();
+  // ---- accumulate: dq (intra + inter), dk intra, dk inter
+  f32x16 aq = zero16(), ak1 = zero16(), ak2 = zero16();
+  const int jend = (rw + 1) * 32;
+  for (int js = 0; js < jend; js += 16)
+    aq = Elem<T>::mfma32(lds_frag32<T>(sdA, LDT, rw * 32, js, lane), lds_frag32<T>(sKtT, LDT, cw * 32, js, lane), aq);
+  for (int is = rw * 32; is < BT; is += 16)
+    ak1 = Elem<T>::mfma32(lds_frag32<T>(sdAT, LDT, rw * 32, is, lane), lds_frag32<T>(sQtT, LDT, cw * 32, is, lane), ak1);
+#pragma unroll
+  for (int vt = 0; vt < VT32; ++vt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      aq = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aq);
+      ak2 = Elem<T>::mfma32(lds_frag32_perm<T>(sV, LDV, rw * 32, vt * 32 + half * 16, lane), dhf[vt][half], ak2);
+    }
+  __syncthreads();  // every MFMA operand read is done: the tiles become fp32 staging
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    int o = (rw * 32 + c32_row(r, lane)) * LDM + cw * 32 + (lane & 31);
+    stA[o] = aq[r];
+    stB[o] = ak1[r];
+    stC[o] = ak2[r];
+  }
+  __syncthreads();
+  // ---- epilogue in the load mapping (4 rows x 4 key channels per lane)
+  float x[4][4], ksum[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = rg * 4 + i;
+    f32x4 a = *(const f32x4*)&stA[row * LDM + c4];
+    f32x4 b = *(const f32x4*)&stB[row * LDM + c4];
+    f32x4 c = *(const f32x4*)&stC[row * LDM + c4];
+    v4 dqv, dkv;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float dq = p.scale * __expf(G[i][j]) * a[j];
+      float dki = __expf(glast[j] - G[i][j]) * c[j];
+      float dk = p.scale * einv[i][j] * b[j] + dki;
+      dqv[j] = (T)dq;
+      dkv[j] = (T)dk;
+      x[i][j] = qq[i][j] * dq - kk[i][j] * dk;
+      ksum[j] += kk[i][j] * dki;
+    }
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
+      *(v4*)((T*)p.dq + off) = dqv;
+      *(v4*)((T*)p.dk + off) = dkv;
+    }
+  }
+  // reverse cumsum over rows + column sums of k*dk_inter
+  float suf[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 3; i >= 0; --i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      suf[j] += x[i][j];
+      x[i][j] = suf[j];
+    }
+  *(f32x4*)&sPart[rg * 64 + c4] = f32x4{suf[0], suf[1], suf[2], suf[3]};
+  *(f32x4*)&sPart2[rg * 64 + c4] = f32x4{ksum[0], ksum[1], ksum[2], ksum[3]};
+  __syncthreads();
+  float add[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    f32x4 s1 = *(const f32x4*)&sPart[r * 64 + c4];
+    f32x4 s2 = *(const f32x4*)&sPart2[r * 64 + c4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (r > rg) add[j] += s1[j];
+      add[j] += s2[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float hd = 0.f;
+    for (int vt = 0; vt < VT32; ++vt)
+      hd += p.hdh[(((int64_t)vt * p.total_chunks + cl.cglob) * H + hh) * K + kb + c4 + j];
+    add[j] += __expf(glast[j]) * hd;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = rg * 4 + i;
+    if (row < L) {
+      f32x4 o = {x[i][0] + add[0], x[i][1] + add[1], x[i][2] + add[2], x[i][3] + add[3]};
+      *(f32x4*)(p.dg + ((row0 + row) * H + hh) * (int64_t)K + kb + c4) = o;
+    }
+  }
+}
+
+template <typename T, typename GT>
+int launch_bwd(const void* q, const void* k, const void* v, const void* g, const void* dout, const float* dht,
+               const void* hT, void* dhf, void* dhtf, float* hdh, void* dq, void* dk, void* dv, float* dg, float* dh0,
+               const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
+               int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  const int64_t total_chunks = grid.x;
+  {
+    BDhParams p{q, g, dout, dht, hT, dhf, dhtf, hdh, dh0, offsets, chunk_offsets, T_, total_chunks,
+                (int)H, (int)K, (int)V, (int)N, scale};
+    int64_t total = (K / 64) * (V / 64) * N * H;
+    FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+    hipLaunchKernelGGL((gla_bwd_dh_kernel<T, GT>), dim3((unsigned)total), dim3(256), 0, st, p);
+    FLA_CHECK_LAUNCH();
+  }
+  {
+    BDvParams p{q, k, g, dout, dhf, dv, offsets, indices, T_, (int)H, ntfix, scale};
+#define FLA_CASE(KK, VV)                                                                            \
+  if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_dv_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
+    FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
+#undef FLA_CASE
+    FLA_CHECK_LAUNCH();
+  }
+  {
+    BDqkgParams p{q, k, v, g, dout, hT, dhtf, hdh, dq, dk, dg, offsets, indices, T_, total_chunks,
+                  (int)H, (int)K, ntfix, scale};
+    dim3 g3(grid.x, grid.y, (unsigned)(K / 64));
+    if (V == 64) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 64>), g3, dim3(256), 0, st, p);
+    else if (V == 128) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 128>), g3, dim3(256), 0, st, p);
+    else return FLA_E_UNSUPPORTED;
+    FLA_CHECK_LAUNCH();
+  }
+  return FLA_OK;
+}
+
+}  // namespace
+
+extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
+                                 const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
+                                 void* dq, void* dk, void* dv, float* dg, float* dh0, const int64_t* offsets,
+                                 const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
+                                 int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                 float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag && dh_frag_t && hdh && dq && dk && dv && dg,
+              FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)dout | (uintptr_t)hT |
+               (uintptr_t)dh_frag | (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
+               (uintptr_t)dg) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  hipStream_t st = (hipStream_t)stream;
+#define FLA_BWD(TT, GG)                                                                                           \
+  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag, dh_frag_t, hdh, dq, dk, dv, dg, dh0, offsets, \
+                            indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_BWD(bf16, float);
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_BWD(bf16, bf16);
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) FLA_BWD(f16, float);
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) FLA_BWD(f16, f16);
+#undef FLA_BWD
+  return FLA_E_UNSUPPORTED;
+}

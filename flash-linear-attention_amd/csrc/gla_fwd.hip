@@ -127,11 +127,17 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
   // accumulator tile of this wave: rows k = kq*32.., cols v = vq*32..
   const int kq = wave & 1, vq = wave >> 1;
   const int vcol = vbase + vq * 32 + (lane & 31);
+  // HL == 3 keeps the tile transposed (rows v, cols k) so that its registers can
+  // feed MFMA operands of products that contract over v (used by the backward pass).
+  constexpr bool TR = (HL == 3);
+  const int kcol = kbase + kq * 32 + (lane & 31);
   f32x16 acc = zero16();
   if (p.h0) {
     const float* h0p = p.h0 + (int64_t)nh * K * V;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = h0p[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
+    for (int r = 0; r < 16; ++r)
+      acc[r] = TR ? h0p[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)]
+                  : h0p[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
   }
 
   struct Regs {
@@ -168,8 +174,10 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
     // ---- state entering chunk c
     if (p.h) {
       int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
-      if (HL == 1) {
-        T* hp = (T*)p.h + blk + (((int64_t)(kbase / 32 + kq) * (V / 32) + (vbase / 32 + vq)) * 64 + lane) * 16;
+      if (HL == 1 || HL == 3) {
+        T* hp = (T*)p.h + blk +
+                (TR ? (((int64_t)(vbase / 32 + vq) * (K / 32) + (kbase / 32 + kq)) * 64 + lane) * 16
+                    : (((int64_t)(kbase / 32 + kq) * (V / 32) + (vbase / 32 + vq)) * 64 + lane) * 16);
         v8 lo, hi;
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
@@ -251,23 +259,36 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
       if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
     }
     __syncthreads();  // tiles of chunk c complete; buffer buf^1 is free again after the next barrier
+    if (TR) {
+      const float d = sDecay[buf][kq * 32 + (lane & 31)];
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];
+      for (int r = 0; r < 16; ++r) acc[r] *= d;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) acc[4 * a + b] *= d[b];
+      for (int s = 0; s < BT; s += 16)
+        acc = Elem<T>::mfma32(lds_frag32<T>(sVt[buf], LDT, vq * 32, s, lane),
+                              lds_frag32<T>(sKt[buf], LDT, kq * 32, s, lane), acc);
+    } else {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[4 * a + b] *= d[b];
+      }
+#pragma unroll
+      for (int s = 0; s < BT; s += 16)
+        acc = Elem<T>::mfma32(lds_frag32<T>(sKt[buf], LDT, kq * 32, s, lane),
+                              lds_frag32<T>(sVt[buf], LDT, vq * 32, s, lane), acc);
     }
-#pragma unroll
-    for (int s = 0; s < BT; s += 16)
-      acc = Elem<T>::mfma32(lds_frag32<T>(sKt[buf], LDT, kq * 32, s, lane),
-                            lds_frag32<T>(sVt[buf], LDT, vq * 32, s, lane), acc);
     R0 = R1;
     R1 = R2;
   }
   if (p.ht) {
     float* htp = p.ht + (int64_t)nh * K * V;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) htp[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc[r];
+    for (int r = 0; r < 16; ++r) {
+      if (TR) htp[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)] = acc[r];
+      else htp[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc[r];
+    }
   }
 }
 
@@ -496,6 +517,8 @@ int launch_h(const HParams& p, int h_dtype, int h_layout, hipStream_t st) {
   dim3 grid((unsigned)total), block(256);
   if (h_layout == FLA_H_FRAGMENT) {
     hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 1>), grid, block, 0, st, p);
+  } else if (h_layout == FLA_H_FRAGMENT_T) {
+    hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 3>), grid, block, 0, st, p);
   } else if (h_dtype == FLA_F32) {
     hipLaunchKernelGGL((gla_fwd_h_kernel<T, GT, GCUM, 2>), grid, block, 0, st, p);
   } else {
@@ -544,8 +567,9 @@ extern "C" int fla_chunk_gla_fwd_h(const void* k, const void* v, const void* gat
   FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 512 && V <= 512 && H <= 65535, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(chunk_offsets != nullptr && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
-  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT, FLA_E_INVALID);
-  if (h_layout == FLA_H_FRAGMENT) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT || h_layout == FLA_H_FRAGMENT_T,
+              FLA_E_INVALID);
+  if (h_layout != FLA_H_ROW_MAJOR) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
   else FLA_REQUIRE(h_dtype == qkv_dtype || h_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   if (gates_are_cumsum) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)h) % 16 == 0, FLA_E_ALIGNMENT);

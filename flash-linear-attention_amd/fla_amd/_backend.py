@@ -15,7 +15,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
-FLA_H_ROW_MAJOR, FLA_H_FRAGMENT = 0, 1
+FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
 ABI_VERSION = 1
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
@@ -41,6 +41,7 @@ SIGNATURES = {
     "fla_chunk_gated_delta_rule_fwd_h": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                                  I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gla_bwd": (c_int, [P] * 18 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_selftest_mfma": (c_int, [P, P, P, I64, I64, I64, I, P]),
 }
 

@@ -26,6 +26,7 @@ def chunk_fwd_h(
     *,
     gates_are_cumsum: bool = True,
     fragment_layout: bool = False,
+    transposed_fragments: bool = False,
     chunk_offsets: Optional[torch.Tensor] = None,
     store_states: bool = True,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
@@ -65,6 +66,7 @@ def chunk_fwd_h(
     be.check(be.lib().fla_chunk_gla_fwd_h(
         be.ptr(k), be.ptr(v), be.ptr(gk), int(gates_are_cumsum), be.ptr(h0), be.ptr(h), be.ptr(ht),
         be.ptr(offsets), be.ptr(chunk_offsets), be.dt(k), be.dt(gk), be._DTYPES[h_dtype],
-        be.FLA_H_FRAGMENT if fragment_layout else be.FLA_H_ROW_MAJOR,
+        (be.FLA_H_FRAGMENT_T if transposed_fragments else be.FLA_H_FRAGMENT) if fragment_layout
+        else be.FLA_H_ROW_MAJOR,
         B, T, H, K, V, N, be.stream_of(k)), "fla_chunk_gla_fwd_h")
     return h, ht

@@ -97,16 +97,46 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
     return g_cumsum, A, h, ht, o
 
 
+def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets):
+    """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
+    Returns ``(dq, dk, dv, dg, dh0)``; recomputes the per-chunk states as the
+    reference does (``fla/ops/gla/chunk.py:1239-1253``)."""
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    offs = None if plan is None else plan.offsets
+    idx = None if plan is None else plan.indices
+    co = None if plan is None else plan.chunk_offsets
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    N = B if plan is None else plan.N
+    NT = 0 if plan is None else plan.NT
+    hT, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=False,
+                        offsets=offs, indices=idx, head_first=False, chunk_size=BT, gates_are_cumsum=False,
+                        fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
+    total_chunks = hT.shape[0] * hT.shape[1]
+    dhf, dhtf = torch.empty_like(hT), torch.empty_like(hT)
+    hdh = q.new_empty(V // 32, total_chunks, H, K, dtype=torch.float32)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dg = q.new_empty(B, T, H, K, dtype=torch.float32)
+    dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
+    if dht is not None:
+        dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
+    be.check(be.lib().fla_chunk_gla_bwd(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(dhf), be.ptr(dhtf),
+        be.ptr(hdh), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(offs), be.ptr(idx),
+        be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_bwd")
+    return dq, dk, dv, dg, dh0
+
+
 class ChunkGLAFunction(torch.autograd.Function):
 
     @staticmethod
     @contiguous
     def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, offsets, head_first):
         be.require_gpu(q, k, v, g)
+        in_dtypes = (q.dtype, k.dtype, v.dtype, g.dtype)
         if head_first:
             q, k, v, g = (x.transpose(1, 2).contiguous() for x in (q, k, v, g))
-        dtype = q.dtype
-        if dtype == torch.float32:
+        if q.dtype == torch.float32:
             warnings.warn("fla_amd chunk_gla: fp32 q/k/v are rounded to bf16 for the MFMA kernels "
                           "(state and gates stay fp32)", stacklevel=3)
             q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
@@ -125,12 +155,15 @@ class ChunkGLAFunction(torch.autograd.Function):
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
         o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets)
+        # like the reference, keep the inputs and recompute everything else in backward
+        ctx.save_for_backward(q, k, v, g, h0, offsets)
+        ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
+        ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
             o = o[..., :V]
             if ht is not None:
                 ht = ht[..., :K, :V].contiguous()
-        if dtype == torch.float32:
-            o = o.float()
+        o = o.to(in_dtypes[2])
         if head_first:
             o = o.transpose(1, 2).contiguous()
         return o, ht
@@ -138,7 +171,27 @@ class ChunkGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        raise NotImplementedError("fla_amd chunk_gla: the backward kernels are not built yet")
+        q, k, v, g, h0, offsets = ctx.saved_tensors
+        K, V, KP, VP = ctx.dims
+        if ctx.head_first:
+            do = do.transpose(1, 2)
+        do = do.to(q.dtype)
+        if VP != V:
+            do = F.pad(do, (0, VP - V))
+        do = do.contiguous()
+        if dht is not None and (KP, VP) != (K, V):
+            dht = F.pad(dht, (0, VP - V, 0, KP - K))
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets)
+        if (KP, VP) != (K, V):
+            dq, dk, dg, dv = dq[..., :K], dk[..., :K], dg[..., :K], dv[..., :V]
+            if dh0 is not None:
+                dh0 = dh0[..., :K, :V]
+        if ctx.head_first:
+            dq, dk, dv, dg = (x.transpose(1, 2) for x in (dq, dk, dv, dg))
+        qd, kd, vd, gd = ctx.in_dtypes
+        if dh0 is not None:
+            dh0 = dh0.to(ctx.h0_dtype)
+        return dq.to(qd), dk.to(kd), dv.to(vd), dg.to(gd), None, dh0, None, None, None
 
 
 def chunk_gla(

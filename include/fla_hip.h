@@ -107,7 +107,10 @@ int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const void* k, const
  * [1,NT_total,H,K,V], addressed through chunk_offsets [N+1]); h_layout selects
  *   FLA_H_ROW_MAJOR  plain [K,V] tiles of dtype h_dtype (the reference layout),
  *   FLA_H_FRAGMENT   bf16/fp16 tiles in MFMA-fragment order, consumed only by
- *                    fla_chunk_gla_fwd_o / fla_chunk_fwd_o (same byte size).
+ *                    fla_chunk_gla_fwd_o / fla_chunk_fwd_o (same byte size),
+ *   FLA_H_FRAGMENT_T the same with every tile transposed ([V,K] orientation), the
+ *                    operand order of products that contract over V; consumed
+ *                    only by the backward entry points.
  * h may be NULL when only ht is wanted.  h0, ht fp32 [N,H,K,V] or NULL.
  *
  * fla_chunk_gla_fwd_o: fused cumsum + intra-chunk gated scores + output,
@@ -116,7 +119,7 @@ int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const void* k, const
  * h must be FLA_H_FRAGMENT.  A_out (optional, fp32 [B,T,H,64]) receives the
  * lower-triangular score matrix the reference saves for backward.
  * ---------------------------------------------------------------------- */
-enum fla_h_layout { FLA_H_ROW_MAJOR = 0, FLA_H_FRAGMENT = 1 };
+enum fla_h_layout { FLA_H_ROW_MAJOR = 0, FLA_H_FRAGMENT = 1, FLA_H_FRAGMENT_T = 2 };
 
 int fla_chunk_gla_fwd_h(const void* k, const void* v, const void* gates, int gates_are_cumsum,
                         const float* h0, void* h, float* ht,
@@ -169,6 +172,28 @@ int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, const void* u
 int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_cumsum, const void* h, void* o,
                     const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Chunked GLA backward (chunk size 64), replaces chunk_gla_bwd
+ * (fla/ops/gla/chunk.py:1217-1320: chunk_bwd_dh common/chunk_h.py:338-402,
+ * chunk_gla_bwd_dv :1018, _dA :982, _dqk_intra :1057, _dqkg :1102).
+ * Three launches on `stream`: reverse state scan, dv, dq/dk/dg.
+ *   gates   raw log-gates [B,T,H,K] (fp32 or the q/k/v dtype)
+ *   dout    gradient of o, [B,T,H,V] in the q/k/v dtype; dht fp32 [N,H,K,V] or NULL
+ *   hT      forward states recomputed by fla_chunk_gla_fwd_h with FLA_H_FRAGMENT_T
+ *   dh_frag, dh_frag_t   workspaces, each the size of hT (gradient of the
+ *           per-chunk states in the two fragment orientations)
+ *   hdh     workspace fp32 [V/32, chunks, H, K]
+ *   dq, dk [B,T,H,K] and dv [B,T,H,V] in the q/k/v dtype; dg fp32 [B,T,H,K]
+ *   (gradient w.r.t. the raw gates); dh0 fp32 [N,H,K,V] or NULL.
+ * ---------------------------------------------------------------------- */
+int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
+                      const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
+                      void* dq, void* dk, void* dv, float* dg, float* dh0,
+                      const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                      int qkv_dtype, int gate_dtype,
+                      int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                      float scale, fla_stream_t stream);
 
 /* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
  * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,

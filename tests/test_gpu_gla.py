@@ -114,3 +114,71 @@ def test_chunk_gla_segment_chaining(device):
     o2, h2 = _run(device, q[:, cut:], k[:, cut:], v[:, cut:], g[:, cut:], h1.cpu())
     assert_close("o chained", o_full.float(), torch.cat([o1, o2], 1).float(), 4e-3)
     assert_close("ht chained", ht_full, h2, 1e-5)
+
+
+# ---------------------------------------------------------------- backward
+def _grads_ref(q, k, v, g, h0, do, dht, offsets=None, scale=None):
+    """Autograd through the fp32 naive recurrence (tests/ops/test_gla.py:59-64)."""
+    from oracle.recurrent import naive_recurrent_gla
+    leaves = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    h0l = None if h0 is None else h0.detach().float().requires_grad_()
+    o, ht = naive_recurrent_gla(*leaves, scale=scale, initial_state=h0l, output_final_state=True, offsets=offsets)
+    loss = (o * do.float()).sum() + (ht * dht.float()).sum()
+    loss.backward()
+    return [x.grad for x in leaves] + [None if h0l is None else h0l.grad]
+
+
+def _grads_dev(device, q, k, v, g, h0, do, dht, offsets=None, scale=None, head_first=False):
+    from fla_amd.ops.gla import chunk_gla
+    dev = lambda x: None if x is None else x.to(device)
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    leaves = [tr(dev(x)).detach().requires_grad_() for x in (q, k, v, g)]
+    h0l = None if h0 is None else dev(h0).detach().requires_grad_()
+    o, ht = chunk_gla(*leaves, scale=scale, initial_state=h0l, output_final_state=True, offsets=dev(offsets),
+                      head_first=head_first)
+    loss = (o.float() * tr(dev(do)).float()).sum() + (ht * dev(dht)).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    return [tr(x.grad) for x in leaves] + [None if h0l is None else h0l.grad]
+
+
+@pytest.mark.parametrize("T", [64, 130, 300])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
+def test_chunk_gla_backward(device, T, K, V):
+    """Gradients against autograd through the naive recurrence
+    (reference tolerances: tests/ops/test_gla.py:90-146 uses 0.005 on bf16 grads)."""
+    B, H = 2, 2
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=31 + T, normalizer=16.0, h0_std=1.0)
+    gen = torch.Generator().manual_seed(5)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    print(f"chunk_gla backward T={T} K={K} V={V}", flush=True)
+    got = _grads_dev(device, q, k, v, g, h0, do, dht)
+    ref = _grads_ref(q, k, v, g, h0, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(name, r, x, tol)
+    assert got[0].dtype == torch.bfloat16 and got[3].dtype == torch.float32
+
+
+def test_chunk_gla_backward_varlen_headfirst_odd(device):
+    gen = torch.Generator().manual_seed(6)
+    T, N, H, D = 500, 4, 2, 100
+    offs = random_offsets(T, N, gen, min_len=1)
+    q, k, v, g, h0 = gla_inputs(1, T, H, D, D, seed=41, N=N, normalizer=4.0, h0_std=1.0)
+    do = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(N, H, D, D, generator=gen) * 0.1
+    print(f"chunk_gla backward varlen offs={offs.tolist()}", flush=True)
+    got = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    ref = _grads_ref(q, k, v, g, h0, do, dht, offsets=offs.tolist())
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(name, r, x, tol)
+    # head-first, bf16 gates, no initial state
+    q, k, v, g, _ = gla_inputs(2, 150, 2, 64, 64, seed=42, h0=False)
+    g = g.bfloat16()
+    do = torch.randn(2, 150, 2, 64, generator=gen).bfloat16()
+    dht = torch.randn(2, 2, 64, 64, generator=gen) * 0.1
+    got = _grads_dev(device, q, k, v, g, None, do, dht, head_first=True)
+    ref = _grads_ref(q, k, v, g, None, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg"), ref, got, (8e-3, 8e-3, 8e-3, 2e-2)):
+        assert_close(name, r, x, tol)
+    assert got[3].dtype == torch.bfloat16
