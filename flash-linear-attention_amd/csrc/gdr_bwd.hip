@@ -1,0 +1,1059 @@
+// Chunked gated delta rule backward for gfx950 (chunk size 64).
+//
+// Notation (per chunk and head): gamma = chunk-local prefix sum of g, Gamma_ij =
+// e^{gamma_i-gamma_j} (j<=i), kb = beta*k, vb = beta*v, M = strict_lower(kb k^T),
+// Aw = (I+M)^-1, Au = Aw*Gamma, w = Aw kb, u = Au vb, v_new = u - (w e^gamma) h_c,
+// dH_c = gradient w.r.t. the state LEAVING chunk c.  Follows
+// fla/ops/gated_delta_rule/chunk.py:76-177:
+//
+//   gdr_bwd_dvlocal_kernel   dv_loc = (s tril(q k^T * Gamma))^T do               (chunk_o.py:379-441)
+//   gdr_bwd_dhu_kernel       reverse scan per (sequence, head, 32 value columns):
+//                              store dH_c;  dv2 = dv_loc + (k e^{gamma_last-gamma}) dH_c;
+//                              dH <- e^{gamma_last} dH + (s q e^gamma)^T do - (w e^gamma)^T dv2
+//                                                                                (chunk_delta_h.py:136-237)
+//   gdr_bwd_dqkwg_kernel     per (chunk, head, 64-wide half of K):
+//                              ds = s tril((do v_new^T) * Gamma)
+//                              dq = s e^gamma (do h_c^T) + ds k
+//                              dk = e^{gamma_last-gamma} (v_new dH_c^T) + ds^T q
+//                              dw = -e^gamma (dv2 h_c^T)
+//                              dgamma_i = sum_k (q*dq - k*dk + w*dw)_ik
+//                                         + [i last] (sum_jk k*dk_inter + e^{gamma_last} <h_c, dH_c>)
+//                            (chunk_o.py:118-265; the row/column sums of ds*(q k^T) there equal
+//                            sum_k q*dq_intra - k*dk_intra, so no second score matrix is formed)
+//   gdr_bwd_wy_kernel        gradient through the WY representation:
+//                              d(kb) = Aw^T dw, d(vb) = Au^T du,
+//                              dAw = strict_lower(dw kb^T) + strict_lower(du vb^T) * Gamma,
+//                              dM = -strict_lower(Aw^T dAw Aw^T),
+//                              d(kb) += dM k, dk = beta d(kb) + dM^T kb, dv = beta d(vb),
+//                              dbeta = sum d(kb)*k + sum d(vb)*v,
+//                              dgamma_i += rowsum_i(X) - colsum_i(X), X = strict_lower(du vb^T) * Au
+//                            (wy_fast.py:440-562, written for the single inverse Aw).
+#include "chunk_common.h"
+
+namespace {
+
+// ---------------------------------------------------------------------------
+struct DvlParams {
+  const void* q;
+  const void* k;
+  const void* dout;
+  const float* gam;
+  void* dvl;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+template <typename T, int K, int V>
+__global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int C8 = K / 8, NP = BT * C8 / 256;
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int TV = V / 64;
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sDt[V * LDT];
+  __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];
+  __shared__ float sGam[BT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, hh = blockIdx.y;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    v8 qv, kv;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c8;
+      qv = *(const v8*)((const T*)p.q + off);
+      kv = *(const v8*)((const T*)p.k + off);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) qv[j] = kv[j] = (T)0.f;
+    }
+    *(v8*)&sQ[row * LDK + c8] = qv;
+    *(v8*)&sK[row * LDK + c8] = kv;
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+  v4 dreg[RPTV];
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) {
+    int row = rgv * RPTV + i;
+    if (row < L) dreg[i] = *(const v4*)((const T*)p.dout + ((row0 + row) * H + hh) * (int64_t)V + cv4);
+    else dreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    T* dst = &sDt[(cv4 + j) * LDT + rgv * RPTV];
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) dst[i] = dreg[i][j];
+  }
+  if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
+  __syncthreads();
+  {
+    const int qi = wave >> 1, qj = wave & 1;
+    if (qj <= qi) {
+      f32x16 s = zero16();
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 16)
+        s = Elem<T>::mfma32(lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
+      const int j = qj * 32 + (lane & 31);
+      const float gj = sGam[j];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        int i0 = qi * 32 + 8 * a + 4 * (lane >> 5);
+        v4 x;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          x[b] = (T)((j <= i0 + b) ? s[4 * a + b] * p.scale * __expf(sGam[i0 + b] - gj) : 0.f);
+        *(v4*)&sPT[j * LDT + i0] = x;
+      }
+    }
+  }
+  __syncthreads();
+  const int rw = wave >> 1, cw = wave & 1;
+  f32x16 acc[TV];
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+  for (int is = rw * 32; is < BT; is += 16) {
+    v8 a = lds_frag32<T>(sPT, LDT, rw * 32, is, lane);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), acc[tv]);
+  }
+  T* op = (T*)p.dvl + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = rw * 32 + c32_row(r, lane);
+      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    }
+}
+
+// ---------------------------------------------------------------------------
+struct DhuParams {
+  const void* q;
+  const void* k;
+  const void* w;
+  const void* dout;
+  const void* dvl;
+  const float* gam;
+  const float* dht;
+  void* dv2;
+  void* dhtf;   // dH, FLA_H_FRAGMENT_T
+  float* dh0;
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int H, V, N;
+  float scale;
+};
+
+// One workgroup: all K rows x 32 value columns.  Two barriers per chunk:
+//   phase A: dv2 from (k^, dH^T, dv_loc^T); stage (q~^T, -w~^T, do^T) of the same chunk
+//   phase B: update dH; stage (k^, dv_loc^T) and publish dH for the next (earlier) chunk
+// X = (q, w, do, gamma) and Y = (k, dv_loc, gamma) are prefetched one full iteration ahead.
+template <typename T, int K>
+__global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  constexpr int BV = 32;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int KT32 = K / 32;
+  constexpr int NKT = (KT32 + 3) / 4;
+  __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];    // k e^{gamma_last-gamma}, row-major
+  __shared__ __attribute__((aligned(16))) T sQt[K * LDT];     // (s q e^gamma)^T
+  __shared__ __attribute__((aligned(16))) T sWt[K * LDT];     // -(w e^gamma)^T
+  __shared__ __attribute__((aligned(16))) T sDoT[BV * LDT];   // do^T
+  __shared__ __attribute__((aligned(16))) T sDvl[BV * LDT];   // dv_loc^T
+  __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];   // dH^T in 16-bit
+  __shared__ __attribute__((aligned(16))) T sDv2T[BV * LDT];  // dv2^T
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, V = p.V;
+  const int nvt = V / BV;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vt = (int)(id % nvt);
+  const int nh = (int)(id / nvt);
+  const int n = nh / H, hh = nh % H;
+  const int vbase = vt * BV;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+
+  f32x16 acc[NKT], acct[NKT];
+#pragma unroll
+  for (int a = 0; a < NKT; ++a) {
+    acc[a] = zero16();
+    acct[a] = zero16();
+    int kt = wave + 4 * a;
+    if (p.dht && kt < KT32) {
+      const float* d0 = p.dht + (int64_t)nh * K * V;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[a][r] = d0[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
+        acct[a][r] = d0[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + c32_row(r, lane)];
+      }
+    }
+  }
+
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  const int urg = tid >> 4, uc2 = (tid & 15) * 2;
+  struct XRegs {
+    v4 q[RPT];
+    v4 w[RPT];
+    float gam[RPT];
+    t2 d[4];
+  };
+  struct YRegs {
+    v4 k[RPT];
+    float gam[RPT];
+    t2 dvl[4];
+    float glast;
+  };
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+  auto load_x = [&](int64_t c, XRegs& R) {
+    bool live = c >= 0;
+    int L = chunk_len(c);
+    int64_t rbase = sp.bos + c * BT;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      if (live && row < L) {
+        int64_t off = ((rbase + row) * H + hh) * (int64_t)K + c4;
+        R.q[i] = *(const v4*)((const T*)p.q + off);
+        R.w[i] = *(const v4*)((const T*)p.w + off);
+        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
+      } else {
+        R.q[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.w[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.gam[i] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int row = urg * 4 + i;
+      if (live && row < L)
+        R.d[i] = *(const t2*)((const T*)p.dout + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
+      else R.d[i] = t2{(T)0.f, (T)0.f};
+    }
+  };
+  auto load_y = [&](int64_t c, YRegs& R) {
+    bool live = c >= 0;
+    int L = chunk_len(c);
+    int64_t rbase = sp.bos + c * BT;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      if (live && row < L) {
+        R.k[i] = *(const v4*)((const T*)p.k + ((rbase + row) * H + hh) * (int64_t)K + c4);
+        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
+      } else {
+        R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.gam[i] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int row = urg * 4 + i;
+      if (live && row < L)
+        R.dvl[i] = *(const t2*)((const T*)p.dvl + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
+      else R.dvl[i] = t2{(T)0.f, (T)0.f};
+    }
+    R.glast = (live && p.gam) ? p.gam[(rbase + L - 1) * H + hh] : 0.f;
+  };
+  auto stage_x = [&](const XRegs& R) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      T* dq = &sQt[(c4 + j) * LDT + rg * RPT];
+      T* dw = &sWt[(c4 + j) * LDT + rg * RPT];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        float eg = __expf(R.gam[i]);
+        dq[i] = (T)((float)R.q[i][j] * p.scale * eg);
+        dw[i] = (T)(-(float)R.w[i][j] * eg);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      v4 dv = v4{R.d[0][j], R.d[1][j], R.d[2][j], R.d[3][j]};
+      *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
+    }
+  };
+  auto stage_y = [&](const YRegs& R, int L) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      float e = (row < L) ? __expf(R.glast - R.gam[i]) : 0.f;
+      v4 kv;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) kv[j] = (T)((float)R.k[i][j] * e);
+      *(v4*)&sKh[row * LDK + c4] = kv;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      v4 dv = v4{R.dvl[0][j], R.dvl[1][j], R.dvl[2][j], R.dvl[3][j]};
+      *(v4*)&sDvl[(uc2 + j) * LDT + urg * 4] = dv;
+    }
+  };
+  // gradient w.r.t. the state leaving chunk c: 16-bit transpose in LDS, FRAGMENT_T copy in HBM
+  auto publish = [&](int64_t c) {
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          v4 x;
+#pragma unroll
+          for (int b = 0; b < 4; ++b) x[b] = (T)acc[a][4 * q4 + b];
+          *(v4*)&sDHt[(lane & 31) * LDK + kt * 32 + 8 * q4 + 4 * (lane >> 5)] = x;
+        }
+        v8 lo, hi;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          lo[r] = (T)acct[a][r];
+          hi[r] = (T)acct[a][r + 8];
+        }
+        T* hp = (T*)p.dhtf + ((chunk0 + c) * H + hh) * (int64_t)K * V + (((int64_t)vt * (K / 32) + kt) * 64 + lane) * 16;
+        *(v8*)hp = lo;
+        *(v8*)(hp + 8) = hi;
+      }
+    }
+  };
+
+  XRegs X;
+  YRegs Y;
+  load_x(nchunks - 1, X);
+  load_y(nchunks - 1, Y);
+  float dec = 1.f;
+  if (nchunks > 0) {
+    stage_y(Y, chunk_len(nchunks - 1));
+    dec = __expf(Y.glast);
+    publish(nchunks - 1);
+  }
+  load_y(nchunks - 2, Y);
+  for (int64_t c = nchunks - 1; c >= 0; --c) {
+    const int L = chunk_len(c);
+    const int64_t rbase = sp.bos + c * BT;
+    __syncthreads();  // (1)
+    // ---- dv2 = dv_loc + k^ dH : wave w owns rows 16w..16w+15, two 16-column tiles
+    {
+      f32x4 d[2] = {zero4(), zero4()};
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 32) {
+        v8 a = lds_frag16<T>(sKh, LDK, wave * 16, ks, lane);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, lds_frag16<T>(sDHt, LDK, j * 16, ks, lane), d[j]);
+      }
+      const int tr = wave * 16 + 4 * (lane >> 4);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        int vc = j * 16 + (lane & 15);
+        v4 dl = *(const v4*)&sDvl[vc * LDT + tr];
+        v4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = (T)((float)dl[r] + d[j][r]);
+        *(v4*)&sDv2T[vc * LDT + tr] = o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (tr + r < L) ((T*)p.dv2)[((rbase + tr + r) * H + hh) * (int64_t)V + vbase + vc] = o[r];
+      }
+    }
+    stage_x(X);
+    const float dec_c = dec;
+    load_x(c - 1, X);
+    __syncthreads();  // (2)
+    // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          acc[a][r] *= dec_c;
+          acct[a][r] *= dec_c;
+        }
+#pragma unroll
+        for (int s = 0; s < BT; s += 16) {
+          v8 fq = lds_frag32<T>(sQt, LDT, kt * 32, s, lane);
+          v8 fd = lds_frag32<T>(sDoT, LDT, 0, s, lane);
+          v8 fw = lds_frag32<T>(sWt, LDT, kt * 32, s, lane);
+          v8 f2 = lds_frag32<T>(sDv2T, LDT, 0, s, lane);
+          acc[a] = Elem<T>::mfma32(fq, fd, acc[a]);
+          acc[a] = Elem<T>::mfma32(fw, f2, acc[a]);
+          acct[a] = Elem<T>::mfma32(fd, fq, acct[a]);
+          acct[a] = Elem<T>::mfma32(f2, fw, acct[a]);
+        }
+      }
+    }
+    if (c > 0) {
+      stage_y(Y, chunk_len(c - 1));
+      dec = __expf(Y.glast);
+      publish(c - 1);
+      load_y(c - 2, Y);
+    }
+  }
+  if (p.dh0) {
+    float* o = p.dh0 + (int64_t)nh * K * V;
+#pragma unroll
+    for (int a = 0; a < NKT; ++a) {
+      int kt = wave + 4 * a;
+      if (kt < KT32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[a][r];
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct DqkwgParams {
+  const void* q;
+  const void* k;
+  const void* vnew;
+  const void* w;
+  const void* dout;
+  const void* dv2;
+  const float* gam;
+  const void* hT;     // forward states, FLA_H_FRAGMENT_T
+  const void* dhtf;   // dH, FLA_H_FRAGMENT_T
+  void* dq;
+  void* dk;           // partial: everything except the WY path
+  void* dw;
+  float* dgam;        // [K/64][B*T][H] partial per key slice
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int64_t total_rows;
+  int H, K, NTfix;
+  float scale;
+};
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDV = V + 8;
+  constexpr int C8 = V / 8, NP = BT * C8 / 256;
+  constexpr int VT32 = V / 32;
+  constexpr int ROWB = BT * LDV * 2;
+  constexpr int STG = BT * LDM * 4;
+  constexpr int REG_A = ROWB > STG ? ROWB : STG;
+  constexpr int REG_C = (2 * BT * LDT * 2 > STG) ? 2 * BT * LDT * 2 : STG;
+  __shared__ __attribute__((aligned(16))) char sRA[REG_A];  // do row-major -> dv2 row-major -> staging (dq)
+  __shared__ __attribute__((aligned(16))) char sRB[REG_A];  // v_new row-major -> staging (dk intra)
+  __shared__ __attribute__((aligned(16))) char sRC[REG_C];  // k^T | q^T -> staging (dk inter)
+  __shared__ __attribute__((aligned(16))) char sRD[REG_C];  // ds | ds^T -> staging (dw)
+  __shared__ float sGam[BT];
+  T* sDo = (T*)sRA;
+  T* sVn = (T*)sRB;
+  T* sKT = (T*)sRC;
+  T* sQT = sKT + BT * LDT;
+  T* sDs = (T*)sRD;
+  T* sDsT = sDs + BT * LDT;
+  float* stA = (float*)sRA;
+  float* stB = (float*)sRB;
+  float* stC = (float*)sRC;
+  float* stD = (float*)sRD;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, hh = blockIdx.y;
+  const int kb = blockIdx.z * 64;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+
+  // ---- loads
+  const int rg = tid >> 4, c4 = (tid & 15) * 4;
+  float qq[4][4], kk[4][4], ww[4][4], gam4[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = rg * 4 + i;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
+      Load<T>::x4((const T*)p.q + off, qq[i]);
+      Load<T>::x4((const T*)p.k + off, kk[i]);
+      Load<T>::x4((const T*)p.w + off, ww[i]);
+      gam4[i] = p.gam ? p.gam[(row0 + row) * H + hh] : 0.f;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qq[i][j] = kk[i][j] = ww[i][j] = 0.f;
+      gam4[i] = 0.f;
+    }
+  }
+  const float glast = p.gam ? p.gam[(row0 + L - 1) * H + hh] : 0.f;
+  v8 dreg[NP], vreg[NP], d2reg[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)V + c8;
+      dreg[i] = *(const v8*)((const T*)p.dout + off);
+      vreg[i] = *(const v8*)((const T*)p.vnew + off);
+      d2reg[i] = *(const v8*)((const T*)p.dv2 + off);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dreg[i][j] = vreg[i][j] = d2reg[i][j] = (T)0.f;
+    }
+  }
+  const int rw = wave >> 1, cw = wave & 1;
+  const int kt32 = kb / 32 + cw;
+  v8 hf[VT32][2], dhf[VT32][2];
+  {
+    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int vt = 0; vt < VT32; ++vt) {
+      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
+      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
+      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
+      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
+      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
+    }
+  }
+  if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sDo[row * LDV + c8] = dreg[i];
+    *(v8*)&sVn[row * LDV + c8] = vreg[i];
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v4 kt, qt;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kt[i] = (T)kk[i][j];
+      qt[i] = (T)qq[i][j];
+    }
+    *(v4*)&sKT[(c4 + j) * LDT + rg * 4] = kt;
+    *(v4*)&sQT[(c4 + j) * LDT + rg * 4] = qt;
+  }
+  // <h_c, dH_c> over this wave's tiles (same fragment order on both sides)
+  float hd = 0.f;
+#pragma unroll
+  for (int vt = 0; vt < VT32; ++vt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) hd += (float)hf[vt][half][e] * (float)dhf[vt][half][e];
+  __syncthreads();
+  // ---- ds = s tril((do v_new^T) * Gamma), both orientations
+  {
+    const int ib = wave >> 1, jb = wave & 1;
+    if (jb <= ib) {
+      f32x16 s1 = zero16(), s2 = zero16();
+#pragma unroll
+      for (int vs = 0; vs < V; vs += 16) {
+        v8 fd = lds_frag32<T>(sDo, LDV, ib * 32, vs, lane);
+        v8 fv = lds_frag32<T>(sVn, LDV, jb * 32, vs, lane);
+        s1 = Elem<T>::mfma32(fd, fv, s1);  // rows i, cols j
+        s2 = Elem<T>::mfma32(fv, fd, s2);  // rows j, cols i
+      }
+      const int c = lane & 31;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        int r0 = 8 * a + 4 * (lane >> 5);
+        v4 x1, x2;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          int i1 = ib * 32 + r0 + b, j1 = jb * 32 + c;
+          x1[b] = (T)((j1 <= i1) ? s1[4 * a + b] * p.scale * __expf(sGam[i1] - sGam[j1]) : 0.f);
+          int j2 = jb * 32 + r0 + b, i2 = ib * 32 + c;
+          x2[b] = (T)((j2 <= i2) ? s2[4 * a + b] * p.scale * __expf(sGam[i2] - sGam[j2]) : 0.f);
+        }
+        *(v4*)&sDsT[(jb * 32 + c) * LDT + ib * 32 + r0] = x1;
+        *(v4*)&sDs[(ib * 32 + c) * LDT + jb * 32 + r0] = x2;
+      }
+    }
+  }
+  __syncthreads();
+  // ---- dq = s e^gamma (do h^T) + ds k ; dk_intra = ds^T q ; dk_inter = v_new dH^T
+  f32x16 aq = zero16(), ak1 = zero16(), ak2 = zero16(), aw = zero16();
+#pragma unroll
+  for (int vt = 0; vt < VT32; ++vt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      aq = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aq);
+      ak2 = Elem<T>::mfma32(lds_frag32_perm<T>(sVn, LDV, rw * 32, vt * 32 + half * 16, lane), dhf[vt][half], ak2);
+    }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float g = sGam[rw * 32 + c32_row(r, lane)];
+    aq[r] *= p.scale * __expf(g);
+    ak2[r] *= __expf(glast - g);
+  }
+  const int jend = (rw + 1) * 32;
+  for (int js = 0; js < jend; js += 16)
+    aq = Elem<T>::mfma32(lds_frag32<T>(sDs, LDT, rw * 32, js, lane), lds_frag32<T>(sKT, LDT, cw * 32, js, lane), aq);
+  for (int is = rw * 32; is < BT; is += 16)
+    ak1 = Elem<T>::mfma32(lds_frag32<T>(sDsT, LDT, rw * 32, is, lane), lds_frag32<T>(sQT, LDT, cw * 32, is, lane), ak1);
+  __syncthreads();  // do is consumed: its tile takes dv2
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sDo[row * LDV + c8] = d2reg[i];
+  }
+  __syncthreads();
+  // ---- dw = -e^gamma (dv2 h^T)
+#pragma unroll
+  for (int vt = 0; vt < VT32; ++vt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      aw = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aw);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) aw[r] *= -__expf(sGam[rw * 32 + c32_row(r, lane)]);
+  __syncthreads();  // all operand reads done: tiles become fp32 staging
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    int o = (rw * 32 + c32_row(r, lane)) * LDM + cw * 32 + (lane & 31);
+    stA[o] = aq[r];
+    stB[o] = ak1[r];
+    stC[o] = ak2[r];
+    stD[o] = aw[r];
+  }
+  // <h, dH> of the whole key slice: reduce over the 4 waves through LDS
+  __shared__ float sHd[4];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) hd += __shfl_xor(hd, off, 64);
+  if (lane == 0) sHd[wave] = hd;
+  __syncthreads();
+  // waves (rw=0,cw) and (rw=1,cw) loaded the same fragments: count each key tile once
+  const float hd_all = sHd[0] + sHd[1];
+  // ---- epilogue in the load mapping (4 rows x 4 key channels per lane)
+  float rowsum[4], kin = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = rg * 4 + i;
+    f32x4 a = *(const f32x4*)&stA[row * LDM + c4];
+    f32x4 b = *(const f32x4*)&stB[row * LDM + c4];
+    f32x4 c = *(const f32x4*)&stC[row * LDM + c4];
+    f32x4 d = *(const f32x4*)&stD[row * LDM + c4];
+    v4 dqv, dkv, dwv;
+    float rs = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float dk = b[j] + c[j];
+      dqv[j] = (T)a[j];
+      dkv[j] = (T)dk;
+      dwv[j] = (T)d[j];
+      rs += qq[i][j] * a[j] - kk[i][j] * dk + ww[i][j] * d[j];
+      kin += kk[i][j] * c[j];
+    }
+    rowsum[i] = rs;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
+      *(v4*)((T*)p.dq + off) = dqv;
+      *(v4*)((T*)p.dk + off) = dkv;
+      *(v4*)((T*)p.dw + off) = dwv;
+    }
+  }
+  // row sums over the 16 lanes that share a row group; total of k*dk_inter over the workgroup
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rowsum[i] += __shfl_xor(rowsum[i], off, 64);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) kin += __shfl_xor(kin, off, 64);
+  __shared__ float sKin[4];
+  if (lane == 0) sKin[wave] = kin;
+  __syncthreads();
+  const float kin_all = sKin[0] + sKin[1] + sKin[2] + sKin[3];
+  if ((tid & 15) == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int row = rg * 4 + i;
+      if (row < L) {
+        float val = rowsum[i];
+        if (row == L - 1) val += kin_all + __expf(glast) * hd_all;
+        p.dgam[((int64_t)blockIdx.z * p.total_rows + row0 + row) * H + hh] = val;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+struct WyBwdParams {
+  const void* k;
+  const void* v;
+  const float* beta;
+  const float* gam;
+  const void* Aw;
+  const void* dw;
+  const void* du;
+  const void* dk_in;   // partial dk from the dq/dk/dw kernel, added before the single rounding
+  void* dk;
+  void* dv;
+  float* dbeta;
+  float* dgam2;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+};
+
+// 64 x N product helper: C[64 x 32*NTILE per wave] with A from a [64][lda] tile (rows = output
+// rows, contraction contiguous) and B from a [cols][ldb] tile (contraction contiguous).
+template <typename T, int NT_>
+FLA_DEVICE void mm64(const T* A, int lda, const T* Bt, int ldb, int rw, int col0, int c_begin, int c_end, int lane,
+                     f32x16* acc) {
+  typedef typename Elem<T>::v8 v8;
+  for (int cs = c_begin; cs < c_end; cs += 16) {
+    v8 a = lds_frag32<T>(A, lda, rw * 32, cs, lane);
+#pragma unroll
+    for (int t = 0; t < NT_; ++t) acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(Bt, ldb, col0 + t * 32, cs, lane), acc[t]);
+  }
+}
+
+template <typename T, int K, int V>
+__global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int D = K > V ? K : V;
+  constexpr int LDD = D + 8;
+  constexpr int TK = K / 64, TV = V / 64;
+  __shared__ __attribute__((aligned(16))) T sRow1[BT * LDD];   // dw | du            row-major [t][d]
+  __shared__ __attribute__((aligned(16))) T sRow2[BT * LDD];   // kb | vb | k         row-major
+  __shared__ __attribute__((aligned(16))) T sTr1[D * LDT];     // dw^T | du^T | k^T   [d][t]
+  __shared__ __attribute__((aligned(16))) T sTr2[D * LDT];     // kb^T
+  __shared__ __attribute__((aligned(16))) T sAw[BT * LDT];     // Aw [i][j]
+  __shared__ __attribute__((aligned(16))) T sAwT[BT * LDT];    // Aw^T
+  __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA (masked) -> dM
+  __shared__ __attribute__((aligned(16))) T sS2[BT * LDT];     // X1^T -> dM^T
+  __shared__ float sBeta[BT], sGam[BT], sDb[BT], sDg[BT];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, hh = blockIdx.y;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+  const int rw = wave >> 1, cw = wave & 1;
+
+  if (tid < BT) {
+    bool ok = tid < L;
+    sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
+    sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
+    sDb[tid] = 0.f;
+    sDg[tid] = 0.f;
+  }
+  // Aw and Aw^T (rows beyond L: identity)
+  {
+    const int i = tid >> 2, j0 = (tid & 3) * 16;
+    v8 a0, a1;
+    if (i < L) {
+      const T* ap = (const T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + j0;
+      a0 = *(const v8*)ap;
+      a1 = *(const v8*)(ap + 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        a0[e] = (T)((j0 + e == i) ? 1.f : 0.f);
+        a1[e] = (T)((j0 + 8 + e == i) ? 1.f : 0.f);
+      }
+    }
+    *(v8*)&sAw[i * LDT + j0] = a0;
+    *(v8*)&sAw[i * LDT + j0 + 8] = a1;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sAwT[(j0 + e) * LDT + i] = a0[e];
+      sAwT[(j0 + 8 + e) * LDT + i] = a1[e];
+    }
+  }
+  __syncthreads();
+
+  // generic tile loaders: row-major [64][DIM] (optionally scaled per row) and its transpose
+  auto load_rows = [&](const void* src, int DIM, bool scale_beta, T* dst_row, T* dst_tr) {
+    const int c8n = DIM / 8;
+    for (int e = tid; e < BT * c8n; e += 256) {
+      int row = e / c8n, c8 = (e % c8n) * 8;
+      v8 x;
+      if (row < L) x = *(const v8*)((const T*)src + ((row0 + row) * H + hh) * (int64_t)DIM + c8);
+      else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = (T)0.f;
+      }
+      if (scale_beta) {
+        float b = sBeta[row];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = (T)((float)x[j] * b);
+      }
+      if (dst_row) *(v8*)&dst_row[row * LDD + c8] = x;
+      if (dst_tr) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dst_tr[(c8 + j) * LDT + row] = x[j];
+      }
+    }
+  };
+
+  // ================= key side: d(kb)_1 = Aw^T dw ; dAw_1 = dw kb^T
+  load_rows(p.dw, K, false, sRow1, sTr1);
+  load_rows(p.k, K, true, sRow2, sTr2);   // kb, kb^T
+  __syncthreads();
+  f32x16 dkb[TK];   // d(kb), rows j = 32rw.., cols (cw*TK+t)*32..
+#pragma unroll
+  for (int t = 0; t < TK; ++t) dkb[t] = zero16();
+  // Aw^T is upper triangular: row j contracts over i >= j
+  mm64<T, TK>(sAwT, LDT, sTr1, LDT, rw, cw * TK * 32, rw * 32, BT, lane, dkb);
+  // dA quadrants (lower triangular incl. diagonal block): waves 0,2,3 -> (ib,jb) = (0,0),(1,0),(1,1)
+  const int ib = wave >> 1, jb = wave & 1;
+  f32x16 dA = zero16();
+  if (jb <= ib) {
+    for (int ks = 0; ks < K; ks += 16)
+      dA = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, ks, lane), lds_frag32<T>(sRow2, LDD, jb * 32, ks, lane), dA);
+  }
+  __syncthreads();
+  // ================= value side: d(vb) = Au^T du ; dAu = du vb^T
+  load_rows(p.du, V, false, sRow1, sTr1);
+  load_rows(p.v, V, true, sRow2, nullptr);   // vb
+  {
+    // Au^T[j][i] = Aw^T[j][i] * e^{gamma_i - gamma_j}, i >= j
+    const int j = tid >> 2, i0 = (tid & 3) * 16;
+    const float gj = sGam[j];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      int i = i0 + e;
+      float a = (float)sAwT[j * LDT + i];
+      sS1[j * LDT + i] = (T)((i >= j) ? a * __expf(sGam[i] - gj) : 0.f);
+    }
+  }
+  __syncthreads();
+  f32x16 dvb[TV];
+#pragma unroll
+  for (int t = 0; t < TV; ++t) dvb[t] = zero16();
+  mm64<T, TV>(sS1, LDT, sTr1, LDT, rw, cw * TV * 32, rw * 32, BT, lane, dvb);
+  f32x16 dAu = zero16();
+  if (jb <= ib) {
+    for (int vs = 0; vs < V; vs += 16)
+      dAu = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, vs, lane), lds_frag32<T>(sRow2, LDD, jb * 32, vs, lane),
+                            dAu);
+  }
+  // dv = beta d(vb);  dbeta += sum_v d(vb) * v   (v = vb / beta is re-read from HBM)
+  {
+    T* dvp = (T*)p.dv + (row0 * H + hh) * (int64_t)V;
+    const T* vp = (const T*)p.v + (row0 * H + hh) * (int64_t)V;
+    float part[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[r] = 0.f;
+#pragma unroll
+    for (int t = 0; t < TV; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int j = rw * 32 + c32_row(r, lane);
+        int col = (cw * TV + t) * 32 + (lane & 31);
+        if (j < L) {
+          dvp[(int64_t)j * H * V + col] = (T)(dvb[t][r] * sBeta[j]);
+          part[r] += dvb[t][r] * (float)vp[(int64_t)j * H * V + col];
+        }
+      }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float s = part[r];
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+      if ((lane & 31) == 0) atomicAdd(&sDb[rw * 32 + c32_row(r, lane)], s);
+    }
+  }
+  __syncthreads();  // Au^T and the value tiles are consumed
+  // ================= dA_total (strictly lower) and the gate gradient through Gamma
+  if (jb <= ib) {
+    const int j = jb * 32 + (lane & 31);
+    const float gj = sGam[j];
+    float colsum = 0.f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      int i0 = ib * 32 + 8 * a + 4 * (lane >> 5);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        int i = i0 + b, r = 4 * a + b;
+        bool low = j < i;
+        float gamma = low ? __expf(sGam[i] - gj) : 0.f;
+        float au = (float)sAw[i * LDT + j] * gamma;         // Au_ij
+        float x = low ? dAu[r] * au : 0.f;                  // dAu * Au
+        float tot = low ? dA[r] + dAu[r] * gamma : 0.f;     // dAw total
+        sS1[i * LDT + j] = (T)tot;                          // dA (masked) [i][j]
+        // row sums: reduce over the 32 lanes holding the same row
+        float rs = x;
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) rs += __shfl_xor(rs, off, 64);
+        if ((lane & 31) == 0) atomicAdd(&sDg[i], rs);
+        colsum += x;
+      }
+    }
+    colsum += __shfl_xor(colsum, 32, 64);
+    if (lane < 32) atomicAdd(&sDg[j], -colsum);
+  } else {
+    // quadrant (0,1) lies strictly above the diagonal
+    for (int e = lane; e < 32 * 32; e += 64) sS1[(e >> 5) * LDT + 32 + (e & 31)] = (T)0.f;
+  }
+  __syncthreads();
+  // ================= X1 = dA Aw^T  (stored transposed), dM = -strict_lower(Aw^T X1)
+  {
+    // wave (rw, cw): rows a = 32rw.., cols j = 32cw..  ; contraction over b
+    f32x16 x1 = zero16();
+    for (int bs = 0; bs < BT; bs += 16)
+      x1 = Elem<T>::mfma32(lds_frag32<T>(sS1, LDT, rw * 32, bs, lane), lds_frag32<T>(sAw, LDT, cw * 32, bs, lane), x1);
+    const int j = cw * 32 + (lane & 31);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      int a0 = rw * 32 + 8 * a + 4 * (lane >> 5);
+      v4 x;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) x[b] = (T)x1[4 * a + b];
+      *(v4*)&sS2[j * LDT + a0] = x;   // X1^T[j][a]
+    }
+  }
+  __syncthreads();
+  {
+    f32x16 m = zero16();
+    for (int as = 0; as < BT; as += 16)
+      m = Elem<T>::mfma32(lds_frag32<T>(sAwT, LDT, rw * 32, as, lane), lds_frag32<T>(sS2, LDT, cw * 32, as, lane), m);
+    __syncthreads();  // every wave has read dA (sS1) and X1^T (sS2)
+    const int j = cw * 32 + (lane & 31);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      int i0 = rw * 32 + 8 * a + 4 * (lane >> 5);
+      v4 x;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        float val = (j < i0 + b) ? -m[4 * a + b] : 0.f;
+        x[b] = (T)val;
+        sS1[(i0 + b) * LDT + j] = (T)val;     // dM[i][j]
+      }
+      *(v4*)&sS2[j * LDT + i0] = x;           // dM^T[j][i]
+    }
+  }
+  // ================= d(kb) += dM k ; dk = beta d(kb) + dM^T kb ; dbeta += sum_k d(kb) * k
+  load_rows(p.k, K, false, nullptr, sTr1);     // k^T (kb^T still in sTr2)
+  __syncthreads();
+  // dM is strictly lower: row i contracts over j < i ; dM^T row j contracts over i > j
+  mm64<T, TK>(sS1, LDT, sTr1, LDT, rw, cw * TK * 32, 0, (rw + 1) * 32, lane, dkb);
+  f32x16 dk2[TK];
+#pragma unroll
+  for (int t = 0; t < TK; ++t) dk2[t] = zero16();
+  mm64<T, TK>(sS2, LDT, sTr2, LDT, rw, cw * TK * 32, rw * 32, BT, lane, dk2);
+  {
+    T* dkp = (T*)p.dk + (row0 * H + hh) * (int64_t)K;
+    const T* kp = (const T*)p.k + (row0 * H + hh) * (int64_t)K;
+    const T* dip = p.dk_in ? (const T*)p.dk_in + (row0 * H + hh) * (int64_t)K : nullptr;
+    float part[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) part[r] = 0.f;
+#pragma unroll
+    for (int t = 0; t < TK; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int j = rw * 32 + c32_row(r, lane);
+        int col = (cw * TK + t) * 32 + (lane & 31);
+        if (j < L) {
+          int64_t o = (int64_t)j * H * K + col;
+          float val = dkb[t][r] * sBeta[j] + dk2[t][r] + (dip ? (float)dip[o] : 0.f);
+          dkp[o] = (T)val;
+          part[r] += dkb[t][r] * (float)kp[o];
+        }
+      }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float s = part[r];
+#pragma unroll
+      for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+      if ((lane & 31) == 0) atomicAdd(&sDb[rw * 32 + c32_row(r, lane)], s);
+    }
+  }
+  __syncthreads();
+  if (tid < L) {
+    p.dbeta[(row0 + tid) * H + hh] = sDb[tid];
+    p.dgam2[(row0 + tid) * H + hh] = sDg[tid];
+  }
+}
+
+template <typename T>
+int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, const void* vnew, const float* beta,
+                   const float* gam, const void* Aw, const void* dout, const float* dht, const void* hT, void* dvl,
+                   void* dv2, void* dhtf, void* dw, void* dkp, float* dgam_part, void* dq, void* dk, void* dv,
+                   float* dbeta, float* dgam2, float* dh0, const int64_t* offsets, const int64_t* indices,
+                   const int64_t* chunk_offsets, int64_t NT, int64_t B, int64_t T_, int64_t H, int64_t K, int64_t V,
+                   int64_t N, float scale, hipStream_t st) {
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+#define FLA_KV(STMT)                                   \
+  if (K == 64 && V == 64) { STMT(64, 64) }             \
+  else if (K == 128 && V == 128) { STMT(128, 128) }    \
+  else if (K == 64 && V == 128) { STMT(64, 128) }      \
+  else if (K == 128 && V == 64) { STMT(128, 64) }      \
+  else return FLA_E_UNSUPPORTED;
+  {
+    DvlParams p{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
+#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+    FLA_KV(L1)
+#undef L1
+    FLA_CHECK_LAUNCH();
+  }
+  {
+    DhuParams p{q, k, w, dout, dvl, gam, dht, dv2, dhtf, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N, scale};
+    int64_t total = (V / 32) * N * H;
+    FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+    if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(256), 0, st, p);
+    FLA_CHECK_LAUNCH();
+  }
+  {
+    DqkwgParams p{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
+                  B * T_, (int)H, (int)K, ntfix, scale};
+    dim3 g3(grid.x, grid.y, (unsigned)(K / 64));
+    if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p);
+    FLA_CHECK_LAUNCH();
+  }
+  {
+    WyBwdParams p{k, v, beta, gam, Aw, dw, dv2, dkp, dk, dv, dbeta, dgam2, offsets, indices, T_, (int)H, ntfix};
+#define L4(KK, VV) hipLaunchKernelGGL((gdr_bwd_wy_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+    FLA_KV(L4)
+#undef L4
+    FLA_CHECK_LAUNCH();
+  }
+#undef FLA_KV
+  return FLA_OK;
+}
+
+}  // namespace
+
+extern "C" int fla_chunk_gated_delta_rule_bwd(
+    const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,
+    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT,
+    void* ws_dv_local, void* ws_dv2, void* ws_dh_frag_t, void* ws_dw, void* ws_dk_partial, float* ws_dgam_partial,
+    void* dq, void* dk, void* dv, float* dbeta, float* dgam2, float* dh0,
+    const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
+    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && w && v_new && beta && Aw && dout && hT && ws_dv_local && ws_dv2 && ws_dh_frag_t &&
+                  ws_dw && ws_dk_partial && ws_dgam_partial && dq && dk && dv && dbeta && dgam2,
+              FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  hipStream_t st = (hipStream_t)stream;
+  if (qkv_dtype == FLA_BF16)
+    return launch_gdr_bwd<bf16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, ws_dv_local, ws_dv2,
+                                ws_dh_frag_t, ws_dw, ws_dk_partial, ws_dgam_partial, dq, dk, dv, dbeta, dgam2, dh0,
+                                offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st);
+  if (qkv_dtype == FLA_F16)
+    return launch_gdr_bwd<f16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, ws_dv_local, ws_dv2,
+                               ws_dh_frag_t, ws_dw, ws_dk_partial, ws_dgam_partial, dq, dk, dv, dbeta, dgam2, dh0,
+                               offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st);
+  return FLA_E_UNSUPPORTED;
+}

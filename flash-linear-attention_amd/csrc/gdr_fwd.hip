@@ -340,15 +340,23 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   const int64_t nchunks = (sp.len + BT - 1) / BT;
   const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
 
+  // HL == 3 additionally keeps every tile transposed (rows v, cols k): the global copy is
+  // then written in FLA_H_FRAGMENT_T order for the backward kernels, which contract over v.
+  constexpr bool TR = (HL == 3);
   f32x16 acc[NKT];
+  f32x16 acct[TR ? NKT : 1];
 #pragma unroll
   for (int a = 0; a < NKT; ++a) {
     acc[a] = zero16();
+    if (TR) acct[a] = zero16();
     int kt = wave + 4 * a;
     if (p.h0 && kt < KT32) {
       const float* h0p = p.h0 + (int64_t)nh * K * V;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
+      for (int r = 0; r < 16; ++r) {
+        acc[a][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
+        if (TR) acct[a][r] = h0p[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + c32_row(r, lane)];
+      }
     }
   }
 
@@ -444,6 +452,16 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
             T* hp = (T*)p.h + blk + (((int64_t)kt * (V / 32) + vt) * 64 + lane) * 16;
             *(v8*)hp = lo;
             *(v8*)(hp + 8) = hi;
+          } else if (HL == 3) {
+            T* hp = (T*)p.h + blk + (((int64_t)vt * (K / 32) + kt) * 64 + lane) * 16;
+            v8 tl, th;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+              tl[r] = (T)acct[a][r];
+              th[r] = (T)acct[a][r + 8];
+            }
+            *(v8*)hp = tl;
+            *(v8*)(hp + 8) = th;
           } else if (HL == 0) {
             T* hp = (T*)p.h + blk;
 #pragma unroll
@@ -513,10 +531,17 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
       if (kt < KT32) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a][r] *= dec;
+        if (TR) {
 #pragma unroll
-        for (int s = 0; s < BT; s += 16)
-          acc[a] = Elem<T>::mfma32(lds_frag32<T>(sKt, LDT, kt * 32, s, lane), lds_frag32<T>(sVnT, LDT, 0, s, lane),
-                                   acc[a]);
+          for (int r = 0; r < 16; ++r) acct[a][r] *= dec;
+        }
+#pragma unroll
+        for (int s = 0; s < BT; s += 16) {
+          v8 fk = lds_frag32<T>(sKt, LDT, kt * 32, s, lane);
+          v8 fv = lds_frag32<T>(sVnT, LDT, 0, s, lane);
+          acc[a] = Elem<T>::mfma32(fk, fv, acc[a]);
+          if (TR) acct[a] = Elem<T>::mfma32(fv, fk, acct[a]);
+        }
       }
     }
     if (c + 1 < nchunks) {
@@ -698,15 +723,15 @@ int launch_dh(const DHParams& p, int K, int h_dtype, int h_layout, hipStream_t s
   if (total == 0) return FLA_OK;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   dim3 grid((unsigned)total), block(256);
-  int hl = (h_layout == FLA_H_FRAGMENT) ? 1 : (h_dtype == FLA_F32 ? 2 : 0);
+  int hl = (h_layout == FLA_H_FRAGMENT) ? 1 : (h_layout == FLA_H_FRAGMENT_T) ? 3 : (h_dtype == FLA_F32 ? 2 : 0);
 #define FLA_CASE(KK, HL)                                                           \
   if (K == KK && hl == HL) {                                                       \
     hipLaunchKernelGGL((gdr_fwd_h_kernel<T, KK, HL>), grid, block, 0, st, p);      \
     FLA_CHECK_LAUNCH();                                                            \
     return FLA_OK;                                                                 \
   }
-  FLA_CASE(64, 0) FLA_CASE(64, 1) FLA_CASE(64, 2)
-  FLA_CASE(128, 0) FLA_CASE(128, 1) FLA_CASE(128, 2)
+  FLA_CASE(64, 0) FLA_CASE(64, 1) FLA_CASE(64, 2) FLA_CASE(64, 3)
+  FLA_CASE(128, 0) FLA_CASE(128, 1) FLA_CASE(128, 2) FLA_CASE(128, 3)
 #undef FLA_CASE
   return FLA_E_UNSUPPORTED;
 }
@@ -769,8 +794,9 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, co
   FLA_REQUIRE(V % 32 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(chunk_offsets != nullptr && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
-  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT, FLA_E_INVALID);
-  if (h_layout == FLA_H_FRAGMENT) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(h_layout == FLA_H_ROW_MAJOR || h_layout == FLA_H_FRAGMENT || h_layout == FLA_H_FRAGMENT_T,
+              FLA_E_INVALID);
+  if (h_layout != FLA_H_ROW_MAJOR) FLA_REQUIRE(h_dtype == qkv_dtype, FLA_E_UNSUPPORTED);
   else FLA_REQUIRE(h_dtype == qkv_dtype || h_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)h | (uintptr_t)v_new) % 16 == 0,
               FLA_E_ALIGNMENT);

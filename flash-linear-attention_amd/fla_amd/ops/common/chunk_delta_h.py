@@ -24,6 +24,7 @@ def chunk_gated_delta_rule_fwd_h(
     *,
     states_in_fp32: bool = False,
     fragment_layout: bool = False,
+    transposed_fragments: bool = False,
     chunk_offsets: Optional[torch.Tensor] = None,
     store_v_new: bool = True,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
@@ -56,6 +57,7 @@ def chunk_gated_delta_rule_fwd_h(
     be.check(be.lib().fla_chunk_gated_delta_rule_fwd_h(
         be.ptr(k), be.ptr(w), be.ptr(u), be.ptr(g), be.ptr(h0), be.ptr(h), be.ptr(v_new), be.ptr(ht),
         be.ptr(offsets), be.ptr(chunk_offsets), be.dt(k), be._DTYPES[h_dtype],
-        be.FLA_H_FRAGMENT if fragment_layout else be.FLA_H_ROW_MAJOR,
+        (be.FLA_H_FRAGMENT_T if transposed_fragments else be.FLA_H_FRAGMENT) if fragment_layout
+        else be.FLA_H_ROW_MAJOR,
         B, T, H, K, V, N, be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_h")
     return h, v_new, ht

@@ -49,6 +49,48 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     return g, o, Aw, Au, final_state
 
 
+def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do, dht, offsets=None):
+    """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims; ``g_cumsum``
+    the fp32 chunk-local cumsum saved by the forward).  Recomputes w, u, Aw, the per-chunk
+    states and v_new like the reference (``fla/ops/gated_delta_rule/chunk.py:95-116``).
+    Returns ``(dq, dk, dv, dbeta, dg, dh0)``."""
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    offs = None if plan is None else plan.offsets
+    idx = None if plan is None else plan.indices
+    co = None if plan is None else plan.chunk_offsets
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    N = B if plan is None else plan.N
+    NT = 0 if plan is None else plan.NT
+    beta = beta.float().contiguous()
+    w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g_cumsum, offsets=offs, indices=idx, head_first=False,
+                                      chunk_size=BT, store_A=True, store_Au=False)
+    hT, v_new, _ = chunk_gated_delta_rule_fwd_h(
+        k=k, w=w, u=u, g=g_cumsum, initial_state=initial_state, output_final_state=False, offsets=offs, indices=idx,
+        head_first=False, chunk_size=BT, fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
+    ws_dvl, ws_dv2 = torch.empty_like(v), torch.empty_like(v)
+    ws_dh = torch.empty_like(hT)
+    ws_dw, ws_dkp = torch.empty_like(k), torch.empty_like(k)
+    ws_dgam = q.new_empty(K // 64, B * T, H, dtype=torch.float32)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dbeta = q.new_empty(B, T, H, dtype=torch.float32)
+    dgam2 = q.new_empty(B, T, H, dtype=torch.float32)
+    dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
+    if dht is not None:
+        dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
+    be.check(be.lib().fla_chunk_gated_delta_rule_bwd(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(w), be.ptr(v_new), be.ptr(beta), be.ptr(g_cumsum), be.ptr(Aw),
+        be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(ws_dvl), be.ptr(ws_dv2), be.ptr(ws_dh), be.ptr(ws_dw),
+        be.ptr(ws_dkp), be.ptr(ws_dgam), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dbeta), be.ptr(dgam2),
+        be.ptr(dh0), be.ptr(offs), be.ptr(idx), be.ptr(co), NT, be.dt(q), B, T, H, K, V, N, float(scale),
+        be.stream_of(q)), "fla_chunk_gated_delta_rule_bwd")
+    dg = None
+    if g_cumsum is not None:
+        dgam = ws_dgam.sum(0).view(B, T, H) + dgam2
+        dg = chunk_local_cumsum(dgam, BT, reverse=True, offsets=offs, indices=idx, head_first=False)
+    return dq, dk, dv, dbeta, dg, dh0
+
+
 class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
 
     @staticmethod
@@ -56,6 +98,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
     @autocast_custom_fwd
     def forward(ctx, q, k, v, g, beta, scale, initial_state, output_final_state, offsets=None, head_first=True):
         be.require_gpu(q, k, v, beta)
+        in_dtypes = (q.dtype, k.dtype, v.dtype, None if g is None else g.dtype, beta.dtype)
         if head_first:
             q, k, v = (x.transpose(1, 2).contiguous() for x in (q, k, v))
             beta = beta.transpose(1, 2).contiguous()
@@ -71,21 +114,46 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             v = F.pad(v, (0, VP - V))
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
-        _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
-                                                    offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+        gc, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
+                                                     offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+        ctx.save_for_backward(q, k, v, gc, beta, h0, offsets)
+        ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
+        ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
             o = o[..., :V]
             if ht is not None:
                 ht = ht[..., :K, :V].contiguous()
         if head_first:
             o = o.transpose(1, 2).contiguous()
-        return o.to(q.dtype), ht
+        return o.to(in_dtypes[0]), ht
 
     @staticmethod
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        raise NotImplementedError("fla_amd chunk_gated_delta_rule: the backward kernels are not built yet")
+        q, k, v, gc, beta, h0, offsets = ctx.saved_tensors
+        K, V, KP, VP = ctx.dims
+        if ctx.head_first:
+            do = do.transpose(1, 2)
+        do = do.to(q.dtype)
+        if VP != V:
+            do = F.pad(do, (0, VP - V))
+        do = do.contiguous()
+        if dht is not None and (KP, VP) != (K, V):
+            dht = F.pad(dht, (0, VP - V, 0, KP - K))
+        dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(q, k, v, gc, beta, ctx.scale, h0, do, dht, offsets)
+        if (KP, VP) != (K, V):
+            dq, dk, dv = dq[..., :K], dk[..., :K], dv[..., :V]
+            if dh0 is not None:
+                dh0 = dh0[..., :K, :V]
+        if ctx.head_first:
+            dq, dk, dv, db = (x.transpose(1, 2) for x in (dq, dk, dv, db))
+            dg = None if dg is None else dg.transpose(1, 2)
+        qd, kd, vd, gd, bd = ctx.in_dtypes
+        if dh0 is not None:
+            dh0 = dh0.to(ctx.h0_dtype)
+        return (dq.to(qd), dk.to(kd), dv.to(vd), None if dg is None else dg.to(gd), db.to(bd), None, dh0,
+                None, None, None)
 
 
 def chunk_gated_delta_rule(

@@ -20,6 +20,7 @@ def fwd_prepare_wy_repr(
     chunk_size: int = 64,
     *,
     store_A: bool = True,
+    store_Au: bool = True,
 ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """Returns ``(w, u, Aw, Au)`` with ``Aw = (I + strict_lower(diag(beta) K K^T))^-1``,
     ``Au = Aw * exp(g_i - g_j)``, ``w = Aw (beta K)``, ``u = Au (beta V)``; ``g`` is the
@@ -38,7 +39,7 @@ def fwd_prepare_wy_repr(
         g = g.float().contiguous()
     w, u = torch.empty_like(k), torch.empty_like(v)
     Aw = k.new_empty(B, T, H, BT) if store_A else None
-    Au = k.new_empty(B, T, H, BT) if store_A else None
+    Au = k.new_empty(B, T, H, BT) if (store_A and store_Au) else None
     be.check(be.lib().fla_gdr_fwd_wy(
         be.ptr(k), be.ptr(v), be.ptr(beta), be.ptr(g), be.ptr(w), be.ptr(u), be.ptr(Aw), be.ptr(Au),
         be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, V, be.stream_of(k)), "fla_gdr_fwd_wy")

@@ -195,6 +195,29 @@ int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* g
                       int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                       float scale, fla_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Chunked gated delta rule backward (chunk size 64), replaces
+ * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):
+ * chunk_bwd_dv_local (common/chunk_o.py:551), chunk_gated_delta_rule_bwd_dhu
+ * (common/chunk_delta_h.py:323), chunk_bwd_dqkwg (common/chunk_o.py:602) and
+ * bwd_prepare_wy_repr (gated_delta_rule/wy_fast.py:565).  Four launches.
+ * Inputs recomputed by the caller with the forward entry points: w, v_new, Aw
+ * (fla_gdr_fwd_wy, fla_chunk_gated_delta_rule_fwd_h) and hT (the per-chunk
+ * states in FLA_H_FRAGMENT_T order).  g_cumsum fp32 [B,T,H] or NULL.
+ * Workspaces: ws_dv_local, ws_dv2 like v; ws_dh_frag_t like hT; ws_dw,
+ * ws_dk_partial like k; ws_dgam_partial fp32 [K/64, B*T, H].
+ * Outputs: dq, dk [B,T,H,K], dv [B,T,H,V] (q/k/v dtype); dbeta and dgam2 fp32
+ * [B,T,H]; dh0 fp32 [N,H,K,V] or NULL.  The gradient w.r.t. the raw gate is the
+ * reverse chunk-local cumsum of (sum over slices of ws_dgam_partial) + dgam2.
+ * ---------------------------------------------------------------------- */
+int fla_chunk_gated_delta_rule_bwd(
+    const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,
+    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT,
+    void* ws_dv_local, void* ws_dv2, void* ws_dh_frag_t, void* ws_dw, void* ws_dk_partial, float* ws_dgam_partial,
+    void* dq, void* dk, void* dv, float* dbeta, float* dgam2, float* dh0,
+    const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
+    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
+
 /* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
  * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,
  * mode 1: 16x16x32 tiles, mode 2: 32x32x16 with the permuted contraction order

@@ -108,3 +108,68 @@ def test_chunk_gdr_varlen(device, T, N, H):
                                                offsets=offs.tolist())
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
+
+
+# ---------------------------------------------------------------- backward
+def _grads_ref(q, k, v, g, beta, h0, do, dht, offsets=None, scale=None):
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    leaves = [x.detach().float().requires_grad_() for x in (q, k, v, g, beta)]
+    h0l = None if h0 is None else h0.detach().float().requires_grad_()
+    o, ht = naive_recurrent_gated_delta_rule(*leaves, scale=scale, initial_state=h0l, output_final_state=True,
+                                             offsets=offsets)
+    ((o * do.float()).sum() + (ht * dht.float()).sum()).backward()
+    return [x.grad for x in leaves] + [None if h0l is None else h0l.grad]
+
+
+def _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=None, scale=None, head_first=False):
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    dev = lambda x: None if x is None else x.to(device)
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    leaves = [tr(dev(x)).detach().requires_grad_() for x in (q, k, v, g, beta)]
+    h0l = None if h0 is None else dev(h0).detach().requires_grad_()
+    o, ht = chunk_gated_delta_rule(*leaves, scale=scale, initial_state=h0l, output_final_state=True,
+                                   offsets=dev(offsets), head_first=head_first)
+    ((o.float() * tr(dev(do)).float()).sum() + (ht * dev(dht)).sum()).backward()
+    torch.cuda.synchronize()
+    return [tr(x.grad) for x in leaves] + [None if h0l is None else h0l.grad]
+
+
+NAMES = ("dq", "dk", "dv", "dg", "dbeta", "dh0")
+# reference tolerances (tests/ops/test_gated_delta.py:220-294): dq,dk,dv,dh0 0.008; dbeta, dg 0.02
+TOLS = (8e-3, 8e-3, 8e-3, 2e-2, 2e-2, 8e-3)
+
+
+@pytest.mark.parametrize("T", [64, 130, 300])
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 64), (64, 128), (128, 64)])
+def test_chunk_gdr_backward(device, T, K, V):
+    B, H = 2, 2
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=51 + T, h0_std=1.0)
+    gen = torch.Generator().manual_seed(7)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    print(f"chunk_gdr backward T={T} K={K} V={V}", flush=True)
+    got = _grads_dev(device, q, k, v, g, beta, h0, do, dht)
+    ref = _grads_ref(q, k, v, g, beta, h0, do, dht)
+    for name, r, x, tol in zip(NAMES, ref, got, TOLS):
+        assert_close(name, r, x, tol)
+
+
+def test_chunk_gdr_backward_varlen_and_headfirst(device):
+    gen = torch.Generator().manual_seed(8)
+    T, N, H, D = 500, 4, 2, 128
+    offs = random_offsets(T, N, gen, min_len=1)
+    q, k, v, g, beta, h0 = gdr_inputs(1, T, H, D, D, seed=61, N=N, h0_std=1.0)
+    do = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(N, H, D, D, generator=gen) * 0.1
+    print(f"chunk_gdr backward varlen offs={offs.tolist()}", flush=True)
+    got = _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs, scale=0.1)
+    ref = _grads_ref(q, k, v, g, beta, h0, do, dht, offsets=offs.tolist(), scale=0.1)
+    for name, r, x, tol in zip(NAMES, ref, got, TOLS):
+        assert_close(name, r, x, tol)
+    q, k, v, g, beta, _ = gdr_inputs(2, 150, 2, 100, 100, seed=62, h0=False)
+    do = torch.randn(2, 150, 2, 100, generator=gen).bfloat16()
+    dht = torch.randn(2, 2, 100, 100, generator=gen) * 0.1
+    got = _grads_dev(device, q, k, v, g, beta, None, do, dht, head_first=True)
+    ref = _grads_ref(q, k, v, g, beta, None, do, dht)
+    for name, r, x, tol in zip(NAMES[:5], ref, got, TOLS):
+        assert_close(name, r, x, tol)
