@@ -1,0 +1,383 @@
+// Fused chunked GLA forward for gfx950: one pass over q, k, v, g produces o and the
+// final state; the per-chunk states never leave the chip.
+//
+// One workgroup of 8 or 12 waves owns one (sequence, head, 64 value columns) and walks the
+// chunks serially.  The waves are specialised:
+//   waves 4..   ("staging")  load chunk c+1 (refilling each register as it is consumed), form the
+//                          chunk-local prefix sum G of the log-gates with wave shuffles,
+//                          and write the gated operand tiles of chunk c+1 to LDS:
+//                          q~ = s q e^{G}, k~ = k e^{-G} (row-major), k^ = k e^{G_last-G}
+//                          and v (time-contiguous), e^{G_last};
+//   waves 0-3 ("matrix")   for chunk c:  S = q~ k~^T,  P = tril(S),
+//                          o = q~ h + P v,  h <- diag(e^{G_last}) h + k^^T v,
+//                          with the fp32 state in MFMA accumulators.
+// Every SIMD therefore hosts one matrix wave and one or two staging waves, so the transcendental
+// and LDS-write work of the next chunk overlaps the MFMAs of the current one.  Operand
+// tiles are double-buffered; both groups meet at two workgroup barriers per chunk.
+// The state is handed from the accumulators to the q~ h product in MFMA-fragment order
+// through LDS (each lane writes and reads its own 32 contiguous bytes per tile).
+//
+// Math: fla/ops/common/chunk_h.py:73-137, fla/ops/gla/chunk.py:29-170 and :320-393.
+// HBM traffic is the operator's floor (q, k, v, g read once per 64-column slab, o
+// written once, h0/ht once) instead of that plus a [B,NT,H,K,V] state round trip.
+#include "chunk_common.h"
+
+namespace {
+
+struct FusedParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const float* h0;
+  void* o;
+  float* ht;
+  const int64_t* offsets;
+  int64_t T;
+  int H, V, N;
+  float scale;
+};
+
+// NSTG: number of staging waves (4 or 8); the workgroup has 4 + NSTG waves.
+template <typename T, typename GT, int K, int NSTG>
+__global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  constexpr int BV = 64;
+  constexpr int LDK = K + 8;
+  constexpr int KT32 = K / 32;                 // 32-row state tiles
+  constexpr int NKT = (KT32 + 3) / 4;          // state tiles per matrix wave (x2 value tiles)
+  constexpr int CPW = K / NSTG;                // key columns per staging wave
+  constexpr int CPL = CPW / 8;                 // key columns per staging lane
+  static_assert(CPL == 4 || CPL == 2, "8 lanes of a staging wave cover its key columns in vectors of 2 or 4");
+  constexpr float LOG2E = 1.4426950408889634f;
+  __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDK];     // q~  [t][k]
+  __shared__ __attribute__((aligned(16))) T sK[2][BT * LDK];     // k~  [t][k]
+  __shared__ __attribute__((aligned(16))) T sKh[2][K * LDT];     // k^  [k][t]
+  __shared__ __attribute__((aligned(16))) T sVt[2][BV * LDT];    // v   [v][t]
+  __shared__ __attribute__((aligned(16))) float sDecay[2][K];
+  __shared__ __attribute__((aligned(16))) T sP[BT * LDT];        // tril(S) [i][j]
+  __shared__ __attribute__((aligned(16))) T sHf[KT32 * 2 * 64 * 16];  // state, fragment order [kt][vt][lane][16]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  // wave-uniform by construction: keeps the role split and the barriers on scalar branches
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = p.H, V = p.V;
+  const int nvb = V / BV;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vb = (int)(id % nvb);
+  const int nh = (int)(id / nvb);
+  const int n = nh / H, hh = nh % H;
+  const int vbase = vb * BV;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+
+  if (wave >= 4) {
+    // =========================== staging waves ===========================
+    const int pw = wave - 4;
+    const int rg = lane >> 3;                         // 8 row groups of 8 rows
+    const int kc = pw * CPW + (lane & 7) * CPL;       // first key column of this lane
+    const int vc = (pw & 3) * 16 + (lane & 7) * 2;    // first value column of this lane
+    const bool has_v = (NSTG == 4) || pw < 4;                        // the value tile is staged by the first four staging waves
+    const int64_t kstride = (int64_t)H * K, vstride = (int64_t)H * V;
+    const T* qp = (const T*)p.q + (sp.bos * H + hh) * (int64_t)K + kc;
+    const T* kp = (const T*)p.k + (sp.bos * H + hh) * (int64_t)K + kc;
+    const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kc;
+    const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + vc;
+    typedef T kvec __attribute__((ext_vector_type(CPL)));
+    typedef GT gvec __attribute__((ext_vector_type(CPL)));
+    struct Regs {
+      gvec g[8];
+      kvec q[8];
+      kvec k[8];
+      t2 v[8];
+    };
+    // Loads are unconditional: rows past the end of the sequence are redirected to its last
+    // row and zeroed afterwards (only a sequence's last chunk can be short), so the compiler
+    // is free to batch and interleave them.
+    const int64_t last_row = sp.len - 1;
+    auto row_of = [&](int64_t c, int i) {
+      int64_t r = c * BT + rg * 8 + i;
+      return r < last_row ? r : last_row;
+    };
+    auto mask_tail = [&](Regs& R, int L) {
+      if (L < BT) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (rg * 8 + i >= L) {
+#pragma unroll
+            for (int j = 0; j < CPL; ++j) {
+              R.g[i][j] = (GT)0.f;
+              R.q[i][j] = (T)0.f;
+              R.k[i][j] = (T)0.f;
+            }
+            R.v[i] = t2{(T)0.f, (T)0.f};
+          }
+        }
+      }
+    };
+    // Stage the tiles of chunk c (held in R) into buffer `buf` and refill R, register by
+    // register as each is consumed, with chunk c+1: the loads of the next chunk are spread
+    // through the arithmetic of this one.  With MID_BARRIER the workgroup barrier that
+    // separates the two halves of the matrix waves' chunk is executed half way through.
+    auto stage = [&](Regs& R, int buf, int64_t c, auto mid_barrier) {
+      mask_tail(R, chunk_len(c));
+      float G[8][CPL], tot[CPL], elast[CPL];
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        float run = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          run = fmaf((float)R.g[i][j], LOG2E, run);   // prefix sums in the log2 domain
+          G[i][j] = run;
+        }
+        float s = run;
+#pragma unroll
+        for (int d = 8; d < 64; d <<= 1) {
+          float u = __shfl_up(s, d, 64);
+          if (lane >= d) s += u;
+        }
+        tot[j] = s - run;
+        elast[j] = __builtin_amdgcn_exp2f(__shfl(s, 56 + (lane & 7), 64));
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 1, i) * kstride);
+      T* dq = sQ[buf];
+      T* dk = sK[buf];
+      T khat[CPL][8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int row = rg * 8 + i;
+        T qv[CPL], kv[CPL];
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+          float e = __builtin_amdgcn_exp2f(G[i][j] + tot[j]);           // e^{G}
+          float einv = __builtin_amdgcn_rcpf(fmaxf(e, 1e-35f));         // e^{-G}, finite
+          float kt = (float)R.k[i][j] * einv;
+          qv[j] = (T)((float)R.q[i][j] * (p.scale * e));
+          kv[j] = (T)kt;
+          khat[j][i] = (T)(kt * elast[j]);                              // k e^{G_last-G}
+        }
+        R.q[i] = *(const kvec*)(qp + row_of(c + 1, i) * kstride);
+        R.k[i] = *(const kvec*)(kp + row_of(c + 1, i) * kstride);
+        if (CPL == 4) {
+          *(v4*)&dq[row * LDK + kc] = v4{qv[0], qv[1], qv[2], qv[3]};
+          *(v4*)&dk[row * LDK + kc] = v4{kv[0], kv[1], kv[2], kv[3]};
+        } else {
+          *(t2*)&dq[row * LDK + kc] = t2{qv[0], qv[1]};
+          *(t2*)&dk[row * LDK + kc] = t2{kv[0], kv[1]};
+        }
+        if (i == 3) mid_barrier();
+      }
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) {
+        v8 x;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = khat[j][i];
+        *(v8*)&sKh[buf][(kc + j) * LDT + rg * 8] = x;
+      }
+      if (has_v) {
+        v8 a, b;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          a[i] = R.v[i][0];
+          b[i] = R.v[i][1];
+        }
+        *(v8*)&sVt[buf][(vc + 0) * LDT + rg * 8] = a;
+        *(v8*)&sVt[buf][(vc + 1) * LDT + rg * 8] = b;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) R.v[i] = *(const t2*)(vp + row_of(c + 1, i) * vstride);
+      }
+      if (rg == 0) {
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) sDecay[buf][kc + j] = elast[j];
+      }
+    };
+
+    if (nchunks > 0) {
+      Regs R0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        R0.g[i] = *(const gvec*)(gp + row_of(0, i) * kstride);
+        R0.q[i] = *(const kvec*)(qp + row_of(0, i) * kstride);
+        R0.k[i] = *(const kvec*)(kp + row_of(0, i) * kstride);
+        if (has_v) R0.v[i] = *(const t2*)(vp + row_of(0, i) * vstride);
+      }
+      stage(R0, 0, 0, [] {});
+      for (int64_t c = 0; c < nchunks; ++c) {
+        __syncthreads();  // B1(c): tiles of chunk c published; buffer (c+1)&1 is free
+        if (c + 1 < nchunks) stage(R0, (int)((c + 1) & 1), c + 1, [] { __syncthreads(); });  // contains B2(c)
+        else __syncthreads();  // B2(c)
+      }
+    }
+  } else {
+    // =========================== matrix waves ===========================
+    const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
+    f32x16 acc[NKT][2];                         // state tiles kt = wave + 4a, value tiles 0/1
+#pragma unroll
+    for (int a = 0; a < NKT; ++a)
+#pragma unroll
+      for (int vt = 0; vt < 2; ++vt) {
+        acc[a][vt] = zero16();
+        int kt = wave + 4 * a;
+        if (p.h0 && kt < KT32) {
+          const float* h0p = p.h0 + (int64_t)nh * K * V;
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[a][vt][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + vt * 32 + (lane & 31)];
+        }
+      }
+    auto publish_state = [&]() {
+#pragma unroll
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
+#pragma unroll
+          for (int vt = 0; vt < 2; ++vt) {
+            v8 lo, hi;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+              lo[r] = (T)acc[a][vt][r];
+              hi[r] = (T)acc[a][vt][r + 8];
+            }
+            T* dst = &sHf[((kt * 2 + vt) * 64 + lane) * 16];
+            *(v8*)dst = lo;
+            *(v8*)(dst + 8) = hi;
+          }
+        }
+      }
+    };
+    publish_state();
+    for (int64_t c = 0; c < nchunks; ++c) {
+      const int buf = (int)(c & 1);
+      const int L = chunk_len(c);
+      const int64_t row0 = sp.bos + c * BT;
+      __syncthreads();  // B1(c)
+      // ---- scores on the lower-triangular quadrants and the inter-chunk part of o
+      const int qi = wave >> 1, qj = wave & 1;
+      f32x16 s = zero16();
+      if (qj <= qi) {
+#pragma unroll
+        for (int ks = 0; ks < K; ks += 16)
+          s = Elem<T>::mfma32(lds_frag32<T>(sQ[buf], LDK, qi * 32, ks, lane),
+                              lds_frag32<T>(sK[buf], LDK, qj * 32, ks, lane), s);
+      }
+      f32x16 o = zero16();
+#pragma unroll
+      for (int kt = 0; kt < KT32; ++kt) {
+        const T* hf = &sHf[((kt * 2 + cw) * 64 + lane) * 16];
+        v8 h0v = *(const v8*)hf, h1v = *(const v8*)(hf + 8);
+        o = Elem<T>::mfma32(lds_frag32_perm<T>(sQ[buf], LDK, rw * 32, kt * 32, lane), h0v, o);
+        o = Elem<T>::mfma32(lds_frag32_perm<T>(sQ[buf], LDK, rw * 32, kt * 32 + 16, lane), h1v, o);
+      }
+      {
+        const int j = qj * 32 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int i = qi * 32 + c32_row(r, lane);
+          sP[i * LDT + j] = (T)((j <= i) ? s[r] : 0.f);
+        }
+      }
+      __syncthreads();  // B2(c): P visible; nobody reads the state fragments any more
+      if (rw == 0) {
+#pragma unroll
+        for (int js = 0; js < 32; js += 16)
+          o = Elem<T>::mfma32(lds_frag32<T>(sP, LDT, 0, js, lane), lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), o);
+      } else {
+#pragma unroll
+        for (int js = 0; js < 64; js += 16)
+          o = Elem<T>::mfma32(lds_frag32<T>(sP, LDT, 32, js, lane), lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), o);
+      }
+      {
+        T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V + vbase + cw * 32 + (lane & 31);
+        if (L == BT) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) op[(int64_t)(rw * 32 + c32_row(r, lane)) * H * V] = (T)o[r];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            int i = rw * 32 + c32_row(r, lane);
+            if (i < L) op[(int64_t)i * H * V] = (T)o[r];
+          }
+        }
+      }
+      // ---- state update
+#pragma unroll
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            f32x4 d = *(const f32x4*)&sDecay[buf][kt * 32 + 8 * q4 + 4 * (lane >> 5)];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+              acc[a][0][4 * q4 + b] *= d[b];
+              acc[a][1][4 * q4 + b] *= d[b];
+            }
+          }
+#pragma unroll
+          for (int ts = 0; ts < BT; ts += 16) {
+            v8 fk = lds_frag32<T>(sKh[buf], LDT, kt * 32, ts, lane);
+            acc[a][0] = Elem<T>::mfma32(fk, lds_frag32<T>(sVt[buf], LDT, 0, ts, lane), acc[a][0]);
+            acc[a][1] = Elem<T>::mfma32(fk, lds_frag32<T>(sVt[buf], LDT, 32, ts, lane), acc[a][1]);
+          }
+        }
+      }
+      publish_state();
+    }
+    if (p.ht) {
+      float* htp = p.ht + (int64_t)nh * K * V;
+#pragma unroll
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
+#pragma unroll
+          for (int vt = 0; vt < 2; ++vt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+              htp[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + vt * 32 + (lane & 31)] = acc[a][vt][r];
+        }
+      }
+    }
+  }
+}
+
+template <typename T, typename GT>
+int launch_fused(const FusedParams& p, int K, hipStream_t st) {
+  int64_t total = (int64_t)(p.V / 64) * p.N * p.H;
+  if (total == 0) return FLA_OK;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  dim3 grid((unsigned)total);
+  if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4>), grid, dim3(512), 0, st, p);
+  else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4>), grid, dim3(512), 0, st, p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+}  // namespace
+
+extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates, const float* h0,
+                                       void* o, float* ht, const int64_t* offsets, int qkv_dtype, int gate_dtype,
+                                       int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                       fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE((K == 64 || K == 128) && V % 64 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)o) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  FusedParams p{q, k, v, gates, h0, o, ht, offsets, T, (int)H, (int)V, (int)N, scale};
+  hipStream_t st = (hipStream_t)stream;
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) return launch_fused<bf16, float>(p, (int)K, st);
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) return launch_fused<bf16, bf16>(p, (int)K, st);
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) return launch_fused<f16, float>(p, (int)K, st);
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) return launch_fused<f16, f16>(p, (int)K, st);
+  return FLA_E_UNSUPPORTED;
+}

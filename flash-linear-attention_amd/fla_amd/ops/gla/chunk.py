@@ -51,8 +51,29 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
     return o
 
 
-def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False):
+def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None):
+    """One-launch forward (``fla_chunk_gla_fwd_fused``): seq-first, K in {64,128}, V % 64 == 0."""
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    N = B if offsets is None else len(offsets) - 1
+    o = torch.empty_like(v)
+    ht = q.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
+    h0 = None
+    if initial_state is not None:
+        h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
+    if offsets is not None:
+        offsets = offsets.to(torch.int64).contiguous()
+    be.check(be.lib().fla_chunk_gla_fwd_fused(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(offsets),
+        be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_fused")
+    return o, ht
+
+
+def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False, fused=True):
     """Seq-first forward on 64-aligned head dims.  Returns (o, ht, A)."""
+    if fused and not want_A and q.shape[-1] in (64, 128):
+        o, ht = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets)
+        return o, ht, None
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     B, T, H, K = q.shape
     h, ht = chunk_fwd_h(

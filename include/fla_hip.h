@@ -135,6 +135,16 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
                         int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                         float scale, fla_stream_t stream);
 
+/* Fused chunked GLA forward: o and the final state in one pass, the per-chunk
+ * states stay on the chip.  Same result as fla_chunk_gla_fwd_h followed by
+ * fla_chunk_gla_fwd_o (the launches of chunk_gla_fwd, fla/ops/gla/chunk.py:1156-1214)
+ * with raw log-gates.  K in {64, 128}, V a multiple of 64.  h0, ht, offsets may be NULL. */
+int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates,
+                            const float* h0, void* o, float* ht, const int64_t* offsets,
+                            int qkv_dtype, int gate_dtype,
+                            int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                            float scale, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Chunked gated delta rule forward (chunk size 64).  g_cumsum is the fp32
  * chunk-local prefix sum of the per-head log-gate [B,T,H] (from
