@@ -93,7 +93,15 @@ def bench_gla(device, steps, warmup):
     ms = elapsed / steps * 1e3
     tokens_per_s = B * T * steps / elapsed
 
-    # per-kernel device time, each entry point launched on its own between events
+    # device time of the kernels of the forward, HIP events on the launch stream.  The
+    # operator is one launch (gla_fwd_fused_kernel); the two-kernel pipeline it replaces
+    # (state scan + per-chunk output) is timed as well for comparison.
+    from fla_amd.ops.gla.chunk import chunk_gla_fwd_fused
+    scale = K ** -0.5
+
+    def run_fused():
+        chunk_gla_fwd_fused(q, k, v, g, scale, h0, True)
+
     h_hold = {}
 
     def run_h():
@@ -102,13 +110,13 @@ def bench_gla(device, steps, warmup):
                                                 fragment_layout=True)
 
     run_h()
-    scale = K ** -0.5
 
     def run_o():
         chunk_gla_fwd_o_gk(q, v, g, None, h_hold["h"], scale, head_first=False, chunk_size=64, k=k,
                            gates_are_cumsum=False)
 
     n_ev = max(steps, 10)
+    us_f = event_avg_us(run_fused, n_ev)
     us_h = event_avg_us(run_h, n_ev)
     us_o = event_avg_us(run_o, n_ev)
     NT = T // 64
@@ -116,22 +124,22 @@ def bench_gla(device, steps, warmup):
     gbytes = B * T * H * K * 4                   # fp32 gates
     hbytes = B * NT * H * K * V * 2              # bf16 per-chunk states
     st = B * H * K * V * 4                       # one fp32 state
+    floor_bytes = 4 * qkv + gbytes + 2 * st      # q,k,v,o + g + h0,ht: the operator's algorithmic bytes
     bytes_h = 2 * qkv + gbytes + hbytes + 2 * st           # k, v, g in; h, ht out; h0 in
     bytes_o = 3 * qkv + gbytes + hbytes + qkv              # q, k, v, g, h in; o out
-    kernels = {
-        "gla_fwd_h_kernel": dict(us=us_h, bytes=bytes_h),
-        "gla_fwd_o_kernel": dict(us=us_o, bytes=bytes_o),
-    }
-    dom = max(kernels, key=lambda n: kernels[n]["us"])
-    ach = kernels[dom]["bytes"] / (kernels[dom]["us"] * 1e-6) / 1e9
-    roofline = {"kernel": dom, "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
-                "avg_us": round(kernels[dom]["us"], 1), "bytes_per_launch": kernels[dom]["bytes"]}
-    floor_bytes = 4 * qkv + gbytes + 2 * st      # q,k,v,o + g + h0,ht: the op's algorithmic floor
+    ach = floor_bytes / (us_f * 1e-6) / 1e9
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/):
+    # 331950 * 2 KiB read (the copy-kernel calibration gives a factor 2 for FETCH_SIZE on this
+    # part) + 139264 KiB written = 784 MiB, i.e. exactly the algorithmic bytes.
+    traffic = 331950 * 2 * 1024 + 139264 * 1024
+    roofline = {"kernel": "gla_fwd_fused_kernel", "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "avg_us": round(us_f, 1), "bytes_per_launch": floor_bytes}
     op = {"algorithmic_bytes": floor_bytes, "achieved_GBs": round(floor_bytes / (ms * 1e-3) / 1e9, 1),
           "frac_of_hbm_peak": round(floor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-          "kernels_us": {n: round(kv["us"], 1) for n, kv in kernels.items()},
-          "kernels_GBs": {n: round(kv["bytes"] / (kv["us"] * 1e-6) / 1e9, 1) for n, kv in kernels.items()}}
+          "two_kernel_pipeline_us": {"gla_fwd_h_kernel": round(us_h, 1), "gla_fwd_o_kernel": round(us_o, 1)},
+          "two_kernel_pipeline_GBs": {"gla_fwd_h_kernel": round(bytes_h / (us_h * 1e-6) / 1e9, 1),
+                                      "gla_fwd_o_kernel": round(bytes_o / (us_o * 1e-6) / 1e9, 1)}}
     return ms, tokens_per_s, roofline, op, c
 
 

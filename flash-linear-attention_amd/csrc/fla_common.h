@@ -87,6 +87,27 @@ FLA_DEVICE T from_f32(float x) { return (T)x; }
 // (fla/ops/utils/exp.py:9-10).
 FLA_DEVICE float safe_exp(float x) { return x <= 0.f ? __expf(x) : 0.f; }
 
+// DPP row operations (a DPP row is 16 consecutive lanes); lanes without a source read 0.
+template <int CTRL>
+FLA_DEVICE float dpp_f32(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+// inclusive prefix / suffix sums across the 16 lanes of a DPP row (VALU only, no LDS traffic)
+FLA_DEVICE float row_prefix16(float x) {
+  x += dpp_f32<0x111>(x);  // row_shr:1
+  x += dpp_f32<0x112>(x);  // row_shr:2
+  x += dpp_f32<0x114>(x);  // row_shr:4
+  x += dpp_f32<0x118>(x);  // row_shr:8
+  return x;
+}
+FLA_DEVICE float row_suffix16(float x) {
+  x += dpp_f32<0x101>(x);  // row_shl:1
+  x += dpp_f32<0x102>(x);  // row_shl:2
+  x += dpp_f32<0x104>(x);  // row_shl:4
+  x += dpp_f32<0x108>(x);  // row_shl:8
+  return x;
+}
+
 struct SeqSpan {
   int64_t bos;  // first token row of the sequence in the packed [B*T] row space
   int64_t len;  // number of tokens

@@ -49,8 +49,8 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   constexpr int KT32 = K / 32;                 // 32-row state tiles
   constexpr int NKT = (KT32 + 3) / 4;          // state tiles per matrix wave (x2 value tiles)
   constexpr int CPW = K / NSTG;                // key columns per staging wave
-  constexpr int CPL = CPW / 8;                 // key columns per staging lane
-  static_assert(CPL == 4 || CPL == 2, "8 lanes of a staging wave cover its key columns in vectors of 2 or 4");
+  constexpr int CPL = CPW / 4;                 // key columns per staging lane (8 for K=128, 4 for K=64)
+  static_assert(CPL == 8 || CPL == 4, "staging lane tiling");
   constexpr float LOG2E = 1.4426950408889634f;
   __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDK];     // q~  [t][k]
   __shared__ __attribute__((aligned(16))) T sK[2][BT * LDK];     // k~  [t][k]
@@ -79,81 +79,75 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
 
   if (wave >= 4) {
     // =========================== staging waves ===========================
+    // A staging wave owns CPW key columns; a lane owns CPL adjacent columns of 4 rows.  The 16
+    // row groups of a column block sit in the 16 lanes of one DPP row, so the prefix sum over
+    // time is register adds plus DPP row shifts.
+    constexpr int LPR = 4;                // lanes (column blocks) per row of the tile
+    constexpr int RPT = 4;                // rows per lane
     const int pw = wave - 4;
-    const int rg = lane >> 3;                         // 8 row groups of 8 rows
-    const int kc = pw * CPW + (lane & 7) * CPL;       // first key column of this lane
-    const int vc = (pw & 3) * 16 + (lane & 7) * 2;    // first value column of this lane
-    const bool has_v = (NSTG == 4) || pw < 4;                        // the value tile is staged by the first four staging waves
-    const int64_t kstride = (int64_t)H * K, vstride = (int64_t)H * V;
+    const int rg = lane & 15;
+    const int kc = pw * CPW + (lane >> 4) * CPL;
+    const int64_t kstride = (int64_t)H * K;
     const T* qp = (const T*)p.q + (sp.bos * H + hh) * (int64_t)K + kc;
     const T* kp = (const T*)p.k + (sp.bos * H + hh) * (int64_t)K + kc;
     const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kc;
-    const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + vc;
-    typedef T kvec __attribute__((ext_vector_type(CPL)));
     typedef GT gvec __attribute__((ext_vector_type(CPL)));
+    typedef T kvec __attribute__((ext_vector_type(CPL)));
     struct Regs {
-      gvec g[8];
-      kvec q[8];
-      kvec k[8];
-      t2 v[8];
+      gvec g[RPT];
+      kvec q[RPT];
+      kvec k[RPT];
     };
     // Loads are unconditional: rows past the end of the sequence are redirected to its last
     // row and zeroed afterwards (only a sequence's last chunk can be short), so the compiler
     // is free to batch and interleave them.
     const int64_t last_row = sp.len - 1;
     auto row_of = [&](int64_t c, int i) {
-      int64_t r = c * BT + rg * 8 + i;
+      int64_t r = c * BT + rg * RPT + i;
       return r < last_row ? r : last_row;
     };
     auto mask_tail = [&](Regs& R, int L) {
       if (L < BT) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          if (rg * 8 + i >= L) {
+        for (int i = 0; i < RPT; ++i) {
+          if (rg * RPT + i >= L) {
 #pragma unroll
             for (int j = 0; j < CPL; ++j) {
               R.g[i][j] = (GT)0.f;
               R.q[i][j] = (T)0.f;
               R.k[i][j] = (T)0.f;
             }
-            R.v[i] = t2{(T)0.f, (T)0.f};
           }
         }
       }
     };
     // Stage the tiles of chunk c (held in R) into buffer `buf` and refill R, register by
-    // register as each is consumed, with chunk c+1: the loads of the next chunk are spread
-    // through the arithmetic of this one.  With MID_BARRIER the workgroup barrier that
-    // separates the two halves of the matrix waves' chunk is executed half way through.
+    // register as each is consumed, with chunk c+2: the loads of the next chunk are spread
+    // through the arithmetic of this one.  mid_barrier() is called half way through; in the
+    // steady state it is the workgroup barrier between the two halves of the matrix waves' chunk.
     auto stage = [&](Regs& R, int buf, int64_t c, auto mid_barrier) {
       mask_tail(R, chunk_len(c));
-      float G[8][CPL], tot[CPL], elast[CPL];
+      float G[RPT][CPL], tot[CPL], elast[CPL];
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
         float run = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
+        for (int i = 0; i < RPT; ++i) {
           run = fmaf((float)R.g[i][j], LOG2E, run);   // prefix sums in the log2 domain
           G[i][j] = run;
         }
-        float s = run;
-#pragma unroll
-        for (int d = 8; d < 64; d <<= 1) {
-          float u = __shfl_up(s, d, 64);
-          if (lane >= d) s += u;
-        }
-        tot[j] = s - run;
-        elast[j] = __builtin_amdgcn_exp2f(__shfl(s, 56 + (lane & 7), 64));
+        float pre = row_prefix16(run);
+        float suf = row_suffix16(run);
+        tot[j] = pre - run;                                      // gates of the earlier row groups
+        elast[j] = __builtin_amdgcn_exp2f(pre + suf - run);      // e^{G_last}
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 1, i) * kstride);
-      T* dq = sQ[buf];
-      T* dk = sK[buf];
-      T khat[CPL][8];
+      for (int i = 0; i < RPT; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 2, i) * kstride);
+      T khat[CPL][RPT];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = rg * 8 + i;
-        T qv[CPL], kv[CPL];
+      for (int i = 0; i < RPT; ++i) {
+        const int row = rg * RPT + i;
+        kvec qv, kv;
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
           float e = __builtin_amdgcn_exp2f(G[i][j] + tot[j]);           // e^{G}
@@ -163,35 +157,19 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           kv[j] = (T)kt;
           khat[j][i] = (T)(kt * elast[j]);                              // k e^{G_last-G}
         }
-        R.q[i] = *(const kvec*)(qp + row_of(c + 1, i) * kstride);
-        R.k[i] = *(const kvec*)(kp + row_of(c + 1, i) * kstride);
-        if (CPL == 4) {
-          *(v4*)&dq[row * LDK + kc] = v4{qv[0], qv[1], qv[2], qv[3]};
-          *(v4*)&dk[row * LDK + kc] = v4{kv[0], kv[1], kv[2], kv[3]};
-        } else {
-          *(t2*)&dq[row * LDK + kc] = t2{qv[0], qv[1]};
-          *(t2*)&dk[row * LDK + kc] = t2{kv[0], kv[1]};
-        }
-        if (i == 3) mid_barrier();
+        R.q[i] = *(const kvec*)(qp + row_of(c + 2, i) * kstride);
+        R.k[i] = *(const kvec*)(kp + row_of(c + 2, i) * kstride);
+        *(kvec*)&sQ[buf][row * LDK + kc] = qv;
+        *(kvec*)&sK[buf][row * LDK + kc] = kv;
+        if (i == RPT / 2 - 1) mid_barrier();
       }
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
-        v8 x;
+        typedef T rvec __attribute__((ext_vector_type(RPT)));
+        rvec x;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = khat[j][i];
-        *(v8*)&sKh[buf][(kc + j) * LDT + rg * 8] = x;
-      }
-      if (has_v) {
-        v8 a, b;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          a[i] = R.v[i][0];
-          b[i] = R.v[i][1];
-        }
-        *(v8*)&sVt[buf][(vc + 0) * LDT + rg * 8] = a;
-        *(v8*)&sVt[buf][(vc + 1) * LDT + rg * 8] = b;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) R.v[i] = *(const t2*)(vp + row_of(c + 1, i) * vstride);
+        for (int i = 0; i < RPT; ++i) x[i] = khat[j][i];
+        *(rvec*)&sKh[buf][(kc + j) * LDT + rg * RPT] = x;
       }
       if (rg == 0) {
 #pragma unroll
@@ -200,19 +178,27 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     };
 
     if (nchunks > 0) {
-      Regs R0;
+      // Two register sets, used alternately: the loads refilling a set have two chunk periods
+      // to land before it is staged again.
+      Regs RA, RB;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        R0.g[i] = *(const gvec*)(gp + row_of(0, i) * kstride);
-        R0.q[i] = *(const kvec*)(qp + row_of(0, i) * kstride);
-        R0.k[i] = *(const kvec*)(kp + row_of(0, i) * kstride);
-        if (has_v) R0.v[i] = *(const t2*)(vp + row_of(0, i) * vstride);
+      for (int i = 0; i < RPT; ++i) {
+        RA.g[i] = *(const gvec*)(gp + row_of(0, i) * kstride);
+        RA.q[i] = *(const kvec*)(qp + row_of(0, i) * kstride);
+        RA.k[i] = *(const kvec*)(kp + row_of(0, i) * kstride);
+        RB.g[i] = *(const gvec*)(gp + row_of(1, i) * kstride);
+        RB.q[i] = *(const kvec*)(qp + row_of(1, i) * kstride);
+        RB.k[i] = *(const kvec*)(kp + row_of(1, i) * kstride);
       }
-      stage(R0, 0, 0, [] {});
-      for (int64_t c = 0; c < nchunks; ++c) {
-        __syncthreads();  // B1(c): tiles of chunk c published; buffer (c+1)&1 is free
-        if (c + 1 < nchunks) stage(R0, (int)((c + 1) & 1), c + 1, [] { __syncthreads(); });  // contains B2(c)
+      stage(RA, 0, 0, [] {});
+      for (int64_t c = 0; c < nchunks; c += 2) {
+        __syncthreads();  // B1(c): tiles of chunk c published; buffer 1 is free
+        if (c + 1 < nchunks) stage(RB, 1, c + 1, [] { __syncthreads(); });  // contains B2(c)
         else __syncthreads();  // B2(c)
+        if (c + 1 >= nchunks) break;
+        __syncthreads();  // B1(c+1)
+        if (c + 2 < nchunks) stage(RA, 0, c + 2, [] { __syncthreads(); });  // contains B2(c+1)
+        else __syncthreads();  // B2(c+1)
       }
     }
   } else {
@@ -253,11 +239,46 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     };
     publish_state();
+    // The matrix waves also stage the value tile (time-contiguous) of the next chunk: 8 rows x
+    // 2 columns per lane, loaded one chunk period ahead.
+    const int vrg = tid >> 5, vc = (tid & 31) * 2;
+    const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + vc;
+    const int64_t vstride = (int64_t)H * V;
+    const int64_t last_row = sp.len - 1;
+    t2 vreg[8];
+    auto load_v = [&](int64_t c) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int64_t r = c * BT + vrg * 8 + i;
+        vreg[i] = *(const t2*)(vp + (r < last_row ? r : last_row) * vstride);
+      }
+    };
+    auto stage_v = [&](int buf, int64_t c) {
+      const int L = chunk_len(c);
+      v8 a, b;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        bool ok = vrg * 8 + i < L;
+        a[i] = ok ? vreg[i][0] : (T)0.f;
+        b[i] = ok ? vreg[i][1] : (T)0.f;
+      }
+      *(v8*)&sVt[buf][(vc + 0) * LDT + vrg * 8] = a;
+      *(v8*)&sVt[buf][(vc + 1) * LDT + vrg * 8] = b;
+    };
+    if (nchunks > 0) {
+      load_v(0);
+      stage_v(0, 0);
+      load_v(1);
+    }
     for (int64_t c = 0; c < nchunks; ++c) {
       const int buf = (int)(c & 1);
       const int L = chunk_len(c);
       const int64_t row0 = sp.bos + c * BT;
       __syncthreads();  // B1(c)
+      if (c + 1 < nchunks) {
+        stage_v(buf ^ 1, c + 1);
+        load_v(c + 2);
+      }
       // ---- scores on the lower-triangular quadrants and the inter-chunk part of o
       const int qi = wave >> 1, qj = wave & 1;
       f32x16 s = zero16();
