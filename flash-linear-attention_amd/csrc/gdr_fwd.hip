@@ -374,30 +374,58 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
     int64_t rem = sp.len - c * BT;
     return (int)(rem < BT ? rem : BT);
   };
+  // Addressing: a wave-uniform 64-bit base per chunk plus 32-bit per-lane element offsets that
+  // are computed once, so a load costs no per-lane 64-bit arithmetic.  Rows past the end of a
+  // short (last) chunk are redirected to its last row and zeroed afterwards.
+  const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
+  uint32_t offk[RPT], offg[RPT], offu[4];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    offk[i] = (uint32_t)(rg * RPT + i) * HK + c4;
+    offg[i] = (uint32_t)(rg * RPT + i) * H;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) offu[i] = (uint32_t)(urg * 4 + i) * HV + uc2;
   auto load_chunk = [&](int64_t c, Regs& R) {
-    int L = chunk_len(c);
-    bool live = c < nchunks;
-    int64_t rbase = sp.bos + c * BT;
+    if (c >= nchunks) return;  // wave-uniform
+    const int L = chunk_len(c);
+    const int64_t rbase = (sp.bos + c * BT) * H + hh;
+    const T* wb = (const T*)p.w + rbase * K;
+    const T* kb = (const T*)p.k + rbase * K;
+    const T* ub = (const T*)p.u + rbase * V + vbase;
+    const float* gb = p.gam ? p.gam + rbase : nullptr;
+    if (L == BT) {
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      if (live && row < L) {
-        R.w[i] = *(const v4*)((const T*)p.w + ((rbase + row) * H + hh) * (int64_t)K + c4);
-        R.k[i] = *(const v4*)((const T*)p.k + ((rbase + row) * H + hh) * (int64_t)K + c4);
-        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
-      } else {
-        R.w[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.gam[i] = 0.f;
+      for (int i = 0; i < RPT; ++i) {
+        R.w[i] = *(const v4*)(wb + offk[i]);
+        R.k[i] = *(const v4*)(kb + offk[i]);
+        R.gam[i] = gb ? gb[offg[i]] : 0.f;
       }
-    }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int row = urg * 4 + i;
-      if (live && row < L) R.u[i] = *(const t2*)((const T*)p.u + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
-      else R.u[i] = t2{(T)0.f, (T)0.f};
+      for (int i = 0; i < 4; ++i) R.u[i] = *(const t2*)(ub + offu[i]);
+      R.glast = gb ? gb[(uint32_t)(BT - 1) * H] : 0.f;
+    } else {
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        int row = rg * RPT + i;
+        bool ok = row < L;
+        uint32_t rr = (uint32_t)(ok ? row : L - 1);
+        v4 wv = *(const v4*)(wb + rr * HK + c4);
+        v4 kv = *(const v4*)(kb + rr * HK + c4);
+        float gv = gb ? gb[rr * H] : 0.f;
+        R.w[i] = ok ? wv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.k[i] = ok ? kv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        R.gam[i] = ok ? gv : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int row = urg * 4 + i;
+        bool ok = row < L;
+        t2 uv = *(const t2*)(ub + (uint32_t)(ok ? row : L - 1) * HV + uc2);
+        R.u[i] = ok ? uv : t2{(T)0.f, (T)0.f};
+      }
+      R.glast = gb ? gb[(uint32_t)(L - 1) * H] : 0.f;
     }
-    R.glast = (live && p.gam) ? p.gam[(rbase + L - 1) * H + hh] : 0.f;
   };
   // state-independent operand tiles of one chunk
   auto stage_wu = [&](const Regs& R) {
@@ -484,9 +512,9 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   // Rc holds the chunk whose tiles are staged next, Rn the one after; loads run a full
   // iteration ahead of their use.
   Regs Rc, Rn;
-  load_chunk(0, Rc);
-  load_chunk(1, Rn);
   if (nchunks > 0) {
+    load_chunk(0, Rc);
+    load_chunk(1, Rn);
     stage_wu(Rc);
     publish_h(0);
   }

@@ -33,6 +33,9 @@ struct FusedParams {
   void* o;
   float* ht;
   const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int* wide;        // [chunks, H]: 1 where a chunk's gates leave the single-reference range
+  void* hwide;      // states entering those chunks, FLA_H_FRAGMENT order, [chunks, H, K*V]
   int64_t T;
   int H, V, N;
   float scale;
@@ -59,6 +62,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   __shared__ __attribute__((aligned(16))) float sDecay[2][K];
   __shared__ __attribute__((aligned(16))) T sP[BT * LDT];        // tril(S) [i][j]
   __shared__ __attribute__((aligned(16))) T sHf[KT32 * 2 * 64 * 16];  // state, fragment order [kt][vt][lane][16]
+  __shared__ int sWide[2][NSTG];                                   // per staging wave: gates out of range
 
   const int tid = threadIdx.x, lane = tid & 63;
   // wave-uniform by construction: keeps the role split and the barriers on scalar branches
@@ -72,6 +76,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   const int vbase = vb * BV;
   SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
   auto chunk_len = [&](int64_t c) {
     int64_t rem = sp.len - c * BT;
     return (int)(rem < BT ? rem : BT);
@@ -127,7 +132,8 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     // steady state it is the workgroup barrier between the two halves of the matrix waves' chunk.
     auto stage = [&](Regs& R, int buf, int64_t c, auto mid_barrier) {
       mask_tail(R, chunk_len(c));
-      float G[RPT][CPL], tot[CPL], elast[CPL];
+      float G[RPT][CPL], tot[CPL], glast[CPL];
+      float gabs = 0.f;
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
         float run = 0.f;
@@ -139,7 +145,16 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         float pre = row_prefix16(run);
         float suf = row_suffix16(run);
         tot[j] = pre - run;                                      // gates of the earlier row groups
-        elast[j] = __builtin_amdgcn_exp2f(pre + suf - run);      // e^{G_last}
+        glast[j] = pre + suf - run;                              // G_last (log2 domain)
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) gabs = fmaxf(gabs, fabsf(G[i][j] + tot[j]));
+      }
+      // The scores use one reference point per chunk (e^{G} on q, e^{-G} on k), exact while
+      // |G| stays below kMaxInvDecayExp.  Chunks beyond that are flagged and recomputed by
+      // the exact kernel afterwards.
+      {
+        const int out_of_range = __any(gabs > kMaxInvDecayExp * LOG2E);
+        if (lane == 0) sWide[buf][pw] = out_of_range;
       }
 #pragma unroll
       for (int i = 0; i < RPT; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 2, i) * kstride);
@@ -150,12 +165,13 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         kvec qv, kv;
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
-          float e = __builtin_amdgcn_exp2f(G[i][j] + tot[j]);           // e^{G}
+          const float Gij = G[i][j] + tot[j];
+          float e = __builtin_amdgcn_exp2f(Gij);                        // e^{G}
           float einv = __builtin_amdgcn_rcpf(fmaxf(e, 1e-35f));         // e^{-G}, finite
-          float kt = (float)R.k[i][j] * einv;
+          const float kf = (float)R.k[i][j];
           qv[j] = (T)((float)R.q[i][j] * (p.scale * e));
-          kv[j] = (T)kt;
-          khat[j][i] = (T)(kt * elast[j]);                              // k e^{G_last-G}
+          kv[j] = (T)(kf * einv);
+          khat[j][i] = (T)(kf * __builtin_amdgcn_exp2f(glast[j] - Gij));  // k e^{G_last-G}, exponent <= 0
         }
         R.q[i] = *(const kvec*)(qp + row_of(c + 2, i) * kstride);
         R.k[i] = *(const kvec*)(kp + row_of(c + 2, i) * kstride);
@@ -173,7 +189,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       if (rg == 0) {
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) sDecay[buf][kc + j] = elast[j];
+        for (int j = 0; j < CPL; ++j) sDecay[buf][kc + j] = __builtin_amdgcn_exp2f(glast[j]);
       }
     };
 
@@ -275,6 +291,22 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       const int L = chunk_len(c);
       const int64_t row0 = sp.bos + c * BT;
       __syncthreads();  // B1(c)
+      if (p.wide) {
+        int wide = 0;
+#pragma unroll
+        for (int w2 = 0; w2 < NSTG; ++w2) wide |= sWide[buf][w2];
+        if (tid == 0) p.wide[(chunk0 + c) * H + hh] = wide;
+        if (wide) {
+          // hand the state entering this chunk to the exact kernel (fragment order, this slab's columns)
+          T* hw = (T*)p.hwide + ((chunk0 + c) * H + hh) * (int64_t)K * V;
+          for (int e = tid; e < KT32 * 2 * 64 * 2; e += 256) {
+            int piece = e & 1, ln = (e >> 1) & 63, tile = e >> 7;  // tile = kt*2 + vt
+            int kt = tile >> 1, vt = tile & 1;
+            v8 x = *(const v8*)&sHf[(tile * 64 + ln) * 16 + piece * 8];
+            *(v8*)(hw + (((int64_t)kt * (V / 32) + (vbase / 32 + vt)) * 64 + ln) * 16 + piece * 8) = x;
+          }
+        }
+      }
       if (c + 1 < nchunks) {
         stage_v(buf ^ 1, c + 1);
         load_v(c + 2);
@@ -368,6 +400,178 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   }
 }
 
+// Exact recomputation of the output rows of flagged chunks: the scores
+//   A_ij = s sum_k q_ik k_jk e^{G_ik - G_jk}   (j <= i)
+// are evaluated pair by pair in fp32 with every exponent <= 0, as the reference does on its
+// diagonal sub-blocks (fla/ops/gla/chunk.py:113-170), then o = (s q e^{G}) h_c + A v on MFMA.
+struct ExactParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const int* wide;
+  const void* hwide;
+  void* o;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+template <typename T, typename GT, int K, int V>
+__global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int LDG = K + 4;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int KT32 = K / 32, TV = V / 64;
+  const int hh = blockIdx.y, H = p.H;
+  if (p.wide[(int64_t)blockIdx.x * H + hh] == 0) return;  // workgroup-uniform
+  __shared__ __attribute__((aligned(16))) float sG[BT * LDG];
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
+  __shared__ __attribute__((aligned(16))) T sVt[V * LDT];
+  __shared__ __attribute__((aligned(16))) T sP[BT * LDT];
+  __shared__ __attribute__((aligned(16))) float sPart[RG * K];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+  const int rg = tid / CG, c4 = (tid % CG) * 4;
+  float gq[RPT][4];
+  v4 qreg[RPT], kreg[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    if (row < L) {
+      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
+      Load<GT>::x4((const GT*)p.g + off, gq[i]);
+      qreg[i] = *(const v4*)((const T*)p.q + off);
+      kreg[i] = *(const v4*)((const T*)p.k + off);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) gq[i][j] = 0.f;
+      qreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      kreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    }
+  }
+  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) {
+    int row = rgv * RPTV + i;
+    v4 x = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    if (row < L) x = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + cv4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sVt[(cv4 + j) * LDT + row] = x[j];
+  }
+  float run[4] = {0.f, 0.f, 0.f, 0.f};
+  float G[RPT][4];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      run[j] += gq[i][j];
+      G[i][j] = run[j];
+    }
+  *(f32x4*)&sPart[rg * K + c4] = f32x4{run[0], run[1], run[2], run[3]};
+  __syncthreads();
+  float off[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < rg; ++r) {
+    f32x4 pr = *(const f32x4*)&sPart[r * K + c4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) off[j] += pr[j];
+  }
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    *(f32x4*)&sG[row * LDG + c4] = f32x4{G[i][0] + off[0], G[i][1] + off[1], G[i][2] + off[2], G[i][3] + off[3]};
+    *(v4*)&sQ[row * LDK + c4] = qreg[i];
+    *(v4*)&sK[row * LDK + c4] = kreg[i];
+  }
+  __syncthreads();
+  // ---- exact scores: lane handles row i and every fourth column j <= i
+  {
+    const int i = tid >> 2, jq = tid & 3;
+    for (int j = 0; j < BT; ++j) {
+      if ((j & 3) != jq) continue;
+      float a = 0.f;
+      if (j <= i) {
+        for (int kk = 0; kk < K; kk += 4) {
+          f32x4 gi = *(const f32x4*)&sG[i * LDG + kk];
+          f32x4 gj = *(const f32x4*)&sG[j * LDG + kk];
+          v4 qv = *(const v4*)&sQ[i * LDK + kk];
+          v4 kv = *(const v4*)&sK[j * LDK + kk];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a += (float)qv[e] * (float)kv[e] * __expf(gi[e] - gj[e]);
+        }
+      }
+      sP[i * LDT + j] = (T)(a * p.scale);
+    }
+  }
+  __syncthreads();
+  // ---- q~ = s q e^{G} over the raw q tile (every lane rewrites exactly what it reads)
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    int row = rg * RPT + i;
+    f32x4 gg = *(const f32x4*)&sG[row * LDG + c4];
+    v4 qv = *(const v4*)&sQ[row * LDK + c4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) qv[j] = (T)((float)qv[j] * p.scale * __expf(gg[j]));
+    *(v4*)&sQ[row * LDK + c4] = qv;
+  }
+  __syncthreads();
+  const int rw = wave >> 1, cw = wave & 1;
+  f32x16 acc[TV];
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+  const T* hp = (const T*)p.hwide + ((int64_t)blockIdx.x * H + hh) * (int64_t)K * V;
+#pragma unroll
+  for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      v8 a = lds_frag32_perm<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) {
+        v8 b = *(const v8*)(hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16 + half * 8);
+        acc[tv] = Elem<T>::mfma32(a, b, acc[tv]);
+      }
+    }
+  const int jend = (rw + 1) * 32;
+  for (int js = 0; js < jend; js += 16) {
+    v8 a = lds_frag32<T>(sP, LDT, rw * 32, js, lane);
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
+  }
+  T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
+#pragma unroll
+  for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int i = rw * 32 + c32_row(r, lane);
+      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    }
+}
+
+template <typename T, typename GT>
+int launch_exact(const ExactParams& p, int K, int V, dim3 grid, hipStream_t st) {
+#define FLA_CASE(KK, VV)                                                                              \
+  if (K == KK && V == VV) {                                                                           \
+    hipLaunchKernelGGL((gla_fwd_o_exact_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);           \
+    FLA_CHECK_LAUNCH();                                                                               \
+    return FLA_OK;                                                                                    \
+  }
+  FLA_CASE(64, 64)
+  FLA_CASE(128, 128)
+  FLA_CASE(64, 128)
+  FLA_CASE(128, 64)
+#undef FLA_CASE
+  return FLA_E_UNSUPPORTED;
+}
+
 template <typename T, typename GT>
 int launch_fused(const FusedParams& p, int K, hipStream_t st) {
   int64_t total = (int64_t)(p.V / 64) * p.N * p.H;
@@ -384,21 +588,38 @@ int launch_fused(const FusedParams& p, int K, hipStream_t st) {
 }  // namespace
 
 extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates, const float* h0,
-                                       void* o, float* ht, const int64_t* offsets, int qkv_dtype, int gate_dtype,
-                                       int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
-                                       fla_stream_t stream) {
+                                       void* o, float* ht, int* ws_wide, void* ws_hwide, const int64_t* offsets,
+                                       const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                                       int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
+                                       int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
-  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE((K == 64 || K == 128) && V % 64 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
-  if (offsets) FLA_REQUIRE(B == 1, FLA_E_INVALID);
+  FLA_REQUIRE((ws_wide == nullptr) == (ws_hwide == nullptr), FLA_E_INVALID);
+  if (offsets) FLA_REQUIRE(B == 1 && (!ws_wide || (indices && chunk_offsets)), FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)o) % 16 == 0,
+  if (ws_wide) FLA_REQUIRE(V <= 128, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)o | (uintptr_t)ws_hwide) % 16 == 0,
               FLA_E_ALIGNMENT);
-  FusedParams p{q, k, v, gates, h0, o, ht, offsets, T, (int)H, (int)V, (int)N, scale};
+  FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, ws_wide, ws_hwide, T, (int)H, (int)V, (int)N, scale};
   hipStream_t st = (hipStream_t)stream;
-  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) return launch_fused<bf16, float>(p, (int)K, st);
-  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) return launch_fused<bf16, bf16>(p, (int)K, st);
-  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) return launch_fused<f16, float>(p, (int)K, st);
-  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) return launch_fused<f16, f16>(p, (int)K, st);
+  dim3 grid;
+  int ntfix = 0;
+  if (ws_wide) {
+    int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+    if (rc) return rc;
+  }
+  ExactParams e{q, k, v, gates, ws_wide, ws_hwide, o, offsets, indices, T, (int)H, ntfix, scale};
+#define FLA_FUSED(TT, GG)                                                \
+  {                                                                      \
+    int rc = launch_fused<TT, GG>(p, (int)K, st);                        \
+    if (rc || !ws_wide || grid.x == 0) return rc;                        \
+    return launch_exact<TT, GG>(e, (int)K, (int)V, grid, st);            \
+  }
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_FUSED(bf16, float)
+  if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_FUSED(bf16, bf16)
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) FLA_FUSED(f16, float)
+  if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) FLA_FUSED(f16, f16)
+#undef FLA_FUSED
   return FLA_E_UNSUPPORTED;
 }

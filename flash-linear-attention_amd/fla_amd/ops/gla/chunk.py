@@ -51,20 +51,28 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
     return o
 
 
-def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None):
-    """One-launch forward (``fla_chunk_gla_fwd_fused``): seq-first, K in {64,128}, V % 64 == 0."""
+def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True):
+    """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
+    With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
+    single-reference range are detected on the device and recomputed exactly."""
     B, T, H, K = q.shape
     V = v.shape[-1]
-    N = B if offsets is None else len(offsets) - 1
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    N = B if plan is None else plan.N
     o = torch.empty_like(v)
     ht = q.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
     h0 = None
     if initial_state is not None:
         h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
-    if offsets is not None:
-        offsets = offsets.to(torch.int64).contiguous()
+    wide = hwide = None
+    if exact_guard and V <= 128:
+        chunks = plan.NT if plan is not None else B * (-(-T // BT))
+        wide = q.new_empty(chunks, H, dtype=torch.int32)
+        hwide = q.new_empty(chunks, H, K * V)
     be.check(be.lib().fla_chunk_gla_fwd_fused(
-        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(offsets),
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide),
+        be.ptr(None if plan is None else plan.offsets), be.ptr(None if plan is None else plan.indices),
+        be.ptr(None if plan is None else plan.chunk_offsets), 0 if plan is None else plan.NT,
         be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_fused")
     return o, ht
 

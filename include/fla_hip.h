@@ -138,10 +138,18 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
 /* Fused chunked GLA forward: o and the final state in one pass, the per-chunk
  * states stay on the chip.  Same result as fla_chunk_gla_fwd_h followed by
  * fla_chunk_gla_fwd_o (the launches of chunk_gla_fwd, fla/ops/gla/chunk.py:1156-1214)
- * with raw log-gates.  K in {64, 128}, V a multiple of 64.  h0, ht, offsets may be NULL. */
+ * with raw log-gates.  K in {64, 128}, V a multiple of 64.  h0, ht, offsets may be NULL.
+ * The fused kernel scores a chunk with one reference point (exact while the
+ * chunk-cumulative log-gate stays within +-80 per channel).  With the workspaces
+ * ws_wide (int32 [chunks, H]) and ws_hwide (q/k/v dtype, [chunks, H, K*V]) given
+ * (V <= 128), chunks outside that range are flagged on the device and their
+ * output rows recomputed by a second launch with exact pairwise exponents
+ * (the reference's diagonal sub-block arithmetic, fla/ops/gla/chunk.py:113-170);
+ * packed batches then also need indices [NT,2] and chunk_offsets [N+1]. */
 int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates,
-                            const float* h0, void* o, float* ht, const int64_t* offsets,
-                            int qkv_dtype, int gate_dtype,
+                            const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                            const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
+                            int64_t NT, int qkv_dtype, int gate_dtype,
                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                             float scale, fla_stream_t stream);
 

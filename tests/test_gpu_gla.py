@@ -182,3 +182,33 @@ def test_chunk_gla_backward_varlen_headfirst_odd(device):
     for name, r, x, tol in zip(("dq", "dk", "dv", "dg"), ref, got, (8e-3, 8e-3, 8e-3, 2e-2)):
         assert_close(name, r, x, tol)
     assert got[3].dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("normalizer", [0.05, 0.3])
+@pytest.mark.parametrize("T", [100, 300])
+def test_chunk_gla_extreme_gates(device, normalizer, T):
+    """Gate magnitudes of the reference sweep (normalizer 0.05, tests/ops/test_gla.py:90-146) where the
+    chunk-cumulative log-gate runs into the hundreds: the device-side range guard routes those
+    chunks through the exact pairwise path."""
+    from oracle.recurrent import naive_recurrent_gla
+    q, k, v, g, h0 = gla_inputs(2, T, 2, 128, 128, seed=71, normalizer=normalizer, h0_std=1.0)
+    print(f"chunk_gla extreme gates normalizer={normalizer} T={T} min g={g.min().item():.1f}", flush=True)
+    o, ht = _run(device, q, k, v, g, h0)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+def test_chunk_gla_extreme_gates_mixed_varlen(device):
+    """Only some chunks (and some channels) leave the safe range; packed batch, K != V."""
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(72)
+    T, N = 700, 3
+    offs = random_offsets(T, N, gen, min_len=70)
+    q, k, v, g, h0 = gla_inputs(1, T, 2, 64, 128, seed=72, N=N, normalizer=16.0)
+    g[:, 200:330, :, :17] *= 400.0      # a stretch of very strong decay on a few channels
+    print(f"chunk_gla mixed extreme gates offs={offs.tolist()}", flush=True)
+    o, ht = _run(device, q, k, v, g, h0, offsets=offs)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True, offsets=offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
