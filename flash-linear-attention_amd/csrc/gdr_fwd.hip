@@ -41,37 +41,24 @@ struct ChunkLoc {
   int64_t cglob;  // global chunk index (addresses per-chunk states)
 };
 
-FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix) {
+FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix, int64_t cidx) {
   ChunkLoc c;
   int64_t bos, len, ic;
   if (offsets) {
-    int64_t n = indices[2 * (int64_t)blockIdx.x];
-    ic = indices[2 * (int64_t)blockIdx.x + 1];
+    int64_t n = indices[2 * cidx];
+    ic = indices[2 * cidx + 1];
     bos = offsets[n];
     len = offsets[n + 1] - bos;
   } else {
-    bos = (blockIdx.x / ntfix) * T;
-    ic = blockIdx.x % ntfix;
+    bos = (cidx / ntfix) * T;
+    ic = cidx % ntfix;
     len = T;
   }
   c.row0 = bos + ic * BT;
   int64_t rem = len - ic * BT;
   c.L = (int)(rem < BT ? rem : BT);
-  c.cglob = blockIdx.x;
+  c.cglob = cidx;
   return c;
-}
-
-// C[n x n] (+)= sign * A[n x n] B[n x n], fp32 in LDS, spread over `nthr` threads.
-template <int N>
-FLA_DEVICE void lds_mm(const float* A, int lda, const float* B, int ldb, float* C, int ldc, float sign, int t,
-                       int nthr) {
-  for (int e = t; e < N * N; e += nthr) {
-    int i = e / N, j = e % N;
-    float acc = 0.f;
-#pragma unroll 8
-    for (int k = 0; k < N; ++k) acc += A[i * lda + k] * B[k * ldb + j];
-    C[i * ldc + j] = sign * acc;
-  }
 }
 
 struct WyParams {
@@ -89,60 +76,128 @@ struct WyParams {
   int H, NTfix;
 };
 
+// out^T tile = X^T-tile A^T for a lower-triangular 16-bit A [64 x 64] in LDS and
+// X^T [columns][t] in LDS.  The transposed product leaves each lane with four
+// consecutive output columns of one row (8-byte LDS writes in wy_store).
+template <typename T, int N>
+FLA_DEVICE void wy_apply(const T* sA, const T* sXT, f32x16* acc, int wave, int lane) {
+  typedef typename Elem<T>::v8 v8;
+  constexpr int TN = N / 64;
+  const int rw = wave >> 1, cw = wave & 1;
+  const int jsteps = (rw + 1) * 2;  // A is lower triangular
+#pragma unroll
+  for (int t = 0; t < TN; ++t) acc[t] = zero16();
+  for (int js = 0; js < jsteps; ++js) {
+    v8 a = lds_frag32<T>(sA, LDT, rw * 32, js * 16, lane);
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+      acc[t] = Elem<T>::mfma32(lds_frag32<T>(sXT, LDT, (cw * TN + t) * 32, js * 16, lane), a, acc[t]);
+  }
+}
+
+// accumulators of wy_apply -> row-major 16-bit tile [64][N + 8] in LDS
+template <typename T, int N>
+FLA_DEVICE void wy_acc_to_lds(T* sOut, const f32x16* acc, int wave, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  constexpr int TN = N / 64;
+  const int rw = wave >> 1, cw = wave & 1;
+  T* op = sOut + (rw * 32 + (lane & 31)) * (N + 8) + 4 * (lane >> 5);
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      v4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (T)acc[t][4 * r4 + e];
+      *(v4*)(op + (cw * TN + t) * 32 + 8 * r4) = o;
+    }
+}
+
+// LDS tile [64][N + 8] -> global rows of pitch row_pitch, 16 bytes per lane, whole rows per wave
+template <typename T, int N>
+FLA_DEVICE void wy_store(const T* sOut, T* out, int64_t row_pitch, int L, int tid) {
+  typedef typename Elem<T>::v8 v8;
+  constexpr int CPR = N / 8, RPI = 256 / CPR;  // 16-byte columns per row, rows per pass
+  const int c8 = (tid % CPR) * 8, r = tid / CPR;
+#pragma unroll
+  for (int i = r; i < BT; i += RPI)
+    if (i < L) *(v8*)(out + (int64_t)i * row_pitch + c8) = *(const v8*)(sOut + i * (N + 8) + c8);
+}
+
+// rows [r0, r0+R) x four columns held in registers -> beta-scaled transposed 16-bit tile [column][t]
+template <typename T, int R>
+FLA_DEVICE void wy_stage_t(T* dstT, const typename Elem<T>::v4* reg, const float* sBeta, int r0, int c4) {
+  typedef T tv __attribute__((ext_vector_type(R)));
+  float b[R];
+#pragma unroll
+  for (int i = 0; i < R; i += 4) *(f32x4*)&b[i] = *(const f32x4*)&sBeta[r0 + i];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    tv o;
+#pragma unroll
+    for (int i = 0; i < R; ++i) o[i] = (T)((float)reg[i][j] * b[i]);
+    *(tv*)&dstT[(c4 + j) * LDT + r0] = o;
+  }
+}
+
+// The inversion keeps M and X = (I + M)^-1 in fp32.  Two LDS regions are
+// reused over the kernel's life so that four workgroups fit a CU:
+//   region A: k row-major -> M (fp32) -> Aw | Au (16-bit)
+//   region B: X (fp32; its always-zero upper right quadrant doubles as the
+//             scratch tile of the block merges) -> (beta k)^T -> (beta v)^T
+// k and v stay in registers from the initial load until their transposed,
+// beta-scaled tiles are written.
 template <typename T, int K, int V>
-__global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
+__global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
   constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
-  constexpr int SA_ELEMS = (BT * LDK > 2 * BT * LDT) ? BT * LDK : 2 * BT * LDT;
-  constexpr int R1_BYTES = (2 * BT * LDM * 4 > V * LDT * 2) ? 2 * BT * LDM * 4 : V * LDT * 2;
-  __shared__ __attribute__((aligned(16))) T sA[SA_ELEMS];          // k row-major, later Aw | Au
-  __shared__ __attribute__((aligned(16))) T sKbT[K * LDT];         // (beta k)^T  [k][t]
-  __shared__ __attribute__((aligned(16))) char sR1[R1_BYTES];      // M, X fp32; later (beta v)^T
-  __shared__ __attribute__((aligned(16))) float sT[32 * 36];
-  __shared__ float sBeta[BT], sGam[BT];
-  T* sK = sA;
-  T* sAw = sA;
-  T* sAu = sA + BT * LDT;
-  float* sM = (float*)sR1;
-  float* sX = sM + BT * LDM;
-  T* sVbT = (T*)sR1;
+  constexpr int KV = K > V ? K : V;
+  constexpr int RA_BYTES = (BT * LDK * 2 > 2 * BT * LDT * 2) ? BT * LDK * 2 : 2 * BT * LDT * 2;
+  constexpr int RB_BYTES = (KV * LDT * 2 > BT * LDM * 4) ? KV * LDT * 2 : BT * LDM * 4;
+  static_assert(RA_BYTES >= BT * LDM * 4 && RA_BYTES >= BT * LDK * 2, "region A holds M and the w tile");
+  static_assert(RB_BYTES >= BT * (V + 8) * 2, "region B holds the u tile");
+  __shared__ __attribute__((aligned(16))) char sRA[RA_BYTES];
+  __shared__ __attribute__((aligned(16))) char sRB[RB_BYTES];
+  __shared__ __attribute__((aligned(16))) float sBeta[BT];
+  __shared__ float sGam[BT];
+  T* sK = (T*)sRA;
+  float* sM = (float*)sRA;
+  T* sAw = (T*)sRA;
+  T* sAu = sAw + BT * LDT;
+  float* sX = (float*)sRB;
+  float* sT = sX + 32;  // rows 0..31, columns 32..63 of X
+  T* sXbT = (T*)sRB;    // (beta k)^T, later (beta v)^T
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, hh = blockIdx.y;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  // workgroups that run together take different heads of the same chunks: their rows are
+  // adjacent in memory, so the traffic spreads over all memory channels
+  const int H = p.H;
+  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+  const int hh = (int)(lin % H);
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, lin / H);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
   // ---- loads
   const int rg = tid / CG, c4 = (tid % CG) * 4;
-  v4 kreg[RPT];
-  float brow[RPT];
-#pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    int row = rg * RPT + i;
-    if (row < L) {
-      kreg[i] = *(const v4*)((const T*)p.k + ((row0 + row) * H + hh) * (int64_t)K + c4);
-      brow[i] = p.beta[(row0 + row) * H + hh];
-    } else {
-      kreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      brow[i] = 0.f;
-    }
-  }
   const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
-  v4 vreg[RPTV];
-  float bvrow[RPTV];
+  v4 kreg[RPT], vreg[RPTV];
+  {
+    const T* kp = (const T*)p.k + (row0 * H + hh) * (int64_t)K + c4;
+    const T* vp = (const T*)p.v + (row0 * H + hh) * (int64_t)V + cv4;
+    const v4 z = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
 #pragma unroll
-  for (int i = 0; i < RPTV; ++i) {
-    int row = rgv * RPTV + i;
-    if (row < L) {
-      vreg[i] = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + cv4);
-      bvrow[i] = p.beta[(row0 + row) * H + hh];
-    } else {
-      vreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      bvrow[i] = 0.f;
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      kreg[i] = row < L ? *(const v4*)(kp + (int64_t)row * H * K) : z;
+    }
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) {
+      int row = rgv * RPTV + i;
+      vreg[i] = row < L ? *(const v4*)(vp + (int64_t)row * H * V) : z;
     }
   }
   if (tid < BT) {
@@ -150,15 +205,8 @@ __global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
     sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
     sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
   }
-  // ---- k row-major and (beta k)^T to LDS
 #pragma unroll
   for (int i = 0; i < RPT; ++i) *(v4*)&sK[(rg * RPT + i) * LDK + c4] = kreg[i];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    T* dst = &sKbT[(c4 + j) * LDT + rg * RPT];
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) dst[i] = (T)((float)kreg[i][j] * brow[i]);
-  }
   __syncthreads();
 
   // ---- S = k k^T on the lower-triangular 32x32 quadrants; M = beta_i S_ij (j < i)
@@ -170,13 +218,20 @@ __global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
       for (int ks = 0; ks < K; ks += 16)
         s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
     }
-    const int j = qj * 32 + (lane & 31);
+    __syncthreads();  // k row-major fully consumed: its storage becomes M
+    if (qj <= qi) {
+      const int j = qj * 32 + (lane & 31);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = qi * 32 + c32_row(r, lane);
-      sM[i * LDM + j] = (j < i) ? sBeta[i] * s[r] : 0.f;
+      for (int r = 0; r < 16; ++r) {
+        int i = qi * 32 + c32_row(r, lane);
+        sM[i * LDM + j] = (j < i) ? sBeta[i] * s[r] : 0.f;
+      }
     }
-    for (int e = tid; e < BT * LDM; e += 256) sX[e] = 0.f;
+    // the 16x16 blocks (0,1) and (2,3) of X are read by the 32x32 merges but never written
+    for (int e = tid; e < 512; e += 256) {
+      int blk = e >> 8, i = (e >> 4) & 15, j = e & 15;
+      sX[(32 * blk + i) * LDM + 32 * blk + 16 + j] = 0.f;
+    }
   }
   __syncthreads();
 
@@ -187,28 +242,33 @@ __global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
     float x[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
+      float m[16];
+#pragma unroll
+      for (int q = 0; 4 * q < i; ++q) *(f32x4*)&m[4 * q] = *(const f32x4*)&Mb[i * LDM + 4 * q];
       float s = (i == col) ? 1.f : 0.f;
 #pragma unroll
-      for (int j = 0; j < i; ++j) s -= Mb[i * LDM + j] * x[j];
+      for (int j = 0; j < i; ++j) s -= m[j] * x[j];
       x[i] = s;
     }
 #pragma unroll
     for (int i = 0; i < 16; ++i) sX[(16 * b + i) * LDM + 16 * b + col] = x[i];
   }
   __syncthreads();
-  // ---- 32x32 diagonal blocks: X_lo = -X_bb M_lo X_aa for the block pairs (1,0) and (3,2)
+  // ---- 32x32 diagonal blocks: X_ba = -X_bb (M_ba X_aa) for the block pairs (1,0) and (3,2)
   {
-    const int pr = tid >> 7, t = tid & 127;
-    const int a0 = 32 * pr, b0 = 32 * pr + 16;
-    lds_mm<16>(sM + b0 * LDM + a0, LDM, sX + a0 * LDM + a0, LDM, sT + pr * 256, 16, 1.f, t, 128);
+    const int a0 = 32 * (wave & 1), b0 = a0 + 16;  // waves 0 and 1 take one pair each
+    if (wave < 2) lds_mm16_f32(sM + b0 * LDM + a0, LDM, sX + a0 * LDM + a0, LDM, sT + 16 * wave, LDM, 16, 1.f, lane);
     __syncthreads();
-    lds_mm<16>(sX + b0 * LDM + b0, LDM, sT + pr * 256, 16, sX + b0 * LDM + a0, LDM, -1.f, t, 128);
+    if (wave < 2) lds_mm16_f32(sX + b0 * LDM + b0, LDM, sT + 16 * wave, LDM, sX + b0 * LDM + a0, LDM, 16, -1.f, lane);
   }
   __syncthreads();
-  // ---- 64x64: X_BA = -X_BB M_BA X_AA
-  lds_mm<32>(sM + 32 * LDM, LDM, sX, LDM, sT, 36, 1.f, tid, 256);
-  __syncthreads();
-  lds_mm<32>(sX + 32 * LDM + 32, LDM, sT, 36, sX + 32 * LDM, LDM, -1.f, tid, 256);
+  // ---- 64x64: X_BA = -X_BB (M_BA X_AA), one 16x16 output tile per wave
+  {
+    const int i0 = 16 * (wave >> 1), j0 = 16 * (wave & 1);
+    lds_mm16_f32(sM + (32 + i0) * LDM, LDM, sX + j0, LDM, sT + i0 * LDM + j0, LDM, 32, 1.f, lane);
+    __syncthreads();
+    lds_mm16_f32(sX + (32 + i0) * LDM + 32, LDM, sT + j0, LDM, sX + (32 + i0) * LDM + j0, LDM, 32, -1.f, lane);
+  }
   __syncthreads();
 
   // ---- Aw, Au in 16-bit (LDS for the products, optionally global for the backward pass)
@@ -217,12 +277,16 @@ __global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
     const float gi = sGam[i];
     v8 aw[2], au[2];
 #pragma unroll
-    for (int jj = 0; jj < 16; ++jj) {
-      int j = j0 + jj;
-      float x = sX[i * LDM + j];
-      float gamma = (j <= i) ? __expf(gi - sGam[j]) : 0.f;
-      aw[jj >> 3][jj & 7] = (T)x;
-      au[jj >> 3][jj & 7] = (T)(x * gamma);
+    for (int q = 0; q < 4; ++q) {
+      f32x4 xv = *(const f32x4*)&sX[i * LDM + j0 + 4 * q];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int jj = 4 * q + e, j = j0 + jj;
+        float x = (j <= i) ? xv[e] : 0.f;  // the upper right quadrant held merge scratch
+        float gamma = (j <= i) ? __expf(gi - sGam[j]) : 0.f;
+        aw[jj >> 3][jj & 7] = (T)x;
+        au[jj >> 3][jj & 7] = (T)(x * gamma);
+      }
     }
     *(v8*)&sAw[i * LDT + j0] = aw[0];
     *(v8*)&sAw[i * LDT + j0 + 8] = aw[1];
@@ -240,57 +304,23 @@ __global__ __launch_bounds__(256) void gdr_fwd_wy_kernel(WyParams p) {
       }
     }
   }
-  __syncthreads();  // X fully consumed: its storage becomes (beta v)^T
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    T* dst = &sVbT[(cv4 + j) * LDT + rgv * RPTV];
-#pragma unroll
-    for (int i = 0; i < RPTV; ++i) dst[i] = (T)((float)vreg[i][j] * bvrow[i]);
-  }
-  // ---- w = Aw (beta k)
-  const int rw = wave >> 1, cw = wave & 1;
-  const int jsteps = (rw + 1) * 2;  // Aw, Au are lower triangular
-  {
-    constexpr int TK = K / 64;
-    f32x16 acc[TK];
-#pragma unroll
-    for (int t = 0; t < TK; ++t) acc[t] = zero16();
-    for (int js = 0; js < jsteps; ++js) {
-      v8 a = lds_frag32<T>(sAw, LDT, rw * 32, js * 16, lane);
-#pragma unroll
-      for (int t = 0; t < TK; ++t)
-        acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(sKbT, LDT, (cw * TK + t) * 32, js * 16, lane), acc[t]);
-    }
-    T* wp = (T*)p.w + (row0 * H + hh) * (int64_t)K;
-#pragma unroll
-    for (int t = 0; t < TK; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int i = rw * 32 + c32_row(r, lane);
-        if (i < L) wp[(int64_t)i * H * K + (cw * TK + t) * 32 + (lane & 31)] = (T)acc[t][r];
-      }
-  }
-  __syncthreads();  // (beta v)^T complete
-  {
-    constexpr int TV = V / 64;
-    f32x16 acc[TV];
-#pragma unroll
-    for (int t = 0; t < TV; ++t) acc[t] = zero16();
-    for (int js = 0; js < jsteps; ++js) {
-      v8 a = lds_frag32<T>(sAu, LDT, rw * 32, js * 16, lane);
-#pragma unroll
-      for (int t = 0; t < TV; ++t)
-        acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(sVbT, LDT, (cw * TV + t) * 32, js * 16, lane), acc[t]);
-    }
-    T* up = (T*)p.u + (row0 * H + hh) * (int64_t)V;
-#pragma unroll
-    for (int t = 0; t < TV; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int i = rw * 32 + c32_row(r, lane);
-        if (i < L) up[(int64_t)i * H * V + (cw * TV + t) * 32 + (lane & 31)] = (T)acc[t][r];
-      }
-  }
+  __syncthreads();  // X fully consumed: its storage becomes (beta k)^T
+  f32x16 accw[K / 64], accu[V / 64];
+  wy_stage_t<T, RPT>(sXbT, kreg, sBeta, rg * RPT, c4);
+  __syncthreads();
+  wy_apply<T, K>(sAw, sXbT, accw, wave, lane);
+  __syncthreads();  // (beta k)^T fully consumed: its storage becomes (beta v)^T
+  wy_stage_t<T, RPTV>(sXbT, vreg, sBeta, rgv * RPTV, cv4);
+  __syncthreads();
+  wy_apply<T, V>(sAu, sXbT, accu, wave, lane);
+  __syncthreads();  // both operand regions are free: they carry the output tiles to whole-row stores
+  T* sWo = (T*)sRA;
+  T* sUo = (T*)sRB;
+  wy_acc_to_lds<T, K>(sWo, accw, wave, lane);
+  wy_acc_to_lds<T, V>(sUo, accu, wave, lane);
+  __syncthreads();
+  wy_store<T, K>(sWo, (T*)p.w + (row0 * H + hh) * (int64_t)K, (int64_t)H * K, L, tid);
+  wy_store<T, V>(sUo, (T*)p.u + (row0 * H + hh) * (int64_t)V, (int64_t)H * V, L, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -621,8 +651,12 @@ __global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
   T* sP = sK;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, hh = blockIdx.y;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  // workgroups that run together take different heads of the same chunks: their rows are
+  // adjacent in memory, so the traffic spreads over all memory channels
+  const int H = p.H;
+  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+  const int hh = (int)(lin % H);
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, lin / H);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 

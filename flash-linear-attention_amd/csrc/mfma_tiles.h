@@ -29,6 +29,22 @@ FLA_DEVICE typename Elem<T>::v8 lds_frag16(const T* tile, int ld, int row0, int 
   return *(const typename Elem<T>::v8*)(tile + (row0 + (lane & 15)) * ld + k0 + 8 * (lane >> 4));
 }
 
+FLA_DEVICE f32x4 zero4();
+
+// One 16x16 fp32 tile C = sign * A B with A [16 x nk] and B [nk x 16] in LDS
+// (fp32, nk a multiple of 4), on the fp32 matrix instruction 16x16x4:
+//   A lane l holds A[l%16][l/16], B lane l holds B[l/16][l%16],
+//   C reg r of lane l is C[4*(l/16) + r][l%16].
+FLA_DEVICE void lds_mm16_f32(const float* A, int lda, const float* B, int ldb, float* C, int ldc, int nk, float sign,
+                             int lane) {
+  const int r = lane & 15, q = lane >> 4;
+  f32x4 acc = zero4();
+  for (int k0 = 0; k0 < nk; k0 += 4)
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(A[r * lda + k0 + q], B[(k0 + q) * ldb + r], acc, 0, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) C[(4 * q + i) * ldc + r] = sign * acc[i];
+}
+
 FLA_DEVICE f32x16 zero16() {
   f32x16 z;
 #pragma unroll
