@@ -70,6 +70,9 @@ struct WyParams {
   void* u;
   void* Aw;
   void* Au;
+  const void* q;  // optional: with Aqk, also emit the gated causal scores of the chunk
+  void* Aqk;      // [rows, H, 64]: scale * (q_i . k_j) e^{gamma_i - gamma_j} for j <= i, else 0
+  float scale;
   const int64_t* offsets;
   const int64_t* indices;
   int64_t T;
@@ -143,8 +146,9 @@ FLA_DEVICE void wy_stage_t(T* dstT, const typename Elem<T>::v4* reg, const float
 // The inversion keeps M and X = (I + M)^-1 in fp32.  Two LDS regions are
 // reused over the kernel's life so that four workgroups fit a CU:
 //   region A: k row-major -> M (fp32) -> Aw | Au (16-bit)
-//   region B: X (fp32; its always-zero upper right quadrant doubles as the
-//             scratch tile of the block merges) -> (beta k)^T -> (beta v)^T
+//   region B: [q row-major -> score tile] -> X (fp32; its always-zero upper
+//             right quadrant doubles as the scratch tile of the block merges)
+//             -> (beta k)^T -> (beta v)^T
 // k and v stay in registers from the initial load until their transposed,
 // beta-scaled tiles are written.
 template <typename T, int K, int V>
@@ -156,7 +160,8 @@ __global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int KV = K > V ? K : V;
   constexpr int RA_BYTES = (BT * LDK * 2 > 2 * BT * LDT * 2) ? BT * LDK * 2 : 2 * BT * LDT * 2;
-  constexpr int RB_BYTES = (KV * LDT * 2 > BT * LDM * 4) ? KV * LDT * 2 : BT * LDM * 4;
+  constexpr int RB_BYTES0 = (KV * LDT * 2 > BT * LDM * 4) ? KV * LDT * 2 : BT * LDM * 4;
+  constexpr int RB_BYTES = RB_BYTES0 > BT * LDK * 2 ? RB_BYTES0 : BT * LDK * 2;
   static_assert(RA_BYTES >= BT * LDM * 4 && RA_BYTES >= BT * LDK * 2, "region A holds M and the w tile");
   static_assert(RB_BYTES >= BT * (V + 8) * 2, "region B holds the u tile");
   __shared__ __attribute__((aligned(16))) char sRA[RA_BYTES];
@@ -185,6 +190,17 @@ __global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
   const int rg = tid / CG, c4 = (tid % CG) * 4;
   const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
   v4 kreg[RPT], vreg[RPTV];
+  const bool scores = p.q != nullptr;  // uniform over the launch
+  if (scores) {
+    const T* qp = (const T*)p.q + (row0 * H + hh) * (int64_t)K + c4;
+    T* sQ = (T*)sRB;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      v4 qv = *(const v4*)(qp + (int64_t)(row < L ? row : L - 1) * H * K);
+      *(v4*)&sQ[row * LDK + c4] = row < L ? qv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    }
+  }
   {
     const T* kp = (const T*)p.k + (row0 * H + hh) * (int64_t)K + c4;
     const T* vp = (const T*)p.v + (row0 * H + hh) * (int64_t)V + cv4;
@@ -218,7 +234,30 @@ __global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
       for (int ks = 0; ks < K; ks += 16)
         s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
     }
-    __syncthreads();  // k row-major fully consumed: its storage becomes M
+    // transposed scores (k q^T): a lane ends up with four consecutive j of one row i
+    f32x16 sq = zero16();
+    if (scores && qj <= qi) {
+      const T* sQ = (const T*)sRB;
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 16)
+        sq = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qj * 32, ks, lane), lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), sq);
+    }
+    __syncthreads();  // k (and q) row-major fully consumed: their storage becomes M (and the score tile)
+    if (scores) {
+      T* sPo = (T*)sRB;
+      const int i = qi * 32 + (lane & 31);
+      const float gi = sGam[i];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        v4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          int j = qj * 32 + 8 * r4 + 4 * (lane >> 5) + e;
+          o[e] = (T)((qj <= qi && j <= i) ? p.scale * sq[4 * r4 + e] * __expf(gi - sGam[j]) : 0.f);
+        }
+        *(v4*)&sPo[i * LDT + qj * 32 + 8 * r4 + 4 * (lane >> 5)] = o;
+      }
+    }
     if (qj <= qi) {
       const int j = qj * 32 + (lane & 31);
 #pragma unroll
@@ -226,6 +265,17 @@ __global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
         int i = qi * 32 + c32_row(r, lane);
         sM[i * LDM + j] = (j < i) ? sBeta[i] * s[r] : 0.f;
       }
+    }
+    if (scores) {
+      __syncthreads();
+      const T* sPo = (const T*)sRB;
+      T* ap = (T*)p.Aqk + (row0 * H + hh) * (int64_t)BT;
+#pragma unroll
+      for (int e = tid; e < BT * 8; e += 256) {
+        int i = e >> 3, c8 = (e & 7) * 8;
+        if (i < L) *(v8*)(ap + (int64_t)i * H * BT + c8) = *(const v8*)&sPo[i * LDT + c8];
+      }
+      __syncthreads();  // score tile stored: region B becomes X
     }
     // the 16x16 blocks (0,1) and (2,3) of X are read by the 32x32 merges but never written
     for (int e = tid; e < 512; e += 256) {
@@ -828,19 +878,21 @@ int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B, int64_
 }  // namespace
 
 extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum, void* w, void* u,
-                              void* Aw, void* Au, const int64_t* offsets, const int64_t* indices, int64_t NT,
-                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
-                              fla_stream_t stream) {
+                              void* Aw, void* Au, const void* q, void* Aqk, float scale, const int64_t* offsets,
+                              const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                              int64_t K, int64_t V, fla_stream_t stream) {
   FLA_REQUIRE(k && v && beta && w && u, FLA_E_INVALID);
+  FLA_REQUIRE((q == nullptr) == (Aqk == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au) % 16 == 0,
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au |
+               (uintptr_t)q | (uintptr_t)Aqk) % 16 == 0,
               FLA_E_ALIGNMENT);
   dim3 grid;
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, offsets, indices, T, (int)H, ntfix};
+  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, q, Aqk, scale, offsets, indices, T, (int)H, ntfix};
   if (qkv_dtype == FLA_BF16) return launch_wy<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_wy<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

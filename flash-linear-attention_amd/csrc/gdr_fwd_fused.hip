@@ -1,0 +1,479 @@
+// Fused gated-delta-rule forward for gfx950: state scan and output in one pass;
+// neither the per-chunk states nor v_new leave the chip.
+//
+// Inputs are the chunk-parallel products of fla_gdr_fwd_wy: w, u and the gated
+// causal scores Aqk, plus q, k and the chunk-local gate prefix sums gamma.
+// One workgroup of 8 waves owns one (sequence, head, 64 value columns) and walks the
+// chunks serially:
+//   waves 4-7 ("staging")  copy w, q, Aqk of chunk c+1 to LDS, transpose k and u into
+//                          time-contiguous tiles, and write the finished o tile of
+//                          chunk c-1 to global memory in whole 128-byte rows;
+//   waves 0-3 ("matrix")   each own 16 value columns of the fp32 state (all K rows, in
+//                          16x16 accumulator tiles).  The delta rule is independent per value
+//                          column, so a matrix wave never exchanges data with another:
+//                            v_new = u - e^{gamma} * (w h)
+//                            o     = s e^{gamma} * (q h) + Aqk v_new
+//                            h    <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} * v_new)
+//                          (fla/ops/common/chunk_delta_h.py:71-119, chunk_o.py:68-101).
+//                          State and v_new go from accumulators straight back into MFMA
+//                          operands: the contraction index of the LDS-side operand is
+//                          permuted to the accumulator row order instead.
+// Operand tiles are double-buffered and the two groups meet at one barrier per chunk.
+// The o tile takes the place of the u tile it was computed from (same lanes, same
+// addresses), so it needs no storage of its own.
+#include "chunk_common.h"
+
+namespace {
+
+struct GdrFusedParams {
+  const void* q;
+  const void* k;
+  const void* w;
+  const void* u;
+  const void* Aqk;
+  const float* gam;
+  const float* h0;
+  void* o;
+  float* ht;
+  const int64_t* offsets;
+  int64_t T;
+  int H, V, N;
+  float scale;
+};
+
+// LDS tiles of this kernel.  An MFMA operand fragment is two 8-byte reads per lane, served
+// 16 lanes (16 consecutive rows) at a time by the 32 four-byte banks, so all row pitches are
+// 8 bytes past a multiple of 128: sixteen consecutive rows then start in sixteen different
+// 8-byte bank pairs (measured: the 16-byte-aligned pitches K+8 / 72 cost ~7x the bank
+// conflict cycles).  Rows are therefore only 8-byte aligned, and every access is 8 bytes wide.
+constexpr int LDS_T = BT + 4;  // pitch of time-contiguous tiles and of the score tile
+
+// Time-contiguous tiles ([row][t]) are written by lanes that own four adjacent rows each,
+// i.e. with a row stride of four between neighbouring lanes; XOR-ing row bits 4-5 into the
+// 8-byte granule index spreads those writes over all banks (the fragment reads see a
+// lane-uniform term and stay conflict-free).
+FLA_DEVICE int swz_t(int row, int t) { return t ^ ((row >> 2) & 12); }
+
+// 16x16x32 operand fragment with the contraction slots in stacked-accumulator order
+// (see lds_frag16_perm); TC selects the swizzled time-contiguous addressing.
+template <typename T, bool TC>
+FLA_DEVICE typename Elem<T>::v8 frag16(const T* tile, int ld, int row0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const int row = row0 + (lane & 15), e = k0 + 4 * (lane >> 4);
+  const T* p = tile + row * ld;
+  v4 lo = *(const v4*)(p + (TC ? swz_t(row, e) : e));
+  v4 hi = *(const v4*)(p + (TC ? swz_t(row, e + 16) : e + 16));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <typename T, int K>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_fused_kernel(
+    GdrFusedParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int BV = 64;
+  constexpr int LDR = K + 4;  // pitch of the row-major w and q tiles
+  constexpr int KS = K / 32;  // 32-wide contraction slices of the state
+  constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
+  __shared__ __attribute__((aligned(16))) T sW[2][BT * LDR];     // w    [t][k]
+  __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDR];     // q    [t][k]
+  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDS_T];   // k^T  [k][t]
+  __shared__ __attribute__((aligned(16))) T sUt[2][BV * LDS_T];  // u^T  [v][t], later o^T
+  __shared__ __attribute__((aligned(16))) T sP[2][BT * LDS_T];   // Aqk  [i][j]
+  __shared__ __attribute__((aligned(16))) float sEg[2][BT];      // e^{gamma_t}
+  __shared__ __attribute__((aligned(16))) float sEd[2][BT];      // e^{gamma_last - gamma_t}
+  __shared__ float sDec[2];                                      // e^{gamma_last}
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  // wave-uniform by construction: keeps the role split and the barriers on scalar branches
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = p.H, V = p.V;
+  const int nvb = V / BV;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vb = (int)(id % nvb);
+  const int nh = (int)(id / nvb);
+  const int n = nh / H, hh = nh % H;
+  const int vbase = vb * BV;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int nchunks = (int)((sp.len + BT - 1) / BT);
+  auto chunk_len = [&](int c) {
+    int64_t rem = sp.len - (int64_t)c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+
+  if (wave >= 4) {
+    // =========================== staging waves ===========================
+    if (nchunks == 0) return;
+    const int st = tid - 256;
+    constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (w, q)
+    constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;  // k: a lane owns RPT rows x 4 columns
+    const int rg = st / CG, c4 = (st % CG) * 4;
+    const int urg = st >> 4, uc4 = (st & 15) * 4;            // u, o: a lane owns 4 rows x 4 columns
+    const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V, HB = (uint32_t)H * BT;
+    // 16-byte pieces of the w/q tiles: sixteen consecutive lanes take eight pieces of each of two
+    // consecutive rows, so that the two 8-byte halves of their LDS writes (rows 8 bytes apart in
+    // bank phase) are conflict-free.
+    auto wq_row = [&](int e) { return C8 == 16 ? 2 * (e >> 5) + ((e >> 3) & 1) : e / C8; };
+    auto wq_col = [&](int e) { return C8 == 16 ? ((e & 7) + 8 * ((e >> 4) & 1)) * 8 : (e % C8) * 8; };
+    struct Regs {
+      v8 w[NPW], q[NPW], a[2];
+      v4 k[RPT], u[4];
+      uint32_t gam;  // fp32 bits
+    };
+    // A wave issues at most one instruction every few cycles, so the steady state is kept
+    // short: byte offsets of this lane's pieces from the chunk's first row are computed once,
+    // the chunk base pointers are advanced by constant strides (loads and stores both walk the
+    // chunks in order), and only a sequence's last, short chunk takes the masked path.
+    uint32_t offw[NPW], offa[2], offk[RPT], offu[4];
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) offw[i] = 2 * ((uint32_t)wq_row(st + 256 * i) * HK + wq_col(st + 256 * i));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) offa[i] = 2 * ((uint32_t)((st + 256 * i) >> 3) * HB + ((st + 256 * i) & 7) * 8);
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) offk[i] = 2 * ((uint32_t)(rg * RPT + i) * HK + c4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) offu[i] = 2 * ((uint32_t)(urg * 4 + i) * HV + uc4);
+    const uint32_t offg = 4 * (uint32_t)lane * H;
+    const int64_t row00 = sp.bos * H + hh;
+    const char* lw = (const char*)p.w + row00 * K * 2;
+    const char* lq = (const char*)p.q + row00 * K * 2;
+    const char* lk = (const char*)p.k + row00 * K * 2;
+    const char* lu = (const char*)p.u + (row00 * V + vbase) * 2;
+    const char* la = (const char*)p.Aqk + row00 * BT * 2;
+    // The gate load is unconditional in every staging wave (a load under a branch would force
+    // the wave to drain its whole load queue at the join); without gates it reads a dummy
+    // address and the bits are masked to zero.
+    const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
+    const char* lg = p.gam ? (const char*)p.gam + row00 * 4 : lw;
+    char* so = (char*)p.o + (row00 * V + vbase) * 2;
+    const int64_t strk = (int64_t)BT * HK * 2, stru = (int64_t)BT * HV * 2, stra = (int64_t)BT * HB * 2;
+    const int64_t strg = p.gam ? (int64_t)BT * H * 4 : 0;
+    const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
+    int lc = 0;  // next chunk to load
+    auto load = [&](Regs& R) __attribute__((always_inline)) {
+      if (lc != nchunks - 1 || Llast == BT) {
+#pragma unroll
+        for (int i = 0; i < NPW; ++i) {
+          R.w[i] = *(const v8*)(lw + offw[i]);
+          R.q[i] = *(const v8*)(lq + offw[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) R.a[i] = *(const v8*)(la + offa[i]);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + offk[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) R.u[i] = *(const v4*)(lu + offu[i]);
+        R.gam = *(const uint32_t*)(lg + offg);
+      } else {
+        // rows past the end of the sequence are redirected to its last row (zeroed in write())
+        const uint32_t last = (uint32_t)Llast - 1;
+        auto cl = [&](uint32_t row) { return row < last ? row : last; };
+#pragma unroll
+        for (int i = 0; i < NPW; ++i) {
+          uint32_t e = st + 256 * i, off = 2 * (cl(wq_row(e)) * HK + wq_col(e));
+          R.w[i] = *(const v8*)(lw + off);
+          R.q[i] = *(const v8*)(lq + off);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          uint32_t e = st + 256 * i;
+          R.a[i] = *(const v8*)(la + 2 * (cl(e >> 3) * HB + (e & 7) * 8));
+        }
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + 2 * (cl(rg * RPT + i) * HK + c4));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) R.u[i] = *(const v4*)(lu + 2 * (cl(urg * 4 + i) * HV + uc4));
+        R.gam = *(const uint32_t*)(lg + 4 * cl(lane) * H);
+      }
+      lw += strk;
+      lq += strk;
+      lk += strk;
+      lu += stru;
+      la += stra;
+      lg += strg;
+      ++lc;
+    };
+    // LDS destinations of this lane (element offsets inside a tile)
+    constexpr int KV = 4;  // elements per k^T write
+    int dw[NPW], dp[2], dk[4][RPT / KV], du[4];
+#pragma unroll
+    for (int i = 0; i < NPW; ++i) dw[i] = wq_row(st + 256 * i) * LDR + wq_col(st + 256 * i);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dp[i] = ((st + 256 * i) >> 3) * LDS_T + ((st + 256 * i) & 7) * 8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int i0 = 0; i0 < RPT / KV; ++i0) dk[j][i0] = (c4 + j) * LDS_T + swz_t(c4 + j, rg * RPT + KV * i0);
+      du[j] = (uc4 + j) * LDS_T + swz_t(uc4 + j, urg * 4);
+    }
+    auto put8 = [&](T* dst, v8 x) {  // 16 bytes at an 8-byte aligned address
+      *(v4*)dst = __builtin_shufflevector(x, x, 0, 1, 2, 3);
+      *(v4*)(dst + 4) = __builtin_shufflevector(x, x, 4, 5, 6, 7);
+    };
+    int wc = 0;  // next chunk to write to LDS
+    auto write = [&](Regs& R) __attribute__((always_inline)) {
+      const int b = wc & 1;
+      if (wc == nchunks - 1 && Llast < BT) {  // zero the rows past the end of the sequence
+        const int L = Llast;
+#pragma unroll
+        for (int i = 0; i < NPW; ++i)
+          if (wq_row(st + 256 * i) >= L)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) R.w[i][j] = R.q[i][j] = (T)0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+          if (((st + 256 * i) >> 3) >= L)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) R.a[i][j] = (T)0.f;
+#pragma unroll
+        for (int i = 0; i < RPT; ++i)
+          if (rg * RPT + i >= L) R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (urg * 4 + i >= L) R.u[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      }
+#pragma unroll
+      for (int i = 0; i < NPW; ++i) {
+        put8(&sW[b][dw[i]], R.w[i]);
+        put8(&sQ[b][dw[i]], R.q[i]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) put8(&sP[b][dp[i]], R.a[i]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i0 = 0; i0 < RPT / KV; ++i0) {
+          v4 kc = {R.k[4 * i0][j], R.k[4 * i0 + 1][j], R.k[4 * i0 + 2][j], R.k[4 * i0 + 3][j]};
+          *(v4*)&sKt[b][dk[j][i0]] = kc;
+        }
+        v4 uc = {R.u[0][j], R.u[1][j], R.u[2][j], R.u[3][j]};
+        *(v4*)&sUt[b][du[j]] = uc;
+      }
+      if (wave == 4) {
+        // lanes past the end of a short chunk carry the last row's gate
+        const float gam = __uint_as_float(R.gam & gmask);
+        const float glast = __uint_as_float(__builtin_amdgcn_readlane(R.gam & gmask, 63));
+        sEg[b][lane] = __expf(gam);
+        sEd[b][lane] = __expf(glast - gam);
+        if (lane == 0) sDec[b] = __expf(glast);
+      }
+      ++wc;
+    };
+    // The matrix waves left o^T of a chunk where u^T of that chunk was; each lane reads back
+    // exactly the addresses it writes in write(), so the tile can be refilled right after.
+    int oc = 0;  // next chunk whose output is stored
+    auto store_o = [&]() __attribute__((always_inline)) {
+      const int b = oc & 1;
+      v4 x[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) x[j] = *(const v4*)&sUt[b][du[j]];
+      if (oc != nchunks - 1 || Llast == BT) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(v4*)(so + offu[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (urg * 4 + i < Llast) *(v4*)(so + offu[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+      }
+      so += stru;
+      ++oc;
+    };
+    // Two register sets: a chunk is loaded three iterations before the matrix waves use it
+    // (two before it is written to LDS), so the loads have a whole chunk period to land.
+    Regs R0, R1;
+    load(R0);
+    if (nchunks > 1) load(R1);
+    write(R0);
+    if (nchunks > 2) load(R0);
+    lds_barrier();
+    // iteration c (the matrix waves work on chunk c): R holds chunk c+1
+    auto iter = [&](int c, Regs& R) __attribute__((always_inline)) {
+      if (c >= 1) store_o();
+      if (c + 1 < nchunks) {
+        write(R);
+        if (c + 3 < nchunks) load(R);
+      }
+      lds_barrier();
+    };
+    for (int c = 0; c < nchunks; c += 2) {
+      iter(c, R1);
+      if (c + 1 < nchunks) iter(c + 1, R0);
+    }
+    store_o();
+  } else {
+    // =========================== matrix waves ===========================
+    const int cb = 16 * wave;  // first of this wave's 16 columns within the slab
+    const int c = lane & 15, g = lane >> 4;
+    f32x4 acc[KT];  // acc[kt][r] = h[16 kt + 4 g + r][cb + c]
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      acc[kt] = zero4();
+      if (p.h0) {
+        const float* h0p = p.h0 + (int64_t)nh * K * V + vbase + cb + c;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[kt][r] = h0p[(int64_t)(16 * kt + 4 * g + r) * V];
+      }
+    }
+    if (nchunks > 0) {
+      lds_barrier();
+      for (int ci = 0; ci < nchunks; ++ci) {
+        const int b = ci & 1;
+        const T* W = sW[b];
+        const T* Q = sQ[b];
+        const T* Kt = sKt[b];
+        const T* P = sP[b];
+        const int urow = cb + c;
+        T* ut = &sUt[b][urow * LDS_T];
+        // LDS reads are issued a group ahead of the MFMAs that consume them; the scheduling
+        // fences keep the compiler from sinking them back next to their use.
+        v8 fa[2 * KS], fb[2 * KS];
+        auto load_wq = [&](int tt, v8* f) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            f[ks] = frag16<T, false>(W, LDR, 16 * tt, 32 * ks, lane);
+            f[KS + ks] = frag16<T, false>(Q, LDR, 16 * tt, 32 * ks, lane);
+          }
+        };
+        auto load_kt = [&](int half, v8* f) {
+#pragma unroll
+          for (int i = 0; i < KT / 2; ++i)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16<T, true>(Kt, LDS_T, 16 * (half * (KT / 2) + i), 32 * s, lane);
+        };
+        load_wq(0, fa);
+        load_wq(1, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        // the state as the other MFMA operand: two stacked accumulators per 32-slice
+        v8 hb[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            hb[ks][e] = (T)acc[2 * ks][e];
+            hb[ks][4 + e] = (T)acc[2 * ks + 1][e];
+          }
+        f32x4 d[4], oq[4];
+        auto mm_wq = [&](int tt, const v8* f) {
+          d[tt] = zero4();
+          oq[tt] = zero4();
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            d[tt] = Elem<T>::mfma16(f[ks], hb[ks], d[tt]);
+            oq[tt] = Elem<T>::mfma16(f[KS + ks], hb[ks], oq[tt]);
+          }
+        };
+        mm_wq(0, fa);
+        __builtin_amdgcn_sched_barrier(0);
+        load_wq(2, fa);
+        __builtin_amdgcn_sched_barrier(0);
+        mm_wq(1, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        load_wq(3, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        mm_wq(2, fa);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 eg[4], ed[4];
+        v4 uu[4];
+        v8 fp[6];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          eg[tt] = *(const f32x4*)&sEg[b][16 * tt + 4 * g];
+          ed[tt] = *(const f32x4*)&sEd[b][16 * tt + 4 * g];
+          uu[tt] = *(const v4*)(ut + swz_t(urow, 16 * tt + 4 * g));
+        }
+        const float dec = sDec[b];
+        fp[0] = frag16<T, false>(P, LDS_T, 0, 0, lane);
+        fp[1] = frag16<T, false>(P, LDS_T, 16, 0, lane);
+        fp[2] = frag16<T, false>(P, LDS_T, 32, 0, lane);
+        fp[3] = frag16<T, false>(P, LDS_T, 32, 32, lane);
+        fp[4] = frag16<T, false>(P, LDS_T, 48, 0, lane);
+        fp[5] = frag16<T, false>(P, LDS_T, 48, 32, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        mm_wq(3, fb);
+        __builtin_amdgcn_sched_barrier(0);
+        load_kt(0, fa);
+        __builtin_amdgcn_sched_barrier(0);
+        v8 vnb[2], vsb[2];  // v_new and its decayed copy as operands contracting over time
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float vn = (float)uu[tt][r] - d[tt][r] * eg[tt][r];
+            vnb[tt >> 1][(tt & 1) * 4 + r] = (T)vn;
+            vsb[tt >> 1][(tt & 1) * 4 + r] = (T)(vn * ed[tt][r]);
+            oq[tt][r] *= p.scale * eg[tt][r];
+          }
+        }
+        // Aqk is lower triangular: row tiles 0 and 1 only meet the first 32 columns
+        oq[0] = Elem<T>::mfma16(fp[0], vnb[0], oq[0]);
+        oq[1] = Elem<T>::mfma16(fp[1], vnb[0], oq[1]);
+        oq[2] = Elem<T>::mfma16(fp[2], vnb[0], oq[2]);
+        oq[3] = Elem<T>::mfma16(fp[4], vnb[0], oq[3]);
+        oq[2] = Elem<T>::mfma16(fp[3], vnb[1], oq[2]);
+        oq[3] = Elem<T>::mfma16(fp[5], vnb[1], oq[3]);
+        __builtin_amdgcn_sched_barrier(0);
+        load_kt(1, fb);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[kt][r] *= dec;
+#pragma unroll
+        for (int i = 0; i < KT / 2; ++i)
+#pragma unroll
+          for (int s = 0; s < 2; ++s) acc[i] = Elem<T>::mfma16(fa[2 * i + s], vsb[s], acc[i]);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          v4 ov;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) ov[r] = (T)oq[tt][r];
+          *(v4*)(ut + swz_t(urow, 16 * tt + 4 * g)) = ov;
+        }
+#pragma unroll
+        for (int i = 0; i < KT / 2; ++i)
+#pragma unroll
+          for (int s = 0; s < 2; ++s) acc[KT / 2 + i] = Elem<T>::mfma16(fb[2 * i + s], vsb[s], acc[KT / 2 + i]);
+        lds_barrier();
+      }
+    }
+    if (p.ht) {
+      float* htp = p.ht + (int64_t)nh * K * V + vbase + cb + c;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) htp[(int64_t)(16 * kt + 4 * g + r) * V] = acc[kt][r];
+    }
+  }
+}
+
+template <typename T>
+int launch_fused(const GdrFusedParams& p, int K, hipStream_t st) {
+  const int64_t nblk = (int64_t)p.N * p.H * (p.V / 64);
+  FLA_REQUIRE(nblk <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  if (nblk == 0) return FLA_OK;
+  dim3 grid((unsigned)nblk), block(512);
+  if (K == 64) hipLaunchKernelGGL((gdr_fwd_fused_kernel<T, 64>), grid, block, 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_fused_kernel<T, 128>), grid, block, 0, st, p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+}  // namespace
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
+                                                    const void* Aqk, const float* g_cumsum, const float* h0, void* o,
+                                                    float* ht, const int64_t* offsets, int qkv_dtype, int64_t B,
+                                                    int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                                    fla_stream_t stream) {
+  FLA_REQUIRE(q && k && w && u && Aqk && o, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(offsets ? B == 1 : N == B, FLA_E_INVALID);
+  FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aqk | (uintptr_t)o) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  GdrFusedParams p{q, k, w, u, Aqk, g_cumsum, h0, o, ht, offsets, T, (int)H, (int)V, (int)N, scale};
+  if (qkv_dtype == FLA_BF16) return launch_fused<bf16>(p, (int)K, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_fused<f16>(p, (int)K, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}

@@ -29,6 +29,19 @@ FLA_DEVICE typename Elem<T>::v8 lds_frag16(const T* tile, int ld, int row0, int 
   return *(const typename Elem<T>::v8*)(tile + (row0 + (lane & 15)) * ld + k0 + 8 * (lane >> 4));
 }
 
+// 16x16x32 operand with the contraction index permuted inside the 32-slice: slot
+// (g = lane/16, e) holds k0 + 16*(e/4) + 4*g + e%4.  This is the order in which two
+// stacked 16x16 accumulators (rows k0.. and k0+16..) enumerate their rows, so a pair
+// of accumulators converted to 16-bit is the other operand without a shuffle.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 lds_frag16_perm(const T* tile, int ld, int row0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const T* p = tile + (row0 + (lane & 15)) * ld + k0 + 4 * (lane >> 4);
+  v4 lo = *(const v4*)p;
+  v4 hi = *(const v4*)(p + 16);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 FLA_DEVICE f32x4 zero4();
 
 // One 16x16 fp32 tile C = sign * A B with A [16 x nk] and B [nk x 16] in LDS

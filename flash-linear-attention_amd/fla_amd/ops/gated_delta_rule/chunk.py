@@ -2,8 +2,10 @@
 (``fla/ops/gated_delta_rule/chunk.py:258-363``).
 
 Forward pipeline on the device (chunk size 64): ``fla_chunk_local_cumsum`` (gate)
--> ``fla_gdr_fwd_wy`` (KK^T, block inverse, w/u) -> ``fla_chunk_gated_delta_rule_fwd_h``
-(state scan, v_new) -> ``fla_chunk_fwd_o``.
+-> ``fla_gdr_fwd_wy`` (KK^T, block inverse, w/u, gated causal q k^T scores)
+-> ``fla_chunk_gated_delta_rule_fwd_fused`` (state scan and output in one launch).
+The backward recomputes w, u, the per-chunk states and v_new with
+``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
 """
 from typing import Optional, Tuple
 
@@ -13,7 +15,7 @@ import torch.nn.functional as F
 from ... import _backend as be
 from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
                       resolve_offsets)
-from ..common.chunk_delta_h import chunk_gated_delta_rule_fwd_h
+from ..common.chunk_delta_h import chunk_gated_delta_rule_fwd_fused, chunk_gated_delta_rule_fwd_h
 from ..common.chunk_o import chunk_fwd_o
 from ..utils.cumsum import chunk_local_cumsum
 from .wy_fast import fwd_prepare_wy_repr
@@ -28,9 +30,10 @@ def _round64(d: int) -> int:
 
 def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
                                offsets=None, indices=None, head_first=True, chunk_size=64,
-                               *, plan: Optional[VarlenPlan] = None, store_A: bool = True):
+                               *, plan: Optional[VarlenPlan] = None, store_A: bool = True, fused: bool = True):
     """Reference-shaped forward (``fla/ops/gated_delta_rule/chunk.py:20-73``): returns
-    ``(g_cumsum, o, Aw, Au, final_state)``."""
+    ``(g_cumsum, o, Aw, Au, final_state)``.  ``fused=False`` runs the state scan and the
+    output stage as the reference's two separate steps."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd: seq-first, chunk size 64 only")
     if offsets is not None and plan is None:
@@ -39,6 +42,12 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     idx = None if plan is None else plan.indices
     co = None if plan is None else plan.chunk_offsets
     g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
+    if fused:
+        w, u, Aw, Au, Aqk = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False,
+                                                chunk_size=BT, store_A=store_A, q=q, scale=scale)
+        o, final_state = chunk_gated_delta_rule_fwd_fused(q, k, w, u, Aqk, g, scale, initial_state,
+                                                          output_final_state, offsets=offs)
+        return g, o, Aw, Au, final_state
     w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
                                        store_A=store_A)
     h, v_new, final_state = chunk_gated_delta_rule_fwd_h(

@@ -164,7 +164,10 @@ int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const v
  * :111-236; :379-426 kernel :250-317): Aw = (I + strict_lower(diag(beta) K K^T))^-1,
  * Au = Aw * exp(g_i - g_j), w = Aw (beta K) [B,T,H,K], u = Au (beta V) [B,T,H,V].
  * Aw, Au (optional outputs, [B,T,H,64] in the q/k/v dtype) are what the
- * reference saves for backward.
+ * reference saves for backward.  With q and Aqk (both or neither) the same
+ * launch also emits the gated causal scores of chunk_fwd_o
+ * (fla/ops/common/chunk_o.py:86-97): Aqk[i,j] = scale (q_i . k_j) exp(g_i - g_j)
+ * for j <= i, else 0, [B,T,H,64] in the q/k/v dtype.
  *
  * fla_chunk_gated_delta_rule_fwd_h: state scan, replaces
  * chunk_gated_delta_rule_fwd_h (fla/ops/common/chunk_delta_h.py:248-320,
@@ -176,7 +179,7 @@ int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const v
  * FLA_H_FRAGMENT; v is v_new for the delta rule.
  * ---------------------------------------------------------------------- */
 int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum,
-                   void* w, void* u, void* Aw, void* Au,
+                   void* w, void* u, void* Aw, void* Au, const void* q, void* Aqk, float scale,
                    const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, fla_stream_t stream);
 
@@ -190,6 +193,19 @@ int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, const void* u
 int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_cumsum, const void* h, void* o,
                     const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream);
+
+/* fla_chunk_gated_delta_rule_fwd_fused: state scan and output in one launch;
+ * replaces chunk_gated_delta_rule_fwd_h followed by chunk_fwd_o in
+ * chunk_gated_delta_rule_fwd (fla/ops/gated_delta_rule/chunk.py:47-72; kernels
+ * fla/ops/common/chunk_delta_h.py:27-119 and chunk_o.py:23-101) when neither the
+ * per-chunk states nor v_new are wanted.  w, u and Aqk come from
+ * fla_gdr_fwd_wy (called with q, scale).  o [B,T,H,V] in the q/k/v dtype;
+ * h0, ht fp32 [N,H,K,V] or NULL.  K in {64,128}, V a multiple of 64. */
+int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
+                                         const void* Aqk, const float* g_cumsum, const float* h0,
+                                         void* o, float* ht, const int64_t* offsets, int qkv_dtype,
+                                         int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                         float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Chunked GLA backward (chunk size 64), replaces chunk_gla_bwd

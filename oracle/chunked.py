@@ -96,6 +96,7 @@ def chunked_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, c
     gam = torch.zeros_like(g)
     Aw = torch.zeros(B, T, H, BT, dtype=dtype)
     Au = torch.zeros(B, T, H, BT, dtype=dtype)
+    Aqk = torch.zeros(B, T, H, BT, dtype=dtype)
     w = torch.zeros_like(k)
     u = torch.zeros_like(v)
     v_new = torch.zeros_like(v)
@@ -129,6 +130,7 @@ def chunked_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, c
             vn = uc - torch.einsum('ihk,hkv->ihv', wc * eg[..., None], h)
             v_new[b, s:e] = vn
             P = torch.einsum('ihk,jhk->hij', qc, kc) * Gam       # tril by Gam's mask
+            Aqk[b, s:e, :, :L] = scale * P.permute(1, 0, 2)
             o[b, s:e] = scale * (eg[..., None] * torch.einsum('ihk,hkv->ihv', qc, h)
                                  + torch.einsum('hij,jhv->ihv', P, vn))
             glast = gc[-1]                                      # [H]
@@ -140,5 +142,5 @@ def chunked_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, c
         h_all = torch.stack(hs, 0).reshape(B, NT, H, K, V) if hs else torch.zeros(B, 0, H, K, V)
     else:
         h_all = torch.stack(hs, 0)[None]
-    return dict(g_cumsum=gam, Aw=Aw, Au=Au, w=w, u=u, h=h_all, v_new=v_new, o=o,
+    return dict(g_cumsum=gam, Aw=Aw, Au=Au, Aqk=Aqk, w=w, u=u, h=h_all, v_new=v_new, o=o,
                 ht=torch.stack(finals, 0))

@@ -54,6 +54,36 @@ def test_gdr_kernel_by_kernel(device):
     o = chunk_fwd_o(dev(q), dev(k), v_new2, hf, gc, 128 ** -0.5, head_first=False)
     torch.cuda.synchronize()
     assert_close("o", ref['o'], o, TOL_O)
+    # the fused scan + output launch, fed by the WY launch that also emits the gated scores
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_fused
+    w2, u2, Aw2, Au2, Aqk = fwd_prepare_wy_repr(dev(k), dev(v), dev(beta), gc, head_first=False, q=dev(q),
+                                                scale=128 ** -0.5)
+    torch.cuda.synchronize()
+    assert torch.equal(w, w2) and torch.equal(u, u2) and torch.equal(Aw, Aw2) and torch.equal(Au, Au2)
+    assert_close("Aqk", ref['Aqk'], Aqk, 5e-3)
+    o2, ht2 = chunk_gated_delta_rule_fwd_fused(dev(q), dev(k), w2, u2, Aqk, gc, 128 ** -0.5, dev(h0), True)
+    torch.cuda.synchronize()
+    assert_close("o fused", ref['o'], o2, TOL_O)
+    assert_close("ht fused", ref['ht'], ht2, TOL_HT)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_gdr_unfused_pipeline(device, varlen):
+    """The reference's two-step form (state scan, then output stage) stays available."""
+    from fla_amd.ops.gated_delta_rule.chunk import chunk_gated_delta_rule_fwd
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    T, N = 500, 3
+    offs = random_offsets(T, N, torch.Generator().manual_seed(5), min_len=1) if varlen else None
+    q, k, v, g, beta, h0 = gdr_inputs(1 if varlen else 2, T, 2, 128, 128, seed=31, N=N if varlen else None)
+    dev = lambda x: None if x is None else x.to(device)
+    print(f"gdr unfused varlen={varlen}", flush=True)
+    _, o, _, _, ht = chunk_gated_delta_rule_fwd(dev(q), dev(k), dev(v), dev(g), dev(beta), 128 ** -0.5, dev(h0), True,
+                                                offsets=dev(offs), head_first=False, fused=False)
+    torch.cuda.synchronize()
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
 
 
 # reference ladder: tests/ops/test_gated_delta.py:220-294 (T in {7,63,286,300,1000}, scale in {1, 0.1})
