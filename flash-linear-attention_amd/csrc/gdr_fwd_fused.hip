@@ -41,28 +41,40 @@ struct GdrFusedParams {
   float scale;
 };
 
-// LDS tiles of this kernel.  An MFMA operand fragment is two 8-byte reads per lane, served
-// 16 lanes (16 consecutive rows) at a time by the 32 four-byte banks, so all row pitches are
-// 8 bytes past a multiple of 128: sixteen consecutive rows then start in sixteen different
-// 8-byte bank pairs (measured: the 16-byte-aligned pitches K+8 / 72 cost ~7x the bank
-// conflict cycles).  Rows are therefore only 8-byte aligned, and every access is 8 bytes wide.
-constexpr int LDS_T = BT + 4;  // pitch of time-contiguous tiles and of the score tile
-
-// Time-contiguous tiles ([row][t]) are written by lanes that own four adjacent rows each,
-// i.e. with a row stride of four between neighbouring lanes; XOR-ing row bits 4-5 into the
-// 8-byte granule index spreads those writes over all banks (the fragment reads see a
-// lane-uniform term and stay conflict-free).
-FLA_DEVICE int swz_t(int row, int t) { return t ^ ((row >> 2) & 12); }
-
-// 16x16x32 operand fragment with the contraction slots in stacked-accumulator order
-// (see lds_frag16_perm); TC selects the swizzled time-contiguous addressing.
-template <typename T, bool TC>
+// LDS tiles of this kernel.  Measured on gfx950 (one wave per SIMD): LDS reads peak at
+// 256 B/clk per CU, writes near 80 B/clk.  For the access shape of an MFMA operand
+// fragment (16 consecutive rows x 4 column groups per wave) the full read rate is reached
+// by 8-byte reads whose groups are 8 bytes apart and whose row pitch is 16 bytes past a
+// multiple of 256 (or 144 bytes); the same bytes fetched as one 16-byte read, or as a
+// paired two-address read, run at half that rate.  A fragment is therefore two separate
+// 8-byte reads (volatile, so that they are not fused into a paired read): accumulator rows
+// {4g..4g+3} and {16+4g..16+4g+3} of a 32-slice, the order in which stacked 16x16
+// accumulators fed straight back as the other operand enumerate their rows.
+template <typename T>
 FLA_DEVICE typename Elem<T>::v8 frag16(const T* tile, int ld, int row0, int k0, int lane) {
   typedef typename Elem<T>::v4 v4;
-  const int row = row0 + (lane & 15), e = k0 + 4 * (lane >> 4);
-  const T* p = tile + row * ld;
-  v4 lo = *(const v4*)(p + (TC ? swz_t(row, e) : e));
-  v4 hi = *(const v4*)(p + (TC ? swz_t(row, e + 16) : e + 16));
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + (row0 + (lane & 15)) * ld + k0 + 4 * (lane >> 4);
+  v4 lo = *(lds_v4*)p;
+  v4 hi = *(lds_v4*)(p + 16);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Time-contiguous tiles ([row][t], pitch LDT = 144 bytes) are written by lanes that own
+// four adjacent rows each, i.e. with a row stride of four between neighbouring lanes
+// (64 bytes modulo 256: unswizzled, such writes run 5x slower); XOR-ing row bits 4-5
+// into the 16-byte slot index spreads them over all banks.  A fragment read covers the 16
+// rows of one 16-row tile and sees a lane-uniform term.
+FLA_DEVICE int swz_t(int row, int t) { return t ^ ((row >> 1) & 24); }
+
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag16_t(const T* tile, int row0, int t0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const int row = row0 + (lane & 15), t = t0 + 4 * (lane >> 4);
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + row * LDT;
+  v4 lo = *(lds_v4*)(p + swz_t(row, t));
+  v4 hi = *(lds_v4*)(p + swz_t(row, t + 16));
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
@@ -72,14 +84,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int BV = 64;
-  constexpr int LDR = K + 4;  // pitch of the row-major w and q tiles
+  constexpr int LDR = K + 8;  // pitch of the row-major w and q tiles
   constexpr int KS = K / 32;  // 32-wide contraction slices of the state
   constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
   __shared__ __attribute__((aligned(16))) T sW[2][BT * LDR];     // w    [t][k]
   __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDR];     // q    [t][k]
-  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDS_T];   // k^T  [k][t]
-  __shared__ __attribute__((aligned(16))) T sUt[2][BV * LDS_T];  // u^T  [v][t], later o^T
-  __shared__ __attribute__((aligned(16))) T sP[2][BT * LDS_T];   // Aqk  [i][j]
+  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDT];   // k^T  [k][t]
+  __shared__ __attribute__((aligned(16))) T sUt[2][BV * LDT];  // u^T  [v][t], later o^T
+  __shared__ __attribute__((aligned(16))) T sP[2][BT * LDT];   // Aqk  [i][j]
   __shared__ __attribute__((aligned(16))) float sEg[2][BT];      // e^{gamma_t}
   __shared__ __attribute__((aligned(16))) float sEd[2][BT];      // e^{gamma_last - gamma_t}
   __shared__ float sDec[2];                                      // e^{gamma_last}
@@ -110,11 +122,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int rg = st / CG, c4 = (st % CG) * 4;
     const int urg = st >> 4, uc4 = (st & 15) * 4;            // u, o: a lane owns 4 rows x 4 columns
     const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V, HB = (uint32_t)H * BT;
-    // 16-byte pieces of the w/q tiles: sixteen consecutive lanes take eight pieces of each of two
-    // consecutive rows, so that the two 8-byte halves of their LDS writes (rows 8 bytes apart in
-    // bank phase) are conflict-free.
-    auto wq_row = [&](int e) { return C8 == 16 ? 2 * (e >> 5) + ((e >> 3) & 1) : e / C8; };
-    auto wq_col = [&](int e) { return C8 == 16 ? ((e & 7) + 8 * ((e >> 4) & 1)) * 8 : (e % C8) * 8; };
+    // 16-byte pieces of the w/q tiles: row and first column of piece e
+    auto wq_row = [&](int e) { return e / C8; };
+    auto wq_col = [&](int e) { return (e % C8) * 8; };
     struct Regs {
       v8 w[NPW], q[NPW], a[2];
       v4 k[RPT], u[4];
@@ -194,22 +204,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       ++lc;
     };
     // LDS destinations of this lane (element offsets inside a tile)
-    constexpr int KV = 4;  // elements per k^T write
+    constexpr int KV = RPT == 8 ? 8 : 4;  // elements per k^T write
     int dw[NPW], dp[2], dk[4][RPT / KV], du[4];
 #pragma unroll
     for (int i = 0; i < NPW; ++i) dw[i] = wq_row(st + 256 * i) * LDR + wq_col(st + 256 * i);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dp[i] = ((st + 256 * i) >> 3) * LDS_T + ((st + 256 * i) & 7) * 8;
+    for (int i = 0; i < 2; ++i) dp[i] = ((st + 256 * i) >> 3) * LDT + ((st + 256 * i) & 7) * 8;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int i0 = 0; i0 < RPT / KV; ++i0) dk[j][i0] = (c4 + j) * LDS_T + swz_t(c4 + j, rg * RPT + KV * i0);
-      du[j] = (uc4 + j) * LDS_T + swz_t(uc4 + j, urg * 4);
+      for (int i0 = 0; i0 < RPT / KV; ++i0) dk[j][i0] = (c4 + j) * LDT + swz_t(c4 + j, rg * RPT + KV * i0);
+      du[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
     }
-    auto put8 = [&](T* dst, v8 x) {  // 16 bytes at an 8-byte aligned address
-      *(v4*)dst = __builtin_shufflevector(x, x, 0, 1, 2, 3);
-      *(v4*)(dst + 4) = __builtin_shufflevector(x, x, 4, 5, 6, 7);
-    };
+    auto put8 = [&](T* dst, v8 x) { *(v8*)dst = x; };
     int wc = 0;  // next chunk to write to LDS
     auto write = [&](Regs& R) __attribute__((always_inline)) {
       const int b = wc & 1;
@@ -243,8 +250,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
         for (int i0 = 0; i0 < RPT / KV; ++i0) {
-          v4 kc = {R.k[4 * i0][j], R.k[4 * i0 + 1][j], R.k[4 * i0 + 2][j], R.k[4 * i0 + 3][j]};
-          *(v4*)&sKt[b][dk[j][i0]] = kc;
+          if constexpr (KV == 8) {
+            v4 lo = {R.k[0][j], R.k[1][j], R.k[2][j], R.k[3][j]};
+            v4 hi = {R.k[4][j], R.k[5][j], R.k[6][j], R.k[7][j]};
+            *(v8*)&sKt[b][dk[j][i0]] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          } else {
+            v4 kc = {R.k[4 * i0][j], R.k[4 * i0 + 1][j], R.k[4 * i0 + 2][j], R.k[4 * i0 + 3][j]};
+            *(v4*)&sKt[b][dk[j][i0]] = kc;
+          }
         }
         v4 uc = {R.u[0][j], R.u[1][j], R.u[2][j], R.u[3][j]};
         *(v4*)&sUt[b][du[j]] = uc;
@@ -323,22 +336,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const T* Kt = sKt[b];
         const T* P = sP[b];
         const int urow = cb + c;
-        T* ut = &sUt[b][urow * LDS_T];
+        T* ut = &sUt[b][urow * LDT];
         // LDS reads are issued a group ahead of the MFMAs that consume them; the scheduling
         // fences keep the compiler from sinking them back next to their use.
         v8 fa[2 * KS], fb[2 * KS];
         auto load_wq = [&](int tt, v8* f) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            f[ks] = frag16<T, false>(W, LDR, 16 * tt, 32 * ks, lane);
-            f[KS + ks] = frag16<T, false>(Q, LDR, 16 * tt, 32 * ks, lane);
+            f[ks] = frag16<T>(W, LDR, 16 * tt, 32 * ks, lane);
+            f[KS + ks] = frag16<T>(Q, LDR, 16 * tt, 32 * ks, lane);
           }
         };
         auto load_kt = [&](int half, v8* f) {
 #pragma unroll
           for (int i = 0; i < KT / 2; ++i)
 #pragma unroll
-            for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16<T, true>(Kt, LDS_T, 16 * (half * (KT / 2) + i), 32 * s, lane);
+            for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16_t<T>(Kt, 16 * (half * (KT / 2) + i), 32 * s, lane);
         };
         load_wq(0, fa);
         load_wq(1, fb);
@@ -382,12 +395,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           uu[tt] = *(const v4*)(ut + swz_t(urow, 16 * tt + 4 * g));
         }
         const float dec = sDec[b];
-        fp[0] = frag16<T, false>(P, LDS_T, 0, 0, lane);
-        fp[1] = frag16<T, false>(P, LDS_T, 16, 0, lane);
-        fp[2] = frag16<T, false>(P, LDS_T, 32, 0, lane);
-        fp[3] = frag16<T, false>(P, LDS_T, 32, 32, lane);
-        fp[4] = frag16<T, false>(P, LDS_T, 48, 0, lane);
-        fp[5] = frag16<T, false>(P, LDS_T, 48, 32, lane);
+        fp[0] = frag16<T>(P, LDT, 0, 0, lane);
+        fp[1] = frag16<T>(P, LDT, 16, 0, lane);
+        fp[2] = frag16<T>(P, LDT, 32, 0, lane);
+        fp[3] = frag16<T>(P, LDT, 32, 32, lane);
+        fp[4] = frag16<T>(P, LDT, 48, 0, lane);
+        fp[5] = frag16<T>(P, LDT, 48, 32, lane);
         __builtin_amdgcn_sched_barrier(0);
         mm_wq(3, fb);
         __builtin_amdgcn_sched_barrier(0);
