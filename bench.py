@@ -13,8 +13,9 @@ returned), inputs resident in HBM.  Prints ONE JSON line:
                    here with HIP events on the launch stream
 * cpu_baseline     the oracle's fp32 naive recurrence timed on the host cores on
                    a bounded sample of the same workload
-* extra            the other measured rows (chunk_gated_delta_rule forward on
-                   config 2 when built, the T=1 decode steps of config 3)
+* extra            the other measured rows: the T=1 decode steps of config 3,
+                   chunk_gated_delta_rule forward on config 2, forward + backward
+                   of both chunk operators on config 4
 """
 import argparse
 import json
@@ -183,6 +184,78 @@ def bench_decode(device, steps=1000):
     return out
 
 
+def bench_gdr(device, steps=20):
+    """chunk_gated_delta_rule forward: BASELINE config 2 (packed, 12 sequences, 32768 tokens)
+    and the fixed-length shape B=8, T=4096 of the headline metric."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    torch.manual_seed(0)
+    T, H, K, V, N = 32768, 16, 128, 128, 12
+    lens = torch.randint(256, 6001, (N,)).double()
+    lens = (lens / lens.sum() * T).round().long()
+    lens[-1] += T - lens.sum()
+    offs = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]).to(device)
+    q = torch.randn(1, T, H, K, device=device).bfloat16()
+    k = F.normalize(torch.randn(1, T, H, K, device=device), dim=-1).bfloat16()
+    v = torch.randn(1, T, H, V, device=device).bfloat16()
+    g = F.logsigmoid(torch.randn(1, T, H, device=device))
+    beta = torch.randn(1, T, H, device=device).sigmoid()
+    # q, k, v, o in 16 bit + g, beta fp32 + the final states: what the operator must move
+    floor = 4 * T * H * K * 2 + 2 * T * H * 4
+    out = {}
+    us = event_avg_us(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs,
+                                                     head_first=False), steps)
+    out["config2_varlen"] = {"us": round(us, 1), "tokens_per_s": round(T / (us * 1e-6), 1),
+                             "sequence_lengths": lens.tolist(),
+                             "operator_floor_bytes": floor + N * H * K * V * 4,
+                             "frac_of_hbm_peak": round((floor + N * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    B, T2 = 8, 4096
+    q, k, v = (x.view(B, T2, H, -1) for x in (q, k, v))
+    g, beta = g.view(B, T2, H), beta.view(B, T2, H)
+    us = event_avg_us(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
+                      steps)
+    out["B8_T4096"] = {"us": round(us, 1), "tokens_per_s": round(B * T2 / (us * 1e-6), 1),
+                       "operator_floor_bytes": floor + B * H * K * V * 4,
+                       "frac_of_hbm_peak": round((floor + B * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
+
+
+def bench_backward(device, steps=10):
+    """BASELINE config 4: forward + backward of both chunk operators, B=4, T=4096, H=16, K=V=128."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_amd.ops.gla import chunk_gla
+    torch.manual_seed(0)
+    B, T, H, K, V = 4, 4096, 16, 128, 128
+    mk = lambda *sh: torch.randn(*sh, device=device)
+    q, v = mk(B, T, H, K).bfloat16().requires_grad_(), mk(B, T, H, V).bfloat16().requires_grad_()
+    h0 = (mk(B, H, K, V) * 0.1).requires_grad_()
+    do, dht = mk(B, T, H, V).bfloat16(), mk(B, H, K, V) * 0.1
+    out = {}
+    k = mk(B, T, H, K).bfloat16().requires_grad_()
+    gk = (F.logsigmoid(mk(B, T, H, K)) / 16).requires_grad_()
+
+    def gla_step():
+        o, ht = chunk_gla(q, k, v, gk, initial_state=h0, output_final_state=True, head_first=False)
+        torch.autograd.backward((o, ht), (do, dht))
+
+    kn = F.normalize(mk(B, T, H, K), dim=-1).bfloat16().requires_grad_()
+    g = F.logsigmoid(mk(B, T, H)).requires_grad_()
+    beta = mk(B, T, H).sigmoid().requires_grad_()
+
+    def gdr_step():
+        o, ht = chunk_gated_delta_rule(q, kn, v, g, beta, initial_state=h0, output_final_state=True,
+                                       head_first=False)
+        torch.autograd.backward((o, ht), (do, dht))
+
+    for name, fn in (("chunk_gla", gla_step), ("chunk_gated_delta_rule", gdr_step)):
+        us = event_avg_us(fn, steps)
+        out[name] = {"fwd_bwd_us": round(us, 1), "tokens_per_s": round(B * T / (us * 1e-6), 1)}
+    return out
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -227,6 +300,8 @@ def main():
     extra = {"chunk_gla_fwd": op}
     if not a.no_extra:
         extra["decode_step"] = bench_decode(device)
+        extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
+        extra["fwd_bwd_config4"] = bench_backward(device)
     out = {
         "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

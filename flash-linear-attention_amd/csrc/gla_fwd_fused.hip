@@ -41,6 +41,28 @@ struct FusedParams {
   float scale;
 };
 
+// The row-major q~ / k~ tiles are written by lanes that own four adjacent rows each, i.e.
+// with a row stride of four between neighbouring lanes (64 bytes modulo 256: measured 2.5x
+// slower than conflict-free writes).  XOR-ing row bits 4-5 into the 16-byte chunk index
+// spreads the writes over all banks; every fragment read stays one (or two half-) chunk reads.
+FLA_DEVICE int swz_rm(int row, int col) { return col ^ (((row >> 4) & 3) << 3); }
+
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag32_swz(const T* tile, int ld, int row0, int k0, int lane) {
+  const int row = row0 + (lane & 31);
+  return *(const typename Elem<T>::v8*)(tile + row * ld + swz_rm(row, k0 + 8 * (lane >> 5)));
+}
+// lds_frag32_perm on a swizzled tile
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag32_perm_swz(const T* tile, int ld, int row0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const int row = row0 + (lane & 31), c = k0 + 4 * (lane >> 5);
+  const T* p = tile + row * ld;
+  v4 lo = *(const v4*)(p + swz_rm(row, c));
+  v4 hi = *(const v4*)(p + swz_rm(row, c + 8));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // NSTG: number of staging waves (4 or 8); the workgroup has 4 + NSTG waves.
 template <typename T, typename GT, int K, int NSTG>
 __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
@@ -152,10 +174,11 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       // The scores use one reference point per chunk (e^{G} on q, e^{-G} on k), exact while
       // |G| stays below kMaxInvDecayExp.  Chunks beyond that are flagged and recomputed by
       // the exact kernel afterwards.
-      {
-        const int out_of_range = __any(gabs > kMaxInvDecayExp * LOG2E);
-        if (lane == 0) sWide[buf][pw] = out_of_range;
-      }
+      const int out_of_range = __any(gabs > kMaxInvDecayExp * LOG2E);  // wave-uniform
+      if (lane == 0) sWide[buf][pw] = out_of_range;
+      float eglast[CPL];
+#pragma unroll
+      for (int j = 0; j < CPL; ++j) eglast[j] = __builtin_amdgcn_exp2f(glast[j]);
 #pragma unroll
       for (int i = 0; i < RPT; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 2, i) * kstride);
       T khat[CPL][RPT];
@@ -163,20 +186,31 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       for (int i = 0; i < RPT; ++i) {
         const int row = rg * RPT + i;
         kvec qv, kv;
+        float kt[CPL];
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
           const float Gij = G[i][j] + tot[j];
           float e = __builtin_amdgcn_exp2f(Gij);                        // e^{G}
           float einv = __builtin_amdgcn_rcpf(fmaxf(e, 1e-35f));         // e^{-G}, finite
-          const float kf = (float)R.k[i][j];
-          qv[j] = (T)((float)R.q[i][j] * (p.scale * e));
-          kv[j] = (T)(kf * einv);
-          khat[j][i] = (T)(kf * __builtin_amdgcn_exp2f(glast[j] - Gij));  // k e^{G_last-G}, exponent <= 0
+          kt[j] = (float)R.k[i][j] * einv;
+          qv[j] = (T)((float)R.q[i][j] * e);   // the matrix waves apply the scale to the fp32 output
+          kv[j] = (T)kt[j];
+        }
+        // k^ = k e^{G_last-G}: inside the guarded range the product of the two factors is exact
+        // to rounding; beyond it e^{-G} is clamped, so the exponent (always <= 0) is formed
+        // directly (wave-uniform branch, rare)
+        if (out_of_range) {
+#pragma unroll
+          for (int j = 0; j < CPL; ++j)
+            khat[j][i] = (T)((float)R.k[i][j] * __builtin_amdgcn_exp2f(glast[j] - (G[i][j] + tot[j])));
+        } else {
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) khat[j][i] = (T)(kt[j] * eglast[j]);
         }
         R.q[i] = *(const kvec*)(qp + row_of(c + 2, i) * kstride);
         R.k[i] = *(const kvec*)(kp + row_of(c + 2, i) * kstride);
-        *(kvec*)&sQ[buf][row * LDK + kc] = qv;
-        *(kvec*)&sK[buf][row * LDK + kc] = kv;
+        *(kvec*)&sQ[buf][row * LDK + swz_rm(row, kc)] = qv;
+        *(kvec*)&sK[buf][row * LDK + swz_rm(row, kc)] = kv;
         if (i == RPT / 2 - 1) mid_barrier();
       }
 #pragma unroll
@@ -189,7 +223,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       if (rg == 0) {
 #pragma unroll
-        for (int j = 0; j < CPL; ++j) sDecay[buf][kc + j] = __builtin_amdgcn_exp2f(glast[j]);
+        for (int j = 0; j < CPL; ++j) sDecay[buf][kc + j] = eglast[j];
       }
     };
 
@@ -208,13 +242,13 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       stage(RA, 0, 0, [] {});
       for (int64_t c = 0; c < nchunks; c += 2) {
-        __syncthreads();  // B1(c): tiles of chunk c published; buffer 1 is free
-        if (c + 1 < nchunks) stage(RB, 1, c + 1, [] { __syncthreads(); });  // contains B2(c)
-        else __syncthreads();  // B2(c)
+        lds_barrier();  // B1(c): tiles of chunk c published; buffer 1 is free
+        if (c + 1 < nchunks) stage(RB, 1, c + 1, [] { lds_barrier(); });  // contains B2(c)
+        else lds_barrier();  // B2(c)
         if (c + 1 >= nchunks) break;
-        __syncthreads();  // B1(c+1)
-        if (c + 2 < nchunks) stage(RA, 0, c + 2, [] { __syncthreads(); });  // contains B2(c+1)
-        else __syncthreads();  // B2(c+1)
+        lds_barrier();  // B1(c+1)
+        if (c + 2 < nchunks) stage(RA, 0, c + 2, [] { lds_barrier(); });  // contains B2(c+1)
+        else lds_barrier();  // B2(c+1)
       }
     }
   } else {
@@ -290,7 +324,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       const int buf = (int)(c & 1);
       const int L = chunk_len(c);
       const int64_t row0 = sp.bos + c * BT;
-      __syncthreads();  // B1(c)
+      lds_barrier();  // B1(c)
       if (p.wide) {
         int wide = 0;
 #pragma unroll
@@ -317,16 +351,17 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       if (qj <= qi) {
 #pragma unroll
         for (int ks = 0; ks < K; ks += 16)
-          s = Elem<T>::mfma32(lds_frag32<T>(sQ[buf], LDK, qi * 32, ks, lane),
-                              lds_frag32<T>(sK[buf], LDK, qj * 32, ks, lane), s);
+          s = Elem<T>::mfma32(frag32_swz<T>(sQ[buf], LDK, qi * 32, ks, lane),
+                              frag32_swz<T>(sK[buf], LDK, qj * 32, ks, lane), s);
       }
       f32x16 o = zero16();
 #pragma unroll
       for (int kt = 0; kt < KT32; ++kt) {
         const T* hf = &sHf[((kt * 2 + cw) * 64 + lane) * 16];
         v8 h0v = *(const v8*)hf, h1v = *(const v8*)(hf + 8);
-        o = Elem<T>::mfma32(lds_frag32_perm<T>(sQ[buf], LDK, rw * 32, kt * 32, lane), h0v, o);
-        o = Elem<T>::mfma32(lds_frag32_perm<T>(sQ[buf], LDK, rw * 32, kt * 32 + 16, lane), h1v, o);
+        // transposed product (h^T q~^T): a lane ends up with four consecutive value columns of one row
+        o = Elem<T>::mfma32(h0v, frag32_perm_swz<T>(sQ[buf], LDK, rw * 32, kt * 32, lane), o);
+        o = Elem<T>::mfma32(h1v, frag32_perm_swz<T>(sQ[buf], LDK, rw * 32, kt * 32 + 16, lane), o);
       }
       {
         const int j = qj * 32 + (lane & 31);
@@ -336,26 +371,27 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           sP[i * LDT + j] = (T)((j <= i) ? s[r] : 0.f);
         }
       }
-      __syncthreads();  // B2(c): P visible; nobody reads the state fragments any more
+      lds_barrier();  // B2(c): P visible; nobody reads the state fragments any more
       if (rw == 0) {
 #pragma unroll
         for (int js = 0; js < 32; js += 16)
-          o = Elem<T>::mfma32(lds_frag32<T>(sP, LDT, 0, js, lane), lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), o);
+          o = Elem<T>::mfma32(lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), lds_frag32<T>(sP, LDT, 0, js, lane), o);
       } else {
 #pragma unroll
         for (int js = 0; js < 64; js += 16)
-          o = Elem<T>::mfma32(lds_frag32<T>(sP, LDT, 32, js, lane), lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), o);
+          o = Elem<T>::mfma32(lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), lds_frag32<T>(sP, LDT, 32, js, lane), o);
       }
       {
-        T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V + vbase + cw * 32 + (lane & 31);
-        if (L == BT) {
+        // o^T tile: lane <-> time row, registers <-> value columns 8 (r/4) + 4 (lane/32) + r%4
+        const int i = rw * 32 + (lane & 31);
+        if (i < L) {
+          T* op = (T*)p.o + ((row0 + i) * H + hh) * (int64_t)V + vbase + cw * 32 + 4 * (lane >> 5);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) op[(int64_t)(rw * 32 + c32_row(r, lane)) * H * V] = (T)o[r];
-        } else {
+          for (int r4 = 0; r4 < 4; ++r4) {
+            v4 ov;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            int i = rw * 32 + c32_row(r, lane);
-            if (i < L) op[(int64_t)i * H * V] = (T)o[r];
+            for (int e = 0; e < 4; ++e) ov[e] = (T)(o[4 * r4 + e] * p.scale);
+            *(v4*)(op + 8 * r4) = ov;
           }
         }
       }
