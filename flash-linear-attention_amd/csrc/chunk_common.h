@@ -41,6 +41,28 @@ FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
   return (id % 8) * (total / 8) + id / 8;
 }
 
+// Work items of the serial scan kernels: one per (sequence, head, value-column slab).
+// Workgroups are dispatched in blockIdx order and dealt round-robin to the 8 XCDs; the slabs
+// of one (sequence, head) are placed on the same XCD (they read the same q/k/gate rows, which
+// then hit in that XCD's L2), and (sequence, head) items are taken in dispatch order, so that
+// with `seq_order` (sequence ids, longest first) the longest sequences start first.
+struct ScanItem {
+  int slab;       // value-column slab
+  int64_t item;   // (position in seq_order) * H + head
+};
+FLA_DEVICE ScanItem scan_item(int nslab) {
+  const int64_t p = blockIdx.x, tot = gridDim.x;
+  ScanItem s;
+  if (tot % (8 * nslab) == 0) {
+    s.slab = (int)((p / 8) % nslab);
+    s.item = (p / (8 * nslab)) * 8 + p % 8;
+  } else {
+    s.slab = (int)(p % nslab);
+    s.item = p / nslab;
+  }
+  return s;
+}
+
 struct ChunkLoc {
   int64_t row0;   // first token row of the chunk in the flattened [B*T] space
   int L;          // valid rows

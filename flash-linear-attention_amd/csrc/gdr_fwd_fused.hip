@@ -36,6 +36,7 @@ struct GdrFusedParams {
   void* o;
   float* ht;
   const int64_t* offsets;
+  const int64_t* seq_order;  // sequence ids, longest first (or NULL)
   int64_t T;
   int H, V, N;
   float scale;
@@ -101,10 +102,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int H = p.H, V = p.V;
   const int nvb = V / BV;
-  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
-  const int vb = (int)(id % nvb);
-  const int nh = (int)(id / nvb);
-  const int n = nh / H, hh = nh % H;
+  const ScanItem wi = scan_item(nvb);
+  const int vb = wi.slab;
+  const int hh = (int)(wi.item % H);
+  const int n = p.seq_order ? (int)p.seq_order[wi.item / H] : (int)(wi.item / H);
+  const int nh = n * H + hh;
   const int vbase = vb * BV;
   SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int nchunks = (int)((sp.len + BT - 1) / BT);
@@ -476,7 +478,8 @@ int launch_fused(const GdrFusedParams& p, int K, hipStream_t st) {
 
 extern "C" int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
                                                     const void* Aqk, const float* g_cumsum, const float* h0, void* o,
-                                                    float* ht, const int64_t* offsets, int qkv_dtype, int64_t B,
+                                                    float* ht, const int64_t* offsets, const int64_t* seq_order, int qkv_dtype,
+                                                    int64_t B,
                                                     int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                                     fla_stream_t stream) {
   FLA_REQUIRE(q && k && w && u && Aqk && o, FLA_E_INVALID);
@@ -485,7 +488,7 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k
   FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aqk | (uintptr_t)o) % 16 == 0,
               FLA_E_ALIGNMENT);
-  GdrFusedParams p{q, k, w, u, Aqk, g_cumsum, h0, o, ht, offsets, T, (int)H, (int)V, (int)N, scale};
+  GdrFusedParams p{q, k, w, u, Aqk, g_cumsum, h0, o, ht, offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
   if (qkv_dtype == FLA_BF16) return launch_fused<bf16>(p, (int)K, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_fused<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

@@ -34,6 +34,7 @@ struct FusedParams {
   float* ht;
   const int64_t* offsets;
   const int64_t* chunk_offsets;
+  const int64_t* seq_order;  // sequence ids, longest first (or NULL)
   int* wide;        // [chunks, H]: 1 where a chunk's gates leave the single-reference range
   void* hwide;      // states entering those chunks, FLA_H_FRAGMENT order, [chunks, H, K*V]
   int64_t T;
@@ -91,10 +92,11 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int H = p.H, V = p.V;
   const int nvb = V / BV;
-  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
-  const int vb = (int)(id % nvb);
-  const int nh = (int)(id / nvb);
-  const int n = nh / H, hh = nh % H;
+  const ScanItem wi = scan_item(nvb);
+  const int vb = wi.slab;
+  const int hh = (int)(wi.item % H);
+  const int n = p.seq_order ? (int)p.seq_order[wi.item / H] : (int)(wi.item / H);
+  const int nh = n * H + hh;
   const int vbase = vb * BV;
   SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int64_t nchunks = (sp.len + BT - 1) / BT;
@@ -625,7 +627,8 @@ int launch_fused(const FusedParams& p, int K, hipStream_t st) {
 
 extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates, const float* h0,
                                        void* o, float* ht, int* ws_wide, void* ws_hwide, const int64_t* offsets,
-                                       const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                                       const int64_t* indices, const int64_t* chunk_offsets,
+                                       const int64_t* seq_order, int64_t NT,
                                        int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                                        int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
@@ -637,7 +640,8 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
   if (ws_wide) FLA_REQUIRE(V <= 128, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)o | (uintptr_t)ws_hwide) % 16 == 0,
               FLA_E_ALIGNMENT);
-  FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, ws_wide, ws_hwide, T, (int)H, (int)V, (int)N, scale};
+  FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
+                T, (int)H, (int)V, (int)N, scale};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;

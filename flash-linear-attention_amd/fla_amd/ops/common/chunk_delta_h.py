@@ -74,12 +74,14 @@ def chunk_gated_delta_rule_fwd_fused(
     initial_state: Optional[torch.Tensor],
     output_final_state: bool,
     offsets: Optional[torch.Tensor] = None,
+    seq_order: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """State scan and output in one launch (``fla_chunk_gated_delta_rule_fwd_fused``): the work of
     ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o``
     (``fla/ops/gated_delta_rule/chunk.py:47-72``) without materialising the per-chunk states
     or ``v_new``.  ``w, u, Aqk`` come from ``fwd_prepare_wy_repr(..., q=q, scale=scale)``;
-    ``g`` is the fp32 chunk-local cumsum.  Seq-first layout.  Returns ``(o, final_state)``."""
+    ``g`` is the fp32 chunk-local cumsum.  Seq-first layout.  ``seq_order`` (int64 ``[N]``, sequence
+    ids longest first) balances a packed batch.  Returns ``(o, final_state)``."""
     be.require_gpu(q, k, w, u, Aqk)
     B, T, H, K = k.shape
     V = u.shape[-1]
@@ -96,6 +98,6 @@ def chunk_gated_delta_rule_fwd_fused(
         g = g.float()
     be.check(be.lib().fla_chunk_gated_delta_rule_fwd_fused(
         be.ptr(q), be.ptr(k), be.ptr(w), be.ptr(u), be.ptr(Aqk), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht),
-        be.ptr(offsets), be.dt(k), B, T, H, K, V, N, float(scale), be.stream_of(k)),
+        be.ptr(offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale), be.stream_of(k)),
         "fla_chunk_gated_delta_rule_fwd_fused")
     return o, ht

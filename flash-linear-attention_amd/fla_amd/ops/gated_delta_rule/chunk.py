@@ -46,7 +46,8 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
         w, u, Aw, Au, Aqk = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False,
                                                 chunk_size=BT, store_A=store_A, q=q, scale=scale)
         o, final_state = chunk_gated_delta_rule_fwd_fused(q, k, w, u, Aqk, g, scale, initial_state,
-                                                          output_final_state, offsets=offs)
+                                                          output_final_state, offsets=offs,
+                                                          seq_order=None if plan is None else plan.seq_order)
         return g, o, Aw, Au, final_state
     w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
                                        store_A=store_A)

@@ -72,7 +72,8 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     be.check(be.lib().fla_chunk_gla_fwd_fused(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide),
         be.ptr(None if plan is None else plan.offsets), be.ptr(None if plan is None else plan.indices),
-        be.ptr(None if plan is None else plan.chunk_offsets), 0 if plan is None else plan.NT,
+        be.ptr(None if plan is None else plan.chunk_offsets), be.ptr(None if plan is None else plan.seq_order),
+        0 if plan is None else plan.NT,
         be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_fused")
     return o, ht
 

@@ -80,6 +80,10 @@ class VarlenPlan:
         self.chunk_offsets = co.to(dev, non_blocking=True)
         self.N = len(host) - 1
         self.NT = idx.shape[0]
+        # sequence ids, longest first: the order in which the serial scan kernels start sequences
+        lens = [host[i + 1] - host[i] for i in range(self.N)]
+        order = sorted(range(self.N), key=lambda i: -lens[i])
+        self.seq_order = torch.tensor(order, dtype=torch.int64).to(dev, non_blocking=True)
 
 
 def resolve_offsets(offsets: Optional[torch.Tensor], cu_seqlens: Optional[torch.Tensor]):

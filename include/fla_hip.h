@@ -145,11 +145,14 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
  * (V <= 128), chunks outside that range are flagged on the device and their
  * output rows recomputed by a second launch with exact pairwise exponents
  * (the reference's diagonal sub-block arithmetic, fla/ops/gla/chunk.py:113-170);
- * packed batches then also need indices [NT,2] and chunk_offsets [N+1]. */
+ * packed batches then also need indices [NT,2] and chunk_offsets [N+1].
+ * seq_order (int64 [N], a permutation of the sequence ids, or NULL) is the order
+ * in which sequences are handed to the hardware; longest first balances a
+ * packed batch. */
 int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates,
                             const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
                             const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
-                            int64_t NT, int qkv_dtype, int gate_dtype,
+                            const int64_t* seq_order, int64_t NT, int qkv_dtype, int gate_dtype,
                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                             float scale, fla_stream_t stream);
 
@@ -200,10 +203,12 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * fla/ops/common/chunk_delta_h.py:27-119 and chunk_o.py:23-101) when neither the
  * per-chunk states nor v_new are wanted.  w, u and Aqk come from
  * fla_gdr_fwd_wy (called with q, scale).  o [B,T,H,V] in the q/k/v dtype;
- * h0, ht fp32 [N,H,K,V] or NULL.  K in {64,128}, V a multiple of 64. */
+ * h0, ht fp32 [N,H,K,V] or NULL.  K in {64,128}, V a multiple of 64.
+ * seq_order as for fla_chunk_gla_fwd_fused. */
 int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
                                          const void* Aqk, const float* g_cumsum, const float* h0,
-                                         void* o, float* ht, const int64_t* offsets, int qkv_dtype,
+                                         void* o, float* ht, const int64_t* offsets,
+                                         const int64_t* seq_order, int qkv_dtype,
                                          int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                          float scale, fla_stream_t stream);
 
