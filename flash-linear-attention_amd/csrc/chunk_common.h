@@ -69,24 +69,32 @@ struct ChunkLoc {
   int64_t cglob;  // global chunk index (addresses per-chunk states)
 };
 
-// blockIdx.x enumerates chunks: (batch, chunk) for equal lengths, rows of `indices` otherwise.
-FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix) {
+// Chunk-parallel kernels run on a grid (chunks, H[, slices]); (batch, chunk) for equal lengths,
+// rows of `indices` otherwise.  Workgroups are dispatched x-fastest, so the linear id is split
+// head-fastest: workgroups that run together take different heads of the same chunks, whose rows
+// are adjacent in memory, and the traffic spreads evenly over the memory channels (a
+// chunk-fastest order makes concurrent workgroups hit the same address bits 8-11).
+FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix, int H,
+                                 int* head) {
+  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+  const int64_t cidx = lin / H;
+  *head = (int)(lin % H);
   ChunkLoc c;
   int64_t bos, len, ic;
   if (offsets) {
-    int64_t n = indices[2 * (int64_t)blockIdx.x];
-    ic = indices[2 * (int64_t)blockIdx.x + 1];
+    int64_t n = indices[2 * cidx];
+    ic = indices[2 * cidx + 1];
     bos = offsets[n];
     len = offsets[n + 1] - bos;
   } else {
-    bos = (blockIdx.x / ntfix) * T;
-    ic = blockIdx.x % ntfix;
+    bos = (cidx / ntfix) * T;
+    ic = cidx % ntfix;
     len = T;
   }
   c.row0 = bos + ic * BT;
   int64_t rem = len - ic * BT;
   c.L = (int)(rem < BT ? rem : BT);
-  c.cglob = blockIdx.x;
+  c.cglob = cidx;
   return c;
 }
 

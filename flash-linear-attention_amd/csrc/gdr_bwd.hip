@@ -60,8 +60,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];
   __shared__ float sGam[BT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, hh = blockIdx.y;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int H = p.H;
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 #pragma unroll
@@ -469,9 +470,10 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
   float* stD = (float*)sRD;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, K = p.K, hh = blockIdx.y;
+  const int H = p.H, K = p.K;
   const int kb = blockIdx.z * 64;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -735,8 +737,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   __shared__ float sBeta[BT], sGam[BT], sDb[BT], sDg[BT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, hh = blockIdx.y;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int H = p.H;
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
   const int rw = wave >> 1, cw = wave & 1;

@@ -251,8 +251,9 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   __shared__ __attribute__((aligned(16))) float sPart[RG * K];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, hh = blockIdx.y;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  const int H = p.H;
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -439,9 +440,10 @@ __global__ __launch_bounds__(256) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   float* stC = (float*)sRC;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int H = p.H, K = p.K, hh = blockIdx.y;
+  const int H = p.H, K = p.K;
   const int kb = blockIdx.z * 64;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 

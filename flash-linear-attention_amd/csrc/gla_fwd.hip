@@ -325,20 +325,22 @@ __global__ __launch_bounds__(256) void gla_fwd_o_kernel(OParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H;
-  const int hh = blockIdx.y;
-  int64_t bos, len, ic, cglob;
+  // workgroups that run together take different heads of the same chunks: their rows are
+  // adjacent in memory, so the traffic spreads over all memory channels
+  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+  const int hh = (int)(lin % H);
+  const int64_t cglob = lin / H;
+  int64_t bos, len, ic;
   if (p.offsets) {
-    int64_t n = p.indices[2 * (int64_t)blockIdx.x];
-    ic = p.indices[2 * (int64_t)blockIdx.x + 1];
+    int64_t n = p.indices[2 * cglob];
+    ic = p.indices[2 * cglob + 1];
     bos = p.offsets[n];
     len = p.offsets[n + 1] - bos;
-    cglob = blockIdx.x;
   } else {
-    int64_t b = blockIdx.x / p.NTfix;
-    ic = blockIdx.x % p.NTfix;
+    int64_t b = cglob / p.NTfix;
+    ic = cglob % p.NTfix;
     bos = b * p.T;
     len = p.T;
-    cglob = blockIdx.x;
   }
   const int64_t t0 = ic * BT;
   const int L = (int)((len - t0) < BT ? (len - t0) : BT);

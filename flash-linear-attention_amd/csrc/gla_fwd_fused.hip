@@ -466,8 +466,10 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
   constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int KT32 = K / 32, TV = V / 64;
-  const int hh = blockIdx.y, H = p.H;
-  if (p.wide[(int64_t)blockIdx.x * H + hh] == 0) return;  // workgroup-uniform
+  const int H = p.H;
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  if (p.wide[cl.cglob * H + hh] == 0) return;  // workgroup-uniform
   __shared__ __attribute__((aligned(16))) float sG[BT * LDG];
   __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
   __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
@@ -475,7 +477,6 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
   __shared__ __attribute__((aligned(16))) T sP[BT * LDT];
   __shared__ __attribute__((aligned(16))) float sPart[RG * K];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
   const int rg = tid / CG, c4 = (tid % CG) * 4;
@@ -565,7 +566,7 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
   f32x16 acc[TV];
 #pragma unroll
   for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
-  const T* hp = (const T*)p.hwide + ((int64_t)blockIdx.x * H + hh) * (int64_t)K * V;
+  const T* hp = (const T*)p.hwide + (cl.cglob * H + hh) * (int64_t)K * V;
 #pragma unroll
   for (int kt = 0; kt < KT32; ++kt)
 #pragma unroll
