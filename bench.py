@@ -262,21 +262,26 @@ def cpu_baseline(c, budget_s=15.0):
     import torch
     from oracle.recurrent import naive_recurrent_gla
     B = c["B"]
-    tokens, spent, used = 0, 0.0, 0
-    for b in range(B):
-        q, k, v, g, h0 = (c[n][b:b + 1].float().cpu() for n in ("q", "k", "v", "g", "h0"))
-        t0 = time.perf_counter()
-        naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
-        dt = time.perf_counter() - t0
-        tokens += q.shape[1]
-        spent += dt
-        used += 1
+    tokens, spent, used, reps = 0, 0.0, 0, 0
+    host = [tuple(c[n][b:b + 1].float().cpu() for n in ("q", "k", "v", "g", "h0")) for b in range(B)]
+    while spent < 10.0:
+        for b in range(B):
+            q, k, v, g, h0 = host[b]
+            t0 = time.perf_counter()
+            naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+            dt = time.perf_counter() - t0
+            tokens += q.shape[1]
+            spent += dt
+            used = max(used, b + 1)
+            if spent + dt > budget_s:
+                break
+        reps += 1
         if spent + dt > budget_s:
             break
     return {"value": round(tokens / spent, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
             "kind": "port", "seconds": round(spent, 2),
             "sample": f"oracle naive_recurrent_gla (torch CPU fp32) on batch elements 0..{used - 1} of {B} "
-                      f"(T={c['T']}, H={c['H']}, K=V=128 each), one repetition"}
+                      f"(T={c['T']}, H={c['H']}, K=V=128 each), {reps} pass(es) over them"}
 
 
 def main():
@@ -286,6 +291,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known traffic, used to scale the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build measures one GPU only (every (sequence, head) pair is independent; "
@@ -314,6 +322,11 @@ def main():
         "extra": extra,
     }
     print(json.dumps(out))
+    if a.copy_calibration:
+        x = torch.empty(1 << 28, device=device, dtype=torch.float32)
+        y = torch.empty_like(x)
+        y.copy_(x)
+        torch.cuda.synchronize()
 
 
 if __name__ == "__main__":
