@@ -21,8 +21,9 @@ def install() -> list:
     import importlib
     patched = []
     table = {name: getattr(ops, name) for name in ops.__all__}
-    targets = ['fla.ops.gla', 'fla.ops.gated_delta_rule', 'fla.ops.utils', 'fla.ops',
-               'fla.layers.gla', 'fla.layers.gated_deltanet', 'fla.layers.hgrn2']
+    targets = ['fla.ops.gla', 'fla.ops.gated_delta_rule', 'fla.ops.delta_rule', 'fla.ops.simple_gla', 'fla.ops.utils',
+               'fla.ops', 'fla.layers.gla', 'fla.layers.gated_deltanet', 'fla.layers.hgrn2', 'fla.layers.delta_net',
+               'fla.layers.simple_gla']
     for modname in targets:
         try:
             mod = importlib.import_module(modname)

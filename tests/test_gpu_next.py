@@ -1,0 +1,108 @@
+"""GPU: the operators that are pure compositions of the hot-path kernels
+(``chunk_delta_rule``, ``chunk_simple_gla``, ``fused_recurrent_simple_gla``) against the
+fp32 naive recurrences, forward and backward."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import assert_close, gdr_inputs, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+TOL_O, TOL_HT, TOL_G = 1e-2, 5e-3, 2e-2
+
+
+def _dev(device):
+    return lambda x: None if x is None else x.to(device)
+
+
+# reference ladder: tests/ops/test_delta.py (T in {63, 300, 1000}-style lengths, packed batches)
+@pytest.mark.parametrize("T", [63, 300, 1000])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_delta_rule(device, T, varlen):
+    from fla_amd.ops.delta_rule import chunk_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    N = 3
+    offs = random_offsets(T, N, torch.Generator().manual_seed(T), min_len=1) if varlen else None
+    q, k, v, _, beta, h0 = gdr_inputs(1 if varlen else 2, T, 2, 128, 128, seed=T, N=N if varlen else None)
+    dev = _dev(device)
+    print(f"chunk_delta_rule T={T} varlen={varlen}", flush=True)
+    do = torch.randn(v.shape, generator=torch.Generator().manual_seed(1)).to(v.dtype)
+    dht = torch.randn(h0.shape, generator=torch.Generator().manual_seed(2)) * 0.1
+    # device
+    leaves = [dev(x).detach().requires_grad_() for x in (q, k, v, beta)]
+    h0l = dev(h0).detach().requires_grad_()
+    o, ht = chunk_delta_rule(*leaves, initial_state=h0l, output_final_state=True, offsets=dev(offs), head_first=False)
+    torch.autograd.backward((o, ht), (dev(do), dev(dht)))
+    torch.cuda.synchronize()
+    # oracle
+    rl = [x.detach().float().requires_grad_() for x in (q, k, v, beta)]
+    rh0 = h0.detach().float().requires_grad_()
+    ro, rht = naive_recurrent_gated_delta_rule(rl[0], rl[1], rl[2], None, rl[3], initial_state=rh0,
+                                               output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    for name, a, b in zip(("dq", "dk", "dv", "dbeta"), rl, leaves):
+        assert_close(name, a.grad, b.grad, TOL_G)
+    assert_close("dh0", rh0.grad, h0l.grad, TOL_G)
+
+
+@pytest.mark.parametrize("T", [64, 300, 1000])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_simple_gla(device, T, varlen):
+    from fla_amd.ops.simple_gla import chunk_simple_gla
+    from oracle.recurrent import naive_recurrent_gla
+    N, H, K, V = 3, 2, 128, 64
+    B = 1 if varlen else 2
+    gen = torch.Generator().manual_seed(T + 7)
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    h0 = torch.randn(N if varlen else B, H, K, V, generator=gen) * 0.1
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"chunk_simple_gla T={T} varlen={varlen}", flush=True)
+    leaves = [dev(x).detach().requires_grad_() for x in (q, k, v, g)]
+    h0l = dev(h0).detach().requires_grad_()
+    o, ht = chunk_simple_gla(*leaves, initial_state=h0l, output_final_state=True, cu_seqlens=dev(offs),
+                             head_first=False)
+    torch.autograd.backward((o, ht), (dev(do), dev(dht)))
+    torch.cuda.synchronize()
+    rl = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.detach().float().requires_grad_()
+    ro, rht = naive_recurrent_gla(rl[0], rl[1], rl[2], None, g=rl[3], initial_state=rh0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    # the head-wise gate gradient is the sum over the 128 key channels of the channel-wise one; the
+    # terms largely cancel, so its relative error is a few times that of a single channel
+    for name, a, b, tol in zip(("dq", "dk", "dv", "dg"), rl, leaves, (TOL_G, TOL_G, TOL_G, 4e-2)):
+        assert_close(name, a.grad, b.grad, tol)
+    assert_close("dh0", rh0.grad, h0l.grad, TOL_G)
+
+
+@pytest.mark.parametrize("T", [1, 100])
+def test_fused_recurrent_simple_gla(device, T):
+    from fla_amd.ops.simple_gla import fused_recurrent_simple_gla
+    from oracle.recurrent import naive_recurrent_gla
+    B, H, K, V = 2, 3, 128, 128
+    gen = torch.Generator().manual_seed(T)
+    q = torch.randn(B, T, H, K, generator=gen)
+    k = torch.randn(B, T, H, K, generator=gen)
+    v = torch.randn(B, T, H, V, generator=gen)
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    h0 = torch.randn(B, H, K, V, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"fused_recurrent_simple_gla T={T}", flush=True)
+    o, ht = fused_recurrent_simple_gla(dev(q), dev(k), dev(v), dev(g), initial_state=dev(h0), output_final_state=True,
+                                       head_first=False)
+    torch.cuda.synchronize()
+    ro, rht = naive_recurrent_gla(q, k, v, None, g=g, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, 1e-5)
+    assert_close("ht", rht, ht, 1e-5)
