@@ -109,12 +109,6 @@ inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B,
   return FLA_OK;
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a fence over
-// global memory as well: a wave with global stores in flight then drains its whole vector
-// memory queue (loads included) at every barrier, which exposes the full memory latency of
-// register prefetches once per chunk.  Use only where the waves exchange data through LDS.
-FLA_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 // Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps
 // the operand finite in 16-bit storage.
 constexpr float kMaxInvDecayExp = 80.f;

@@ -108,6 +108,12 @@ FLA_DEVICE float row_suffix16(float x) {
   return x;
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a fence over
+// global memory as well: a wave with global stores in flight then drains its whole vector
+// memory queue (loads included) at every barrier, which exposes the full memory latency of
+// register prefetches once per chunk.  Use only where the waves exchange data through LDS.
+FLA_DEVICE void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 struct SeqSpan {
   int64_t bos;  // first token row of the sequence in the packed [B*T] row space
   int64_t len;  // number of tokens

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   for (int64_t c = nchunks - 1; c >= 0; --c) {
     const int L = chunk_len(c);
     const int64_t rbase = sp.bos + c * BT;
-    __syncthreads();  // (1)
+    lds_barrier();  // (1)
     // ---- dv2 = dv_loc + k^ dH : wave w owns rows 16w..16w+15, two 16-column tiles
     {
       f32x4 d[2] = {zero4(), zero4()};
@@ -375,7 +375,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
     stage_x(X);
     const float dec_c = dec;
     load_x(c - 1, X);
-    __syncthreads();  // (2)
+    lds_barrier();  // (2)
     // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
 #pragma unroll
     for (int a = 0; a < NKT; ++a) {

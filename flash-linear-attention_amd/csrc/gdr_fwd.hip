@@ -601,7 +601,7 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   for (int64_t c = 0; c < nchunks; ++c) {
     const int L = chunk_len(c);
     const int64_t rbase = sp.bos + c * BT;
-    __syncthreads();  // (1)
+    lds_barrier();  // (1)
     // ---- v_new = u - (w e^gamma) h : wave w owns rows 16w..16w+15, two 16-column tiles
     {
       f32x4 d[2] = {zero4(), zero4()};
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
     const float dec = __expf(Rc.glast);
     Rc = Rn;
     load_chunk(c + 2, Rn);
-    __syncthreads();  // (2)
+    lds_barrier();  // (2)
     // ---- h <- e^{gamma_last} h + (k e^{gamma_last-gamma})^T v_new
 #pragma unroll
     for (int a = 0; a < NKT; ++a) {

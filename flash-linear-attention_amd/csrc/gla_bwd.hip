@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       *(v8*)&sDt[buf][(c2 + 1) * LDT + rg * 8] = db;
       if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
     }
-    __syncthreads();
+    lds_barrier();
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];

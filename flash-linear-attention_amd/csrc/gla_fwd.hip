@@ -258,7 +258,7 @@ __global__ __launch_bounds__(256) void gla_fwd_h_kernel(HParams p) {
       *(v8*)&sVt[buf][(c2 + 1) * LDT + rg * 8] = vb;
       if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
     }
-    __syncthreads();  // tiles of chunk c complete; buffer buf^1 is free again after the next barrier
+    lds_barrier();  // tiles of chunk c complete; buffer buf^1 is free again after the next barrier
     if (TR) {
       const float d = sDecay[buf][kq * 32 + (lane & 31)];
 #pragma unroll
