@@ -706,18 +706,55 @@ struct WyBwdParams {
   int H, NTfix;
 };
 
-// 64 x N product helper: C[64 x 32*NTILE per wave] with A from a [64][lda] tile (rows = output
-// rows, contraction contiguous) and B from a [cols][ldb] tile (contraction contiguous).
+// Transposed 64 x N product: acc[t] (+)= X^T-tile A^T, i.e. C[column][time row] with
+//   X^T  [columns][ldx]  (contraction contiguous), columns col0 + 32 t ..
+//   A    [64][lda]       (rows = output time rows 32 rw .., contraction contiguous).
+// A lane ends up with one time row (32 rw + lane % 32) and, per tile, registers
+// r <-> column col0 + 32 t + 8 (r/4) + 4 (lane/32) + r%4: four consecutive columns per
+// register quad, so the epilogues use 8-byte accesses and row sums stay in the lane.
 template <typename T, int NT_>
-FLA_DEVICE void mm64(const T* A, int lda, const T* Bt, int ldb, int rw, int col0, int c_begin, int c_end, int lane,
-                     f32x16* acc) {
+FLA_DEVICE void mm64t(const T* Xt, int ldx, int col0, const T* A, int lda, int rw, int c_begin, int c_end, int lane,
+                      f32x16* acc) {
   typedef typename Elem<T>::v8 v8;
   for (int cs = c_begin; cs < c_end; cs += 16) {
     v8 a = lds_frag32<T>(A, lda, rw * 32, cs, lane);
 #pragma unroll
-    for (int t = 0; t < NT_; ++t) acc[t] = Elem<T>::mfma32(a, lds_frag32<T>(Bt, ldb, col0 + t * 32, cs, lane), acc[t]);
+    for (int t = 0; t < NT_; ++t) acc[t] = Elem<T>::mfma32(lds_frag32<T>(Xt, ldx, col0 + t * 32, cs, lane), a, acc[t]);
   }
 }
+
+// A thread of the tile loaders owns RPT rows x 4 columns of a [64][DIM] tile: 8-byte global
+// loads, 8-byte row-major LDS writes and time-contiguous vectors for the transposed copy.
+template <typename T, int DIM>
+struct TileIO {
+  typedef typename Elem<T>::v4 v4;
+  static constexpr int CG = DIM / 4, RG = 256 / CG, RPT = BT / RG;
+  typedef T tvec __attribute__((ext_vector_type(RPT)));
+  static FLA_DEVICE void load(const void* src, int64_t row0, int L, int H, int hh, int tid, v4* reg) {
+    const int rg = tid / CG, c4 = (tid % CG) * 4;
+    const T* p = (const T*)src + (row0 * H + hh) * (int64_t)DIM + c4;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      reg[i] = row < L ? *(const v4*)(p + (int64_t)row * H * DIM) : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    }
+  }
+  static FLA_DEVICE void put_rows(T* dst, int ld, int tid, const v4* reg) {
+    const int rg = tid / CG, c4 = (tid % CG) * 4;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) *(v4*)&dst[(rg * RPT + i) * ld + c4] = reg[i];
+  }
+  static FLA_DEVICE void put_tr(T* dst, int tid, const v4* reg) {
+    const int rg = tid / CG, c4 = (tid % CG) * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      tvec x;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) x[i] = reg[i][j];
+      *(tvec*)&dst[(c4 + j) * LDT + rg * RPT] = x;
+    }
+  }
+};
 
 template <typename T, int K, int V>
 __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
@@ -726,14 +763,16 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   constexpr int D = K > V ? K : V;
   constexpr int LDD = D + 8;
   constexpr int TK = K / 64, TV = V / 64;
-  __shared__ __attribute__((aligned(16))) T sRow1[BT * LDD];   // dw | du            row-major [t][d]
-  __shared__ __attribute__((aligned(16))) T sRow2[BT * LDD];   // kb | vb | k         row-major
-  __shared__ __attribute__((aligned(16))) T sTr1[D * LDT];     // dw^T | du^T | k^T   [d][t]
-  __shared__ __attribute__((aligned(16))) T sTr2[D * LDT];     // kb^T
+  typedef TileIO<T, K> IOK;
+  typedef TileIO<T, V> IOV;
+  typedef TileIO<T, BT> IOA;
+  __shared__ __attribute__((aligned(16))) T sRow1[BT * LDD];   // du, then dw          row-major [t][d]
+  __shared__ __attribute__((aligned(16))) T sRow2[BT * LDD];   // v,  then k           row-major
+  __shared__ __attribute__((aligned(16))) T sTr1[D * LDT];     // du^T, dw^T, k^T      [d][t]
   __shared__ __attribute__((aligned(16))) T sAw[BT * LDT];     // Aw [i][j]
   __shared__ __attribute__((aligned(16))) T sAwT[BT * LDT];    // Aw^T
   __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA (masked) -> dM
-  __shared__ __attribute__((aligned(16))) T sS2[BT * LDT];     // X1^T -> dM^T
+  __shared__ __attribute__((aligned(16))) T sS2[BT * LDT];     // X1^T -> dM^T diag(beta)
   __shared__ float sBeta[BT], sGam[BT], sDb[BT], sDg[BT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -744,6 +783,11 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   const int64_t row0 = cl.row0;
   const int rw = wave >> 1, cw = wave & 1;
 
+  // ---- issue the loads of the value side and of Aw
+  v4 rdu[IOV::RPT], rv[IOV::RPT], ra[IOA::RPT];
+  IOV::load(p.du, row0, L, H, hh, tid, rdu);
+  IOV::load(p.v, row0, L, H, hh, tid, rv);
+  IOA::load(p.Aw, row0, L, H, hh, tid, ra);
   if (tid < BT) {
     bool ok = tid < L;
     sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
@@ -751,124 +795,101 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
     sDb[tid] = 0.f;
     sDg[tid] = 0.f;
   }
-  // Aw and Aw^T (rows beyond L: identity)
   {
-    const int i = tid >> 2, j0 = (tid & 3) * 16;
-    v8 a0, a1;
-    if (i < L) {
-      const T* ap = (const T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + j0;
-      a0 = *(const v8*)ap;
-      a1 = *(const v8*)(ap + 8);
-    } else {
+    // rows beyond L: identity
+    const int rg = tid / IOA::CG, c4 = (tid % IOA::CG) * 4;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        a0[e] = (T)((j0 + e == i) ? 1.f : 0.f);
-        a1[e] = (T)((j0 + 8 + e == i) ? 1.f : 0.f);
-      }
-    }
-    *(v8*)&sAw[i * LDT + j0] = a0;
-    *(v8*)&sAw[i * LDT + j0 + 8] = a1;
+    for (int i = 0; i < IOA::RPT; ++i) {
+      int row = rg * IOA::RPT + i;
+      if (row >= L)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      sAwT[(j0 + e) * LDT + i] = a0[e];
-      sAwT[(j0 + 8 + e) * LDT + i] = a1[e];
+        for (int j = 0; j < 4; ++j) ra[i][j] = (T)((c4 + j == row) ? 1.f : 0.f);
     }
   }
+  IOA::put_rows(sAw, LDT, tid, ra);
+  IOA::put_tr(sAwT, tid, ra);
+  IOV::put_rows(sRow1, LDD, tid, rdu);
+  IOV::put_tr(sTr1, tid, rdu);
+  IOV::put_rows(sRow2, LDD, tid, rv);
+  // the key side is loaded while the value side computes
+  v4 rdw[IOK::RPT], rk[IOK::RPT];
+  IOK::load(p.dw, row0, L, H, hh, tid, rdw);
+  IOK::load(p.k, row0, L, H, hh, tid, rk);
   __syncthreads();
-
-  // generic tile loaders: row-major [64][DIM] (optionally scaled per row) and its transpose
-  auto load_rows = [&](const void* src, int DIM, bool scale_beta, T* dst_row, T* dst_tr) {
-    const int c8n = DIM / 8;
-    for (int e = tid; e < BT * c8n; e += 256) {
-      int row = e / c8n, c8 = (e % c8n) * 8;
-      v8 x;
-      if (row < L) x = *(const v8*)((const T*)src + ((row0 + row) * H + hh) * (int64_t)DIM + c8);
-      else {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = (T)0.f;
-      }
-      if (scale_beta) {
-        float b = sBeta[row];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) x[j] = (T)((float)x[j] * b);
-      }
-      if (dst_row) *(v8*)&dst_row[row * LDD + c8] = x;
-      if (dst_tr) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dst_tr[(c8 + j) * LDT + row] = x[j];
-      }
-    }
-  };
-
-  // ================= key side: d(kb)_1 = Aw^T dw ; dAw_1 = dw kb^T
-  load_rows(p.dw, K, false, sRow1, sTr1);
-  load_rows(p.k, K, true, sRow2, sTr2);   // kb, kb^T
-  __syncthreads();
-  f32x16 dkb[TK];   // d(kb), rows j = 32rw.., cols (cw*TK+t)*32..
-#pragma unroll
-  for (int t = 0; t < TK; ++t) dkb[t] = zero16();
-  // Aw^T is upper triangular: row j contracts over i >= j
-  mm64<T, TK>(sAwT, LDT, sTr1, LDT, rw, cw * TK * 32, rw * 32, BT, lane, dkb);
-  // dA quadrants (lower triangular incl. diagonal block): waves 0,2,3 -> (ib,jb) = (0,0),(1,0),(1,1)
-  const int ib = wave >> 1, jb = wave & 1;
-  f32x16 dA = zero16();
-  if (jb <= ib) {
-    for (int ks = 0; ks < K; ks += 16)
-      dA = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, ks, lane), lds_frag32<T>(sRow2, LDD, jb * 32, ks, lane), dA);
-  }
-  __syncthreads();
-  // ================= value side: d(vb) = Au^T du ; dAu = du vb^T
-  load_rows(p.du, V, false, sRow1, sTr1);
-  load_rows(p.v, V, true, sRow2, nullptr);   // vb
   {
     // Au^T[j][i] = Aw^T[j][i] * e^{gamma_i - gamma_j}, i >= j
     const int j = tid >> 2, i0 = (tid & 3) * 16;
     const float gj = sGam[j];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      int i = i0 + e;
-      float a = (float)sAwT[j * LDT + i];
-      sS1[j * LDT + i] = (T)((i >= j) ? a * __expf(sGam[i] - gj) : 0.f);
+    for (int h8 = 0; h8 < 2; ++h8) {
+      v8 a = *(const v8*)&sAwT[j * LDT + i0 + 8 * h8], o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        int i = i0 + 8 * h8 + e;
+        o[e] = (T)((i >= j) ? (float)a[e] * __expf(sGam[i] - gj) : 0.f);
+      }
+      *(v8*)&sS1[j * LDT + i0 + 8 * h8] = o;
     }
   }
   __syncthreads();
-  f32x16 dvb[TV];
-#pragma unroll
-  for (int t = 0; t < TV; ++t) dvb[t] = zero16();
-  mm64<T, TV>(sS1, LDT, sTr1, LDT, rw, cw * TV * 32, rw * 32, BT, lane, dvb);
+
+  const int jrow = rw * 32 + (lane & 31);      // this lane's time row in the transposed products
+  const float bj = sBeta[jrow];
+  // ================= value side: d(vb) = Au^T du ; dAu = (du v^T) diag(beta)
+  const int ib = wave >> 1, jb = wave & 1;     // score quadrants: waves 0,2,3 -> (0,0),(1,0),(1,1)
   f32x16 dAu = zero16();
-  if (jb <= ib) {
-    for (int vs = 0; vs < V; vs += 16)
-      dAu = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, vs, lane), lds_frag32<T>(sRow2, LDD, jb * 32, vs, lane),
-                            dAu);
-  }
-  // dv = beta d(vb);  dbeta += sum_v d(vb) * v   (v = vb / beta is re-read from HBM)
   {
-    T* dvp = (T*)p.dv + (row0 * H + hh) * (int64_t)V;
-    const T* vp = (const T*)p.v + (row0 * H + hh) * (int64_t)V;
-    float part[16];
+    f32x16 dvb[TV];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) part[r] = 0.f;
+    for (int t = 0; t < TV; ++t) dvb[t] = zero16();
+    // Au^T is upper triangular: row j contracts over i >= j
+    mm64t<T, TV>(sTr1, LDT, cw * TV * 32, sS1, LDT, rw, rw * 32, BT, lane, dvb);
+    if (jb <= ib) {
+      for (int vs = 0; vs < V; vs += 16)
+        dAu = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, vs, lane), lds_frag32<T>(sRow2, LDD, jb * 32, vs, lane),
+                              dAu);
+      const float bcol = sBeta[jb * 32 + (lane & 31)];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dAu[r] *= bcol;
+    }
+    // dv = beta d(vb);  dbeta += sum_v d(vb) * v
+    float part = 0.f;
+    T* dvp = (T*)p.dv + ((row0 + jrow) * H + hh) * (int64_t)V;
 #pragma unroll
     for (int t = 0; t < TV; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int j = rw * 32 + c32_row(r, lane);
-        int col = (cw * TV + t) * 32 + (lane & 31);
-        if (j < L) {
-          dvp[(int64_t)j * H * V + col] = (T)(dvb[t][r] * sBeta[j]);
-          part[r] += dvb[t][r] * (float)vp[(int64_t)j * H * V + col];
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int col = (cw * TV + t) * 32 + 8 * r4 + 4 * (lane >> 5);
+        v4 vv = *(const v4*)&sRow2[jrow * LDD + col], o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float d = dvb[t][4 * r4 + e];
+          part += d * (float)vv[e];
+          o[e] = (T)(d * bj);
         }
+        if (jrow < L) *(v4*)(dvp + col) = o;
       }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float s = part[r];
-#pragma unroll
-      for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-      if ((lane & 31) == 0) atomicAdd(&sDb[rw * 32 + c32_row(r, lane)], s);
-    }
+    part += __shfl_xor(part, 32, 64);
+    if (lane < 32) atomicAdd(&sDb[jrow], part);
   }
-  __syncthreads();  // Au^T and the value tiles are consumed
+  __syncthreads();  // the value tiles and Au^T are consumed
+  // ================= key side: d(kb)_1 = Aw^T dw ; dAw_1 = (dw k^T) diag(beta)
+  IOK::put_rows(sRow1, LDD, tid, rdw);
+  IOK::put_tr(sTr1, tid, rdw);
+  IOK::put_rows(sRow2, LDD, tid, rk);
+  __syncthreads();
+  f32x16 dkb[TK];   // d(kb)^T: columns (cw*TK+t)*32.., time row jrow
+#pragma unroll
+  for (int t = 0; t < TK; ++t) dkb[t] = zero16();
+  mm64t<T, TK>(sTr1, LDT, cw * TK * 32, sAwT, LDT, rw, rw * 32, BT, lane, dkb);
+  f32x16 dA = zero16();
+  if (jb <= ib) {
+    for (int ks = 0; ks < K; ks += 16)
+      dA = Elem<T>::mfma32(lds_frag32<T>(sRow1, LDD, ib * 32, ks, lane), lds_frag32<T>(sRow2, LDD, jb * 32, ks, lane), dA);
+    const float bcol = sBeta[jb * 32 + (lane & 31)];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dA[r] *= bcol;
+  }
   // ================= dA_total (strictly lower) and the gate gradient through Gamma
   if (jb <= ib) {
     const int j = jb * 32 + (lane & 31);
@@ -900,7 +921,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
     // quadrant (0,1) lies strictly above the diagonal
     for (int e = lane; e < 32 * 32; e += 64) sS1[(e >> 5) * LDT + 32 + (e & 31)] = (T)0.f;
   }
-  __syncthreads();
+  __syncthreads();  // dA complete; dw^T consumed
+  IOK::put_tr(sTr1, tid, rk);   // k^T
   // ================= X1 = dA Aw^T  (stored transposed), dM = -strict_lower(Aw^T X1)
   {
     // wave (rw, cw): rows a = 32rw.., cols j = 32cw..  ; contraction over b
@@ -919,60 +941,66 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   }
   __syncthreads();
   {
-    f32x16 m = zero16();
-    for (int as = 0; as < BT; as += 16)
-      m = Elem<T>::mfma32(lds_frag32<T>(sAwT, LDT, rw * 32, as, lane), lds_frag32<T>(sS2, LDT, cw * 32, as, lane), m);
+    // both orientations of Aw^T X1 so that dM and dM^T are written with 8-byte vectors
+    f32x16 m = zero16(), mt = zero16();
+    for (int as = 0; as < BT; as += 16) {
+      v8 fa = lds_frag32<T>(sAwT, LDT, rw * 32, as, lane), fx = lds_frag32<T>(sS2, LDT, cw * 32, as, lane);
+      m = Elem<T>::mfma32(fa, fx, m);     // rows i = 32rw.. (registers), column j = 32cw + lane%32
+      mt = Elem<T>::mfma32(fx, fa, mt);   // rows j = 32cw.. (registers), column i = 32rw + lane%32
+    }
     __syncthreads();  // every wave has read dA (sS1) and X1^T (sS2)
-    const int j = cw * 32 + (lane & 31);
+    {
+      const int j = cw * 32 + (lane & 31);
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      int i0 = rw * 32 + 8 * a + 4 * (lane >> 5);
-      v4 x;
+      for (int a = 0; a < 4; ++a) {
+        int i0 = rw * 32 + 8 * a + 4 * (lane >> 5);
+        v4 x;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        float val = (j < i0 + b) ? -m[4 * a + b] : 0.f;
-        x[b] = (T)val;
-        sS1[(i0 + b) * LDT + j] = (T)val;     // dM[i][j]
+        for (int b = 0; b < 4; ++b) x[b] = (T)((j < i0 + b) ? -m[4 * a + b] * sBeta[i0 + b] : 0.f);
+        *(v4*)&sS2[j * LDT + i0] = x;           // (dM^T diag(beta))[j][i]
       }
-      *(v4*)&sS2[j * LDT + i0] = x;           // dM^T[j][i]
+      const int i = rw * 32 + (lane & 31);
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        int j0 = cw * 32 + 8 * a + 4 * (lane >> 5);
+        v4 x;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) x[b] = (T)((j0 + b < i) ? -mt[4 * a + b] : 0.f);
+        *(v4*)&sS1[i * LDT + j0] = x;           // dM[i][j]
+      }
     }
   }
-  // ================= d(kb) += dM k ; dk = beta d(kb) + dM^T kb ; dbeta += sum_k d(kb) * k
-  load_rows(p.k, K, false, nullptr, sTr1);     // k^T (kb^T still in sTr2)
   __syncthreads();
+  // ================= d(kb) += dM k ; dk = beta d(kb) + (dM^T diag(beta)) k ; dbeta += sum_k d(kb) * k
   // dM is strictly lower: row i contracts over j < i ; dM^T row j contracts over i > j
-  mm64<T, TK>(sS1, LDT, sTr1, LDT, rw, cw * TK * 32, 0, (rw + 1) * 32, lane, dkb);
+  mm64t<T, TK>(sTr1, LDT, cw * TK * 32, sS1, LDT, rw, 0, (rw + 1) * 32, lane, dkb);
   f32x16 dk2[TK];
 #pragma unroll
   for (int t = 0; t < TK; ++t) dk2[t] = zero16();
-  mm64<T, TK>(sS2, LDT, sTr2, LDT, rw, cw * TK * 32, rw * 32, BT, lane, dk2);
+  mm64t<T, TK>(sTr1, LDT, cw * TK * 32, sS2, LDT, rw, rw * 32, BT, lane, dk2);
   {
-    T* dkp = (T*)p.dk + (row0 * H + hh) * (int64_t)K;
-    const T* kp = (const T*)p.k + (row0 * H + hh) * (int64_t)K;
-    const T* dip = p.dk_in ? (const T*)p.dk_in + (row0 * H + hh) * (int64_t)K : nullptr;
-    float part[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) part[r] = 0.f;
+    float part = 0.f;
+    const int64_t rowoff = ((row0 + jrow) * H + hh) * (int64_t)K;
+    T* dkp = (T*)p.dk + rowoff;
+    const T* dip = p.dk_in ? (const T*)p.dk_in + rowoff : nullptr;
 #pragma unroll
     for (int t = 0; t < TK; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int j = rw * 32 + c32_row(r, lane);
-        int col = (cw * TK + t) * 32 + (lane & 31);
-        if (j < L) {
-          int64_t o = (int64_t)j * H * K + col;
-          float val = dkb[t][r] * sBeta[j] + dk2[t][r] + (dip ? (float)dip[o] : 0.f);
-          dkp[o] = (T)val;
-          part[r] += dkb[t][r] * (float)kp[o];
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int col = (cw * TK + t) * 32 + 8 * r4 + 4 * (lane >> 5);
+        v4 kk = *(const v4*)&sRow2[jrow * LDD + col], o;
+        v4 din = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        if (dip && jrow < L) din = *(const v4*)(dip + col);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float d = dkb[t][4 * r4 + e];
+          part += d * (float)kk[e];
+          o[e] = (T)(d * bj + dk2[t][4 * r4 + e] + (float)din[e]);
         }
+        if (jrow < L) *(v4*)(dkp + col) = o;
       }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float s = part[r];
-#pragma unroll
-      for (int off = 16; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-      if ((lane & 31) == 0) atomicAdd(&sDb[rw * 32 + c32_row(r, lane)], s);
-    }
+    part += __shfl_xor(part, 32, 64);
+    if (lane < 32) atomicAdd(&sDb[jrow], part);
   }
   __syncthreads();
   if (tid < L) {
