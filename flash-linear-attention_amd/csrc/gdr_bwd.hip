@@ -766,14 +766,16 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   typedef TileIO<T, K> IOK;
   typedef TileIO<T, V> IOV;
   typedef TileIO<T, BT> IOA;
-  __shared__ __attribute__((aligned(16))) T sRow1[BT * LDD];   // du, then dw          row-major [t][d]
+  __shared__ __attribute__((aligned(16))) T sRow1[BT * LDD];   // du, then dw          row-major [t][d]; later sS2
   __shared__ __attribute__((aligned(16))) T sRow2[BT * LDD];   // v,  then k           row-major
   __shared__ __attribute__((aligned(16))) T sTr1[D * LDT];     // du^T, dw^T, k^T      [d][t]
   __shared__ __attribute__((aligned(16))) T sAw[BT * LDT];     // Aw [i][j]
   __shared__ __attribute__((aligned(16))) T sAwT[BT * LDT];    // Aw^T
   __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA (masked) -> dM
-  __shared__ __attribute__((aligned(16))) T sS2[BT * LDT];     // X1^T -> dM^T diag(beta)
   __shared__ float sBeta[BT], sGam[BT], sDb[BT], sDg[BT];
+  // X1^T, then dM^T diag(beta): lives in the du/dw tile, which is dead once dA has been formed
+  // (two workgroups then fit a CU)
+  T* sS2 = sRow1;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H;

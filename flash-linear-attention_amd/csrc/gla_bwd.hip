@@ -414,7 +414,7 @@ struct BDqkgParams {
 
 // grid (chunks, H, K/64): one workgroup per 64-wide slice of the key dim.
 template <typename T, typename GT, int V>
-__global__ __launch_bounds__(256) void gla_bwd_dqkg_kernel(BDqkgParams p) {
+__global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDV = V + 8;
@@ -479,18 +479,6 @@ __global__ __launch_bounds__(256) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   // operand fragments: wave (rw, cw) produces rows 32rw.., key columns kb + 32cw..
   const int rw = wave >> 1, cw = wave & 1;
   const int kt32 = kb / 32 + cw;
-  v8 hf[VT32][2], dhf[VT32][2];
-  {
-    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
-#pragma unroll
-    for (int vt = 0; vt < VT32; ++vt) {
-      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
-      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
-      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
-      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
-      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
-    }
-  }
   // ---- prefix sums of the gates over the 16 row groups
   float G[4][4], glast[4];
   {
@@ -545,6 +533,19 @@ __global__ __launch_bounds__(256) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     *(v4*)&sQtT[(c4 + j) * LDT + rg * 4] = qt;
   }
   __syncthreads();
+  // state fragments for the inter-chunk terms: issued here, consumed after the score phase
+  v8 hf[VT32][2], dhf[VT32][2];
+  {
+    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int vt = 0; vt < VT32; ++vt) {
+      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
+      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
+      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
+      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
+      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
+    }
+  }
   // ---- dA = tril(do v^T) in both orientations (each gives 8-byte LDS writes)
   {
     const int ib = wave >> 1, jb = wave & 1;
