@@ -237,7 +237,15 @@ def bench_backward(device, steps=10):
     k = mk(B, T, H, K).bfloat16().requires_grad_()
     gk = (F.logsigmoid(mk(B, T, H, K)) / 16).requires_grad_()
 
+    leaves = []
+
+    def clear():
+        # gradients are produced, not accumulated: a step is one forward + one backward of the operator
+        for x in leaves:
+            x.grad = None
+
     def gla_step():
+        clear()
         o, ht = chunk_gla(q, k, v, gk, initial_state=h0, output_final_state=True, head_first=False)
         torch.autograd.backward((o, ht), (do, dht))
 
@@ -246,9 +254,12 @@ def bench_backward(device, steps=10):
     beta = mk(B, T, H).sigmoid().requires_grad_()
 
     def gdr_step():
+        clear()
         o, ht = chunk_gated_delta_rule(q, kn, v, g, beta, initial_state=h0, output_final_state=True,
                                        head_first=False)
         torch.autograd.backward((o, ht), (do, dht))
+
+    leaves.extend([q, k, v, gk, h0, kn, g, beta])
 
     for name, fn in (("chunk_gla", gla_step), ("chunk_gated_delta_rule", gdr_step)):
         us = event_avg_us(fn, steps)

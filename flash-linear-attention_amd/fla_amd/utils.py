@@ -7,6 +7,7 @@ The reference caches bookkeeping results keyed on ``data_ptr``
 """
 import ctypes
 import functools
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -28,10 +29,26 @@ autocast_custom_fwd = functools.partial(torch.amp.custom_fwd, device_type="cuda"
 autocast_custom_bwd = functools.partial(torch.amp.custom_bwd, device_type="cuda")
 
 
+# Host copies of device-resident offsets, keyed by tensor identity: a model passes the same
+# cu_seqlens tensor to every layer, and reading it back costs a device synchronisation.
+# An entry is valid only for the very same, unmodified tensor object.
+_HOST_OFFSETS_CACHE = {}
+
+
 def _host_offsets(offsets) -> Tuple[int, ...]:
-    if isinstance(offsets, torch.Tensor):
-        return tuple(int(x) for x in offsets.detach().cpu().tolist())
-    return tuple(int(x) for x in offsets)
+    if not isinstance(offsets, torch.Tensor):
+        return tuple(int(x) for x in offsets)
+    key = id(offsets)
+    hit = _HOST_OFFSETS_CACHE.get(key)
+    if hit is not None:
+        ref, version, host = hit
+        if ref() is offsets and version == offsets._version:
+            return host
+    host = tuple(int(x) for x in offsets.detach().cpu().tolist())
+    if len(_HOST_OFFSETS_CACHE) > 256:
+        _HOST_OFFSETS_CACHE.clear()
+    _HOST_OFFSETS_CACHE[key] = (weakref.ref(offsets), offsets._version, host)
+    return host
 
 
 @functools.lru_cache(maxsize=64)
@@ -69,9 +86,27 @@ def prepare_chunk_offsets(offsets, chunk_size: int, device=None) -> torch.Tensor
 
 
 class VarlenPlan:
-    """Everything the kernels need to address a packed batch."""
+    """Everything the kernels need to address a packed batch.  Plans are cached per offsets
+    tensor (same object, unmodified), so the layers of a model that share one ``cu_seqlens``
+    build the device tables once."""
 
-    def __init__(self, offsets: torch.Tensor, chunk_size: int):
+    _cache = {}
+
+    def __new__(cls, offsets: torch.Tensor, chunk_size: int):
+        key = (id(offsets), int(chunk_size))
+        hit = cls._cache.get(key)
+        if hit is not None:
+            ref, version, plan = hit
+            if ref() is offsets and version == offsets._version:
+                return plan
+        plan = super().__new__(cls)
+        plan._build(offsets, chunk_size)
+        if len(cls._cache) > 256:
+            cls._cache.clear()
+        cls._cache[key] = (weakref.ref(offsets), offsets._version, plan)
+        return plan
+
+    def _build(self, offsets: torch.Tensor, chunk_size: int):
         host = _host_offsets(offsets)
         idx, co = _chunk_tables(host, int(chunk_size))
         dev = offsets.device
