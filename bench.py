@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-A step is one chunk_gla forward over BASELINE config 1 (B=8, T=4096, H=16,
+A step is one chunk_gla forward on the headline workload (B=8, T=4096, H=16,
 K=V=128, bf16 q/k/v, fp32 log-gates and state, initial state given, final state
 returned), inputs resident in HBM.  Prints ONE JSON line:
 
@@ -13,9 +13,9 @@ returned), inputs resident in HBM.  Prints ONE JSON line:
                    here with HIP events on the launch stream
 * cpu_baseline     the oracle's fp32 naive recurrence timed on the host cores on
                    a bounded sample of the same workload
-* extra            the other measured rows: the T=1 decode steps of config 3,
-                   chunk_gated_delta_rule forward on config 2, forward + backward
-                   of both chunk operators on config 4
+* extra            the other measured rows: the T=1 decode steps (B=256, H=32),
+                   chunk_gated_delta_rule forward on a packed batch, forward + backward
+                   of both chunk operators (B=4, T=4096)
 """
 import argparse
 import json
@@ -145,7 +145,7 @@ def bench_gla(device, steps, warmup):
 
 
 def bench_decode(device, steps=1000):
-    """BASELINE config 3: B=256, H=32, K=V=128 single-token step, state in place."""
+    """Decode workload: B=256, H=32, K=V=128 single-token step, state in place."""
     import torch
     import torch.nn.functional as F
     from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
@@ -185,7 +185,7 @@ def bench_decode(device, steps=1000):
 
 
 def bench_gdr(device, steps=20):
-    """chunk_gated_delta_rule forward: BASELINE config 2 (packed, 12 sequences, 32768 tokens)
+    """chunk_gated_delta_rule forward: the packed workload (packed, 12 sequences, 32768 tokens)
     and the fixed-length shape B=8, T=4096 of the headline metric."""
     import torch
     import torch.nn.functional as F
@@ -222,7 +222,7 @@ def bench_gdr(device, steps=20):
 
 
 def bench_backward(device, steps=10):
-    """BASELINE config 4: forward + backward of both chunk operators, B=4, T=4096, H=16, K=V=128."""
+    """Training workload: forward + backward of both chunk operators, B=4, T=4096, H=16, K=V=128."""
     import torch
     import torch.nn.functional as F
     from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
@@ -326,7 +326,7 @@ def main():
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "chunk_gla forward, BASELINE config 1: B=8 T=4096 H=16 K=V=128, bf16 q/k/v, "
+        "config": {"workload": "chunk_gla forward: B=8 T=4096 H=16 K=V=128, bf16 q/k/v, "
                                "fp32 log-gates logsigmoid(N(0,1))/16, fp32 initial state, final state returned"},
         "roofline": roofline,
         "cpu_baseline": None if a.no_cpu_baseline else cpu_baseline(cfg),

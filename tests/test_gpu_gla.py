@@ -24,7 +24,7 @@ def _run(device, q, k, v, g, h0, offsets=None, head_first=False, scale=None):
 
 
 def test_chunk_gla_config0(device):
-    """BASELINE config 0 shape (B=2, T=256, H=4, K=V=64, zero initial state), bf16 storage."""
+    """The CPU-runnable reference shape (B=2, T=256, H=4, K=V=64, zero initial state), bf16 storage."""
     from oracle.recurrent import naive_recurrent_gla
     q, k, v, g, _ = gla_inputs(2, 256, 4, 64, 64, seed=0, h0=False)
     print("chunk_gla config0", flush=True)
