@@ -228,6 +228,7 @@ struct BDvParams {
   const void* g;
   const void* dout;
   const void* dhf;
+  const int* wide;   // [chunks, H] or null: chunks whose intra-chunk part is left to the exact kernel
   void* dv;
   const int64_t* offsets;
   const int64_t* indices;
@@ -257,6 +258,9 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
+  // gates beyond the single-reference range: the scores are left out here and added by
+  // gla_bwd_intra_exact_kernel
+  const bool flagged = p.wide && p.wide[cl.cglob * H + hh];
   const int rg = tid / CG, c4 = (tid % CG) * 4;
   float gq[RPT][4], qq[RPT][4], kk[RPT][4];
 #pragma unroll
@@ -357,7 +361,7 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
         int i0 = qi * 32 + 8 * a + 4 * (lane >> 5);
         v4 x;
 #pragma unroll
-        for (int b = 0; b < 4; ++b) x[b] = (T)((j <= i0 + b) ? s[4 * a + b] : 0.f);
+        for (int b = 0; b < 4; ++b) x[b] = (T)((j <= i0 + b && !flagged) ? s[4 * a + b] : 0.f);
         *(v4*)&sPT[j * LDT + i0] = x;
       }
     }
@@ -401,6 +405,7 @@ struct BDqkgParams {
   const void* hT;     // forward states, FLA_H_FRAGMENT_T
   const void* dhtf;   // dH, FLA_H_FRAGMENT_T
   const float* hdh;   // [V/32][chunks][H][K]
+  const int* wide;    // [chunks, H] or null: chunks whose intra-chunk part is left to the exact kernel
   void* dq;
   void* dk;
   float* dg;
@@ -447,6 +452,9 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
+  // gates beyond the single-reference range: dA is left out here and the intra-chunk terms are
+  // added by gla_bwd_intra_exact_kernel
+  const bool flagged = p.wide && p.wide[cl.cglob * H + hh];
   // ---- loads: q,k,g slice as 4 rows x 4 cols per lane; do, v whole rows in 16-byte pieces
   const int rg = tid >> 4, c4 = (tid & 15) * 4;
   float gq[4][4], qq[4][4], kk[4][4];
@@ -566,9 +574,9 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
           int i1 = ib * 32 + r0 + b, j1 = jb * 32 + c;      // s1 element (i1, j1)
-          x1[b] = (T)((j1 <= i1) ? s1[4 * a + b] : 0.f);
+          x1[b] = (T)((j1 <= i1 && !flagged) ? s1[4 * a + b] : 0.f);
           int j2 = jb * 32 + r0 + b, i2 = ib * 32 + c;      // s2 element (j2, i2)
-          x2[b] = (T)((j2 <= i2) ? s2[4 * a + b] : 0.f);
+          x2[b] = (T)((j2 <= i2 && !flagged) ? s2[4 * a + b] : 0.f);
         }
         *(v4*)&sdAT[(jb * 32 + c) * LDT + ib * 32 + r0] = x1;  // dA^T[j][i..i+3]
         *(v4*)&sdA[(ib * 32 + c) * LDT + jb * 32 + r0] = x2;   // dA[i][j..j+3]
@@ -671,9 +679,179 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Intra-chunk part of the backward for chunks whose cumulative log-gate leaves the range in
+// which one reference point per chunk is exact.  gla_bwd_dv_kernel and gla_bwd_dqkg_kernel
+// leave the score terms of such chunks out; this kernel adds them with pairwise exponents
+// G_i - G_j <= 0, the arithmetic of the reference's diagonal sub-blocks
+// (fla/ops/gla/chunk.py:409-567):
+//   A_ij  = s sum_k q_ik k_jk e^{G_ik-G_jk},  dA_ij = do_i . v_j            (j <= i)
+//   dv_j += sum_{i>=j} A_ij do_i
+//   dq_ik += s sum_{j<=i} dA_ij k_jk e^{G_ik-G_jk},  dk_jk += s sum_{i>=j} dA_ij q_ik e^{G_ik-G_jk}
+//   dg_ik += sum_{t>=i} (q_tk dq'_tk - k_tk dk'_tk)          (dq', dk': the terms added here)
+// Plain fp32 arithmetic on the vector ALU: it only runs for flagged chunks.
+struct BExactParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const void* dout;
+  const int* wide;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* dg;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+};
+
+template <typename T, typename GT, int K, int V>
+__global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p) {
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDG = K + 1, LDQ = K + 8, LDVV = V + 8, LDA = BT + 1;
+  constexpr int VD_BYTES = 2 * BT * LDVV * 2;
+  constexpr int X_BYTES = BT * LDG * 4;
+  const int H = p.H;
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  if (p.wide[cl.cglob * H + hh] == 0) return;  // workgroup-uniform
+  __shared__ float sG[BT * LDG];
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDQ];
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDQ];
+  __shared__ __attribute__((aligned(16))) char sVD[VD_BYTES > X_BYTES ? VD_BYTES : X_BYTES];  // v | do, later x
+  __shared__ float sA[BT * LDA];
+  __shared__ float sdA[BT * LDA];
+  T* sV = (T*)sVD;
+  T* sDo = sV + BT * LDVV;
+  float* sX = (float*)sVD;
+  const int tid = threadIdx.x;
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+  const int64_t strideK = (int64_t)H * K, strideV = (int64_t)H * V;
+  const int64_t baseK = (row0 * H + hh) * (int64_t)K, baseV = (row0 * H + hh) * (int64_t)V;
+
+  for (int e = tid; e < BT * (K / 4); e += 256) {
+    int row = e / (K / 4), c4 = (e % (K / 4)) * 4;
+    float gv[4] = {0.f, 0.f, 0.f, 0.f};
+    v4 qv = {(T)0.f, (T)0.f, (T)0.f, (T)0.f}, kv = qv;
+    if (row < L) {
+      int64_t off = baseK + row * strideK + c4;
+      Load<GT>::x4((const GT*)p.g + off, gv);
+      qv = *(const v4*)((const T*)p.q + off);
+      kv = *(const v4*)((const T*)p.k + off);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sG[row * LDG + c4 + j] = gv[j];
+    *(v4*)&sQ[row * LDQ + c4] = qv;
+    *(v4*)&sK[row * LDQ + c4] = kv;
+  }
+  for (int e = tid; e < BT * (V / 4); e += 256) {
+    int row = e / (V / 4), c4 = (e % (V / 4)) * 4;
+    v4 vv = {(T)0.f, (T)0.f, (T)0.f, (T)0.f}, dv = vv;
+    if (row < L) {
+      int64_t off = baseV + row * strideV + c4;
+      vv = *(const v4*)((const T*)p.v + off);
+      dv = *(const v4*)((const T*)p.dout + off);
+    }
+    *(v4*)&sV[row * LDVV + c4] = vv;
+    *(v4*)&sDo[row * LDVV + c4] = dv;
+  }
+  __syncthreads();
+  // prefix sums of the gates along time, one channel per thread
+  for (int c = tid; c < K; c += 256) {
+    float run = 0.f;
+    for (int t = 0; t < BT; ++t) {
+      run += sG[t * LDG + c];
+      sG[t * LDG + c] = run;
+    }
+  }
+  __syncthreads();
+  // A and dA, one (i, j) pair at a time
+  for (int e = tid; e < BT * BT; e += 256) {
+    int i = e >> 6, j = e & 63;
+    float a = 0.f, da = 0.f;
+    if (j <= i && i < L) {
+      for (int c = 0; c < K; ++c)
+        a += (float)sQ[i * LDQ + c] * (float)sK[j * LDQ + c] * __expf(sG[i * LDG + c] - sG[j * LDG + c]);
+      for (int c = 0; c < V; ++c) da += (float)sDo[i * LDVV + c] * (float)sV[j * LDVV + c];
+    }
+    sA[i * LDA + j] = a * p.scale;
+    sdA[i * LDA + j] = da * p.scale;
+  }
+  __syncthreads();
+  // dv_j += sum_{i>=j} A_ij do_i
+  for (int e = tid; e < BT * (V / 4); e += 256) {
+    int j = e / (V / 4), c4 = (e % (V / 4)) * 4;
+    if (j >= L) continue;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int i = j; i < L; ++i) {
+      float a = sA[i * LDA + j];
+      v4 d = *(const v4*)&sDo[i * LDVV + c4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) acc[x] += a * (float)d[x];
+    }
+    T* dst = (T*)p.dv + baseV + j * strideV + c4;
+    v4 old = *(const v4*)dst, nw;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) nw[x] = (T)((float)old[x] + acc[x]);
+    *(v4*)dst = nw;
+  }
+  __syncthreads();  // v and do are consumed: their storage becomes x = q dq' - k dk'
+  for (int e = tid; e < BT * (K / 4); e += 256) {
+    int r = e / (K / 4), c4 = (e % (K / 4)) * 4;
+    float xq[4] = {0.f, 0.f, 0.f, 0.f}, xk[4] = {0.f, 0.f, 0.f, 0.f};
+    if (r < L) {
+      float dq[4] = {0.f, 0.f, 0.f, 0.f}, dk[4] = {0.f, 0.f, 0.f, 0.f};
+      float gr[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) gr[x] = sG[r * LDG + c4 + x];
+      for (int j = 0; j <= r; ++j) {       // row r as the query row i
+        float da = sdA[r * LDA + j];
+        v4 kj = *(const v4*)&sK[j * LDQ + c4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) dq[x] += da * (float)kj[x] * __expf(gr[x] - sG[j * LDG + c4 + x]);
+      }
+      for (int i = r; i < L; ++i) {        // row r as the key row j
+        float da = sdA[i * LDA + r];
+        v4 qi = *(const v4*)&sQ[i * LDQ + c4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) dk[x] += da * (float)qi[x] * __expf(sG[i * LDG + c4 + x] - gr[x]);
+      }
+      v4 qr = *(const v4*)&sQ[r * LDQ + c4], kr = *(const v4*)&sK[r * LDQ + c4];
+      T* dqp = (T*)p.dq + baseK + r * strideK + c4;
+      T* dkp = (T*)p.dk + baseK + r * strideK + c4;
+      v4 oq = *(const v4*)dqp, ok = *(const v4*)dkp, nq, nk;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        nq[x] = (T)((float)oq[x] + dq[x]);
+        nk[x] = (T)((float)ok[x] + dk[x]);
+        xq[x] = (float)qr[x] * dq[x];
+        xk[x] = (float)kr[x] * dk[x];
+      }
+      *(v4*)dqp = nq;
+      *(v4*)dkp = nk;
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) sX[r * LDG + c4 + x] = xq[x] - xk[x];
+  }
+  __syncthreads();
+  // dg_ik += sum_{t>=i} x_tk, one channel per thread
+  for (int c = tid; c < K; c += 256) {
+    float run = 0.f;
+    for (int t = L - 1; t >= 0; --t) {
+      run += sX[t * LDG + c];
+      p.dg[baseK + t * strideK + c] += run;
+    }
+  }
+}
+
 template <typename T, typename GT>
 int launch_bwd(const void* q, const void* k, const void* v, const void* g, const void* dout, const float* dht,
                const void* hT, void* dhf, void* dhtf, float* hdh, void* dq, void* dk, void* dv, float* dg, float* dh0,
+               const int* wide,
                const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
                int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
   dim3 grid;
@@ -691,7 +869,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   {
-    BDvParams p{q, k, g, dout, dhf, dv, offsets, indices, T_, (int)H, ntfix, scale};
+    BDvParams p{q, k, g, dout, dhf, wide, dv, offsets, indices, T_, (int)H, ntfix, scale};
 #define FLA_CASE(KK, VV)                                                                            \
   if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_dv_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
     FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
@@ -699,12 +877,20 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   {
-    BDqkgParams p{q, k, v, g, dout, hT, dhtf, hdh, dq, dk, dg, offsets, indices, T_, total_chunks,
+    BDqkgParams p{q, k, v, g, dout, hT, dhtf, hdh, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
                   (int)H, (int)K, ntfix, scale};
     dim3 g3(grid.x, grid.y, (unsigned)(K / 64));
     if (V == 64) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 64>), g3, dim3(256), 0, st, p);
     else if (V == 128) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 128>), g3, dim3(256), 0, st, p);
     else return FLA_E_UNSUPPORTED;
+    FLA_CHECK_LAUNCH();
+  }
+  if (wide) {
+    BExactParams p{q, k, v, g, dout, wide, dq, dk, dv, dg, offsets, indices, T_, (int)H, ntfix, scale};
+#define FLA_CASE(KK, VV)                                                                                      \
+  if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_intra_exact_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
+    FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
+#undef FLA_CASE
     FLA_CHECK_LAUNCH();
   }
   return FLA_OK;
@@ -714,8 +900,9 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
 
 extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
                                  const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
-                                 void* dq, void* dk, void* dv, float* dg, float* dh0, const int64_t* offsets,
-                                 const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
+                                 void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                                 const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
+                                 int64_t NT, int qkv_dtype,
                                  int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                  float scale, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag && dh_frag_t && hdh && dq && dk && dv && dg,
@@ -730,8 +917,8 @@ extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, co
               FLA_E_ALIGNMENT);
   hipStream_t st = (hipStream_t)stream;
 #define FLA_BWD(TT, GG)                                                                                           \
-  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag, dh_frag_t, hdh, dq, dk, dv, dg, dh0, offsets, \
-                            indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
+  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag, dh_frag_t, hdh, dq, dk, dv, dg, dh0, wide,   \
+                            offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_BWD(bf16, float);
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_BWD(bf16, bf16);
   if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) FLA_BWD(f16, float);

@@ -43,7 +43,7 @@ SIGNATURES = {
                                                  I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_fused": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
-    "fla_chunk_gla_bwd": (c_int, [P] * 18 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gla_bwd": (c_int, [P] * 19 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 26 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_selftest_mfma": (c_int, [P, P, P, I64, I64, I64, I, P]),
 }

@@ -51,10 +51,12 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
     return o
 
 
-def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True):
+def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,
+                        return_flags=False):
     """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
     With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
-    single-reference range are detected on the device and recomputed exactly."""
+    single-reference range are detected on the device and recomputed exactly; ``return_flags``
+    also returns the int32 ``[chunks, H]`` flags (for the backward pass)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
@@ -75,13 +77,20 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         be.ptr(None if plan is None else plan.chunk_offsets), be.ptr(None if plan is None else plan.seq_order),
         0 if plan is None else plan.NT,
         be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_fused")
+    if return_flags:
+        return o, ht, wide
     return o, ht
 
 
-def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False, fused=True):
-    """Seq-first forward on 64-aligned head dims.  Returns (o, ht, A)."""
+def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False, fused=True,
+                 flags_out=None):
+    """Seq-first forward on 64-aligned head dims.  Returns (o, ht, A); with a list ``flags_out`` the
+    gate-range flags of the fused kernel are appended to it."""
     if fused and not want_A and q.shape[-1] in (64, 128):
-        o, ht = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets)
+        o, ht, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets,
+                                          return_flags=True)
+        if flags_out is not None:
+            flags_out.append(wide)
         return o, ht, None
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     B, T, H, K = q.shape
@@ -127,10 +136,13 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
     return g_cumsum, A, h, ht, o
 
 
-def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets):
+def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
     Returns ``(dq, dk, dv, dg, dh0)``; recomputes the per-chunk states as the
-    reference does (``fla/ops/gla/chunk.py:1239-1253``)."""
+    reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``wide``: the forward's
+    gate-range flags (int32 ``[chunks, H]``); flagged chunks get their intra-chunk terms
+    from the exact kernel.  Without it the result is exact only while the chunk-cumulative
+    log-gate stays within +-80."""
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
@@ -152,8 +164,8 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets):
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
     be.check(be.lib().fla_chunk_gla_bwd(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(dhf), be.ptr(dhtf),
-        be.ptr(hdh), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(offs), be.ptr(idx),
-        be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_bwd")
+        be.ptr(hdh), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
+        be.ptr(idx), be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_bwd")
     return dq, dk, dv, dg, dh0
 
 
@@ -184,9 +196,11 @@ class ChunkGLAFunction(torch.autograd.Function):
             v = _pad_dim(v, VP)
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
-        o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets)
-        # like the reference, keep the inputs and recompute everything else in backward
-        ctx.save_for_backward(q, k, v, g, h0, offsets)
+        flags = []
+        o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets, flags_out=flags)
+        # like the reference, keep the inputs and recompute everything else in backward (plus the
+        # small table of chunks whose gates need the exact intra-chunk arithmetic)
+        ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
@@ -201,7 +215,7 @@ class ChunkGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        q, k, v, g, h0, offsets = ctx.saved_tensors
+        q, k, v, g, h0, offsets, wide = ctx.saved_tensors
         K, V, KP, VP = ctx.dims
         if ctx.head_first:
             do = do.transpose(1, 2)
@@ -211,7 +225,7 @@ class ChunkGLAFunction(torch.autograd.Function):
         do = do.contiguous()
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
-        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide)
         if (KP, VP) != (K, V):
             dq, dk, dg, dv = dq[..., :K], dk[..., :K], dg[..., :K], dv[..., :V]
             if dh0 is not None:

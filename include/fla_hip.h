@@ -225,10 +225,16 @@ int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const voi
  *   hdh     workspace fp32 [V/32, chunks, H, K]
  *   dq, dk [B,T,H,K] and dv [B,T,H,V] in the q/k/v dtype; dg fp32 [B,T,H,K]
  *   (gradient w.r.t. the raw gates); dh0 fp32 [N,H,K,V] or NULL.
+ *   wide    int32 [chunks, H] flags written by fla_chunk_gla_fwd_fused (ws_wide), or
+ *           NULL.  The kernels score a chunk with one reference point (exact while
+ *           the chunk-cumulative log-gate stays within +-80); for flagged chunks the
+ *           intra-chunk terms are instead added by a fourth launch with pairwise
+ *           exponents <= 0 (the reference's sub-block arithmetic,
+ *           fla/ops/gla/chunk.py:409-567).
  * ---------------------------------------------------------------------- */
 int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
                       const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
-                      void* dq, void* dk, void* dv, float* dg, float* dh0,
+                      void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
                       const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                       int qkv_dtype, int gate_dtype,
                       int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,

@@ -212,3 +212,36 @@ def test_chunk_gla_extreme_gates_mixed_varlen(device):
     ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True, offsets=offs.tolist())
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("normalizer", [0.05, 0.3])
+def test_chunk_gla_backward_extreme_gates(device, normalizer):
+    """Backward with gates far outside the single-reference range (the reference sweeps
+    normalizer 0.05 for the gradients too, tests/ops/test_gla.py:90-146): the flagged chunks get
+    their intra-chunk terms from the exact pairwise kernel."""
+    B, T, H, K, V = 2, 200, 2, 128, 128
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=81, normalizer=normalizer, h0_std=1.0)
+    gen = torch.Generator().manual_seed(8)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    print(f"chunk_gla backward extreme gates normalizer={normalizer} min g={g.min().item():.1f}", flush=True)
+    got = _grads_dev(device, q, k, v, g, h0, do, dht)
+    ref = _grads_ref(q, k, v, g, h0, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (1e-2, 1e-2, 1e-2, 2e-2, 5e-3)):
+        assert_close(name, r, x, tol)
+
+
+def test_chunk_gla_backward_extreme_gates_mixed_varlen(device):
+    """Only some chunks and channels are flagged; packed batch, K != V."""
+    gen = torch.Generator().manual_seed(82)
+    T, N = 500, 3
+    offs = random_offsets(T, N, gen, min_len=70)
+    q, k, v, g, h0 = gla_inputs(1, T, 2, 64, 128, seed=82, N=N, normalizer=16.0)
+    g[:, 150:290, :, :17] *= 400.0
+    do = torch.randn(1, T, 2, 128, generator=gen).bfloat16()
+    dht = torch.randn(N, 2, 64, 128, generator=gen) * 0.1
+    print(f"chunk_gla backward mixed extreme gates offs={offs.tolist()}", flush=True)
+    got = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    ref = _grads_ref(q, k, v, g, h0, do, dht, offsets=offs.tolist())
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (1e-2, 1e-2, 1e-2, 2e-2, 5e-3)):
+        assert_close(name, r, x, tol)
