@@ -1,0 +1,101 @@
+"""GPU: storage types other than the default (bf16 q/k/v, fp32 gates, fp32 state): fp16 q/k/v,
+gates / beta / initial state in the q/k/v type, as the reference's own tests build them
+(tests/ops/test_gla.py:110-121 draws g and h0 in the test dtype; tests/ops/test_gated_delta.py:180-192
+draws beta in it).  Forward and backward against the fp32 naive recurrences."""
+import pytest
+import torch
+
+from helpers import assert_close, gdr_inputs, gla_inputs, random_offsets
+from test_gpu_gdr import NAMES as GDR_NAMES, TOLS as GDR_TOLS, _grads_dev as gdr_grads_dev, _grads_ref as gdr_grads_ref
+from test_gpu_gla import _grads_dev as gla_grads_dev, _grads_ref as gla_grads_ref
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_storage_types(device, dtype, varlen):
+    """q, k, v, g, h0 and the incoming gradients all in `dtype`."""
+    T, H, K, V = 300, 2, 128, 128
+    gen = torch.Generator().manual_seed(3)
+    offs = random_offsets(T, 3, gen, min_len=1) if varlen else None
+    B, N = (1, 3) if varlen else (2, 2)
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=71, dtype=dtype, normalizer=16.0, N=N, h0_std=1.0)
+    g, h0 = g.to(dtype), h0.to(dtype)
+    do = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    dht = (torch.randn(N, H, K, V, generator=gen) * 0.1)
+    print(f"chunk_gla storage {dtype} varlen={varlen}", flush=True)
+    got = gla_grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    ref = gla_grads_ref(q, k, v, g, h0, do, dht, offsets=None if offs is None else offs.tolist())
+    # gradients of tensors stored in 16 bits are rounded once more on the way out
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (8e-3, 8e-3, 8e-3, 1.2e-2, 8e-3)):
+        assert x.dtype == dtype, (name, x.dtype)
+        assert_close(name, r, x, tol)
+
+    from fla_amd.ops.gla import chunk_gla
+    from oracle.recurrent import naive_recurrent_gla
+    dev = lambda x: None if x is None else x.to(device)
+    o, ht = chunk_gla(dev(q), dev(k), dev(v), dev(g), initial_state=dev(h0), output_final_state=True,
+                      offsets=dev(offs), head_first=False)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gdr_storage_types(device, dtype, varlen):
+    """q, k, v, beta and the incoming gradient in `dtype`; log-gates and state fp32 as in the reference's test."""
+    T, H, K, V = 300, 2, 128, 128
+    gen = torch.Generator().manual_seed(4)
+    offs = random_offsets(T, 3, gen, min_len=1) if varlen else None
+    B, N = (1, 3) if varlen else (2, 2)
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=72, dtype=dtype, N=N, h0_std=1.0)
+    beta = beta.to(dtype)
+    do = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    dht = torch.randn(N, H, K, V, generator=gen) * 0.1
+    print(f"chunk_gdr storage {dtype} varlen={varlen}", flush=True)
+    got = gdr_grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs)
+    ref = gdr_grads_ref(q, k, v, g, beta, h0, do, dht, offsets=None if offs is None else offs.tolist())
+    for name, r, x, tol in zip(GDR_NAMES, ref, got, GDR_TOLS):
+        assert_close(name, r, x, tol)
+    assert got[0].dtype == dtype and got[4].dtype == dtype and got[3].dtype == torch.float32
+
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    dev = lambda x: None if x is None else x.to(device)
+    o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), initial_state=dev(h0),
+                                   output_final_state=True, offsets=dev(offs), head_first=False)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    assert o.dtype == dtype and ht.dtype == torch.float32
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_fused_recurrent_storage_types(device, dtype):
+    """The decode step and a short prefill in every storage type the reference's tests use
+    (tests/ops/test_gla.py:33 runs fused_recurrent_gla in fp32)."""
+    from fla_amd.ops.gla import fused_recurrent_gla
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule, naive_recurrent_gla
+    dev = lambda x: None if x is None else x.to(device)
+    tol = 1e-4 if dtype == torch.float32 else 1e-2
+    for T in (1, 40):
+        q, k, v, g, h0 = gla_inputs(2, T, 3, 128, 128, seed=73 + T, dtype=dtype, normalizer=4.0, h0_std=1.0)
+        print(f"fused_recurrent_gla {dtype} T={T}", flush=True)
+        o, ht = fused_recurrent_gla(dev(q), dev(k), dev(v), gk=dev(g.to(dtype)), initial_state=dev(h0),
+                                    output_final_state=True, head_first=False)
+        ro, rht = naive_recurrent_gla(q, k, v, g.to(dtype), initial_state=h0, output_final_state=True)
+        assert_close("o", ro, o, tol)
+        assert_close("ht", rht, ht, 5e-3 if dtype != torch.float32 else 1e-5)
+        q, k, v, g, beta, h0 = gdr_inputs(2, T, 3, 128, 128, seed=74 + T, dtype=dtype, h0_std=1.0)
+        print(f"fused_recurrent_gated_delta_rule {dtype} T={T}", flush=True)
+        o, ht = fused_recurrent_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta.to(dtype)), initial_state=dev(h0),
+                                                 output_final_state=True, head_first=False)
+        ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta.to(dtype), initial_state=h0, output_final_state=True)
+        assert_close("o", ro, o, tol)
+        assert_close("ht", rht, ht, 5e-3 if dtype != torch.float32 else 1e-5)
