@@ -116,10 +116,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     const int pw = wave - 4;
     const int rg = lane & 15;
     const int kc = pw * CPW + (lane >> 4) * CPL;
-    const int64_t kstride = (int64_t)H * K;
-    const T* qp = (const T*)p.q + (sp.bos * H + hh) * (int64_t)K + kc;
-    const T* kp = (const T*)p.k + (sp.bos * H + hh) * (int64_t)K + kc;
-    const GT* gp = (const GT*)p.g + (sp.bos * H + hh) * (int64_t)K + kc;
     typedef GT gvec __attribute__((ext_vector_type(CPL)));
     typedef T kvec __attribute__((ext_vector_type(CPL)));
     struct Regs {
@@ -127,15 +123,48 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       kvec q[RPT];
       kvec k[RPT];
     };
-    // Loads are unconditional: rows past the end of the sequence are redirected to its last
-    // row and zeroed afterwards (only a sequence's last chunk can be short), so the compiler
-    // is free to batch and interleave them.
-    const int64_t last_row = sp.len - 1;
-    auto row_of = [&](int64_t c, int i) {
-      int64_t r = c * BT + rg * RPT + i;
-      return r < last_row ? r : last_row;
+    // A wave issues at most one instruction every few cycles and this path is arithmetic-bound,
+    // so the steady state carries no address arithmetic: the byte offsets of this lane's rows
+    // from the first row of a chunk are computed once, the (uniform) chunk base pointers are
+    // advanced by a constant stride, and rows past the end of a sequence's last chunk are
+    // redirected to its last row by one unsigned minimum (they are zeroed before use).
+    // Loads are unconditional, so the compiler is free to batch and interleave them; past the
+    // last chunk the pointers stay on it.
+    constexpr int GSH = sizeof(GT) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
+    const uint32_t pitch = (uint32_t)H * K * (uint32_t)sizeof(T);
+    uint32_t offk[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) offk[i] = (uint32_t)(rg * RPT + i) * pitch + (uint32_t)kc * (uint32_t)sizeof(T);
+    const int64_t row00 = (sp.bos * H + hh) * (int64_t)K;
+    const char* lq = (const char*)p.q + row00 * (int64_t)sizeof(T);
+    const char* lk = (const char*)p.k + row00 * (int64_t)sizeof(T);
+    const char* lg = (const char*)p.g + row00 * (int64_t)sizeof(GT);
+    const int64_t strk = (int64_t)BT * pitch;
+    const int Llast = (int)(sp.len - (nchunks - 1) * BT);
+    const uint32_t lim_full = (uint32_t)(BT - 1) * pitch, lim_last = (uint32_t)(Llast - 1) * pitch;
+    int64_t lc = 0;  // chunk the load pointers are on
+    uint32_t lim = 0;
+    auto begin_loads = [&]() __attribute__((always_inline)) {
+      lim = (lc >= nchunks - 1 ? lim_last : lim_full) + (uint32_t)kc * (uint32_t)sizeof(T);
     };
-    auto mask_tail = [&](Regs& R, int L) {
+    auto load_g = [&](Regs& R, int i) __attribute__((always_inline)) {
+      uint32_t o = offk[i] < lim ? offk[i] : lim;
+      R.g[i] = *(const gvec*)(lg + (o << GSH));
+    };
+    auto load_qk = [&](Regs& R, int i) __attribute__((always_inline)) {
+      uint32_t o = offk[i] < lim ? offk[i] : lim;
+      R.q[i] = *(const kvec*)(lq + o);
+      R.k[i] = *(const kvec*)(lk + o);
+    };
+    auto end_loads = [&]() __attribute__((always_inline)) {
+      if (lc + 1 < nchunks) {
+        lq += strk;
+        lk += strk;
+        lg += strk << GSH;
+      }
+      ++lc;
+    };
+    auto mask_tail = [&](Regs& R, int L) __attribute__((always_inline)) {
       if (L < BT) {
 #pragma unroll
         for (int i = 0; i < RPT; ++i) {
@@ -150,13 +179,20 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
     };
+    // LDS destinations of this lane
+    int dq[RPT], dkh[CPL];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) dq[i] = (rg * RPT + i) * LDK + swz_rm(rg * RPT + i, kc);
+#pragma unroll
+    for (int j = 0; j < CPL; ++j) dkh[j] = (kc + j) * LDT + rg * RPT;
     // Stage the tiles of chunk c (held in R) into buffer `buf` and refill R, register by
-    // register as each is consumed, with chunk c+2: the loads of the next chunk are spread
-    // through the arithmetic of this one.  mid_barrier() is called half way through; in the
+    // register as each is consumed, with the chunk two further on: the loads of that chunk are
+    // spread through the arithmetic of this one.  mid_barrier() is called half way through; in the
     // steady state it is the workgroup barrier between the two halves of the matrix waves' chunk.
-    auto stage = [&](Regs& R, int buf, int64_t c, auto mid_barrier) {
+    auto stage = [&](Regs& R, int buf, int64_t c, auto mid_barrier) __attribute__((always_inline)) {
       mask_tail(R, chunk_len(c));
-      float G[RPT][CPL], tot[CPL], glast[CPL];
+      begin_loads();
+      float G[RPT][CPL], glast[CPL];
       float gabs = 0.f;
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
@@ -166,62 +202,63 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           run = fmaf((float)R.g[i][j], LOG2E, run);   // prefix sums in the log2 domain
           G[i][j] = run;
         }
-        float pre = row_prefix16(run);
-        float suf = row_suffix16(run);
-        tot[j] = pre - run;                                      // gates of the earlier row groups
-        glast[j] = pre + suf - run;                              // G_last (log2 domain)
+        const float pre = row_prefix16(run);
+        const float tot = pre - run;                             // gates of the earlier row groups
+        glast[j] = dpp_f32<0x15f>(pre);                          // G_last: lane 15 of the row, broadcast
 #pragma unroll
-        for (int i = 0; i < RPT; ++i) gabs = fmaxf(gabs, fabsf(G[i][j] + tot[j]));
+        for (int i = 0; i < RPT; ++i) {
+          G[i][j] += tot;
+          gabs = fmaxf(gabs, fabsf(G[i][j]));
+        }
       }
       // The scores use one reference point per chunk (e^{G} on q, e^{-G} on k), exact while
       // |G| stays below kMaxInvDecayExp.  Chunks beyond that are flagged and recomputed by
-      // the exact kernel afterwards.
+      // the exact kernel afterwards (their q~, k~ tiles may hold infinities: only the scores
+      // use them, and those are recomputed).
       const int out_of_range = __any(gabs > kMaxInvDecayExp * LOG2E);  // wave-uniform
       if (lane == 0) sWide[buf][pw] = out_of_range;
       float eglast[CPL];
 #pragma unroll
       for (int j = 0; j < CPL; ++j) eglast[j] = __builtin_amdgcn_exp2f(glast[j]);
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) R.g[i] = *(const gvec*)(gp + row_of(c + 2, i) * kstride);
+      for (int i = 0; i < RPT; ++i) load_g(R, i);
       T khat[CPL][RPT];
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        const int row = rg * RPT + i;
         kvec qv, kv;
         float kt[CPL];
 #pragma unroll
         for (int j = 0; j < CPL; ++j) {
-          const float Gij = G[i][j] + tot[j];
-          float e = __builtin_amdgcn_exp2f(Gij);                        // e^{G}
-          float einv = __builtin_amdgcn_rcpf(fmaxf(e, 1e-35f));         // e^{-G}, finite
+          const float e = __builtin_amdgcn_exp2f(G[i][j]);       // e^{G}
+          const float einv = __builtin_amdgcn_exp2f(-G[i][j]);   // e^{-G}
           kt[j] = (float)R.k[i][j] * einv;
           qv[j] = (T)((float)R.q[i][j] * e);   // the matrix waves apply the scale to the fp32 output
           kv[j] = (T)kt[j];
         }
         // k^ = k e^{G_last-G}: inside the guarded range the product of the two factors is exact
-        // to rounding; beyond it e^{-G} is clamped, so the exponent (always <= 0) is formed
-        // directly (wave-uniform branch, rare)
+        // to rounding; beyond it e^{-G} may overflow, so the exponent (always <= 0 for
+        // non-positive gates) is formed directly (wave-uniform branch, rare)
         if (out_of_range) {
 #pragma unroll
           for (int j = 0; j < CPL; ++j)
-            khat[j][i] = (T)((float)R.k[i][j] * __builtin_amdgcn_exp2f(glast[j] - (G[i][j] + tot[j])));
+            khat[j][i] = (T)((float)R.k[i][j] * __builtin_amdgcn_exp2f(glast[j] - G[i][j]));
         } else {
 #pragma unroll
           for (int j = 0; j < CPL; ++j) khat[j][i] = (T)(kt[j] * eglast[j]);
         }
-        R.q[i] = *(const kvec*)(qp + row_of(c + 2, i) * kstride);
-        R.k[i] = *(const kvec*)(kp + row_of(c + 2, i) * kstride);
-        *(kvec*)&sQ[buf][row * LDK + swz_rm(row, kc)] = qv;
-        *(kvec*)&sK[buf][row * LDK + swz_rm(row, kc)] = kv;
+        load_qk(R, i);
+        *(kvec*)&sQ[buf][dq[i]] = qv;
+        *(kvec*)&sK[buf][dq[i]] = kv;
         if (i == RPT / 2 - 1) mid_barrier();
       }
+      end_loads();
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
         typedef T rvec __attribute__((ext_vector_type(RPT)));
         rvec x;
 #pragma unroll
         for (int i = 0; i < RPT; ++i) x[i] = khat[j][i];
-        *(rvec*)&sKh[buf][(kc + j) * LDT + rg * RPT] = x;
+        *(rvec*)&sKh[buf][dkh[j]] = x;
       }
       if (rg == 0) {
 #pragma unroll
@@ -233,15 +270,20 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       // Two register sets, used alternately: the loads refilling a set have two chunk periods
       // to land before it is staged again.
       Regs RA, RB;
+      begin_loads();
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        RA.g[i] = *(const gvec*)(gp + row_of(0, i) * kstride);
-        RA.q[i] = *(const kvec*)(qp + row_of(0, i) * kstride);
-        RA.k[i] = *(const kvec*)(kp + row_of(0, i) * kstride);
-        RB.g[i] = *(const gvec*)(gp + row_of(1, i) * kstride);
-        RB.q[i] = *(const kvec*)(qp + row_of(1, i) * kstride);
-        RB.k[i] = *(const kvec*)(kp + row_of(1, i) * kstride);
+        load_g(RA, i);
+        load_qk(RA, i);
       }
+      end_loads();
+      begin_loads();
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        load_g(RB, i);
+        load_qk(RB, i);
+      }
+      end_loads();
       stage(RA, 0, 0, [] {});
       for (int64_t c = 0; c < nchunks; c += 2) {
         lds_barrier();  // B1(c): tiles of chunk c published; buffer 1 is free
@@ -294,33 +336,44 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     // The matrix waves also stage the value tile (time-contiguous) of the next chunk: 8 rows x
     // 2 columns per lane, loaded one chunk period ahead.
     const int vrg = tid >> 5, vc = (tid & 31) * 2;
-    const T* vp = (const T*)p.v + (sp.bos * H + hh) * (int64_t)V + vbase + vc;
-    const int64_t vstride = (int64_t)H * V;
-    const int64_t last_row = sp.len - 1;
-    t2 vreg[8];
-    auto load_v = [&](int64_t c) {
+    const uint32_t vpitch = (uint32_t)H * V * (uint32_t)sizeof(T);
+    const char* lv = (const char*)p.v + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const int64_t strv = (int64_t)BT * vpitch;
+    const int Llast = (int)(sp.len - (nchunks - 1) * BT);
+    uint32_t offv[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        int64_t r = c * BT + vrg * 8 + i;
-        vreg[i] = *(const t2*)(vp + (r < last_row ? r : last_row) * vstride);
-      }
+    for (int i = 0; i < 8; ++i) offv[i] = (uint32_t)(vrg * 8 + i) * vpitch + (uint32_t)vc * (uint32_t)sizeof(T);
+    const uint32_t vlim_full = (uint32_t)(BT - 1) * vpitch, vlim_last = (uint32_t)(Llast - 1) * vpitch;
+    int64_t lvc = 0;  // chunk the value pointer is on (stays on the last one)
+    t2 vreg[8];
+    auto load_v = [&]() __attribute__((always_inline)) {
+      const uint32_t lim = (lvc >= nchunks - 1 ? vlim_last : vlim_full) + (uint32_t)vc * (uint32_t)sizeof(T);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) vreg[i] = *(const t2*)(lv + (offv[i] < lim ? offv[i] : lim));
+      if (lvc + 1 < nchunks) lv += strv;
+      ++lvc;
     };
-    auto stage_v = [&](int buf, int64_t c) {
+    const int dv0 = (vc + 0) * LDT + vrg * 8, dv1 = (vc + 1) * LDT + vrg * 8;
+    auto stage_v = [&](int buf, int64_t c) __attribute__((always_inline)) {
       const int L = chunk_len(c);
       v8 a, b;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        bool ok = vrg * 8 + i < L;
-        a[i] = ok ? vreg[i][0] : (T)0.f;
-        b[i] = ok ? vreg[i][1] : (T)0.f;
+        a[i] = vreg[i][0];
+        b[i] = vreg[i][1];
       }
-      *(v8*)&sVt[buf][(vc + 0) * LDT + vrg * 8] = a;
-      *(v8*)&sVt[buf][(vc + 1) * LDT + vrg * 8] = b;
+      if (L < BT) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (vrg * 8 + i >= L) a[i] = b[i] = (T)0.f;
+      }
+      *(v8*)&sVt[buf][dv0] = a;
+      *(v8*)&sVt[buf][dv1] = b;
     };
     if (nchunks > 0) {
-      load_v(0);
+      load_v();
       stage_v(0, 0);
-      load_v(1);
+      load_v();
     }
     for (int64_t c = 0; c < nchunks; ++c) {
       const int buf = (int)(c & 1);
@@ -345,16 +398,18 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       if (c + 1 < nchunks) {
         stage_v(buf ^ 1, c + 1);
-        load_v(c + 2);
+        load_v();
       }
       // ---- scores on the lower-triangular quadrants and the inter-chunk part of o
       const int qi = wave >> 1, qj = wave & 1;
+      // transposed scores (k~ q~^T): a lane ends up with one row i of P and four consecutive
+      // columns j per register quad, so P is written with 8-byte stores
       f32x16 s = zero16();
       if (qj <= qi) {
 #pragma unroll
         for (int ks = 0; ks < K; ks += 16)
-          s = Elem<T>::mfma32(frag32_swz<T>(sQ[buf], LDK, qi * 32, ks, lane),
-                              frag32_swz<T>(sK[buf], LDK, qj * 32, ks, lane), s);
+          s = Elem<T>::mfma32(frag32_swz<T>(sK[buf], LDK, qj * 32, ks, lane),
+                              frag32_swz<T>(sQ[buf], LDK, qi * 32, ks, lane), s);
       }
       f32x16 o = zero16();
 #pragma unroll
@@ -366,11 +421,25 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         o = Elem<T>::mfma32(h1v, frag32_perm_swz<T>(sQ[buf], LDK, rw * 32, kt * 32 + 16, lane), o);
       }
       {
-        const int j = qj * 32 + (lane & 31);
+        const int i = qi * 32 + (lane & 31);
+        T* prow = &sP[i * LDT + qj * 32 + 4 * (lane >> 5)];
+        if (qi == qj) {            // diagonal quadrant: keep j <= i
+          const int il = (lane & 31) - 4 * (lane >> 5);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          int i = qi * 32 + c32_row(r, lane);
-          sP[i * LDT + j] = (T)((j <= i) ? s[r] : 0.f);
+          for (int r4 = 0; r4 < 4; ++r4) {
+            v4 x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = (T)((8 * r4 + e <= il) ? s[4 * r4 + e] : 0.f);
+            *(v4*)(prow + 8 * r4) = x;
+          }
+        } else {                   // below the diagonal, or the all-zero quadrant above it
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            v4 x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = (T)s[4 * r4 + e];
+            *(v4*)(prow + 8 * r4) = x;
+          }
         }
       }
       lds_barrier();  // B2(c): P visible; nobody reads the state fragments any more

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       int row = rg + RG * i;
-      if (h0p && colok && row < K) h[i] = *(const f32x4*)(h0p + (int64_t)row * V);
+      if (h0p && colok && row < K) h[i] = __builtin_nontemporal_load((const f32x4*)(h0p + (int64_t)row * V));
       else h[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   }
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       int row = rg + RG * i;
-      if (row < K) *(f32x4*)(htp + (int64_t)row * V) = h[i];
+      if (row < K) __builtin_nontemporal_store(h[i], (f32x4*)(htp + (int64_t)row * V));
     }
   }
 }
