@@ -267,6 +267,52 @@ def bench_backward(device, steps=10):
     return out
 
 
+def bench_layer_steps(device, steps=20):
+    """The row-wise steps either side of the operators at the operators' benchmark shape
+    (B=8, T=4096, H=16, D=128; the convolution on 2048 channels, kernel 4): device time of each
+    kernel (HIP events) and its algorithmic bytes (each tensor read or written once)."""
+    import torch
+    from fla_amd.modules.convolution import ShortConvolution
+    from fla_amd.modules.fused_norm_gate import norm_gate_bwd, norm_gate_fwd
+    from fla_amd.modules.l2norm import l2norm_bwd, l2norm_fwd
+    B, T, H, D = 8, 4096, 16, 128
+    gen = torch.Generator(device=device).manual_seed(4)
+    x = torch.randn(B * T * H, D, device=device, generator=gen).bfloat16()
+    o = torch.randn(B * T * H, D, device=device, generator=gen).bfloat16()
+    dy = torch.randn(B * T * H, D, device=device, generator=gen).bfloat16()
+    w = torch.ones(D, device=device)
+    nb = x.numel() * 2
+    out = {}
+
+    def rec(name, fn, nbytes):
+        us = event_avg_us(fn, steps)
+        out[name] = {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    rec("l2norm_fwd", lambda: l2norm_fwd(x), 2 * nb)
+    rec("l2norm_bwd", lambda: l2norm_bwd(x, dy), 3 * nb)
+    rec("rmsnorm_swish_gate_fwd", lambda: norm_gate_fwd(x, o, w, None, 1e-5, True), 3 * nb)
+    y, mean, rstd = norm_gate_fwd(x, o, w, None, 1e-5, True)
+    rec("rmsnorm_swish_gate_bwd", lambda: norm_gate_bwd(dy, x, o, w, None, 1e-5, mean, rstd, True), 5 * nb)
+    Dc = 2048
+    xc = torch.randn(B, T, Dc, device=device, generator=gen).bfloat16()
+    dyc = torch.randn(B, T, Dc, device=device, generator=gen).bfloat16()
+    conv = ShortConvolution(Dc, 4, activation="silu").to(device)
+    nbc = xc.numel() * 2
+    with torch.no_grad():
+        rec("short_conv_fwd", lambda: conv(xc), 2 * nbc)
+    xg = xc.clone().requires_grad_()
+
+    def conv_fb():
+        yc, _ = conv(xg)
+        yc.backward(dyc)
+        xg.grad = None
+        conv.weight.grad = None
+
+    rec("short_conv_fwd_bwd", conv_fb, 5 * nbc)
+    return out
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -321,6 +367,7 @@ def main():
         extra["decode_step"] = bench_decode(device)
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
+        extra["layer_steps"] = bench_layer_steps(device)
     out = {
         "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

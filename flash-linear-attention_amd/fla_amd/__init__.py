@@ -4,7 +4,7 @@ chunked linear-attention hot path (``chunk_gla``, ``chunk_gated_delta_rule``,
 ``from fla.ops.gla import chunk_gla`` for ``from fla_amd.ops.gla import chunk_gla``,
 or call :func:`install` to rebind the names inside an importable upstream ``fla``.
 """
-from . import ops  # noqa: F401
+from . import modules, ops  # noqa: F401
 from ._backend import lib, lib_path  # noqa: F401
 
 __version__ = '0.1.0'
@@ -21,9 +21,14 @@ def install() -> list:
     import importlib
     patched = []
     table = {name: getattr(ops, name) for name in ops.__all__}
+    # the steps either side of the operators: fla/modules/l2norm.py, fused_norm_gate.py, convolution.py
+    table.update({name: getattr(modules, name) for name in (
+        'l2_norm', 'l2norm_fwd', 'l2norm_bwd', 'L2NormFunction', 'FusedRMSNormSwishGate', 'FusedLayerNormSwishGate',
+        'rms_norm_swish_gate_fn', 'layer_norm_swish_gate_fn', 'LayerNormSwishGateFn', 'ShortConvolution')})
     targets = ['fla.ops.gla', 'fla.ops.gated_delta_rule', 'fla.ops.delta_rule', 'fla.ops.simple_gla', 'fla.ops.utils',
                'fla.ops', 'fla.layers.gla', 'fla.layers.gated_deltanet', 'fla.layers.hgrn2', 'fla.layers.delta_net',
-               'fla.layers.simple_gla']
+               'fla.layers.simple_gla', 'fla.modules', 'fla.modules.l2norm', 'fla.modules.fused_norm_gate',
+               'fla.modules.convolution']
     for modname in targets:
         try:
             mod = importlib.import_module(modname)

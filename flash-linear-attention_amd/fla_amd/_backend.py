@@ -45,6 +45,15 @@ SIGNATURES = {
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 19 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 26 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_l2norm_fwd": (c_int, [P, P, I64, I64, F, I, I, P]),
+    "fla_l2norm_bwd": (c_int, [P, P, P, I64, I64, F, I, I, P]),
+    "fla_norm_swish_gate_workgroups": (c_int, [I64, I64]),
+    "fla_norm_swish_gate_fwd": (c_int, [P, P, P, P, P, P, P, I64, I64, F, I, I, P]),
+    "fla_norm_swish_gate_bwd": (c_int, [P] * 11 + [I64, I64, F, I, I, P]),
+    "fla_causal_conv1d_fwd": (c_int, [P, P, P, P, I64, I64, I64, I64, I, I, P]),
+    "fla_causal_conv1d_bwd_partials": (c_int, [I64, I64]),
+    "fla_causal_conv1d_bwd": (c_int, [P] * 7 + [I64, I64, I64, I64, I, I, P]),
+    "fla_causal_conv1d_update": (c_int, [P] * 5 + [I64, I64, I64, I, I, P]),
     "fla_selftest_mfma": (c_int, [P, P, P, I64, I64, I64, I, P]),
 }
 

@@ -263,6 +263,59 @@ int fla_chunk_gated_delta_rule_bwd(
     const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
+/* ------------------------------------------------------------------------
+ * Row-wise steps either side of the chunk operators inside the layers
+ * (fla/layers/gated_deltanet.py:234-235, fla/layers/gla.py:203-218).
+ * Rows are the leading dimensions flattened: x is [M, N], N % 8 == 0, N <= 2048.
+ *
+ * fla_l2norm_fwd / _bwd replace l2norm_fwd / l2norm_bwd
+ * (fla/modules/l2norm.py:91-132, :135-166): y = x / sqrt(sum x^2 + eps),
+ * dx = dy*rstd - (sum dy*x) * rstd^3 * x.  x/dx in x_dtype, y in y_dtype, dy in dy_dtype.
+ * ---------------------------------------------------------------------- */
+int fla_l2norm_fwd(const void* x, void* y, int64_t M, int64_t N, float eps, int x_dtype, int y_dtype,
+                   fla_stream_t stream);
+int fla_l2norm_bwd(const void* x, const void* dy, void* dx, int64_t M, int64_t N, float eps, int x_dtype,
+                   int dy_dtype, fla_stream_t stream);
+
+/* fla_norm_swish_gate_fwd / _bwd replace layer_norm_fwd / layer_norm_bwd of the gated
+ * norms (fla/modules/fused_norm_gate.py:186-256, :333-397) without residual:
+ *   y = norm(x) * weight (+ bias) * gate * sigmoid(gate),
+ * norm = RMS norm (is_rms_norm != 0) or layer norm.  x, gate, y, dy, dx, dgate [M,N] in
+ * `dtype`; weight, bias fp32 [N] or NULL; mean (layer norm only) and rstd fp32 [M] are
+ * written by the forward and read by the backward.  The backward leaves per-workgroup
+ * column sums of the weight / bias gradients in dw_partial / db_partial, fp32
+ * [fla_norm_swish_gate_workgroups(M, N), N] (either may be NULL); their sum over the first
+ * dimension is the gradient. */
+int fla_norm_swish_gate_workgroups(int64_t M, int64_t N);
+int fla_norm_swish_gate_fwd(const void* x, const void* gate, const float* weight, const float* bias, void* y,
+                            float* mean, float* rstd, int64_t M, int64_t N, float eps, int is_rms_norm,
+                            int dtype, fla_stream_t stream);
+int fla_norm_swish_gate_bwd(const void* dy, const void* x, const void* gate, const float* weight,
+                            const float* bias, const float* mean, const float* rstd, void* dx, void* dgate,
+                            float* dw_partial, float* db_partial, int64_t M, int64_t N, float eps,
+                            int is_rms_norm, int dtype, fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Depthwise causal convolution over time, channels last, replaces the external
+ * causal_conv1d_fn / causal_conv1d_update calls of ShortConvolution
+ * (fla/modules/convolution.py:171-186 and :188-211):
+ *   y[b,t,d] = act(bias[d] + sum_{i<W} weight[d,i] * x[b, t-(W-1)+i, d]),  act = SiLU or identity.
+ * x, y, dy, dx [B,T,D] in `dtype`, D % 8 == 0; weight fp32 [D,W], 2 <= W <= 4; bias fp32 [D]
+ * or NULL.  The backward leaves per-workgroup partial sums of the weight / bias gradients in
+ * dw_partial (fp32 [P,D,W]) and db_partial (fp32 [P,D] or NULL), P =
+ * fla_causal_conv1d_bwd_partials(B, T); their sum over P is the gradient (deterministic, no
+ * atomics).  The update is the single-token step: cache [B,D,W] (in `dtype`) is
+ * shifted left by one and x [B,D] appended in place, y [B,D] = act(bias + sum cache*weight).
+ * ---------------------------------------------------------------------- */
+int fla_causal_conv1d_fwd(const void* x, const float* weight, const float* bias, void* y, int64_t B, int64_t T,
+                          int64_t D, int64_t W, int silu, int dtype, fla_stream_t stream);
+int fla_causal_conv1d_bwd_partials(int64_t B, int64_t T);
+int fla_causal_conv1d_bwd(const void* x, const float* weight, const float* bias, const void* dy, void* dx,
+                          float* dw_partial, float* db_partial, int64_t B, int64_t T, int64_t D, int64_t W, int silu,
+                          int dtype, fla_stream_t stream);
+int fla_causal_conv1d_update(const void* x, void* cache, const float* weight, const float* bias, void* y,
+                             int64_t B, int64_t D, int64_t W, int silu, int dtype, fla_stream_t stream);
+
 /* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
  * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,
  * mode 1: 16x16x32 tiles, mode 2: 32x32x16 with the permuted contraction order

@@ -1,0 +1,157 @@
+"""GPU: the row-wise steps either side of the chunk operators (l2 norm, gated norms, short causal
+convolution and its single-token step), forward and backward, against the torch restatements in
+oracle/modules.py.  Tolerances (rel-L2): 1e-5 for fp32 storage; for 16-bit storage the outputs are
+rounded once to bf16/fp16, 4e-3 forward and 8e-3 for gradients (the bar of the chunk operators)."""
+import pytest
+import torch
+
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _tols(dtype):
+    return (1e-5, 1e-5) if dtype == torch.float32 else (4e-3, 8e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("N", [64, 128, 200, 256, 512, 1024])
+def test_l2norm(device, dtype, N):
+    from fla_amd.modules import l2_norm
+    from oracle.modules import l2norm
+    gen = torch.Generator().manual_seed(N)
+    x = (torch.randn(3, 37, 2, N, generator=gen) * 1.5).to(dtype)
+    dy = torch.randn(3, 37, 2, N, generator=gen).to(dtype)
+    print(f"l2_norm {dtype} N={N}", flush=True)
+    xd = x.to(device).requires_grad_()
+    y = l2_norm(xd)
+    y.backward(dy.to(device))
+    xr = x.float().requires_grad_()
+    yr = l2norm(xr)
+    yr.backward(dy.float())
+    ft, bt = _tols(dtype)
+    assert y.dtype == dtype and xd.grad.dtype == dtype
+    assert_close("y", yr, y, ft)
+    assert_close("dx", xr.grad, xd.grad, bt)
+
+
+def test_l2norm_output_dtype_and_empty(device):
+    from fla_amd.modules import l2_norm
+    from oracle.modules import l2norm
+    x = torch.randn(5, 128).bfloat16()
+    y = l2_norm(x.to(device), output_dtype=torch.float32)
+    assert y.dtype == torch.float32
+    assert_close("y", l2norm(x), y, 1e-5)
+    assert l2_norm(torch.empty(0, 128, device=device)).shape == (0, 128)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("is_rms", [True, False])
+@pytest.mark.parametrize("N,affine", [(128, True), (128, False), (64, True), (256, True), (1024, True), (1536, True)])
+def test_norm_swish_gate(device, dtype, is_rms, N, affine):
+    from fla_amd.modules import FusedLayerNormSwishGate, FusedRMSNormSwishGate
+    from oracle.modules import norm_swish_gate
+    gen = torch.Generator().manual_seed(N + is_rms)
+    shape = (2, 300, 3, N) if N <= 256 else (2, 77, N)
+    x = (torch.randn(*shape, generator=gen) * 2 + 0.3).to(dtype)
+    o = torch.randn(*shape, generator=gen).to(dtype)
+    dy = torch.randn(*shape, generator=gen).to(dtype)
+    w = torch.randn(N, generator=gen) * 0.5 + 1.0
+    print(f"norm gate {dtype} rms={is_rms} N={N} affine={affine}", flush=True)
+    mod = (FusedRMSNormSwishGate if is_rms else FusedLayerNormSwishGate)(N, elementwise_affine=affine, eps=1e-5).to(device)
+    if affine:
+        with torch.no_grad():
+            mod.weight.copy_(w)
+    xd, od = x.to(device).requires_grad_(), o.to(device).requires_grad_()
+    y = mod(xd, od)
+    y.backward(dy.to(device))
+    xr, orr = x.float().requires_grad_(), o.float().requires_grad_()
+    wr = w.clone().requires_grad_() if affine else None
+    yr = norm_swish_gate(xr, orr, wr, None, eps=1e-5, is_rms_norm=is_rms)
+    yr.backward(dy.float())
+    ft, bt = _tols(dtype)
+    assert y.dtype == dtype
+    assert_close("y", yr, y, ft)
+    assert_close("dx", xr.grad, xd.grad, bt)
+    assert_close("do", orr.grad, od.grad, bt)
+    if affine:
+        assert_close("dw", wr.grad, mod.weight.grad, 2e-3 if dtype != torch.float32 else 1e-5)
+
+
+def test_norm_swish_gate_with_bias_function(device):
+    from fla_amd.modules import layer_norm_swish_gate_fn
+    from oracle.modules import norm_swish_gate
+    gen = torch.Generator().manual_seed(5)
+    N = 128
+    x, o, dy = (torch.randn(4, 50, N, generator=gen) for _ in range(3))
+    w, b = torch.randn(N, generator=gen), torch.randn(N, generator=gen)
+    leaves = [t.to(device).requires_grad_() for t in (x, o, w, b)]
+    y = layer_norm_swish_gate_fn(*leaves, eps=1e-6)
+    y.backward(dy.to(device))
+    refs = [t.clone().requires_grad_() for t in (x, o, w, b)]
+    yr = norm_swish_gate(*refs, eps=1e-6, is_rms_norm=False)
+    yr.backward(dy)
+    assert_close("y", yr, y, 1e-5)
+    for name, r, d in zip(("dx", "do", "dw", "db"), refs, leaves):
+        assert_close(name, r.grad, d.grad, 1e-5)
+    with pytest.raises(NotImplementedError):
+        layer_norm_swish_gate_fn(leaves[0], leaves[1], leaves[2], leaves[3], residual=leaves[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("W", [2, 3, 4])
+@pytest.mark.parametrize("T,D,bias,act", [(1, 64, False, "silu"), (5, 64, True, "silu"), (64, 200, False, None),
+                                          (300, 512, True, "silu"), (1000, 2048, False, "silu")])
+def test_causal_conv1d(device, dtype, W, T, D, bias, act):
+    from fla_amd.modules import ShortConvolution
+    from oracle.modules import causal_conv1d
+    gen = torch.Generator().manual_seed(T + W)
+    B = 2
+    x = torch.randn(B, T, D, generator=gen).to(dtype)
+    dy = torch.randn(B, T, D, generator=gen).to(dtype)
+    print(f"short conv {dtype} W={W} T={T} D={D} bias={bias} act={act}", flush=True)
+    conv = ShortConvolution(D, W, bias=bias, activation=act).to(device)
+    w = conv.weight.detach().cpu().reshape(D, W).clone()
+    b = conv.bias.detach().cpu().clone() if bias else None
+    xd = x.to(device).requires_grad_()
+    # with a cache a single token takes the (non-differentiable) decode step, as in the reference
+    y, cache = conv(xd, output_final_state=T > 1)
+    y.backward(dy.to(device))
+    xr = x.float().requires_grad_()
+    wr = w.clone().requires_grad_()
+    br = b.clone().requires_grad_() if bias else None
+    yr = causal_conv1d(xr, wr, br, act)
+    yr.backward(dy.float())
+    ft, bt = _tols(dtype)
+    assert y.dtype == dtype and y.shape == x.shape
+    assert_close("y", yr, y, ft)
+    assert_close("dx", xr.grad, xd.grad, bt)
+    # weight/bias gradients are fp32 sums over B*T terms of 16-bit inputs
+    assert_close("dw", wr.grad, conv.weight.grad.reshape(D, W), 2e-3 if dtype != torch.float32 else 2e-5)
+    if bias:
+        assert_close("db", br.grad, conv.bias.grad, 2e-3 if dtype != torch.float32 else 2e-5)
+    # final state: the last W inputs, zero-padded on the left, [B,D,W]
+    if T > 1:
+        ref_cache = torch.nn.functional.pad(x.transpose(1, 2), (W - T, 0))
+        assert torch.equal(cache.cpu(), ref_cache)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("W", [2, 4])
+def test_short_convolution_step(device, dtype, W):
+    """Prefill T tokens then decode 3 more one at a time == one pass over T+3 tokens."""
+    from fla_amd.modules import ShortConvolution
+    gen = torch.Generator().manual_seed(9)
+    B, T, D = 3, 20, 256
+    x = torch.randn(B, T + 3, D, generator=gen).to(dtype).to(device)
+    conv = ShortConvolution(D, W, bias=True, activation="silu").to(device).to(dtype)
+    with torch.no_grad():
+        full, _ = conv(x)
+        y, cache = conv(x[:, :T].contiguous(), output_final_state=True)
+        outs = [y]
+        for t in range(T, T + 3):
+            yt, cache = conv(x[:, t:t + 1].contiguous(), cache=cache)
+            outs.append(yt)
+    got = torch.cat(outs, dim=1)
+    assert_close("y", full, got, 1e-6 if dtype == torch.float32 else 4e-3)
+    assert torch.equal(cache, x[:, -W:].transpose(1, 2))
