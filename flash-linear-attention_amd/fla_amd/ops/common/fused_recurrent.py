@@ -60,6 +60,10 @@ def fused_recurrent_fwd(q, k, v, g=None, gk=None, gv=None, scale=None, initial_s
 
 
 class FusedRecurrentFunction(torch.autograd.Function):
+    """Forward: the token-by-token kernel.  Backward: the recurrence equals the chunked operator on
+    the same inputs, so the gradients come from ``chunk_gla``'s backward kernels (the reference runs
+    a second token-by-token pass, ``fla/ops/common/fused_recurrent.py:381-468``, and a global
+    reverse cumsum for the gates, ``:462-467``)."""
 
     @staticmethod
     @contiguous
@@ -68,15 +72,43 @@ class FusedRecurrentFunction(torch.autograd.Function):
                 output_final_state=False, reverse=False, offsets=None, head_first=True, inplace_state=False):
         o, ht = fused_recurrent_fwd(q, k, v, g, gk, gv, scale, initial_state, output_final_state, reverse,
                                     offsets, head_first, inplace_state)
+        if any(t is not None and t.requires_grad for t in (q, k, v, g, gk, gv, initial_state)):
+            if inplace_state:
+                raise ValueError("inplace_state=True overwrites the initial state the backward needs")
+            ctx.save_for_backward(q, k, v, g, gk, gv, initial_state, offsets)
+            ctx.scale, ctx.reverse, ctx.head_first = scale, reverse, head_first
         return o.to(q.dtype), ht
 
     @staticmethod
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        raise NotImplementedError(
-            "fla_amd: the backward of the token-by-token recurrence is not built; "
-            "use the chunked operators (chunk_gla, chunk_gated_delta_rule) for training.")
+        import warnings
+
+        from ..gla.chunk import chunk_gla
+        q, k, v, g, gk, gv, h0, offsets = ctx.saved_tensors
+        if gv is not None or ctx.reverse:
+            raise NotImplementedError("fla_amd fused_recurrent backward: value gates (gv) and reverse=True are not covered")
+        leaves = [None if t is None else t.detach().requires_grad_() for t in (q, k, v, g, gk, h0)]
+        ql, kl, vl, gl, gkl, h0l = leaves
+        with torch.enable_grad(), warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            # one per-key log-gate: gk, plus the per-head scalar g broadcast over the key channels
+            gate = gkl.float() if gkl is not None else None
+            if gl is not None:
+                gs = gl.float().unsqueeze(-1).expand(*kl.shape)
+                gate = gs if gate is None else gate + gs
+            if gate is None:
+                gate = torch.zeros(kl.shape, dtype=torch.float32, device=kl.device)
+            o, ht = chunk_gla(ql, kl, vl, gate.contiguous(), scale=ctx.scale, initial_state=h0l, output_final_state=True,
+                              offsets=offsets, head_first=ctx.head_first)
+            outs, grads = [o], [do.to(o.dtype)]
+            if dht is not None:
+                outs.append(ht)
+                grads.append(dht.to(ht.dtype))
+            torch.autograd.backward(outs, grads)
+        dq, dk, dv, dg, dgk, dh0 = (None if t is None else t.grad for t in leaves)
+        return dq, dk, dv, dg, dgk, None, None, dh0, None, None, None, None, None
 
 
 def fused_recurrent(

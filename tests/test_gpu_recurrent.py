@@ -132,3 +132,58 @@ def test_decode_inplace_matches_out_of_place(device, op):
         assert torch.equal(o_a, o_b) and torch.equal(state_a, state_b)
         assert torch.equal(o_a, o_all[:, t:t + 1])
     assert torch.equal(state_b, ht_all)
+
+
+# ---------------------------------------------------------------- backward of fused_recurrent_gla
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,D,head_first", [(1, 128, False), (20, 64, False), (64, 128, True), (100, 100, False)])
+def test_fused_recurrent_gla_backward(device, dtype, T, D, head_first):
+    """Gradients of the token-by-token operator (the layers' path for sequences of at most 64
+    tokens) against autograd through the naive recurrence, at the reference's tolerance for this
+    operator (tests/ops/test_gla.py:66-87 uses 0.005 in fp32; the kernels behind the backward
+    round q, k, v to bf16, hence the bar of the chunked operator here)."""
+    from fla_amd.ops.gla import fused_recurrent_gla
+    from oracle.recurrent import naive_recurrent_gla
+    B, H = 2, 2
+    q, k, v, g, h0 = gla_inputs(B, T, H, D, D, seed=40 + T, dtype=dtype, normalizer=4.0, h0_std=1.0)
+    gen = torch.Generator().manual_seed(6)
+    do = torch.randn(B, T, H, D, generator=gen).to(dtype)
+    dht = torch.randn(B, H, D, D, generator=gen) * 0.1
+    print(f"fused_recurrent_gla backward {dtype} T={T} D={D} head_first={head_first}", flush=True)
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    leaves = [tr(x.to(device)).detach().requires_grad_() for x in (q, k, v, g)]
+    h0l = h0.to(device).requires_grad_()
+    o, ht = fused_recurrent_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=head_first)
+    ((o.float() * tr(do.to(device)).float()).sum() + (ht * dht.to(device)).sum()).backward()
+    refs = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gla(*refs, initial_state=rh0, output_final_state=True)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg"), refs, leaves, (8e-3, 8e-3, 8e-3, 1e-2)):
+        assert x.grad.dtype == x.dtype
+        assert_close(name, r.grad, tr(x.grad), tol)
+    assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
+
+
+def test_fused_recurrent_scalar_gate_backward_and_guards(device):
+    """Per-head scalar gates (the simple-GLA form) through the same backward; value gates and
+    reverse scans are refused loudly."""
+    from fla_amd.ops.common.fused_recurrent import fused_recurrent
+    from oracle.recurrent import naive_recurrent_gla
+    B, T, H, D = 2, 50, 2, 64
+    gen = torch.Generator().manual_seed(8)
+    q, k, v = (torch.randn(B, T, H, D, generator=gen).bfloat16() for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
+    leaves = [x.to(device).requires_grad_() for x in (q, k, v, g)]
+    o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], g=leaves[3], head_first=False)
+    (o.float() * do.to(device).float()).sum().backward()
+    refs = [x.float().requires_grad_() for x in (q, k, v, g)]
+    ro, _ = naive_recurrent_gla(refs[0], refs[1], refs[2], None, g=refs[3])
+    (ro * do.float()).sum().backward()
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg"), refs, leaves, (8e-3, 8e-3, 8e-3, 4e-2)):
+        assert_close(name, r.grad, x.grad, tol)
+    gv = F.logsigmoid(torch.randn(B, T, H, D, generator=gen)).to(device)
+    o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], gv=gv, head_first=False)
+    with pytest.raises(NotImplementedError):
+        o.sum().backward()
