@@ -120,6 +120,76 @@ int launch_cumsum(const void* g, float* out, int64_t B, int64_t T, int64_t H, in
   return FLA_OK;
 }
 
+// Second pass of the whole-sequence cumulative sum: out = local + (sum of the totals of the
+// chunks before (reverse: after) this one in the same sequence).  `local` holds the chunk-local
+// sums of the first pass, so a chunk's total is its last (reverse: first) row.
+template <typename OT, int VEC>
+__global__ __launch_bounds__(256) void cumsum_carry_kernel(const float* __restrict__ local, OT* __restrict__ out,
+                                                           int64_t T, int64_t HS, int BT, int reverse,
+                                                           const int64_t* __restrict__ offsets,
+                                                           const int64_t* __restrict__ indices) {
+  int64_t col = ((int64_t)blockIdx.y * 256 + threadIdx.x) * VEC;
+  if (col >= HS) return;
+  int64_t bos, len, ic;
+  if (offsets) {
+    int64_t n = indices[2 * (int64_t)blockIdx.x];
+    ic = indices[2 * (int64_t)blockIdx.x + 1];
+    bos = offsets[n];
+    len = offsets[n + 1] - bos;
+  } else {
+    bos = (int64_t)blockIdx.z * T;
+    len = T;
+    ic = blockIdx.x;
+  }
+  const int64_t t0 = ic * BT;
+  const int L = (int)((len - t0) < BT ? (len - t0) : BT);
+  if (L <= 0) return;
+  const int64_t nchunks = (len + BT - 1) / BT;
+  float carry[VEC];
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) carry[i] = 0.f;
+  const int64_t c_lo = reverse ? ic + 1 : 0, c_hi = reverse ? nchunks : ic;
+  for (int64_t c = c_lo; c < c_hi; ++c) {
+    int64_t row = c * BT;
+    if (!reverse) {
+      int64_t rem = len - row;
+      row += (rem < BT ? rem : BT) - 1;
+    }
+    float x[VEC];
+    VecLoad<float, VEC>::load(local + (bos + row) * HS + col, x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) carry[i] += x[i];
+  }
+  for (int r = 0; r < L; ++r) {
+    float x[VEC];
+    VecLoad<float, VEC>::load(local + (bos + t0 + r) * HS + col, x);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) out[(bos + t0 + r) * HS + col + i] = (OT)(x[i] + carry[i]);
+  }
+}
+
+template <typename OT>
+int launch_carry(const float* local, void* out, int64_t B, int64_t T, int64_t H, int64_t S, int BT, int reverse,
+                 const int64_t* offsets, const int64_t* indices, int64_t NT, hipStream_t stream) {
+  int64_t HS = H * S;
+  bool vec4 = (HS % 4 == 0) && (((uintptr_t)local) % 16 == 0);
+  int64_t nt = offsets ? NT : fla_cdiv(T, BT);
+  int64_t nb = offsets ? 1 : B;
+  if (nt == 0 || nb == 0 || HS == 0) return FLA_OK;
+  FLA_REQUIRE(nt <= 0x7fffffffLL && nb <= 65535 && fla_cdiv(HS, 256) <= 65535, FLA_E_UNSUPPORTED);
+  if (vec4) {
+    dim3 grid((unsigned)nt, (unsigned)fla_cdiv(HS / 4, 256), (unsigned)nb);
+    hipLaunchKernelGGL((cumsum_carry_kernel<OT, 4>), grid, dim3(256), 0, stream, local, (OT*)out, T, HS, BT, reverse,
+                       offsets, indices);
+  } else {
+    dim3 grid((unsigned)nt, (unsigned)fla_cdiv(HS, 256), (unsigned)nb);
+    hipLaunchKernelGGL((cumsum_carry_kernel<OT, 1>), grid, dim3(256), 0, stream, local, (OT*)out, T, HS, BT, reverse,
+                       offsets, indices);
+  }
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
 }  // namespace
 
 extern "C" int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype, int64_t B, int64_t T, int64_t H,
@@ -135,6 +205,22 @@ extern "C" int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype, in
     case FLA_F32: return launch_cumsum<float>(g, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
     case FLA_BF16: return launch_cumsum<bf16>(g, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
     case FLA_F16: return launch_cumsum<f16>(g, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
+    default: return FLA_E_UNSUPPORTED;
+  }
+}
+
+extern "C" int fla_chunk_global_cumsum(const void* s, float* ws_local, void* out, int s_dtype, int out_dtype, int64_t B,
+                                       int64_t T, int64_t H, int64_t S, int64_t chunk_size, int reverse,
+                                       const int64_t* offsets, const int64_t* indices, int64_t NT,
+                                       fla_stream_t stream) {
+  FLA_REQUIRE(s && ws_local && out, FLA_E_INVALID);
+  int rc = fla_chunk_local_cumsum(s, ws_local, s_dtype, B, T, H, S, chunk_size, reverse, offsets, indices, NT, stream);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  switch (out_dtype) {
+    case FLA_F32: return launch_carry<float>(ws_local, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
+    case FLA_BF16: return launch_carry<bf16>(ws_local, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
+    case FLA_F16: return launch_carry<f16>(ws_local, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
     default: return FLA_E_UNSUPPORTED;
   }
 }

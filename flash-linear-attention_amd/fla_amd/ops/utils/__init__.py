@@ -1,3 +1,3 @@
-from .cumsum import chunk_local_cumsum
+from .cumsum import chunk_global_cumsum, chunk_local_cumsum
 
-__all__ = ['chunk_local_cumsum']
+__all__ = ['chunk_global_cumsum', 'chunk_local_cumsum']

@@ -1,5 +1,6 @@
-"""``chunk_local_cumsum`` with the reference's signature
-(``fla/ops/utils/cumsum.py:389-407``), served by ``fla_chunk_local_cumsum``."""
+"""``chunk_local_cumsum`` and ``chunk_global_cumsum`` with the reference's signatures
+(``fla/ops/utils/cumsum.py:389-407`` and ``:366-386``), served by ``fla_chunk_local_cumsum`` and
+``fla_chunk_global_cumsum``."""
 from typing import Optional
 
 import torch
@@ -43,4 +44,46 @@ def chunk_local_cumsum(
     be.check(be.lib().fla_chunk_local_cumsum(
         be.ptr(g), be.ptr(out), be.dt(g), B, T, H, S, chunk_size, int(bool(reverse)),
         be.ptr(offsets), be.ptr(indices), NT, be.stream_of(g)), "fla_chunk_local_cumsum")
+    return out
+
+
+def chunk_global_cumsum(
+    s: torch.Tensor,
+    dtype: Optional[torch.dtype] = None,
+    reverse: bool = False,
+    offsets: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+) -> torch.Tensor:
+    """Cumulative sum along time over each whole sequence; ``s`` is ``[B,H,T]`` / ``[B,H,T,D]``
+    (``[B,T,H]`` / ``[B,T,H,D]`` if not ``head_first``), the result has dtype ``dtype or s.dtype``."""
+    if offsets is not None:
+        assert s.shape[0] == 1, "Only batch size 1 is supported when offsets are provided"
+    if s.dim() not in (3, 4):
+        raise ValueError(f"Unsupported input shape {s.shape}. "
+                         f"which should be [B, H, T]/[B, H, T, D] if `head_first=True` "
+                         f"or [B, T, H]/[B, T, H, D] otherwise")
+    be.require_gpu(s)
+    if head_first:
+        out = chunk_global_cumsum(s.transpose(1, 2), dtype, reverse, offsets, head_first=False)
+        return out.transpose(1, 2).contiguous()
+    s = s.contiguous()
+    B, T, H = s.shape[:3]
+    S = s.shape[3] if s.dim() == 4 else 1
+    out = torch.empty_like(s, dtype=dtype or s.dtype)
+    if s.numel() == 0:
+        return out
+    # parallel grain: at most about 64 chunks per sequence, so the carry pass stays short
+    longest = T
+    chunk_size = 64
+    while chunk_size * 64 < longest:
+        chunk_size *= 2
+    indices, NT = None, 0
+    if offsets is not None:
+        plan = VarlenPlan(offsets, chunk_size)
+        offsets, indices = plan.offsets.to(torch.int64).contiguous(), plan.indices.to(torch.int64).contiguous()
+        NT = indices.shape[0]
+    ws = torch.empty_like(s, dtype=torch.float32)
+    be.check(be.lib().fla_chunk_global_cumsum(
+        be.ptr(s), be.ptr(ws), be.ptr(out), be.dt(s), be.dt(out), B, T, H, S, chunk_size, int(bool(reverse)),
+        be.ptr(offsets), be.ptr(indices), NT, be.stream_of(s)), "fla_chunk_global_cumsum")
     return out

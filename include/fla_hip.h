@@ -67,6 +67,16 @@ int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype,
                            const int64_t* offsets, const int64_t* indices, int64_t NT,
                            fla_stream_t stream);
 
+/* Cumulative sum over the whole sequence (not restarted at chunk boundaries), replaces
+ * chunk_global_cumsum (fla/ops/utils/cumsum.py:308-386).  Two launches: chunk-local sums into
+ * ws_local (fp32, same shape as s), then each chunk adds the totals of the chunks before
+ * (reverse: after) it.  chunk_size is the caller's choice of parallel grain (a power of two;
+ * sequence length / 64 keeps the second pass short); offsets/indices as for the local sum,
+ * built for the same chunk_size.  out in out_dtype. */
+int fla_chunk_global_cumsum(const void* s, float* ws_local, void* out, int s_dtype, int out_dtype, int64_t B,
+                            int64_t T, int64_t H, int64_t S, int64_t chunk_size, int reverse,
+                            const int64_t* offsets, const int64_t* indices, int64_t NT, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Token-by-token recurrence, forward (fla/ops/common/fused_recurrent.py:322-378,
  * kernel :27-128).  Any of g [B,T,H], gk [B,T,H,K], gv [B,T,H,V] may be NULL;

@@ -57,3 +57,40 @@ def test_cumsum_varlen(device, T, N, S, reverse):
     out = chunk_local_cumsum(g.to(device), 64, reverse=reverse, offsets=offs.to(device), head_first=False)
     ref = ref_cumsum(g, 64, reverse=reverse, offsets=offs.tolist())
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("shape", [(2, 1, 3), (2, 300, 3), (1, 5000, 2, 64), (2, 130, 4, 20), (1, 70, 3, 1)])
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_global_cumsum(device, shape, reverse, dtype):
+    """Whole-sequence cumulative sum against torch.cumsum in fp64 (fp32 accumulation on the device:
+    1e-5 relative for fp32 output; one rounding for bf16 output)."""
+    from fla_amd.ops.utils import chunk_global_cumsum
+    gen = torch.Generator().manual_seed(len(shape) + shape[1])
+    s = torch.randn(*shape, generator=gen).to(dtype)
+    print(f"global cumsum {shape} reverse={reverse} {dtype}", flush=True)
+    out = chunk_global_cumsum(s.to(device), reverse=reverse, head_first=False)
+    x = s.double()
+    ref = x.flip(1).cumsum(1).flip(1) if reverse else x.cumsum(1)
+    assert out.dtype == dtype and out.shape == s.shape
+    assert_close("cumsum", ref, out, 1e-5 if dtype == torch.float32 else 4e-3)
+    out32 = chunk_global_cumsum(s.transpose(1, 2).contiguous().to(device), dtype=torch.float32, reverse=reverse,
+                                head_first=True)
+    assert out32.dtype == torch.float32
+    assert_close("cumsum head-first fp32", ref.transpose(1, 2), out32, 1e-5)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_global_cumsum_varlen(device, reverse):
+    from fla_amd.ops.utils import chunk_global_cumsum
+    gen = torch.Generator().manual_seed(17)
+    T, N = 700, 5
+    offs = random_offsets(T, N, gen, min_len=1)
+    s = torch.randn(1, T, 3, 8, generator=gen)
+    print(f"global cumsum varlen offs={offs.tolist()} reverse={reverse}", flush=True)
+    out = chunk_global_cumsum(s.to(device), reverse=reverse, offsets=offs.to(device), head_first=False)
+    ref = torch.empty_like(s, dtype=torch.float64)
+    for a, b in zip(offs[:-1].tolist(), offs[1:].tolist()):
+        x = s[:, a:b].double()
+        ref[:, a:b] = x.flip(1).cumsum(1).flip(1) if reverse else x.cumsum(1)
+    assert_close("cumsum", ref, out, 1e-5)
