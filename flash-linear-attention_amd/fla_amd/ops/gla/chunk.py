@@ -169,6 +169,19 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     return dq, dk, dv, dg, dh0
 
 
+def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
+                  offsets=None, indices=None, head_first=True, chunk_size=64):
+    """Reference-shaped backward (``fla/ops/gla/chunk.py:1217-1320``) for internal callers:
+    returns ``(dq, dk, dv, dg, dh0)`` with ``dg`` the gradient of the raw gates ``g``.  The
+    per-chunk states and scores are recomputed on chip, so ``g_cumsum``, ``h`` and ``A`` are
+    accepted and ignored; tensors must be seq-first, 16-bit, with head dims of 64 or 128."""
+    if head_first:
+        raise NotImplementedError("fla_amd chunk_gla_bwd: seq-first layout only")
+    if g is None:
+        raise NotImplementedError("fla_amd chunk_gla_bwd: needs the raw gates g (the kernels form the cumulative sums)")
+    return chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht, offsets)
+
+
 class ChunkGLAFunction(torch.autograd.Function):
 
     @staticmethod

@@ -245,3 +245,22 @@ def test_chunk_gla_backward_extreme_gates_mixed_varlen(device):
     ref = _grads_ref(q, k, v, g, h0, do, dht, offsets=offs.tolist())
     for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, got, (1e-2, 1e-2, 1e-2, 2e-2, 5e-3)):
         assert_close(name, r, x, tol)
+
+
+def test_chunk_gla_internal_fwd_bwd_signatures(device):
+    """The reference-shaped internal entry points other operators build on (chunk_gla_fwd /
+    chunk_gla_bwd, fla/ops/gla/chunk.py:1156-1320): same gradients as the public operator."""
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd, chunk_gla_fwd
+    B, T, H, D = 2, 200, 2, 128
+    q, k, v, g, h0 = gla_inputs(B, T, H, D, D, seed=33, h0_std=1.0)
+    gen = torch.Generator().manual_seed(9)
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(B, H, D, D, generator=gen) * 0.1
+    dev = lambda x: x.to(device)
+    print("chunk_gla_fwd / chunk_gla_bwd internal signatures", flush=True)
+    gc, A, h, ht, o = chunk_gla_fwd(dev(q), dev(k), dev(v), dev(g), None, D ** -0.5, dev(h0), True, head_first=False)
+    dq, dk, dv, dg, dh0 = chunk_gla_bwd(dev(q), dev(k), dev(v), dev(g), gc, D ** -0.5, dev(h0), h, A, dev(do), dev(dht),
+                                        head_first=False)
+    ref = _grads_ref(q, k, v, g, h0, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, (dq, dk, dv, dg, dh0), (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(name, r, x, tol)
