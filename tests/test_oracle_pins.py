@@ -18,12 +18,21 @@ def _rand(*shape, seed=0):
 
 
 # ---------------------------------------------------------------- bookkeeping (integer, bit exact)
+def _known_answer():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "chunk_indices_known_answer.json")) as f:
+        return json.load(f)
+
+
 def test_chunk_indices_known_answer():
-    # fla/ops/gla/chunk.py:1352-1355: offsets [0,100,356], chunk 64
-    idx = bookkeeping.prepare_chunk_indices([0, 100, 356], 64)
+    # the reference's stored known answer (fla/ops/gla/chunk.py:1352-1355), kept as a fixture
+    ka = _known_answer()
+    idx = bookkeeping.prepare_chunk_indices(ka["offsets"], ka["chunk_size"])
     assert idx.dtype == np.int64
-    assert idx.tolist() == [[0, 0], [0, 1], [1, 0], [1, 1], [1, 2], [1, 3]]
-    assert bookkeeping.prepare_chunk_offsets([0, 100, 356], 64).tolist() == [0, 2, 6]
+    assert idx.tolist() == ka["indices"]
+    assert ka["offsets"] == [0, 100, 356] and ka["chunk_size"] == 64
+    assert bookkeeping.prepare_chunk_offsets(ka["offsets"], ka["chunk_size"]).tolist() == [0, 2, 6]
 
 
 @pytest.mark.parametrize("bt", [16, 32, 64])
