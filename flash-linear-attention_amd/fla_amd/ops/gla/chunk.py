@@ -281,5 +281,29 @@ def chunk_gla(
     check_varlen_args(q, offsets, head_first, initial_state)
     if scale is None:
         scale = q.shape[-1] ** -0.5
+    K, V = q.shape[-1], v.shape[-1]
+    if K > 128:
+        # every key channel carries its own row of the state and o sums over them: wider key heads
+        # run as slabs of 128 channels whose outputs are added (in fp32)
+        o_sum, states = None, []
+        for k0 in range(0, K, 128):
+            ks = slice(k0, k0 + 128)
+            h0 = None if initial_state is None else initial_state[..., ks, :]
+            o, ht = chunk_gla(q[..., ks], k[..., ks], v, g[..., ks], scale=scale, initial_state=h0,
+                              output_final_state=output_final_state, offsets=offsets, head_first=head_first)
+            o_sum = o.float() if o_sum is None else o_sum + o.float()
+            states.append(ht)
+        return o_sum.to(v.dtype), (torch.cat(states, dim=-2) if output_final_state else None)
+    if V > 128:
+        # value columns are independent in the recurrence: wider heads run as slabs of 128 columns
+        # (autograd sums the slabs' gradients of q, k and g)
+        outs, states = [], []
+        for v0 in range(0, V, 128):
+            h0 = None if initial_state is None else initial_state[..., v0:v0 + 128]
+            o, ht = ChunkGLAFunction.apply(q, k, v[..., v0:v0 + 128], g, scale, h0, output_final_state, offsets,
+                                           head_first)
+            outs.append(o)
+            states.append(ht)
+        return torch.cat(outs, dim=-1), (torch.cat(states, dim=-1) if output_final_state else None)
     o, final_state = ChunkGLAFunction.apply(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
     return o, final_state

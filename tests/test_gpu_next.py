@@ -5,7 +5,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import assert_close, gdr_inputs, random_offsets
+from helpers import assert_close, gdr_inputs, gla_inputs, random_offsets
 
 pytestmark = pytest.mark.gpu
 
@@ -106,3 +106,56 @@ def test_fused_recurrent_simple_gla(device, T):
     ro, rht = naive_recurrent_gla(q, k, v, None, g=g, initial_state=h0, output_final_state=True)
     assert_close("o", ro, o, 1e-5)
     assert_close("ht", rht, ht, 1e-5)
+
+
+@pytest.mark.parametrize("K,V", [(128, 256), (256, 128), (192, 320)])
+def test_chunk_gla_wide_heads(device, K, V):
+    """Head dims above the built 128-wide tiles: key channels and value columns are independent
+    in the GLA recurrence, so the operator runs slabs of 128 (the reference allows K <= 256)."""
+    from fla_amd.ops.gla import chunk_gla
+    from oracle.recurrent import naive_recurrent_gla
+    B, T, H = 2, 150, 2
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=K + V, h0_std=1.0)
+    gen = torch.Generator().manual_seed(3)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"chunk_gla wide heads K={K} V={V}", flush=True)
+    leaves = [dev(x).requires_grad_() for x in (q, k, v, g)]
+    h0l = dev(h0).requires_grad_()
+    o, ht = chunk_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=False)
+    ((o.float() * dev(do).float()).sum() + (ht * dev(dht)).sum()).backward()
+    refs = [x.float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gla(*refs, initial_state=rh0, output_final_state=True)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), refs, leaves):
+        assert_close(name, a.grad, b.grad, 1e-2)
+    assert_close("dh0", rh0.grad, h0l.grad, TOL_G)
+
+
+def test_chunk_gdr_wide_values(device):
+    """Value head dims above 128 for the gated delta rule (independent per value column)."""
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    B, T, H, K, V = 2, 150, 2, 128, 256
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=77, h0_std=1.0)
+    gen = torch.Generator().manual_seed(4)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dev = _dev(device)
+    print("chunk_gated_delta_rule V=256", flush=True)
+    leaves = [dev(x).requires_grad_() for x in (q, k, v, g, beta)]
+    h0l = dev(h0).requires_grad_()
+    o, ht = chunk_gated_delta_rule(*leaves, initial_state=h0l, output_final_state=True, head_first=False)
+    (o.float() * dev(do).float()).sum().backward()
+    refs = [x.float().requires_grad_() for x in (q, k, v, g, beta)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gated_delta_rule(*refs, initial_state=rh0, output_final_state=True)
+    (ro * do.float()).sum().backward()
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    for name, a, b, tol in zip(("dq", "dk", "dv", "dg", "dbeta"), refs, leaves, (8e-3, 8e-3, 8e-3, 2e-2, 2e-2)):
+        assert_close(name, a.grad, b.grad, tol)
+    assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
