@@ -85,6 +85,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   __shared__ __attribute__((aligned(16))) float sDecay[2][K];
   __shared__ __attribute__((aligned(16))) T sP[BT * LDT];        // tril(S) [i][j]
   __shared__ __attribute__((aligned(16))) T sHf[KT32 * 2 * 64 * 16];  // state, fragment order [kt][vt][lane][16]
+  __shared__ __attribute__((aligned(16))) T sO[BT * LDT];        // finished output tile [t][v]
   __shared__ int sWide[2][NSTG];                                   // per staging wave: gates out of range
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -266,6 +267,33 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     };
 
+    // The matrix waves leave each finished output tile in LDS; the staging waves write it to
+    // memory one chunk period later as whole 128-byte rows (8 lanes x 16 bytes per row).
+    constexpr int NPO = BT * (BV / 8) / (64 * NSTG);
+    const uint32_t opitch = (uint32_t)H * V * (uint32_t)sizeof(T);
+    uint32_t offo[NPO];
+    int ldo[NPO], orow[NPO];
+#pragma unroll
+    for (int i = 0; i < NPO; ++i) {
+      const int e = (tid - 256) + 64 * NSTG * i;
+      orow[i] = e >> 3;
+      ldo[i] = orow[i] * LDT + (e & 7) * 8;
+      offo[i] = (uint32_t)orow[i] * opitch + (uint32_t)((e & 7) * 8) * (uint32_t)sizeof(T);
+    }
+    char* po = (char*)p.o + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const int64_t stro = (int64_t)BT * opitch;
+    int64_t oc = 0;  // chunk whose output tile is stored next
+    auto store_o = [&]() __attribute__((always_inline)) {
+      const int Lc = oc == nchunks - 1 ? Llast : BT;
+#pragma unroll
+      for (int i = 0; i < NPO; ++i) {
+        const v8 x = *(const v8*)&sO[ldo[i]];
+        if (orow[i] < Lc) *(v8*)(po + offo[i]) = x;
+      }
+      po += stro;
+      ++oc;
+    };
+
     if (nchunks > 0) {
       // Two register sets, used alternately: the loads refilling a set have two chunk periods
       // to land before it is staged again.
@@ -286,14 +314,18 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       end_loads();
       stage(RA, 0, 0, [] {});
       for (int64_t c = 0; c < nchunks; c += 2) {
-        lds_barrier();  // B1(c): tiles of chunk c published; buffer 1 is free
+        lds_barrier();  // B1(c): tiles of chunk c and the output tile of chunk c-1 published; buffer 1 is free
+        if (c > 0) store_o();
         if (c + 1 < nchunks) stage(RB, 1, c + 1, [] { lds_barrier(); });  // contains B2(c)
         else lds_barrier();  // B2(c)
         if (c + 1 >= nchunks) break;
         lds_barrier();  // B1(c+1)
+        store_o();
         if (c + 2 < nchunks) stage(RA, 0, c + 2, [] { lds_barrier(); });  // contains B2(c+1)
         else lds_barrier();  // B2(c+1)
       }
+      lds_barrier();  // the last output tile is published
+      store_o();
     }
   } else {
     // =========================== matrix waves ===========================
@@ -453,17 +485,15 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           o = Elem<T>::mfma32(lds_frag32<T>(sVt[buf], LDT, cw * 32, js, lane), lds_frag32<T>(sP, LDT, 32, js, lane), o);
       }
       {
-        // o^T tile: lane <-> time row, registers <-> value columns 8 (r/4) + 4 (lane/32) + r%4
-        const int i = rw * 32 + (lane & 31);
-        if (i < L) {
-          T* op = (T*)p.o + ((row0 + i) * H + hh) * (int64_t)V + vbase + cw * 32 + 4 * (lane >> 5);
+        // o^T tile: lane <-> time row, registers <-> value columns 8 (r/4) + 4 (lane/32) + r%4.
+        // Left in LDS for the staging waves (rows past the end of a short chunk are not stored).
+        T* orow_ = &sO[(rw * 32 + (lane & 31)) * LDT + cw * 32 + 4 * (lane >> 5)];
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            v4 ov;
+        for (int r4 = 0; r4 < 4; ++r4) {
+          v4 ov;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) ov[e] = (T)(o[4 * r4 + e] * p.scale);
-            *(v4*)(op + 8 * r4) = ov;
-          }
+          for (int e = 0; e < 4; ++e) ov[e] = (T)(o[4 * r4 + e] * p.scale);
+          *(v4*)(orow_ + 8 * r4) = ov;
         }
       }
       // ---- state update
@@ -490,6 +520,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       publish_state();
     }
+    if (nchunks > 0) lds_barrier();  // hands the last output tile to the staging waves
     if (p.ht) {
       float* htp = p.ht + (int64_t)nh * K * V;
 #pragma unroll
