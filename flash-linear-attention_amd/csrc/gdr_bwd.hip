@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   constexpr int C8 = K / 8, NP = BT * C8 / 256;
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int TV = V / 64;
-  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
+  constexpr int LDV = V + 8;
+  __shared__ __attribute__((aligned(16))) T sQ[BT * (K > V ? LDK : LDV)];   // q; later the dv tile [t][v]
   __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
   __shared__ __attribute__((aligned(16))) T sDt[V * LDT];
   __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];
@@ -121,20 +122,35 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   f32x16 acc[TV];
 #pragma unroll
   for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+  // transposed product (do^T A): a lane ends up with one time row and four consecutive value
+  // columns per register quad; the tile leaves through LDS (the q tile is dead) as whole rows
   for (int is = rw * 32; is < BT; is += 16) {
     v8 a = lds_frag32<T>(sPT, LDT, rw * 32, is, lane);
 #pragma unroll
     for (int tv = 0; tv < TV; ++tv)
-      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), acc[tv]);
+      acc[tv] = Elem<T>::mfma32(lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), a, acc[tv]);
   }
+  T* sO = sQ;
+  {
+    T* orow = &sO[(rw * 32 + (lane & 31)) * LDV + cw * TV * 32 + 4 * (lane >> 5)];
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        v4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = (T)acc[tv][4 * r4 + e];
+        *(v4*)(orow + tv * 32 + 8 * r4) = x;
+      }
+  }
+  __syncthreads();
+  constexpr int C8V = V / 8;
   T* op = (T*)p.dvl + (row0 * H + hh) * (int64_t)V;
 #pragma unroll
-  for (int tv = 0; tv < TV; ++tv)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = rw * 32 + c32_row(r, lane);
-      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
-    }
+  for (int i = 0; i < BT * C8V / 256; ++i) {
+    const int e = tid + 256 * i, row = e / C8V, c8 = (e % C8V) * 8;
+    if (row < L) *(v8*)(op + (int64_t)row * H * V + c8) = *(const v8*)&sO[row * LDV + c8];
+  }
 }
 
 // ---------------------------------------------------------------------------

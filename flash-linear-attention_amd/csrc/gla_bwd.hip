@@ -245,7 +245,8 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int KT32 = K / 32, TV = V / 64;
-  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];    // s q e^{G-G_last}
+  constexpr int LDV = V + 8;
+  __shared__ __attribute__((aligned(16))) T sQ[BT * (K > V ? LDK : LDV)];   // s q e^{G-G_last}; later the dv tile [t][v]
   __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];   // k e^{G_last-G}
   __shared__ __attribute__((aligned(16))) T sDt[V * LDT];    // do^T [v][i]
   __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];   // A^T [j][i]
@@ -367,7 +368,8 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     }
   }
   __syncthreads();
-  // ---- dv = A^T do + k^ dH
+  // ---- dv^T = do^T A + dH^T k^^T (transposed products: a lane ends up with one time row and four
+  // consecutive value columns per register quad)
   f32x16 acc[TV];
 #pragma unroll
   for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     v8 a = lds_frag32<T>(sPT, LDT, rw * 32, is, lane);
 #pragma unroll
     for (int tv = 0; tv < TV; ++tv)
-      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), acc[tv]);
+      acc[tv] = Elem<T>::mfma32(lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), a, acc[tv]);
   }
 #pragma unroll
   for (int kt = 0; kt < KT32; ++kt)
@@ -383,16 +385,30 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     for (int half = 0; half < 2; ++half) {
       v8 a = lds_frag32_perm<T>(sKh, LDK, rw * 32, kt * 32 + half * 16, lane);
 #pragma unroll
-      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(a, hf[kt][tv][half], acc[tv]);
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(hf[kt][tv][half], a, acc[tv]);
     }
+  // the q tile is dead since the score phase: the dv tile goes through it and leaves as whole rows
+  T* sO = sQ;
+  {
+    T* orow = &sO[(rw * 32 + (lane & 31)) * LDV + cw * TV * 32 + 4 * (lane >> 5)];
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        v4 x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = (T)acc[tv][4 * r4 + e];
+        *(v4*)(orow + tv * 32 + 8 * r4) = x;
+      }
+  }
+  __syncthreads();
+  constexpr int C8V = V / 8;
   T* op = (T*)p.dv + (row0 * H + hh) * (int64_t)V;
 #pragma unroll
-  for (int tv = 0; tv < TV; ++tv)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = rw * 32 + c32_row(r, lane);
-      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
-    }
+  for (int i = 0; i < BT * C8V / 256; ++i) {
+    const int e = tid + 256 * i, row = e / C8V, c8 = (e % C8V) * 8;
+    if (row < L) *(v8*)(op + (int64_t)row * H * V + c8) = *(const v8*)&sO[row * LDV + c8];
+  }
 }
 
 // ---------------------------------------------------------------------------
