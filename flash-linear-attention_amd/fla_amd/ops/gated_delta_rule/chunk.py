@@ -7,6 +7,7 @@ Forward pipeline on the device (chunk size 64): ``fla_chunk_local_cumsum`` (gate
 The backward recomputes w, u, the per-chunk states and v_new with
 ``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
 """
+import warnings
 from typing import Optional, Tuple
 
 import torch
@@ -200,7 +201,25 @@ def chunk_gated_delta_rule(
         scale = k.shape[-1] ** -0.5
     else:
         assert scale > 0, "Scale must be positive."
-    V = v.shape[-1]
+    K, V = k.shape[-1], v.shape[-1]
+    if 128 < K <= 256:
+        # The chunk kernels hold at most 128 key channels of the state (the delta rule couples all of
+        # them, so there are no independent slabs).  Without gradients the token-by-token kernel
+        # computes the same operator for up to 256 channels: slower (serial in time), not approximate.
+        if torch.is_grad_enabled() and any(t is not None and t.requires_grad
+                                           for t in (q, k, v, g, beta, initial_state)):
+            raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: the backward needs the chunk kernels, which "
+                                      f"cover key head dims up to 128 (got {K})")
+        from .fused_recurrent import fused_recurrent_gated_delta_rule
+        if not getattr(chunk_gated_delta_rule, "_warned_wide_k", False):
+            warnings.warn(f"fla_amd chunk_gated_delta_rule: key head dim {K} > 128 runs on the token-by-token "
+                          f"kernel (forward only)", stacklevel=2)
+            chunk_gated_delta_rule._warned_wide_k = True
+        if g is None:
+            g = torch.zeros_like(beta, dtype=torch.float32)
+        return fused_recurrent_gated_delta_rule(q, k, v, g, beta, scale=scale, initial_state=initial_state,
+                                                output_final_state=output_final_state, offsets=offsets,
+                                                head_first=head_first)
     if V > 128:
         # the delta rule is independent per value column: wider heads run as slabs of 128 columns
         # (autograd sums the slabs' gradients of q, k, g and beta)

@@ -159,3 +159,24 @@ def test_chunk_gdr_wide_values(device):
     for name, a, b, tol in zip(("dq", "dk", "dv", "dg", "dbeta"), refs, leaves, (8e-3, 8e-3, 8e-3, 2e-2, 2e-2)):
         assert_close(name, a.grad, b.grad, tol)
     assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
+
+
+def test_chunk_gdr_wide_keys_forward_only(device):
+    """Key head dim 256 (the default of the reference's GatedDeltaNet layer): served without gradients
+    by the token-by-token kernel; with gradients the operator refuses loudly."""
+    import warnings
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    B, T, H, K, V = 1, 200, 2, 256, 128
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=78, h0_std=1.0)
+    dev = _dev(device)
+    print("chunk_gated_delta_rule K=256 (forward only)", flush=True)
+    with torch.no_grad(), warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), initial_state=dev(h0),
+                                       output_final_state=True, head_first=False)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    with pytest.raises(NotImplementedError):
+        chunk_gated_delta_rule(dev(q).requires_grad_(), dev(k), dev(v), dev(g), dev(beta), head_first=False)
