@@ -74,9 +74,8 @@ struct ChunkLoc {
 // head-fastest: workgroups that run together take different heads of the same chunks, whose rows
 // are adjacent in memory, and the traffic spreads evenly over the memory channels (a
 // chunk-fastest order makes concurrent workgroups hit the same address bits 8-11).
-FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix, int H,
-                                 int* head) {
-  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+FLA_DEVICE ChunkLoc locate_chunk_at(int64_t lin, const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix,
+                                    int H, int* head) {
   const int64_t cidx = lin / H;
   *head = (int)(lin % H);
   ChunkLoc c;
@@ -96,6 +95,10 @@ FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices,
   c.L = (int)(rem < BT ? rem : BT);
   c.cglob = cidx;
   return c;
+}
+FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix, int H,
+                                 int* head) {
+  return locate_chunk_at((int64_t)blockIdx.y * gridDim.x + blockIdx.x, offsets, indices, T, ntfix, H, head);
 }
 
 inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B, int64_t T, int64_t H, int64_t NT,

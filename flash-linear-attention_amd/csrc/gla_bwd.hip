@@ -722,6 +722,7 @@ struct BExactParams {
   int64_t T;
   int H, NTfix;
   float scale;
+  int64_t total;   // (chunk, head) pairs
 };
 
 template <typename T, typename GT, int K, int V>
@@ -731,9 +732,12 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
   constexpr int VD_BYTES = 2 * BT * LDVV * 2;
   constexpr int X_BYTES = BT * LDG * 4;
   const int H = p.H;
+  // a few hundred workgroups walk the (chunk, head) flags (almost always none is set)
+  for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
+  if (p.wide[lin] == 0) continue;  // workgroup-uniform
+  __syncthreads();                 // the tiles of the previous flagged chunk are free
   int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
-  if (p.wide[cl.cglob * H + hh] == 0) return;  // workgroup-uniform
+  ChunkLoc cl = locate_chunk_at(lin, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   __shared__ float sG[BT * LDG];
   __shared__ __attribute__((aligned(16))) T sQ[BT * LDQ];
   __shared__ __attribute__((aligned(16))) T sK[BT * LDQ];
@@ -862,6 +866,7 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
       p.dg[baseK + t * strideK + c] += run;
     }
   }
+  }
 }
 
 template <typename T, typename GT>
@@ -902,9 +907,11 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   if (wide) {
-    BExactParams p{q, k, v, g, dout, wide, dq, dk, dv, dg, offsets, indices, T_, (int)H, ntfix, scale};
+    BExactParams p{q, k, v, g, dout, wide, dq, dk, dv, dg, offsets, indices, T_, (int)H, ntfix, scale,
+                   (int64_t)grid.x * grid.y};
+    const dim3 gx((unsigned)(p.total < 512 ? p.total : 512));
 #define FLA_CASE(KK, VV)                                                                                      \
-  if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_intra_exact_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
+  if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_intra_exact_kernel<T, GT, KK, VV>), gx, dim3(256), 0, st, p);
     FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
 #undef FLA_CASE
     FLA_CHECK_LAUNCH();

@@ -555,6 +555,7 @@ struct ExactParams {
   int64_t T;
   int H, NTfix;
   float scale;
+  int64_t total;   // (chunk, head) pairs
 };
 
 template <typename T, typename GT, int K, int V>
@@ -567,9 +568,13 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int KT32 = K / 32, TV = V / 64;
   const int H = p.H;
+  // A few hundred workgroups walk the (chunk, head) flags: almost always none is set, and a
+  // launch of one workgroup per chunk would cost more than the scan.
+  for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
+  if (p.wide[lin] == 0) continue;  // workgroup-uniform
+  __syncthreads();                 // the tiles of the previous flagged chunk are free
   int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
-  if (p.wide[cl.cglob * H + hh] == 0) return;  // workgroup-uniform
+  ChunkLoc cl = locate_chunk_at(lin, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   __shared__ __attribute__((aligned(16))) float sG[BT * LDG];
   __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
   __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
@@ -693,6 +698,7 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
       int i = rw * 32 + c32_row(r, lane);
       if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
     }
+  }
 }
 
 template <typename T, typename GT>
@@ -750,7 +756,9 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
     int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
     if (rc) return rc;
   }
-  ExactParams e{q, k, v, gates, ws_wide, ws_hwide, o, offsets, indices, T, (int)H, ntfix, scale};
+  ExactParams e{q, k, v, gates, ws_wide, ws_hwide, o, offsets, indices, T, (int)H, ntfix, scale,
+                (int64_t)grid.x * grid.y};
+  if (ws_wide) grid = dim3((unsigned)(e.total < 512 ? e.total : 512));
 #define FLA_FUSED(TT, GG)                                                \
   {                                                                      \
     int rc = launch_fused<TT, GG>(p, (int)K, st);                        \
