@@ -112,7 +112,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     // A staging wave owns CPW key columns; a lane owns CPL adjacent columns of 4 rows.  The 16
     // row groups of a column block sit in the 16 lanes of one DPP row, so the prefix sum over
     // time is register adds plus DPP row shifts.
-    constexpr int LPR = 4;                // lanes (column blocks) per row of the tile
     constexpr int RPT = 4;                // rows per lane
     const int pw = wave - 4;
     const int rg = lane & 15;
@@ -409,8 +408,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     }
     for (int64_t c = 0; c < nchunks; ++c) {
       const int buf = (int)(c & 1);
-      const int L = chunk_len(c);
-      const int64_t row0 = sp.bos + c * BT;
       lds_barrier();  // B1(c)
       if (p.wide) {
         int wide = 0;
