@@ -183,7 +183,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   typedef T t2 __attribute__((ext_vector_type(2)));
   constexpr int BV = 32;
   constexpr int LDK = K + 8;
-  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;   // q, w, k: a lane owns RPT rows x 4 columns
   constexpr int KT32 = K / 32;
   constexpr int NKT = (KT32 + 3) / 4;
   __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];    // k e^{gamma_last-gamma}, row-major
@@ -240,71 +240,87 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
     int64_t rem = sp.len - c * BT;
     return (int)(rem < BT ? rem : BT);
   };
-  auto load_x = [&](int64_t c, XRegs& R) {
-    bool live = c >= 0;
-    int L = chunk_len(c);
-    int64_t rbase = sp.bos + c * BT;
+  // Loads are unconditional (a load under a branch makes the wave drain its whole load queue at the
+  // join): byte offsets of this lane's rows from the first row of a chunk are computed once, rows past
+  // the end of a short chunk are redirected to its last row, chunks before the first one to chunk 0;
+  // the staging functions zero what must not count.
+  const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
+  const uint32_t pitchG = (uint32_t)H * 4u;
+  uint32_t offk[RPT], offg[RPT], offv[4];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    offk[i] = (uint32_t)(rg * RPT + i) * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
+    offg[i] = (uint32_t)(rg * RPT + i) * pitchG;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) offv[i] = (uint32_t)(urg * 4 + i) * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+  const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
+  const char* gq = (const char*)p.q + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+  const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+  const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+  const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+  const char* gl = (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+  const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : gq;
+  auto load_x = [&](int64_t c, XRegs& R) __attribute__((always_inline)) {
+    c = c < 0 ? 0 : c;
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      if (live && row < L) {
-        int64_t off = ((rbase + row) * H + hh) * (int64_t)K + c4;
-        R.q[i] = *(const v4*)((const T*)p.q + off);
-        R.w[i] = *(const v4*)((const T*)p.w + off);
-        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
-      } else {
-        R.q[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.w[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.gam[i] = 0.f;
-      }
+      const uint32_t lk = last * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
+      const uint32_t o = offk[i] < lk ? offk[i] : lk;
+      R.q[i] = *(const v4*)(gq + ck + o);
+      R.w[i] = *(const v4*)(gw + ck + o);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      int row = urg * 4 + i;
-      if (live && row < L)
-        R.d[i] = *(const t2*)((const T*)p.dout + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
-      else R.d[i] = t2{(T)0.f, (T)0.f};
+      const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+      R.d[i] = *(const t2*)(gd + cv + (offv[i] < lv ? offv[i] : lv));
     }
   };
-  auto load_y = [&](int64_t c, YRegs& R) {
-    bool live = c >= 0;
-    int L = chunk_len(c);
-    int64_t rbase = sp.bos + c * BT;
+  auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
+    c = c < 0 ? 0 : c;
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV, cg = p.gam ? c * BT * (int64_t)pitchG : 0;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      if (live && row < L) {
-        R.k[i] = *(const v4*)((const T*)p.k + ((rbase + row) * H + hh) * (int64_t)K + c4);
-        R.gam[i] = p.gam ? p.gam[(rbase + row) * H + hh] : 0.f;
-      } else {
-        R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.gam[i] = 0.f;
-      }
+      const uint32_t lk = last * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
+      R.k[i] = *(const v4*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
+      const uint32_t og = offg[i] < last * pitchG ? offg[i] : last * pitchG;
+      R.gam[i] = __uint_as_float(*(const uint32_t*)(gg + cg + (p.gam ? og : 0u)) & gmask);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      int row = urg * 4 + i;
-      if (live && row < L)
-        R.dvl[i] = *(const t2*)((const T*)p.dvl + ((rbase + row) * H + hh) * (int64_t)V + vbase + uc2);
-      else R.dvl[i] = t2{(T)0.f, (T)0.f};
+      const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+      R.dvl[i] = *(const t2*)(gl + cv + (offv[i] < lv ? offv[i] : lv));
     }
-    R.glast = (live && p.gam) ? p.gam[(rbase + L - 1) * H + hh] : 0.f;
+    R.glast = __uint_as_float(*(const uint32_t*)(gg + cg + (p.gam ? last * pitchG : 0u)) & gmask);
   };
-  auto stage_x = [&](const XRegs& R) {
+  auto stage_x = [&](const XRegs& R, int L) {
+    // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
+    typedef T rvec __attribute__((ext_vector_type(RPT)));
+    float eg[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) eg[i] = (rg * RPT + i < L) ? __expf(R.gam[i]) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      T* dq = &sQt[(c4 + j) * LDT + rg * RPT];
-      T* dw = &sWt[(c4 + j) * LDT + rg * RPT];
+      rvec xq, xw;
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        float eg = __expf(R.gam[i]);
-        dq[i] = (T)((float)R.q[i][j] * p.scale * eg);
-        dw[i] = (T)(-(float)R.w[i][j] * eg);
+        xq[i] = (T)((float)R.q[i][j] * p.scale * eg[i]);
+        xw[i] = (T)(-(float)R.w[i][j] * eg[i]);
       }
+      *(rvec*)&sQt[(c4 + j) * LDT + rg * RPT] = xq;
+      *(rvec*)&sWt[(c4 + j) * LDT + rg * RPT] = xw;
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       v4 dv = v4{R.d[0][j], R.d[1][j], R.d[2][j], R.d[3][j]};
+      if (L < BT) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (urg * 4 + i >= L) dv[i] = (T)0.f;
+      }
       *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
     }
   };
@@ -321,6 +337,11 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       v4 dv = v4{R.dvl[0][j], R.dvl[1][j], R.dvl[2][j], R.dvl[3][j]};
+      if (L < BT) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (urg * 4 + i >= L) dv[i] = (T)0.f;
+      }
       *(v4*)&sDvl[(uc2 + j) * LDT + urg * 4] = dv;
     }
   };
@@ -352,15 +373,17 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
 
   XRegs X;
   YRegs Y;
-  load_x(nchunks - 1, X);
-  load_y(nchunks - 1, Y);
   float dec = 1.f;
   if (nchunks > 0) {
+    load_x(nchunks - 1, X);
+    load_y(nchunks - 1, Y);
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) X.gam[i] = Y.gam[i];
     stage_y(Y, chunk_len(nchunks - 1));
     dec = __expf(Y.glast);
     publish(nchunks - 1);
+    load_y(nchunks - 2, Y);
   }
-  load_y(nchunks - 2, Y);
   for (int64_t c = nchunks - 1; c >= 0; --c) {
     const int L = chunk_len(c);
     const int64_t rbase = sp.bos + c * BT;
@@ -383,14 +406,23 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) o[r] = (T)((float)dl[r] + d[j][r]);
         *(v4*)&sDv2T[vc * LDT + tr] = o;
+      }
+      // The wave reads its own 16 rows back in row-major order (its writes only: no barrier) and
+      // stores each row's 32 columns as four 16-byte pieces.
+      {
+        const int row = wave * 16 + (lane >> 2), v0 = (lane & 3) * 8;
+        v8 x;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (tr + r < L) ((T*)p.dv2)[((rbase + tr + r) * H + hh) * (int64_t)V + vbase + vc] = o[r];
+        for (int e = 0; e < 8; ++e) x[e] = sDv2T[(v0 + e) * LDT + row];
+        if (row < L) *(v8*)((T*)p.dv2 + ((rbase + row) * H + hh) * (int64_t)V + vbase + v0) = x;
       }
     }
-    stage_x(X);
+    stage_x(X, L);
     const float dec_c = dec;
     load_x(c - 1, X);
+    // Y holds chunk c-1 at this point, with the same row mapping: its gates serve X as well
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) X.gam[i] = Y.gam[i];
     lds_barrier();  // (2)
     // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
 #pragma unroll
