@@ -28,6 +28,8 @@
 //                              dbeta = sum d(kb)*k + sum d(vb)*v,
 //                              dgamma_i += rowsum_i(X) - colsum_i(X), X = strict_lower(du vb^T) * Au
 //                            (wy_fast.py:440-562, written for the single inverse Aw).
+#include <type_traits>
+
 #include "chunk_common.h"
 
 namespace {
@@ -153,6 +155,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   }
 }
 
+// a word of zeros in device memory: the target of gate loads when an operator has no gates
+__device__ const float kZeroWord = 0.f;
+
 // ---------------------------------------------------------------------------
 struct DhuParams {
   const void* q;
@@ -227,7 +232,6 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   struct XRegs {
     v4 q[RPT];
     v4 w[RPT];
-    float gam[RPT];
     t2 d[4];
   };
   struct YRegs {
@@ -254,13 +258,14 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) offv[i] = (uint32_t)(urg * 4 + i) * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-  const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
   const char* gq = (const char*)p.q + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
   const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
   const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
   const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
   const char* gl = (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
-  const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : gq;
+  // without gates every gate load reads one zero word (no select on the loaded value: it would
+  // make the wave wait for the load where it is issued)
+  const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : (const char*)&kZeroWord;
   auto load_x = [&](int64_t c, XRegs& R) __attribute__((always_inline)) {
     c = c < 0 ? 0 : c;
     const uint32_t last = (uint32_t)(chunk_len(c) - 1);
@@ -287,21 +292,24 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
       const uint32_t lk = last * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
       R.k[i] = *(const v4*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
       const uint32_t og = offg[i] < last * pitchG ? offg[i] : last * pitchG;
-      R.gam[i] = __uint_as_float(*(const uint32_t*)(gg + cg + (p.gam ? og : 0u)) & gmask);
+      R.gam[i] = *(const float*)(gg + cg + (p.gam ? og : 0u));
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
       R.dvl[i] = *(const t2*)(gl + cv + (offv[i] < lv ? offv[i] : lv));
     }
-    R.glast = __uint_as_float(*(const uint32_t*)(gg + cg + (p.gam ? last * pitchG : 0u)) & gmask);
+    R.glast = *(const float*)(gg + cg + (p.gam ? last * pitchG : 0u));
   };
-  auto stage_x = [&](const XRegs& R, int L) {
+  // e^{gamma} of the rows of the chunk held in X (zero past its end): formed when the same chunk is
+  // staged as Y, one iteration earlier, so that nothing loop-carried depends on a load in flight
+  float egx[RPT];
+  auto stage_x = [&](const XRegs& R) {
     // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
     typedef T rvec __attribute__((ext_vector_type(RPT)));
     float eg[RPT];
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) eg[i] = (rg * RPT + i < L) ? __expf(R.gam[i]) : 0.f;
+    for (int i = 0; i < RPT; ++i) eg[i] = egx[i];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       rvec xq, xw;
@@ -316,11 +324,6 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       v4 dv = v4{R.d[0][j], R.d[1][j], R.d[2][j], R.d[3][j]};
-      if (L < BT) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i >= L) dv[i] = (T)0.f;
-      }
       *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
     }
   };
@@ -328,6 +331,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       int row = rg * RPT + i;
+      egx[i] = (row < L) ? __expf(R.gam[i]) : 0.f;
       float e = (row < L) ? __expf(R.glast - R.gam[i]) : 0.f;
       v4 kv;
 #pragma unroll
@@ -377,14 +381,14 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   if (nchunks > 0) {
     load_x(nchunks - 1, X);
     load_y(nchunks - 1, Y);
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) X.gam[i] = Y.gam[i];
     stage_y(Y, chunk_len(nchunks - 1));
     dec = __expf(Y.glast);
     publish(nchunks - 1);
     load_y(nchunks - 2, Y);
   }
-  for (int64_t c = nchunks - 1; c >= 0; --c) {
+  // One chunk of the reverse scan.  The first chunk of the sequence (processed last) is peeled off
+  // so that the steady-state loop has no memory operation under a branch.
+  auto step = [&](int64_t c, auto more) __attribute__((always_inline)) {
     const int L = chunk_len(c);
     const int64_t rbase = sp.bos + c * BT;
     lds_barrier();  // (1)
@@ -417,12 +421,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
         if (row < L) *(v8*)((T*)p.dv2 + ((rbase + row) * H + hh) * (int64_t)V + vbase + v0) = x;
       }
     }
-    stage_x(X, L);
+    stage_x(X);
     const float dec_c = dec;
     load_x(c - 1, X);
-    // Y holds chunk c-1 at this point, with the same row mapping: its gates serve X as well
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) X.gam[i] = Y.gam[i];
     lds_barrier();  // (2)
     // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
 #pragma unroll
@@ -447,13 +448,15 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
         }
       }
     }
-    if (c > 0) {
+    if constexpr (decltype(more)::value) {
       stage_y(Y, chunk_len(c - 1));
       dec = __expf(Y.glast);
       publish(c - 1);
       load_y(c - 2, Y);
     }
-  }
+  };
+  for (int64_t c = nchunks - 1; c >= 1; --c) step(c, std::true_type{});
+  if (nchunks > 0) step(0, std::false_type{});
   if (p.dh0) {
     float* o = p.dh0 + (int64_t)nh * K * V;
 #pragma unroll
