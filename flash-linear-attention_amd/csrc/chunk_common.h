@@ -10,6 +10,10 @@ constexpr int BT = 64;        // chunk length
 constexpr int LDT = BT + 8;   // row pitch of time-contiguous 16-bit LDS tiles
 constexpr int LDM = BT + 4;   // row pitch of fp32 64-column LDS tiles
 
+// A word of zeros in device memory: where the gate loads of an operator without gates point, so
+// that the loaded value needs no select (a select right behind a load makes the wave wait for it).
+__device__ float kZeroWord = 0.f;  // never written; not const, so that it lives in the global address space like the tensors
+
 template <typename X>
 struct Load;
 template <>

@@ -155,9 +155,6 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   }
 }
 
-// a word of zeros in device memory: the target of gate loads when an operator has no gates
-__device__ const float kZeroWord = 0.f;
-
 // ---------------------------------------------------------------------------
 struct DhuParams {
   const void* q;

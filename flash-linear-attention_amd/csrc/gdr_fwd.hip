@@ -21,10 +21,16 @@
 //                       (fla/ops/common/chunk_o.py:68-101).  The scalar gate is
 //                       applied to the fp32 scores / accumulators, so every
 //                       exponent is <= 0 whatever the gate magnitude.
+#include <type_traits>
+
 #include "fla_common.h"
 #include "mfma_tiles.h"
 
 namespace {
+
+// A word of zeros in device memory: where the gate loads of a call without gates point, so that
+// the loaded value needs no select (a select right behind a load makes the wave wait for it).
+__device__ float kZeroWord = 0.f;  // never written; not const, so that it lives in the global address space like the tensors
 
 constexpr int BT = 64;
 constexpr int LDT = BT + 8;  // pitch of time-contiguous 16-bit tiles
@@ -392,7 +398,8 @@ struct DHParams {
 // One workgroup: all K rows x 32 value columns of one (sequence, head) state.
 // Wave w keeps the 32x32 state tiles kt = w, w+4, ... in MFMA accumulators.
 // HL: 0 row-major [K,V] in T, 1 fragment order in T, 2 row-major fp32.
-template <typename T, int K, int HL>
+// VN: v_new is written (its store is unconditional, so the choice is made at compile time).
+template <typename T, int K, int HL, bool VN>
 __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
@@ -440,78 +447,74 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
     }
   }
 
-  // prefetch registers: w, k as (RPT rows x 4 cols), u as (4 rows x 2 cols), gamma per row
+  // Prefetch registers.  Two independent sets, each refilled right after the staging step that
+  // consumed it, one full iteration before its next use, so that no register copy and no wait
+  // sits between issuing a load and the end of the iteration:
+  //   WU: w as (RPT rows x 4 cols), u as (4 rows x 2 cols), gamma per row  -> sW, sUt
+  //   KR: k as (RPT rows x 4 cols), gamma of the chunk's last row          -> sKt
   const int rg = tid / CG, c4 = (tid % CG) * 4;
   const int urg = tid >> 4, uc2 = (tid & 15) * 2;
-  struct Regs {
+  struct WURegs {
     v4 w[RPT];
-    v4 k[RPT];
     float gam[RPT];
     t2 u[4];
+  };
+  struct KRegs {
+    v4 k[RPT];
     float glast;
   };
   auto chunk_len = [&](int64_t c) {
     int64_t rem = sp.len - c * BT;
     return (int)(rem < BT ? rem : BT);
   };
-  // Addressing: a wave-uniform 64-bit base per chunk plus 32-bit per-lane element offsets that
-  // are computed once, so a load costs no per-lane 64-bit arithmetic.  Rows past the end of a
-  // short (last) chunk are redirected to its last row and zeroed afterwards.
-  const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
+  // Addressing: a wave-uniform 64-bit base per chunk plus 32-bit per-lane byte offsets that are
+  // computed once.  Every load is unconditional: rows past the end of a short (last) chunk are
+  // redirected to its last row (one unsigned minimum) and masked where they are used.
+  const uint32_t pitchK = (uint32_t)H * K * sizeof(T), pitchV = (uint32_t)H * V * sizeof(T), pitchG = (uint32_t)H * 4;
   uint32_t offk[RPT], offg[RPT], offu[4];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    offk[i] = (uint32_t)(rg * RPT + i) * HK + c4;
-    offg[i] = (uint32_t)(rg * RPT + i) * H;
+    offk[i] = (uint32_t)(rg * RPT + i) * pitchK + c4 * sizeof(T);
+    offg[i] = p.gam ? (uint32_t)(rg * RPT + i) * pitchG : 0u;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) offu[i] = (uint32_t)(urg * 4 + i) * HV + uc2;
-  auto load_chunk = [&](int64_t c, Regs& R) {
-    if (c >= nchunks) return;  // wave-uniform
-    const int L = chunk_len(c);
-    const int64_t rbase = (sp.bos + c * BT) * H + hh;
-    const T* wb = (const T*)p.w + rbase * K;
-    const T* kb = (const T*)p.k + rbase * K;
-    const T* ub = (const T*)p.u + rbase * V + vbase;
-    const float* gb = p.gam ? p.gam + rbase : nullptr;
-    if (L == BT) {
+  for (int i = 0; i < 4; ++i) offu[i] = (uint32_t)(urg * 4 + i) * pitchV + uc2 * sizeof(T);
+  const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * sizeof(T);
+  const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * sizeof(T);
+  const char* gu = (const char*)p.u + ((sp.bos * H + hh) * (int64_t)V + vbase) * sizeof(T);
+  const char* gg = p.gam ? (const char*)(p.gam + sp.bos * H + hh) : (const char*)&kZeroWord;
+  const int64_t stepG = p.gam ? (int64_t)BT * pitchG : 0;
+  auto load_wu = [&](int64_t c, WURegs& R) {
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const uint32_t limk = last * pitchK + c4 * sizeof(T), limu = last * pitchV + uc2 * sizeof(T);
+    const uint32_t limg = p.gam ? last * pitchG : 0u;
+    const char* wb = gw + c * (int64_t)BT * pitchK;
+    const char* ub = gu + c * (int64_t)BT * pitchV;
+    const char* gb = gg + c * stepG;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        R.w[i] = *(const v4*)(wb + offk[i]);
-        R.k[i] = *(const v4*)(kb + offk[i]);
-        R.gam[i] = gb ? gb[offg[i]] : 0.f;
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) R.u[i] = *(const t2*)(ub + offu[i]);
-      R.glast = gb ? gb[(uint32_t)(BT - 1) * H] : 0.f;
-    } else {
-#pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        int row = rg * RPT + i;
-        bool ok = row < L;
-        uint32_t rr = (uint32_t)(ok ? row : L - 1);
-        v4 wv = *(const v4*)(wb + rr * HK + c4);
-        v4 kv = *(const v4*)(kb + rr * HK + c4);
-        float gv = gb ? gb[rr * H] : 0.f;
-        R.w[i] = ok ? wv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.k[i] = ok ? kv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        R.gam[i] = ok ? gv : 0.f;
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int row = urg * 4 + i;
-        bool ok = row < L;
-        t2 uv = *(const t2*)(ub + (uint32_t)(ok ? row : L - 1) * HV + uc2);
-        R.u[i] = ok ? uv : t2{(T)0.f, (T)0.f};
-      }
-      R.glast = gb ? gb[(uint32_t)(L - 1) * H] : 0.f;
+    for (int i = 0; i < RPT; ++i) {
+      R.w[i] = *(const v4*)(wb + (offk[i] < limk ? offk[i] : limk));
+      R.gam[i] = *(const float*)(gb + (offg[i] < limg ? offg[i] : limg));
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) R.u[i] = *(const t2*)(ub + (offu[i] < limu ? offu[i] : limu));
   };
-  // state-independent operand tiles of one chunk
-  auto stage_wu = [&](const Regs& R) {
+  auto load_k = [&](int64_t c, KRegs& R) {
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const uint32_t limk = last * pitchK + c4 * sizeof(T);
+    const char* kb = gk + c * (int64_t)BT * pitchK;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(kb + (offk[i] < limk ? offk[i] : limk));
+    R.glast = *(const float*)(gg + c * stepG + (p.gam ? last * pitchG : 0u));
+  };
+  // state-independent operand tiles of one chunk; the gates of its rows stay in registers for
+  // the key tile of the same chunk, which is staged half an iteration later
+  float grow[RPT];
+  auto stage_wu = [&](const WURegs& R) {
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       int row = rg * RPT + i;
+      grow[i] = R.gam[i];
       float eg = __expf(R.gam[i]);
       v4 wv;
 #pragma unroll
@@ -524,15 +527,18 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
       *(v4*)&sUt[(uc2 + j) * LDT + urg * 4] = uv;
     }
   };
-  auto stage_k = [&](const Regs& R, int L) {
+  // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
+  auto stage_k = [&](const KRegs& R, int L) {
+    typedef T rvec __attribute__((ext_vector_type(RPT)));
+    float e[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) e[i] = (rg * RPT + i) < L ? __expf(R.glast - grow[i]) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      T* dst = &sKt[(c4 + j) * LDT + rg * RPT];
+      rvec x;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        bool valid = (rg * RPT + i) < L;
-        dst[i] = (T)(valid ? (float)R.k[i][j] * __expf(R.glast - R.gam[i]) : 0.f);
-      }
+      for (int i = 0; i < RPT; ++i) x[i] = (T)((float)R.k[i][j] * e[i]);
+      *(rvec*)&sKt[(c4 + j) * LDT + rg * RPT] = x;
     }
   };
   // state entering chunk c: 16-bit transpose in LDS for the MFMA, global copy for the output kernel
@@ -588,19 +594,13 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
 
   // Two barriers per chunk and single-buffered tiles:
   //   phase A (after barrier 1): v_new from sW, sUt, sHt;  stage sKt of the same chunk
-  //   phase B (after barrier 2): state update from sKt, sVnT;  stage sW, sUt, sHt of the next chunk
-  // Rc holds the chunk whose tiles are staged next, Rn the one after; loads run a full
-  // iteration ahead of their use.
-  Regs Rc, Rn;
-  if (nchunks > 0) {
-    load_chunk(0, Rc);
-    load_chunk(1, Rn);
-    stage_wu(Rc);
-    publish_h(0);
-  }
-  for (int64_t c = 0; c < nchunks; ++c) {
+  //   phase B (after barrier 2): state update from sKt, sVnT;  v_new leaves as 16-byte row pieces;
+  //                              stage sW, sUt, sHt of the next chunk
+  WURegs WU;
+  KRegs KR;
+  const int st = tid >> 2, sp8 = (tid & 3) * 8;  // v_new store: time row, first of 8 value columns
+  auto step = [&](int64_t c, auto more) {
     const int L = chunk_len(c);
-    const int64_t rbase = sp.bos + c * BT;
     lds_barrier();  // (1)
     // ---- v_new = u - (w e^gamma) h : wave w owns rows 16w..16w+15, two 16-column tiles
     {
@@ -620,17 +620,11 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) vn[r] = (T)((float)uu[r] - d[j][r]);
         *(v4*)&sVnT[vc * LDT + tr] = vn;
-        if (p.v_new) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (tr + r < L) ((T*)p.v_new)[((rbase + tr + r) * H + hh) * (int64_t)V + vbase + vc] = vn[r];
-        }
       }
     }
-    stage_k(Rc, L);
-    const float dec = __expf(Rc.glast);
-    Rc = Rn;
-    load_chunk(c + 2, Rn);
+    stage_k(KR, L);
+    const float dec = __expf(KR.glast);
+    if constexpr (decltype(more)::value) load_k(c + 1, KR);
     lds_barrier();  // (2)
     // ---- h <- e^{gamma_last} h + (k e^{gamma_last-gamma})^T v_new
 #pragma unroll
@@ -652,10 +646,32 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
         }
       }
     }
-    if (c + 1 < nchunks) {
-      stage_wu(Rc);
-      publish_h(c + 1);
+    if constexpr (VN) {
+      // rows past the end of a short chunk repeat its last row (same address, same data), so the
+      // store is unconditional and the waits for the loads in flight stay exact
+      const int sr = st < L ? st : L - 1;
+      v8 x;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) x[j] = sVnT[(sp8 + j) * LDT + sr];
+      *(v8*)((T*)p.v_new + ((sp.bos + c * BT + sr) * H + hh) * (int64_t)V + vbase + sp8) = x;
     }
+    if constexpr (decltype(more)::value) {
+      stage_wu(WU);
+      publish_h(c + 1);
+      load_wu(c + 2 < nchunks ? c + 2 : nchunks - 1, WU);
+      // keeps the loads here, at the end of the iteration: without it they are merged with the
+      // prologue's copy at the top of the loop and start half an iteration later
+      asm volatile("" ::: "memory");
+    }
+  };
+  if (nchunks > 0) {
+    load_wu(0, WU);
+    stage_wu(WU);
+    publish_h(0);
+    load_wu(nchunks > 1 ? 1 : 0, WU);
+    load_k(0, KR);
+    for (int64_t c = 0; c + 1 < nchunks; ++c) step(c, std::true_type{});
+    step(nchunks - 1, std::false_type{});
   }
   if (p.ht) {
     float* htp = p.ht + (int64_t)nh * K * V;
@@ -838,7 +854,8 @@ int launch_dh(const DHParams& p, int K, int h_dtype, int h_layout, hipStream_t s
   int hl = (h_layout == FLA_H_FRAGMENT) ? 1 : (h_layout == FLA_H_FRAGMENT_T) ? 3 : (h_dtype == FLA_F32 ? 2 : 0);
 #define FLA_CASE(KK, HL)                                                           \
   if (K == KK && hl == HL) {                                                       \
-    hipLaunchKernelGGL((gdr_fwd_h_kernel<T, KK, HL>), grid, block, 0, st, p);      \
+    if (p.v_new) hipLaunchKernelGGL((gdr_fwd_h_kernel<T, KK, HL, true>), grid, block, 0, st, p);   \
+    else hipLaunchKernelGGL((gdr_fwd_h_kernel<T, KK, HL, false>), grid, block, 0, st, p);          \
     FLA_CHECK_LAUNCH();                                                            \
     return FLA_OK;                                                                 \
   }
