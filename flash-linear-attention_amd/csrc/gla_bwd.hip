@@ -18,6 +18,8 @@
 //                        (fla/ops/gla/chunk.py:409-567 intra, :726-837 inter incl. the dg formula
 //                        :818-823).  As in the forward, one reference point per chunk replaces
 //                        the 16x16 sub-block scheme.
+#include <type_traits>
+
 #include "chunk_common.h"
 
 namespace {
@@ -87,39 +89,40 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
     t2 d[8];
     v8 h[2];
   };
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+  // Every load is unconditional: rows past the end of a short (last) chunk are redirected to its
+  // last row (one unsigned minimum on a byte offset) and masked where they are used.
+  const uint32_t pitchK = (uint32_t)kstride * sizeof(T), pitchG = (uint32_t)kstride * sizeof(GT);
+  const uint32_t pitchV = (uint32_t)vstride * sizeof(T);
   auto load_chunk = [&](int64_t c, Regs& R) {
-    bool live = c >= 0;
-    int64_t t0 = c * BT;
-    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const uint32_t limk = last * pitchK, limg = last * pitchG, limv = last * pitchV;
+    const char* qb = (const char*)(qp + c * BT * kstride);
+    const char* gb = (const char*)(gp + c * BT * kstride);
+    const char* db = (const char*)(dp + c * BT * vstride);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      int row = rg * 8 + i;
-      if (live && row < L) {
-        R.g[i] = *(const g2*)(gp + (t0 + row) * kstride);
-        R.q[i] = *(const t2*)(qp + (t0 + row) * kstride);
-        R.d[i] = *(const t2*)(dp + (t0 + row) * vstride);
-      } else {
-        R.g[i] = g2{(GT)0.f, (GT)0.f};
-        R.q[i] = t2{(T)0.f, (T)0.f};
-        R.d[i] = t2{(T)0.f, (T)0.f};
-      }
+      const uint32_t row = (uint32_t)(rg * 8 + i);
+      uint32_t ok = row * pitchK, og = row * pitchG, ov = row * pitchV;
+      R.g[i] = *(const g2*)(gb + (og < limg ? og : limg));
+      R.q[i] = *(const t2*)(qb + (ok < limk ? ok : limk));
+      R.d[i] = *(const t2*)(db + (ov < limv ? ov : limv));
     }
-    if (live) {
-      const T* hp = (const T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V +
-                    (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
-      R.h[0] = *(const v8*)hp;
-      R.h[1] = *(const v8*)(hp + 8);
-    }
+    const T* hp = (const T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V +
+                  (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
+    R.h[0] = *(const v8*)hp;
+    R.h[1] = *(const v8*)(hp + 8);
   };
 
-  Regs R0, R1, R2;
-  load_chunk(nchunks - 1, R0);
-  load_chunk(nchunks - 2, R1);
-  for (int64_t c = nchunks - 1; c >= 0; --c) {
+  // One barrier per chunk, operand tiles double-buffered in LDS.  Two register sets, each
+  // refilled right after the staging step that consumed it: a chunk is in flight for almost two
+  // iterations and no register copy sits between a load and its use.
+  auto step = [&](int64_t c, Regs& R, auto more) {
     const int buf = (int)(c & 1);
-    int64_t t0 = c * BT;
-    int L = (int)((sp.len - t0) < BT ? (sp.len - t0) : BT);
-    load_chunk(c - 2, R2);
+    const int L = chunk_len(c);
     // ---- gradient w.r.t. the state leaving chunk c, both orientations, fragment order
     {
       int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
@@ -143,7 +146,7 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       // sum over this wave's 32 value columns of h_c * dH_c, one key channel per lane
       float part = 0.f;
 #pragma unroll
-      for (int r = 0; r < 8; ++r) part += (float)R0.h[0][r] * acc2[r] + (float)R0.h[1][r] * acc2[r + 8];
+      for (int r = 0; r < 8; ++r) part += (float)R.h[0][r] * acc2[r] + (float)R.h[1][r] * acc2[r + 8];
       part += __shfl_xor(part, 32, 64);
       if (lane < 32) p.hdh[(((int64_t)vt32 * p.total_chunks + chunk0 + c) * H + hh) * K + kcol] = part;
     }
@@ -153,8 +156,9 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       float r0 = 0.f, r1 = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        r0 += (float)R0.g[i][0];
-        r1 += (float)R0.g[i][1];
+        bool valid = (rg * 8 + i) < L;
+        r0 += valid ? (float)R.g[i][0] : 0.f;
+        r1 += valid ? (float)R.g[i][1] : 0.f;
         G[i][0] = r0;
         G[i][1] = r1;
       }
@@ -181,16 +185,20 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         bool valid = (rg * 8 + i) < L;
-        qa[i] = (T)(valid ? (float)R0.q[i][0] * p.scale * __expf(G[i][0]) : 0.f);
-        qb[i] = (T)(valid ? (float)R0.q[i][1] * p.scale * __expf(G[i][1]) : 0.f);
-        da[i] = R0.d[i][0];
-        db[i] = R0.d[i][1];
+        qa[i] = (T)(valid ? (float)R.q[i][0] * p.scale * __expf(G[i][0]) : 0.f);
+        qb[i] = (T)(valid ? (float)R.q[i][1] * p.scale * __expf(G[i][1]) : 0.f);
+        da[i] = R.d[i][0];
+        db[i] = R.d[i][1];
       }
       *(v8*)&sQt[buf][(c2 + 0) * LDT + rg * 8] = qa;
       *(v8*)&sQt[buf][(c2 + 1) * LDT + rg * 8] = qb;
       *(v8*)&sDt[buf][(c2 + 0) * LDT + rg * 8] = da;
       *(v8*)&sDt[buf][(c2 + 1) * LDT + rg * 8] = db;
       if (rg == 0) *(f32x2*)&sDecay[buf][c2] = f32x2{__expf(glast0), __expf(glast1)};
+    }
+    if constexpr (decltype(more)::value) {
+      load_chunk(c >= 2 ? c - 2 : 0, R);
+      asm volatile("" ::: "memory");  // the loads stay here, ahead of the barrier
     }
     lds_barrier();
 #pragma unroll
@@ -211,8 +219,27 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       acc1 = Elem<T>::mfma32(fq, fd, acc1);
       acc2 = Elem<T>::mfma32(fd, fq, acc2);
     }
-    R0 = R1;
-    R1 = R2;
+  };
+  Regs R0, R1;
+  if (nchunks > 0) {
+    load_chunk(nchunks - 1, R0);
+    asm volatile("" ::: "memory");  // the two sets are issued one after the other, as in the loop:
+    load_chunk(nchunks > 1 ? nchunks - 2 : 0, R1);  // interleaved, the loop's first wait would cover both
+    asm volatile("" ::: "memory");
+    int64_t c = nchunks - 1;
+    for (; c >= 3; c -= 2) {
+      step(c, R0, std::true_type{});
+      step(c - 1, R1, std::true_type{});
+    }
+    // the last one to three chunks: nothing is left to prefetch for the final two
+    if (c == 2) {
+      step(2, R0, std::true_type{});
+      step(1, R1, std::false_type{});
+      step(0, R0, std::false_type{});
+    } else {
+      step(c, R0, std::false_type{});
+      if (c == 1) step(0, R1, std::false_type{});
+    }
   }
   if (p.dh0) {
     float* o = p.dh0 + (int64_t)nh * K * V;
