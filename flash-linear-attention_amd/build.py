@@ -26,6 +26,11 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# Keeps MFMA accumulators in ordinary vector registers: elementwise work on them (decay, scaling,
+# conversion for stores) then needs no copies out of and back into the accumulation registers.
+# Only where it measured faster (gdr_bwd_dhu 216 -> 204 us); the forward state scans lose with it.
+VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+VGPR_FORM_SOURCES = {"gdr_bwd.hip"}
 
 
 def sources():
@@ -44,7 +49,7 @@ def _compile(src, force):
     if (not force and os.path.exists(obj)
             and os.path.getmtime(obj) >= max(os.path.getmtime(path), _newest_header())):
         return obj, ""
-    cmd = [HIPCC] + FLAGS + ["-c", path, "-o", obj]
+    cmd = [HIPCC] + FLAGS + (VGPR_FORM if src in VGPR_FORM_SOURCES else []) + ["-c", path, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
                     if "not a recognized feature" not in l)

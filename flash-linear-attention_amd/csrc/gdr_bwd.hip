@@ -189,8 +189,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   constexpr int KT32 = K / 32;
   constexpr int NKT = (KT32 + 3) / 4;
   __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];    // k e^{gamma_last-gamma}, row-major
-  __shared__ __attribute__((aligned(16))) T sQt[K * LDT];     // (s q e^gamma)^T
-  __shared__ __attribute__((aligned(16))) T sWt[K * LDT];     // -(w e^gamma)^T
+  __shared__ __attribute__((aligned(16))) T sQt[K * LDT];     // (s q e^gamma)^T, swz16
+  __shared__ __attribute__((aligned(16))) T sWt[K * LDT];     // -(w e^gamma)^T, swz16
   __shared__ __attribute__((aligned(16))) T sDoT[BV * LDT];   // do^T
   __shared__ __attribute__((aligned(16))) T sDvl[BV * LDT];   // dv_loc^T
   __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];   // dH^T in 16-bit
@@ -315,8 +315,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
         xq[i] = (T)((float)R.q[i][j] * p.scale * eg[i]);
         xw[i] = (T)(-(float)R.w[i][j] * eg[i]);
       }
-      *(rvec*)&sQt[(c4 + j) * LDT + rg * RPT] = xq;
-      *(rvec*)&sWt[(c4 + j) * LDT + rg * RPT] = xw;
+      *(rvec*)&sQt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = xq;
+      *(rvec*)&sWt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = xw;
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -434,9 +434,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
         }
 #pragma unroll
         for (int s = 0; s < BT; s += 16) {
-          v8 fq = lds_frag32<T>(sQt, LDT, kt * 32, s, lane);
+          v8 fq = lds_frag32_swz<T>(sQt, LDT, kt * 32, s, lane);
           v8 fd = lds_frag32<T>(sDoT, LDT, 0, s, lane);
-          v8 fw = lds_frag32<T>(sWt, LDT, kt * 32, s, lane);
+          v8 fw = lds_frag32_swz<T>(sWt, LDT, kt * 32, s, lane);
           v8 f2 = lds_frag32<T>(sDv2T, LDT, 0, s, lane);
           acc[a] = Elem<T>::mfma32(fq, fd, acc[a]);
           acc[a] = Elem<T>::mfma32(fw, f2, acc[a]);

@@ -410,7 +410,7 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   constexpr int KT32 = K / 32;
   constexpr int NKT = (KT32 + 3) / 4;  // state tiles per wave
   __shared__ __attribute__((aligned(16))) T sW[BT * LDK];    // w e^gamma, row-major
-  __shared__ __attribute__((aligned(16))) T sKt[K * LDT];    // (k e^{gamma_last-gamma})^T
+  __shared__ __attribute__((aligned(16))) T sKt[K * LDT];    // (k e^{gamma_last-gamma})^T, swz16
   __shared__ __attribute__((aligned(16))) T sUt[BV * LDT];   // u^T
   __shared__ __attribute__((aligned(16))) T sHt[BV * LDK];   // h^T in 16-bit
   __shared__ __attribute__((aligned(16))) T sVnT[BV * LDT];  // v_new^T
@@ -538,7 +538,7 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
       rvec x;
 #pragma unroll
       for (int i = 0; i < RPT; ++i) x[i] = (T)((float)R.k[i][j] * e[i]);
-      *(rvec*)&sKt[(c4 + j) * LDT + rg * RPT] = x;
+      *(rvec*)&sKt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = x;
     }
   };
   // state entering chunk c: 16-bit transpose in LDS for the MFMA, global copy for the output kernel
@@ -639,7 +639,7 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
         }
 #pragma unroll
         for (int s = 0; s < BT; s += 16) {
-          v8 fk = lds_frag32<T>(sKt, LDT, kt * 32, s, lane);
+          v8 fk = lds_frag32_swz<T>(sKt, LDT, kt * 32, s, lane);
           v8 fv = lds_frag32<T>(sVnT, LDT, 0, s, lane);
           acc[a] = Elem<T>::mfma32(fk, fv, acc[a]);
           if (TR) acct[a] = Elem<T>::mfma32(fv, fk, acct[a]);

@@ -10,6 +10,18 @@ FLA_DEVICE typename Elem<T>::v8 lds_frag32(const T* tile, int ld, int row0, int 
   return *(const typename Elem<T>::v8*)(tile + (row0 + (lane & 31)) * ld + k0 + 8 * (lane >> 5));
 }
 
+// Time-contiguous 16-bit tiles ([row][t], pitch 144 bytes) that are written by lanes owning four
+// adjacent rows each see a lane stride of 64 bytes modulo 256, i.e. a quarter of the banks.
+// XOR-ing row bits 4-5 into the index of the 16-byte slot along t spreads such writes over all
+// banks; a fragment read stays conflict-free.  Writer and reader both map t through swz16.
+FLA_DEVICE int swz16(int row, int t) { return t ^ (((row >> 4) & 3) << 3); }
+
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 lds_frag32_swz(const T* tile, int ld, int row0, int k0, int lane) {
+  const int row = row0 + (lane & 31);
+  return *(const typename Elem<T>::v8*)(tile + row * ld + swz16(row, k0 + 8 * (lane >> 5)));
+}
+
 // Same slice with the contraction index permuted inside the 16-slice: slot
 // (g = lane/32, e) holds k0 + 8*(e/4) + 4*g + e%4.  This is the order in which
 // a 32x32 accumulator's registers enumerate rows, so an accumulator converted
