@@ -303,20 +303,25 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   float egx[RPT];
   auto stage_x = [&](const XRegs& R) {
     // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
-    typedef T rvec __attribute__((ext_vector_type(RPT)));
+    // (in pieces of at most one 16-byte slot, the unit the swizzle permutes)
+    constexpr int PW = RPT < 8 ? RPT : 8;
+    typedef T rvec __attribute__((ext_vector_type(PW)));
     float eg[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; ++i) eg[i] = egx[i];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      rvec xq, xw;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        xq[i] = (T)((float)R.q[i][j] * p.scale * eg[i]);
-        xw[i] = (T)(-(float)R.w[i][j] * eg[i]);
+      for (int i0 = 0; i0 < RPT; i0 += PW) {
+        rvec xq, xw;
+#pragma unroll
+        for (int i = 0; i < PW; ++i) {
+          xq[i] = (T)((float)R.q[i0 + i][j] * p.scale * eg[i0 + i]);
+          xw[i] = (T)(-(float)R.w[i0 + i][j] * eg[i0 + i]);
+        }
+        *(rvec*)&sQt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT + i0)] = xq;
+        *(rvec*)&sWt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT + i0)] = xw;
       }
-      *(rvec*)&sQt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = xq;
-      *(rvec*)&sWt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = xw;
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -1076,6 +1081,8 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   else if (K == 128 && V == 128) { STMT(128, 128) }    \
   else if (K == 64 && V == 128) { STMT(64, 128) }      \
   else if (K == 128 && V == 64) { STMT(128, 64) }      \
+  else if (K == 256 && V == 64) { STMT(256, 64) }      \
+  else if (K == 256 && V == 128) { STMT(256, 128) }    \
   else return FLA_E_UNSUPPORTED;
   {
     DvlParams p{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
@@ -1089,6 +1096,7 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
     int64_t total = (V / 32) * N * H;
     FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
     if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(256), 0, st, p);
+    else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(256), 0, st, p);
     else hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(256), 0, st, p);
     FLA_CHECK_LAUNCH();
   }
@@ -1124,7 +1132,7 @@ extern "C" int fla_chunk_gated_delta_rule_bwd(
                   ws_dw && ws_dk_partial && ws_dgam_partial && dq && dk && dv && dbeta && dgam2,
               FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE((K == 64 || K == 128 || K == 256) && (V == 64 || V == 128), FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
   hipStream_t st = (hipStream_t)stream;

@@ -529,16 +529,21 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
   };
   // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
   auto stage_k = [&](const KRegs& R, int L) {
-    typedef T rvec __attribute__((ext_vector_type(RPT)));
+    // (in pieces of at most one 16-byte slot, the unit the swizzle permutes)
+    constexpr int PW = RPT < 8 ? RPT : 8;
+    typedef T rvec __attribute__((ext_vector_type(PW)));
     float e[RPT];
 #pragma unroll
     for (int i = 0; i < RPT; ++i) e[i] = (rg * RPT + i) < L ? __expf(R.glast - grow[i]) : 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      rvec x;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) x[i] = (T)((float)R.k[i][j] * e[i]);
-      *(rvec*)&sKt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT)] = x;
+      for (int i0 = 0; i0 < RPT; i0 += PW) {
+        rvec x;
+#pragma unroll
+        for (int i = 0; i < PW; ++i) x[i] = (T)((float)R.k[i0 + i][j] * e[i0 + i]);
+        *(rvec*)&sKt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT + i0)] = x;
+      }
     }
   };
   // state entering chunk c: 16-bit transpose in LDS for the MFMA, global copy for the output kernel
@@ -841,6 +846,8 @@ int launch_wy(const WyParams& p, int K, int V, dim3 grid, hipStream_t st) {
   FLA_CASE(128, 128)
   FLA_CASE(64, 128)
   FLA_CASE(128, 64)
+  FLA_CASE(256, 64)
+  FLA_CASE(256, 128)
 #undef FLA_CASE
   return FLA_E_UNSUPPORTED;
 }
@@ -861,6 +868,7 @@ int launch_dh(const DHParams& p, int K, int h_dtype, int h_layout, hipStream_t s
   }
   FLA_CASE(64, 0) FLA_CASE(64, 1) FLA_CASE(64, 2) FLA_CASE(64, 3)
   FLA_CASE(128, 0) FLA_CASE(128, 1) FLA_CASE(128, 2) FLA_CASE(128, 3)
+  FLA_CASE(256, 0) FLA_CASE(256, 1) FLA_CASE(256, 2) FLA_CASE(256, 3)
 #undef FLA_CASE
   return FLA_E_UNSUPPORTED;
 }
@@ -877,6 +885,8 @@ int launch_do(const DOParams& p, int K, int V, dim3 grid, hipStream_t st) {
   FLA_CASE(128, 128)
   FLA_CASE(64, 128)
   FLA_CASE(128, 64)
+  FLA_CASE(256, 64)
+  FLA_CASE(256, 128)
 #undef FLA_CASE
   return FLA_E_UNSUPPORTED;
 }

@@ -22,11 +22,17 @@ from ..utils.cumsum import chunk_local_cumsum
 from .wy_fast import fwd_prepare_wy_repr
 
 BT = 64
-_SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
+_SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64), (256, 64), (256, 128)}
+_FUSED_MAX_K = 128  # the one-pass forward kernel holds at most 128 key channels of the state
 
 
 def _round64(d: int) -> int:
     return -(-d // 64) * 64
+
+
+def _round_k(d: int) -> int:
+    """Key head dims run on tiles of 64, 128 or 256 channels (zero padding is exact)."""
+    return 64 if d <= 64 else 128 if d <= 128 else 256 if d <= 256 else _round64(d)
 
 
 def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
@@ -115,7 +121,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             beta = beta.transpose(1, 2).contiguous()
             g = None if g is None else g.transpose(1, 2).contiguous()
         K, V = q.shape[-1], v.shape[-1]
-        KP, VP = _round64(K), _round64(V)
+        KP, VP = _round_k(K), _round64(V)
         if (KP, VP) not in _SUPPORTED_KV:
             raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: head dims K={K}, V={V} are outside the built "
                                       f"tiles {sorted(_SUPPORTED_KV)} (after rounding up to multiples of 64)")
@@ -126,7 +132,8 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
         gc, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
-                                                     offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+                                                     offsets=offsets, head_first=False, chunk_size=BT, store_A=False,
+                                                     fused=KP <= _FUSED_MAX_K)
         ctx.save_for_backward(q, k, v, gc, beta, h0, offsets)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
@@ -202,24 +209,9 @@ def chunk_gated_delta_rule(
     else:
         assert scale > 0, "Scale must be positive."
     K, V = k.shape[-1], v.shape[-1]
-    if 128 < K <= 256:
-        # The chunk kernels hold at most 128 key channels of the state (the delta rule couples all of
-        # them, so there are no independent slabs).  Without gradients the token-by-token kernel
-        # computes the same operator for up to 256 channels: slower (serial in time), not approximate.
-        if torch.is_grad_enabled() and any(t is not None and t.requires_grad
-                                           for t in (q, k, v, g, beta, initial_state)):
-            raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: the backward needs the chunk kernels, which "
-                                      f"cover key head dims up to 128 (got {K})")
-        from .fused_recurrent import fused_recurrent_gated_delta_rule
-        if not getattr(chunk_gated_delta_rule, "_warned_wide_k", False):
-            warnings.warn(f"fla_amd chunk_gated_delta_rule: key head dim {K} > 128 runs on the token-by-token "
-                          f"kernel (forward only)", stacklevel=2)
-            chunk_gated_delta_rule._warned_wide_k = True
-        if g is None:
-            g = torch.zeros_like(beta, dtype=torch.float32)
-        return fused_recurrent_gated_delta_rule(q, k, v, g, beta, scale=scale, initial_state=initial_state,
-                                                output_final_state=output_final_state, offsets=offsets,
-                                                head_first=head_first)
+    if K > 256:
+        raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: key head dims up to 256 are covered (got {K}), "
+                                  f"as in the reference (fla/ops/common/chunk_delta_h.py:272)")
     if V > 128:
         # the delta rule is independent per value column: wider heads run as slabs of 128 columns
         # (autograd sums the slabs' gradients of q, k, g and beta)

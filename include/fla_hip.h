@@ -170,7 +170,7 @@ int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const v
  * Chunked gated delta rule forward (chunk size 64).  g_cumsum is the fp32
  * chunk-local prefix sum of the per-head log-gate [B,T,H] (from
  * fla_chunk_local_cumsum), or NULL for the un-gated delta rule; beta is fp32
- * [B,T,H].
+ * [B,T,H].  K in {64,128,256}, V in {64,128} for the three entry points below.
  *
  * fla_gdr_fwd_wy: WY representation, replaces fwd_prepare_wy_repr +
  * fwd_recompute_w_u (fla/ops/gated_delta_rule/wy_fast.py:320-376 kernel
@@ -264,6 +264,7 @@ int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* g
  * Outputs: dq, dk [B,T,H,K], dv [B,T,H,V] (q/k/v dtype); dbeta and dgam2 fp32
  * [B,T,H]; dh0 fp32 [N,H,K,V] or NULL.  The gradient w.r.t. the raw gate is the
  * reverse chunk-local cumsum of (sum over slices of ws_dgam_partial) + dgam2.
+ * K in {64,128,256}, V in {64,128}.
  * ---------------------------------------------------------------------- */
 int fla_chunk_gated_delta_rule_bwd(
     const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,

@@ -203,3 +203,31 @@ def test_chunk_gdr_backward_varlen_and_headfirst(device):
     ref = _grads_ref(q, k, v, g, beta, None, do, dht)
     for name, r, x, tol in zip(NAMES[:5], ref, got, TOLS):
         assert_close(name, r, x, tol)
+
+
+# The reference's own ladder (tests/ops/test_gated_delta.py:220-294): head dims 50, 100, 200 (not
+# multiples of 64, 200 needing 256 key channels), both layouts, strong and weak decays.
+@pytest.mark.parametrize("D,T,scale,normalizer,head_first", [
+    (50, 63, 1.0, 1.0, False),
+    (100, 286, 0.1, 0.05, True),
+    (200, 7, 1.0, 1.0, True),
+    (200, 300, 0.1, 20.0, False),
+    (200, 1000, 1.0, 0.05, False),
+])
+def test_chunk_gdr_reference_ladder(device, D, T, scale, normalizer, head_first):
+    B, H = 2, 2
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, D, D, seed=71 + T, h0_std=1.0, normalizer=normalizer)
+    gen = torch.Generator().manual_seed(9)
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(B, H, D, D, generator=gen) * 0.1
+    print(f"chunk_gdr ladder D={D} T={T} scale={scale} normalizer={normalizer} head_first={head_first}", flush=True)
+    o, ht = _run(device, q, k, v, g, beta, h0, scale=scale, head_first=head_first)
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, scale=scale, initial_state=h0,
+                                               output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    got = _grads_dev(device, q, k, v, g, beta, h0, do, dht, scale=scale, head_first=head_first)
+    ref = _grads_ref(q, k, v, g, beta, h0, do, dht, scale=scale)
+    for name, r, x, tol in zip(NAMES, ref, got, TOLS):
+        assert_close(name, r, x, tol)

@@ -161,22 +161,44 @@ def test_chunk_gdr_wide_values(device):
     assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
 
 
-def test_chunk_gdr_wide_keys_forward_only(device):
-    """Key head dim 256 (the default of the reference's GatedDeltaNet layer): served without gradients
-    by the token-by-token kernel; with gradients the operator refuses loudly."""
-    import warnings
+@pytest.mark.parametrize("B,T,H,K,V,varlen", [
+    (2, 150, 2, 256, 128, False),
+    (1, 200, 2, 200, 200, False),   # the reference's own test dims: padded to 256 keys, two value slabs
+    (1, 300, 2, 256, 64, True),
+])
+def test_chunk_gdr_wide_keys(device, B, T, H, K, V, varlen):
+    """Key head dims up to 256 (the default of the reference's GatedDeltaNet layer), forward and
+    backward through the chunk kernels."""
     from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
     from oracle.recurrent import naive_recurrent_gated_delta_rule
-    B, T, H, K, V = 1, 200, 2, 256, 128
     q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=78, h0_std=1.0)
+    offsets = torch.tensor([0, 70, 71, 199, T]) if varlen else None
+    N = B if offsets is None else len(offsets) - 1
+    gen = torch.Generator().manual_seed(5)
+    h0 = torch.randn(N, H, K, V, generator=gen)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(N, H, K, V, generator=gen) * 0.1
     dev = _dev(device)
-    print("chunk_gated_delta_rule K=256 (forward only)", flush=True)
-    with torch.no_grad(), warnings.catch_warnings():
-        warnings.simplefilter("ignore")
-        o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), initial_state=dev(h0),
-                                       output_final_state=True, head_first=False)
-    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    print(f"chunk_gated_delta_rule K={K} V={V} varlen={varlen}", flush=True)
+    leaves = [dev(x).requires_grad_() for x in (q, k, v, g, beta)]
+    h0l = dev(h0).requires_grad_()
+    o, ht = chunk_gated_delta_rule(*leaves, initial_state=h0l, output_final_state=True, head_first=False,
+                                   offsets=None if offsets is None else dev(offsets))
+    ((o.float() * dev(do).float()).sum() + (ht * dev(dht)).sum()).backward()
+    refs = [x.float().requires_grad_() for x in (q, k, v, g, beta)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gated_delta_rule(*refs, initial_state=rh0, output_final_state=True, offsets=offsets)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
     assert_close("o", ro, o, 1e-2)
     assert_close("ht", rht, ht, 5e-3)
+    for name, a, b, tol in zip(("dq", "dk", "dv", "dg", "dbeta"), refs, leaves, (8e-3, 8e-3, 8e-3, 2e-2, 2e-2)):
+        assert_close(name, a.grad, b.grad, tol)
+    assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
+
+
+def test_chunk_gdr_keys_above_256_refused(device):
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    q, k, v, g, beta, _ = gdr_inputs(1, 64, 1, 320, 64, seed=3, h0_std=1.0)
+    dev = _dev(device)
     with pytest.raises(NotImplementedError):
-        chunk_gated_delta_rule(dev(q).requires_grad_(), dev(k), dev(v), dev(g), dev(beta), head_first=False)
+        chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), head_first=False)
