@@ -668,12 +668,23 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     v4 dqv, dkv;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float dq = p.scale * __expf(G[i][j]) * a[j];
-      float dki = __expf(glast[j] - G[i][j]) * c[j];
-      float dk = p.scale * einv[i][j] * b[j] + dki;
+      // (the gate factors go through an opaque copy: the rounded operands below are recomputed
+      // here instead of being kept in registers from the staging step to this point)
+      float gij = G[i][j], ei = einv[i][j];
+      asm volatile("" : "+v"(gij), "+v"(ei));
+      const float eg = __expf(gij);
+      float dq = p.scale * eg * a[j];
+      float dki = __expf(glast[j] - gij) * c[j];
+      float dk = p.scale * ei * b[j] + dki;
       dqv[j] = (T)dq;
       dkv[j] = (T)dk;
-      x[i][j] = qq[i][j] * dq - kk[i][j] * dk;
+      // dg sums q*dq - k*dk over later rows: an intra-chunk pair (i, j) enters q*dq at row i and
+      // k*dk at row j and cancels unless it straddles the row.  Formed with the rounded operands
+      // the matrix products used, the two copies are equal and cancel exactly; with strong gates,
+      // where dg is small against either sum, this is what keeps its error at rounding level.
+      const float qr = (float)(T)(qq[i][j] * eg);
+      const float kr = (float)(T)(kk[i][j] * ei);
+      x[i][j] = p.scale * (qr * a[j] - kr * b[j]) - kk[i][j] * dki;
       ksum[j] += kk[i][j] * dki;
     }
     if (row < L) {

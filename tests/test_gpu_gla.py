@@ -264,3 +264,38 @@ def test_chunk_gla_internal_fwd_bwd_signatures(device):
     ref = _grads_ref(q, k, v, g, h0, do, dht)
     for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), ref, (dq, dk, dv, dg, dh0), (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
         assert_close(name, r, x, tol)
+
+
+# The reference's own ladder (tests/ops/test_gla.py:90-146): head dims 300 and 100 (key and value
+# slabs of 128 after padding), both layouts, gate_logit_normalizer 1 / 0.05 / 20.
+@pytest.mark.parametrize("D,T,normalizer,head_first", [
+    (300, 130, 1.0, False),
+    (300, 178, 0.05, True),
+    (300, 300, 20.0, False),
+    (100, 146, 0.05, False),
+    (100, 2048, 20.0, True),
+])
+def test_chunk_gla_reference_ladder(device, D, T, normalizer, head_first):
+    from fla_amd.ops.gla import chunk_gla
+    from helpers import gla_inputs
+    from oracle.recurrent import naive_recurrent_gla
+    B, H = 2, 2
+    q, k, v, g, h0 = gla_inputs(B, T, H, D, D, seed=81 + T, normalizer=normalizer, h0_std=1.0)
+    gen = torch.Generator().manual_seed(11)
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(B, H, D, D, generator=gen) * 0.1
+    print(f"chunk_gla ladder D={D} T={T} normalizer={normalizer} head_first={head_first}", flush=True)
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    leaves = [tr(x.to(device)).detach().requires_grad_() for x in (q, k, v, g)]
+    h0l = h0.to(device).requires_grad_()
+    o, ht = chunk_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=head_first)
+    ((o.float() * tr(do.to(device)).float()).sum() + (ht * dht.to(device)).sum()).backward()
+    refs = [x.float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gla(*refs, initial_state=rh0, output_final_state=True)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, tr(o), 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), refs, leaves):
+        assert_close(name, a.grad, tr(b.grad), 1e-2)
+    assert_close("dh0", rh0.grad, h0l.grad, 1e-2)
