@@ -4,7 +4,7 @@ chunked linear-attention hot path (``chunk_gla``, ``chunk_gated_delta_rule``,
 ``from fla.ops.gla import chunk_gla`` for ``from fla_amd.ops.gla import chunk_gla``,
 or call :func:`install` to rebind the names inside an importable upstream ``fla``.
 """
-from . import modules, ops  # noqa: F401
+from . import models, modules, ops  # noqa: F401
 from ._backend import lib, lib_path  # noqa: F401
 
 __version__ = '0.1.0'
@@ -38,4 +38,6 @@ def install() -> list:
             if hasattr(mod, name):
                 setattr(mod, name, fn)
                 patched.append(f'{modname}.{name}')
+    # fla.models.utils.Cache is left alone: the upstream models subclass-check it against
+    # transformers' Cache; fla_amd.models.Cache is for callers that drive the operators directly
     return patched

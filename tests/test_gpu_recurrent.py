@@ -187,3 +187,45 @@ def test_fused_recurrent_scalar_gate_backward_and_guards(device):
     o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], gv=gv, head_first=False)
     with pytest.raises(NotImplementedError):
         o.sum().backward()
+
+
+# ---------------------------------------------------------------- prefill + decode through the Cache
+@pytest.mark.parametrize("op", ["gla", "gdr"])
+def test_cache_prefill_then_decode(device, op):
+    """A layer's call pattern (fla/layers/gla.py:232-263, gated_deltanet.py:241-275): chunk operator on the
+    prompt, state into the Cache, then single-token steps that read it back.  With in-place steps the
+    Cache holds one buffer from the first step to the last."""
+    from fla_amd.models import Cache
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
+    from fla_amd.ops.gla import chunk_gla, fused_recurrent_gla
+    from oracle.recurrent import naive_recurrent_gated_delta_rule, naive_recurrent_gla
+    B, H, D, Tp, steps = 2, 2, 128, 150, 6
+    T = Tp + steps
+    if op == "gla":
+        q, k, v, g, _ = gla_inputs(B, T, H, D, D, seed=91)
+        cpu = (q, k, v, g)
+        chunk, step_fn = chunk_gla, fused_recurrent_gla
+        ro, rht = naive_recurrent_gla(q, k, v, g, output_final_state=True)
+    else:
+        q, k, v, g, beta, _ = gdr_inputs(B, T, H, D, D, seed=91)
+        cpu = (q, k, v, g, beta)
+        chunk, step_fn = chunk_gated_delta_rule, fused_recurrent_gated_delta_rule
+        ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, output_final_state=True)
+    args = [x.to(device) for x in cpu]
+    print(f"cache prefill+decode {op}", flush=True)
+    cache = Cache()
+    o_p, ht = chunk(*[x[:, :Tp].contiguous() for x in args], initial_state=None, output_final_state=True,
+                    head_first=False)
+    cache.update(recurrent_state=ht, layer_idx=0, offset=Tp)
+    outs = [o_p]
+    ptr = cache[0]['recurrent_state'].data_ptr()
+    for t in range(Tp, T):
+        state = cache[0]['recurrent_state']
+        o_t, new_state = step_fn(*[x[:, t:t + 1].contiguous() for x in args], initial_state=state,
+                                 output_final_state=True, head_first=False, inplace_state=True)
+        cache.update(recurrent_state=new_state, layer_idx=0, offset=1)
+        outs.append(o_t)
+        assert cache[0]['recurrent_state'].data_ptr() == ptr
+    assert cache.get_seq_length() == T
+    assert_close("o", ro, torch.cat(outs, 1), 1e-2)
+    assert_close("ht", rht, cache[0]['recurrent_state'], 5e-3)
