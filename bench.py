@@ -28,6 +28,7 @@ for _p in (ROOT, os.path.join(ROOT, "flash-linear-attention_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+MFMA_PEAK_FLOPS = 2.5e15   # dense bf16 MFMA, FLOP/s
 HBM_PEAK_GBS = 8000.0
 MIB = 1 << 20
 
@@ -136,8 +137,10 @@ def bench_gla(device, steps, warmup):
     roofline = {"kernel": "gla_fwd_fused_kernel", "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "avg_us": round(us_f, 1), "bytes_per_launch": floor_bytes}
+    flops = B * T * H * (4 * K * V + 2 * 64 * K + 2 * 64 * V)   # dense-tile count of the chunked algorithm
     op = {"algorithmic_bytes": floor_bytes, "achieved_GBs": round(floor_bytes / (ms * 1e-3) / 1e9, 1),
           "frac_of_hbm_peak": round(floor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+          "algorithmic_flops": flops, "frac_of_mfma_peak": round(flops / (ms * 1e-3) / MFMA_PEAK_FLOPS, 4),
           "two_kernel_pipeline_us": {"gla_fwd_h_kernel": round(us_h, 1), "gla_fwd_o_kernel": round(us_o, 1)},
           "two_kernel_pipeline_GBs": {"gla_fwd_h_kernel": round(bytes_h / (us_h * 1e-6) / 1e9, 1),
                                       "gla_fwd_o_kernel": round(bytes_o / (us_o * 1e-6) / 1e9, 1)}}
@@ -203,13 +206,17 @@ def bench_gdr(device, steps=20):
     beta = torch.randn(1, T, H, device=device).sigmoid()
     # q, k, v, o in 16 bit + g, beta fp32 + the final states: what the operator must move
     floor = 4 * T * H * K * 2 + 2 * T * H * 4
+    # state products 6KV, the chunk-local products 3*2*BT*K + 2*2*BT*V, and the 64x64 triangular solve per chunk
+    gdr_flops = T * H * (6 * K * V + 6 * 64 * K + 4 * 64 * V + 5500)
     out = {}
     us = event_avg_us(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs,
                                                      head_first=False), steps)
     out["config2_varlen"] = {"us": round(us, 1), "tokens_per_s": round(T / (us * 1e-6), 1),
                              "sequence_lengths": lens.tolist(),
                              "operator_floor_bytes": floor + N * H * K * V * 4,
-                             "frac_of_hbm_peak": round((floor + N * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+                             "frac_of_hbm_peak": round((floor + N * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                             "algorithmic_flops": gdr_flops,
+                             "frac_of_mfma_peak": round(gdr_flops / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
     B, T2 = 8, 4096
     q, k, v = (x.view(B, T2, H, -1) for x in (q, k, v))
     g, beta = g.view(B, T2, H), beta.view(B, T2, H)
@@ -217,7 +224,9 @@ def bench_gdr(device, steps=20):
                       steps)
     out["B8_T4096"] = {"us": round(us, 1), "tokens_per_s": round(B * T2 / (us * 1e-6), 1),
                        "operator_floor_bytes": floor + B * H * K * V * 4,
-                       "frac_of_hbm_peak": round((floor + B * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+                       "frac_of_hbm_peak": round((floor + B * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                       "algorithmic_flops": gdr_flops,
+                       "frac_of_mfma_peak": round(gdr_flops / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
     return out
 
 
@@ -263,7 +272,11 @@ def bench_backward(device, steps=10):
 
     for name, fn in (("chunk_gla", gla_step), ("chunk_gated_delta_rule", gdr_step)):
         us = event_avg_us(fn, steps)
-        out[name] = {"fwd_bwd_us": round(us, 1), "tokens_per_s": round(B * T / (us * 1e-6), 1)}
+        # forward + backward FLOPs (dense-tile counts): GLA 10KV + 4*BT*(K+V); delta rule 16KV + 2*BT*(9K+5V) + 8*BT^2
+        fl = B * T * H * ((10 * K * V + 4 * 64 * (K + V)) if name == "chunk_gla"
+                          else (16 * K * V + 2 * 64 * (9 * K + 5 * V) + 8 * 64 * 64))
+        out[name] = {"fwd_bwd_us": round(us, 1), "tokens_per_s": round(B * T / (us * 1e-6), 1),
+                     "algorithmic_flops": fl, "frac_of_mfma_peak": round(fl / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
     return out
 
 
