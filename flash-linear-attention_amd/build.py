@@ -28,9 +28,10 @@ FLAGS = [
 ]
 # Keeps MFMA accumulators in ordinary vector registers: elementwise work on them (decay, scaling,
 # conversion for stores) then needs no copies out of and back into the accumulation registers.
-# Only where it measured faster (gdr_bwd_dhu 216 -> 204 us); the forward state scans lose with it.
+# Only where it measured faster (gdr_bwd_dhu 216 -> 204 us, gla_bwd_dh 166 -> 162 us); the forward state
+# scans lose with it.
 VGPR_FORM = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
-VGPR_FORM_SOURCES = {"gdr_bwd.hip"}
+VGPR_FORM_SOURCES = {"gdr_bwd.hip", "gla_bwd.hip"}
 
 
 def sources():
