@@ -9,7 +9,7 @@ from typing import Optional, Tuple
 import torch
 
 from ...utils import check_varlen_args, resolve_offsets
-from ..gated_delta_rule.chunk import ChunkGatedDeltaRuleFunction
+from ..gated_delta_rule.chunk import apply_in_value_slabs
 
 
 def chunk_delta_rule(
@@ -41,5 +41,4 @@ def chunk_delta_rule(
     offsets = resolve_offsets(offsets, cu_seqlens)
     check_varlen_args(q, offsets, head_first, initial_state)
     scale = k.shape[-1] ** -0.5 if scale is None else scale
-    return ChunkGatedDeltaRuleFunction.apply(q, k, v, None, beta, scale, initial_state, output_final_state, offsets,
-                                             head_first)
+    return apply_in_value_slabs(q, k, v, None, beta, scale, initial_state, output_final_state, offsets, head_first)

@@ -174,6 +174,27 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
                 None, None, None)
 
 
+def apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first):
+    """The autograd function on heads of any supported width (``g`` may be None: un-gated rule)."""
+    K, V = k.shape[-1], v.shape[-1]
+    if K > 256:
+        raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: key head dims up to 256 are covered (got {K}), "
+                                  f"as in the reference (fla/ops/common/chunk_delta_h.py:272)")
+    if V > 128:
+        # the delta rule is independent per value column: wider heads run as slabs of 128 columns
+        # (autograd sums the slabs' gradients of q, k, g and beta)
+        outs, states = [], []
+        for v0 in range(0, V, 128):
+            h0 = None if initial_state is None else initial_state[..., v0:v0 + 128]
+            o, ht = ChunkGatedDeltaRuleFunction.apply(q, k, v[..., v0:v0 + 128], g, beta, scale, h0, output_final_state,
+                                                      offsets, head_first)
+            outs.append(o)
+            states.append(ht)
+        return torch.cat(outs, dim=-1), (torch.cat(states, dim=-1) if output_final_state else None)
+    return ChunkGatedDeltaRuleFunction.apply(q, k, v, g, beta, scale, initial_state, output_final_state, offsets,
+                                             head_first)
+
+
 def chunk_gated_delta_rule(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -208,20 +229,4 @@ def chunk_gated_delta_rule(
         scale = k.shape[-1] ** -0.5
     else:
         assert scale > 0, "Scale must be positive."
-    K, V = k.shape[-1], v.shape[-1]
-    if K > 256:
-        raise NotImplementedError(f"fla_amd chunk_gated_delta_rule: key head dims up to 256 are covered (got {K}), "
-                                  f"as in the reference (fla/ops/common/chunk_delta_h.py:272)")
-    if V > 128:
-        # the delta rule is independent per value column: wider heads run as slabs of 128 columns
-        # (autograd sums the slabs' gradients of q, k, g and beta)
-        outs, states = [], []
-        for v0 in range(0, V, 128):
-            h0 = None if initial_state is None else initial_state[..., v0:v0 + 128]
-            o, ht = ChunkGatedDeltaRuleFunction.apply(q, k, v[..., v0:v0 + 128], g, beta, scale, h0, output_final_state,
-                                                      offsets, head_first)
-            outs.append(o)
-            states.append(ht)
-        return torch.cat(outs, dim=-1), (torch.cat(states, dim=-1) if output_final_state else None)
-    return ChunkGatedDeltaRuleFunction.apply(q, k, v, g, beta, scale, initial_state, output_final_state, offsets,
-                                             head_first)
+    return apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first)

@@ -17,16 +17,16 @@ def _dev(device):
 
 
 # reference ladder: tests/ops/test_delta.py (T in {63, 300, 1000}-style lengths, packed batches)
-@pytest.mark.parametrize("T", [63, 300, 1000])
+@pytest.mark.parametrize("T,K,V", [(63, 128, 128), (300, 128, 128), (1000, 128, 128), (300, 256, 256), (150, 200, 100)])
 @pytest.mark.parametrize("varlen", [False, True])
-def test_chunk_delta_rule(device, T, varlen):
+def test_chunk_delta_rule(device, T, K, V, varlen):
     from fla_amd.ops.delta_rule import chunk_delta_rule
     from oracle.recurrent import naive_recurrent_gated_delta_rule
     N = 3
     offs = random_offsets(T, N, torch.Generator().manual_seed(T), min_len=1) if varlen else None
-    q, k, v, _, beta, h0 = gdr_inputs(1 if varlen else 2, T, 2, 128, 128, seed=T, N=N if varlen else None)
+    q, k, v, _, beta, h0 = gdr_inputs(1 if varlen else 2, T, 2, K, V, seed=T, N=N if varlen else None)
     dev = _dev(device)
-    print(f"chunk_delta_rule T={T} varlen={varlen}", flush=True)
+    print(f"chunk_delta_rule T={T} K={K} V={V} varlen={varlen}", flush=True)
     do = torch.randn(v.shape, generator=torch.Generator().manual_seed(1)).to(v.dtype)
     dht = torch.randn(h0.shape, generator=torch.Generator().manual_seed(2)) * 0.1
     # device
