@@ -393,6 +393,7 @@ struct DHParams {
   const int64_t* chunk_offsets;
   int64_t T;
   int H, V, N;
+  void* h2;  // with the transposed fragment layout: a second copy in FLA_H_FRAGMENT order, or NULL
 };
 
 // One workgroup: all K rows x 32 value columns of one (sequence, head) state.
@@ -581,6 +582,11 @@ __global__ __launch_bounds__(256) void gdr_fwd_h_kernel(DHParams p) {
             }
             *(v8*)hp = tl;
             *(v8*)(hp + 8) = th;
+            if (p.h2) {
+              T* hq = (T*)p.h2 + blk + (((int64_t)kt * (V / 32) + vt) * 64 + lane) * 16;
+              *(v8*)hq = lo;
+              *(v8*)(hq + 8) = hi;
+            }
           } else if (HL == 0) {
             T* hp = (T*)p.h + blk;
 #pragma unroll
@@ -941,9 +947,27 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, co
   else FLA_REQUIRE(h_dtype == qkv_dtype || h_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)h | (uintptr_t)v_new) % 16 == 0,
               FLA_E_ALIGNMENT);
-  DHParams p{k, w, u, g_cumsum, h0, h, v_new, ht, offsets, chunk_offsets, T, (int)H, (int)V, (int)N};
+  DHParams p{k, w, u, g_cumsum, h0, h, v_new, ht, offsets, chunk_offsets, T, (int)H, (int)V, (int)N, nullptr};
   if (qkv_dtype == FLA_BF16) return launch_dh<bf16>(p, (int)K, h_dtype, h_layout, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_dh<f16>(p, (int)K, h_dtype, h_layout, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_h_both(const void* k, const void* w, const void* u,
+                                                     const float* g_cumsum, const float* h0, void* h_frag,
+                                                     void* h_frag_t, void* v_new, float* ht, const int64_t* offsets,
+                                                     const int64_t* chunk_offsets, int qkv_dtype, int64_t B, int64_t T,
+                                                     int64_t H, int64_t K, int64_t V, int64_t N, fla_stream_t stream) {
+  FLA_REQUIRE(k && w && u && h_frag && h_frag_t, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(V % 32 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(chunk_offsets != nullptr && B == 1, FLA_E_INVALID);
+  else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)h_frag | (uintptr_t)h_frag_t |
+               (uintptr_t)v_new) % 16 == 0, FLA_E_ALIGNMENT);
+  DHParams p{k, w, u, g_cumsum, h0, h_frag_t, v_new, ht, offsets, chunk_offsets, T, (int)H, (int)V, (int)N, h_frag};
+  if (qkv_dtype == FLA_BF16) return launch_dh<bf16>(p, (int)K, qkv_dtype, FLA_H_FRAGMENT_T, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_dh<f16>(p, (int)K, qkv_dtype, FLA_H_FRAGMENT_T, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
 }
 

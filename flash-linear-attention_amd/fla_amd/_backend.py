@@ -42,6 +42,7 @@ SIGNATURES = {
     "fla_gdr_fwd_wy": (c_int, [P, P, P, P, P, P, P, P, P, P, F, P, P, I64, I, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                                  I64, I64, I64, I64, I64, I64, P]),
+    "fla_chunk_gated_delta_rule_fwd_h_both": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_fused": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 19 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),

@@ -63,6 +63,48 @@ def chunk_gated_delta_rule_fwd_h(
     return h, v_new, ht
 
 
+def chunk_gated_delta_rule_fwd_h_both(
+    k: torch.Tensor,
+    w: torch.Tensor,
+    u: torch.Tensor,
+    g: Optional[torch.Tensor],
+    initial_state: Optional[torch.Tensor],
+    output_final_state: bool,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    chunk_offsets: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """The state scan for a forward pass whose states are kept for the backward pass: returns
+    ``(h, hT, v_new, final_state)`` with the per-chunk states in MFMA-fragment order (for
+    ``chunk_fwd_o``) and in transposed fragment order (for ``fla_chunk_gated_delta_rule_bwd``).
+    Seq-first, chunk size 64; served by ``fla_chunk_gated_delta_rule_fwd_h_both``."""
+    be.require_gpu(k, w, u)
+    B, T, H, K = k.shape
+    V = u.shape[-1]
+    if offsets is None:
+        N, NT = B, -(-T // BT)
+    else:
+        if chunk_offsets is None:
+            chunk_offsets = prepare_chunk_offsets(offsets, BT, device=k.device)
+        N = len(offsets) - 1
+        NT = int(indices.shape[0]) if indices is not None else int(prepare_chunk_offsets(offsets, BT)[-1])
+        offsets = offsets.to(torch.int64).contiguous()
+    h = k.new_empty(B, NT, H, K, V)
+    hT = k.new_empty(B, NT, H, K, V)
+    v_new = torch.empty_like(u)
+    ht = k.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
+    h0 = None
+    if initial_state is not None:
+        h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
+    if g is not None and g.dtype != torch.float32:
+        g = g.float()
+    be.check(be.lib().fla_chunk_gated_delta_rule_fwd_h_both(
+        be.ptr(k), be.ptr(w), be.ptr(u), be.ptr(g), be.ptr(h0), be.ptr(h), be.ptr(hT), be.ptr(v_new), be.ptr(ht),
+        be.ptr(offsets), be.ptr(chunk_offsets), be.dt(k), B, T, H, K, V, N, be.stream_of(k)),
+        "fla_chunk_gated_delta_rule_fwd_h_both")
+    return h, hT, v_new, ht
+
+
 def chunk_gated_delta_rule_fwd_fused(
     q: torch.Tensor,
     k: torch.Tensor,

@@ -4,9 +4,12 @@
 Forward pipeline on the device (chunk size 64): ``fla_chunk_local_cumsum`` (gate)
 -> ``fla_gdr_fwd_wy`` (KK^T, block inverse, w/u, gated causal q k^T scores)
 -> ``fla_chunk_gated_delta_rule_fwd_fused`` (state scan and output in one launch).
-The backward recomputes w, u, the per-chunk states and v_new with
+A forward pass that will be differentiated runs the two-launch form instead (state scan, output
+stage) and keeps w, Aw, v_new and the per-chunk states for the backward; with
+``KEEP_STATES_FOR_BACKWARD = False`` the backward recomputes them with
 ``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
 """
+import os
 import warnings
 from typing import Optional, Tuple
 
@@ -16,7 +19,8 @@ import torch.nn.functional as F
 from ... import _backend as be
 from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
                       resolve_offsets)
-from ..common.chunk_delta_h import chunk_gated_delta_rule_fwd_fused, chunk_gated_delta_rule_fwd_h
+from ..common.chunk_delta_h import (chunk_gated_delta_rule_fwd_fused, chunk_gated_delta_rule_fwd_h,
+                                    chunk_gated_delta_rule_fwd_h_both)
 from ..common.chunk_o import chunk_fwd_o
 from ..utils.cumsum import chunk_local_cumsum
 from .wy_fast import fwd_prepare_wy_repr
@@ -24,6 +28,13 @@ from .wy_fast import fwd_prepare_wy_repr
 BT = 64
 _SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64), (256, 64), (256, 128)}
 _FUSED_MAX_K = 128  # the one-pass forward kernel holds at most 128 key channels of the state
+
+# A forward pass that will be differentiated keeps w, Aw, v_new and the per-chunk states for its
+# backward pass (about 2.3 bytes per q/k/v byte) instead of recomputing them there as the reference
+# does (fla/ops/gated_delta_rule/chunk.py:95-116): with 288 GB of HBM the second WY launch and the
+# second state scan cost more than the memory.  FLA_AMD_RECOMPUTE_STATES=1 (or setting this flag to
+# False) restores the reference's behaviour.
+KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("", "0")
 
 
 def _round64(d: int) -> int:
@@ -66,10 +77,29 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     return g, o, Aw, Au, final_state
 
 
-def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do, dht, offsets=None):
+def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, output_final_state, offsets=None):
+    """Forward of a pass that will be differentiated: the two-launch form (state scan, output stage),
+    whose intermediates are what the backward needs.  Returns ``(g_cumsum, o, final_state, kept)``
+    with ``kept = (w, Aw, v_new, hT)`` for :func:`chunk_gated_delta_rule_bwd`."""
+    plan = VarlenPlan(offsets, BT) if offsets is not None else None
+    offs = None if plan is None else plan.offsets
+    idx = None if plan is None else plan.indices
+    co = None if plan is None else plan.chunk_offsets
+    g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
+    beta = beta.float().contiguous()
+    w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
+                                      store_A=True, store_Au=False)
+    h, hT, v_new, final_state = chunk_gated_delta_rule_fwd_h_both(
+        k, w, u, g, initial_state, output_final_state, offsets=offs, indices=idx, chunk_offsets=co)
+    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False,
+                    chunk_size=BT)
+    return g, o, final_state, (w, Aw, v_new, hT)
+
+
+def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do, dht, offsets=None, kept=None):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims; ``g_cumsum``
-    the fp32 chunk-local cumsum saved by the forward).  Recomputes w, u, Aw, the per-chunk
-    states and v_new like the reference (``fla/ops/gated_delta_rule/chunk.py:95-116``).
+    the fp32 chunk-local cumsum saved by the forward).  Without ``kept`` it recomputes w, u, Aw, the
+    per-chunk states and v_new like the reference (``fla/ops/gated_delta_rule/chunk.py:95-116``).
     Returns ``(dq, dk, dv, dbeta, dg, dh0)``."""
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
@@ -80,11 +110,15 @@ def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do
     N = B if plan is None else plan.N
     NT = 0 if plan is None else plan.NT
     beta = beta.float().contiguous()
-    w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g_cumsum, offsets=offs, indices=idx, head_first=False,
-                                      chunk_size=BT, store_A=True, store_Au=False)
-    hT, v_new, _ = chunk_gated_delta_rule_fwd_h(
-        k=k, w=w, u=u, g=g_cumsum, initial_state=initial_state, output_final_state=False, offsets=offs, indices=idx,
-        head_first=False, chunk_size=BT, fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
+    if kept is not None:
+        w, Aw, v_new, hT = kept
+    else:
+        w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g_cumsum, offsets=offs, indices=idx, head_first=False,
+                                          chunk_size=BT, store_A=True, store_Au=False)
+        hT, v_new, _ = chunk_gated_delta_rule_fwd_h(
+            k=k, w=w, u=u, g=g_cumsum, initial_state=initial_state, output_final_state=False, offsets=offs,
+            indices=idx, head_first=False, chunk_size=BT, fragment_layout=True, transposed_fragments=True,
+            chunk_offsets=co)
     ws_dvl, ws_dv2 = torch.empty_like(v), torch.empty_like(v)
     ws_dh = torch.empty_like(hT)
     ws_dw, ws_dkp = torch.empty_like(k), torch.empty_like(k)
@@ -131,10 +165,15 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             v = F.pad(v, (0, VP - V))
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
-        gc, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
-                                                     offsets=offsets, head_first=False, chunk_size=BT, store_A=False,
-                                                     fused=KP <= _FUSED_MAX_K)
-        ctx.save_for_backward(q, k, v, gc, beta, h0, offsets)
+        kept = ()
+        if KEEP_STATES_FOR_BACKWARD and any(ctx.needs_input_grad):
+            gc, o, ht, kept = chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, h0, output_final_state,
+                                                              offsets=offsets)
+        else:
+            gc, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
+                                                         offsets=offsets, head_first=False, chunk_size=BT,
+                                                         store_A=False, fused=KP <= _FUSED_MAX_K)
+        ctx.save_for_backward(q, k, v, gc, beta, h0, offsets, *kept)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
@@ -149,7 +188,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        q, k, v, gc, beta, h0, offsets = ctx.saved_tensors
+        q, k, v, gc, beta, h0, offsets, *kept = ctx.saved_tensors
         K, V, KP, VP = ctx.dims
         if ctx.head_first:
             do = do.transpose(1, 2)
@@ -159,7 +198,8 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         do = do.contiguous()
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
-        dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(q, k, v, gc, beta, ctx.scale, h0, do, dht, offsets)
+        dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(q, k, v, gc, beta, ctx.scale, h0, do, dht, offsets,
+                                                             kept=tuple(kept) if kept else None)
         if (KP, VP) != (K, V):
             dq, dk, dv = dq[..., :K], dk[..., :K], dv[..., :V]
             if dh0 is not None:

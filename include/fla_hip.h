@@ -203,6 +203,17 @@ int fla_chunk_gated_delta_rule_fwd_h(const void* k, const void* w, const void* u
                                      int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                      fla_stream_t stream);
 
+/* The same scan with the per-chunk states written in both fragment orders: h_frag (FLA_H_FRAGMENT, for
+ * fla_chunk_fwd_o) and h_frag_t (FLA_H_FRAGMENT_T, for fla_chunk_gated_delta_rule_bwd), both
+ * [chunks, H, K*V] in the q/k/v dtype.  For callers that keep the states of the forward pass for the
+ * backward pass instead of recomputing them as chunk_gated_delta_rule_bwd does
+ * (fla/ops/gated_delta_rule/chunk.py:105-116). */
+int fla_chunk_gated_delta_rule_fwd_h_both(const void* k, const void* w, const void* u, const float* g_cumsum,
+                                          const float* h0, void* h_frag, void* h_frag_t, void* v_new, float* ht,
+                                          const int64_t* offsets, const int64_t* chunk_offsets, int qkv_dtype,
+                                          int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                          fla_stream_t stream);
+
 int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_cumsum, const void* h, void* o,
                     const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream);

@@ -231,3 +231,33 @@ def test_chunk_gdr_reference_ladder(device, D, T, scale, normalizer, head_first)
     ref = _grads_ref(q, k, v, g, beta, h0, do, dht, scale=scale)
     for name, r, x, tol in zip(NAMES, ref, got, TOLS):
         assert_close(name, r, x, tol)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gdr_keep_vs_recompute(device, varlen, monkeypatch):
+    """The backward from kept forward states and the reference-style backward that recomputes them
+    run the same kernels on the same operands: identical gradients; both forwards within tolerance."""
+    import fla_amd.ops.gated_delta_rule.chunk as mod
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(12)
+    T, N, H, D = 400, 3, 2, 128
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q, k, v, g, beta, h0 = gdr_inputs(1 if varlen else 2, T, H, D, D, seed=63, N=N if varlen else None, h0_std=1.0)
+    do = torch.randn(q.shape[0], T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    print(f"chunk_gdr keep vs recompute varlen={varlen}", flush=True)
+    assert mod.KEEP_STATES_FOR_BACKWARD
+    kept = _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs)
+    o_keep, ht_keep = _run(device, *[x.requires_grad_() for x in (q.clone(), k.clone(), v.clone())], g, beta, h0,
+                           offsets=offs)
+    monkeypatch.setattr(mod, "KEEP_STATES_FOR_BACKWARD", False)
+    rec = _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs)
+    for name, a, b in zip(NAMES, kept, rec):
+        if name in ("dg", "dbeta"):   # summed with LDS atomics: the order of the additions is not fixed
+            assert_close(name, a, b, 1e-5)
+        else:
+            assert torch.equal(a, b), name
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    assert_close("o (two launches, states kept)", ro, o_keep, TOL_O)
+    assert_close("ht (two launches, states kept)", rht, ht_keep, TOL_HT)
