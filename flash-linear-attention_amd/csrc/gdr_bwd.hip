@@ -893,6 +893,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   // ================= value side: d(vb) = Au^T du ; dAu = (du v^T) diag(beta)
   const int ib = wave >> 1, jb = wave & 1;     // score quadrants: waves 0,2,3 -> (0,0),(1,0),(1,1)
   f32x16 dAu = zero16();
+  v4 dvst[TV][4];
   {
     f32x16 dvb[TV];
 #pragma unroll
@@ -907,9 +908,9 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) dAu[r] *= bcol;
     }
-    // dv = beta d(vb);  dbeta += sum_v d(vb) * v
+    // dv = beta d(vb), kept in registers until the tiles are free to carry it to whole-row stores;
+    // dbeta += sum_v d(vb) * v
     float part = 0.f;
-    T* dvp = (T*)p.dv + ((row0 + jrow) * H + hh) * (int64_t)V;
 #pragma unroll
     for (int t = 0; t < TV; ++t)
 #pragma unroll
@@ -922,7 +923,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
           part += d * (float)vv[e];
           o[e] = (T)(d * bj);
         }
-        if (jrow < L) *(v4*)(dvp + col) = o;
+        dvst[t][r4] = o;
       }
     part += __shfl_xor(part, 32, 64);
     if (lane < 32) atomicAdd(&sDb[jrow], part);
@@ -933,6 +934,19 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   IOK::put_tr(sTr1, tid, rdw);
   IOK::put_rows(sRow2, LDD, tid, rk);
   __syncthreads();
+  // the partial dk of the previous launch is needed only in the last step: fetched now, so that its
+  // latency hides behind the products
+  v4 dinr[TK][4];
+  {
+    const T* dip = p.dk_in ? (const T*)p.dk_in + ((row0 + jrow) * H + hh) * (int64_t)K : nullptr;
+#pragma unroll
+    for (int t = 0; t < TK; ++t)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        dinr[t][r4] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        if (dip && jrow < L) dinr[t][r4] = *(const v4*)(dip + (cw * TK + t) * 32 + 8 * r4 + 4 * (lane >> 5));
+      }
+  }
   f32x16 dkb[TK];   // d(kb)^T: columns (cw*TK+t)*32.., time row jrow
 #pragma unroll
   for (int t = 0; t < TK; ++t) dkb[t] = zero16();
@@ -1035,32 +1049,48 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   mm64t<T, TK>(sTr1, LDT, cw * TK * 32, sS2, LDT, rw, rw * 32, BT, lane, dk2);
   {
     float part = 0.f;
-    const int64_t rowoff = ((row0 + jrow) * H + hh) * (int64_t)K;
-    T* dkp = (T*)p.dk + rowoff;
-    const T* dip = p.dk_in ? (const T*)p.dk_in + rowoff : nullptr;
 #pragma unroll
     for (int t = 0; t < TK; ++t)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int col = (cw * TK + t) * 32 + 8 * r4 + 4 * (lane >> 5);
         v4 kk = *(const v4*)&sRow2[jrow * LDD + col], o;
-        v4 din = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        if (dip && jrow < L) din = *(const v4*)(dip + col);
+        const v4 din = dinr[t][r4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float d = dkb[t][4 * r4 + e];
           part += d * (float)kk[e];
           o[e] = (T)(d * bj + dk2[t][4 * r4 + e] + (float)din[e]);
         }
-        if (jrow < L) *(v4*)(dkp + col) = o;
+        // dk takes the place of the k element this lane has just read (nobody else reads the tile any more)
+        *(v4*)&sRow2[jrow * LDD + col] = o;
       }
     part += __shfl_xor(part, 32, 64);
     if (lane < 32) atomicAdd(&sDb[jrow], part);
   }
-  __syncthreads();
+  __syncthreads();  // every wave is past its last read of X1^T / dM^T, which share storage with the dv tile
   if (tid < L) {
     p.dbeta[(row0 + tid) * H + hh] = sDb[tid];
     p.dgam2[(row0 + tid) * H + hh] = sDg[tid];
+  }
+#pragma unroll
+  for (int t = 0; t < TV; ++t)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4)
+      *(v4*)&sRow1[jrow * LDD + (cw * TV + t) * 32 + 8 * r4 + 4 * (lane >> 5)] = dvst[t][r4];
+  __syncthreads();
+  // dk and dv leave as whole rows, 16 bytes per lane (8-byte pieces scattered over 32 rows cost
+  // several times their bytes)
+  {
+    constexpr int CK = K / 8, CV = V / 8;
+    for (int e = tid; e < BT * CK; e += 256) {
+      const int row = e / CK, c8 = (e % CK) * 8;
+      if (row < L) *(v8*)((T*)p.dk + ((row0 + row) * H + hh) * (int64_t)K + c8) = *(const v8*)&sRow2[row * LDD + c8];
+    }
+    for (int e = tid; e < BT * CV; e += 256) {
+      const int row = e / CV, c8 = (e % CV) * 8;
+      if (row < L) *(v8*)((T*)p.dv + ((row0 + row) * H + hh) * (int64_t)V + c8) = *(const v8*)&sRow1[row * LDD + c8];
+    }
   }
 }
 
