@@ -721,10 +721,11 @@ __global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
   constexpr int NP = BT * C8 / 256;          // pieces per thread
   constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
   constexpr int KT32 = K / 32, TV = V / 64;
-  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
-  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];  // later P
+  __shared__ __attribute__((aligned(16))) T sQK[2 * BT * LDK];  // q | k (later P); at the end the output tile
   __shared__ __attribute__((aligned(16))) T sVt[V * LDT];
   __shared__ float sGam[BT];
+  T* sQ = sQK;
+  T* sK = sQK + BT * LDK;
   T* sP = sK;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -778,35 +779,49 @@ __global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
     *(v8*)&sQ[row * LDK + c8] = qreg[i];
     *(v8*)&sK[row * LDK + c8] = kreg[i];
   }
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    T* dst = &sVt[(cv4 + j) * LDT + rgv * RPTV];
-#pragma unroll
-    for (int i = 0; i < RPTV; ++i) dst[i] = vreg[i][j];
-  }
-  __syncthreads();
-
-  const int qi = wave >> 1, qj = wave & 1;
-  f32x16 s = zero16();
-  if (qj <= qi) {
-#pragma unroll
-    for (int ks = 0; ks < K; ks += 16)
-      s = Elem<T>::mfma32(lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
-  }
-  __syncthreads();  // all reads of sK done before P overwrites it
   {
-    const int j = qj * 32 + (lane & 31);
-    const float gj = sGam[j];
+    // a lane owns RPTV consecutive time rows of 4 value columns: one vector write per column
+    typedef T rvec __attribute__((ext_vector_type(RPTV)));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = qi * 32 + c32_row(r, lane);
-      float val = (j <= i) ? s[r] * p.scale * __expf(sGam[i] - gj) : 0.f;
-      sP[i * LDT + j] = (T)val;
+    for (int j = 0; j < 4; ++j) {
+      rvec x;
+#pragma unroll
+      for (int i = 0; i < RPTV; ++i) x[i] = vreg[i][j];
+      *(rvec*)&sVt[(cv4 + j) * LDT + rgv * RPTV] = x;
     }
   }
   __syncthreads();
 
-  f32x16 acc[TV];
+  // Every product is formed transposed (operands swapped): a lane then holds one time row and four
+  // consecutive columns per register quad, so the score tile and the output tile are written to
+  // LDS with 8-byte vectors and the output leaves as whole rows.
+  const int qi = wave >> 1, qj = wave & 1;
+  f32x16 s = zero16();   // s[4a+b] = (q k^T)[i][j0+b], i = 32 qi + lane%32, j0 = 32 qj + 8a + 4 (lane/32)
+  if (qj <= qi) {
+#pragma unroll
+    for (int ks = 0; ks < K; ks += 16)
+      s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qj * 32, ks, lane), lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), s);
+  }
+  __syncthreads();  // all reads of sK done before P overwrites it
+  {
+    const int i = qi * 32 + (lane & 31);
+    const float gi = sGam[i];
+#pragma unroll
+    for (int a4 = 0; a4 < 4; ++a4) {
+      const int j0 = qj * 32 + 8 * a4 + 4 * (lane >> 5);
+      v4 x;
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) {
+        const int j = j0 + b4;
+        x[b4] = (T)((j <= i) ? s[4 * a4 + b4] * p.scale * __expf(gi - sGam[j]) : 0.f);
+      }
+      *(v4*)&sP[i * LDT + j0] = x;
+    }
+  }
+  __syncthreads();
+
+  const int trow = rw * 32 + (lane & 31);   // this lane's time row in the transposed output tiles
+  f32x16 acc[TV];                           // acc[tv][4a+b] = o[trow][32 (cw TV + tv) + 8a + 4 (lane/32) + b]
 #pragma unroll
   for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
 #pragma unroll
@@ -815,29 +830,44 @@ __global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
     for (int half = 0; half < 2; ++half) {
       v8 a = lds_frag32_perm<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
 #pragma unroll
-      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(a, hf[kt][tv][half], acc[tv]);
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(hf[kt][tv][half], a, acc[tv]);
     }
+  {
+    const float rs = p.scale * __expf(sGam[trow]);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float rs = p.scale * __expf(sGam[rw * 32 + c32_row(r, lane)]);
+    for (int tv = 0; tv < TV; ++tv)
 #pragma unroll
-    for (int tv = 0; tv < TV; ++tv) acc[tv][r] *= rs;
+      for (int r = 0; r < 16; ++r) acc[tv][r] *= rs;
   }
   const int jend = (rw + 1) * 32;
   for (int js = 0; js < jend; js += 16) {
     v8 a = lds_frag32<T>(sP, LDT, rw * 32, js, lane);
 #pragma unroll
     for (int tv = 0; tv < TV; ++tv)
-      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
+      acc[tv] = Elem<T>::mfma32(lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), a, acc[tv]);
   }
-  T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
+  __syncthreads();  // q is consumed: its tile carries the output
+  constexpr int LDO = V + 8;
+  static_assert(LDO <= 2 * LDK, "the output tile fits the q and k tiles");
+  T* sO = sQK;  // [t][v]; with V > K it runs on into the k tile (P), which is consumed as well
 #pragma unroll
   for (int tv = 0; tv < TV; ++tv)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = rw * 32 + c32_row(r, lane);
-      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+    for (int a4 = 0; a4 < 4; ++a4) {
+      v4 x;
+#pragma unroll
+      for (int b4 = 0; b4 < 4; ++b4) x[b4] = (T)acc[tv][4 * a4 + b4];
+      *(v4*)&sO[trow * LDO + (cw * TV + tv) * 32 + 8 * a4 + 4 * (lane >> 5)] = x;
     }
+  __syncthreads();
+  {
+    constexpr int CV = V / 8;
+    T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
+    for (int e = tid; e < BT * CV; e += 256) {
+      const int row = e / CV, c8 = (e % CV) * 8;
+      if (row < L) *(v8*)(op + (int64_t)row * H * V + c8) = *(const v8*)&sO[row * LDO + c8];
+    }
+  }
 }
 
 template <typename T>
