@@ -53,9 +53,9 @@ struct ConvParams {
   int D, silu;
 };
 
-FLA_DEVICE float silu_f(float z) { return z / (1.f + __expf(-z)); }
+FLA_DEVICE float silu_f(float z) { return z * __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
 FLA_DEVICE float silu_grad(float z) {
-  const float s = 1.f / (1.f + __expf(-z));
+  const float s = __builtin_amdgcn_rcpf(1.f + __expf(-z));  // hardware reciprocal (1 ulp), not an IEEE division
   return s * (1.f + z * (1.f - s));
 }
 
