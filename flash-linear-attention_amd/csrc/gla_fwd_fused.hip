@@ -40,6 +40,7 @@ struct FusedParams {
   int64_t T;
   int H, V, N;
   float scale;
+  void* hT;         // HT variant: the state entering every chunk, FLA_H_FRAGMENT_T order, [chunks, H, K*V]
 };
 
 // The row-major q~ / k~ tiles are written by lanes that own four adjacent rows each, i.e.
@@ -65,7 +66,10 @@ FLA_DEVICE typename Elem<T>::v8 frag32_perm_swz(const T* tile, int ld, int row0,
 }
 
 // NSTG: number of staging waves (4 or 8); the workgroup has 4 + NSTG waves.
-template <typename T, typename GT, int K, int NSTG>
+// HT: the matrix waves keep a transposed copy of their state tiles as well and write the state
+// entering every chunk to p.hT (what the backward kernels contract over v with), for a forward pass
+// whose states are kept instead of being recomputed by the backward pass.
+template <typename T, typename GT, int K, int NSTG, bool HT>
 __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
@@ -330,19 +334,47 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     // =========================== matrix waves ===========================
     const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
     f32x16 acc[NKT][2];                         // state tiles kt = wave + 4a, value tiles 0/1
+    f32x16 acct[HT ? NKT : 1][2];               // HT: the same tiles transposed (rows v, columns k)
 #pragma unroll
     for (int a = 0; a < NKT; ++a)
 #pragma unroll
       for (int vt = 0; vt < 2; ++vt) {
         acc[a][vt] = zero16();
+        if (HT) acct[a][vt] = zero16();
         int kt = wave + 4 * a;
         if (p.h0 && kt < KT32) {
           const float* h0p = p.h0 + (int64_t)nh * K * V;
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
+          for (int r = 0; r < 16; ++r) {
             acc[a][vt][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + vt * 32 + (lane & 31)];
+            if (HT) acct[a][vt][r] = h0p[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + vt * 32 + c32_row(r, lane)];
+          }
         }
       }
+    // HT: state entering chunk c, transposed fragment order, straight from the accumulators
+    auto store_ht = [&](int64_t c) {
+      if constexpr (HT) {
+        T* hb = (T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V;
+#pragma unroll
+        for (int a = 0; a < NKT; ++a) {
+          int kt = wave + 4 * a;
+          if (kt < KT32) {
+#pragma unroll
+            for (int vt = 0; vt < 2; ++vt) {
+              v8 lo, hi;
+#pragma unroll
+              for (int r = 0; r < 8; ++r) {
+                lo[r] = (T)acct[a][vt][r];
+                hi[r] = (T)acct[a][vt][r + 8];
+              }
+              T* dst = hb + (((int64_t)(vbase / 32 + vt) * (K / 32) + kt) * 64 + lane) * 16;
+              *(v8*)dst = lo;
+              *(v8*)(dst + 8) = hi;
+            }
+          }
+        }
+      }
+    };
     auto publish_state = [&]() {
 #pragma unroll
       for (int a = 0; a < NKT; ++a) {
@@ -364,6 +396,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     };
     publish_state();
+    if (nchunks > 0) store_ht(0);
     // The matrix waves also stage the value tile (time-contiguous) of the next chunk: 8 rows x
     // 2 columns per lane, loaded one chunk period ahead.
     const int vrg = tid >> 5, vc = (tid & 31) * 2;
@@ -507,15 +540,29 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
               acc[a][1][4 * q4 + b] *= d[b];
             }
           }
+          if (HT) {
+            const float dcol = sDecay[buf][kt * 32 + (lane & 31)];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              acct[a][0][r] *= dcol;
+              acct[a][1][r] *= dcol;
+            }
+          }
 #pragma unroll
           for (int ts = 0; ts < BT; ts += 16) {
             v8 fk = lds_frag32<T>(sKh[buf], LDT, kt * 32, ts, lane);
-            acc[a][0] = Elem<T>::mfma32(fk, lds_frag32<T>(sVt[buf], LDT, 0, ts, lane), acc[a][0]);
-            acc[a][1] = Elem<T>::mfma32(fk, lds_frag32<T>(sVt[buf], LDT, 32, ts, lane), acc[a][1]);
+            v8 fv0 = lds_frag32<T>(sVt[buf], LDT, 0, ts, lane), fv1 = lds_frag32<T>(sVt[buf], LDT, 32, ts, lane);
+            acc[a][0] = Elem<T>::mfma32(fk, fv0, acc[a][0]);
+            acc[a][1] = Elem<T>::mfma32(fk, fv1, acc[a][1]);
+            if (HT) {
+              acct[a][0] = Elem<T>::mfma32(fv0, fk, acct[a][0]);
+              acct[a][1] = Elem<T>::mfma32(fv1, fk, acct[a][1]);
+            }
           }
         }
       }
       publish_state();
+      if (c + 1 < nchunks) store_ht(c + 1);
     }
     if (nchunks > 0) lds_barrier();  // hands the last output tile to the staging waves
     if (p.ht) {
@@ -720,21 +767,26 @@ int launch_fused(const FusedParams& p, int K, hipStream_t st) {
   if (total == 0) return FLA_OK;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   dim3 grid((unsigned)total);
-  if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4>), grid, dim3(512), 0, st, p);
-  else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4>), grid, dim3(512), 0, st, p);
-  else return FLA_E_UNSUPPORTED;
+  if (p.hT) {
+    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, true>), grid, dim3(512), 0, st, p);
+    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, true>), grid, dim3(512), 0, st, p);
+    else return FLA_E_UNSUPPORTED;
+  } else {
+    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, false>), grid, dim3(512), 0, st, p);
+    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, false>), grid, dim3(512), 0, st, p);
+    else return FLA_E_UNSUPPORTED;
+  }
   FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
 
 }  // namespace
 
-extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates, const float* h0,
-                                       void* o, float* ht, int* ws_wide, void* ws_hwide, const int64_t* offsets,
-                                       const int64_t* indices, const int64_t* chunk_offsets,
-                                       const int64_t* seq_order, int64_t NT,
-                                       int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
-                                       int64_t V, int64_t N, float scale, fla_stream_t stream) {
+static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const void* gates, const float* h0,
+                              void* o, float* ht, int* ws_wide, void* ws_hwide, void* h_frag_t, const int64_t* offsets,
+                              const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                              int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
+                              int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE((K == 64 || K == 128) && V % 64 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
@@ -744,8 +796,12 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
   if (ws_wide) FLA_REQUIRE(V <= 128, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)o | (uintptr_t)ws_hwide) % 16 == 0,
               FLA_E_ALIGNMENT);
+  if (h_frag_t) {
+    FLA_REQUIRE((uintptr_t)h_frag_t % 16 == 0, FLA_E_ALIGNMENT);
+    if (offsets) FLA_REQUIRE(chunk_offsets != nullptr, FLA_E_INVALID);
+  }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
-                T, (int)H, (int)V, (int)N, scale};
+                T, (int)H, (int)V, (int)N, scale, h_frag_t};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;
@@ -768,4 +824,25 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
   if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) FLA_FUSED(f16, f16)
 #undef FLA_FUSED
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const void* gates, const float* h0,
+                                       void* o, float* ht, int* ws_wide, void* ws_hwide, const int64_t* offsets,
+                                       const int64_t* indices, const int64_t* chunk_offsets,
+                                       const int64_t* seq_order, int64_t NT,
+                                       int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
+                                       int64_t V, int64_t N, float scale, fla_stream_t stream) {
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, offsets, indices, chunk_offsets,
+                            seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, const void* v, const void* gates,
+                                              const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                              void* h_frag_t, const int64_t* offsets, const int64_t* indices,
+                                              const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                                              int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
+                                              int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(h_frag_t, FLA_E_INVALID);
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, offsets, indices, chunk_offsets,
+                            seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
 }

@@ -4,6 +4,7 @@ Forward pipeline on the device (chunk size 64):
 ``fla_chunk_gla_fwd_h`` (state scan, cumsum of the gates formed in-kernel)
 -> ``fla_chunk_gla_fwd_o`` (fused cumsum + gated scores + output).
 """
+import os
 import warnings
 from typing import Optional, Tuple
 
@@ -17,6 +18,12 @@ from ..utils.cumsum import chunk_local_cumsum
 
 BT = 64
 _SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
+
+# A forward pass that will be differentiated has the fused launch write the state entering every
+# chunk (one more [K, V] tile in the q/k/v dtype per chunk and head) and keeps it for the backward
+# pass, which the reference starts by recomputing those states (fla/ops/gla/chunk.py:1239-1253).
+# FLA_AMD_RECOMPUTE_STATES=1 (or setting this flag to False) restores the reference's behaviour.
+KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("", "0")
 
 
 def _pad_dim(x: Optional[torch.Tensor], size: int) -> Optional[torch.Tensor]:
@@ -52,11 +59,13 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
 
 
 def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,
-                        return_flags=False):
+                        return_flags=False, states_out=None):
     """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
     With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
     single-reference range are detected on the device and recomputed exactly; ``return_flags``
-    also returns the int32 ``[chunks, H]`` flags (for the backward pass)."""
+    also returns the int32 ``[chunks, H]`` flags (for the backward pass).  With a list
+    ``states_out`` the launch also writes the state entering every chunk (transposed fragment
+    order, what the backward kernels read) and appends it."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
@@ -71,24 +80,30 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         chunks = plan.NT if plan is not None else B * (-(-T // BT))
         wide = q.new_empty(chunks, H, dtype=torch.int32)
         hwide = q.new_empty(chunks, H, K * V)
-    be.check(be.lib().fla_chunk_gla_fwd_fused(
-        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide),
-        be.ptr(None if plan is None else plan.offsets), be.ptr(None if plan is None else plan.indices),
-        be.ptr(None if plan is None else plan.chunk_offsets), be.ptr(None if plan is None else plan.seq_order),
-        0 if plan is None else plan.NT,
-        be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_fused")
+    tail = (be.ptr(None if plan is None else plan.offsets), be.ptr(None if plan is None else plan.indices),
+            be.ptr(None if plan is None else plan.chunk_offsets), be.ptr(None if plan is None else plan.seq_order),
+            0 if plan is None else plan.NT,
+            be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q))
+    head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide))
+    if states_out is not None:
+        hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
+        be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
+        states_out.append(hT)
+    else:
+        be.check(be.lib().fla_chunk_gla_fwd_fused(*head, *tail), "fla_chunk_gla_fwd_fused")
     if return_flags:
         return o, ht, wide
     return o, ht
 
 
 def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, want_A=False, fused=True,
-                 flags_out=None):
+                 flags_out=None, states_out=None):
     """Seq-first forward on 64-aligned head dims.  Returns (o, ht, A); with a list ``flags_out`` the
-    gate-range flags of the fused kernel are appended to it."""
+    gate-range flags of the fused kernel are appended to it, with a list ``states_out`` the per-chunk
+    states it kept for the backward pass."""
     if fused and not want_A and q.shape[-1] in (64, 128):
         o, ht, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets,
-                                          return_flags=True)
+                                          return_flags=True, states_out=states_out)
         if flags_out is not None:
             flags_out.append(wide)
         return o, ht, None
@@ -136,10 +151,10 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
     return g_cumsum, A, h, ht, o
 
 
-def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None):
+def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None, hT=None):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
-    Returns ``(dq, dk, dv, dg, dh0)``; recomputes the per-chunk states as the
-    reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``wide``: the forward's
+    Returns ``(dq, dk, dv, dg, dh0)``; without ``hT`` (the states a forward pass kept) it
+    recomputes the per-chunk states as the reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``wide``: the forward's
     gate-range flags (int32 ``[chunks, H]``); flagged chunks get their intra-chunk terms
     from the exact kernel.  Without it the result is exact only while the chunk-cumulative
     log-gate stays within +-80."""
@@ -151,9 +166,10 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     V = v.shape[-1]
     N = B if plan is None else plan.N
     NT = 0 if plan is None else plan.NT
-    hT, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=False,
-                        offsets=offs, indices=idx, head_first=False, chunk_size=BT, gates_are_cumsum=False,
-                        fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
+    if hT is None:
+        hT, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=False,
+                            offsets=offs, indices=idx, head_first=False, chunk_size=BT, gates_are_cumsum=False,
+                            fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
     total_chunks = hT.shape[0] * hT.shape[1]
     dhf, dhtf = torch.empty_like(hT), torch.empty_like(hT)
     hdh = q.new_empty(V // 32, total_chunks, H, K, dtype=torch.float32)
@@ -210,10 +226,12 @@ class ChunkGLAFunction(torch.autograd.Function):
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
         flags = []
-        o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets, flags_out=flags)
-        # like the reference, keep the inputs and recompute everything else in backward (plus the
-        # small table of chunks whose gates need the exact intra-chunk arithmetic)
-        ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None)
+        states = [] if KEEP_STATES_FOR_BACKWARD and any(ctx.needs_input_grad) else None
+        o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets, flags_out=flags,
+                                states_out=states)
+        # the inputs, the small table of chunks whose gates need the exact intra-chunk arithmetic, and
+        # (unless recomputation is asked for) the per-chunk states the fused launch wrote on its way
+        ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None, states[0] if states else None)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
@@ -228,7 +246,7 @@ class ChunkGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        q, k, v, g, h0, offsets, wide = ctx.saved_tensors
+        q, k, v, g, h0, offsets, wide, hT = ctx.saved_tensors
         K, V, KP, VP = ctx.dims
         if ctx.head_first:
             do = do.transpose(1, 2)
@@ -238,7 +256,7 @@ class ChunkGLAFunction(torch.autograd.Function):
         do = do.contiguous()
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
-        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide, hT=hT)
         if (KP, VP) != (K, V):
             dq, dk, dg, dv = dq[..., :K], dk[..., :K], dg[..., :K], dv[..., :V]
             if dh0 is not None:

@@ -299,3 +299,26 @@ def test_chunk_gla_reference_ladder(device, D, T, normalizer, head_first):
     for name, a, b in zip(("dq", "dk", "dv", "dg"), refs, leaves):
         assert_close(name, a.grad, tr(b.grad), 1e-2)
     assert_close("dh0", rh0.grad, h0l.grad, 1e-2)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_keep_vs_recompute(device, varlen, monkeypatch):
+    """The backward from the states the fused forward kept and the reference-style backward that
+    recomputes them agree to the rounding of the 16-bit states; both meet the oracle's tolerances
+    (the default, state-keeping mode is what every other backward test exercises)."""
+    import fla_amd.ops.gla.chunk as mod
+    gen = torch.Generator().manual_seed(13)
+    T, N, H, D = 400, 3, 2, 128
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q, k, v, g, h0 = gla_inputs(1 if varlen else 2, T, H, D, D, seed=64, N=N if varlen else None, h0_std=1.0)
+    do = torch.randn(q.shape[0], T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    print(f"chunk_gla keep vs recompute varlen={varlen}", flush=True)
+    assert mod.KEEP_STATES_FOR_BACKWARD
+    kept = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    monkeypatch.setattr(mod, "KEEP_STATES_FOR_BACKWARD", False)
+    rec = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    ref = _grads_ref(q, k, v, g, h0, do, dht, offsets=None if offs is None else offs.tolist())
+    for name, a, b, r, tol in zip(("dq", "dk", "dv", "dg", "dh0"), kept, rec, ref, (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(f"{name} kept vs recomputed", b, a, 2e-3)
+        assert_close(f"{name} recomputed vs oracle", r, b, tol)
