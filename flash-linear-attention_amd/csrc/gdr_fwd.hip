@@ -158,7 +158,7 @@ FLA_DEVICE void wy_stage_t(T* dstT, const typename Elem<T>::v4* reg, const float
 // k and v stay in registers from the initial load until their transposed,
 // beta-scaled tiles are written.
 template <typename T, int K, int V>
-__global__ __launch_bounds__(256, 4) void gdr_fwd_wy_kernel(WyParams p) {
+__global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
