@@ -524,9 +524,13 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H, K = p.K;
-  const int kb = blockIdx.z * 64;
+  // The key slices of one (chunk, head) share do, v_new and dv2: they get consecutive logical
+  // ids on the same XCD, so the second slice finds those tiles in that XCD's L2.
+  const int nz = K / 64;
+  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kb = (int)(lid % nz) * 64;
   int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  ChunkLoc cl = locate_chunk_at(lid / nz, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -733,7 +737,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
       if (row < L) {
         float val = rowsum[i];
         if (row == L - 1) val += kin_all + __expf(glast) * hd_all;
-        p.dgam[((int64_t)blockIdx.z * p.total_rows + row0 + row) * H + hh] = val;
+        p.dgam[((int64_t)(kb / 64) * p.total_rows + row0 + row) * H + hh] = val;
       }
     }
   }
@@ -1133,7 +1137,9 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   {
     DqkwgParams p{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
                   B * T_, (int)H, (int)K, ntfix, scale};
-    dim3 g3(grid.x, grid.y, (unsigned)(K / 64));
+    const int64_t nwg = (int64_t)grid.x * grid.y * (K / 64);
+    FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+    dim3 g3((unsigned)nwg);
     if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p);
     else hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p);
     FLA_CHECK_LAUNCH();
