@@ -489,9 +489,13 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H, K = p.K;
-  const int kb = blockIdx.z * 64;
+  // The key slices of one (chunk, head) share v and do: they get consecutive logical ids on the
+  // same XCD, so the second slice finds those tiles in that XCD's L2.
+  const int nz = K / 64;
+  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int kb = (int)(lid % nz) * 64;
   int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  ChunkLoc cl = locate_chunk_at(lid / nz, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -938,7 +942,9 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   {
     BDqkgParams p{q, k, v, g, dout, hT, dhtf, hdh, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
                   (int)H, (int)K, ntfix, scale};
-    dim3 g3(grid.x, grid.y, (unsigned)(K / 64));
+    const int64_t nwg = (int64_t)grid.x * grid.y * (K / 64);
+    FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+    dim3 g3((unsigned)nwg);
     if (V == 64) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 64>), g3, dim3(256), 0, st, p);
     else if (V == 128) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 128>), g3, dim3(256), 0, st, p);
     else return FLA_E_UNSUPPORTED;
