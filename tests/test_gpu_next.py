@@ -202,3 +202,41 @@ def test_chunk_gdr_keys_above_256_refused(device):
     dev = _dev(device)
     with pytest.raises(NotImplementedError):
         chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), head_first=False)
+
+
+@pytest.mark.parametrize("op", ["gla", "gdr"])
+def test_packed_batch_with_empty_sequence(device, op):
+    """A packed batch may contain a sequence of length zero: it has no chunks, its final state is its
+    initial state and the gradient of that state passes straight through."""
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_amd.ops.gla import chunk_gla
+    from oracle.recurrent import naive_recurrent_gated_delta_rule, naive_recurrent_gla
+    T, H, D = 200, 2, 128
+    offs = torch.tensor([0, 70, 70, 199, 200])          # the second sequence is empty, the last has one token
+    N = 4
+    gen = torch.Generator().manual_seed(21)
+    do = torch.randn(1, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(N, H, D, D, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"packed batch with an empty sequence: {op}", flush=True)
+    if op == "gla":
+        q, k, v, g, h0 = gla_inputs(1, T, H, D, D, seed=22, N=N, h0_std=1.0)
+        cpu, fn, naive = (q, k, v, g), chunk_gla, naive_recurrent_gla
+    else:
+        q, k, v, g, beta, h0 = gdr_inputs(1, T, H, D, D, seed=22, N=N, h0_std=1.0)
+        cpu, fn, naive = (q, k, v, g, beta), chunk_gated_delta_rule, naive_recurrent_gated_delta_rule
+    leaves = [dev(x).requires_grad_() for x in cpu]
+    h0l = dev(h0).requires_grad_()
+    o, ht = fn(*leaves, initial_state=h0l, output_final_state=True, offsets=dev(offs), head_first=False)
+    ((o.float() * dev(do).float()).sum() + (ht * dev(dht)).sum()).backward()
+    torch.cuda.synchronize()
+    refs = [x.float().requires_grad_() for x in cpu]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive(*refs, initial_state=rh0, output_final_state=True, offsets=offs.tolist())
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    assert torch.equal(ht[1].cpu(), h0[1]) and torch.equal(h0l.grad[1].cpu(), dht[1])
+    for name, a, b in zip(("dq", "dk", "dv", "dg", "dbeta"), refs, leaves):
+        assert_close(name, a.grad, b.grad, 2e-2)
+    assert_close("dh0", rh0.grad, h0l.grad, 1e-2)
