@@ -280,6 +280,17 @@ def bench_backward(device, steps=10):
     return out
 
 
+def bench_copy(device, steps=20):
+    """The runtime's device-to-device copy of 1 GiB (1 GiB read + 1 GiB written): what a pure stream of
+    this size reaches on the box, beside the 8 TB/s the roofline fractions are quoted against."""
+    import torch
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    dst = torch.empty_like(src)
+    us = event_avg_us(lambda: dst.copy_(src), steps)
+    return {"us": round(us, 1), "GBs": round(2 * (1 << 30) / us / 1e3, 1),
+            "frac_of_hbm_peak": round(2 * (1 << 30) / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+
 def bench_layer_steps(device, steps=20):
     """The row-wise steps either side of the operators at the operators' benchmark shape
     (B=8, T=4096, H=16, D=128; the convolution on 2048 channels, kernel 4): device time of each
@@ -381,6 +392,7 @@ def main():
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
         extra["layer_steps"] = bench_layer_steps(device)
+        extra["device_copy_1GiB"] = bench_copy(device)
     out = {
         "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
