@@ -396,7 +396,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     };
     publish_state();
-    if (nchunks > 0) store_ht(0);
     // The matrix waves also stage the value tile (time-contiguous) of the next chunk: 8 rows x
     // 2 columns per lane, loaded one chunk period ahead.
     const int vrg = tid >> 5, vc = (tid & 31) * 2;
@@ -442,6 +441,12 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     for (int64_t c = 0; c < nchunks; ++c) {
       const int buf = (int)(c & 1);
       lds_barrier();  // B1(c)
+      // the next chunk's values first: the wait for their loads then covers no store issued after them
+      if (c + 1 < nchunks) {
+        stage_v(buf ^ 1, c + 1);
+        load_v();
+      }
+      store_ht(c);  // unconditional and a whole chunk period ahead of the next wait for the value loads
       if (p.wide) {
         int wide = 0;
 #pragma unroll
@@ -457,10 +462,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
             *(v8*)(hw + (((int64_t)kt * (V / 32) + (vbase / 32 + vt)) * 64 + ln) * 16 + piece * 8) = x;
           }
         }
-      }
-      if (c + 1 < nchunks) {
-        stage_v(buf ^ 1, c + 1);
-        load_v();
       }
       // ---- scores on the lower-triangular quadrants and the inter-chunk part of o
       const int qi = wave >> 1, qj = wave & 1;
@@ -562,7 +563,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
       publish_state();
-      if (c + 1 < nchunks) store_ht(c + 1);
     }
     if (nchunks > 0) lds_barrier();  // hands the last output tile to the staging waves
     if (p.ht) {
