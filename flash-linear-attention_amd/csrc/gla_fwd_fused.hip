@@ -275,23 +275,28 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     constexpr int NPO = BT * (BV / 8) / (64 * NSTG);
     const uint32_t opitch = (uint32_t)H * V * (uint32_t)sizeof(T);
     uint32_t offo[NPO];
-    int ldo[NPO], orow[NPO];
+    int ldo[NPO];
+    const int ocol = (tid & 7) * 8;   // element offset inside a row: the same for every piece of a lane
 #pragma unroll
     for (int i = 0; i < NPO; ++i) {
-      const int e = (tid - 256) + 64 * NSTG * i;
-      orow[i] = e >> 3;
-      ldo[i] = orow[i] * LDT + (e & 7) * 8;
-      offo[i] = (uint32_t)orow[i] * opitch + (uint32_t)((e & 7) * 8) * (uint32_t)sizeof(T);
+      const int orow = ((tid - 256) + 64 * NSTG * i) >> 3;
+      ldo[i] = orow * LDT + ocol;
+      offo[i] = (uint32_t)orow * opitch + (uint32_t)ocol * (uint32_t)sizeof(T);
     }
     char* po = (char*)p.o + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
     const int64_t stro = (int64_t)BT * opitch;
     int64_t oc = 0;  // chunk whose output tile is stored next
+    // Rows past the end of a short last chunk are redirected to its last row (LDS source and
+    // destination alike, so the duplicates rewrite the same bytes): the stores stay unconditional
+    // and the compiler's wait counts around them exact.
     auto store_o = [&]() __attribute__((always_inline)) {
       const int Lc = oc == nchunks - 1 ? Llast : BT;
 #pragma unroll
       for (int i = 0; i < NPO; ++i) {
-        const v8 x = *(const v8*)&sO[ldo[i]];
-        if (orow[i] < Lc) *(v8*)(po + offo[i]) = x;
+        const int ls = min(ldo[i], (Lc - 1) * LDT + ocol);
+        const uint32_t os = min(offo[i], (uint32_t)(Lc - 1) * opitch + (uint32_t)ocol * (uint32_t)sizeof(T));
+        const v8 x = *(const v8*)&sO[ls];
+        *(v8*)(po + os) = x;
       }
       po += stro;
       ++oc;
@@ -316,16 +321,33 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
       end_loads();
       stage(RA, 0, 0, [] {});
-      for (int64_t c = 0; c < nchunks; c += 2) {
-        lds_barrier();  // B1(c): tiles of chunk c and the output tile of chunk c-1 published; buffer 1 is free
-        if (c > 0) store_o();
-        if (c + 1 < nchunks) stage(RB, 1, c + 1, [] { lds_barrier(); });  // contains B2(c)
-        else lds_barrier();  // B2(c)
-        if (c + 1 >= nchunks) break;
-        lds_barrier();  // B1(c+1)
+      // Chunk c: B1(c) publishes its tiles and the output tile of chunk c-1, then the tiles of
+      // chunk c+1 are staged around B2(c).  The steady-state loop runs whole pairs of chunks and
+      // leaves only at its latch (the odd chunk out is handled after it): every path round it
+      // issues the same loads, so the wait counts keep the two register sets two chunk periods
+      // apart instead of waiting for the set that was refilled last.
+      lds_barrier();  // B1(0)
+      if (nchunks > 1) {
+        stage(RB, 1, 1, [] { lds_barrier(); });  // contains B2(0)
+        int64_t c = 1;
+        for (int64_t pairs = (nchunks - 2) >> 1; pairs > 0; --pairs, c += 2) {
+          lds_barrier();  // B1(c), c odd
+          store_o();
+          stage(RA, 0, c + 1, [] { lds_barrier(); });  // contains B2(c)
+          lds_barrier();  // B1(c+1)
+          store_o();
+          stage(RB, 1, c + 2, [] { lds_barrier(); });  // contains B2(c+1)
+        }
+        lds_barrier();  // B1(c)
         store_o();
-        if (c + 2 < nchunks) stage(RA, 0, c + 2, [] { lds_barrier(); });  // contains B2(c+1)
-        else lds_barrier();  // B2(c+1)
+        if (c + 1 < nchunks) {
+          stage(RA, 0, c + 1, [] { lds_barrier(); });  // contains B2(c)
+          lds_barrier();  // B1(c+1)
+          store_o();
+        }
+        lds_barrier();  // B2 of the last chunk
+      } else {
+        lds_barrier();  // B2(0)
       }
       lds_barrier();  // the last output tile is published
       store_o();
