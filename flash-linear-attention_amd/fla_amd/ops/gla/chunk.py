@@ -36,15 +36,74 @@ def _round64(d: int) -> int:
     return -(-d // 64) * 64
 
 
+def _piece_chunk_size(T: int, chunk_size: int) -> int:
+    """The reference's chunk length for a launch over T tokens (``fla/ops/gla/chunk.py:995``)."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd: the chunk kernels are built for chunk_size=64")
+    return min(chunk_size, max(16, 1 << (max(T, 1) - 1).bit_length()))
+
+
+def _piece_k(K: int) -> int:
+    if K > 256:
+        raise NotImplementedError("fla_amd: the chunk-parallel GLA stages are built for K <= 256")
+    return 64 if K <= 64 else 128 if K <= 128 else 256
+
+
+def _seq_first(x: Optional[torch.Tensor], head_first: bool) -> Optional[torch.Tensor]:
+    """[B, H, T|NT, ...] -> [B, T|NT, H, ...] (a copy) for head-first callers."""
+    if x is None or not head_first:
+        return x
+    return x.transpose(1, 2).contiguous()
+
+
+def _pad_state(m: torch.Tensor, Kp: int, Vp: int) -> torch.Tensor:
+    K, V = m.shape[-2:]
+    if (K, V) == (Kp, Vp):
+        return m.contiguous()
+    return F.pad(m, (0, Vp - V, 0, Kp - K)).contiguous()
+
+
+def _check_piece_dtypes(x: torch.Tensor, A: torch.Tensor, m: torch.Tensor, g: torch.Tensor):
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError("fla_amd: q/k/v/do must be bf16 or fp16")
+    for name, t in (("A", A), ("the states", m)):
+        if t.dtype not in (torch.float32, x.dtype):
+            raise NotImplementedError(f"fla_amd: {name} must be fp32 or of the q/k/v dtype")
+    if g.dtype != torch.float32:
+        raise NotImplementedError("fla_amd: the cumulative gates must be fp32")
+
+
+def _chunk_gla_fwd_o_gk_plain(q, v, g, A, h, scale, offsets, indices, head_first, chunk_size):
+    """``chunk_gla_fwd_o_gk`` on the reference's operands (``fla/ops/gla/chunk.py:941-979``):
+    scores ``A`` [B,T,H,BT] and row-major states ``h`` [B,NT,H,K,V] as the caller computed them."""
+    q, v, g, A, h = (_seq_first(t, head_first) for t in (q, v, g, A, h))
+    B, T, H, K = q.shape
+    V = v.shape[-1]
+    bt = _piece_chunk_size(T, chunk_size)
+    _check_piece_dtypes(q, A, h, g)
+    Kp, Vp = _piece_k(K), _round64(V)
+    qp, gp = _pad_dim(q, Kp).contiguous(), _pad_dim(g, Kp).contiguous()
+    vp, Ap, hp = _pad_dim(v, Vp).contiguous(), _pad_dim(A, BT).contiguous(), _pad_state(h, Kp, Vp)
+    NT = 0 if offsets is None else indices.shape[0]
+    o = torch.empty_like(vp)
+    be.check(be.lib().fla_chunk_gla_fwd_o_gk(
+        be.ptr(qp), be.ptr(vp), be.ptr(gp), be.ptr(Ap), be.ptr(hp), be.ptr(o), be.ptr(offsets), be.ptr(indices), NT,
+        be.dt(qp), be.dt(Ap), be.dt(hp), B, T, H, Kp, Vp, float(scale), be.stream_of(q)), "fla_chunk_gla_fwd_o_gk")
+    o = o[..., :V]
+    return o.transpose(1, 2) if head_first else o
+
+
 def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_first=True, chunk_size=64,
                        *, k=None, gates_are_cumsum=True, A_out=None):
-    """Output kernel.  Unlike the reference (``fla/ops/gla/chunk.py:941-979``) the
-    device kernel recomputes the scores from ``q, k, g`` instead of reading ``A``,
-    so ``k`` must be given and ``h`` must be in fragment layout."""
-    if head_first or chunk_size != BT:
-        raise NotImplementedError("fla_amd chunk_gla_fwd_o_gk: seq-first, chunk size 64 only")
+    """Output stage ``o = (scale q e^{g}) h + tril(A) v`` (``fla/ops/gla/chunk.py:941-979``).
+
+    Called as the reference calls it (``k`` not given), ``A`` and the row-major ``h`` are read as
+    they are.  The operator's own pipeline passes ``k=``: the device kernel then recomputes the
+    scores from ``q, k, g`` and takes ``h`` in MFMA-fragment order (seq-first only)."""
     if k is None:
-        raise NotImplementedError("fla_amd chunk_gla_fwd_o_gk: pass k=; scores are recomputed in the kernel")
+        return _chunk_gla_fwd_o_gk_plain(q, v, g, A, h, scale, offsets, indices, head_first, chunk_size)
+    if head_first or chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gla_fwd_o_gk with k=: seq-first, chunk size 64 only")
     B, T, H, K = q.shape
     V = v.shape[-1]
     NT = 0
@@ -56,6 +115,46 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
         be.ptr(offsets), be.ptr(indices), NT, be.dt(q), be.dt(g), B, T, H, K, V, float(scale),
         be.stream_of(q)), "fla_chunk_gla_fwd_o")
     return o
+
+
+def chunk_gla_bwd_dA(v, do, scale, offsets=None, indices=None, head_first=True, chunk_size=64):
+    """``dA = scale tril(do v^T)``, fp32 [B,T,H,BT] (``fla/ops/gla/chunk.py:982-1015``)."""
+    v, do = _seq_first(v, head_first), _seq_first(do, head_first)
+    B, T, H, V = v.shape
+    bt = _piece_chunk_size(T, chunk_size)
+    if v.dtype not in (torch.bfloat16, torch.float16) or do.dtype != v.dtype:
+        raise NotImplementedError("fla_amd chunk_gla_bwd_dA: v and do must both be bf16 or fp16")
+    if V > 256:
+        raise NotImplementedError("fla_amd chunk_gla_bwd_dA: V <= 256")
+    Vp = _piece_k(V)
+    vp, dop = _pad_dim(v, Vp).contiguous(), _pad_dim(do, Vp).contiguous()
+    NT = 0 if offsets is None else indices.shape[0]
+    dA = v.new_empty(B, T, H, BT, dtype=torch.float32)
+    be.check(be.lib().fla_chunk_gla_bwd_dA(
+        be.ptr(vp), be.ptr(dop), be.ptr(dA), be.ptr(offsets), be.ptr(indices), NT, be.dt(vp), B, T, H, Vp,
+        float(scale), be.stream_of(v)), "fla_chunk_gla_bwd_dA")
+    dA = dA[..., :bt]
+    return dA.transpose(1, 2) if head_first else dA
+
+
+def chunk_gla_bwd_dv(k, g, A, do, dh, offsets=None, indices=None, head_first=True, chunk_size=64):
+    """``dv = triu(A^T) do + (k e^{g_last-g}) dh`` with row-major ``dh`` [B,NT,H,K,V]
+    (``fla/ops/gla/chunk.py:1018-1054``)."""
+    k, g, A, do, dh = (_seq_first(t, head_first) for t in (k, g, A, do, dh))
+    B, T, H, K = k.shape
+    V = do.shape[-1]
+    _piece_chunk_size(T, chunk_size)
+    _check_piece_dtypes(k, A, dh, g)
+    Kp, Vp = _piece_k(K), _round64(V)
+    kp, gp = _pad_dim(k, Kp).contiguous(), _pad_dim(g, Kp).contiguous()
+    dop, Ap, dhp = _pad_dim(do, Vp).contiguous(), _pad_dim(A, BT).contiguous(), _pad_state(dh, Kp, Vp)
+    NT = 0 if offsets is None else indices.shape[0]
+    dv = torch.empty_like(dop)
+    be.check(be.lib().fla_chunk_gla_bwd_dv(
+        be.ptr(kp), be.ptr(gp), be.ptr(Ap), be.ptr(dop), be.ptr(dhp), be.ptr(dv), be.ptr(offsets), be.ptr(indices), NT,
+        be.dt(kp), be.dt(Ap), be.dt(dhp), B, T, H, Kp, Vp, be.stream_of(k)), "fla_chunk_gla_bwd_dv")
+    dv = dv[..., :V]
+    return dv.transpose(1, 2) if head_first else dv
 
 
 def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,

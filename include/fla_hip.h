@@ -274,6 +274,35 @@ int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* g
                       float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * The chunk-parallel stages of GLA under the operand layouts of the reference's internal
+ * functions, for sibling operators that bring their own scores and states (RWKV6:
+ * fla/ops/rwkv6/chunk.py:1163, 1227, 1236).  g_cumsum is the fp32 chunk-local prefix sum of the
+ * log-gates [B,T,H,K]; A is [B,T,H,64] (fp32 or the q/k/v dtype, a_dtype); the states h / dh are
+ * row-major [chunks, H, K, V] (fp32 or the q/k/v dtype), chunk index as in `indices` (packed)
+ * or b * ceil(T/64) + c.  K in {64,128,256}, V a multiple of 64 (dA: V in {64,128,256}).
+ *
+ * fla_chunk_gla_fwd_o_gk replaces chunk_gla_fwd_o_gk (fla/ops/gla/chunk.py:941-979, kernel :320-393):
+ *   o = (scale q e^{g}) h + tril(A) v.
+ * fla_chunk_gla_bwd_dA replaces chunk_gla_bwd_dA (fla/ops/gla/chunk.py:982-1015, kernel :582-624):
+ *   dA = scale tril(do v^T), fp32 [B,T,H,64].
+ * fla_chunk_gla_bwd_dv replaces chunk_gla_bwd_dv (fla/ops/gla/chunk.py:1018-1054, kernel :642-710):
+ *   dv = triu(A^T) do + (k e^{g_last - g}) dh, g_last the gate row of the chunk's last token.
+ * ---------------------------------------------------------------------- */
+int fla_chunk_gla_fwd_o_gk(const void* q, const void* v, const float* g_cumsum, const void* A, const void* h,
+                           void* o, const int64_t* offsets, const int64_t* indices, int64_t NT,
+                           int qkv_dtype, int a_dtype, int h_dtype, int64_t B, int64_t T, int64_t H,
+                           int64_t K, int64_t V, float scale, fla_stream_t stream);
+
+int fla_chunk_gla_bwd_dA(const void* v, const void* dout, float* dA, const int64_t* offsets,
+                         const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T,
+                         int64_t H, int64_t V, float scale, fla_stream_t stream);
+
+int fla_chunk_gla_bwd_dv(const void* k, const float* g_cumsum, const void* A, const void* dout,
+                         const void* dh, void* dv, const int64_t* offsets, const int64_t* indices,
+                         int64_t NT, int qkv_dtype, int a_dtype, int dh_dtype, int64_t B, int64_t T,
+                         int64_t H, int64_t K, int64_t V, fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * Chunked gated delta rule backward (chunk size 64), replaces
  * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):
  * chunk_bwd_dv_local (common/chunk_o.py:551), chunk_gated_delta_rule_bwd_dhu

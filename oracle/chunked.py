@@ -25,6 +25,12 @@ No rounding to bf16 anywhere: this is the exact-arithmetic target, so kernel
 intermediates are compared with a tolerance, final outputs against the naive
 recurrences.  Chunks never straddle sequences; tail chunks are short.
 
+The three ``gla_*`` functions at the end restate single stages of the GLA pipeline on the
+operands the reference's internal callers pass (scores ``A`` and row-major per-chunk states):
+``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  They are pinned
+by the recurrence (output stage on ``chunked_gla``'s intermediates) and by autograd through the
+chunk step (dA, dv) in ``tests/test_oracle_pins.py``.
+
 Test infrastructure only.
 """
 from typing import Dict, Optional, Sequence
@@ -144,3 +150,60 @@ def chunked_gated_delta_rule(q, k, v, g, beta, scale=None, initial_state=None, c
         h_all = torch.stack(hs, 0)[None]
     return dict(g_cumsum=gam, Aw=Aw, Au=Au, Aqk=Aqk, w=w, u=u, h=h_all, v_new=v_new, o=o,
                 ht=torch.stack(finals, 0))
+
+
+def _chunk_list(B, T, BT, offsets):
+    """(global chunk index, batch row, first token, end token) in the order the states are stored."""
+    out = []
+    for b, bos, eos in _spans(B, T, offsets):
+        for s, e in _chunks(bos, eos, BT):
+            out.append((len(out), b, s, e))
+    return out
+
+
+def _state_of(m, c, B, offsets):
+    """State of global chunk c from [B, NT, H, K, V] (equal lengths) or [1, NT_total, H, K, V]."""
+    if offsets is None:
+        NT = m.shape[1]
+        return m[c // NT, c % NT]
+    return m[0, c]
+
+
+def gla_fwd_o_gk(q, v, g_cumsum, A, h, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """o_i = (s q_i e^{G_i})^T h_c + sum_{j<=i} A_ij v_j   (fla/ops/gla/chunk.py:353-393)."""
+    q, v, G, A, h = (x.to(dtype) for x in (q, v, g_cumsum, A, h))
+    B, T, H, _ = q.shape
+    o = torch.zeros(B, T, H, v.shape[-1], dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        L = e - s
+        Ac = torch.tril(A[b, s:e, :, :L].permute(1, 0, 2)).permute(1, 0, 2)        # [i, H, j], j <= i
+        o[b, s:e] = (torch.einsum('ihk,hkv->ihv', scale * q[b, s:e] * G[b, s:e].exp(), _state_of(h, c, B, offsets))
+                     + torch.einsum('ihj,jhv->ihv', Ac, v[b, s:e]))
+    return o
+
+
+def gla_bwd_dA(v, do, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """dA_ij = s * (do_i . v_j) for j <= i, else 0   (fla/ops/gla/chunk.py:607-624)."""
+    v, do = v.to(dtype), do.to(dtype)
+    B, T, H, _ = v.shape
+    dA = torch.zeros(B, T, H, chunk_size, dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        L = e - s
+        d = scale * torch.einsum('ihv,jhv->hij', do[b, s:e], v[b, s:e])
+        dA[b, s:e, :, :L] = torch.tril(d).permute(1, 0, 2)
+    return dA
+
+
+def gla_bwd_dv(k, g_cumsum, A, do, dh, chunk_size=64, offsets=None, dtype=torch.float32):
+    """dv_j = sum_{i>=j} A_ij do_i + (k_j e^{G_last-G_j})^T dh_c, dh_c the gradient w.r.t. the state
+    LEAVING chunk c   (fla/ops/gla/chunk.py:681-710)."""
+    k, G, A, do, dh = (x.to(dtype) for x in (k, g_cumsum, A, do, dh))
+    B, T, H, _ = k.shape
+    dv = torch.zeros(B, T, H, do.shape[-1], dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        L = e - s
+        Ac = torch.tril(A[b, s:e, :, :L].permute(1, 0, 2))                          # [H, i, j], j <= i
+        kd = k[b, s:e] * (G[b, e - 1][None] - G[b, s:e]).exp()
+        dv[b, s:e] = (torch.einsum('hij,ihv->jhv', Ac, do[b, s:e])
+                      + torch.einsum('jhk,hkv->jhv', kd, _state_of(dh, c, B, offsets)))
+    return dv

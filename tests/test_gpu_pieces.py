@@ -1,0 +1,146 @@
+"""GPU: the chunk-parallel GLA stages under the reference's internal signatures
+(``chunk_gla_fwd_o_gk``, ``chunk_gla_bwd_dA``, ``chunk_gla_bwd_dv`` of ``fla/ops/gla/chunk.py``,
+called that way by RWKV6) against the fp32 oracle, with the scores ``A`` and the row-major
+per-chunk states supplied by the caller.
+
+Tolerances (rel-L2): 1e-2 on o and dv (bf16 operands of two matrix products), 5e-3 on dA (one
+product, fp32 output)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import assert_close, gla_inputs, random_offsets
+
+pytestmark = pytest.mark.gpu
+
+TOL_O, TOL_DA = 1e-2, 5e-3
+
+
+def _case(B, T, H, K, V, varlen, seed, dtype=torch.bfloat16):
+    from oracle import chunked
+    N = 4
+    offs = random_offsets(T, N, torch.Generator().manual_seed(seed), min_len=1) if varlen else None
+    q, k, v, g, _ = gla_inputs(1 if varlen else B, T, H, K, V, seed=seed, dtype=dtype, h0=False)
+    ol = None if offs is None else offs.tolist()
+    r = chunked.chunked_gla(q, k, v, g, offsets=ol)
+    gen = torch.Generator().manual_seed(seed + 1)
+    do = torch.randn(v.shape, generator=gen).to(dtype)
+    dh = torch.randn(r["h"].shape, generator=gen) * 0.1
+    return dict(q=q, k=k, v=v, g=g, G=r["g_cumsum"].float(), A=r["A"].float(), h=r["h"].float(), o=r["o"], do=do, dh=dh,
+                offs=offs, ol=ol, scale=K ** -0.5)
+
+
+def _plan(offs, device):
+    if offs is None:
+        return None, None
+    from fla_amd.utils import VarlenPlan
+    plan = VarlenPlan(offs.to(device), 64)
+    return plan.offsets, plan.indices
+
+
+SHAPES = [
+    # B, T, H, K, V
+    (2, 256, 3, 128, 128),
+    (2, 200, 2, 64, 64),
+    (1, 300, 2, 128, 64),
+    (2, 130, 2, 256, 256),
+    (2, 150, 2, 100, 50),   # neither a power of two nor a multiple of 64: padded by the wrapper
+    (2, 40, 2, 64, 64),     # shorter than a chunk: the reference shrinks BT to 64 here as well
+    (1, 20, 2, 32, 32),     # BT = 32
+]
+
+
+@pytest.mark.parametrize("B,T,H,K,V", SHAPES)
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("state_dtype", ["fp32", "same"])
+def test_chunk_gla_fwd_o_gk_reference_operands(device, B, T, H, K, V, varlen, state_dtype):
+    from fla_amd.ops.gla.chunk import chunk_gla_fwd_o_gk
+    if varlen and T < 64:
+        pytest.skip("packed case covered at the longer shapes")
+    c = _case(B, T, H, K, V, varlen, seed=T + K)
+    print(f"o_gk B={B} T={T} H={H} K={K} V={V} varlen={varlen} states={state_dtype}", flush=True)
+    offsets, indices = _plan(c["offs"], device)
+    bt = min(64, max(16, 1 << (T - 1).bit_length()))
+    A, h = c["A"][..., :bt], c["h"]
+    if state_dtype == "same":
+        A, h = A.to(c["q"].dtype), h.to(c["q"].dtype)
+    o = chunk_gla_fwd_o_gk(c["q"].to(device), c["v"].to(device), c["G"].to(device), A.to(device), h.to(device),
+                           c["scale"], offsets=offsets, indices=indices, head_first=False, chunk_size=64)
+    torch.cuda.synchronize()
+    assert o.dtype == c["v"].dtype
+    assert_close("o", c["o"], o, TOL_O)
+
+
+@pytest.mark.parametrize("B,T,H,K,V", SHAPES)
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_bwd_dA_and_dv_reference_operands(device, B, T, H, K, V, varlen):
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd_dA, chunk_gla_bwd_dv
+    from oracle import chunked
+    if varlen and T < 64:
+        pytest.skip("packed case covered at the longer shapes")
+    c = _case(B, T, H, K, V, varlen, seed=T + V + 1)
+    print(f"dA/dv B={B} T={T} H={H} K={K} V={V} varlen={varlen}", flush=True)
+    offsets, indices = _plan(c["offs"], device)
+    bt = min(64, max(16, 1 << (T - 1).bit_length()))
+    dA = chunk_gla_bwd_dA(c["v"].to(device), c["do"].to(device), c["scale"], offsets=offsets, indices=indices,
+                          head_first=False, chunk_size=64)
+    dv = chunk_gla_bwd_dv(c["k"].to(device), c["G"].to(device), c["A"][..., :bt].to(device), c["do"].to(device),
+                          c["dh"].to(device), offsets=offsets, indices=indices, head_first=False, chunk_size=64)
+    torch.cuda.synchronize()
+    assert dA.dtype == torch.float32 and dA.shape[-1] == bt and dv.dtype == c["do"].dtype
+    ref_dA = chunked.gla_bwd_dA(c["v"], c["do"], c["scale"], offsets=c["ol"])[..., :bt]
+    ref_dv = chunked.gla_bwd_dv(c["k"], c["G"], c["A"], c["do"], c["dh"], offsets=c["ol"])
+    assert_close("dA", ref_dA, dA, TOL_DA)
+    # nothing above the diagonal, bit for bit
+    pos = torch.arange(T) % 64 if c["offs"] is None else torch.cat(
+        [torch.arange(int(e - s)) % 64 for s, e in zip(c["offs"][:-1], c["offs"][1:])])
+    upper = torch.arange(bt)[None, :] > pos[:, None]
+    assert (dA.cpu()[:, upper.nonzero()[:, 0], :, upper.nonzero()[:, 1]] == 0).all()
+    assert_close("dv", ref_dv, dv, TOL_O)
+
+
+def test_gla_stages_head_first_and_fp16(device):
+    """head_first=True (the reference's default for these functions) and fp16 operands."""
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd_dA, chunk_gla_bwd_dv, chunk_gla_fwd_o_gk
+    from oracle import chunked
+    B, T, H, K, V = 2, 192, 3, 64, 128
+    c = _case(B, T, H, K, V, False, seed=5, dtype=torch.float16)
+    hf = lambda x: x.transpose(1, 2).contiguous().to(device)
+    o = chunk_gla_fwd_o_gk(hf(c["q"]), hf(c["v"]), hf(c["G"]), hf(c["A"]), hf(c["h"]), c["scale"])
+    dA = chunk_gla_bwd_dA(hf(c["v"]), hf(c["do"]), c["scale"])
+    dv = chunk_gla_bwd_dv(hf(c["k"]), hf(c["G"]), hf(c["A"]), hf(c["do"]), hf(c["dh"]))
+    torch.cuda.synchronize()
+    assert o.shape == (B, H, T, V) and dA.shape == (B, H, T, 64) and dv.shape == (B, H, T, V)
+    assert_close("o", c["o"], o.transpose(1, 2), TOL_O)
+    assert_close("dA", chunked.gla_bwd_dA(c["v"], c["do"], c["scale"]), dA.transpose(1, 2), TOL_DA)
+    assert_close("dv", chunked.gla_bwd_dv(c["k"], c["G"], c["A"], c["do"], c["dh"]), dv.transpose(1, 2), TOL_O)
+
+
+def test_gla_stages_compose_with_the_operator(device):
+    """The stages fed with this library's own scores and row-major states reproduce chunk_gla's output,
+    and dv assembled from dA-independent pieces matches chunk_gla's gradient w.r.t. v."""
+    from fla_amd.ops.common.chunk_h import chunk_fwd_h
+    from fla_amd.ops.gla import chunk_gla
+    from fla_amd.ops.gla.chunk import chunk_gla_fwd_o_gk
+    from fla_amd.ops.utils.cumsum import chunk_local_cumsum
+    from oracle import chunked
+    B, T, H, K, V = 2, 512, 4, 128, 128
+    q, k, v, g, _ = gla_inputs(B, T, H, K, V, seed=9, h0=False)
+    q, k, v, g = (x.to(device) for x in (q, k, v, g))
+    o_ref, _ = chunk_gla(q, k, v, g, head_first=False)
+    G = chunk_local_cumsum(g, 64, head_first=False)
+    h, _ = chunk_fwd_h(k, v, None, G, None, None, False, head_first=False, chunk_size=64, states_in_fp32=True)
+    A = chunked.chunked_gla(q.cpu(), k.cpu(), v.cpu(), g.cpu())["A"].to(device)
+    o = chunk_gla_fwd_o_gk(q, v, G, A, h, K ** -0.5, head_first=False)
+    torch.cuda.synchronize()
+    assert_close("o vs chunk_gla", o_ref.float(), o, TOL_O)
+
+
+def test_gla_stage_argument_errors(device):
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd_dA, chunk_gla_fwd_o_gk
+    c = _case(1, 64, 1, 64, 64, False, seed=1)
+    d = lambda x: x.to(device)
+    with pytest.raises(NotImplementedError):
+        chunk_gla_bwd_dA(d(c["v"]), d(c["do"]), 1.0, head_first=False, chunk_size=32)
+    with pytest.raises(NotImplementedError):
+        chunk_gla_fwd_o_gk(d(c["q"]).float(), d(c["v"]), d(c["G"]), d(c["A"]), d(c["h"]), 1.0, head_first=False)

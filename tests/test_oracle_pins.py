@@ -275,3 +275,59 @@ def test_oracle_gradcheck():
     f2 = lambda q, k, v, g, beta, h0: recurrent.naive_recurrent_gated_delta_rule(
         q, k, v, g, beta, initial_state=h0, output_final_state=True, dtype=D)
     assert torch.autograd.gradcheck(f2, (q, k, v, g, beta, h0), atol=1e-6)
+
+
+# ---------------------------------------------------------------- single GLA stages on the reference's internal operands
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_gla_stage_output_on_chunked_intermediates_equals_recurrence(offsets):
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    q, k, v = _rand(B, T, H, K, seed=11), _rand(B, T, H, K, seed=12), _rand(B, T, H, V, seed=13)
+    gk = F.logsigmoid(_rand(B, T, H, K, seed=14))
+    o, _ = recurrent.naive_recurrent_gla(q, k, v, gk, offsets=offsets, dtype=D)
+    r = chunked.chunked_gla(q, k, v, gk, offsets=offsets, dtype=D)
+    # garbage above the diagonal of A must not matter (the stage masks it)
+    A = r['A'] + torch.triu(torch.ones(64, 64, dtype=D), 1)[torch.arange(T) % 64 if offsets is None else _pos_in_chunk(offsets, T)][None, :, None, :]
+    got = chunked.gla_fwd_o_gk(q, v, r['g_cumsum'], A, r['h'], K ** -0.5, offsets=offsets, dtype=D)
+    torch.testing.assert_close(got, o, rtol=1e-10, atol=1e-10)
+
+
+def _pos_in_chunk(offsets, T):
+    pos = torch.zeros(T, dtype=torch.long)
+    for bos, eos in zip(offsets[:-1], offsets[1:]):
+        pos[bos:eos] = torch.arange(eos - bos) % 64
+    return pos
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_gla_stage_gradients_match_autograd_through_the_chunk_step(offsets):
+    """dA and dv are the gradients of  sum(do * o) + sum(dh_next * h_next)  w.r.t. the unscaled scores
+    and v, where o = (s q e^G) h + tril(s S) v and h_next = e^{G_last} h + (k e^{G_last - G})^T v
+    (the chunk step that chunked_gla, pinned against the recurrence, is built from)."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    q, k = _rand(B, T, H, K, seed=21), _rand(B, T, H, K, seed=22)
+    v = _rand(B, T, H, V, seed=23).requires_grad_()
+    G = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, K, seed=24)), 64, offsets=offsets).to(D)
+    S = _rand(B, T, H, 64, seed=25).requires_grad_()
+    do = _rand(B, T, H, V, seed=26)
+    spans = recurrent._spans(B, T, offsets)
+    chunks = [(b, s, min(s + 64, eos)) for b, bos, eos in spans for s in range(bos, eos, 64)]
+    NT = len(chunks)
+    h = _rand(NT, H, K, V, seed=27)
+    dh_next = _rand(NT, H, K, V, seed=28)
+    scale = 0.37
+    loss = 0.
+    for c, (b, s, e) in enumerate(chunks):
+        L = e - s
+        Ac = torch.tril((scale * S[b, s:e, :, :L]).permute(1, 0, 2))                    # [H, i, j]
+        o = (torch.einsum('ihk,hkv->ihv', scale * q[b, s:e] * G[b, s:e].exp(), h[c])
+             + torch.einsum('hij,jhv->ihv', Ac, v[b, s:e]))
+        kd = k[b, s:e] * (G[b, e - 1][None] - G[b, s:e]).exp()
+        h_next = h[c] * G[b, e - 1].exp()[:, :, None] + torch.einsum('jhk,jhv->hkv', kd, v[b, s:e])
+        loss = loss + (do[b, s:e] * o).sum() + (dh_next[c] * h_next).sum()
+    gv, gS = torch.autograd.grad(loss, [v, S])
+    states = dh_next.reshape(B, NT // B, H, K, V) if offsets is None else dh_next[None]
+    dv = chunked.gla_bwd_dv(k, G, (scale * S).detach(), do, states, offsets=offsets, dtype=D)
+    dA = chunked.gla_bwd_dA(v.detach(), do, scale, offsets=offsets, dtype=D)
+    torch.testing.assert_close(dv, gv, rtol=1e-10, atol=1e-10)
+    # autograd leaves the entries of S above the diagonal (and beyond a short chunk) at zero, as dA does
+    torch.testing.assert_close(dA, gS, rtol=1e-10, atol=1e-10)
