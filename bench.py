@@ -337,6 +337,37 @@ def bench_layer_steps(device, steps=20):
     return out
 
 
+def bench_gla_stages(device, steps=20):
+    """The chunk-parallel GLA stages on the reference's internal operands (scores A [B,T,H,64] fp32,
+    row-major fp32 states [B,NT,H,K,V]) at B=4, T=4096, H=16, K=V=128: device time per launch and
+    algorithmic bytes (every operand read once, the result written once)."""
+    import torch
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd_dA, chunk_gla_bwd_dv, chunk_gla_fwd_o_gk
+    B, T, H, K, V = 4, 4096, 16, 128, 128
+    NT = T // 64
+    gen = torch.Generator(device=device).manual_seed(5)
+    q, k = (torch.randn(B, T, H, K, device=device, generator=gen).bfloat16() for _ in range(2))
+    v, do = (torch.randn(B, T, H, V, device=device, generator=gen).bfloat16() for _ in range(2))
+    G = -torch.rand(B, T, H, K, device=device, generator=gen)
+    A = torch.randn(B, T, H, 64, device=device, generator=gen)
+    h = torch.randn(B, NT, H, K, V, device=device, generator=gen)
+    tok = B * T * H
+    b_qk, b_v, b_g, b_a, b_h = tok * K * 2, tok * V * 2, tok * K * 4, tok * 64 * 4, h.numel() * 4
+    out = {}
+
+    def rec(name, fn, nbytes):
+        us = event_avg_us(fn, steps)
+        out[name] = {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+
+    rec("chunk_gla_fwd_o_gk", lambda: chunk_gla_fwd_o_gk(q, v, G, A, h, K ** -0.5, head_first=False),
+        b_qk + b_g + b_a + b_h + 2 * b_v)
+    rec("chunk_gla_bwd_dA", lambda: chunk_gla_bwd_dA(v, do, K ** -0.5, head_first=False), 2 * b_v + b_a)
+    rec("chunk_gla_bwd_dv", lambda: chunk_gla_bwd_dv(k, G, A, do, h, head_first=False),
+        b_qk + b_g + b_a + b_h + 2 * b_v)
+    return out
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -392,6 +423,7 @@ def main():
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
         extra["layer_steps"] = bench_layer_steps(device)
+        extra["gla_stages_reference_operands"] = bench_gla_stages(device)
         extra["device_copy_1GiB"] = bench_copy(device)
     out = {
         "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
