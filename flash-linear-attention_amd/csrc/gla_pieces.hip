@@ -6,6 +6,7 @@
 //   fla_chunk_gla_fwd_o_gk : o  = (s q e^{g}) h + tril(A) v            fla/ops/gla/chunk.py:320-393
 //   fla_chunk_gla_bwd_dA   : dA = s tril(do v^T)                       fla/ops/gla/chunk.py:582-624
 //   fla_chunk_gla_bwd_dv   : dv = triu(A^T) do + (k e^{g_last-g}) dh   fla/ops/gla/chunk.py:642-710
+//   fla_chunk_bwd_dh       : the reverse state scan with row-major dh  fla/ops/common/chunk_h.py:146-262
 //
 // The operator's own forward and backward never take this route (they keep the states in MFMA
 // fragment order and recompute A on the fly); these are one workgroup per (chunk, head[, 64 value
@@ -244,6 +245,115 @@ __global__ __launch_bounds__(256) void gla_bwd_dA_kernel(DAParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Reverse state scan with row-major output (chunk_bwd_kernel_dh, fla/ops/common/chunk_h.py:146-262):
+// for c = last .. 0:  store dh_c;  dh <- e^{g_last} diag(e^{gk_last}) dh + (s q e^{g} e^{gk})^T do.
+// One workgroup per (sequence, head, 64 key channels x 64 value columns), serial over chunks.
+struct RowDhParams {
+  const void* q;
+  const float* g;     // [B*T, H] or null
+  const float* gk;    // [B*T, H, K] or null
+  const void* dout;
+  const float* dht;   // [N, H, K, V] or null
+  void* dh;           // [chunks, H, K, V]
+  float* dh0;         // [N, H, K, V] or null
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int H, K, V;
+  float scale;
+  int dh_is_f32;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void chunk_bwd_dh_rowmajor_kernel(RowDhParams p) {
+  __shared__ __attribute__((aligned(16))) T sQt[64 * LDT];   // [k][t]
+  __shared__ __attribute__((aligned(16))) T sDt[64 * LDT];   // [v][t]
+  __shared__ float sDecay[64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, V = p.V;
+  const int nv = V / 64;
+  const int kbase = (blockIdx.x / nv) * 64, vbase = (blockIdx.x % nv) * 64;
+  const int n = blockIdx.y / H, hh = blockIdx.y % H;
+  const SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t boh = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+  const int kq = wave >> 1, vq = wave & 1;
+  const int vcol = vbase + vq * 32 + (lane & 31);
+  f32x16 acc = zero16();
+  if (p.dht) {
+    const float* s = p.dht + ((int64_t)n * H + hh) * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = s[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
+  }
+  const int tp = tid >> 3, c8 = (tid & 7) * 8;
+  for (int64_t c = nchunks - 1; c >= 0; --c) {
+    const int64_t row0 = sp.bos + c * BT;
+    const int L = (int)(sp.len - c * BT < BT ? sp.len - c * BT : BT);
+    {
+      const int64_t base = ((boh + c) * H + hh) * (int64_t)K * V;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t idx = base + (int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol;
+        if (p.dh_is_f32) ((float*)p.dh)[idx] = acc[r];
+        else ((T*)p.dh)[idx] = (T)acc[r];
+      }
+    }
+    // q~^T and do^T, two rows x 8 columns per thread, written as (t, t+1) pairs
+    float qa[8], qb[8], da[8], db[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qa[e] = qb[e] = da[e] = db[e] = 0.f;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int t = 2 * tp + half;
+      if (t < L) {
+        float* qo = half ? qb : qa;
+        float* dd = half ? db : da;
+        const int64_t tok = (row0 + t) * H + hh;
+        Load<T>::x4((const T*)p.q + tok * K + kbase + c8, qo);
+        Load<T>::x4((const T*)p.q + tok * K + kbase + c8 + 4, qo + 4);
+        Load<T>::x4((const T*)p.dout + tok * V + vbase + c8, dd);
+        Load<T>::x4((const T*)p.dout + tok * V + vbase + c8 + 4, dd + 4);
+        float gs = p.scale;
+        if (p.g) gs *= __expf(p.g[tok]);
+        float gv[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) gv[e] = 0.f;
+        if (p.gk) {
+          Load<float>::x4(p.gk + tok * K + kbase + c8, gv);
+          Load<float>::x4(p.gk + tok * K + kbase + c8 + 4, gv + 4);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qo[e] *= gs * __expf(gv[e]);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      store_pair<T>(&sQt[(c8 + e) * LDT + 2 * tp], qa[e], qb[e]);
+      store_pair<T>(&sDt[(c8 + e) * LDT + 2 * tp], da[e], db[e]);
+    }
+    if (tid < 64) {
+      const int64_t tok = (row0 + L - 1) * H + hh;
+      float d = p.g ? p.g[tok] : 0.f;
+      if (p.gk) d += p.gk[tok * K + kbase + tid];
+      sDecay[tid] = __expf(d);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] *= sDecay[kq * 32 + c32_row(r, lane)];
+#pragma unroll
+    for (int s = 0; s < BT; s += 16)
+      acc = Elem<T>::mfma32(lds_frag32<T>(sQt, LDT, kq * 32, s, lane), lds_frag32<T>(sDt, LDT, vq * 32, s, lane), acc);
+    __syncthreads();
+  }
+  if (p.dh0) {
+    float* o = p.dh0 + ((int64_t)n * H + hh) * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc[r];
+  }
+}
+
+
 template <typename T, bool DV>
 int launch_piece(const PieceParams& p, int K, dim3 grid, hipStream_t stream) {
   switch (K) {
@@ -332,4 +442,27 @@ extern "C" int fla_chunk_gla_bwd_dA(const void* v, const void* dout, float* dA, 
   if (qkv_dtype == FLA_BF16) return launch_dA<bf16>(p, (int)V, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_dA<f16>(p, (int)V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, const void* dout, const float* dht,
+                                void* dh, float* dh0, const int64_t* offsets, const int64_t* chunk_offsets,
+                                int qkv_dtype, int dh_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                int64_t N, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q && dout && dh, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 64 == 0 && V % 64 == 0, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)gk | (uintptr_t)dout | (uintptr_t)dh) % 16 == 0, FLA_E_ALIGNMENT);
+  const int64_t tiles = (K / 64) * (V / 64);
+  FLA_REQUIRE(tiles <= 0x7fffffffLL && N * H <= 65535, FLA_E_UNSUPPORTED);
+  if (N == 0 || T == 0) return FLA_OK;
+  RowDhParams p{q, g, gk, dout, dht, dh, dh0, offsets, chunk_offsets, T, (int)H, (int)K, (int)V, scale, 0};
+  int rc = is_f32_code(dh_dtype, qkv_dtype, &p.dh_is_f32);
+  if (rc) return rc;
+  dim3 grid((unsigned)tiles, (unsigned)(N * H));
+  if (qkv_dtype == FLA_BF16) chunk_bwd_dh_rowmajor_kernel<bf16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+  else if (qkv_dtype == FLA_F16) chunk_bwd_dh_rowmajor_kernel<f16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
 }

@@ -302,6 +302,18 @@ int fla_chunk_gla_bwd_dv(const void* k, const float* g_cumsum, const void* A, co
                          int64_t NT, int qkv_dtype, int a_dtype, int dh_dtype, int64_t B, int64_t T,
                          int64_t H, int64_t K, int64_t V, fla_stream_t stream);
 
+/* Reverse state scan with row-major output, replaces chunk_bwd_dh for per-head (g, fp32 [B,T,H]) and / or
+ * per-key (gk, fp32 [B,T,H,K]) chunk-cumulative log-gates, either may be NULL
+ * (fla/ops/common/chunk_h.py:338-410, kernel :146-262):
+ *   for c = last .. 0:  dh[c] <- dH;  dH <- e^{g_last} diag(e^{gk_last}) dH + (scale q e^{g} e^{gk})^T do,
+ * starting from dht (fp32 [N,H,K,V] or NULL = 0); dh [chunks,H,K,V] (fp32 or the q/k/v dtype, dh_dtype) is the
+ * gradient w.r.t. the state LEAVING each chunk, dh0 (fp32 [N,H,K,V] or NULL) what is left after chunk 0.
+ * K and V multiples of 64; packed batches need chunk_offsets [N+1].  q and do have as many heads as the gates. */
+int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, const void* dout, const float* dht,
+                     void* dh, float* dh0, const int64_t* offsets, const int64_t* chunk_offsets,
+                     int qkv_dtype, int dh_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                     int64_t N, float scale, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Chunked gated delta rule backward (chunk size 64), replaces
  * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):

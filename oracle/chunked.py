@@ -27,9 +27,10 @@ recurrences.  Chunks never straddle sequences; tail chunks are short.
 
 The three ``gla_*`` functions at the end restate single stages of the GLA pipeline on the
 operands the reference's internal callers pass (scores ``A`` and row-major per-chunk states):
-``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  They are pinned
+``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  ``chunk_bwd_dh`` restates the reverse
+state scan of ``fla/ops/common/chunk_h.py:146-262``.  They are pinned
 by the recurrence (output stage on ``chunked_gla``'s intermediates) and by autograd through the
-chunk step (dA, dv) in ``tests/test_oracle_pins.py``.
+chunk step (dA, dv, dh) in ``tests/test_oracle_pins.py``.
 
 Test infrastructure only.
 """
@@ -207,3 +208,37 @@ def gla_bwd_dv(k, g_cumsum, A, do, dh, chunk_size=64, offsets=None, dtype=torch.
         dv[b, s:e] = (torch.einsum('hij,ihv->jhv', Ac, do[b, s:e])
                       + torch.einsum('jhk,hkv->jhv', kd, _state_of(dh, c, B, offsets)))
     return dv
+
+
+def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """For c = last .. 0:  dh[c] = dH;  dH = e^{g_last} diag(e^{gk_last}) dH + (s q e^{g} e^{gk})^T do, from dH = dht.
+    g [B,T,H] and gk [B,T,H,K] are chunk-cumulative log-gates, either may be None.  Returns dh in the
+    storage order of the states ([B,NT,H,K,V] / [1,NT_total,H,K,V]) and dh0 [N,H,K,V]
+    (fla/ops/common/chunk_h.py:202-262)."""
+    q, do = q.to(dtype), do.to(dtype)
+    B, T, H, K = q.shape
+    V = do.shape[-1]
+    spans = _spans(B, T, offsets)
+    out, dh0 = [], []
+    for n, (b, bos, eos) in enumerate(spans):
+        dH = torch.zeros(H, K, V, dtype=dtype) if dht is None else dht[n].to(dtype).clone()
+        seq = []
+        for s, e in reversed(_chunks(bos, eos, chunk_size)):
+            seq.append(dH)
+            qt = scale * q[b, s:e]
+            decay = torch.ones(H, K, dtype=dtype)
+            if g is not None:
+                qt = qt * g[b, s:e].to(dtype).exp()[..., None]
+                decay = decay * g[b, e - 1].to(dtype).exp()[:, None]
+            if gk is not None:
+                qt = qt * gk[b, s:e].to(dtype).exp()
+                decay = decay * gk[b, e - 1].to(dtype).exp()
+            dH = dH * decay[:, :, None] + torch.einsum('thk,thv->hkv', qt, do[b, s:e])
+        out.extend(reversed(seq))
+        dh0.append(dH)
+    if offsets is None:
+        NT = -(-T // chunk_size)
+        dh = torch.stack(out, 0).reshape(B, NT, H, K, V) if out else torch.zeros(B, 0, H, K, V, dtype=dtype)
+    else:
+        dh = torch.stack(out, 0)[None]
+    return dh, torch.stack(dh0, 0)

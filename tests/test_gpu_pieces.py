@@ -117,8 +117,8 @@ def test_gla_stages_head_first_and_fp16(device):
 
 
 def test_gla_stages_compose_with_the_operator(device):
-    """The stages fed with this library's own scores and row-major states reproduce chunk_gla's output,
-    and dv assembled from dA-independent pieces matches chunk_gla's gradient w.r.t. v."""
+    """The output stage fed with row-major states from this library's own chunk_fwd_h (and the oracle's
+    scores) reproduces chunk_gla's output."""
     from fla_amd.ops.common.chunk_h import chunk_fwd_h
     from fla_amd.ops.gla import chunk_gla
     from fla_amd.ops.gla.chunk import chunk_gla_fwd_o_gk
@@ -144,3 +144,52 @@ def test_gla_stage_argument_errors(device):
         chunk_gla_bwd_dA(d(c["v"]), d(c["do"]), 1.0, head_first=False, chunk_size=32)
     with pytest.raises(NotImplementedError):
         chunk_gla_fwd_o_gk(d(c["q"]).float(), d(c["v"]), d(c["G"]), d(c["A"]), d(c["h"]), 1.0, head_first=False)
+
+
+# chunk_bwd_dh with the reference's arguments (fla/ops/common/chunk_h.py:338-410): row-major dh, 5e-3 on dh / dh0
+# (bf16 q~ and do operands, fp32 accumulation over the whole sequence)
+@pytest.mark.parametrize("B,T,H,K,V", [(2, 256, 3, 128, 128), (2, 200, 2, 64, 128), (1, 1000, 2, 128, 64),
+                                       (2, 130, 2, 256, 256), (2, 150, 2, 100, 50), (2, 40, 2, 64, 64)])
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("gates", ["gk", "g", "none"])
+def test_chunk_bwd_dh_reference_operands(device, B, T, H, K, V, varlen, gates):
+    from fla_amd.ops.common.chunk_h import chunk_bwd_dh
+    from oracle import chunked, cumsum
+    if varlen and T < 64:
+        pytest.skip("packed case covered at the longer shapes")
+    N = 4 if varlen else B
+    gen = torch.Generator().manual_seed(T + K + V)
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    Bq = 1 if varlen else B
+    ol = None if offs is None else offs.tolist()
+    q = torch.randn(Bq, T, H, K, generator=gen).bfloat16()
+    k = torch.randn(Bq, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(Bq, T, H, V, generator=gen).bfloat16()
+    do = torch.randn(Bq, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(N, H, K, V, generator=gen) * 0.1
+    h0 = torch.zeros(N, H, K, V)
+    gk = cumsum.chunk_local_cumsum(F.logsigmoid(torch.randn(Bq, T, H, K, generator=gen)) / 16, 64, offsets=ol) \
+        if gates == "gk" else None
+    g = cumsum.chunk_local_cumsum(F.logsigmoid(torch.randn(Bq, T, H, generator=gen)), 64, offsets=ol) \
+        if gates == "g" else None
+    print(f"chunk_bwd_dh B={B} T={T} H={H} K={K} V={V} varlen={varlen} gates={gates}", flush=True)
+    d = lambda x: None if x is None else x.to(device)
+    indices = None
+    if varlen:
+        from fla_amd.utils import VarlenPlan
+        indices = VarlenPlan(offs.to(device), 64).indices
+    scale = K ** -0.5
+    for fp32 in (True, False):
+        dh, dh0 = chunk_bwd_dh(d(q), d(k), d(v), d(g), d(gk), None, d(do), d(h0), d(dht), scale, offsets=d(offs),
+                               indices=indices, head_first=False, chunk_size=64, states_in_fp32=fp32)
+        torch.cuda.synchronize()
+        ref_dh, ref_dh0 = chunked.chunk_bwd_dh(q, g, gk, do, dht, scale, offsets=ol)
+        assert dh.dtype == (torch.float32 if fp32 else torch.bfloat16) and dh0.dtype == torch.float32
+        assert_close("dh", ref_dh, dh, 5e-3)
+        assert_close("dh0", ref_dh0, dh0, 5e-3)
+    # without h0 no dh0 comes back, as in the reference; without dht the scan starts from zero
+    dh, none = chunk_bwd_dh(d(q), d(k), d(v), d(g), d(gk), None, d(do), None, None, scale, offsets=d(offs),
+                            indices=indices, head_first=False, states_in_fp32=True)
+    torch.cuda.synchronize()
+    assert none is None
+    assert_close("dh (no dht)", chunked.chunk_bwd_dh(q, g, gk, do, None, scale, offsets=ol)[0], dh, 5e-3)

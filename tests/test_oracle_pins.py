@@ -331,3 +331,43 @@ def test_gla_stage_gradients_match_autograd_through_the_chunk_step(offsets):
     torch.testing.assert_close(dv, gv, rtol=1e-10, atol=1e-10)
     # autograd leaves the entries of S above the diagonal (and beyond a short chunk) at zero, as dA does
     torch.testing.assert_close(dA, gS, rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+@pytest.mark.parametrize("gates", ["gk", "g", "both", "none"])
+def test_chunk_bwd_dh_matches_autograd_through_the_state_chain(offsets, gates):
+    """dh[c] is the gradient of  sum(do * o) + sum(dht * ht)  w.r.t. the state leaving chunk c (taken with a
+    zero tap added to every state), dh0 the one w.r.t. the initial state; only the inter-chunk part of o sees
+    the states:  o = (s q e^{g} e^{gk}) h,  h_next = e^{g_last + gk_last} h + (k e^{g_last - g + gk_last - gk})^T v."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q, k, v = _rand(B, T, H, K, seed=31), _rand(B, T, H, K, seed=32), _rand(B, T, H, V, seed=33)
+    gk = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, K, seed=34)), 64, offsets=offsets).to(D)
+    g = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, seed=35)), 64, offsets=offsets).to(D)
+    if gates in ("g", "none"):
+        gk = None
+    if gates in ("gk", "none"):
+        g = None
+    do, dht = _rand(B, T, H, V, seed=36), _rand(N, H, K, V, seed=37)
+    h0 = _rand(N, H, K, V, seed=38).requires_grad_()
+    scale = 0.41
+    taps, loss = [], 0.
+    for n, (b, bos, eos) in enumerate(recurrent._spans(B, T, offsets)):
+        h = h0[n]
+        for s in range(bos, eos, 64):
+            e = min(s + 64, eos)
+            lg = torch.zeros(e - s, H, K, dtype=D)
+            if g is not None:
+                lg = lg + g[b, s:e][..., None]
+            if gk is not None:
+                lg = lg + gk[b, s:e]
+            loss = loss + (do[b, s:e] * torch.einsum('thk,hkv->thv', scale * q[b, s:e] * lg.exp(), h)).sum()
+            kd = k[b, s:e] * (lg[-1][None] - lg).exp()
+            tap = torch.zeros(H, K, V, dtype=D, requires_grad=True)
+            taps.append(tap)
+            h = h * lg[-1].exp()[:, :, None] + torch.einsum('thk,thv->hkv', kd, v[b, s:e]) + tap
+        loss = loss + (dht[n] * h).sum()
+    grads = torch.autograd.grad(loss, [h0] + taps)
+    dh, dh0 = chunked.chunk_bwd_dh(q, g, gk, do, dht, scale, offsets=offsets, dtype=D)
+    torch.testing.assert_close(dh0, grads[0], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(dh.reshape(-1, H, K, V), torch.stack(grads[1:], 0), rtol=1e-10, atol=1e-10)
