@@ -35,10 +35,15 @@ def chunk_fwd_h(
     in the reference, unless ``gates_are_cumsum=False`` (raw gates; the prefix
     sum is formed in the kernel).  ``fragment_layout=True`` stores ``h`` in the
     MFMA-fragment order only ``fla_chunk_gla_fwd_o`` understands."""
-    if g is not None or gv is not None:
-        raise NotImplementedError("fla_amd chunk_fwd_h: only per-key gates (gk) are covered")
+    if gv is not None:
+        raise NotImplementedError("fla_amd chunk_fwd_h: value gates (gv) are not covered")
+    if g is not None:
+        # per-head gates run on the per-key kernel: the same log-gate on every key channel
+        # (what chunk_simple_gla does at the operator level), added to gk when both are given
+        gb = g.float().unsqueeze(-1).expand(*g.shape, k.shape[-1])
+        gk = gb.contiguous() if gk is None else gk.float() + gb
     if gk is None:
-        raise NotImplementedError("fla_amd chunk_fwd_h: gk is required")
+        raise NotImplementedError("fla_amd chunk_fwd_h: g or gk is required")
     if head_first:
         raise NotImplementedError("fla_amd chunk_fwd_h: seq-first layout only (transpose at the operator boundary)")
     if chunk_size != BT:

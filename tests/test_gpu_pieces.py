@@ -193,3 +193,31 @@ def test_chunk_bwd_dh_reference_operands(device, B, T, H, K, V, varlen, gates):
     torch.cuda.synchronize()
     assert none is None
     assert_close("dh (no dht)", chunked.chunk_bwd_dh(q, g, gk, do, None, scale, offsets=ol)[0], dh, 5e-3)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_fwd_h_per_head_gates_row_major(device, varlen):
+    """chunk_fwd_h(g=...) as chunk_simple_gla's pipeline calls it (fla/ops/simple_gla/chunk.py:33-46):
+    per-head chunk-cumulative gates, row-major fp32 states; 5e-3 on the states."""
+    from fla_amd.ops.common.chunk_h import chunk_fwd_h
+    from oracle import chunked, cumsum
+    B, T, H, K, V, N = (1 if varlen else 2), 300, 3, 128, 64, 3
+    gen = torch.Generator().manual_seed(17)
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    ol = None if offs is None else offs.tolist()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    h0 = torch.randn(N if varlen else B, H, K, V, generator=gen) * 0.1
+    r = chunked.chunked_gla(k, k, v, g[..., None].expand(B, T, H, K), initial_state=h0, offsets=ol)
+    G = cumsum.chunk_local_cumsum(g, 64, offsets=ol)
+    d = lambda x: None if x is None else x.to(device)
+    indices = None
+    if varlen:
+        from fla_amd.utils import VarlenPlan
+        indices = VarlenPlan(offs.to(device), 64).indices
+    h, ht = chunk_fwd_h(d(k), d(v), d(G), None, None, d(h0), True, offsets=d(offs), indices=indices,
+                        head_first=False, chunk_size=64, states_in_fp32=True)
+    torch.cuda.synchronize()
+    assert_close("h", r["h"], h, 5e-3)
+    assert_close("ht", r["ht"], ht, 5e-3)
