@@ -354,6 +354,38 @@ __global__ __launch_bounds__(256) void chunk_bwd_dh_rowmajor_kernel(RowDhParams 
 }
 
 
+// ---------------------------------------------------------------------------
+// Row-major [K, V] state tiles -> MFMA fragment order (FLA_H_FRAGMENT, or FLA_H_FRAGMENT_T with
+// every 32x32 tile transposed), 16-bit: what the output-stage and backward kernels read.  One
+// wave per 32x32 tile; lane l, slot r holds element (32 kt + row(r, l), 32 vt + l % 32) of the
+// tile, row(r, l) = 8 (r / 4) + 4 (l / 32) + r % 4 (the accumulator order of the 32x32 MFMA).
+template <typename T>
+__global__ __launch_bounds__(256) void states_to_fragments_kernel(const void* src, int src_is_f32, T* dst, int K, int V,
+                                                                  int transposed, int64_t total_tiles) {
+  typedef typename Elem<T>::v8 v8;
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= total_tiles) return;
+  const int nkt = K / 32, nvt = V / 32;
+  const int64_t state = tile / (nkt * nvt);
+  const int t = (int)(tile % (nkt * nvt)), kt = t / nvt, vt = t % nvt;
+  const int64_t blk = state * (int64_t)K * V;
+  v8 lo, hi;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int kk = kt * 32 + (transposed ? (lane & 31) : c32_row(r, lane));
+    const int vv = vt * 32 + (transposed ? c32_row(r, lane) : (lane & 31));
+    const int64_t idx = blk + (int64_t)kk * V + vv;
+    const float x = src_is_f32 ? ((const float*)src)[idx] : (float)((const T*)src)[idx];
+    if (r < 8) lo[r] = (T)x;
+    else hi[r - 8] = (T)x;
+  }
+  T* d = dst + blk + ((transposed ? (int64_t)vt * nkt + kt : (int64_t)kt * nvt + vt) * 64 + lane) * 16;
+  *(v8*)d = lo;
+  *(v8*)(d + 8) = hi;
+}
+
+
 template <typename T, bool DV>
 int launch_piece(const PieceParams& p, int K, dim3 grid, hipStream_t stream) {
   switch (K) {
@@ -462,6 +494,30 @@ extern "C" int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, 
   dim3 grid((unsigned)tiles, (unsigned)(N * H));
   if (qkv_dtype == FLA_BF16) chunk_bwd_dh_rowmajor_kernel<bf16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
   else if (qkv_dtype == FLA_F16) chunk_bwd_dh_rowmajor_kernel<f16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+extern "C" int fla_states_to_fragments(const void* h_row_major, void* h_frag, int src_dtype, int dst_dtype,
+                                       int transposed, int64_t n_states, int64_t K, int64_t V, fla_stream_t stream) {
+  FLA_REQUIRE(h_row_major && h_frag && h_row_major != h_frag, FLA_E_INVALID);
+  FLA_REQUIRE(n_states >= 0 && K > 0 && V > 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 32 == 0 && V % 32 == 0, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE((uintptr_t)h_frag % 16 == 0, FLA_E_ALIGNMENT);
+  int src_is_f32;
+  int rc = is_f32_code(src_dtype, dst_dtype, &src_is_f32);
+  if (rc) return rc;
+  const int64_t tiles = n_states * (K / 32) * (V / 32);
+  if (tiles == 0) return FLA_OK;
+  const int64_t blocks = (tiles + 3) / 4;
+  FLA_REQUIRE(blocks <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  if (dst_dtype == FLA_BF16)
+    states_to_fragments_kernel<bf16><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
+        h_row_major, src_is_f32, (bf16*)h_frag, (int)K, (int)V, transposed, tiles);
+  else if (dst_dtype == FLA_F16)
+    states_to_fragments_kernel<f16><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
+        h_row_major, src_is_f32, (f16*)h_frag, (int)K, (int)V, transposed, tiles);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;

@@ -72,7 +72,7 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     h, v_new, final_state = chunk_gated_delta_rule_fwd_h(
         k=k, w=w, u=u, g=g, initial_state=initial_state, output_final_state=output_final_state,
         offsets=offs, indices=idx, head_first=False, chunk_size=BT, fragment_layout=True, chunk_offsets=co)
-    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False,
+    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False, fragment_layout=True,
                     chunk_size=BT)
     return g, o, Aw, Au, final_state
 
@@ -91,7 +91,7 @@ def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, outp
                                       store_A=True, store_Au=False)
     h, hT, v_new, final_state = chunk_gated_delta_rule_fwd_h_both(
         k, w, u, g, initial_state, output_final_state, offsets=offs, indices=idx, chunk_offsets=co)
-    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False,
+    o = chunk_fwd_o(q=q, k=k, v=v_new, h=h, g=g, scale=scale, offsets=offs, indices=idx, head_first=False, fragment_layout=True,
                     chunk_size=BT)
     return g, o, final_state, (w, Aw, v_new, hT)
 

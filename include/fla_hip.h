@@ -314,6 +314,14 @@ int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, const void*
                      int qkv_dtype, int dh_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                      int64_t N, float scale, fla_stream_t stream);
 
+/* Row-major states [n_states, K, V] (fp32 or 16-bit, what chunk_fwd_h and chunk_gated_delta_rule_fwd_h return
+ * in the reference: fla/ops/common/chunk_h.py:303, chunk_delta_h.py:289) re-ordered into FLA_H_FRAGMENT
+ * (transposed == 0) or FLA_H_FRAGMENT_T (== 1) tiles of the 16-bit dst_dtype, for callers that hold the
+ * reference's layout and hand the states to fla_chunk_fwd_o / fla_chunk_gla_fwd_o or a backward entry point.
+ * K and V multiples of 32; not in place. */
+int fla_states_to_fragments(const void* h_row_major, void* h_frag, int src_dtype, int dst_dtype,
+                            int transposed, int64_t n_states, int64_t K, int64_t V, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Chunked gated delta rule backward (chunk size 64), replaces
  * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):

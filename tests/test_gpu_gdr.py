@@ -51,9 +51,13 @@ def test_gdr_kernel_by_kernel(device):
     hf, v_new2, _ = chunk_gated_delta_rule_fwd_h(dev(k), w, u, gc, dev(h0), False, head_first=False,
                                                  fragment_layout=True)
     assert torch.equal(v_new, v_new2)
-    o = chunk_fwd_o(dev(q), dev(k), v_new2, hf, gc, 128 ** -0.5, head_first=False)
+    o = chunk_fwd_o(dev(q), dev(k), v_new2, hf, gc, 128 ** -0.5, head_first=False, fragment_layout=True)
     torch.cuda.synchronize()
     assert_close("o", ref['o'], o, TOL_O)
+    # the reference's calling form: row-major states, re-ordered on the way in
+    o_rm = chunk_fwd_o(dev(q), dev(k), v_new2, h, gc, 128 ** -0.5, head_first=False)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_rm)
     # the fused scan + output launch, fed by the WY launch that also emits the gated scores
     from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_fused
     w2, u2, Aw2, Au2, Aqk = fwd_prepare_wy_repr(dev(k), dev(v), dev(beta), gc, head_first=False, q=dev(q),

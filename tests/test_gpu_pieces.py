@@ -221,3 +221,26 @@ def test_chunk_fwd_h_per_head_gates_row_major(device, varlen):
     torch.cuda.synchronize()
     assert_close("h", r["h"], h, 5e-3)
     assert_close("ht", r["ht"], ht, 5e-3)
+
+
+@pytest.mark.parametrize("K,V", [(128, 128), (64, 128), (128, 64)])
+def test_states_to_fragments_matches_the_scan_kernels_own_layouts(device, K, V):
+    """Row-major states re-ordered by fla_states_to_fragments are bit-identical to what the state scan
+    writes directly in fragment order (both orientations), from fp32 and from 16-bit sources."""
+    from fla_amd.ops.common.chunk_h import chunk_fwd_h
+    from fla_amd.ops.common.chunk_o import states_to_fragments
+    from fla_amd.ops.utils.cumsum import chunk_local_cumsum
+    B, T, H = 2, 300, 3
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=K + V)
+    k, v, g, h0 = (x.to(device) for x in (k, v, g, h0))
+    G = chunk_local_cumsum(g, 64, head_first=False)
+    kw = dict(head_first=False, chunk_size=64)
+    h_rm, _ = chunk_fwd_h(k, v, None, G, None, h0, False, **kw)
+    h_f32, _ = chunk_fwd_h(k, v, None, G, None, h0, False, states_in_fp32=True, **kw)
+    h_fr, _ = chunk_fwd_h(k, v, None, G, None, h0, False, fragment_layout=True, **kw)
+    h_frt, _ = chunk_fwd_h(k, v, None, G, None, h0, False, fragment_layout=True, transposed_fragments=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(states_to_fragments(h_rm, k.dtype), h_fr)
+    assert torch.equal(states_to_fragments(h_rm, k.dtype, transposed=True), h_frt)
+    assert torch.equal(states_to_fragments(h_f32, k.dtype), h_fr)
+    assert torch.equal(states_to_fragments(h_f32, k.dtype, transposed=True), h_frt)
