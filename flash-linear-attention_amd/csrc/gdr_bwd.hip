@@ -1155,7 +1155,43 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   return FLA_OK;
 }
 
+template <typename T>
+int launch_dv_local(const DvlParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
+#define FLA_KV(STMT)                                   \
+  if (K == 64 && V == 64) { STMT(64, 64) }             \
+  else if (K == 128 && V == 128) { STMT(128, 128) }    \
+  else if (K == 64 && V == 128) { STMT(64, 128) }      \
+  else if (K == 128 && V == 64) { STMT(128, 64) }      \
+  else if (K == 256 && V == 64) { STMT(256, 64) }      \
+  else if (K == 256 && V == 128) { STMT(256, 128) }    \
+  else return FLA_E_UNSUPPORTED;
+#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+  FLA_KV(L1)
+#undef L1
+#undef FLA_KV
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
 }  // namespace
+
+extern "C" int fla_chunk_bwd_dv_local(const void* q, const void* k, const float* g_cumsum, const void* dout, void* dv,
+                                      const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                                      int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale,
+                                      fla_stream_t stream) {
+  FLA_REQUIRE(q && k && dout && dv, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)dout | (uintptr_t)dv) % 16 == 0, FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  DvlParams p{q, k, dout, g_cumsum, dv, offsets, indices, T, (int)H, ntfix, scale};
+  if (qkv_dtype == FLA_BF16) return launch_dv_local<bf16>(p, K, V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_dv_local<f16>(p, K, V, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
 
 extern "C" int fla_chunk_gated_delta_rule_bwd(
     const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,

@@ -52,6 +52,7 @@ SIGNATURES = {
     "fla_chunk_gla_bwd_dv": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, P]),
     "fla_chunk_bwd_dh": (c_int, [P] * 9 + [I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_states_to_fragments": (c_int, [P, P, I, I, I, I64, I64, I64, P]),
+    "fla_chunk_bwd_dv_local": (c_int, [P] * 7 + [I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 26 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_l2norm_fwd": (c_int, [P, P, I64, I64, F, I, I, P]),
     "fla_l2norm_bwd": (c_int, [P, P, P, I64, I64, F, I, I, P]),

@@ -62,3 +62,58 @@ def states_to_fragments(h: torch.Tensor, dtype: torch.dtype, transposed: bool = 
         be.ptr(h), be.ptr(out), be.dt(h), be._DTYPES[dtype], int(transposed), h.numel() // (K * V), K, V,
         be.stream_of(h)), "fla_states_to_fragments")
     return out
+
+
+def chunk_bwd_dv_local(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    g: Optional[torch.Tensor],
+    do: torch.Tensor,
+    dh: Optional[torch.Tensor],
+    scale: float,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+    chunk_size: int = 64,
+) -> torch.Tensor:
+    """``dv_j = sum_{i>=j} scale (k_j . q_i) exp(g_i - g_j) do_i`` within each chunk
+    (``fla/ops/common/chunk_o.py:551-599``; ``dh`` is unused there as well).  ``g`` is the chunk-local
+    cumsum ``[B,T,H]`` or ``None``.  Key dims up to 256 (zero-padded to 64 / 128 / 256), value dims in
+    slabs of 128."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_bwd_dv_local: chunk size is fixed to 64")
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or do.dtype != q.dtype:
+        raise NotImplementedError("fla_amd chunk_bwd_dv_local: q, k and do must all be bf16 or all fp16")
+    if head_first:
+        q, k, do = (x.transpose(1, 2) for x in (q, k, do))
+        g = None if g is None else g.transpose(1, 2)
+    be.require_gpu(q, k, do)
+    B, T, H, K = k.shape
+    V = do.shape[-1]
+    if K > 256:
+        raise NotImplementedError("fla_amd chunk_bwd_dv_local: K <= 256")
+    Kp = 64 if K <= 64 else 128 if K <= 128 else 256
+    pad = torch.nn.functional.pad
+    qp = (q if Kp == K else pad(q, (0, Kp - K))).contiguous()
+    kp = (k if Kp == K else pad(k, (0, Kp - K))).contiguous()
+    gp = None if g is None else g.float().contiguous()
+    NT = 0
+    if offsets is not None:
+        if indices is None:
+            from ...utils import VarlenPlan
+            indices = VarlenPlan(offsets, BT).indices
+        NT = indices.shape[0]
+        offsets = offsets.to(torch.int64).contiguous()
+    outs = []
+    for v0 in range(0, V, 128):
+        d = do[..., v0:v0 + 128]
+        w = d.shape[-1]
+        wp = 64 if w <= 64 else 128
+        d = (d if wp == w else pad(d, (0, wp - w))).contiguous()
+        dv = torch.empty_like(d)
+        be.check(be.lib().fla_chunk_bwd_dv_local(
+            be.ptr(qp), be.ptr(kp), be.ptr(gp), be.ptr(d), be.ptr(dv), be.ptr(offsets), be.ptr(indices), NT,
+            be.dt(qp), B, T, H, Kp, wp, float(scale), be.stream_of(q)), "fla_chunk_bwd_dv_local")
+        outs.append(dv[..., :w])
+    dv = outs[0] if len(outs) == 1 else torch.cat(outs, -1)
+    return dv.transpose(1, 2) if head_first else dv

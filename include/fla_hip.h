@@ -322,6 +322,16 @@ int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, const void*
 int fla_states_to_fragments(const void* h_row_major, void* h_frag, int src_dtype, int dst_dtype,
                             int transposed, int64_t n_states, int64_t K, int64_t V, fla_stream_t stream);
 
+/* Intra-chunk part of dv for the operators with a per-head gate, replaces chunk_bwd_dv_local
+ * (fla/ops/common/chunk_o.py:551-599, kernel :379-441):
+ *   dv_j = sum_{i>=j} scale (k_j . q_i) exp(g_i - g_j) do_i  within each chunk,
+ * g_cumsum fp32 [B,T,H] (chunk-local prefix sum) or NULL.  K in {64,128,256}, V in {64,128}.
+ * The first launch of fla_chunk_gated_delta_rule_bwd on its own. */
+int fla_chunk_bwd_dv_local(const void* q, const void* k, const float* g_cumsum, const void* dout, void* dv,
+                           const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                           int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale,
+                           fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Chunked gated delta rule backward (chunk size 64), replaces
  * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):

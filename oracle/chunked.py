@@ -28,7 +28,8 @@ recurrences.  Chunks never straddle sequences; tail chunks are short.
 The three ``gla_*`` functions at the end restate single stages of the GLA pipeline on the
 operands the reference's internal callers pass (scores ``A`` and row-major per-chunk states):
 ``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  ``chunk_bwd_dh`` restates the reverse
-state scan of ``fla/ops/common/chunk_h.py:146-262``.  They are pinned
+state scan of ``fla/ops/common/chunk_h.py:146-262``, ``chunk_bwd_dv_local`` the intra-chunk dv of the
+per-head-gate operators (``fla/ops/common/chunk_o.py:379-441``).  They are pinned
 by the recurrence (output stage on ``chunked_gla``'s intermediates) and by autograd through the
 chunk step (dA, dv, dh) in ``tests/test_oracle_pins.py``.
 
@@ -242,3 +243,19 @@ def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=to
     else:
         dh = torch.stack(out, 0)[None]
     return dh, torch.stack(dh0, 0)
+
+
+def chunk_bwd_dv_local(q, k, g_cumsum, do, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """dv_j = sum_{i>=j} s (k_j . q_i) e^{g_i-g_j} do_i within each chunk; g_cumsum [B,T,H] or None
+    (fla/ops/common/chunk_o.py:419-441)."""
+    q, k, do = q.to(dtype), k.to(dtype), do.to(dtype)
+    B, T, H, _ = k.shape
+    dv = torch.zeros(B, T, H, do.shape[-1], dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        A = scale * torch.einsum('jhk,ihk->hji', k[b, s:e], q[b, s:e])               # [H, j, i]
+        if g_cumsum is not None:
+            gc = g_cumsum[b, s:e].to(dtype)                                           # [L, H]
+            x = gc.t()[:, None, :] - gc.t()[:, :, None]                               # g_i - g_j
+            A = A * torch.where(x <= 0, x.exp(), torch.zeros_like(x))                 # safe_exp (fla/ops/utils/exp.py:9-10)
+        dv[b, s:e] = torch.einsum('hji,ihv->jhv', torch.triu(A), do[b, s:e])
+    return dv

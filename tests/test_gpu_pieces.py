@@ -244,3 +244,30 @@ def test_states_to_fragments_matches_the_scan_kernels_own_layouts(device, K, V):
     assert torch.equal(states_to_fragments(h_rm, k.dtype, transposed=True), h_frt)
     assert torch.equal(states_to_fragments(h_f32, k.dtype), h_fr)
     assert torch.equal(states_to_fragments(h_f32, k.dtype, transposed=True), h_frt)
+
+
+@pytest.mark.parametrize("B,T,H,K,V", [(2, 256, 3, 128, 128), (2, 200, 2, 64, 128), (2, 130, 2, 256, 64),
+                                       (2, 150, 2, 100, 50), (1, 300, 2, 128, 256), (2, 40, 2, 64, 64)])
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("gated", [True, False])
+def test_chunk_bwd_dv_local_reference_operands(device, B, T, H, K, V, varlen, gated):
+    """chunk_bwd_dv_local with the reference's arguments (fla/ops/common/chunk_o.py:551-599); 1e-2 on dv
+    (the scores are rounded to bf16 before the second product, as in the reference)."""
+    from fla_amd.ops.common.chunk_o import chunk_bwd_dv_local
+    from oracle import chunked, cumsum
+    if varlen and T < 64:
+        pytest.skip("packed case covered at the longer shapes")
+    gen = torch.Generator().manual_seed(T + K + V + 3)
+    offs = random_offsets(T, 4, gen, min_len=1) if varlen else None
+    ol = None if offs is None else offs.tolist()
+    Bq = 1 if varlen else B
+    q = torch.randn(Bq, T, H, K, generator=gen).bfloat16()
+    k = torch.randn(Bq, T, H, K, generator=gen).bfloat16()
+    do = torch.randn(Bq, T, H, V, generator=gen).bfloat16()
+    g = cumsum.chunk_local_cumsum(F.logsigmoid(torch.randn(Bq, T, H, generator=gen)), 64, offsets=ol) if gated else None
+    print(f"dv_local B={B} T={T} H={H} K={K} V={V} varlen={varlen} gated={gated}", flush=True)
+    d = lambda x: None if x is None else x.to(device)
+    dv = chunk_bwd_dv_local(d(q), d(k), d(g), d(do), None, K ** -0.5, offsets=d(offs), head_first=False)
+    torch.cuda.synchronize()
+    assert dv.shape == do.shape and dv.dtype == do.dtype
+    assert_close("dv_local", chunked.chunk_bwd_dv_local(q, k, g, do, K ** -0.5, offsets=ol), dv, 1e-2)

@@ -371,3 +371,26 @@ def test_chunk_bwd_dh_matches_autograd_through_the_state_chain(offsets, gates):
     dh, dh0 = chunked.chunk_bwd_dh(q, g, gk, do, dht, scale, offsets=offsets, dtype=D)
     torch.testing.assert_close(dh0, grads[0], rtol=1e-10, atol=1e-10)
     torch.testing.assert_close(dh.reshape(-1, H, K, V), torch.stack(grads[1:], 0), rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+@pytest.mark.parametrize("gated", [True, False])
+def test_chunk_bwd_dv_local_matches_autograd_of_the_intra_chunk_output(offsets, gated):
+    """dv_local is the gradient w.r.t. v of  sum(do * o_intra),  o_intra_i = s sum_{j<=i} (q_i . k_j) e^{g_i-g_j} v_j
+    (the intra-chunk term of chunk_fwd_o, fla/ops/common/chunk_o.py:86-101)."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    q, k = _rand(B, T, H, K, seed=41), _rand(B, T, H, K, seed=42)
+    v = _rand(B, T, H, V, seed=43).requires_grad_()
+    do = _rand(B, T, H, V, seed=44)
+    g = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, seed=45)), 64, offsets=offsets).to(D) if gated else None
+    scale, loss = 0.29, 0.
+    for b, bos, eos in recurrent._spans(B, T, offsets):
+        for s in range(bos, eos, 64):
+            e = min(s + 64, eos)
+            A = scale * torch.einsum('ihk,jhk->hij', q[b, s:e], k[b, s:e])
+            if gated:
+                A = A * (g[b, s:e].t()[:, :, None] - g[b, s:e].t()[:, None, :]).exp()
+            loss = loss + (do[b, s:e] * torch.einsum('hij,jhv->ihv', torch.tril(A), v[b, s:e])).sum()
+    gv, = torch.autograd.grad(loss, [v])
+    got = chunked.chunk_bwd_dv_local(q, k, g, do, scale, offsets=offsets, dtype=D)
+    torch.testing.assert_close(got, gv, rtol=1e-10, atol=1e-10)
