@@ -215,3 +215,43 @@ def test_config4_backward_full_size(device, op):
     g3 = grads((do.float() - 0.5 * do2.float()).bfloat16(), dht - 0.5 * dht2)
     for name, a, c, d in zip(names + ("dh0",), got, g2, g3):
         assert_close(f"linearity {name}", a.float() - 0.5 * c.float(), d, 1.5e-2)
+
+
+def test_config4_row_major_stage_pipeline_reproduces_the_operator(device):
+    """At config 4's size, the stages that take the reference's internal operands (scores A [B,T,H,64],
+    row-major fp32 states) rebuild chunk_gla's output and its gradient w.r.t. v from separately computed
+    pieces: h from chunk_fwd_h, A from the output kernel's A_out, dh from chunk_bwd_dh.  Different kernels,
+    layouts and summation orders on the two sides, so the bar is the bf16 tolerance (1e-2), not equality."""
+    from fla_amd.ops.common.chunk_h import chunk_bwd_dh, chunk_fwd_h
+    from fla_amd.ops.gla import chunk_gla
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd_dA, chunk_gla_bwd_dv, chunk_gla_fwd_o_gk
+    from fla_amd.ops.utils.cumsum import chunk_local_cumsum
+    B, T, H, D = 4, 4096, 16, 128
+    q, k, v, gk, h0 = _config1(device, B=B)
+    gen = torch.Generator(device=device).manual_seed(3)
+    do = torch.randn(B, T, H, D, device=device, generator=gen).bfloat16()
+    dht = torch.randn(B, H, D, D, device=device, generator=gen) * 0.1
+    scale = D ** -0.5
+    print("config 4: row-major stage pipeline vs chunk_gla, B=4 T=4096 H=16 D=128", flush=True)
+    vl = v.clone().requires_grad_()
+    o_ref, ht_ref = chunk_gla(q, k, vl, gk, initial_state=h0, output_final_state=True, head_first=False)
+    torch.autograd.backward((o_ref, ht_ref), (do, dht))
+    kw = dict(head_first=False, chunk_size=64)
+    G = chunk_local_cumsum(gk, 64, head_first=False)
+    h, ht = chunk_fwd_h(k, v, None, G, None, h0, True, states_in_fp32=True, **kw)
+    A = torch.empty(B, T, H, 64, device=device, dtype=torch.float32)
+    h_frag, _ = chunk_fwd_h(k, v, None, G, None, h0, False, fragment_layout=True, **kw)
+    chunk_gla_fwd_o_gk(q, v, G, None, h_frag, scale, k=k, A_out=A, **kw)
+    o = chunk_gla_fwd_o_gk(q, v, G, A, h, scale, **kw)
+    dh, dh0 = chunk_bwd_dh(q, k, v, None, G, None, do, h0, dht, scale, states_in_fp32=True, **kw)
+    dv = chunk_gla_bwd_dv(k, G, A, do, dh, **kw)
+    dA = chunk_gla_bwd_dA(v, do, scale, **kw)
+    torch.cuda.synchronize()
+    assert_close("o", o_ref.float(), o, 1e-2)
+    assert_close("ht", ht_ref, ht, 5e-3)
+    assert_close("dv", vl.grad.float(), dv, 1e-2)
+    # dA against a plain matrix product on one chunk of three (batch, head) pairs
+    for b, hh, c in ((0, 0, 0), (2, 7, 31), (3, 15, 63)):
+        sl = slice(c * 64, c * 64 + 64)
+        ref = torch.tril(do[b, sl, hh].float() @ v[b, sl, hh].float().t()) * scale
+        assert_close(f"dA[{b},{hh},{c}]", ref, dA[b, sl, hh], 5e-3)
