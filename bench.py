@@ -368,6 +368,29 @@ def bench_gla_stages(device, steps=20):
     return out
 
 
+def bench_simple_gla(device, steps=20):
+    """chunk_simple_gla forward (one log-gate per token and head) at config 1's shape: the per-head-gate
+    launch against the same operator through the per-key-gate kernel on a materialised gate tensor."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.ops.gla import chunk_gla
+    from fla_amd.ops.simple_gla import chunk_simple_gla
+    B, T, H, D = 8, 4096, 16, 128
+    gen = torch.Generator(device=device).manual_seed(6)
+    q, k, v = (torch.randn(B, T, H, D, device=device, generator=gen).bfloat16() for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, T, H, device=device, generator=gen))
+    h0 = torch.randn(B, H, D, D, device=device, generator=gen) * 0.1
+    nbytes = 4 * q.numel() * 2 + g.numel() * 4 + 2 * h0.numel() * 4
+    with torch.no_grad():
+        us = event_avg_us(lambda: chunk_simple_gla(q, k, v, g, initial_state=h0, output_final_state=True,
+                                                   head_first=False), steps)
+        us_b = event_avg_us(lambda: chunk_gla(q, k, v, g[..., None].expand(B, T, H, D), initial_state=h0,
+                                              output_final_state=True, head_first=False), steps)
+    return {"us": round(us, 1), "tokens_per_s": round(B * T / us * 1e6, 1), "algorithmic_bytes": nbytes,
+            "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+            "through_per_key_gate_kernel_us": round(us_b, 1)}
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -423,6 +446,7 @@ def main():
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
         extra["layer_steps"] = bench_layer_steps(device)
+        extra["chunk_simple_gla_fwd"] = bench_simple_gla(device)
         extra["gla_stages_reference_operands"] = bench_gla_stages(device)
         extra["device_copy_1GiB"] = bench_copy(device)
     out = {

@@ -69,8 +69,11 @@ FLA_DEVICE typename Elem<T>::v8 frag32_perm_swz(const T* tile, int ld, int row0,
 // HT: the matrix waves keep a transposed copy of their state tiles as well and write the state
 // entering every chunk to p.hT (what the backward kernels contract over v with), for a forward pass
 // whose states are kept instead of being recomputed by the backward pass.
-template <typename T, typename GT, int K, int NSTG, bool HT>
+// SG: one log-gate per (token, head), p.g is fp32 [B*T, H] (the simple-GLA / RetNet-style decay): a lane loads one
+// word per row and uses it for all its key channels, so the prefix sums and exponentials of a row are formed once.
+template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false>
 __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
+  static_assert(!SG || sizeof(GT) == 4, "per-head gates are fp32");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   typedef T t2 __attribute__((ext_vector_type(2)));
@@ -142,18 +145,31 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     const int64_t row00 = (sp.bos * H + hh) * (int64_t)K;
     const char* lq = (const char*)p.q + row00 * (int64_t)sizeof(T);
     const char* lk = (const char*)p.k + row00 * (int64_t)sizeof(T);
-    const char* lg = (const char*)p.g + row00 * (int64_t)sizeof(GT);
+    const char* lg = SG ? (const char*)p.g + (sp.bos * H + hh) * (int64_t)sizeof(float)
+                        : (const char*)p.g + row00 * (int64_t)sizeof(GT);
     const int64_t strk = (int64_t)BT * pitch;
+    const uint32_t gpitch = (uint32_t)H * (uint32_t)sizeof(float);   // SG: row pitch of the gates
+    const int64_t strg = SG ? (int64_t)BT * gpitch : (strk << (sizeof(GT) == 4 ? 1 : 0));
+    uint32_t offg[RPT];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) offg[i] = (uint32_t)(rg * RPT + i) * gpitch;
     const int Llast = (int)(sp.len - (nchunks - 1) * BT);
     const uint32_t lim_full = (uint32_t)(BT - 1) * pitch, lim_last = (uint32_t)(Llast - 1) * pitch;
     int64_t lc = 0;  // chunk the load pointers are on
-    uint32_t lim = 0;
+    uint32_t lim = 0, limg = 0;
     auto begin_loads = [&]() __attribute__((always_inline)) {
       lim = (lc >= nchunks - 1 ? lim_last : lim_full) + (uint32_t)kc * (uint32_t)sizeof(T);
+      if (SG) limg = (uint32_t)((lc >= nchunks - 1 ? Llast : BT) - 1) * gpitch;
     };
     auto load_g = [&](Regs& R, int i) __attribute__((always_inline)) {
-      uint32_t o = offk[i] < lim ? offk[i] : lim;
-      R.g[i] = *(const gvec*)(lg + (o << GSH));
+      if constexpr (SG) {
+        const float x = *(const float*)(lg + (offg[i] < limg ? offg[i] : limg));
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) R.g[i][j] = x;
+      } else {
+        uint32_t o = offk[i] < lim ? offk[i] : lim;
+        R.g[i] = *(const gvec*)(lg + (o << GSH));
+      }
     };
     auto load_qk = [&](Regs& R, int i) __attribute__((always_inline)) {
       uint32_t o = offk[i] < lim ? offk[i] : lim;
@@ -164,7 +180,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       if (lc + 1 < nchunks) {
         lq += strk;
         lk += strk;
-        lg += strk << GSH;
+        lg += strg;
       }
       ++lc;
     };
@@ -198,6 +214,30 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       begin_loads();
       float G[RPT][CPL], glast[CPL];
       float gabs = 0.f;
+      if constexpr (SG) {
+        // one gate per row: a single prefix sum, shared by all key channels of the lane (the
+        // exponentials below then collapse to one pair per row)
+        float run = 0.f, Gs[RPT];
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+          run = fmaf((float)R.g[i][0], LOG2E, run);
+          Gs[i] = run;
+        }
+        const float pre = row_prefix16(run);
+        const float tot = pre - run;
+        const float gl = dpp_f32<0x15f>(pre);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) {
+          Gs[i] += tot;
+          gabs = fmaxf(gabs, fabsf(Gs[i]));
+        }
+#pragma unroll
+        for (int j = 0; j < CPL; ++j) {
+          glast[j] = gl;
+#pragma unroll
+          for (int i = 0; i < RPT; ++i) G[i][j] = Gs[i];
+        }
+      } else
 #pragma unroll
       for (int j = 0; j < CPL; ++j) {
         float run = 0.f;
@@ -622,6 +662,7 @@ struct ExactParams {
   int H, NTfix;
   float scale;
   int64_t total;   // (chunk, head) pairs
+  int head_gates;  // g is fp32 [B*T, H]: one log-gate per (token, head)
 };
 
 template <typename T, typename GT, int K, int V>
@@ -658,7 +699,13 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
     int row = rg * RPT + i;
     if (row < L) {
       int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
-      Load<GT>::x4((const GT*)p.g + off, gq[i]);
+      if (p.head_gates) {
+        const float x = ((const float*)p.g)[(row0 + row) * H + hh];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gq[i][j] = x;
+      } else {
+        Load<GT>::x4((const GT*)p.g + off, gq[i]);
+      }
       qreg[i] = *(const v4*)((const T*)p.q + off);
       kreg[i] = *(const v4*)((const T*)p.k + off);
     } else {
@@ -783,19 +830,19 @@ int launch_exact(const ExactParams& p, int K, int V, dim3 grid, hipStream_t st) 
   return FLA_E_UNSUPPORTED;
 }
 
-template <typename T, typename GT>
+template <typename T, typename GT, bool SG = false>
 int launch_fused(const FusedParams& p, int K, hipStream_t st) {
   int64_t total = (int64_t)(p.V / 64) * p.N * p.H;
   if (total == 0) return FLA_OK;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   dim3 grid((unsigned)total);
   if (p.hT) {
-    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, true>), grid, dim3(512), 0, st, p);
-    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, true>), grid, dim3(512), 0, st, p);
+    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, true, SG>), grid, dim3(512), 0, st, p);
+    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, true, SG>), grid, dim3(512), 0, st, p);
     else return FLA_E_UNSUPPORTED;
   } else {
-    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, false>), grid, dim3(512), 0, st, p);
-    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, false>), grid, dim3(512), 0, st, p);
+    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, false, SG>), grid, dim3(512), 0, st, p);
+    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, false, SG>), grid, dim3(512), 0, st, p);
     else return FLA_E_UNSUPPORTED;
   }
   FLA_CHECK_LAUNCH();
@@ -808,8 +855,9 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
                               void* o, float* ht, int* ws_wide, void* ws_hwide, void* h_frag_t, const int64_t* offsets,
                               const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
-                              int64_t V, int64_t N, float scale, fla_stream_t stream) {
+                              int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
+  if (head_gates) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE((K == 64 || K == 128) && V % 64 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
   FLA_REQUIRE((ws_wide == nullptr) == (ws_hwide == nullptr), FLA_E_INVALID);
@@ -832,13 +880,25 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     if (rc) return rc;
   }
   ExactParams e{q, k, v, gates, ws_wide, ws_hwide, o, offsets, indices, T, (int)H, ntfix, scale,
-                (int64_t)grid.x * grid.y};
+                (int64_t)grid.x * grid.y, head_gates ? 1 : 0};
   if (ws_wide) grid = dim3((unsigned)(e.total < 512 ? e.total : 512));
 #define FLA_FUSED(TT, GG)                                                \
   {                                                                      \
     int rc = launch_fused<TT, GG>(p, (int)K, st);                        \
     if (rc || !ws_wide || grid.x == 0) return rc;                        \
     return launch_exact<TT, GG>(e, (int)K, (int)V, grid, st);            \
+  }
+  if (head_gates) {
+#define FLA_FUSED_SG(TT)                                                 \
+  {                                                                      \
+    int rc = launch_fused<TT, float, true>(p, (int)K, st);               \
+    if (rc || !ws_wide || grid.x == 0) return rc;                        \
+    return launch_exact<TT, float>(e, (int)K, (int)V, grid, st);         \
+  }
+    if (qkv_dtype == FLA_BF16) FLA_FUSED_SG(bf16)
+    if (qkv_dtype == FLA_F16) FLA_FUSED_SG(f16)
+#undef FLA_FUSED_SG
+    return FLA_E_UNSUPPORTED;
   }
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_FUSED(bf16, float)
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_FUSED(bf16, bf16)
@@ -867,4 +927,14 @@ extern "C" int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, cons
   FLA_REQUIRE(h_frag_t, FLA_E_INVALID);
   return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, const float* g,
+                                              const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                              void* h_frag_t, const int64_t* offsets, const int64_t* indices,
+                                              const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                              int64_t N, float scale, fla_stream_t stream) {
+  return gla_fwd_fused_impl(q, k, v, g, h0, o, ht, ws_wide, ws_hwide, h_frag_t, offsets, indices, chunk_offsets,
+                            seq_order, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true);
 }

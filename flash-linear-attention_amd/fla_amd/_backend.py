@@ -40,6 +40,7 @@ SIGNATURES = {
                                     I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused": (c_int, [P] * 13 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_states": (c_int, [P] * 14 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 14 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_gdr_fwd_wy": (c_int, [P, P, P, P, P, P, P, P, P, P, F, P, P, I64, I, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                                  I64, I64, I64, I64, I64, I64, P]),

@@ -158,13 +158,14 @@ def chunk_gla_bwd_dv(k, g, A, do, dh, offsets=None, indices=None, head_first=Tru
 
 
 def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,
-                        return_flags=False, states_out=None):
+                        return_flags=False, states_out=None, head_gates=False):
     """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
     With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
     single-reference range are detected on the device and recomputed exactly; ``return_flags``
     also returns the int32 ``[chunks, H]`` flags (for the backward pass).  With a list
     ``states_out`` the launch also writes the state entering every chunk (transposed fragment
-    order, what the backward kernels read) and appends it."""
+    order, what the backward kernels read) and appends it.  ``head_gates``: ``g`` is one fp32 log-gate
+    per (token, head), ``[B,T,H]`` (``fla_chunk_simple_gla_fwd_fused``)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
@@ -184,7 +185,16 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
             0 if plan is None else plan.NT,
             be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q))
     head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide))
-    if states_out is not None:
+    if head_gates:
+        if g.dtype != torch.float32 or g.shape != q.shape[:3]:
+            raise ValueError("head gates must be fp32 [B, T, H]")
+        hT = None
+        if states_out is not None:
+            hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
+            states_out.append(hT)
+        be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), *tail[:5], be.dt(q), *tail[7:]),
+                 "fla_chunk_simple_gla_fwd_fused")
+    elif states_out is not None:
         hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
         be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
         states_out.append(hT)

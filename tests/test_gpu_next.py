@@ -240,3 +240,36 @@ def test_packed_batch_with_empty_sequence(device, op):
     for name, a, b in zip(("dq", "dk", "dv", "dg", "dbeta"), refs, leaves):
         assert_close(name, a.grad, b.grad, 2e-2)
     assert_close("dh0", rh0.grad, h0l.grad, 1e-2)
+
+
+# the forward that is not differentiated reads the per-head gates as they are (no [B,T,H,K] gate tensor)
+@pytest.mark.parametrize("T,K,V", [(64, 128, 128), (300, 128, 64), (1000, 64, 128), (37, 64, 64)])
+@pytest.mark.parametrize("varlen", [False, True])
+@pytest.mark.parametrize("gate_scale", [1.0, 40.0])   # 40: chunk-cumulative gates far beyond the single-reference range
+def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, gate_scale):
+    from fla_amd.ops.simple_gla import chunk_simple_gla
+    from oracle.recurrent import naive_recurrent_gla
+    N, H = 3, 3
+    B = 1 if varlen else 2
+    gen = torch.Generator().manual_seed(T + K + int(gate_scale))
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen)) * gate_scale
+    h0 = torch.randn(N if varlen else B, H, K, V, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"chunk_simple_gla no-grad T={T} K={K} V={V} varlen={varlen} gate x{gate_scale}", flush=True)
+    with torch.no_grad():
+        o, ht = chunk_simple_gla(dev(q), dev(k), dev(v), dev(g), initial_state=dev(h0), output_final_state=True,
+                                 cu_seqlens=dev(offs), head_first=False)
+        # the general route (gates broadcast over the key channels) on the same inputs
+        from fla_amd.ops.gla import chunk_gla
+        o2, ht2 = chunk_gla(dev(q), dev(k), dev(v), dev(g)[..., None].expand(B, T, H, K).contiguous(),
+                            initial_state=dev(h0), output_final_state=True, offsets=dev(offs), head_first=False)
+    torch.cuda.synchronize()
+    ro, rht = naive_recurrent_gla(q.float(), k.float(), v.float(), None, g=g, initial_state=h0,
+                                  output_final_state=True, offsets=None if offs is None else offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)   # same arithmetic on both routes
