@@ -386,9 +386,26 @@ def bench_simple_gla(device, steps=20):
                                                    head_first=False), steps)
         us_b = event_avg_us(lambda: chunk_gla(q, k, v, g[..., None].expand(B, T, H, D), initial_state=h0,
                                               output_final_state=True, head_first=False), steps)
+    # forward + backward at config 4's batch (B=4): per-head-gate forward that keeps the states, GLA backward kernels
+    Bb = 4
+    leaves = [x[:Bb].clone().requires_grad_() for x in (q, k, v, g)]
+    h0b = h0[:Bb].clone().requires_grad_()
+    do = torch.randn(Bb, T, H, D, device=device, generator=gen).bfloat16()
+    dht = torch.randn(Bb, H, D, D, device=device, generator=gen) * 0.1
+
+    def fb(fn, gate):
+        o, ht = fn(leaves[0], leaves[1], leaves[2], gate(leaves[3]), initial_state=h0b, output_final_state=True,
+                   head_first=False)
+        torch.autograd.backward((o, ht), (do, dht))
+        for x in leaves + [h0b]:
+            x.grad = None
+
+    us_fb = event_avg_us(lambda: fb(chunk_simple_gla, lambda x: x), steps)
+    us_fb_b = event_avg_us(lambda: fb(chunk_gla, lambda x: x[..., None].expand(Bb, T, H, D)), steps)
     return {"us": round(us, 1), "tokens_per_s": round(B * T / us * 1e6, 1), "algorithmic_bytes": nbytes,
             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-            "through_per_key_gate_kernel_us": round(us_b, 1)}
+            "through_per_key_gate_kernel_us": round(us_b, 1),
+            "fwd_bwd_B4_us": round(us_fb, 1), "fwd_bwd_B4_through_per_key_gate_kernels_us": round(us_fb_b, 1)}
 
 
 def cpu_baseline(c, budget_s=15.0):

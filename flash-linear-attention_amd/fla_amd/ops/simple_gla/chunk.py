@@ -3,14 +3,52 @@
 Head-wise (scalar) log-decay: ``h_t = e^{g_t} h_{t-1} + k_t v_t^T``, ``o_t = s q_t^T h_t``.  That is
 GLA with the same gate on every key channel, so the operator is served by the GLA kernels
 (forward and backward) on the gate broadcast over K; autograd reduces the gate gradient
-over the key channels.  A forward that will not be differentiated skips the ``[B,T,H,K]`` gate
-tensor: ``fla_chunk_simple_gla_fwd_fused`` reads the per-head gates as they are."""
+over the key channels.  For 16-bit seq-first inputs with K, V in {64, 128} the forward skips the
+``[B,T,H,K]`` gate tensor: ``fla_chunk_simple_gla_fwd_fused`` reads the per-head gates as they are
+(``ChunkSimpleGLAFunction`` when gradients are needed: only its backward forms the gate tensor)."""
 from typing import Optional, Tuple
 
 import torch
 
-from ...utils import check_varlen_args, resolve_offsets
-from ..gla.chunk import chunk_gla, chunk_gla_fwd_fused
+from ... import _backend as be
+from ...utils import check_varlen_args, contiguous, resolve_offsets
+from ..gla import chunk as gla_chunk
+from ..gla.chunk import chunk_gla, chunk_gla_bwd_device, chunk_gla_fwd_fused
+
+
+class ChunkSimpleGLAFunction(torch.autograd.Function):
+    """Seq-first, K and V in {64, 128}, 16-bit q/k/v: the forward reads the per-head gates as they are
+    (``fla_chunk_simple_gla_fwd_fused``, which also keeps the per-chunk states for the backward pass unless
+    recomputation is asked for); only the backward pass, which runs on the GLA kernels, forms the
+    ``[B,T,H,K]`` gate tensor, and reduces the gate gradient over the key channels
+    (the reference: ``fla/ops/simple_gla/chunk.py:134-210``)."""
+
+    @staticmethod
+    @contiguous
+    def forward(ctx, q, k, v, g, scale, initial_state, output_final_state, offsets):
+        be.require_gpu(q, k, v, g)
+        gf = g.float().contiguous()
+        h0 = initial_state
+        flags_states = [] if gla_chunk.KEEP_STATES_FOR_BACKWARD and any(ctx.needs_input_grad) else None
+        o, ht, wide = chunk_gla_fwd_fused(q, k, v, gf, scale, h0, output_final_state, offsets=offsets,
+                                          return_flags=True, states_out=flags_states, head_gates=True)
+        ctx.save_for_backward(q, k, v, gf, h0, offsets, wide, flags_states[0] if flags_states else None)
+        ctx.scale, ctx.g_dtype = scale, g.dtype
+        ctx.h0_dtype = None if initial_state is None else initial_state.dtype
+        return o, ht
+
+    @staticmethod
+    @contiguous
+    def backward(ctx, do, dht):
+        q, k, v, gf, h0, offsets, wide, hT = ctx.saved_tensors
+        K = q.shape[-1]
+        gk = gf.unsqueeze(-1).expand(*gf.shape, K).contiguous()
+        h0f = None if h0 is None else h0.float().contiguous()
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, gk, ctx.scale, h0f, do.to(q.dtype).contiguous(), dht,
+                                                   offsets, wide, hT=hT)
+        if dh0 is not None:
+            dh0 = dh0.to(ctx.h0_dtype)
+        return dq, dk, dv, dg.sum(-1).to(ctx.g_dtype), None, dh0, None, None
 
 
 def chunk_simple_gla(
@@ -44,8 +82,10 @@ def chunk_simple_gla(
     V = v.shape[-1]
     needs_grad = torch.is_grad_enabled() and any(
         t is not None and t.requires_grad for t in (q, k, v, g, initial_state))
-    if (g is not None and not needs_grad and not head_first and K in (64, 128) and V in (64, 128)
+    if (g is not None and not head_first and K in (64, 128) and V in (64, 128)
             and q.dtype in (torch.bfloat16, torch.float16) and k.dtype == q.dtype and v.dtype == q.dtype):
+        if needs_grad:
+            return ChunkSimpleGLAFunction.apply(q, k, v, g, scale, initial_state, output_final_state, offsets)
         return chunk_gla_fwd_fused(q.contiguous(), k.contiguous(), v.contiguous(), g.float().contiguous(), scale,
                                    initial_state, output_final_state, offsets=offsets, head_gates=True)
     if g is None:
