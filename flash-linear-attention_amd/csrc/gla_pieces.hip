@@ -66,10 +66,14 @@ __global__ __launch_bounds__(256) void gla_piece_kernel(PieceParams p) {
   __shared__ __attribute__((aligned(16))) T sS[BT * LDT];    // [row][contraction row]
   __shared__ __attribute__((aligned(16))) T sYt[64 * LDT];   // [v][contraction row]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // 1-D grid, value slabs of one (chunk, head) side by side on one XCD: the second slab finds the
+  // q/k and gate rows of the first in that XCD's L2
   int hh;
-  const ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.ntfix, p.H, &hh);
+  const int nslab = p.V / 64;
+  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
+  const ChunkLoc cl = locate_chunk_at(lid / nslab, p.offsets, p.indices, p.T, p.ntfix, p.H, &hh);
   const int H = p.H, V = p.V, L = cl.L;
-  const int vbase = blockIdx.z * 64;
+  const int vbase = (int)(lid % nslab) * 64;
 
   // X: 8 key channels of one row per unit
   {
@@ -430,7 +434,9 @@ int piece_entry(bool dv, const void* x, const float* g, const void* A, const voi
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  grid.z = (unsigned)(V / 64);
+  const int64_t nwg = (int64_t)grid.x * grid.y * (V / 64);
+  FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  grid = dim3((unsigned)nwg);
   PieceParams p{x, g, A, m, y, out, offsets, indices, T, ntfix, (int)H, (int)V, scale, 0, 0};
   if ((rc = is_f32_code(a_dtype, qkv_dtype, &p.a_is_f32))) return rc;
   if ((rc = is_f32_code(m_dtype, qkv_dtype, &p.m_is_f32))) return rc;
