@@ -365,6 +365,10 @@ def bench_gla_stages(device, steps=20):
     rec("chunk_gla_bwd_dA", lambda: chunk_gla_bwd_dA(v, do, K ** -0.5, head_first=False), 2 * b_v + b_a)
     rec("chunk_gla_bwd_dv", lambda: chunk_gla_bwd_dv(k, G, A, do, h, head_first=False),
         b_qk + b_g + b_a + b_h + 2 * b_v)
+    from fla_amd.ops.common.chunk_h import chunk_bwd_dh
+    h0 = torch.zeros(B, H, K, V, device=device)
+    rec("chunk_bwd_dh", lambda: chunk_bwd_dh(q, k, v, None, G, None, do, h0, h0, K ** -0.5, head_first=False,
+                                             states_in_fp32=True), b_qk + b_g + b_v + b_h)
     return out
 
 

@@ -276,9 +276,12 @@ __global__ __launch_bounds__(256) void chunk_bwd_dh_rowmajor_kernel(RowDhParams 
   __shared__ float sDecay[64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int H = p.H, K = p.K, V = p.V;
-  const int nv = V / 64;
-  const int kbase = (blockIdx.x / nv) * 64, vbase = (blockIdx.x % nv) * 64;
-  const int n = blockIdx.y / H, hh = blockIdx.y % H;
+  // 1-D grid, the tiles of one (sequence, head) side by side on one XCD (they share q, do and the gates)
+  const int nv = V / 64, ntile = (K / 64) * nv;
+  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile = (int)(lid % ntile);
+  const int kbase = (tile / nv) * 64, vbase = (tile % nv) * 64;
+  const int n = (int)((lid / ntile) / H), hh = (int)((lid / ntile) % H);
   const SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int64_t nchunks = (sp.len + BT - 1) / BT;
   const int64_t boh = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
@@ -492,12 +495,12 @@ extern "C" int fla_chunk_bwd_dh(const void* q, const float* g, const float* gk, 
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)gk | (uintptr_t)dout | (uintptr_t)dh) % 16 == 0, FLA_E_ALIGNMENT);
   const int64_t tiles = (K / 64) * (V / 64);
-  FLA_REQUIRE(tiles <= 0x7fffffffLL && N * H <= 65535, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(tiles * N * H <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   if (N == 0 || T == 0) return FLA_OK;
   RowDhParams p{q, g, gk, dout, dht, dh, dh0, offsets, chunk_offsets, T, (int)H, (int)K, (int)V, scale, 0};
   int rc = is_f32_code(dh_dtype, qkv_dtype, &p.dh_is_f32);
   if (rc) return rc;
-  dim3 grid((unsigned)tiles, (unsigned)(N * H));
+  dim3 grid((unsigned)(tiles * N * H));
   if (qkv_dtype == FLA_BF16) chunk_bwd_dh_rowmajor_kernel<bf16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
   else if (qkv_dtype == FLA_F16) chunk_bwd_dh_rowmajor_kernel<f16><<<grid, 256, 0, (hipStream_t)stream>>>(p);
   else return FLA_E_UNSUPPORTED;
