@@ -23,8 +23,13 @@ Pinning status (what independent fact fixes each function; the checks live in
   (pure decay), ``g = 0, beta = 1`` with orthonormal keys (exact overwrite),
   the T=1 closed form, and an independent dense "materialise every transition
   matrix" evaluation.
-* ``chunked.*`` - the chunked algorithms are pinned against the two naive
-  recurrences above plus ``torch.linalg.solve_triangular`` for the WY inverse.
+* ``chunked.chunked_gla`` / ``chunked.chunked_gated_delta_rule`` - the chunked algorithms are pinned
+  against the two naive recurrences above plus ``torch.linalg.solve_triangular`` for the WY inverse.
+* ``chunked.gla_fwd_o_gk`` - pinned by the recurrence: fed with ``chunked_gla``'s scores and states
+  (and garbage above the diagonal of the scores) it must reproduce the recurrence's output.
+* ``chunked.gla_bwd_dA`` / ``gla_bwd_dv`` / ``chunk_bwd_dv_local`` / ``chunk_bwd_dh`` - pinned by
+  ``torch.autograd`` through the fp64 chunk step (the one ``chunked_gla`` is built from), with a zero
+  tap on every per-chunk state for ``dh``.
 * gradients - ``torch.autograd`` through the fp64 recurrences, with
   ``torch.autograd.gradcheck`` on tiny shapes.
 """
