@@ -116,8 +116,16 @@ inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B,
   return FLA_OK;
 }
 
-// Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps
-// the operand finite in 16-bit storage.
-constexpr float kMaxInvDecayExp = 80.f;
+// Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps the operand finite in
+// 16-bit storage.  bf16 has fp32's exponent range; fp16 ends at 65504 (e^{11}), so fp16 chunks leave the
+// single-reference arithmetic much earlier (e^{8} |k| stays representable for |k| up to 20).
+template <typename T>
+struct InvDecayLimit {
+  static constexpr float value = 80.f;
+};
+template <>
+struct InvDecayLimit<f16> {
+  static constexpr float value = 8.f;
+};
 
 }  // namespace

@@ -361,7 +361,7 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     v4 qv, kv;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      float up = fminf(G[i][j] - glast[j], kMaxInvDecayExp);
+      float up = fminf(G[i][j] - glast[j], InvDecayLimit<T>::value);
       qv[j] = (T)(qq[i][j] * p.scale * __expf(up));
       kv[j] = (T)(kk[i][j] * __expf(glast[j] - G[i][j]));
     }
@@ -575,7 +575,7 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) einv[i][j] = __expf(fminf(-G[i][j], kMaxInvDecayExp));
+    for (int j = 0; j < 4; ++j) einv[i][j] = __expf(fminf(-G[i][j], InvDecayLimit<T>::value));
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     v4 kt, qt;

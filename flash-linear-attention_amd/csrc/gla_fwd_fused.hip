@@ -256,10 +256,10 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
       // The scores use one reference point per chunk (e^{G} on q, e^{-G} on k), exact while
-      // |G| stays below kMaxInvDecayExp.  Chunks beyond that are flagged and recomputed by
+      // |G| stays below InvDecayLimit<T>::value.  Chunks beyond that are flagged and recomputed by
       // the exact kernel afterwards (their q~, k~ tiles may hold infinities: only the scores
       // use them, and those are recomputed).
-      const int out_of_range = __any(gabs > kMaxInvDecayExp * LOG2E);  // wave-uniform
+      const int out_of_range = __any(gabs > InvDecayLimit<T>::value * LOG2E);  // wave-uniform
       if (lane == 0) sWide[buf][pw] = out_of_range;
       float eglast[CPL];
 #pragma unroll

@@ -150,7 +150,8 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
  * fla_chunk_gla_fwd_o (the launches of chunk_gla_fwd, fla/ops/gla/chunk.py:1156-1214)
  * with raw log-gates.  K in {64, 128}, V a multiple of 64.  h0, ht, offsets may be NULL.
  * The fused kernel scores a chunk with one reference point (exact while the
- * chunk-cumulative log-gate stays within +-80 per channel).  With the workspaces
+ * chunk-cumulative log-gate stays within +-80 per channel; +-8 for fp16 q/k/v, whose
+ * range ends at 65504).  With the workspaces
  * ws_wide (int32 [chunks, H]) and ws_hwide (q/k/v dtype, [chunks, H, K*V]) given
  * (V <= 128), chunks outside that range are flagged on the device and their
  * output rows recomputed by a second launch with exact pairwise exponents

@@ -99,3 +99,31 @@ def test_fused_recurrent_storage_types(device, dtype):
         ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta.to(dtype), initial_state=h0, output_final_state=True)
         assert_close("o", ro, o, tol)
         assert_close("ht", rht, ht, 5e-3 if dtype != torch.float32 else 1e-5)
+
+
+def test_chunk_gla_fp16_strong_gates(device):
+    """fp16 ends at 65504: with chunk-cumulative log-gates beyond about -8 the factor e^{-G} on k no longer fits,
+    so such chunks must take the exact pairwise arithmetic (bf16 only needs it beyond -80).  Forward and backward
+    against the fp32 recurrence, 1e-2 / 2e-2 as for the other dtypes."""
+    import torch.nn.functional as F
+    from fla_amd.ops.gla import chunk_gla
+    from helpers import assert_close
+    from oracle.recurrent import naive_recurrent_gla
+    B, T, H, K, V = 2, 256, 2, 128, 128
+    gen = torch.Generator().manual_seed(5)
+    q = (torch.randn(B, T, H, K, generator=gen) * 0.5).half()
+    k = (torch.randn(B, T, H, K, generator=gen) * 0.5).half()
+    v = torch.randn(B, T, H, V, generator=gen).half()
+    g = F.logsigmoid(torch.randn(B, T, H, K, generator=gen))          # about -0.8 per step: -50 over a chunk
+    do = torch.randn(B, T, H, V, generator=gen).half()
+    leaves = [x.to(device).detach().requires_grad_() for x in (q, k, v, g)]
+    o, ht = chunk_gla(*leaves, output_final_state=True, head_first=False)
+    o.backward(do.to(device))
+    torch.cuda.synchronize()
+    rl = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    ro, rht = naive_recurrent_gla(*rl, output_final_state=True)
+    (ro * do.float()).sum().backward()
+    assert_close("o", ro, o, 1e-2)
+    assert_close("ht", rht, ht, 5e-3)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
+        assert_close(name, a.grad, b.grad, 2e-2)

@@ -273,3 +273,35 @@ def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, 
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
     assert torch.equal(o, o2) and torch.equal(ht, ht2)   # same arithmetic on both routes
+
+
+def test_chunk_simple_gla_per_head_gate_kernel_fp16_and_gradients(device):
+    """fp16 operands through the per-head-gate launch, forward and backward (the states it keeps feed the GLA
+    backward kernels), against the fp32 recurrence."""
+    from fla_amd.ops.simple_gla import chunk_simple_gla
+    from oracle.recurrent import naive_recurrent_gla
+    B, T, H, K, V = 2, 200, 2, 64, 128
+    gen = torch.Generator().manual_seed(77)
+    q = (torch.randn(B, T, H, K, generator=gen) * 0.5).half()
+    k = (torch.randn(B, T, H, K, generator=gen) * 0.5).half()
+    v = torch.randn(B, T, H, V, generator=gen).half()
+    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
+    h0 = torch.randn(B, H, K, V, generator=gen) * 0.1
+    do = torch.randn(B, T, H, V, generator=gen).half()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    dev = _dev(device)
+    leaves = [dev(x).detach().requires_grad_() for x in (q, k, v, g)]
+    h0l = dev(h0).detach().requires_grad_()
+    o, ht = chunk_simple_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=False)
+    torch.autograd.backward((o, ht), (dev(do), dev(dht)))
+    torch.cuda.synchronize()
+    rl = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.detach().float().requires_grad_()
+    ro, rht = naive_recurrent_gla(rl[0], rl[1], rl[2], None, g=rl[3], initial_state=rh0, output_final_state=True)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    assert o.dtype == torch.float16
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
+        assert_close(name, a.grad, b.grad, TOL_G)
+    assert_close("dh0", rh0.grad, h0l.grad, TOL_G)
