@@ -99,7 +99,10 @@ def chunk_gla_fwd_o_gk(q, v, g, A, h, scale, offsets=None, indices=None, head_fi
 
     Called as the reference calls it (``k`` not given), ``A`` and the row-major ``h`` are read as
     they are.  The operator's own pipeline passes ``k=``: the device kernel then recomputes the
-    scores from ``q, k, g`` and takes ``h`` in MFMA-fragment order (seq-first only)."""
+    scores from ``q, k, g`` and takes ``h`` in MFMA-fragment order (seq-first only); that form scores a
+    chunk with one reference point and has no range guard, so it is exact only while the chunk-cumulative
+    log-gate stays within +-80 (bf16) or +-8 (fp16) - ``chunk_gla`` itself goes through the guarded
+    fused launch."""
     if k is None:
         return _chunk_gla_fwd_o_gk_plain(q, v, g, A, h, scale, offsets, indices, head_first, chunk_size)
     if head_first or chunk_size != BT:
