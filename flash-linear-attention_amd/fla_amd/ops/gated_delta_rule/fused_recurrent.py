@@ -100,5 +100,10 @@ def fused_recurrent_gated_delta_rule(
         assert scale > 0, "scale must be positive"
     if beta is None:
         beta = torch.ones_like(q[..., 0])
+    if not (torch.is_grad_enabled() and any(t is not None and t.requires_grad
+                                            for t in (q, k, v, g, beta, initial_state))):
+        # decode loops: no autograd node to build, and the host time of a step is of the order of its device time
+        return fused_recurrent_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
+                                                    offsets, head_first, inplace_state)
     return FusedRecurrentFunction.apply(q, k, v, g, beta, scale, initial_state, output_final_state, offsets,
                                         head_first, inplace_state)
