@@ -164,8 +164,7 @@ def bench_decode(device, steps=1000):
     beta = torch.rand(B, 1, H, device=device).sigmoid()
     state_bytes = B * H * K * V * 4
     small = B * H * 128 * 2
-    # one state buffer for both recurrences, refilled in place: what a serving loop holds for the whole
-    # generation (a second 512 MiB allocation made late in a process has measured 15 % slower steps)
+    # one state buffer for both recurrences, refilled in place: what a serving loop holds for the whole generation
     S = torch.empty(B, H, K, V, device=device)
     for name in ("gla", "gdr"):
         S.normal_().mul_(0.1)
