@@ -7,10 +7,13 @@ A step is one chunk_gla forward on the headline workload (B=8, T=4096, H=16,
 K=V=128, bf16 q/k/v, fp32 log-gates and state, initial state given, final state
 returned), inputs resident in HBM.  Prints ONE JSON line:
 
-* value            tokens/s of the whole forward (B*T*steps / elapsed)
+* value            tokens/s of the whole forward: B*T / the median step time (every step sits between
+                   two HIP events on the launch stream; min, max, the number of stalled intervals and
+                   the wall time of the same loop are reported in extra.chunk_gla_fwd)
 * roofline         the dominant kernel of that forward against the HBM roofline:
-                   algorithmic bytes per launch / its average duration measured
-                   here with HIP events on the launch stream
+                   algorithmic bytes per launch / its median duration measured
+                   here with HIP events on the launch stream; traffic = HBM bytes per launch from
+                   the counter readings kept in profiles/hbm_traffic_counters.txt
 * cpu_baseline     the oracle's fp32 naive recurrence timed on the host cores on
                    a bounded sample of the same workload
 * extra            the other measured rows: the T=1 decode steps (B=256, H=32),
@@ -38,32 +41,59 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def time_steps(fn, steps, warmup):
-    """Wall time of exactly `steps` calls, bracketed by synchronize on both sides."""
+def event_stats(fn, steps, warmup=3):
+    """Device time of one call from HIP events recorded on the launch stream around every call:
+    median, min, max and mean in microseconds, the number of intervals longer than twice the median
+    (a stalled launch: clock ramp, an allocation, something else on the box) and the wall time of the
+    whole timed loop, which is bracketed by synchronize on both sides."""
+    import statistics
     import torch
     for _ in range(warmup):
         fn()
+    ev = _events(2 * steps)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return time.perf_counter() - t0
-
-
-def event_avg_us(fn, steps, warmup=3):
-    """Average device time of one call, HIP events recorded on the launch stream."""
-    import torch
-    for _ in range(warmup):
-        fn()
-    torch.cuda.synchronize()
-    ev = _events(2 * steps)
     for i in range(steps):
         ev[2 * i].record()
         fn()
         ev[2 * i + 1].record()
     torch.cuda.synchronize()
-    return sum(ev[2 * i].elapsed_time(ev[2 * i + 1]) for i in range(steps)) / steps * 1e3
+    wall = time.perf_counter() - t0
+    us = [ev[2 * i].elapsed_time(ev[2 * i + 1]) * 1e3 for i in range(steps)]
+    med = statistics.median(us)
+    return {"median_us": med, "min_us": min(us), "max_us": max(us), "mean_us": sum(us) / steps, "n": steps,
+            "n_over_2x_median": sum(1 for x in us if x > 2 * med), "wall_us_per_call": wall / steps * 1e6}
+
+
+def spread(st):
+    """The part of event_stats() every row reports beside its median."""
+    return {"min_us": round(st["min_us"], 1), "max_us": round(st["max_us"], 1), "n": st["n"],
+            "n_over_2x_median": st["n_over_2x_median"]}
+
+
+def event_avg_us(fn, steps, warmup=3):
+    """Median device time of one call (see event_stats)."""
+    return event_stats(fn, steps, warmup)["median_us"]
+
+
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
+
+
+def counter_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs whose
+    readings are kept in profiles/hbm_traffic_counters.txt (one tab-separated line per kernel: name,
+    FETCH_SIZE, WRITE_SIZE; a `scale` line holds the bytes per counter unit found with the 1 GiB copy
+    of the same runs; the kernels of the roofline blocks also appear as `roofline:<kernel>:<workload>`).
+    None if the file or the kernel is missing."""
+    try:
+        lines = [l.rstrip("\n").split("\t") for l in open(TRAFFIC_FILE) if l.strip() and not l.startswith("#")]
+    except OSError:
+        return None
+    scale = next((l for l in lines if l[0] == "scale"), None)
+    row = next((l for l in lines if l[0] == kernel), None)
+    if scale is None or row is None:
+        return None
+    return int(round(float(row[1]) * float(scale[1]) + float(row[2]) * float(scale[2])))
 
 
 def gla_config1(device):
@@ -91,18 +121,22 @@ def bench_gla(device, steps, warmup):
     def step():
         return chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
 
-    elapsed = time_steps(step, steps, warmup)
-    ms = elapsed / steps * 1e3
-    tokens_per_s = B * T * steps / elapsed
+    # `warmup` untimed steps, then exactly `steps` steps between two synchronisations, each step between
+    # two HIP events on the launch stream.  value = tokens / median step time; the wall time of the same
+    # loop and the spread of the intervals are reported beside it.
+    st = event_stats(step, steps, warmup)
+    ms = st["median_us"] * 1e-3
+    tokens_per_s = B * T / (st["median_us"] * 1e-6)
 
-    # device time of the kernels of the forward, HIP events on the launch stream.  The
-    # operator is one launch (gla_fwd_fused_kernel); the two-kernel pipeline it replaces
-    # (state scan + per-chunk output) is timed as well for comparison.
+    # device time of the kernels of the forward, HIP events on the launch stream.  The operator is
+    # gla_fwd_fused_kernel followed by the range guard's short second launch; the dominant kernel is
+    # timed on its own in the form the operator runs it (guard workspaces given).  The two-kernel
+    # pipeline it replaces (state scan + per-chunk output) is timed as well for comparison.
     from fla_amd.ops.gla.chunk import chunk_gla_fwd_fused
     scale = K ** -0.5
 
     def run_fused():
-        chunk_gla_fwd_fused(q, k, v, g, scale, h0, True, exact_guard=False)
+        chunk_gla_fwd_fused(q, k, v, g, scale, h0, True, first_launch_only=True)
 
     h_hold = {}
 
@@ -117,30 +151,31 @@ def bench_gla(device, steps, warmup):
         chunk_gla_fwd_o_gk(q, v, g, None, h_hold["h"], scale, head_first=False, chunk_size=64, k=k,
                            gates_are_cumsum=False)
 
-    n_ev = max(steps, 10)
-    us_f = event_avg_us(run_fused, n_ev)
-    us_h = event_avg_us(run_h, n_ev)
-    us_o = event_avg_us(run_o, n_ev)
+    n_ev = max(steps, 20)
+    st_f = event_stats(run_fused, n_ev, warmup=10)
+    us_f = st_f["median_us"]
+    us_h = event_avg_us(run_h, 20)
+    us_o = event_avg_us(run_o, 20)
     NT = T // 64
     qkv = B * T * H * K * 2                      # one bf16 [B,T,H,128] tensor
     gbytes = B * T * H * K * 4                   # fp32 gates
     hbytes = B * NT * H * K * V * 2              # bf16 per-chunk states
-    st = B * H * K * V * 4                       # one fp32 state
-    floor_bytes = 4 * qkv + gbytes + 2 * st      # q,k,v,o + g + h0,ht: the operator's algorithmic bytes
-    bytes_h = 2 * qkv + gbytes + hbytes + 2 * st           # k, v, g in; h, ht out; h0 in
+    stb = B * H * K * V * 4                      # one fp32 state
+    floor_bytes = 4 * qkv + gbytes + 2 * stb     # q,k,v,o + g + h0,ht: the operator's algorithmic bytes
+    bytes_h = 2 * qkv + gbytes + hbytes + 2 * stb          # k, v, g in; h, ht out; h0 in
     bytes_o = 3 * qkv + gbytes + hbytes + qkv              # q, k, v, g, h in; o out
     ach = floor_bytes / (us_f * 1e-6) / 1e9
-    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/):
-    # 331950 * 2 KiB read (the copy-kernel calibration gives a factor 2 for FETCH_SIZE on this
-    # part) + 139264 KiB written = 784 MiB, i.e. exactly the algorithmic bytes.
-    traffic = 331950 * 2 * 1024 + 139264 * 1024
-    roofline = {"kernel": "gla_fwd_fused_kernel", "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": traffic,
-                "avg_us": round(us_f, 1), "bytes_per_launch": floor_bytes}
     flops = B * T * H * (4 * K * V + 2 * 64 * K + 2 * 64 * V)   # dense-tile count of the chunked algorithm
+    roofline = {"kernel": "gla_fwd_fused_kernel", "bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                "traffic": counter_traffic("roofline:gla_fwd_fused_kernel:config1"),
+                "avg_us": round(us_f, 1), "bytes_per_launch": floor_bytes,
+                "frac_of_mfma_peak": round(flops / (us_f * 1e-6) / MFMA_PEAK_FLOPS, 4), **spread(st_f)}
     op = {"algorithmic_bytes": floor_bytes, "achieved_GBs": round(floor_bytes / (ms * 1e-3) / 1e9, 1),
           "frac_of_hbm_peak": round(floor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
           "algorithmic_flops": flops, "frac_of_mfma_peak": round(flops / (ms * 1e-3) / MFMA_PEAK_FLOPS, 4),
+          "step_us": round(st["median_us"], 1), **spread(st),
+          "wall_us_per_step": round(st["wall_us_per_call"], 1),
           "two_kernel_pipeline_us": {"gla_fwd_h_kernel": round(us_h, 1), "gla_fwd_o_kernel": round(us_o, 1)},
           "two_kernel_pipeline_GBs": {"gla_fwd_h_kernel": round(bytes_h / (us_h * 1e-6) / 1e9, 1),
                                       "gla_fwd_o_kernel": round(bytes_o / (us_o * 1e-6) / 1e9, 1)}}
@@ -179,17 +214,33 @@ def bench_decode(device, steps=1000):
                                                           output_final_state=True, head_first=False,
                                                           inplace_state=True)
             nbytes = 2 * state_bytes + 4 * small + 2 * B * H * 4
-        elapsed = time_steps(fn, steps, 20)
-        us = elapsed / steps * 1e6
+        # 1000 consecutive steps: the wall time of the loop per step (what a serving loop sees, host
+        # included) and the median of the per-step HIP-event intervals (the device side)
+        st = event_stats(fn, steps, 20)
+        us = st["wall_us_per_call"]
         assert torch.isfinite(S).all()
         out[name] = {"us_per_step": round(us, 1), "tokens_per_s": round(B / (us * 1e-6), 1),
                      "GBs": round(nbytes / (us * 1e-6) / 1e9, 1),
                      "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                     "bytes_per_step": nbytes, "steps": steps}
+                     "bytes_per_step": nbytes, "steps": steps,
+                     "event_median_us": round(st["median_us"], 1), **spread(st)}
+        # the same step captured once in a HIP graph and replayed: no Python between the launches
+        S.normal_().mul_(0.1)
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        stg = event_stats(graph.replay, steps, 20)
+        usg = stg["wall_us_per_call"]
+        assert torch.isfinite(S).all()
+        out[name]["hip_graph_replay"] = {"us_per_step": round(usg, 1), "tokens_per_s": round(B / (usg * 1e-6), 1),
+                                         "frac_of_hbm_peak": round(nbytes / (usg * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                                         "event_median_us": round(stg["median_us"], 1), **spread(stg)}
     return out
 
 
-def bench_gdr(device, steps=20):
+def bench_gdr(device, steps=50, warmup=20):
     """chunk_gated_delta_rule forward: the packed workload (packed, 12 sequences, 32768 tokens)
     and the fixed-length shape B=8, T=4096 of the headline metric."""
     import torch
@@ -211,9 +262,10 @@ def bench_gdr(device, steps=20):
     # state products 6KV, the chunk-local products 3*2*BT*K + 2*2*BT*V, and the 64x64 triangular solve per chunk
     gdr_flops = T * H * (6 * K * V + 6 * 64 * K + 4 * 64 * V + 5500)
     out = {}
-    us = event_avg_us(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs,
-                                                     head_first=False), steps)
-    out["config2_varlen"] = {"us": round(us, 1), "tokens_per_s": round(T / (us * 1e-6), 1),
+    st = event_stats(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs,
+                                                    head_first=False), steps, warmup)
+    us = st["median_us"]
+    out["config2_varlen"] = {"us": round(us, 1), **spread(st), "tokens_per_s": round(T / (us * 1e-6), 1),
                              "sequence_lengths": lens.tolist(),
                              "operator_floor_bytes": floor + N * H * K * V * 4,
                              "frac_of_hbm_peak": round((floor + N * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
@@ -222,9 +274,10 @@ def bench_gdr(device, steps=20):
     B, T2 = 8, 4096
     q, k, v = (x.view(B, T2, H, -1) for x in (q, k, v))
     g, beta = g.view(B, T2, H), beta.view(B, T2, H)
-    us = event_avg_us(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
-                      steps)
-    out["B8_T4096"] = {"us": round(us, 1), "tokens_per_s": round(B * T2 / (us * 1e-6), 1),
+    st = event_stats(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
+                     steps, warmup)
+    us = st["median_us"]
+    out["B8_T4096"] = {"us": round(us, 1), **spread(st), "tokens_per_s": round(B * T2 / (us * 1e-6), 1),
                        "operator_floor_bytes": floor + B * H * K * V * 4,
                        "frac_of_hbm_peak": round((floor + B * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                        "algorithmic_flops": gdr_flops,
@@ -232,7 +285,7 @@ def bench_gdr(device, steps=20):
     return out
 
 
-def bench_backward(device, steps=10):
+def bench_backward(device, steps=20):
     """Training workload: forward + backward of both chunk operators, B=4, T=4096, H=16, K=V=128."""
     import torch
     import torch.nn.functional as F
@@ -273,11 +326,12 @@ def bench_backward(device, steps=10):
     leaves.extend([q, k, v, gk, h0, kn, g, beta])
 
     for name, fn in (("chunk_gla", gla_step), ("chunk_gated_delta_rule", gdr_step)):
-        us = event_avg_us(fn, steps)
+        st = event_stats(fn, steps, 5)
+        us = st["median_us"]
         # forward + backward FLOPs (dense-tile counts): GLA 10KV + 4*BT*(K+V); delta rule 16KV + 2*BT*(9K+5V) + 8*BT^2
         fl = B * T * H * ((10 * K * V + 4 * 64 * (K + V)) if name == "chunk_gla"
                           else (16 * K * V + 2 * 64 * (9 * K + 5 * V) + 8 * 64 * 64))
-        out[name] = {"fwd_bwd_us": round(us, 1), "tokens_per_s": round(B * T / (us * 1e-6), 1),
+        out[name] = {"fwd_bwd_us": round(us, 1), **spread(st), "tokens_per_s": round(B * T / (us * 1e-6), 1),
                      "algorithmic_flops": fl, "frac_of_mfma_peak": round(fl / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
     return out
 

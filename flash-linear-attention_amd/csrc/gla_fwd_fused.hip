@@ -676,7 +676,14 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
   constexpr int KT32 = K / 32, TV = V / 64;
   const int H = p.H;
   // A few hundred workgroups walk the (chunk, head) flags: almost always none is set, and a
-  // launch of one workgroup per chunk would cost more than the scan.
+  // launch of one workgroup per chunk would cost more than the scan.  The lanes first read all flags
+  // of the workgroup side by side (one memory latency instead of one per flag) and leave if none is set.
+  {
+    int any = 0;
+    for (int64_t lin = blockIdx.x + (int64_t)threadIdx.x * gridDim.x; lin < p.total; lin += (int64_t)256 * gridDim.x)
+      any |= p.wide[lin];
+    if (!__syncthreads_or(any)) return;
+  }
   for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
   if (p.wide[lin] == 0) continue;  // workgroup-uniform
   __syncthreads();                 // the tiles of the previous flagged chunk are free
@@ -855,7 +862,8 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
                               void* o, float* ht, int* ws_wide, void* ws_hwide, void* h_frag_t, const int64_t* offsets,
                               const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
-                              int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false) {
+                              int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false,
+                              bool exact_pass = true) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
   if (head_gates) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
@@ -885,14 +893,14 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
 #define FLA_FUSED(TT, GG)                                                \
   {                                                                      \
     int rc = launch_fused<TT, GG>(p, (int)K, st);                        \
-    if (rc || !ws_wide || grid.x == 0) return rc;                        \
+    if (rc || !ws_wide || grid.x == 0 || !exact_pass) return rc;         \
     return launch_exact<TT, GG>(e, (int)K, (int)V, grid, st);            \
   }
   if (head_gates) {
 #define FLA_FUSED_SG(TT)                                                 \
   {                                                                      \
     int rc = launch_fused<TT, float, true>(p, (int)K, st);               \
-    if (rc || !ws_wide || grid.x == 0) return rc;                        \
+    if (rc || !ws_wide || grid.x == 0 || !exact_pass) return rc;         \
     return launch_exact<TT, float>(e, (int)K, (int)V, grid, st);         \
   }
     if (qkv_dtype == FLA_BF16) FLA_FUSED_SG(bf16)
@@ -916,6 +924,16 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
                                        int64_t V, int64_t N, float scale, fla_stream_t stream) {
   return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_gla_fwd_fused_first_launch(const void* q, const void* k, const void* v, const void* gates,
+                                                    const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                                    const int64_t* offsets, const int64_t* indices,
+                                                    const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                                                    int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
+                                                    int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, offsets, indices, chunk_offsets,
+                            seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream, false, false);
 }
 
 extern "C" int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, const void* v, const void* gates,

@@ -39,6 +39,7 @@ SIGNATURES = {
     "fla_chunk_gla_fwd_o": (c_int, [P, P, P, P, I, P, P, P, P, P, I64, I, I,
                                     I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused": (c_int, [P] * 13 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gla_fwd_fused_first_launch": (c_int, [P] * 13 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_states": (c_int, [P] * 14 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 14 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_gdr_fwd_wy": (c_int, [P, P, P, P, P, P, P, P, P, P, F, P, P, I64, I, I64, I64, I64, I64, I64, P]),

@@ -1,8 +1,11 @@
 """``chunk_gla`` with the reference's signature (``fla/ops/gla/chunk.py:1409-1495``).
 
-Forward pipeline on the device (chunk size 64):
-``fla_chunk_gla_fwd_h`` (state scan, cumsum of the gates formed in-kernel)
--> ``fla_chunk_gla_fwd_o`` (fused cumsum + gated scores + output).
+Forward on the device (chunk size 64): one launch, ``fla_chunk_gla_fwd_fused`` (prefix sums of the
+gates, gated scores, output and state scan in one pass; the per-chunk states stay on the chip),
+followed by a short second launch that recomputes the output rows of chunks whose gates left the
+range of the single-reference-point scores.  The two-kernel form (``fla_chunk_gla_fwd_h`` ->
+``fla_chunk_gla_fwd_o``) serves the reference-shaped internal entry points ``chunk_gla_fwd`` /
+``chunk_fwd_h`` / ``chunk_gla_fwd_o_gk``.
 """
 import os
 import warnings
@@ -160,8 +163,26 @@ def chunk_gla_bwd_dv(k, g, A, do, dh, offsets=None, indices=None, head_first=Tru
     return dv.transpose(1, 2) if head_first else dv
 
 
+# Workspaces of the range guard for forward passes whose flags nobody keeps: one pair per (device,
+# stream, shape, dtype), reused by every call (launches on one stream are ordered, so the next call
+# may overwrite them).  A forward that hands its flags to a backward pass gets fresh ones.
+_GUARD_WS = {}
+
+
+def _guard_workspaces(q, chunks, H, KV, keep):
+    if keep:
+        return q.new_empty(chunks, H, dtype=torch.int32), q.new_empty(chunks, H, KV)
+    key = (q.device, torch.cuda.current_stream(q.device).cuda_stream, chunks, H, KV, q.dtype)
+    ws = _GUARD_WS.get(key)
+    if ws is None:
+        if len(_GUARD_WS) >= 8:
+            _GUARD_WS.clear()
+        ws = _GUARD_WS[key] = (q.new_empty(chunks, H, dtype=torch.int32), q.new_empty(chunks, H, KV))
+    return ws
+
+
 def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,
-                        return_flags=False, states_out=None, head_gates=False):
+                        return_flags=False, states_out=None, head_gates=False, first_launch_only=False):
     """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
     With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
     single-reference range are detected on the device and recomputed exactly; ``return_flags``
@@ -181,8 +202,7 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     wide = hwide = None
     if exact_guard and V <= 128:
         chunks = plan.NT if plan is not None else B * (-(-T // BT))
-        wide = q.new_empty(chunks, H, dtype=torch.int32)
-        hwide = q.new_empty(chunks, H, K * V)
+        wide, hwide = _guard_workspaces(q, chunks, H, K * V, keep=return_flags)
     tail = (be.ptr(None if plan is None else plan.offsets), be.ptr(None if plan is None else plan.indices),
             be.ptr(None if plan is None else plan.chunk_offsets), be.ptr(None if plan is None else plan.seq_order),
             0 if plan is None else plan.NT,
@@ -201,6 +221,8 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
         be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
         states_out.append(hT)
+    elif first_launch_only:   # benchmark hook: the scan without the guard's second launch
+        be.check(be.lib().fla_chunk_gla_fwd_fused_first_launch(*head, *tail), "fla_chunk_gla_fwd_fused_first_launch")
     else:
         be.check(be.lib().fla_chunk_gla_fwd_fused(*head, *tail), "fla_chunk_gla_fwd_fused")
     if return_flags:
@@ -214,10 +236,13 @@ def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, 
     gate-range flags of the fused kernel are appended to it, with a list ``states_out`` the per-chunk
     states it kept for the backward pass."""
     if fused and not want_A and q.shape[-1] in (64, 128):
+        if flags_out is None:
+            o, ht = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets,
+                                        states_out=states_out)
+            return o, ht, None
         o, ht, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets,
                                           return_flags=True, states_out=states_out)
-        if flags_out is not None:
-            flags_out.append(wide)
+        flags_out.append(wide)
         return o, ht, None
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     B, T, H, K = q.shape
@@ -337,8 +362,9 @@ class ChunkGLAFunction(torch.autograd.Function):
             v = _pad_dim(v, VP)
             if h0 is not None:
                 h0 = F.pad(h0, (0, VP - V, 0, KP - K))
-        flags = []
-        states = [] if KEEP_STATES_FOR_BACKWARD and any(ctx.needs_input_grad) else None
+        needs_grad = any(ctx.needs_input_grad)
+        flags = [] if needs_grad else None   # the backward pass reads the guard's flags
+        states = [] if KEEP_STATES_FOR_BACKWARD and needs_grad else None
         o, ht, _ = _gla_forward(q, k, v, g, scale, h0, output_final_state, offsets, flags_out=flags,
                                 states_out=states)
         # the inputs, the small table of chunks whose gates need the exact intra-chunk arithmetic, and

@@ -167,6 +167,16 @@ int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const v
                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                             float scale, fla_stream_t stream);
 
+/* Diagnostics: only the first of the two launches of fla_chunk_gla_fwd_fused (the scan, with the flag and
+ * state hand-over stores of the range guard when the workspaces are given), so that a benchmark can put
+ * events round the dominant kernel in the form the operator runs.  o is incomplete for flagged chunks. */
+int fla_chunk_gla_fwd_fused_first_launch(const void* q, const void* k, const void* v, const void* gates,
+                                         const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                         const int64_t* offsets, const int64_t* indices,
+                                         const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                                         int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
+                                         int64_t V, int64_t N, float scale, fla_stream_t stream);
+
 /* The same launch for a forward pass whose states are kept for the backward pass: additionally
  * writes the state entering every chunk to h_frag_t ([chunks, H, K*V] in the q/k/v dtype,
  * FLA_H_FRAGMENT_T order), i.e. what fla_chunk_gla_fwd_h would recompute for fla_chunk_gla_bwd
