@@ -34,6 +34,7 @@ for _p in (ROOT, os.path.join(ROOT, "flash-linear-attention_amd")):
 MFMA_PEAK_FLOPS = 2.5e15   # dense bf16 MFMA, FLOP/s
 HBM_PEAK_GBS = 8000.0
 MIB = 1 << 20
+RAMP_SECONDS = 0.5         # untimed load ahead of the warm-up steps (clock ramp)
 
 
 def _events(n):
@@ -120,6 +121,15 @@ def bench_gla(device, steps, warmup):
 
     def step():
         return chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
+
+    # The clocks of an idle GPU need a few hundred milliseconds of load to reach their steady state (the
+    # first launches after idle run about 25 % slower): keep the device busy with the step itself for
+    # RAMP_SECONDS before the warm-up steps, whatever --warmup says.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < RAMP_SECONDS:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
 
     # `warmup` untimed steps, then exactly `steps` steps between two synchronisations, each step between
     # two HIP events on the launch stream.  value = tokens / median step time; the wall time of the same
