@@ -9,6 +9,7 @@ extern "C" const char* fla_error_string(int code) {
     case FLA_E_INVALID: return "fla_hip: invalid argument (null pointer, negative size or inconsistent shapes)";
     case FLA_E_UNSUPPORTED: return "fla_hip: shape, dtype or chunk size not supported by the gfx950 kernels";
     case FLA_E_ALIGNMENT: return "fla_hip: pointer or row pitch not aligned for vector access";
+    case FLA_E_SCRATCH: return "fla_hip: input larger than the static scratch buffer of the allocation-free entry point";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);

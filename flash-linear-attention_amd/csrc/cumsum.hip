@@ -6,6 +6,8 @@
 // reads 64*VEC contiguous elements per row.  The reference forms the same
 // sums with a [BT,BT] triangular-mask matmul (fla/ops/utils/cumsum.py:97-109);
 // a running sum in registers needs no matrix unit and no LDS.
+#include <mutex>
+
 #include "fla_common.h"
 
 namespace {
@@ -223,4 +225,57 @@ extern "C" int fla_chunk_global_cumsum(const void* s, float* ws_local, void* out
     case FLA_F16: return launch_carry<f16>(ws_local, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
     default: return FLA_E_UNSUPPORTED;
   }
+}
+
+// ---------------------------------------------------------------------------
+// fla_chunk_global_cumsum for callers that cannot allocate (code under HIP graph capture, serving
+// loops, harnesses that forbid hipMalloc): the chunk-local sums of the first pass live in a
+// file-scope device array instead of a caller workspace.  Each GPU holds its own copy of the array
+// at its own address, so the address is looked up once per device (hipGetSymbolAddress with that
+// device current) and only that pointer is handed to the kernels; the array's name itself is a
+// host-side stand-in and never a kernel argument.  Every element the second pass reads has been
+// written by the first pass of the same call, so nothing needs clearing between calls.  All calls
+// on one GPU share the array: calls that overlap on one GPU (different streams) race.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[FLA_STATIC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices];   // per device; written once under g_scratch_mu
+std::mutex g_scratch_mu;
+
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return FLA_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return FLA_E_INVALID;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FLA_OK;
+}
+}  // namespace
+
+extern "C" int fla_chunk_global_cumsum_static(const void* s, void* out, int s_dtype, int out_dtype, int64_t B, int64_t T,
+                                              int64_t H, int64_t S, int64_t chunk_size, int reverse,
+                                              const int64_t* offsets, const int64_t* indices, int64_t NT,
+                                              fla_stream_t stream) {
+  FLA_REQUIRE(s && out, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H >= 0 && S >= 1, FLA_E_INVALID);
+  // sizes first: an input that does not fit is refused before anything touches the device
+  const int64_t cap = FLA_STATIC_SCRATCH_FLOATS;
+  if (B > 0 && T > 0 && H > 0) {
+    FLA_REQUIRE(B <= cap && T <= cap / B && H <= cap / (B * T) && S <= cap / (B * T * H), FLA_E_SCRATCH);
+  }
+  float* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc) return rc;
+  return fla_chunk_global_cumsum(s, ws, out, s_dtype, out_dtype, B, T, H, S, chunk_size, reverse, offsets, indices, NT,
+                                 stream);
 }

@@ -30,6 +30,7 @@ SIGNATURES = {
     "fla_prepare_chunk_indices": (c_int, [P, I64, I64, P, P]),
     "fla_chunk_local_cumsum": (c_int, [P, P, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
     "fla_chunk_global_cumsum": (c_int, [P, P, P, I, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
+    "fla_chunk_global_cumsum_static": (c_int, [P, P, I, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
     "fla_fused_recurrent_fwd": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                         I64, I64, I64, I64, I64, I64, F, I, P]),
     "fla_fused_recurrent_gated_delta_rule_fwd": (c_int, [P, P, P, P, P, P, P, P, P, I, I, I, I,

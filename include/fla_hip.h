@@ -33,7 +33,8 @@ enum fla_error {
   FLA_OK = 0,
   FLA_E_INVALID = -1,     /* null pointer / negative size / inconsistent arguments */
   FLA_E_UNSUPPORTED = -2, /* shape, dtype or chunk size outside what the kernels cover */
-  FLA_E_ALIGNMENT = -3    /* pointer or row pitch not aligned for vector access */
+  FLA_E_ALIGNMENT = -3,   /* pointer or row pitch not aligned for vector access */
+  FLA_E_SCRATCH = -4      /* input larger than the library's static scratch buffer (allocation-free entry point) */
 };
 
 typedef void* fla_stream_t; /* hipStream_t */
@@ -76,6 +77,19 @@ int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype,
 int fla_chunk_global_cumsum(const void* s, float* ws_local, void* out, int s_dtype, int out_dtype, int64_t B,
                             int64_t T, int64_t H, int64_t S, int64_t chunk_size, int reverse,
                             const int64_t* offsets, const int64_t* indices, int64_t NT, fla_stream_t stream);
+
+/* fla_chunk_global_cumsum without the workspace argument, for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference (whose wrapper allocates its intermediates with torch).  The chunk-local sums go through a
+ * static device array of FLA_STATIC_SCRATCH_FLOATS fp32 elements (16 MiB, held by every GPU the library
+ * runs on until the process ends); B*T*H*S beyond that returns FLA_E_SCRATCH and launches nothing.  The
+ * call allocates nothing; its first call on a device looks the array's address up (do that call outside
+ * graph capture, with the stream's device current).  All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams) race.  Same kernels and results as fla_chunk_global_cumsum. */
+#define FLA_STATIC_SCRATCH_FLOATS (4 * 1024 * 1024)
+int fla_chunk_global_cumsum_static(const void* s, void* out, int s_dtype, int out_dtype, int64_t B, int64_t T,
+                                   int64_t H, int64_t S, int64_t chunk_size, int reverse, const int64_t* offsets,
+                                   const int64_t* indices, int64_t NT, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Token-by-token recurrence, forward (fla/ops/common/fused_recurrent.py:322-378,

@@ -50,6 +50,9 @@ def test_argument_validation_without_device():
     assert lib.fla_chunk_local_cumsum(p, p, 7, 1, 0, 1, 1, 64, 0, None, None, 0, None) == -2     # unknown dtype
     assert lib.fla_chunk_gla_fwd_h(p, p, p, 0, None, p, None, None, None, 1, 0, 1, 1, 1, 64, 1, 100, 64, 1, None) == -2
     assert lib.fla_selftest_mfma(p, p, p, 33, 32, 32, 0, None) == -2
+    # the allocation-free cumsum refuses what its static scratch array (4 Mi floats) cannot hold
+    assert lib.fla_chunk_global_cumsum_static(p, p, 0, 0, 1, 4 * 1024 * 1024 // 64 + 1, 8, 8, 64, 0, None, None, 0, None) == -4
+    assert lib.fla_chunk_global_cumsum_static(None, p, 0, 0, 1, 1, 1, 1, 64, 0, None, None, 0, None) == -1
 
 
 @pytest.mark.parametrize("bt", [16, 64])
