@@ -251,11 +251,16 @@ def bench_decode(device, steps=1000):
 
 
 def bench_gdr(device, steps=50, warmup=20):
-    """chunk_gated_delta_rule forward: the packed workload (packed, 12 sequences, 32768 tokens)
-    and the fixed-length shape B=8, T=4096 of the headline metric."""
+    """chunk_gated_delta_rule forward: the packed workload (12 sequences, 32768 tokens) and the
+    fixed-length shape B=8, T=4096 of the headline metric.  Each row carries a roofline block for its
+    dominant kernel (the serial scan, gdr_fwd_scan_kernel) and the time of the chunk-parallel launch
+    that precedes it (gdr_fwd_prep_kernel), both from HIP events round the single launch."""
     import torch
     import torch.nn.functional as F
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_scan
     from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_scan_operands
+    from fla_amd.utils import VarlenPlan
     torch.manual_seed(0)
     T, H, K, V, N = 32768, 16, 128, 128, 12
     lens = torch.randint(256, 6001, (N,)).double()
@@ -267,31 +272,57 @@ def bench_gdr(device, steps=50, warmup=20):
     v = torch.randn(1, T, H, V, device=device).bfloat16()
     g = F.logsigmoid(torch.randn(1, T, H, device=device))
     beta = torch.randn(1, T, H, device=device).sigmoid()
-    # q, k, v, o in 16 bit + g, beta fp32 + the final states: what the operator must move
+    scale = K ** -0.5
+    # q, k, v, o in 16 bit + g, beta fp32 (+ the final states): what the operator must move
     floor = 4 * T * H * K * 2 + 2 * T * H * 4
     # state products 6KV, the chunk-local products 3*2*BT*K + 2*2*BT*V, and the 64x64 triangular solve per chunk
     gdr_flops = T * H * (6 * K * V + 6 * 64 * K + 4 * 64 * V + 5500)
     out = {}
-    st = event_stats(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs,
-                                                    head_first=False), steps, warmup)
-    us = st["median_us"]
-    out["config2_varlen"] = {"us": round(us, 1), **spread(st), "tokens_per_s": round(T / (us * 1e-6), 1),
-                             "sequence_lengths": lens.tolist(),
-                             "operator_floor_bytes": floor + N * H * K * V * 4,
-                             "frac_of_hbm_peak": round((floor + N * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                             "algorithmic_flops": gdr_flops,
-                             "frac_of_mfma_peak": round(gdr_flops / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
+
+    def row(name, fn, prep, scan, n_states, chunks, tokens):
+        st = event_stats(fn, steps, warmup)
+        us = st["median_us"]
+        st_p = event_stats(prep, steps, 5)
+        st_s = event_stats(scan, steps, 5)
+        state_bytes = n_states * H * K * V * 4
+        tri = chunks * H * 2 * 10 * 256 * 2                     # the packed triangular tiles
+        # algorithmic bytes of each launch: every operand read once, every result written once
+        bytes_prep = 2 * T * H * K * 2 + 2 * T * H * 4 + T * H * 4 + tri          # q, k, g, beta in; gamma, tiles out
+        bytes_scan = 4 * T * H * K * 2 + T * H * 4 + tri + state_bytes            # q, k, v, gamma, tiles in; o, ht out
+        ach = bytes_scan / (st_s["median_us"] * 1e-6) / 1e9
+        out[name] = {
+            "us": round(us, 1), **spread(st), "tokens_per_s": round(tokens / (us * 1e-6), 1),
+            "operator_floor_bytes": floor + state_bytes,
+            "frac_of_hbm_peak": round((floor + state_bytes) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "algorithmic_flops": gdr_flops, "frac_of_mfma_peak": round(gdr_flops / (us * 1e-6) / MFMA_PEAK_FLOPS, 4),
+            "roofline": {"kernel": "gdr_fwd_scan_kernel", "bound": "hbm", "achieved": round(ach, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4),
+                         "traffic": counter_traffic("roofline:gdr_fwd_scan_kernel:" + name),
+                         "avg_us": round(st_s["median_us"], 1), "bytes_per_launch": bytes_scan, **spread(st_s)},
+            "gdr_fwd_prep_kernel": {"avg_us": round(st_p["median_us"], 1), "bytes_per_launch": bytes_prep,
+                                    "GBs": round(bytes_prep / (st_p["median_us"] * 1e-6) / 1e9, 1),
+                                    "traffic": counter_traffic("roofline:gdr_fwd_prep_kernel:" + name),
+                                    **spread(st_p)},
+            "launches_bytes_total": bytes_prep + bytes_scan}
+
+    plan = VarlenPlan(offs, 64)
+    AT, gc = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=plan.offsets, indices=plan.indices)
+    row("config2_varlen",
+        lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs, head_first=False),
+        lambda: fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=plan.offsets, indices=plan.indices),
+        lambda: chunk_gated_delta_rule_fwd_scan(q, k, v, AT, gc, scale, None, True, offsets=plan.offsets,
+                                                chunk_offsets=plan.chunk_offsets, seq_order=plan.seq_order),
+        N, plan.NT, T)
+    out["config2_varlen"]["sequence_lengths"] = lens.tolist()
     B, T2 = 8, 4096
     q, k, v = (x.view(B, T2, H, -1) for x in (q, k, v))
     g, beta = g.view(B, T2, H), beta.view(B, T2, H)
-    st = event_stats(lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
-                     steps, warmup)
-    us = st["median_us"]
-    out["B8_T4096"] = {"us": round(us, 1), **spread(st), "tokens_per_s": round(B * T2 / (us * 1e-6), 1),
-                       "operator_floor_bytes": floor + B * H * K * V * 4,
-                       "frac_of_hbm_peak": round((floor + B * H * K * V * 4) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                       "algorithmic_flops": gdr_flops,
-                       "frac_of_mfma_peak": round(gdr_flops / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
+    AT, gc = fwd_prepare_scan_operands(q, k, beta, g, scale)
+    row("B8_T4096",
+        lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
+        lambda: fwd_prepare_scan_operands(q, k, beta, g, scale),
+        lambda: chunk_gated_delta_rule_fwd_scan(q, k, v, AT, gc, scale, None, True),
+        B, B * T2 // 64, B * T2)
     return out
 
 

@@ -23,49 +23,9 @@
 //                       exponent is <= 0 whatever the gate magnitude.
 #include <type_traits>
 
-#include "fla_common.h"
-#include "mfma_tiles.h"
+#include "chunk_common.h"
 
 namespace {
-
-// A word of zeros in device memory: where the gate loads of a call without gates point, so that
-// the loaded value needs no select (a select right behind a load makes the wave wait for it).
-__device__ float kZeroWord = 0.f;  // never written; not const, so that it lives in the global address space like the tensors
-
-constexpr int BT = 64;
-constexpr int LDT = BT + 8;  // pitch of time-contiguous 16-bit tiles
-constexpr int LDM = BT + 4;  // pitch of fp32 64x64 tiles
-
-FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
-  if (total % 8 != 0) return id;
-  return (id % 8) * (total / 8) + id / 8;
-}
-
-struct ChunkLoc {
-  int64_t row0;   // first token row of the chunk in the flattened [B*T] space
-  int L;          // valid rows
-  int64_t cglob;  // global chunk index (addresses per-chunk states)
-};
-
-FLA_DEVICE ChunkLoc locate_chunk(const int64_t* offsets, const int64_t* indices, int64_t T, int ntfix, int64_t cidx) {
-  ChunkLoc c;
-  int64_t bos, len, ic;
-  if (offsets) {
-    int64_t n = indices[2 * cidx];
-    ic = indices[2 * cidx + 1];
-    bos = offsets[n];
-    len = offsets[n + 1] - bos;
-  } else {
-    bos = (cidx / ntfix) * T;
-    ic = cidx % ntfix;
-    len = T;
-  }
-  c.row0 = bos + ic * BT;
-  int64_t rem = len - ic * BT;
-  c.L = (int)(rem < BT ? rem : BT);
-  c.cglob = cidx;
-  return c;
-}
 
 struct WyParams {
   const void* k;
@@ -76,9 +36,6 @@ struct WyParams {
   void* u;
   void* Aw;
   void* Au;
-  const void* q;  // optional: with Aqk, also emit the gated causal scores of the chunk
-  void* Aqk;      // [rows, H, 64]: scale * (q_i . k_j) e^{gamma_i - gamma_j} for j <= i, else 0
-  float scale;
   const int64_t* offsets;
   const int64_t* indices;
   int64_t T;
@@ -149,6 +106,58 @@ FLA_DEVICE void wy_stage_t(T* dstT, const typename Elem<T>::v4* reg, const float
   }
 }
 
+// X = (I + M)^-1 for a strictly lower triangular fp32 M [64][LDM] in LDS, into sX [64][LDM]
+// (lower triangle valid; the upper right quadrant is used as scratch and holds garbage afterwards).
+// 16x16 diagonal blocks by forward substitution, then block merges X_ba = -X_bb (M_ba X_aa) on the
+// fp32 matrix instruction.  Called by all 256 threads after a barrier behind the writes of M; ends
+// with a barrier, after which X is complete.  The barriers order LDS traffic only.
+FLA_DEVICE void wy_invert(const float* sM, float* sX, int tid) {
+  const int lane = tid & 63, wave = tid >> 6;
+  float* sT = sX + 32;  // rows 0..31, columns 32..63 of X
+  // the 16x16 blocks (0,1) and (2,3) of X are read by the 32x32 merges but never written
+  for (int e = tid; e < 512; e += 256) {
+    int blk = e >> 8, i = (e >> 4) & 15, j = e & 15;
+    sX[(32 * blk + i) * LDM + 32 * blk + 16 + j] = 0.f;
+  }
+  // 16x16 diagonal blocks by forward substitution (one lane per column)
+  if (tid < 64) {
+    const int b = tid >> 4, col = tid & 15;
+    const float* Mb = sM + (16 * b) * LDM + 16 * b;
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float m[16];
+#pragma unroll
+      for (int q = 0; 4 * q < i; ++q) *(f32x4*)&m[4 * q] = *(const f32x4*)&Mb[i * LDM + 4 * q];
+      float s = (i == col) ? 1.f : 0.f;
+#pragma unroll
+      for (int j = 0; j < i; ++j) s -= m[j] * x[j];
+      x[i] = s;
+      if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // keeps the row loads of later rows from piling up in registers
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sX[(16 * b + i) * LDM + 16 * b + col] = x[i];
+  }
+  lds_barrier();
+  // ---- 32x32 diagonal blocks: X_ba = -X_bb (M_ba X_aa) for the block pairs (1,0) and (3,2)
+  {
+    const int a0 = 32 * (wave & 1), b0 = a0 + 16;  // waves 0 and 1 take one pair each
+    if (wave < 2) lds_mm16_f32(sM + b0 * LDM + a0, LDM, sX + a0 * LDM + a0, LDM, sT + 16 * wave, LDM, 16, 1.f, lane);
+    lds_barrier();
+    if (wave < 2) lds_mm16_f32(sX + b0 * LDM + b0, LDM, sT + 16 * wave, LDM, sX + b0 * LDM + a0, LDM, 16, -1.f, lane);
+  }
+  lds_barrier();
+  // ---- 64x64: X_BA = -X_BB (M_BA X_AA), one 16x16 output tile per wave
+  {
+    const int i0 = 16 * (wave >> 1), j0 = 16 * (wave & 1);
+    lds_mm16_f32(sM + (32 + i0) * LDM, LDM, sX + j0, LDM, sT + i0 * LDM + j0, LDM, 32, 1.f, lane);
+    lds_barrier();
+    lds_mm16_f32(sX + (32 + i0) * LDM + 32, LDM, sT + j0, LDM, sX + (32 + i0) * LDM + j0, LDM, 32, -1.f, lane);
+  }
+  lds_barrier();
+
+}
+
 // The inversion keeps M and X = (I + M)^-1 in fp32.  Two LDS regions are
 // reused over the kernel's life so that four workgroups fit a CU:
 //   region A: k row-major -> M (fp32) -> Aw | Au (16-bit)
@@ -179,16 +188,14 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
   T* sAw = (T*)sRA;
   T* sAu = sAw + BT * LDT;
   float* sX = (float*)sRB;
-  float* sT = sX + 32;  // rows 0..31, columns 32..63 of X
   T* sXbT = (T*)sRB;    // (beta k)^T, later (beta v)^T
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   // workgroups that run together take different heads of the same chunks: their rows are
   // adjacent in memory, so the traffic spreads over all memory channels
   const int H = p.H;
-  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
-  const int hh = (int)(lin % H);
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, lin / H);
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -196,17 +203,6 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
   const int rg = tid / CG, c4 = (tid % CG) * 4;
   const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
   v4 kreg[RPT], vreg[RPTV];
-  const bool scores = p.q != nullptr;  // uniform over the launch
-  if (scores) {
-    const T* qp = (const T*)p.q + (row0 * H + hh) * (int64_t)K + c4;
-    T* sQ = (T*)sRB;
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      v4 qv = *(const v4*)(qp + (int64_t)(row < L ? row : L - 1) * H * K);
-      *(v4*)&sQ[row * LDK + c4] = row < L ? qv : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-    }
-  }
   {
     const T* kp = (const T*)p.k + (row0 * H + hh) * (int64_t)K + c4;
     const T* vp = (const T*)p.v + (row0 * H + hh) * (int64_t)V + cv4;
@@ -240,30 +236,7 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
       for (int ks = 0; ks < K; ks += 16)
         s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
     }
-    // transposed scores (k q^T): a lane ends up with four consecutive j of one row i
-    f32x16 sq = zero16();
-    if (scores && qj <= qi) {
-      const T* sQ = (const T*)sRB;
-#pragma unroll
-      for (int ks = 0; ks < K; ks += 16)
-        sq = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qj * 32, ks, lane), lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), sq);
-    }
-    __syncthreads();  // k (and q) row-major fully consumed: their storage becomes M (and the score tile)
-    if (scores) {
-      T* sPo = (T*)sRB;
-      const int i = qi * 32 + (lane & 31);
-      const float gi = sGam[i];
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        v4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          int j = qj * 32 + 8 * r4 + 4 * (lane >> 5) + e;
-          o[e] = (T)((qj <= qi && j <= i) ? p.scale * sq[4 * r4 + e] * __expf(gi - sGam[j]) : 0.f);
-        }
-        *(v4*)&sPo[i * LDT + qj * 32 + 8 * r4 + 4 * (lane >> 5)] = o;
-      }
-    }
+    __syncthreads();  // k row-major fully consumed: its storage becomes M
     if (qj <= qi) {
       const int j = qj * 32 + (lane & 31);
 #pragma unroll
@@ -272,60 +245,10 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
         sM[i * LDM + j] = (j < i) ? sBeta[i] * s[r] : 0.f;
       }
     }
-    if (scores) {
-      __syncthreads();
-      const T* sPo = (const T*)sRB;
-      T* ap = (T*)p.Aqk + (row0 * H + hh) * (int64_t)BT;
-#pragma unroll
-      for (int e = tid; e < BT * 8; e += 256) {
-        int i = e >> 3, c8 = (e & 7) * 8;
-        if (i < L) *(v8*)(ap + (int64_t)i * H * BT + c8) = *(const v8*)&sPo[i * LDT + c8];
-      }
-      __syncthreads();  // score tile stored: region B becomes X
-    }
-    // the 16x16 blocks (0,1) and (2,3) of X are read by the 32x32 merges but never written
-    for (int e = tid; e < 512; e += 256) {
-      int blk = e >> 8, i = (e >> 4) & 15, j = e & 15;
-      sX[(32 * blk + i) * LDM + 32 * blk + 16 + j] = 0.f;
-    }
   }
   __syncthreads();
 
-  // ---- (I + M)^-1: 16x16 diagonal blocks by forward substitution (one lane per column)
-  if (tid < 64) {
-    const int b = tid >> 4, col = tid & 15;
-    const float* Mb = sM + (16 * b) * LDM + 16 * b;
-    float x[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float m[16];
-#pragma unroll
-      for (int q = 0; 4 * q < i; ++q) *(f32x4*)&m[4 * q] = *(const f32x4*)&Mb[i * LDM + 4 * q];
-      float s = (i == col) ? 1.f : 0.f;
-#pragma unroll
-      for (int j = 0; j < i; ++j) s -= m[j] * x[j];
-      x[i] = s;
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sX[(16 * b + i) * LDM + 16 * b + col] = x[i];
-  }
-  __syncthreads();
-  // ---- 32x32 diagonal blocks: X_ba = -X_bb (M_ba X_aa) for the block pairs (1,0) and (3,2)
-  {
-    const int a0 = 32 * (wave & 1), b0 = a0 + 16;  // waves 0 and 1 take one pair each
-    if (wave < 2) lds_mm16_f32(sM + b0 * LDM + a0, LDM, sX + a0 * LDM + a0, LDM, sT + 16 * wave, LDM, 16, 1.f, lane);
-    __syncthreads();
-    if (wave < 2) lds_mm16_f32(sX + b0 * LDM + b0, LDM, sT + 16 * wave, LDM, sX + b0 * LDM + a0, LDM, 16, -1.f, lane);
-  }
-  __syncthreads();
-  // ---- 64x64: X_BA = -X_BB (M_BA X_AA), one 16x16 output tile per wave
-  {
-    const int i0 = 16 * (wave >> 1), j0 = 16 * (wave & 1);
-    lds_mm16_f32(sM + (32 + i0) * LDM, LDM, sX + j0, LDM, sT + i0 * LDM + j0, LDM, 32, 1.f, lane);
-    __syncthreads();
-    lds_mm16_f32(sX + (32 + i0) * LDM + 32, LDM, sT + j0, LDM, sX + (32 + i0) * LDM + j0, LDM, 32, -1.f, lane);
-  }
-  __syncthreads();
+  wy_invert(sM, sX, tid);
 
   // ---- Aw, Au in 16-bit (LDS for the products, optionally global for the backward pass)
   {
@@ -377,6 +300,250 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
   __syncthreads();
   wy_store<T, K>(sWo, (T*)p.w + (row0 * H + hh) * (int64_t)K, (int64_t)H * K, L, tid);
   wy_store<T, V>(sUo, (T*)p.u + (row0 * H + hh) * (int64_t)V, (int64_t)H * V, L, tid);
+}
+
+// ---------------------------------------------------------------------------
+// Chunk-parallel preparation for the one-pass forward (fla_chunk_gated_delta_rule_fwd_scan): per
+// (chunk, head) the two lower-triangular 64x64 matrices the scan applies to value-column slabs,
+//   Tu  = (Aw * Gamma) diag(beta)        Tu_ij  = Aw_ij e^{gamma_i - gamma_j} beta_j   (j <= i)
+//   Aqk = scale tril(q k^T * Gamma)      Aqk_ij = scale (q_i . k_j) e^{gamma_i - gamma_j}
+// With them  v_new = u - e^{gamma} (w h) = Tu (v - e^{gamma} (k h))  (u = Tu v and
+// e^{gamma} w = Tu diag(e^{gamma}) k, since Aw Gamma-scaling is D Aw D^-1 and diagonal matrices
+// commute), so neither w nor u is formed and the scan reads k, q, v and these 10 KB instead of
+// k, q, w, u and a 8 KB score tile.  Only the ten 16x16 blocks on and below the diagonal are stored,
+// block (tt, jb) at index tt (tt + 1) / 2 + jb, each block row-major: at [chunk, head, {Tu, Aqk}, 10, 16, 16].
+// Rows past the end of a short chunk come out as zeros (beta and q are zero there).
+struct PrepParams {
+  const void* q;
+  const void* k;
+  const float* beta;
+  const float* g;      // raw log-gates [rows, H] (g_is_cumsum == 0) or their chunk-local prefix sums, or NULL
+  int g_is_cumsum;
+  float* gam_out;      // [rows, H]: the chunk-local prefix sums (written when g is raw), or NULL
+  void* AT;
+  float scale;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+};
+
+constexpr int kPrepWorkgroups = 3 * 256;        // three resident workgroups (register budget) on each of the 256 CUs
+constexpr int kTriBlocks = 10;                   // 16x16 blocks on and below the diagonal of a 64x64 tile
+constexpr int kTriElems = kTriBlocks * 256;      // elements of one packed triangular tile
+FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
+
+// A workgroup walks several (chunk, head) items (grid-stride) and loads the q, k rows, beta and the gate
+// of its next item into registers once the matrix products of the current one have released their
+// accumulators: the loads land while the inversion runs (measured: worth about 4 %; the launch is a chain
+// of short dependent phases - removing the inversion, the stores or the loads each saves 15-20 % - rather
+// than bound by one resource).
+template <typename T, int K>
+__global__ __launch_bounds__(256, 3) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int R_BYTES = BT * LDK * 2 > BT * LDM * 4 ? BT * LDK * 2 : BT * LDM * 4;
+  __shared__ __attribute__((aligned(16))) char sRA[R_BYTES];   // k row-major -> M (fp32) -> packed Tu tile
+  __shared__ __attribute__((aligned(16))) char sRB[R_BYTES];   // q row-major -> X (fp32)
+  __shared__ __attribute__((aligned(16))) T sPo[kTriElems];    // packed score tile
+  __shared__ __attribute__((aligned(16))) float sBeta[BT];
+  __shared__ __attribute__((aligned(16))) float sGam[BT];
+  T* sK = (T*)sRA;
+  float* sM = (float*)sRA;
+  T* sQ = (T*)sRB;
+  T* sTu = (T*)sRA;
+  float* sX = (float*)sRB;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H;
+  // 16-byte pieces: a lane owns 8 adjacent columns of NPL rows
+  constexpr int C8 = K / 8, RPP = 256 / C8, NPL = BT / RPP;
+  const int r0 = tid / C8, c8 = (tid % C8) * 8;
+  const uint32_t pitch = (uint32_t)H * K * 2;   // bytes between rows of one head
+  uint32_t off[NPL];
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) off[i] = (uint32_t)(r0 + RPP * i) * pitch + c8 * 2;
+  const v8 z = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+
+  struct Item {
+    int L, hh;
+    int64_t row0, cglob;
+    v8 q[NPL], k[NPL];
+    float beta, g;   // wave 0: this lane's row
+  };
+  // Items are numbered head-fastest: item = chunk * H + head.  The walk keeps (chunk, head) and advances
+  // them by the grid size without a division; the chunk's place in its sequence comes from 32-bit
+  // arithmetic on wave-uniform values (scalar loads for a packed batch).
+  const uint32_t step_c = gridDim.x / (uint32_t)H, step_h = gridDim.x % (uint32_t)H;
+  uint32_t it_chunk = blockIdx.x / (uint32_t)H, it_head = blockIdx.x % (uint32_t)H;
+  auto fetch = [&](Item& it) __attribute__((always_inline)) {
+    const uint32_t cidx = __builtin_amdgcn_readfirstlane(it_chunk);
+    const int hh = (int)__builtin_amdgcn_readfirstlane(it_head);
+    ChunkLoc cl;
+    {
+      int64_t bos, len;
+      uint32_t ic;
+      if (p.offsets) {
+        const int64_t n = p.indices[2 * (int64_t)cidx];
+        ic = (uint32_t)p.indices[2 * (int64_t)cidx + 1];
+        bos = p.offsets[n];
+        len = p.offsets[n + 1] - bos;
+      } else {
+        const uint32_t b = cidx / (uint32_t)p.NTfix;
+        ic = cidx - b * (uint32_t)p.NTfix;
+        bos = (int64_t)b * p.T;
+        len = p.T;
+      }
+      cl.row0 = bos + (int64_t)ic * BT;
+      const int64_t rem = len - (int64_t)ic * BT;
+      cl.L = (int)(rem < BT ? rem : BT);
+      cl.cglob = cidx;
+    }
+    it.L = cl.L;
+    it.hh = hh;
+    it.row0 = cl.row0;
+    it.cglob = cl.cglob;
+    const char* qp = (const char*)p.q + (cl.row0 * H + hh) * (int64_t)K * 2;
+    const char* kp = (const char*)p.k + (cl.row0 * H + hh) * (int64_t)K * 2;
+    const uint32_t lim = (uint32_t)(cl.L - 1) * pitch + c8 * 2;   // rows past the end: re-read the last one
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const uint32_t o = off[i] < lim ? off[i] : lim;
+      it.q[i] = *(const v8*)(qp + o);
+      it.k[i] = *(const v8*)(kp + o);
+    }
+    if (wave == 0) {
+      const int64_t gi = (cl.row0 + (lane < cl.L ? lane : cl.L - 1)) * H + hh;
+      it.beta = p.beta[gi];
+      it.g = p.g ? p.g[gi] : 0.f;
+    }
+  };
+
+  auto advance = [&]() {
+    it_chunk += step_c;
+    it_head += step_h;
+    if (it_head >= (uint32_t)H) {
+      it_head -= (uint32_t)H;
+      ++it_chunk;
+    }
+  };
+  Item cur;
+  int64_t lin = blockIdx.x;
+  if (lin >= total) return;
+  fetch(cur);
+  for (;;) {
+    const int L = cur.L;
+    const int hh = cur.hh;
+    const int64_t row0 = cur.row0, cglob = cur.cglob;
+    // ---- q, k row-major (rows past the end of the chunk zero), beta, gamma
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+      const int row = r0 + RPP * i;
+      *(v8*)&sQ[row * LDK + c8] = row < L ? cur.q[i] : z;
+      *(v8*)&sK[row * LDK + c8] = row < L ? cur.k[i] : z;
+    }
+    if (wave == 0) {
+      const bool ok = lane < L;
+      sBeta[lane] = ok ? cur.beta : 0.f;
+      float gam = cur.g;   // a cumulative gate: rows past the end carry the last valid row's
+      if (p.g && !p.g_is_cumsum) {
+        // inclusive prefix sum over the 64 rows: DPP row scans plus the totals of the earlier rows of 16;
+        // rows past the end add zero, so they carry the last valid row's sum
+        float x = row_prefix16(ok ? cur.g : 0.f);
+        const float t0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 15));
+        const float t1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 31));
+        const float t2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 47));
+        const int r = lane >> 4;
+        gam = x + (r >= 1 ? t0 : 0.f) + (r >= 2 ? t1 : 0.f) + (r >= 3 ? t2 : 0.f);
+        if (p.gam_out && ok) p.gam_out[(row0 + lane) * H + hh] = gam;
+      }
+      sGam[lane] = gam;
+    }
+    lds_barrier();   // LDS-only barriers throughout: a full one would wait for the loads issued further down
+    const int64_t next = lin + gridDim.x;
+    const bool more = next < total;   // workgroup-uniform
+
+    // ---- S = k k^T and the transposed scores k q^T on the lower-triangular 32x32 quadrants
+    const int qi = wave >> 1, qj = wave & 1;
+    f32x16 s = zero16(), sq = zero16();
+    if (qj <= qi) {
+#pragma unroll
+      for (int ks = 0; ks < K; ks += 16) {
+        const v8 kj = lds_frag32<T>(sK, LDK, qj * 32, ks, lane);
+        s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), kj, s);
+        sq = Elem<T>::mfma32(kj, lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), sq);
+      }
+    }
+    lds_barrier();  // k and q row-major fully consumed: their storage becomes M and the packed score tile
+    if (qj <= qi) {
+      // sq: lane <-> row i, registers <-> four consecutive columns j per quad
+      const int i = qi * 32 + (lane & 31), tt = i >> 4;
+      const float gi = sGam[i];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int j0 = qj * 32 + 8 * r4 + 4 * (lane >> 5);
+        const f32x4 gj = *(const f32x4*)&sGam[j0];
+        v4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (T)(j0 + e <= i ? p.scale * sq[4 * r4 + e] * __expf(gi - gj[e]) : 0.f);
+        if ((j0 >> 4) <= tt) *(v4*)&sPo[tri_block(tt, j0 >> 4) * 256 + (i & 15) * 16 + (j0 & 15)] = o;
+      }
+      // s: lane <-> column j, registers <-> four consecutive rows i per quad
+      const int j = qj * 32 + (lane & 31);
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int ib = qi * 32 + 8 * r4 + 4 * (lane >> 5);
+        const f32x4 b = *(const f32x4*)&sBeta[ib];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sM[(ib + e) * LDM + j] = (j < ib + e) ? b[e] * s[4 * r4 + e] : 0.f;
+      }
+    }
+    lds_barrier();  // M complete; region B becomes X
+    // the next item's rows start their way to the registers now: the matrix products above no longer
+    // hold their accumulators, and the inversion below needs few registers and no memory
+    if (more) {
+      advance();
+      fetch(cur);
+    }
+
+    wy_invert(sM, sX, tid);
+
+    // ---- Tu = (X * Gamma) diag(beta), one 16-element block row per thread, straight to memory
+    {
+      const int i = tid >> 2, jb = tid & 3, tt = i >> 4;
+      if (jb <= tt) {
+        const float gi = sGam[i];
+        v8 tu[2];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4 xv = *(const f32x4*)&sX[i * LDM + 16 * jb + 4 * q4];
+          const f32x4 gj = *(const f32x4*)&sGam[16 * jb + 4 * q4];
+          const f32x4 bj = *(const f32x4*)&sBeta[16 * jb + 4 * q4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int jj = 4 * q4 + e, j = 16 * jb + jj;
+            tu[jj >> 3][jj & 7] = (T)(j <= i ? xv[e] * __expf(gi - gj[e]) * bj[e] : 0.f);
+          }
+        }
+        T* dst = sTu + tri_block(tt, jb) * 256 + (i & 15) * 16;   // M is dead: its storage takes the packed tile
+        *(v8*)dst = tu[0];
+        *(v8*)(dst + 8) = tu[1];
+      }
+    }
+    lds_barrier();
+    // both tiles leave as one contiguous 10 KB block, 16 bytes per lane
+    {
+      T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)(2 * kTriElems);
+      constexpr int NP = kTriElems / 8;   // 16-byte pieces per tile
+      for (int e = tid; e < 2 * NP; e += 256)
+        *(v8*)(at + e * 8) = e < NP ? *(const v8*)&sTu[e * 8] : *(const v8*)&sPo[(e - NP) * 8];
+    }
+    if (!more) break;
+    lin = next;
+    lds_barrier();  // the packed tiles are on their way: the tiles of the next item may be written
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -732,9 +899,8 @@ __global__ __launch_bounds__(256) void chunk_fwd_o_kernel(DOParams p) {
   // workgroups that run together take different heads of the same chunks: their rows are
   // adjacent in memory, so the traffic spreads over all memory channels
   const int H = p.H;
-  const int64_t lin = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
-  const int hh = (int)(lin % H);
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, lin / H);
+  int hh;
+  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -927,35 +1093,52 @@ int launch_do(const DOParams& p, int K, int V, dim3 grid, hipStream_t st) {
   return FLA_E_UNSUPPORTED;
 }
 
-int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B, int64_t T, int64_t H, int64_t NT,
-               dim3* grid, int* ntfix) {
-  if (offsets) FLA_REQUIRE(indices != nullptr && B == 1, FLA_E_INVALID);
-  int64_t nf = (T + BT - 1) / BT;
-  int64_t nblk = offsets ? NT : B * nf;
-  FLA_REQUIRE(nblk <= 0x7fffffffLL && H <= 65535, FLA_E_UNSUPPORTED);
-  *grid = dim3((unsigned)nblk, (unsigned)H);
-  *ntfix = (int)nf;
+template <typename T>
+int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
+  // (chunk, head) items, head-fastest; as many workgroups as are resident at once, each walking its share of the items
+  const int64_t total = (int64_t)chunk_grid_.x * chunk_grid_.y;
+  dim3 grid((unsigned)(total < kPrepWorkgroups ? total : kPrepWorkgroups));
+  if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64>), grid, dim3(256), 0, st, p, total);
+  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128>), grid, dim3(256), 0, st, p, total);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
 
 }  // namespace
 
+extern "C" int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
+                                float* g_cumsum_out, void* AT, float scale, const int64_t* offsets,
+                                const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                                int64_t K, fla_stream_t stream) {
+  FLA_REQUIRE(q && k && beta && AT, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)AT) % 16 == 0, FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  PrepParams p{q, k, beta, g, g_is_cumsum, g_cumsum_out, AT, scale, offsets, indices, T, (int)H, ntfix};
+  if (qkv_dtype == FLA_BF16) return launch_prep<bf16>(p, (int)K, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_prep<f16>(p, (int)K, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
 extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum, void* w, void* u,
-                              void* Aw, void* Au, const void* q, void* Aqk, float scale, const int64_t* offsets,
-                              const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
-                              int64_t K, int64_t V, fla_stream_t stream) {
+                              void* Aw, void* Au, const int64_t* offsets, const int64_t* indices, int64_t NT,
+                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                              fla_stream_t stream) {
   FLA_REQUIRE(k && v && beta && w && u, FLA_E_INVALID);
-  FLA_REQUIRE((q == nullptr) == (Aqk == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au |
-               (uintptr_t)q | (uintptr_t)Aqk) % 16 == 0,
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au) % 16 == 0,
               FLA_E_ALIGNMENT);
   dim3 grid;
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, q, Aqk, scale, offsets, indices, T, (int)H, ntfix};
+  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, offsets, indices, T, (int)H, ntfix};
   if (qkv_dtype == FLA_BF16) return launch_wy<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_wy<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

@@ -1,46 +1,30 @@
-// Fused gated-delta-rule forward for gfx950: state scan and output in one pass;
-// neither the per-chunk states nor v_new leave the chip.
+// One-pass gated-delta-rule forward for gfx950: state scan and output in one launch; neither w, u,
+// v_new nor the per-chunk states exist in memory.
 //
-// Inputs are the chunk-parallel products of fla_gdr_fwd_wy: w, u and the gated
-// causal scores Aqk, plus q, k and the chunk-local gate prefix sums gamma.
-// One workgroup of 8 waves owns one (sequence, head, 64 value columns) and walks the
+// Inputs are q, k, v, the chunk-local gate prefix sums gamma and the two packed triangular 64x64 tiles
+// per (chunk, head) that fla_gdr_fwd_prep leaves: Tu = (Aw * Gamma) diag(beta) and the gated causal
+// scores Aqk.  One workgroup of 8 waves owns one (sequence, head, 64 value columns) and walks the
 // chunks serially:
-//   waves 4-7 ("staging")  copy w, q, Aqk of chunk c+1 to LDS, transpose k and u into
-//                          time-contiguous tiles, and write the finished o tile of
-//                          chunk c-1 to global memory in whole 128-byte rows;
-//   waves 0-3 ("matrix")   each own 16 value columns of the fp32 state (all K rows, in
-//                          16x16 accumulator tiles).  The delta rule is independent per value
-//                          column, so a matrix wave never exchanges data with another:
-//                            v_new = u - e^{gamma} * (w h)
+//   waves 4-7 ("staging")  copy k, q and the triangular tiles of chunk c+1 to LDS, transpose k and v
+//                          into time-contiguous tiles, and write the finished o tile of chunk c-1 to
+//                          global memory;
+//   waves 0-3 ("matrix")   each own 16 value columns of the fp32 state (all K rows, in 16x16
+//                          accumulator tiles).  The delta rule is independent per value column, so a
+//                          matrix wave never exchanges data with another:
+//                            v_new = Tu (v - e^{gamma} * (k h))
 //                            o     = s e^{gamma} * (q h) + Aqk v_new
 //                            h    <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} * v_new)
-//                          (fla/ops/common/chunk_delta_h.py:71-119, chunk_o.py:68-101).
-//                          State and v_new go from accumulators straight back into MFMA
-//                          operands: the contraction index of the LDS-side operand is
-//                          permuted to the accumulator row order instead.
-// Operand tiles are double-buffered and the two groups meet at one barrier per chunk.
-// The o tile takes the place of the u tile it was computed from (same lanes, same
-// addresses), so it needs no storage of its own.
+//                          (fla/ops/common/chunk_delta_h.py:71-119, chunk_o.py:68-101; v_new equals the
+//                          reference's u - e^{gamma} (w h), see gdr_fwd.hip).  State, k h, the residual
+//                          and v_new go from accumulators straight back into MFMA operands: the
+//                          contraction index of the LDS-side operand is permuted to the accumulator
+//                          row order instead.
+// Operand tiles are double-buffered and the two groups meet at one barrier per chunk.  The o tile
+// takes the place of the v tile it was computed from (same lanes, same addresses), so it needs no
+// storage of its own.
 #include "chunk_common.h"
 
 namespace {
-
-struct GdrFusedParams {
-  const void* q;
-  const void* k;
-  const void* w;
-  const void* u;
-  const void* Aqk;
-  const float* gam;
-  const float* h0;
-  void* o;
-  float* ht;
-  const int64_t* offsets;
-  const int64_t* seq_order;  // sequence ids, longest first (or NULL)
-  int64_t T;
-  int H, V, N;
-  float scale;
-};
 
 // LDS tiles of this kernel.  Measured on gfx950 (one wave per SIMD): LDS reads peak at
 // 256 B/clk per CU, writes near 80 B/clk.  For the access shape of an MFMA operand
@@ -79,20 +63,57 @@ FLA_DEVICE typename Elem<T>::v8 frag16_t(const T* tile, int row0, int t0, int la
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Per chunk and workgroup the kernel reads q, k (16 KB each at K=128), its 64 value columns (8 KB) and
+// 10 KB of triangular blocks, and its time follows those bytes: the launch is bound by the rate at which
+// data reaches the CUs through L2, both value-column slabs of a head pulling q, k and the tiles.
+struct GdrScanParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* AT;   // [chunks, H, 2, 10, 16, 16]: Tu, Aqk
+  const float* gam;
+  const float* h0;
+  void* o;
+  float* ht;
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  const int64_t* seq_order;  // sequence ids, longest first (or NULL)
+  int64_t T;
+  int H, V, N;
+  float scale;
+};
+
+constexpr int kTriElems = 10 * 256;  // one packed triangular tile: ten 16x16 blocks
+
+// A operand (16 rows x 32 contraction indices in accumulator-row order) of row tile tt, column pair s,
+// from a packed triangular tile: block (tt, 2s) gives the first four indices of each group, block
+// (tt, 2s + 1) the second four; above the diagonal that block is not stored and reads as zero.  A
+// block is 512 contiguous bytes and the 64 lanes read each of its 8-byte pieces once.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag_tri(const T* tile, int tt, int s, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + (tt * (tt + 1) / 2 + 2 * s) * 256 + (lane & 15) * 16 + 4 * (lane >> 4);
+  v4 lo = *(lds_v4*)p;
+  v4 hi = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  if (2 * s + 1 <= tt) hi = *(lds_v4*)(p + 256);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 template <typename T, int K>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_fused_kernel(
-    GdrFusedParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
+    GdrScanParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int BV = 64;
-  constexpr int LDR = K + 8;  // pitch of the row-major w and q tiles
+  constexpr int LDR = K + 8;  // pitch of the row-major k and q tiles
   constexpr int KS = K / 32;  // 32-wide contraction slices of the state
   constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
-  __shared__ __attribute__((aligned(16))) T sW[2][BT * LDR];     // w    [t][k]
+  __shared__ __attribute__((aligned(16))) T sK[2][BT * LDR];     // k    [t][k]
   __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDR];     // q    [t][k]
-  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDT];   // k^T  [k][t]
-  __shared__ __attribute__((aligned(16))) T sUt[2][BV * LDT];  // u^T  [v][t], later o^T
-  __shared__ __attribute__((aligned(16))) T sP[2][BT * LDT];   // Aqk  [i][j]
+  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDT];     // k^T  [k][t]
+  __shared__ __attribute__((aligned(16))) T sVt[2][BV * LDT];    // v^T  [v][t], later o^T
+  __shared__ __attribute__((aligned(16))) T sAT[2][2 * kTriElems];  // Tu, Aqk (packed triangular tiles)
   __shared__ __attribute__((aligned(16))) float sEg[2][BT];      // e^{gamma_t}
   __shared__ __attribute__((aligned(16))) float sEd[2][BT];      // e^{gamma_last - gamma_t}
   __shared__ float sDec[2];                                      // e^{gamma_last}
@@ -110,71 +131,63 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int vbase = vb * BV;
   SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int nchunks = (int)((sp.len + BT - 1) / BT);
-  auto chunk_len = [&](int c) {
-    int64_t rem = sp.len - (int64_t)c * BT;
-    return (int)(rem < BT ? rem : BT);
-  };
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
 
   if (wave >= 4) {
     // =========================== staging waves ===========================
     if (nchunks == 0) return;
     const int st = tid - 256;
-    constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (w, q)
+    constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (q)
     constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;  // k: a lane owns RPT rows x 4 columns
+    constexpr int NPA = 2 * kTriElems / 4 / 256;             // 8-byte pieces of the triangular tiles per lane
+    static_assert(NPA * 256 * 4 == 2 * kTriElems, "the triangular tiles split evenly over the staging lanes");
     const int rg = st / CG, c4 = (st % CG) * 4;
-    const int urg = st >> 4, uc4 = (st & 15) * 4;            // u, o: a lane owns 4 rows x 4 columns
-    const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V, HB = (uint32_t)H * BT;
-    // 16-byte pieces of the w/q tiles: row and first column of piece e
-    auto wq_row = [&](int e) { return e / C8; };
-    auto wq_col = [&](int e) { return (e % C8) * 8; };
+    const int urg = st >> 4, uc4 = (st & 15) * 4;            // v, o: a lane owns 4 rows x 4 columns
+    const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
+    auto q_row = [&](int e) { return e / C8; };
+    auto q_col = [&](int e) { return (e % C8) * 8; };
     struct Regs {
-      v8 w[NPW], q[NPW], a[2];
-      v4 k[RPT], u[4];
+      v8 q[NPW];
+      v4 a[NPA];
+      v4 k[RPT], v[4];
       uint32_t gam;  // fp32 bits
     };
-    // A wave issues at most one instruction every few cycles, so the steady state is kept
-    // short: byte offsets of this lane's pieces from the chunk's first row are computed once,
-    // the chunk base pointers are advanced by constant strides (loads and stores both walk the
-    // chunks in order), and only a sequence's last, short chunk takes the masked path.
-    uint32_t offw[NPW], offa[2], offk[RPT], offu[4];
+    // The steady state carries no address arithmetic: byte offsets of this lane's pieces from the
+    // chunk's first row are computed once, the chunk base pointers advance by constant strides, and
+    // only a sequence's last, short chunk takes the masked path.
+    uint32_t offq[NPW], offk[RPT], offv[4];
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) offw[i] = 2 * ((uint32_t)wq_row(st + 256 * i) * HK + wq_col(st + 256 * i));
-#pragma unroll
-    for (int i = 0; i < 2; ++i) offa[i] = 2 * ((uint32_t)((st + 256 * i) >> 3) * HB + ((st + 256 * i) & 7) * 8);
+    for (int i = 0; i < NPW; ++i) offq[i] = 2 * ((uint32_t)q_row(st + 256 * i) * HK + q_col(st + 256 * i));
 #pragma unroll
     for (int i = 0; i < RPT; ++i) offk[i] = 2 * ((uint32_t)(rg * RPT + i) * HK + c4);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) offu[i] = 2 * ((uint32_t)(urg * 4 + i) * HV + uc4);
+    for (int i = 0; i < 4; ++i) offv[i] = 2 * ((uint32_t)(urg * 4 + i) * HV + uc4);
     const uint32_t offg = 4 * (uint32_t)lane * H;
     const int64_t row00 = sp.bos * H + hh;
-    const char* lw = (const char*)p.w + row00 * K * 2;
     const char* lq = (const char*)p.q + row00 * K * 2;
     const char* lk = (const char*)p.k + row00 * K * 2;
-    const char* lu = (const char*)p.u + (row00 * V + vbase) * 2;
-    const char* la = (const char*)p.Aqk + row00 * BT * 2;
-    // The gate load is unconditional in every staging wave (a load under a branch would force
-    // the wave to drain its whole load queue at the join); without gates it reads a dummy
-    // address and the bits are masked to zero.
+    const char* lv = (const char*)p.v + (row00 * V + vbase) * 2;
+    const char* la = (const char*)p.AT + ((chunk0 * H + hh) * (int64_t)(2 * kTriElems) + st * 4) * 2;
+    // The gate load is unconditional (a load under a branch would make the wave drain its whole load
+    // queue at the join); without gates it reads a dummy address and the bits are masked to zero.
     const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
-    const char* lg = p.gam ? (const char*)p.gam + row00 * 4 : lw;
+    const char* lg = p.gam ? (const char*)p.gam + row00 * 4 : lq;
     char* so = (char*)p.o + (row00 * V + vbase) * 2;
-    const int64_t strk = (int64_t)BT * HK * 2, stru = (int64_t)BT * HV * 2, stra = (int64_t)BT * HB * 2;
+    const int64_t strk = (int64_t)BT * HK * 2, strv = (int64_t)BT * HV * 2;
+    const int64_t stra = (int64_t)H * (2 * kTriElems) * 2;
     const int64_t strg = p.gam ? (int64_t)BT * H * 4 : 0;
     const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
     int lc = 0;  // next chunk to load
     auto load = [&](Regs& R) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < NPA; ++i) R.a[i] = *(const v4*)(la + 2048 * i);   // full tiles whatever the chunk length
       if (lc != nchunks - 1 || Llast == BT) {
 #pragma unroll
-        for (int i = 0; i < NPW; ++i) {
-          R.w[i] = *(const v8*)(lw + offw[i]);
-          R.q[i] = *(const v8*)(lq + offw[i]);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) R.a[i] = *(const v8*)(la + offa[i]);
+        for (int i = 0; i < NPW; ++i) R.q[i] = *(const v8*)(lq + offq[i]);
 #pragma unroll
         for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + offk[i]);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) R.u[i] = *(const v4*)(lu + offu[i]);
+        for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + offv[i]);
         R.gam = *(const uint32_t*)(lg + offg);
       } else {
         // rows past the end of the sequence are redirected to its last row (zeroed in write())
@@ -182,43 +195,35 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         auto cl = [&](uint32_t row) { return row < last ? row : last; };
 #pragma unroll
         for (int i = 0; i < NPW; ++i) {
-          uint32_t e = st + 256 * i, off = 2 * (cl(wq_row(e)) * HK + wq_col(e));
-          R.w[i] = *(const v8*)(lw + off);
-          R.q[i] = *(const v8*)(lq + off);
-        }
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
           uint32_t e = st + 256 * i;
-          R.a[i] = *(const v8*)(la + 2 * (cl(e >> 3) * HB + (e & 7) * 8));
+          R.q[i] = *(const v8*)(lq + 2 * (cl(q_row(e)) * HK + q_col(e)));
         }
 #pragma unroll
         for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + 2 * (cl(rg * RPT + i) * HK + c4));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) R.u[i] = *(const v4*)(lu + 2 * (cl(urg * 4 + i) * HV + uc4));
+        for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + 2 * (cl(urg * 4 + i) * HV + uc4));
         R.gam = *(const uint32_t*)(lg + 4 * cl(lane) * H);
       }
-      lw += strk;
       lq += strk;
       lk += strk;
-      lu += stru;
+      lv += strv;
       la += stra;
       lg += strg;
       ++lc;
     };
     // LDS destinations of this lane (element offsets inside a tile)
     constexpr int KV = RPT == 8 ? 8 : 4;  // elements per k^T write
-    int dw[NPW], dp[2], dk[4][RPT / KV], du[4];
+    int dq[NPW], dkr[RPT], dk[4][RPT / KV], dv[4];
 #pragma unroll
-    for (int i = 0; i < NPW; ++i) dw[i] = wq_row(st + 256 * i) * LDR + wq_col(st + 256 * i);
+    for (int i = 0; i < NPW; ++i) dq[i] = q_row(st + 256 * i) * LDR + q_col(st + 256 * i);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dp[i] = ((st + 256 * i) >> 3) * LDT + ((st + 256 * i) & 7) * 8;
+    for (int i = 0; i < RPT; ++i) dkr[i] = (rg * RPT + i) * LDR + c4;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
       for (int i0 = 0; i0 < RPT / KV; ++i0) dk[j][i0] = (c4 + j) * LDT + swz_t(c4 + j, rg * RPT + KV * i0);
-      du[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
+      dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
     }
-    auto put8 = [&](T* dst, v8 x) { *(v8*)dst = x; };
     int wc = 0;  // next chunk to write to LDS
     auto write = [&](Regs& R) __attribute__((always_inline)) {
       const int b = wc & 1;
@@ -226,28 +231,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int L = Llast;
 #pragma unroll
         for (int i = 0; i < NPW; ++i)
-          if (wq_row(st + 256 * i) >= L)
+          if (q_row(st + 256 * i) >= L)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) R.w[i][j] = R.q[i][j] = (T)0.f;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-          if (((st + 256 * i) >> 3) >= L)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) R.a[i][j] = (T)0.f;
+            for (int j = 0; j < 8; ++j) R.q[i][j] = (T)0.f;
 #pragma unroll
         for (int i = 0; i < RPT; ++i)
           if (rg * RPT + i >= L) R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i >= L) R.u[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          if (urg * 4 + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
       }
 #pragma unroll
-      for (int i = 0; i < NPW; ++i) {
-        put8(&sW[b][dw[i]], R.w[i]);
-        put8(&sQ[b][dw[i]], R.q[i]);
-      }
+      for (int i = 0; i < NPW; ++i) *(v8*)&sQ[b][dq[i]] = R.q[i];
 #pragma unroll
-      for (int i = 0; i < 2; ++i) put8(&sP[b][dp[i]], R.a[i]);
+      for (int i = 0; i < NPA; ++i) *(v4*)&sAT[b][st * 4 + 1024 * i] = R.a[i];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) *(v4*)&sK[b][dkr[i]] = R.k[i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -261,8 +260,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             *(v4*)&sKt[b][dk[j][i0]] = kc;
           }
         }
-        v4 uc = {R.u[0][j], R.u[1][j], R.u[2][j], R.u[3][j]};
-        *(v4*)&sUt[b][du[j]] = uc;
+        v4 vc = {R.v[0][j], R.v[1][j], R.v[2][j], R.v[3][j]};
+        *(v4*)&sVt[b][dv[j]] = vc;
       }
       if (wave == 4) {
         // lanes past the end of a short chunk carry the last row's gate
@@ -274,23 +273,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
       ++wc;
     };
-    // The matrix waves left o^T of a chunk where u^T of that chunk was; each lane reads back
+    // The matrix waves left o^T of a chunk where v^T of that chunk was; each lane reads back
     // exactly the addresses it writes in write(), so the tile can be refilled right after.
     int oc = 0;  // next chunk whose output is stored
     auto store_o = [&]() __attribute__((always_inline)) {
       const int b = oc & 1;
       v4 x[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x[j] = *(const v4*)&sUt[b][du[j]];
+      for (int j = 0; j < 4; ++j) x[j] = *(const v4*)&sVt[b][dv[j]];
       if (oc != nchunks - 1 || Llast == BT) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *(v4*)(so + offu[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+        for (int i = 0; i < 4; ++i) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i < Llast) *(v4*)(so + offu[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+          if (urg * 4 + i < Llast) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
       }
-      so += stru;
+      so += strv;
       ++oc;
     };
     // Two register sets: a chunk is loaded three iterations before the matrix waves use it
@@ -333,19 +332,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       lds_barrier();
       for (int ci = 0; ci < nchunks; ++ci) {
         const int b = ci & 1;
-        const T* W = sW[b];
+        const T* Kr = sK[b];
         const T* Q = sQ[b];
         const T* Kt = sKt[b];
-        const T* P = sP[b];
-        const int urow = cb + c;
-        T* ut = &sUt[b][urow * LDT];
+        const T* Tu = sAT[b];
+        const T* P = sAT[b] + kTriElems;
+        const int vrow = cb + c;
+        T* vt = &sVt[b][vrow * LDT];
         // LDS reads are issued a group ahead of the MFMAs that consume them; the scheduling
         // fences keep the compiler from sinking them back next to their use.
         v8 fa[2 * KS], fb[2 * KS];
-        auto load_wq = [&](int tt, v8* f) {
+        auto load_kq = [&](int tt, v8* f) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            f[ks] = frag16<T>(W, LDR, 16 * tt, 32 * ks, lane);
+            f[ks] = frag16<T>(Kr, LDR, 16 * tt, 32 * ks, lane);
             f[KS + ks] = frag16<T>(Q, LDR, 16 * tt, 32 * ks, lane);
           }
         };
@@ -355,8 +355,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16_t<T>(Kt, 16 * (half * (KT / 2) + i), 32 * s, lane);
         };
-        load_wq(0, fa);
-        load_wq(1, fb);
+        load_kq(0, fa);
+        load_kq(1, fb);
         __builtin_amdgcn_sched_barrier(0);
         // the state as the other MFMA operand: two stacked accumulators per 32-slice
         v8 hb[KS];
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             hb[ks][4 + e] = (T)acc[2 * ks + 1][e];
           }
         f32x4 d[4], oq[4];
-        auto mm_wq = [&](int tt, const v8* f) {
+        auto mm_kq = [&](int tt, const v8* f) {
           d[tt] = zero4();
           oq[tt] = zero4();
 #pragma unroll
@@ -377,49 +377,68 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             oq[tt] = Elem<T>::mfma16(f[KS + ks], hb[ks], oq[tt]);
           }
         };
-        mm_wq(0, fa);
+        mm_kq(0, fa);
         __builtin_amdgcn_sched_barrier(0);
-        load_wq(2, fa);
+        load_kq(2, fa);
         __builtin_amdgcn_sched_barrier(0);
-        mm_wq(1, fb);
+        mm_kq(1, fb);
         __builtin_amdgcn_sched_barrier(0);
-        load_wq(3, fb);
+        load_kq(3, fb);
         __builtin_amdgcn_sched_barrier(0);
-        mm_wq(2, fa);
+        mm_kq(2, fa);
         __builtin_amdgcn_sched_barrier(0);
         f32x4 eg[4], ed[4];
-        v4 uu[4];
-        v8 fp[6];
+        v4 vv[4];
+        v8 ft[6];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
           eg[tt] = *(const f32x4*)&sEg[b][16 * tt + 4 * g];
           ed[tt] = *(const f32x4*)&sEd[b][16 * tt + 4 * g];
-          uu[tt] = *(const v4*)(ut + swz_t(urow, 16 * tt + 4 * g));
+          vv[tt] = *(const v4*)(vt + swz_t(vrow, 16 * tt + 4 * g));
         }
         const float dec = sDec[b];
-        fp[0] = frag16<T>(P, LDT, 0, 0, lane);
-        fp[1] = frag16<T>(P, LDT, 16, 0, lane);
-        fp[2] = frag16<T>(P, LDT, 32, 0, lane);
-        fp[3] = frag16<T>(P, LDT, 32, 32, lane);
-        fp[4] = frag16<T>(P, LDT, 48, 0, lane);
-        fp[5] = frag16<T>(P, LDT, 48, 32, lane);
+        ft[0] = frag_tri<T>(Tu, 0, 0, lane);
+        ft[1] = frag_tri<T>(Tu, 1, 0, lane);
+        ft[2] = frag_tri<T>(Tu, 2, 0, lane);
+        ft[3] = frag_tri<T>(Tu, 2, 1, lane);
+        ft[4] = frag_tri<T>(Tu, 3, 0, lane);
+        ft[5] = frag_tri<T>(Tu, 3, 1, lane);
         __builtin_amdgcn_sched_barrier(0);
-        mm_wq(3, fb);
+        mm_kq(3, fb);
         __builtin_amdgcn_sched_barrier(0);
         load_kt(0, fa);
+        v8 fp[6];
+        fp[0] = frag_tri<T>(P, 0, 0, lane);
+        fp[1] = frag_tri<T>(P, 1, 0, lane);
+        fp[2] = frag_tri<T>(P, 2, 0, lane);
+        fp[3] = frag_tri<T>(P, 2, 1, lane);
+        fp[4] = frag_tri<T>(P, 3, 0, lane);
+        fp[5] = frag_tri<T>(P, 3, 1, lane);
         __builtin_amdgcn_sched_barrier(0);
+        // r = v - e^{gamma} (k h), as the operand contracting over time
+        v8 rb[2];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) rb[tt >> 1][(tt & 1) * 4 + r] = (T)((float)vv[tt][r] - d[tt][r] * eg[tt][r]);
+        // v_new = Tu r; Tu is lower triangular: row tiles 0 and 1 only meet the first 32 rows of r
+        f32x4 vn[4];
+        vn[0] = Elem<T>::mfma16(ft[0], rb[0], zero4());
+        vn[1] = Elem<T>::mfma16(ft[1], rb[0], zero4());
+        vn[2] = Elem<T>::mfma16(ft[2], rb[0], zero4());
+        vn[3] = Elem<T>::mfma16(ft[4], rb[0], zero4());
+        vn[2] = Elem<T>::mfma16(ft[3], rb[1], vn[2]);
+        vn[3] = Elem<T>::mfma16(ft[5], rb[1], vn[3]);
         v8 vnb[2], vsb[2];  // v_new and its decayed copy as operands contracting over time
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            float vn = (float)uu[tt][r] - d[tt][r] * eg[tt][r];
-            vnb[tt >> 1][(tt & 1) * 4 + r] = (T)vn;
-            vsb[tt >> 1][(tt & 1) * 4 + r] = (T)(vn * ed[tt][r]);
+            vnb[tt >> 1][(tt & 1) * 4 + r] = (T)vn[tt][r];
+            vsb[tt >> 1][(tt & 1) * 4 + r] = (T)(vn[tt][r] * ed[tt][r]);
             oq[tt][r] *= p.scale * eg[tt][r];
           }
         }
-        // Aqk is lower triangular: row tiles 0 and 1 only meet the first 32 columns
         oq[0] = Elem<T>::mfma16(fp[0], vnb[0], oq[0]);
         oq[1] = Elem<T>::mfma16(fp[1], vnb[0], oq[1]);
         oq[2] = Elem<T>::mfma16(fp[2], vnb[0], oq[2]);
@@ -442,7 +461,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           v4 ov;
 #pragma unroll
           for (int r = 0; r < 4; ++r) ov[r] = (T)oq[tt][r];
-          *(v4*)(ut + swz_t(urow, 16 * tt + 4 * g)) = ov;
+          *(v4*)(vt + swz_t(vrow, 16 * tt + 4 * g)) = ov;
         }
 #pragma unroll
         for (int i = 0; i < KT / 2; ++i)
@@ -462,13 +481,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 template <typename T>
-int launch_fused(const GdrFusedParams& p, int K, hipStream_t st) {
+int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
   const int64_t nblk = (int64_t)p.N * p.H * (p.V / 64);
   FLA_REQUIRE(nblk <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   if (nblk == 0) return FLA_OK;
   dim3 grid((unsigned)nblk), block(512);
-  if (K == 64) hipLaunchKernelGGL((gdr_fwd_fused_kernel<T, 64>), grid, block, 0, st, p);
-  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_fused_kernel<T, 128>), grid, block, 0, st, p);
+  if (K == 64) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64>), grid, block, 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128>), grid, block, 0, st, p);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;
@@ -476,20 +495,19 @@ int launch_fused(const GdrFusedParams& p, int K, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
-                                                    const void* Aqk, const float* g_cumsum, const float* h0, void* o,
-                                                    float* ht, const int64_t* offsets, const int64_t* seq_order, int qkv_dtype,
-                                                    int64_t B,
-                                                    int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
-                                                    fla_stream_t stream) {
-  FLA_REQUIRE(q && k && w && u && Aqk && o, FLA_E_INVALID);
+extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
+                                                   const float* g_cumsum, const float* h0, void* o, float* ht,
+                                                   const int64_t* offsets, const int64_t* chunk_offsets,
+                                                   const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
+                                                   int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                                   fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v && AT && o, FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(offsets ? B == 1 : N == B, FLA_E_INVALID);
+  FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
   FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aqk | (uintptr_t)o) % 16 == 0,
-              FLA_E_ALIGNMENT);
-  GdrFusedParams p{q, k, w, u, Aqk, g_cumsum, h0, o, ht, offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
-  if (qkv_dtype == FLA_BF16) return launch_fused<bf16>(p, (int)K, (hipStream_t)stream);
-  if (qkv_dtype == FLA_F16) return launch_fused<f16>(p, (int)K, (hipStream_t)stream);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o) % 16 == 0, FLA_E_ALIGNMENT);
+  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
+  if (qkv_dtype == FLA_BF16) return launch_scan<bf16>(p, (int)K, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_scan<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
 }

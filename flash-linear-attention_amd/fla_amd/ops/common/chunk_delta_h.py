@@ -105,41 +105,40 @@ def chunk_gated_delta_rule_fwd_h_both(
     return h, hT, v_new, ht
 
 
-def chunk_gated_delta_rule_fwd_fused(
+def chunk_gated_delta_rule_fwd_scan(
     q: torch.Tensor,
     k: torch.Tensor,
-    w: torch.Tensor,
-    u: torch.Tensor,
-    Aqk: torch.Tensor,
+    v: torch.Tensor,
+    AT: torch.Tensor,
     g: Optional[torch.Tensor],
     scale: float,
     initial_state: Optional[torch.Tensor],
     output_final_state: bool,
     offsets: Optional[torch.Tensor] = None,
+    chunk_offsets: Optional[torch.Tensor] = None,
     seq_order: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """State scan and output in one launch (``fla_chunk_gated_delta_rule_fwd_fused``): the work of
-    ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o``
-    (``fla/ops/gated_delta_rule/chunk.py:47-72``) without materialising the per-chunk states
-    or ``v_new``.  ``w, u, Aqk`` come from ``fwd_prepare_wy_repr(..., q=q, scale=scale)``;
-    ``g`` is the fp32 chunk-local cumsum.  Seq-first layout.  ``seq_order`` (int64 ``[N]``, sequence
-    ids longest first) balances a packed batch.  Returns ``(o, final_state)``."""
-    be.require_gpu(q, k, w, u, Aqk)
+    """Serial half of the one-pass forward (``fla_chunk_gated_delta_rule_fwd_scan``): the work of
+    ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o`` (``fla/ops/gated_delta_rule/chunk.py:47-72``)
+    on ``q, k, v`` and the packed triangular tiles ``AT`` of ``fwd_prepare_scan_operands``; neither w, u,
+    v_new nor the per-chunk states are materialised.  ``g`` is the fp32 chunk-local cumsum.  Seq-first.
+    Returns ``(o, final_state)``."""
+    be.require_gpu(q, k, v, AT)
     B, T, H, K = k.shape
-    V = u.shape[-1]
+    V = v.shape[-1]
     N = B
     if offsets is not None:
         N = len(offsets) - 1
         offsets = offsets.to(torch.int64).contiguous()
-    o = torch.empty_like(u)
+    o = torch.empty_like(v)
     ht = k.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
     h0 = None
     if initial_state is not None:
         h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
     if g is not None and g.dtype != torch.float32:
         g = g.float()
-    be.check(be.lib().fla_chunk_gated_delta_rule_fwd_fused(
-        be.ptr(q), be.ptr(k), be.ptr(w), be.ptr(u), be.ptr(Aqk), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht),
-        be.ptr(offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale), be.stream_of(k)),
-        "fla_chunk_gated_delta_rule_fwd_fused")
+    be.check(be.lib().fla_chunk_gated_delta_rule_fwd_scan(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht),
+        be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale),
+        be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan")
     return o, ht

@@ -1,11 +1,12 @@
 """``chunk_gated_delta_rule`` with the reference's signature
 (``fla/ops/gated_delta_rule/chunk.py:258-363``).
 
-Forward pipeline on the device (chunk size 64): ``fla_chunk_local_cumsum`` (gate)
--> ``fla_gdr_fwd_wy`` (KK^T, block inverse, w/u, gated causal q k^T scores)
--> ``fla_chunk_gated_delta_rule_fwd_fused`` (state scan and output in one launch).
-A forward pass that will be differentiated runs the two-launch form instead (state scan, output
-stage) and keeps w, Aw, v_new and the per-chunk states for the backward; with
+Forward on the device (chunk size 64), two launches: ``fla_gdr_fwd_prep`` (chunk-parallel: prefix sum of the
+gate, KK^T, block inverse, gated causal q k^T scores; leaves two packed triangular 64x64 tiles per chunk and
+head) -> ``fla_chunk_gated_delta_rule_fwd_scan`` (state scan and output in one pass over q, k, v; w, u, v_new
+and the per-chunk states are never formed).
+A forward pass that will be differentiated runs the reference's decomposition instead (cumsum, WY launch, state
+scan, output stage) and keeps w, Aw, v_new and the per-chunk states for the backward; with
 ``KEEP_STATES_FOR_BACKWARD = False`` the backward recomputes them with
 ``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
 """
@@ -19,11 +20,11 @@ import torch.nn.functional as F
 from ... import _backend as be
 from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
                       resolve_offsets)
-from ..common.chunk_delta_h import (chunk_gated_delta_rule_fwd_fused, chunk_gated_delta_rule_fwd_h,
-                                    chunk_gated_delta_rule_fwd_h_both)
+from ..common.chunk_delta_h import (chunk_gated_delta_rule_fwd_h, chunk_gated_delta_rule_fwd_h_both,
+                                    chunk_gated_delta_rule_fwd_scan)
 from ..common.chunk_o import chunk_fwd_o
 from ..utils.cumsum import chunk_local_cumsum
-from .wy_fast import fwd_prepare_wy_repr
+from .wy_fast import fwd_prepare_scan_operands, fwd_prepare_wy_repr
 
 BT = 64
 _SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64), (256, 64), (256, 128)}
@@ -50,8 +51,9 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
                                offsets=None, indices=None, head_first=True, chunk_size=64,
                                *, plan: Optional[VarlenPlan] = None, store_A: bool = True, fused: bool = True):
     """Reference-shaped forward (``fla/ops/gated_delta_rule/chunk.py:20-73``): returns
-    ``(g_cumsum, o, Aw, Au, final_state)``.  ``fused=False`` runs the state scan and the
-    output stage as the reference's two separate steps."""
+    ``(g_cumsum, o, Aw, Au, final_state)``.  ``fused=False`` runs the reference's steps one by one
+    (cumsum, WY representation, state scan, output stage); the default two-launch form does not form
+    ``Aw`` / ``Au`` and returns ``None`` for them."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd: seq-first, chunk size 64 only")
     if offsets is not None and plan is None:
@@ -59,14 +61,14 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
     co = None if plan is None else plan.chunk_offsets
-    g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
     if fused:
-        w, u, Aw, Au, Aqk = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False,
-                                                chunk_size=BT, store_A=store_A, q=q, scale=scale)
-        o, final_state = chunk_gated_delta_rule_fwd_fused(q, k, w, u, Aqk, g, scale, initial_state,
-                                                          output_final_state, offsets=offs,
-                                                          seq_order=None if plan is None else plan.seq_order)
-        return g, o, Aw, Au, final_state
+        # two launches; Aw / Au are not formed on this path
+        AT, g = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=offs, indices=idx)
+        o, final_state = chunk_gated_delta_rule_fwd_scan(q, k, v, AT, g, scale, initial_state, output_final_state,
+                                                         offsets=offs, chunk_offsets=co,
+                                                         seq_order=None if plan is None else plan.seq_order)
+        return g, o, None, None, final_state
+    g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
     w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
                                        store_A=store_A)
     h, v_new, final_state = chunk_gated_delta_rule_fwd_h(
@@ -170,9 +172,11 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
             gc, o, ht, kept = chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, h0, output_final_state,
                                                               offsets=offsets)
         else:
-            gc, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
-                                                         offsets=offsets, head_first=False, chunk_size=BT,
-                                                         store_A=False, fused=KP <= _FUSED_MAX_K)
+            _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
+                                                        offsets=offsets, head_first=False, chunk_size=BT,
+                                                        store_A=False, fused=KP <= _FUSED_MAX_K)
+            # a backward that recomputes starts from the raw gate, like the reference's
+            gc = None if g is None else g.float().contiguous()
         ctx.save_for_backward(q, k, v, gc, beta, h0, offsets, *kept)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
@@ -198,6 +202,10 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         do = do.contiguous()
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
+        if not kept and gc is not None:   # the raw gate was saved: its prefix sums as the kept-states forward forms them
+            plan = VarlenPlan(offsets, BT) if offsets is not None else None
+            gc = chunk_local_cumsum(gc, BT, offsets=None if plan is None else plan.offsets,
+                                    indices=None if plan is None else plan.indices, head_first=False)
         dq, dk, dv, db, dg, dh0 = chunk_gated_delta_rule_bwd(q, k, v, gc, beta, ctx.scale, h0, do, dht, offsets,
                                                              kept=tuple(kept) if kept else None)
         if (KP, VP) != (K, V):

@@ -21,16 +21,10 @@ def fwd_prepare_wy_repr(
     *,
     store_A: bool = True,
     store_Au: bool = True,
-    q: Optional[torch.Tensor] = None,
-    scale: float = 1.0,
 ):
     """Returns ``(w, u, Aw, Au)`` with ``Aw = (I + strict_lower(diag(beta) K K^T))^-1``,
     ``Au = Aw * exp(g_i - g_j)``, ``w = Aw (beta K)``, ``u = Au (beta V)``; ``g`` is the
-    fp32 chunk-local cumsum of the log-gate (or ``None``).
-
-    With ``q`` the same launch also produces the gated causal scores of the output stage,
-    ``Aqk[i, j] = scale (q_i . k_j) exp(g_i - g_j)`` for ``j <= i`` (else 0), ``[B, T, H, 64]``,
-    and the return value is ``(w, u, Aw, Au, Aqk)``."""
+    fp32 chunk-local cumsum of the log-gate (or ``None``)."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd fwd_prepare_wy_repr: seq-first, chunk size 64 only")
     be.require_gpu(k, v, beta)
@@ -46,11 +40,58 @@ def fwd_prepare_wy_repr(
     w, u = torch.empty_like(k), torch.empty_like(v)
     Aw = k.new_empty(B, T, H, BT) if store_A else None
     Au = k.new_empty(B, T, H, BT) if (store_A and store_Au) else None
-    Aqk = k.new_empty(B, T, H, BT) if q is not None else None
     be.check(be.lib().fla_gdr_fwd_wy(
         be.ptr(k), be.ptr(v), be.ptr(beta), be.ptr(g), be.ptr(w), be.ptr(u), be.ptr(Aw), be.ptr(Au),
-        be.ptr(q), be.ptr(Aqk), float(scale),
         be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, V, be.stream_of(k)), "fla_gdr_fwd_wy")
-    if q is not None:
-        return w, u, Aw, Au, Aqk
     return w, u, Aw, Au
+
+
+TRI_BLOCKS = 10   # 16x16 blocks on and below the diagonal of a 64x64 tile
+
+
+def fwd_prepare_scan_operands(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    beta: torch.Tensor,
+    g: Optional[torch.Tensor],
+    scale: float,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    g_is_cumsum: bool = False,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Chunk-parallel half of the one-pass forward (``fla_gdr_fwd_prep``): the work of ``chunk_local_cumsum``,
+    ``fwd_prepare_wy_repr`` (``fla/ops/gated_delta_rule/wy_fast.py:320-376``) and the score product of
+    ``chunk_fwd_o`` (``fla/ops/common/chunk_o.py:86-97``), leaving per (chunk, head) the lower-triangular
+    ``Tu = (Aw * Gamma) diag(beta)`` and ``Aqk = scale tril(q k^T * Gamma)`` as packed 16x16 blocks:
+    ``AT`` is ``[chunks, H, 2, 10, 16, 16]`` in the q/k/v dtype.  ``g`` is the raw per-head log-gate
+    ``[B, T, H]`` (or its chunk-local cumsum with ``g_is_cumsum``; ``None`` for the un-gated rule).
+    Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``."""
+    be.require_gpu(q, k, beta)
+    B, T, H, K = k.shape
+    NT = 0
+    chunks = B * (-(-T // BT))
+    if offsets is not None:
+        NT = chunks = indices.shape[0]
+        offsets = offsets.to(torch.int64).contiguous()
+    beta = beta.float().contiguous()
+    gc = None
+    if g is not None:
+        g = g.float().contiguous()
+        gc = g if g_is_cumsum else torch.empty_like(g)
+    AT = k.new_empty(chunks, H, 2, TRI_BLOCKS, 16, 16)
+    be.check(be.lib().fla_gdr_fwd_prep(
+        be.ptr(q), be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
+        be.ptr(AT), float(scale), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, be.stream_of(k)),
+        "fla_gdr_fwd_prep")
+    return AT, gc
+
+
+def unpack_triangular_tiles(AT: torch.Tensor) -> torch.Tensor:
+    """``[chunks, H, 2, 10, 16, 16]`` packed blocks -> dense ``[chunks, H, 2, 64, 64]`` (zeros above the diagonal
+    blocks); for tests and debugging."""
+    chunks, H = AT.shape[:2]
+    out = AT.new_zeros(chunks, H, 2, 64, 64)
+    for i in range(4):
+        for j in range(i + 1):
+            out[..., 16 * i:16 * i + 16, 16 * j:16 * j + 16] = AT[..., i * (i + 1) // 2 + j, :, :]
+    return out

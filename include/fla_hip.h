@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 1
+#define FLA_ABI_VERSION 2
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -226,10 +226,7 @@ int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, 
  * :111-236; :379-426 kernel :250-317): Aw = (I + strict_lower(diag(beta) K K^T))^-1,
  * Au = Aw * exp(g_i - g_j), w = Aw (beta K) [B,T,H,K], u = Au (beta V) [B,T,H,V].
  * Aw, Au (optional outputs, [B,T,H,64] in the q/k/v dtype) are what the
- * reference saves for backward.  With q and Aqk (both or neither) the same
- * launch also emits the gated causal scores of chunk_fwd_o
- * (fla/ops/common/chunk_o.py:86-97): Aqk[i,j] = scale (q_i . k_j) exp(g_i - g_j)
- * for j <= i, else 0, [B,T,H,64] in the q/k/v dtype.
+ * reference saves for backward.
  *
  * fla_chunk_gated_delta_rule_fwd_h: state scan, replaces
  * chunk_gated_delta_rule_fwd_h (fla/ops/common/chunk_delta_h.py:248-320,
@@ -241,7 +238,7 @@ int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, 
  * FLA_H_FRAGMENT; v is v_new for the delta rule.
  * ---------------------------------------------------------------------- */
 int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum,
-                   void* w, void* u, void* Aw, void* Au, const void* q, void* Aqk, float scale,
+                   void* w, void* u, void* Aw, void* Au,
                    const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, fla_stream_t stream);
 
@@ -267,20 +264,33 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
                     const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
                     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream);
 
-/* fla_chunk_gated_delta_rule_fwd_fused: state scan and output in one launch;
- * replaces chunk_gated_delta_rule_fwd_h followed by chunk_fwd_o in
- * chunk_gated_delta_rule_fwd (fla/ops/gated_delta_rule/chunk.py:47-72; kernels
- * fla/ops/common/chunk_delta_h.py:27-119 and chunk_o.py:23-101) when neither the
- * per-chunk states nor v_new are wanted.  w, u and Aqk come from
- * fla_gdr_fwd_wy (called with q, scale).  o [B,T,H,V] in the q/k/v dtype;
- * h0, ht fp32 [N,H,K,V] or NULL.  K in {64,128}, V a multiple of 64.
- * seq_order as for fla_chunk_gla_fwd_fused. */
-int fla_chunk_gated_delta_rule_fwd_fused(const void* q, const void* k, const void* w, const void* u,
-                                         const void* Aqk, const float* g_cumsum, const float* h0,
-                                         void* o, float* ht, const int64_t* offsets,
-                                         const int64_t* seq_order, int qkv_dtype,
-                                         int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
-                                         float scale, fla_stream_t stream);
+/* The two-launch forward that forms neither w, u, v_new nor the per-chunk states (what
+ * chunk_gated_delta_rule runs when nothing is kept for a backward pass).  fla_gdr_fwd_prep is the chunk-parallel part: it replaces
+ * chunk_local_cumsum of the gate, fwd_prepare_wy_repr (fla/ops/gated_delta_rule/wy_fast.py:320-376) and the
+ * score product of chunk_fwd_o (fla/ops/common/chunk_o.py:86-97) and leaves, per (chunk, head), two
+ * lower-triangular 64x64 matrices in the q/k/v dtype:
+ *   Tu  = (Aw * Gamma) diag(beta),  Gamma_ij = exp(gamma_i - gamma_j)   (so that u = Tu v, e^{gamma} w = Tu e^{gamma} k)
+ *   Aqk = scale tril(q k^T * Gamma)
+ * stored as their ten 16x16 blocks on and below the diagonal (block (i, j) at index i (i + 1) / 2 + j, row-major
+ * inside a block): AT is [chunks, H, 2, 10, 16, 16] (chunk index as in `indices`, or b * ceil(T/64) + c).
+ * g is the raw per-head log-gate [B,T,H] (g_is_cumsum == 0; its chunk-local prefix sum is formed in the kernel and
+ * written to g_cumsum_out, fp32 [B,T,H], if that is given), or already the prefix sum (== 1), or NULL (no gate).
+ * K in {64, 128}.
+ * fla_chunk_gated_delta_rule_fwd_scan is the serial part (state scan + output, replaces
+ * chunk_gated_delta_rule_fwd_h + chunk_fwd_o, fla/ops/gated_delta_rule/chunk.py:47-72): with h the state entering
+ * a chunk,  v_new = Tu (v - e^{gamma} (k h)),  o = scale e^{gamma} (q h) + Aqk v_new,
+ * h <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} v_new).  g_cumsum fp32 [B,T,H] or NULL; h0, ht fp32
+ * [N,H,K,V] or NULL; packed batches need chunk_offsets [N+1]; seq_order as for fla_chunk_gla_fwd_fused.
+ * K in {64, 128}, V a multiple of 64. */
+int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
+                     float* g_cumsum_out, void* AT, float scale, const int64_t* offsets, const int64_t* indices,
+                     int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, fla_stream_t stream);
+
+int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
+                                        const float* g_cumsum, const float* h0, void* o, float* ht,
+                                        const int64_t* offsets, const int64_t* chunk_offsets,
+                                        const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                                        int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Chunked GLA backward (chunk size 64), replaces chunk_gla_bwd

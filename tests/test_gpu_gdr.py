@@ -58,17 +58,82 @@ def test_gdr_kernel_by_kernel(device):
     o_rm = chunk_fwd_o(dev(q), dev(k), v_new2, h, gc, 128 ** -0.5, head_first=False)
     torch.cuda.synchronize()
     assert torch.equal(o, o_rm)
-    # the fused scan + output launch, fed by the WY launch that also emits the gated scores
-    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_fused
-    w2, u2, Aw2, Au2, Aqk = fwd_prepare_wy_repr(dev(k), dev(v), dev(beta), gc, head_first=False, q=dev(q),
-                                                scale=128 ** -0.5)
+
+
+def _dense_tiles(ref, beta, B, T, H, offsets=None):
+    """Oracle Tu = Au diag(beta) and Aqk per chunk as dense [chunks, H, 64, 64] (zero outside the chunk's rows)."""
+    spans = [(b, 0, T) for b in range(B)] if offsets is None else [(0, a, e) for a, e in zip(offsets[:-1], offsets[1:])]
+    tu, aqk = [], []
+    for b, bos, eos in spans:
+        for c0 in range(bos, eos, 64):
+            L = min(64, eos - c0)
+            t_, a_ = torch.zeros(H, 64, 64), torch.zeros(H, 64, 64)
+            t_[:, :L, :L] = ref['Au'][b, c0:c0 + L].permute(1, 0, 2)[:, :, :L] * beta[b, c0:c0 + L].t()[:, None, :]
+            a_[:, :L, :L] = ref['Aqk'][b, c0:c0 + L].permute(1, 0, 2)[:, :, :L]
+            tu.append(t_)
+            aqk.append(a_)
+    return torch.stack(tu), torch.stack(aqk)
+
+
+@pytest.mark.parametrize("B,T,H,K,V", [(2, 200, 2, 128, 128), (2, 64, 2, 64, 64), (1, 1, 1, 128, 64), (2, 300, 3, 64, 128)])
+def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
+    """The operator's own decomposition: fla_gdr_fwd_prep (gate prefix sums, Tu = Au diag(beta) and the gated
+    scores as packed triangular tiles) against the fp32 chunked oracle, then the scan on them against the
+    naive recurrence."""
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_scan
+    from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_scan_operands, unpack_triangular_tiles
+    from oracle.chunked import chunked_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=21)
+    ref = chunked_gated_delta_rule(q, k, v, g, beta, initial_state=h0)
+    dev = lambda x: x.to(device)
+    print(f"gdr prep + scan B={B} T={T} H={H} K={K} V={V}", flush=True)
+    AT, gc = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), K ** -0.5)
     torch.cuda.synchronize()
-    assert torch.equal(w, w2) and torch.equal(u, u2) and torch.equal(Aw, Aw2) and torch.equal(Au, Au2)
-    assert_close("Aqk", ref['Aqk'], Aqk, 5e-3)
-    o2, ht2 = chunk_gated_delta_rule_fwd_fused(dev(q), dev(k), w2, u2, Aqk, gc, 128 ** -0.5, dev(h0), True)
+    torch.testing.assert_close(gc.cpu(), ref['g_cumsum'], rtol=1e-5, atol=1e-5)
+    dense = unpack_triangular_tiles(AT).float().cpu()
+    tu_ref, aqk_ref = _dense_tiles(ref, beta, B, T, H)
+    assert_close("Tu", tu_ref, dense[:, :, 0], 5e-3)
+    assert_close("Aqk", aqk_ref, dense[:, :, 1], 5e-3)
+    assert torch.equal(dense.triu(1), torch.zeros_like(dense))          # nothing above the diagonal
+    # the same tiles from gates that are already cumulative
+    AT2, gc2 = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), gc, K ** -0.5, g_is_cumsum=True)
+    assert gc2 is gc and torch.equal(AT, AT2)
+    o, ht = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, K ** -0.5, dev(h0), True)
     torch.cuda.synchronize()
-    assert_close("o fused", ref['o'], o2, TOL_O)
-    assert_close("ht fused", ref['ht'], ht2, TOL_HT)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
+def test_gdr_two_launch_forward_pieces_packed(device):
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_scan
+    from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_scan_operands, unpack_triangular_tiles
+    from fla_amd.utils import VarlenPlan
+    from oracle.chunked import chunked_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    T, N, H = 500, 4, 2
+    offs = random_offsets(T, N, torch.Generator().manual_seed(5), min_len=1)
+    q, k, v, g, beta, h0 = gdr_inputs(1, T, H, 128, 128, seed=31, N=N)
+    ref = chunked_gated_delta_rule(q, k, v, g, beta, initial_state=h0, offsets=offs.tolist())
+    dev = lambda x: x.to(device)
+    plan = VarlenPlan(dev(offs), 64)
+    print(f"gdr prep + scan packed {offs.tolist()}", flush=True)
+    AT, gc = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), 128 ** -0.5, offsets=plan.offsets,
+                                       indices=plan.indices)
+    torch.cuda.synchronize()
+    dense = unpack_triangular_tiles(AT).float().cpu()
+    tu_ref, aqk_ref = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
+    assert_close("Tu", tu_ref, dense[:, :, 0], 5e-3)
+    assert_close("Aqk", aqk_ref, dense[:, :, 1], 5e-3)
+    o, ht = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, 128 ** -0.5, dev(h0), True,
+                                            offsets=plan.offsets, chunk_offsets=plan.chunk_offsets,
+                                            seq_order=plan.seq_order)
+    torch.cuda.synchronize()
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
 
 
 @pytest.mark.parametrize("varlen", [False, True])
