@@ -116,6 +116,21 @@ inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B,
   return FLA_OK;
 }
 
+// dst = src (or zeros when src is NULL), n floats: what the state gradient of a batch without any
+// chunk is (d initial_state = d final_state).  A kernel rather than a memset / memcpy call, so that
+// the launch can sit in a captured graph like the rest.
+__global__ void copy_or_zero_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = src ? src[i] : 0.f;
+}
+inline int copy_or_zero(const float* src, float* dst, int64_t n, hipStream_t st) {
+  if (!dst || n <= 0) return FLA_OK;
+  const int64_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(copy_or_zero_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, st, src, dst, n);
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
 // Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps the operand finite in
 // 16-bit storage.  bf16 has fp32's exponent range; fp16 ends at 65504 (e^{11}), so fp16 chunks leave the
 // single-reference arithmetic much earlier (e^{8} |k| stays representable for |k| up to 20).

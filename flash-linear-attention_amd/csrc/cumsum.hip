@@ -47,7 +47,7 @@ template <typename GT, int VEC, int ROWS>
 __global__ __launch_bounds__(256) void cumsum_kernel(const GT* __restrict__ g, float* __restrict__ out,
                                                      int64_t T, int64_t HS, int BT, int reverse,
                                                      const int64_t* __restrict__ offsets,
-                                                     const int64_t* __restrict__ indices) {
+                                                     const int64_t* __restrict__ indices, int inverse) {
   int64_t col = ((int64_t)blockIdx.y * 256 + threadIdx.x) * VEC;
   if (col >= HS) return;
   int64_t bos, len, ic;
@@ -66,6 +66,8 @@ __global__ __launch_bounds__(256) void cumsum_kernel(const GT* __restrict__ g, f
   if (L <= 0) return;
   const GT* src = g + (bos + t0) * HS + col;
   float* dst = out + (bos + t0) * HS + col;
+  // inverse: the input holds the sums and the output is the differences of consecutive rows (the
+  // first row of the walk keeps its value); `run` then carries the previous row instead of the sum
   float run[VEC];
 #pragma unroll
   for (int i = 0; i < VEC; ++i) run[i] = 0.f;
@@ -86,14 +88,23 @@ __global__ __launch_bounds__(256) void cumsum_kernel(const GT* __restrict__ g, f
     for (int r = 0; r < ROWS; ++r) {
       int row = r0 + r;
       int rr = reverse ? (L - 1 - row) : row;
+      float o[VEC];
 #pragma unroll
-      for (int i = 0; i < VEC; ++i) run[i] += x[r][i];
+      for (int i = 0; i < VEC; ++i) {
+        if (inverse) {
+          o[i] = x[r][i] - run[i];
+          run[i] = x[r][i];
+        } else {
+          run[i] += x[r][i];
+          o[i] = run[i];
+        }
+      }
       if (row < L) {
         if (VEC == 4) {
-          f32x4 o4 = {run[0], run[VEC > 1 ? 1 : 0], run[VEC > 2 ? 2 : 0], run[VEC > 3 ? 3 : 0]};
+          f32x4 o4 = {o[0], o[VEC > 1 ? 1 : 0], o[VEC > 2 ? 2 : 0], o[VEC > 3 ? 3 : 0]};
           *(f32x4*)(dst + (int64_t)rr * HS) = o4;
         } else {
-          dst[(int64_t)rr * HS] = run[0];
+          dst[(int64_t)rr * HS] = o[0];
         }
       }
     }
@@ -102,7 +113,7 @@ __global__ __launch_bounds__(256) void cumsum_kernel(const GT* __restrict__ g, f
 
 template <typename GT>
 int launch_cumsum(const void* g, float* out, int64_t B, int64_t T, int64_t H, int64_t S, int BT, int reverse,
-                  const int64_t* offsets, const int64_t* indices, int64_t NT, hipStream_t stream) {
+                  const int64_t* offsets, const int64_t* indices, int64_t NT, hipStream_t stream, int inverse = 0) {
   int64_t HS = H * S;
   bool vec4 = (HS % 4 == 0) && (((uintptr_t)g) % (4 * sizeof(GT)) == 0) && (((uintptr_t)out) % 16 == 0);
   int64_t nt = offsets ? NT : fla_cdiv(T, BT);
@@ -112,11 +123,11 @@ int launch_cumsum(const void* g, float* out, int64_t B, int64_t T, int64_t H, in
   if (vec4) {
     dim3 grid((unsigned)nt, (unsigned)fla_cdiv(HS / 4, 256), (unsigned)nb);
     hipLaunchKernelGGL((cumsum_kernel<GT, 4, 16>), grid, dim3(256), 0, stream, (const GT*)g, out, T, HS, BT, reverse,
-                       offsets, indices);
+                       offsets, indices, inverse);
   } else {
     dim3 grid((unsigned)nt, (unsigned)fla_cdiv(HS, 256), (unsigned)nb);
     hipLaunchKernelGGL((cumsum_kernel<GT, 1, 16>), grid, dim3(256), 0, stream, (const GT*)g, out, T, HS, BT, reverse,
-                       offsets, indices);
+                       offsets, indices, inverse);
   }
   FLA_CHECK_LAUNCH();
   return FLA_OK;
@@ -209,6 +220,18 @@ extern "C" int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype, in
     case FLA_F16: return launch_cumsum<f16>(g, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT, st);
     default: return FLA_E_UNSUPPORTED;
   }
+}
+
+extern "C" int fla_chunk_local_cumsum_inverse(const float* g_cumsum, float* out, int64_t B, int64_t T, int64_t H,
+                                              int64_t S, int64_t chunk_size, int reverse, const int64_t* offsets,
+                                              const int64_t* indices, int64_t NT, fla_stream_t stream) {
+  FLA_REQUIRE(g_cumsum && out, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H >= 0 && S >= 1 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(chunk_size > 0 && (chunk_size & (chunk_size - 1)) == 0, FLA_E_INVALID);
+  FLA_REQUIRE(chunk_size <= (1 << 20), FLA_E_UNSUPPORTED);
+  if (offsets) FLA_REQUIRE(indices != nullptr && B == 1, FLA_E_INVALID);
+  return launch_cumsum<float>(g_cumsum, out, B, T, H, S, (int)chunk_size, reverse, offsets, indices, NT,
+                              (hipStream_t)stream, 1);
 }
 
 extern "C" int fla_chunk_global_cumsum(const void* s, float* ws_local, void* out, int s_dtype, int out_dtype, int64_t B,

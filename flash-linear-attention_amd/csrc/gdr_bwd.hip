@@ -1109,7 +1109,7 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
   if (rc) return rc;
-  if (grid.x == 0) return FLA_OK;
+  if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
 #define FLA_KV(STMT)                                   \
   if (K == 64 && V == 64) { STMT(64, 64) }             \
   else if (K == 128 && V == 128) { STMT(128, 128) }    \

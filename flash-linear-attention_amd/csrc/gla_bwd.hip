@@ -921,7 +921,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
   if (rc) return rc;
-  if (grid.x == 0) return FLA_OK;
+  if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
   const int64_t total_chunks = grid.x;
   {
     BDhParams p{q, g, dout, dht, hT, dhf, dhtf, hdh, dh0, offsets, chunk_offsets, T_, total_chunks,

@@ -29,10 +29,12 @@ SIGNATURES = {
     "fla_count_chunks": (c_int64, [P, I64, I64]),
     "fla_prepare_chunk_indices": (c_int, [P, I64, I64, P, P]),
     "fla_chunk_local_cumsum": (c_int, [P, P, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
+    "fla_chunk_local_cumsum_inverse": (c_int, [P, P, I64, I64, I64, I64, I64, I, P, P, I64, P]),
     "fla_chunk_global_cumsum": (c_int, [P, P, P, I, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
     "fla_chunk_global_cumsum_static": (c_int, [P, P, I, I, I64, I64, I64, I64, I64, I, P, P, I64, P]),
     "fla_fused_recurrent_fwd": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                         I64, I64, I64, I64, I64, I64, F, I, P]),
+    "fla_fused_recurrent_bwd": (c_int, [P] * 14 + [I, I, I64, I64, I64, I64, I64, I64, F, I, P]),
     "fla_fused_recurrent_gated_delta_rule_fwd": (c_int, [P, P, P, P, P, P, P, P, P, I, I, I, I,
                                                          I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_h": (c_int, [P, P, P, I, P, P, P, P, P, I, I, I, I,

@@ -1,6 +1,6 @@
 """``fused_recurrent`` (``fla/ops/common/fused_recurrent.py:545-574``): the
 token-by-token recurrence with optional scalar / per-key / per-value log-gates,
-served by ``fla_fused_recurrent_fwd``."""
+served by ``fla_fused_recurrent_fwd`` and ``fla_fused_recurrent_bwd``."""
 from typing import Optional, Tuple
 
 import torch
@@ -11,12 +11,12 @@ from ...utils import autocast_custom_bwd, autocast_custom_fwd, contiguous
 
 def fused_recurrent_fwd(q, k, v, g=None, gk=None, gv=None, scale=None, initial_state=None,
                         output_final_state=False, reverse=False, offsets=None, head_first=True,
-                        inplace_state=False):
+                        inplace_state=False, o_dtype=None):
     be.require_gpu(q, k, v)
     if head_first:
         tr = (lambda x: None if x is None else x.transpose(1, 2).contiguous())
         o, ht = fused_recurrent_fwd(tr(q), tr(k), tr(v), tr(g), tr(gk), tr(gv), scale, initial_state,
-                                    output_final_state, reverse, offsets, False, inplace_state)
+                                    output_final_state, reverse, offsets, False, inplace_state, o_dtype)
         return o.transpose(1, 2).contiguous(), ht
     B, T, H, K = k.shape
     V = v.shape[-1]
@@ -46,7 +46,7 @@ def fused_recurrent_fwd(q, k, v, g=None, gk=None, gv=None, scale=None, initial_s
             ht = h0
         else:
             ht = q.new_empty(N, H, K, V, dtype=torch.float32)
-    o = torch.empty_like(v, dtype=qkv_dtype)  # fp32 accumulation, rounded once on store
+    o = torch.empty_like(v, dtype=o_dtype or qkv_dtype)  # fp32 accumulation, rounded once on store
     if offsets is not None:
         offsets = offsets.to(torch.int64).contiguous()
     gate_code = be.FLA_F32 if gdt is None else be._DTYPES[gdt]
@@ -59,56 +59,115 @@ def fused_recurrent_fwd(q, k, v, g=None, gk=None, gv=None, scale=None, initial_s
     return o, ht
 
 
+def _gate_dtype(gates, qkv_dtype):
+    gates = [x for x in gates if x is not None]
+    if not gates:
+        return None
+    gdt = gates[0].dtype
+    if any(x.dtype != gdt for x in gates) or gdt not in (torch.float32, qkv_dtype):
+        gdt = torch.float32
+    return gdt
+
+
+def _per_token(term, B, T, offsets):
+    """A per-sequence tensor [N, ...] repeated over the tokens of its sequence: [B, T, ...]."""
+    if offsets is None:
+        return term.unsqueeze(1)
+    lens = offsets[1:] - offsets[:-1]
+    ids = torch.repeat_interleave(torch.arange(lens.numel(), device=term.device), lens, output_size=T)
+    return term[ids].unsqueeze(0)
+
+
+def fused_recurrent_bwd(q, k, v, g=None, gk=None, gv=None, o=None, do=None, dht=None, scale=None,
+                        initial_state=None, reverse=False, offsets=None, head_first=True, ht=None):
+    """Gradients of the recurrence (``fla/ops/common/fused_recurrent.py:381-468``): a token-by-token
+    kernel for dq, dk, dv, dh0 (fp32 arithmetic) and whole-sequence reverse cumulative sums for the
+    gates.  Returns ``(dq, dk, dv, dg, dgk, dgv, dh0)`` in fp32.  With ``dht`` and gates the final state
+    ``ht`` of the forward pass is needed as well: the last cumulative gate also scales the final state,
+    which adds ``sum(dht * ht)`` over the ungated dims to every token's gate gradient (the reference
+    leaves that term out and refuses the combination, ``:518-525``)."""
+    from ..utils.cumsum import chunk_global_cumsum
+    be.require_gpu(q, k, v, do)
+    if head_first:
+        tr = (lambda x: None if x is None else x.transpose(1, 2).contiguous())
+        outs = fused_recurrent_bwd(tr(q), tr(k), tr(v), tr(g), tr(gk), tr(gv), tr(o), tr(do), dht, scale,
+                                   initial_state, reverse, offsets, False, ht)
+        return tuple(None if x is None else x.transpose(1, 2) for x in outs[:6]) + (outs[6],)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    N = B if offsets is None else len(offsets) - 1
+    if K > 256 or V % 4:
+        raise NotImplementedError("fla_amd fused_recurrent backward: K <= 256 and V a multiple of 4")
+    qkv_dtype = q.dtype
+    q, k, v, do = q.contiguous(), k.to(qkv_dtype).contiguous(), v.to(qkv_dtype).contiguous(), do.to(qkv_dtype).contiguous()
+    gdt = _gate_dtype((g, gk, gv), qkv_dtype)
+    gg, ggk, ggv = (None if x is None else x.to(gdt).contiguous() for x in (g, gk, gv))
+    h0 = None if initial_state is None else initial_state.float().contiguous()
+    dht_ = None if dht is None else dht.float().contiguous()
+    if offsets is not None:
+        offsets = offsets.to(torch.int64).contiguous()
+    NV = -(-V // 64)
+    dq = q.new_empty(NV, B, T, H, K, dtype=torch.float32)
+    dk = q.new_empty(NV, B, T, H, K, dtype=torch.float32)
+    dv = q.new_empty(B, T, H, V, dtype=torch.float32)
+    dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
+    be.check(be.lib().fla_fused_recurrent_bwd(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(gg), be.ptr(ggk), be.ptr(ggv), be.ptr(h0), be.ptr(do), be.ptr(dht_),
+        be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dh0), be.ptr(offsets), be.dt(q),
+        be.FLA_F32 if gdt is None else be._DTYPES[gdt], B, T, H, K, V, N, float(scale), int(bool(reverse)),
+        be.stream_of(q)), "fla_fused_recurrent_bwd")
+    dq, dk = (dq[0] if NV == 1 else dq.sum(0)), (dk[0] if NV == 1 else dk.sum(0))
+    dg = dgk = dgv = None
+    if g is not None or gk is not None:
+        dgk_all = chunk_global_cumsum(dq * q.float() - dk * k.float(), reverse=not reverse, offsets=offsets,
+                                      head_first=False)
+        if dht is not None and ht is not None:
+            dgk_all = dgk_all + _per_token((dht_ * ht.float()).sum(-1), B, T, offsets)
+        if gk is not None:
+            dgk = dgk_all
+        if g is not None:
+            dg = dgk_all.sum(-1)
+    if gv is not None:
+        dgv = chunk_global_cumsum(do.float() * o.float() - dv * v.float(), reverse=not reverse, offsets=offsets,
+                                  head_first=False)
+        if dht is not None and ht is not None:
+            dgv = dgv + _per_token((dht_ * ht.float()).sum(-2), B, T, offsets)
+    return dq, dk, dv, dg, dgk, dgv, dh0
+
+
 class FusedRecurrentFunction(torch.autograd.Function):
-    """Forward: the token-by-token kernel.  Backward: the recurrence equals the chunked operator on
-    the same inputs, so the gradients come from ``chunk_gla``'s backward kernels (the reference runs
-    a second token-by-token pass, ``fla/ops/common/fused_recurrent.py:381-468``, and a global
-    reverse cumsum for the gates, ``:462-467``)."""
+    """Forward and backward are the token-by-token kernels, in fp32 arithmetic whatever the storage type
+    (``fla/ops/common/fused_recurrent.py:471-542``)."""
 
     @staticmethod
     @contiguous
     @autocast_custom_fwd
     def forward(ctx, q, k, v, g=None, gk=None, gv=None, scale=None, initial_state=None,
                 output_final_state=False, reverse=False, offsets=None, head_first=True, inplace_state=False):
-        o, ht = fused_recurrent_fwd(q, k, v, g, gk, gv, scale, initial_state, output_final_state, reverse,
-                                    offsets, head_first, inplace_state)
-        if any(t is not None and t.requires_grad for t in (q, k, v, g, gk, gv, initial_state)):
-            if inplace_state:
-                raise ValueError("inplace_state=True overwrites the initial state the backward needs")
-            ctx.save_for_backward(q, k, v, g, gk, gv, initial_state, offsets)
+        needs_grad = any(t is not None and t.requires_grad for t in (q, k, v, g, gk, gv, initial_state))
+        if needs_grad and inplace_state:
+            raise ValueError("inplace_state=True overwrites the initial state the backward needs")
+        gates_grad = any(t is not None and t.requires_grad for t in (g, gk, gv))
+        # the gate gradients read the unrounded output (gv) and the final state (a gradient of the final state)
+        o, ht = fused_recurrent_fwd(q, k, v, g, gk, gv, scale, initial_state, output_final_state or gates_grad,
+                                    reverse, offsets, head_first, inplace_state,
+                                    o_dtype=torch.float32 if (gv is not None and gv.requires_grad) else None)
+        if needs_grad:
+            ctx.save_for_backward(q, k, v, g, gk, gv, initial_state, offsets,
+                                  o if gv is not None and gv.requires_grad else None, ht if gates_grad else None)
             ctx.scale, ctx.reverse, ctx.head_first = scale, reverse, head_first
-        return o.to(q.dtype), ht
+        return o.to(q.dtype), (ht if output_final_state else None)
 
     @staticmethod
     @contiguous
     @autocast_custom_bwd
     def backward(ctx, do, dht):
-        import warnings
-
-        from ..gla.chunk import chunk_gla
-        q, k, v, g, gk, gv, h0, offsets = ctx.saved_tensors
-        if gv is not None or ctx.reverse:
-            raise NotImplementedError("fla_amd fused_recurrent backward: value gates (gv) and reverse=True are not covered")
-        leaves = [None if t is None else t.detach().requires_grad_() for t in (q, k, v, g, gk, h0)]
-        ql, kl, vl, gl, gkl, h0l = leaves
-        with torch.enable_grad(), warnings.catch_warnings():
-            warnings.simplefilter("ignore")
-            # one per-key log-gate: gk, plus the per-head scalar g broadcast over the key channels
-            gate = gkl.float() if gkl is not None else None
-            if gl is not None:
-                gs = gl.float().unsqueeze(-1).expand(*kl.shape)
-                gate = gs if gate is None else gate + gs
-            if gate is None:
-                gate = torch.zeros(kl.shape, dtype=torch.float32, device=kl.device)
-            o, ht = chunk_gla(ql, kl, vl, gate.contiguous(), scale=ctx.scale, initial_state=h0l, output_final_state=True,
-                              offsets=offsets, head_first=ctx.head_first)
-            outs, grads = [o], [do.to(o.dtype)]
-            if dht is not None:
-                outs.append(ht)
-                grads.append(dht.to(ht.dtype))
-            torch.autograd.backward(outs, grads)
-        dq, dk, dv, dg, dgk, dh0 = (None if t is None else t.grad for t in leaves)
-        return dq, dk, dv, dg, dgk, None, None, dh0, None, None, None, None, None
+        q, k, v, g, gk, gv, h0, offsets, o, ht = ctx.saved_tensors
+        dq, dk, dv, dg, dgk, dgv, dh0 = fused_recurrent_bwd(
+            q, k, v, g, gk, gv, o, do, dht, ctx.scale, h0, ctx.reverse, offsets, ctx.head_first, ht=ht)
+        cast = lambda x, like: None if (x is None or like is None) else x.to(like.dtype)
+        return (cast(dq, q), cast(dk, k), cast(dv, v), cast(dg, g), cast(dgk, gk), cast(dgv, gv), None,
+                cast(dh0, h0), None, None, None, None, None)
 
 
 def fused_recurrent(

@@ -19,7 +19,7 @@ import torch.nn.functional as F
 
 from ... import _backend as be
 from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
-                      resolve_offsets)
+                      empty_batch_result, resolve_offsets)
 from ..common.chunk_delta_h import (chunk_gated_delta_rule_fwd_h, chunk_gated_delta_rule_fwd_h_both,
                                     chunk_gated_delta_rule_fwd_scan)
 from ..common.chunk_o import chunk_fwd_o
@@ -277,4 +277,6 @@ def chunk_gated_delta_rule(
         scale = k.shape[-1] ** -0.5
     else:
         assert scale > 0, "Scale must be positive."
+    if q.numel() == 0:
+        return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
     return apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first)

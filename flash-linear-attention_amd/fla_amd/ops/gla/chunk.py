@@ -15,9 +15,9 @@ import torch
 import torch.nn.functional as F
 
 from ... import _backend as be
-from ...utils import VarlenPlan, check_varlen_args, contiguous, resolve_offsets
+from ...utils import VarlenPlan, check_varlen_args, contiguous, empty_batch_result, resolve_offsets
 from ..common.chunk_h import chunk_fwd_h
-from ..utils.cumsum import chunk_local_cumsum
+from ..utils.cumsum import chunk_local_cumsum, chunk_local_cumsum_inverse
 
 BT = 64
 _SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
@@ -260,31 +260,56 @@ def _gla_forward(q, k, v, g, scale, initial_state, output_final_state, offsets, 
     return o, ht, A
 
 
+def _internal_layout(head_first, *tensors):
+    """Seq-first, contiguous copies of the operands of an internal entry point."""
+    return tuple(None if t is None else (t.transpose(1, 2) if head_first else t).contiguous() for t in tensors)
+
+
+def _check_internal(q, k, v, T):
+    if min(BT, max(16, 1 << (max(T, 1) - 1).bit_length())) != BT:
+        raise NotImplementedError("fla_amd chunk_gla_fwd / chunk_gla_bwd: chunk size is fixed to 64 (needs T > 32)")
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise NotImplementedError("fla_amd chunk_gla_fwd / chunk_gla_bwd: q, k, v must share one 16-bit dtype")
+    if (q.shape[-1], v.shape[-1]) not in _SUPPORTED_KV:
+        raise NotImplementedError(f"fla_amd chunk_gla_fwd / chunk_gla_bwd: head dims {q.shape[-1]}, {v.shape[-1]} "
+                                  f"outside the built tiles {sorted(_SUPPORTED_KV)}")
+
+
 def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state,
                   offsets=None, indices=None, head_first=True, chunk_size=64):
-    """Reference-shaped forward (``fla/ops/gla/chunk.py:1156-1214``) for internal
-    callers: returns ``(g_cumsum, A, h, ht, o)`` with ``h`` row-major
-    ``[B,NT,H,K,V]`` and ``A`` fp32 ``[B,T,H,64]``."""
-    if head_first:
-        raise NotImplementedError("fla_amd chunk_gla_fwd: seq-first layout only")
-    T = q.shape[1]
-    if min(chunk_size, max(16, 1 << (T - 1).bit_length())) != BT:
-        raise NotImplementedError("fla_amd chunk_gla_fwd: chunk size is fixed to 64 (needs T > 32)")
+    """Reference-shaped forward (``fla/ops/gla/chunk.py:1156-1214``) for internal callers
+    (GSA calls it with ``g=None, g_cumsum=...``, ``fla/ops/gsa/chunk.py:622-636``): returns
+    ``(g_cumsum, A, h, ht, o)`` in the caller's layout, ``h`` row-major ``[B,NT,H,K,V]`` in the q/k/v dtype,
+    ``A`` fp32 ``[B,T,H,64]``.  ``o``, ``h`` and ``ht`` are exact for any gate (``o`` comes from the guarded
+    fused launch); ``A`` is scored with one reference point per chunk, i.e. exact while the chunk-cumulative
+    log-gate stays within +-80 (bf16) / +-8 (fp16) - the backward entry below does not read it."""
+    q, k, v, g, g_cumsum = _internal_layout(head_first, q, k, v, g, g_cumsum)
+    B, T, H, K = q.shape
+    _check_internal(q, k, v, T)
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
+    co = None if plan is None else plan.chunk_offsets
     if g_cumsum is None:
         g_cumsum = chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
+    elif g_cumsum.dtype != torch.float32:
+        g_cumsum = g_cumsum.float()
+    if g is None:
+        g = chunk_local_cumsum_inverse(g_cumsum, BT, offsets=offs, indices=idx, head_first=False)
     h, ht = chunk_fwd_h(k=k, v=v, g=None, gk=g_cumsum, gv=None, h0=initial_state,
                         output_final_state=output_final_state, offsets=offs, indices=idx, head_first=False,
-                        chunk_size=BT, chunk_offsets=None if plan is None else plan.chunk_offsets)
-    hf, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g_cumsum, gv=None, h0=initial_state, output_final_state=False,
-                        offsets=offs, indices=idx, head_first=False, chunk_size=BT, fragment_layout=True,
-                        chunk_offsets=None if plan is None else plan.chunk_offsets)
-    B, _, H, _ = q.shape
+                        chunk_size=BT, chunk_offsets=co)
+    # the scores depend on q, k and the gates only: the score launch also forms an output from whatever
+    # states it is given, which is discarded here (the row-major states stand in for the fragment-order ones,
+    # same size), and o comes from the guarded fused launch instead
     A = q.new_empty(B, T, H, BT, dtype=torch.float32)
-    o = chunk_gla_fwd_o_gk(q, v, g_cumsum, None, hf, scale, offsets=offs, indices=idx, head_first=False,
-                           chunk_size=BT, k=k, gates_are_cumsum=True, A_out=A)
+    chunk_gla_fwd_o_gk(q, v, g_cumsum, None, h, scale, offsets=offs, indices=idx, head_first=False,
+                       chunk_size=BT, k=k, gates_are_cumsum=True, A_out=A)
+    o, _ = chunk_gla_fwd_fused(q, k, v, g if g.dtype in (torch.float32, q.dtype) else g.float(), scale, initial_state,
+                               False, offsets)
+    if head_first:
+        g_cumsum, A, o = (x.transpose(1, 2) for x in (g_cumsum, A, o))
+        h = h.transpose(1, 2)
     return g_cumsum, A, h, ht, o
 
 
@@ -324,15 +349,31 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
 
 def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
                   offsets=None, indices=None, head_first=True, chunk_size=64):
-    """Reference-shaped backward (``fla/ops/gla/chunk.py:1217-1320``) for internal callers:
-    returns ``(dq, dk, dv, dg, dh0)`` with ``dg`` the gradient of the raw gates ``g``.  The
-    per-chunk states and scores are recomputed on chip, so ``g_cumsum``, ``h`` and ``A`` are
-    accepted and ignored; tensors must be seq-first, 16-bit, with head dims of 64 or 128."""
-    if head_first:
-        raise NotImplementedError("fla_amd chunk_gla_bwd: seq-first layout only")
+    """Reference-shaped backward (``fla/ops/gla/chunk.py:1217-1320``) for internal callers (GSA:
+    ``g=None, g_cumsum=..., h=..., A=...``, ``fla/ops/gsa/chunk.py:741-757``): returns ``(dq, dk, dv, dg, dh0)`` in
+    the caller's layout, ``dg`` the gradient of the raw gates (the chunk-local reverse cumulative sum already
+    applied, as ``chunk_gla_bwd_kernel_inter`` leaves it, ``fla/ops/gla/chunk.py:818-823``).  Either ``g`` or
+    ``g_cumsum`` may be ``None``.  The per-chunk states and the gate-range flags come from one run of the fused
+    forward launch and the scores are recomputed on chip, so ``h`` and ``A`` are accepted and not read; exact for
+    any gate."""
+    q, k, v, g, g_cumsum, do = _internal_layout(head_first, q, k, v, g, g_cumsum, do)
+    _check_internal(q, k, v, q.shape[1])
     if g is None:
-        raise NotImplementedError("fla_amd chunk_gla_bwd: needs the raw gates g (the kernels form the cumulative sums)")
-    return chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht, offsets)
+        if g_cumsum is None:
+            raise ValueError("chunk_gla_bwd needs g or g_cumsum")
+        plan = VarlenPlan(offsets, BT) if offsets is not None else None
+        g = chunk_local_cumsum_inverse(g_cumsum, BT, offsets=None if plan is None else plan.offsets,
+                                       indices=None if plan is None else plan.indices, head_first=False)
+    elif g.dtype not in (torch.float32, q.dtype):
+        g = g.float()
+    states = []
+    _, _, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, False, offsets, return_flags=True,
+                                     states_out=states)
+    dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht,
+                                               offsets, wide, hT=states[0])
+    if head_first:
+        dq, dk, dv, dg = (x.transpose(1, 2) for x in (dq, dk, dv, dg))
+    return dq, dk, dv, dg, dh0
 
 
 class ChunkGLAFunction(torch.autograd.Function):
@@ -437,6 +478,8 @@ def chunk_gla(
     check_varlen_args(q, offsets, head_first, initial_state)
     if scale is None:
         scale = q.shape[-1] ** -0.5
+    if q.numel() == 0:
+        return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
     K, V = q.shape[-1], v.shape[-1]
     if K > 128:
         # every key channel carries its own row of the state and o sums over them: wider key heads

@@ -47,6 +47,39 @@ def chunk_local_cumsum(
     return out
 
 
+def chunk_local_cumsum_inverse(
+    g_cumsum: torch.Tensor,
+    chunk_size: int,
+    reverse: bool = False,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+) -> torch.Tensor:
+    """The raw values whose ``chunk_local_cumsum`` is ``g_cumsum`` (fp32): differences of consecutive rows
+    inside every chunk (``fla_chunk_local_cumsum_inverse``).  No counterpart in the reference, whose internal
+    entry points take the cumulative gates as they are; the kernels here start from the raw gates."""
+    be.require_gpu(g_cumsum)
+    if head_first:
+        out = chunk_local_cumsum_inverse(g_cumsum.transpose(1, 2), chunk_size, reverse, offsets, indices, head_first=False)
+        return out.transpose(1, 2).contiguous()
+    g = g_cumsum.float().contiguous()
+    B, T, H = g.shape[:3]
+    S = g.shape[3] if g.dim() == 4 else 1
+    out = torch.empty_like(g)
+    NT = 0
+    if offsets is not None:
+        if indices is None:
+            plan = VarlenPlan(offsets, chunk_size)
+            offsets, indices = plan.offsets, plan.indices
+        offsets = offsets.to(torch.int64).contiguous()
+        indices = indices.to(torch.int64).contiguous()
+        NT = indices.shape[0]
+    be.check(be.lib().fla_chunk_local_cumsum_inverse(
+        be.ptr(g), be.ptr(out), B, T, H, S, chunk_size, int(bool(reverse)), be.ptr(offsets), be.ptr(indices), NT,
+        be.stream_of(g)), "fla_chunk_local_cumsum_inverse")
+    return out
+
+
 def chunk_global_cumsum(
     s: torch.Tensor,
     dtype: Optional[torch.dtype] = None,

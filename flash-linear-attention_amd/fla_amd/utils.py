@@ -140,3 +140,19 @@ def check_varlen_args(q, offsets, head_first, initial_state):
         if initial_state is not None and initial_state.shape[0] != len(offsets) - 1:
             raise ValueError(f"The number of initial states is expected to be equal to the number of input sequences, "
                              f"i.e., {len(offsets) - 1} rather than {initial_state.shape[0]}.")
+
+
+def empty_batch_result(q, v, offsets, initial_state, output_final_state):
+    """What a chunk operator returns for a batch without a single token (zero-size tensors have no
+    device address to hand to a kernel): an empty output and the initial states as final states,
+    through ``clone`` so that the gradient of the final states reaches the initial ones."""
+    o = torch.empty_like(v)
+    ht = None
+    if output_final_state:
+        if initial_state is not None:
+            ht = initial_state.float().clone()
+        else:
+            N = q.shape[0] if offsets is None else len(offsets) - 1
+            H = q.shape[2] if q.dim() == 4 else 1
+            ht = q.new_zeros(N, H, q.shape[-1], v.shape[-1], dtype=torch.float32)
+    return o, ht

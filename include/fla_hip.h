@@ -68,6 +68,14 @@ int fla_chunk_local_cumsum(const void* g, float* out, int g_dtype,
                            const int64_t* offsets, const int64_t* indices, int64_t NT,
                            fla_stream_t stream);
 
+/* The inverse of fla_chunk_local_cumsum on fp32 data: out[t] = g_cumsum[t] - g_cumsum[t-1] inside every chunk
+ * (the chunk's first row keeps its value; reverse: last row, differences taken towards the end).  For callers
+ * of the reference's internal entry points that hold only the cumulative gates (chunk_gla_bwd called with
+ * g=None, g_cumsum=..., fla/ops/gsa/chunk.py:741-757) while the kernels here start from the raw ones. */
+int fla_chunk_local_cumsum_inverse(const float* g_cumsum, float* out, int64_t B, int64_t T, int64_t H, int64_t S,
+                                   int64_t chunk_size, int reverse, const int64_t* offsets,
+                                   const int64_t* indices, int64_t NT, fla_stream_t stream);
+
 /* Cumulative sum over the whole sequence (not restarted at chunk boundaries), replaces
  * chunk_global_cumsum (fla/ops/utils/cumsum.py:308-386).  Two launches: chunk-local sums into
  * ws_local (fp32, same shape as s), then each chunk adds the totals of the chunks before
@@ -106,6 +114,19 @@ int fla_fused_recurrent_fwd(const void* q, const void* k, const void* v,
                             int qkv_dtype, int gate_dtype, int o_dtype,
                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                             float scale, int reverse, fla_stream_t stream);
+
+/* Token-by-token backward of the same recurrence, replaces fused_recurrent_bwd
+ * (fla/ops/common/fused_recurrent.py:381-468, kernel :131-319): two passes over the tokens (rebuild h_t and
+ * emit dq; then the reverse scan of dh emitting dk, dv), fp32 arithmetic.  dout [B,T,H,V] in the q/k/v dtype;
+ * h0, dht, dh0 fp32 [N,H,K,V] or NULL.  dq_partial and dk_partial are fp32 [ceil(V/64), B, T, H, K]: one slice
+ * per 64 value columns, their sum over the first dimension is the gradient (the reference sums such partial
+ * tensors as well, :445-447); dv is fp32 [B,T,H,V].  The gate gradients follow from these on the caller's side
+ * (whole-sequence reverse cumulative sums of q*dq - k*dk and do*o - dv*v, :448-467).  K <= 256, V % 4 == 0. */
+int fla_fused_recurrent_bwd(const void* q, const void* k, const void* v, const void* g, const void* gk,
+                            const void* gv, const float* h0, const void* dout, const float* dht,
+                            float* dq_partial, float* dk_partial, float* dv, float* dh0, const int64_t* offsets,
+                            int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                            int64_t N, float scale, int reverse, fla_stream_t stream);
 
 /* Gated delta rule recurrence, forward
  * (fla/ops/gated_delta_rule/fused_recurrent.py:113-167, kernel :19-110).

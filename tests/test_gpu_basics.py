@@ -94,3 +94,25 @@ def test_global_cumsum_varlen(device, reverse):
         x = s[:, a:b].double()
         ref[:, a:b] = x.flip(1).cumsum(1).flip(1) if reverse else x.cumsum(1)
     assert_close("cumsum", ref, out, 1e-5)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_local_cumsum_inverse(device, varlen, reverse):
+    """Differences of consecutive rows inside every chunk: undoes chunk_local_cumsum (to fp32 rounding) and is
+    exact on integers."""
+    from fla_amd.ops.utils.cumsum import chunk_local_cumsum, chunk_local_cumsum_inverse
+    gen = torch.Generator().manual_seed(23)
+    T = 333
+    offs = torch.tensor([0, 5, 5, 200, 333], device=device) if varlen else None
+    x = torch.randint(-8, 9, (1 if varlen else 2, T, 3, 8), generator=gen).float().to(device)
+    print(f"local cumsum inverse varlen={varlen} reverse={reverse}", flush=True)
+    G = chunk_local_cumsum(x, 64, reverse=reverse, offsets=offs, head_first=False)
+    back = chunk_local_cumsum_inverse(G, 64, reverse=reverse, offsets=offs, head_first=False)
+    assert torch.equal(back, x)
+    y = torch.randn(2, T, 3, generator=gen).to(device)
+    Gy = chunk_local_cumsum(y, 64, reverse=reverse, head_first=False)
+    assert_close("round trip", y, chunk_local_cumsum_inverse(Gy, 64, reverse=reverse, head_first=False), 1e-5)
+    Gh = chunk_local_cumsum(y.transpose(1, 2).contiguous(), 64, reverse=reverse, head_first=True)
+    assert torch.equal(chunk_local_cumsum_inverse(Gh, 64, reverse=reverse, head_first=True).transpose(1, 2),
+                       chunk_local_cumsum_inverse(Gy, 64, reverse=reverse, head_first=False))

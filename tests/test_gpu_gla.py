@@ -266,6 +266,94 @@ def test_chunk_gla_internal_fwd_bwd_signatures(device):
         assert_close(name, r, x, tol)
 
 
+@pytest.mark.parametrize("head_first", [False, True])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_internal_entries_as_gsa_calls_them(device, head_first, varlen):
+    """chunk_gla_fwd / chunk_gla_bwd with GSA's argument lists (fla/ops/gsa/chunk.py:622-636 and :741-757):
+    g=None, g_cumsum = the chunk-local cumulative gates, the saved h and A handed back to the backward,
+    either layout, keyword arguments throughout."""
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd, chunk_gla_fwd
+    from fla_amd.utils import prepare_chunk_indices
+    from oracle.chunked import chunked_gla
+    from oracle.cumsum import chunk_local_cumsum as ref_cumsum
+    if varlen and head_first:
+        pytest.skip("packed batches are seq-first")
+    B, T, H, K, V = (1, 300, 2, 128, 64) if varlen else (2, 200, 2, 128, 64)
+    N = 3 if varlen else B
+    offs = torch.tensor([0, 70, 71, 300]) if varlen else None
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=35, h0_std=1.0, N=N)
+    gen = torch.Generator().manual_seed(10)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(N, H, K, V, generator=gen) * 0.1
+    gc = ref_cumsum(g, 64, offsets=None if offs is None else offs.tolist())
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    dev = lambda x: None if x is None else x.to(device)
+    print(f"chunk_gla_fwd / bwd, GSA calling form, head_first={head_first} varlen={varlen}", flush=True)
+    doffs = dev(offs)
+    idx = None if offs is None else prepare_chunk_indices(doffs, 64)
+    A, h, ht, o = chunk_gla_fwd(q=dev(tr(q)), k=dev(tr(k)), v=dev(tr(v)), g=None, g_cumsum=dev(tr(gc)), scale=K ** -0.5,
+                                initial_state=dev(h0), output_final_state=True, offsets=doffs, indices=idx,
+                                head_first=head_first, chunk_size=64)[1:]
+    ref = chunked_gla(q, k, v, g, initial_state=h0, offsets=None if offs is None else offs.tolist())
+    assert_close("o", ref['o'], tr(o) if head_first else o, TOL_O)
+    assert_close("ht", ref['ht'], ht, TOL_HT)
+    assert_close("A", ref['A'], tr(A) if head_first else A, 1e-2)
+    assert_close("h", ref['h'], h.transpose(1, 2) if head_first else h, 5e-3)
+    dq, dk, dv, dg, dh0 = chunk_gla_bwd(q=dev(tr(q)), k=dev(tr(k)), v=dev(tr(v)), g=None, g_cumsum=dev(tr(gc)),
+                                        scale=K ** -0.5, initial_state=dev(h0), h=h, A=A, do=dev(tr(do)), dht=dev(dht),
+                                        offsets=doffs, indices=idx, head_first=head_first, chunk_size=64)
+    grads = _grads_ref(q, k, v, g, h0, do, dht, offsets=offs)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), grads, (dq, dk, dv, dg, dh0), (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(name, r, tr(x) if (head_first and name != "dh0") else x, tol)
+
+
+def test_chunk_gla_internal_entries_strong_gates_fp16(device):
+    """The internal forward and backward stay exact where the single-reference-point scores leave their
+    range (fp16: a chunk-cumulative log-gate beyond 8): o and the gradients come from the guarded launches."""
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd, chunk_gla_fwd
+    from oracle.recurrent import naive_recurrent_gla
+    B, T, H, D = 2, 130, 2, 64
+    q, k, v, g, h0 = gla_inputs(B, T, H, D, D, seed=36, dtype=torch.float16, normalizer=1.0, h0_std=1.0)
+    gen = torch.Generator().manual_seed(11)
+    do = torch.randn(B, T, H, D, generator=gen).half()
+    dht = torch.randn(B, H, D, D, generator=gen) * 0.1
+    dev = lambda x: x.to(device)
+    print("chunk_gla_fwd / bwd, fp16, strong gates", flush=True)
+    gc, A, h, ht, o = chunk_gla_fwd(dev(q), dev(k), dev(v), dev(g), None, D ** -0.5, dev(h0), True, head_first=False)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True)
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    dq, dk, dv, dg, dh0 = chunk_gla_bwd(dev(q), dev(k), dev(v), dev(g), gc, D ** -0.5, dev(h0), h, A, dev(do), dev(dht),
+                                        head_first=False)
+    grads = _grads_ref(q, k, v, g, h0, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), grads, (dq, dk, dv, dg, dh0), (1e-2, 1e-2, 1e-2, 2e-2, 5e-3)):
+        assert_close(name, r, x, tol)
+
+
+def test_chunk_backward_of_an_empty_batch(device):
+    """No chunk at all (a packed batch whose sequences are all empty): the gradient of the initial
+    states is the gradient of the final states, and nothing else is touched."""
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_amd.ops.gla import chunk_gla
+    H, D, N = 2, 64, 2
+    offs = torch.zeros(N + 1, dtype=torch.int64, device=device)
+    z = lambda *sh: torch.zeros(*sh, device=device, dtype=torch.bfloat16).requires_grad_()
+    dht = torch.randn(N, H, D, D, device=device)
+    print("backward of an empty packed batch", flush=True)
+    for name in ("gla", "gdr"):
+        h0 = torch.randn(N, H, D, D, device=device).requires_grad_()
+        if name == "gla":
+            o, ht = chunk_gla(z(1, 0, H, D), z(1, 0, H, D), z(1, 0, H, D), torch.zeros(1, 0, H, D, device=device),
+                              initial_state=h0, output_final_state=True, offsets=offs, head_first=False)
+        else:
+            o, ht = chunk_gated_delta_rule(z(1, 0, H, D), z(1, 0, H, D), z(1, 0, H, D),
+                                           torch.zeros(1, 0, H, device=device), torch.zeros(1, 0, H, device=device),
+                                           initial_state=h0, output_final_state=True, offsets=offs, head_first=False)
+        assert torch.equal(ht, h0.detach())
+        (ht * dht).sum().backward()
+        assert torch.equal(h0.grad, dht), name
+
+
 # The reference's own ladder (tests/ops/test_gla.py:90-146): head dims 300 and 100 (key and value
 # slabs of 128 after padding), both layouts, gate_logit_normalizer 1 / 0.05 / 20.
 @pytest.mark.parametrize("D,T,normalizer,head_first", [

@@ -140,8 +140,7 @@ def test_decode_inplace_matches_out_of_place(device, op):
 def test_fused_recurrent_gla_backward(device, dtype, T, D, head_first):
     """Gradients of the token-by-token operator (the layers' path for sequences of at most 64
     tokens) against autograd through the naive recurrence, at the reference's tolerance for this
-    operator (tests/ops/test_gla.py:66-87 uses 0.005 in fp32; the kernels behind the backward
-    round q, k, v to bf16, hence the bar of the chunked operator here)."""
+    operator (tests/ops/test_gla.py:66-87 uses 0.005 in fp32)."""
     from fla_amd.ops.gla import fused_recurrent_gla
     from oracle.recurrent import naive_recurrent_gla
     B, H = 2, 2
@@ -165,28 +164,98 @@ def test_fused_recurrent_gla_backward(device, dtype, T, D, head_first):
     assert_close("dh0", rh0.grad, h0l.grad, 8e-3)
 
 
-def test_fused_recurrent_scalar_gate_backward_and_guards(device):
-    """Per-head scalar gates (the simple-GLA form) through the same backward; value gates and
-    reverse scans are refused loudly."""
+@pytest.mark.parametrize("reverse", [False, True])
+@pytest.mark.parametrize("gates", ["g", "gk", "gv", "gk+gv", "g+gk+gv", "none"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_recurrent_backward_all_gates(device, gates, reverse, dtype):
+    """dq, dk, dv, every gate gradient and dh0 of the token-by-token operator, with a gradient of the final
+    state as well, against autograd through the fp32 naive recurrence (fla/ops/common/fused_recurrent.py:381-468
+    covers g, gk, gv and reverse).  fp32 inputs: both sides are fp32 recurrences, 1e-4; bf16 inputs: the output is
+    rounded once, the rest is fp32."""
     from fla_amd.ops.common.fused_recurrent import fused_recurrent
     from oracle.recurrent import naive_recurrent_gla
-    B, T, H, D = 2, 50, 2, 64
-    gen = torch.Generator().manual_seed(8)
-    q, k, v = (torch.randn(B, T, H, D, generator=gen).bfloat16() for _ in range(3))
-    g = F.logsigmoid(torch.randn(B, T, H, generator=gen))
-    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
-    leaves = [x.to(device).requires_grad_() for x in (q, k, v, g)]
-    o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], g=leaves[3], head_first=False)
-    (o.float() * do.to(device).float()).sum().backward()
-    refs = [x.float().requires_grad_() for x in (q, k, v, g)]
-    ro, _ = naive_recurrent_gla(refs[0], refs[1], refs[2], None, g=refs[3])
-    (ro * do.float()).sum().backward()
-    for name, r, x, tol in zip(("dq", "dk", "dv", "dg"), refs, leaves, (8e-3, 8e-3, 8e-3, 4e-2)):
+    B, T, H, K, V = 2, 70, 2, 64, 128
+    gen = torch.Generator().manual_seed(8 + len(gates))
+    q, k = (torch.randn(B, T, H, K, generator=gen).to(dtype) for _ in range(2))
+    v = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    gd = {"g": F.logsigmoid(torch.randn(B, T, H, generator=gen)) / 4 if "g" in gates.split("+") else None,
+          "gk": F.logsigmoid(torch.randn(B, T, H, K, generator=gen)) / 4 if "gk" in gates else None,
+          "gv": F.logsigmoid(torch.randn(B, T, H, V, generator=gen)) / 4 if "gv" in gates else None}
+    h0 = torch.randn(B, H, K, V, generator=gen)
+    do = torch.randn(B, T, H, V, generator=gen).to(dtype)
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    print(f"fused_recurrent backward gates={gates} reverse={reverse} {dtype}", flush=True)
+    mk = lambda x: None if x is None else x.to(device).requires_grad_()
+    ql, kl, vl, h0l = mk(q), mk(k), mk(v), mk(h0)
+    gl = {n: mk(x) for n, x in gd.items()}
+    o, ht = fused_recurrent(ql, kl, vl, g=gl["g"], gk=gl["gk"], gv=gl["gv"], initial_state=h0l, output_final_state=True,
+                            reverse=reverse, head_first=False)
+    ((o.float() * do.to(device).float()).sum() + (ht * dht.to(device)).sum()).backward()
+    rq, rk, rv, rh0 = (x.float().requires_grad_() for x in (q, k, v, h0))
+    rg = {n: None if x is None else x.clone().requires_grad_() for n, x in gd.items()}
+    ro, rht = naive_recurrent_gla(rq, rk, rv, rg["gk"], g=rg["g"], gv=rg["gv"], initial_state=rh0,
+                                  output_final_state=True, reverse=reverse)
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    tol = 1e-4 if dtype == torch.float32 else 8e-3
+    assert_close("o", ro, o, 1e-5 if dtype == torch.float32 else 5e-3)
+    for name, r, x in (("dq", rq, ql), ("dk", rk, kl), ("dv", rv, vl), ("dh0", rh0, h0l)):
+        assert x.grad.dtype == x.dtype
         assert_close(name, r.grad, x.grad, tol)
-    gv = F.logsigmoid(torch.randn(B, T, H, D, generator=gen)).to(device)
-    o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], gv=gv, head_first=False)
-    with pytest.raises(NotImplementedError):
-        o.sum().backward()
+    for n in ("g", "gk", "gv"):
+        if gd[n] is not None:
+            assert_close("d" + n, rg[n].grad, gl[n].grad, 5e-4 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_fused_recurrent_backward_packed_and_head_first(device, reverse):
+    from fla_amd.ops.common.fused_recurrent import fused_recurrent
+    from oracle.recurrent import naive_recurrent_gla
+    T, N, H, K, V = 90, 4, 2, 100, 64
+    gen = torch.Generator().manual_seed(77)
+    offs = torch.tensor([0, 1, 40, 40, 90])
+    q, k = (torch.randn(1, T, H, K, generator=gen) for _ in range(2))
+    v = torch.randn(1, T, H, V, generator=gen)
+    gk = F.logsigmoid(torch.randn(1, T, H, K, generator=gen)) / 4
+    gv = F.logsigmoid(torch.randn(1, T, H, V, generator=gen)) / 4
+    h0 = torch.randn(N, H, K, V, generator=gen)
+    do = torch.randn(1, T, H, V, generator=gen)
+    dht = torch.randn(N, H, K, V, generator=gen) * 0.1
+    print(f"fused_recurrent backward packed reverse={reverse}", flush=True)
+    leaves = [x.to(device).requires_grad_() for x in (q, k, v, gk, gv, h0)]
+    o, ht = fused_recurrent(leaves[0], leaves[1], leaves[2], gk=leaves[3], gv=leaves[4], initial_state=leaves[5],
+                            output_final_state=True, reverse=reverse, offsets=offs.to(device), head_first=False)
+    ((o * do.to(device)).sum() + (ht * dht.to(device)).sum()).backward()
+    refs = [x.clone().requires_grad_() for x in (q, k, v, gk, gv, h0)]
+    ro, rht = naive_recurrent_gla(refs[0], refs[1], refs[2], refs[3], gv=refs[4], initial_state=refs[5],
+                                  output_final_state=True, reverse=reverse, offsets=offs.tolist())
+    ((ro * do).sum() + (rht * dht).sum()).backward()
+    for name, r, x in zip(("dq", "dk", "dv", "dgk", "dgv", "dh0"), refs, leaves):
+        assert_close(name, r.grad, x.grad, 5e-4)
+    # head-first, equal lengths, per-head gate
+    B, T2 = 2, 33
+    q, k, v = (torch.randn(B, H, T2, 64, generator=gen) for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, H, T2, generator=gen))
+    do = torch.randn(B, H, T2, 64, generator=gen)
+    leaves = [x.to(device).requires_grad_() for x in (q, k, v, g)]
+    o, _ = fused_recurrent(leaves[0], leaves[1], leaves[2], g=leaves[3], reverse=reverse, head_first=True)
+    (o * do.to(device)).sum().backward()
+    refs = [x.transpose(1, 2).clone().requires_grad_() for x in (q, k, v, g)]
+    ro, _ = naive_recurrent_gla(refs[0], refs[1], refs[2], None, g=refs[3], reverse=reverse)
+    (ro * do.transpose(1, 2)).sum().backward()
+    for name, r, x in zip(("dq", "dk", "dv", "dg"), refs, leaves):
+        assert_close(name + " head-first", r.grad, x.grad.transpose(1, 2), 5e-4)
+
+
+def test_fused_recurrent_inplace_state_refused_before_launch(device):
+    """A state that would be overwritten while a backward needs it is refused before anything runs."""
+    from fla_amd.ops.common.fused_recurrent import fused_recurrent
+    q = torch.randn(1, 1, 1, 64, device=device).requires_grad_()
+    state = torch.ones(1, 1, 64, 64, device=device)
+    with pytest.raises(ValueError, match="inplace_state"):
+        fused_recurrent(q, q.detach(), q.detach(), initial_state=state, output_final_state=True, head_first=False,
+                        inplace_state=True)
+    torch.cuda.synchronize()
+    assert torch.equal(state, torch.ones_like(state))
 
 
 # ---------------------------------------------------------------- prefill + decode through the Cache
