@@ -63,15 +63,19 @@ class Cache:
         Returns the layer's dict."""
         if layer_idx == 0:
             self._seen_tokens += offset
-        window_size = None
         if attn_state is not None:
             if not isinstance(attn_state, (tuple, list)) or len(attn_state) != 2:
                 raise ValueError("`attn_state` must be a tuple of two tensors for key/value states")
+            # key/value states of softmax-attention layers in hybrid models (outside the linear-attention path;
+            # kept for interface parity): appended along the token axis, optionally cut to the newest
+            # `window_size` tokens
+            held = self.states[layer_idx].get('attn_state') if layer_idx < len(self.states) else None
+            if held is not None:
+                attn_state = tuple(torch.cat([h, n], -2) for h, n in zip(held, attn_state))
             window_size = (cache_kwargs or {}).get('window_size', None)
-            input_size = attn_state[0].shape[-2]
-        if len(self.states) <= layer_idx:
-            if attn_state is not None and window_size is not None and input_size > window_size:
+            if window_size is not None and attn_state[0].shape[-2] > window_size:
                 attn_state = tuple(x[..., -window_size:, :].contiguous() for x in attn_state)
+        if len(self.states) <= layer_idx:
             state = dict(recurrent_state=recurrent_state, attn_state=attn_state, conv_state=conv_state,
                          ffn_state=ffn_state)
             self.states.append(state)
@@ -80,16 +84,6 @@ class Cache:
         if recurrent_state is not None:
             state['recurrent_state'] = self._keep(state.get('recurrent_state'), recurrent_state)
         if attn_state is not None:
-            key_state, value_state = state['attn_state']
-            if window_size is not None and key_state.shape[-2] == window_size:
-                # full window: shift left by the number of new tokens inside the held buffers
-                key_state = key_state.roll(-input_size, -2)
-                value_state = value_state.roll(-input_size, -2)
-                key_state[..., -input_size:, :] = attn_state[0]
-                value_state[..., -input_size:, :] = attn_state[1]
-                attn_state = (key_state, value_state)
-            else:
-                attn_state = (torch.cat([key_state, attn_state[0]], -2), torch.cat([value_state, attn_state[1]], -2))
             state['attn_state'] = attn_state
         if conv_state is not None:
             held = state.get('conv_state')

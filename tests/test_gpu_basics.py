@@ -116,3 +116,41 @@ def test_local_cumsum_inverse(device, varlen, reverse):
     Gh = chunk_local_cumsum(y.transpose(1, 2).contiguous(), 64, reverse=reverse, head_first=True)
     assert torch.equal(chunk_local_cumsum_inverse(Gh, 64, reverse=reverse, head_first=True).transpose(1, 2),
                        chunk_local_cumsum_inverse(Gy, 64, reverse=reverse, head_first=False))
+
+
+def _config2_offsets():
+    """The packed workload's boundaries: 12 lengths drawn uniformly in [256, 6000], rescaled to sum to 32768."""
+    gen = torch.Generator().manual_seed(0)
+    lens = torch.randint(256, 6001, (12,), generator=gen).double()
+    lens = (lens / lens.sum() * 32768).round().long()
+    lens[-1] += 32768 - lens.sum()
+    return torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)])
+
+
+@pytest.mark.parametrize("bt", [16, 64])
+def test_varlen_plan_device_tables_bit_exact(device, bt):
+    """The chunk tables a packed launch reads on the device (indices, chunk_offsets, seq_order) against the
+    oracle's, bit for bit, together with the reference-held known answer."""
+    import json
+    import os
+    import numpy as np
+    from fla_amd.utils import VarlenPlan
+    from oracle import bookkeeping
+    with open(os.path.join(os.path.dirname(__file__), "golden", "chunk_indices_known_answer.json")) as f:
+        ka = json.load(f)
+    cases = [_config2_offsets().tolist(), ka["offsets"], [0, 0], [0, 1], [0, 63, 64, 65, 1000], [0, 5, 5, 5, 700]]
+    for offs in cases:
+        print(f"varlen plan bt={bt} offsets={offs}", flush=True)
+        plan = VarlenPlan(torch.tensor(offs, dtype=torch.int64, device=device), bt)
+        assert plan.indices.is_cuda and plan.chunk_offsets.is_cuda and plan.seq_order.is_cuda
+        assert plan.indices.dtype == torch.int64 and plan.chunk_offsets.dtype == torch.int64
+        ref_idx = bookkeeping.prepare_chunk_indices(offs, bt)
+        assert np.array_equal(plan.indices.cpu().numpy().reshape(-1, 2), ref_idx)
+        assert np.array_equal(plan.chunk_offsets.cpu().numpy(), bookkeeping.prepare_chunk_offsets(offs, bt))
+        assert plan.NT == ref_idx.shape[0] and plan.N == len(offs) - 1
+        lens = np.diff(np.asarray(offs))
+        order = plan.seq_order.cpu().numpy()
+        assert sorted(order.tolist()) == list(range(len(lens)))            # a permutation of the sequence ids,
+        assert (np.diff(lens[order]) <= 0).all()                           # longest first
+    plan = VarlenPlan(torch.tensor(ka["offsets"], dtype=torch.int64, device=device), ka["chunk_size"])
+    assert plan.indices.cpu().tolist() == ka["indices"]
