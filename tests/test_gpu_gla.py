@@ -410,3 +410,20 @@ def test_chunk_gla_keep_vs_recompute(device, varlen, monkeypatch):
     for name, a, b, r, tol in zip(("dq", "dk", "dv", "dg", "dh0"), kept, rec, ref, (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
         assert_close(f"{name} kept vs recomputed", b, a, 2e-3)
         assert_close(f"{name} recomputed vs oracle", r, b, tol)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_gradients_are_reproducible(device, varlen):
+    """Same inputs twice: every gradient identical bit for bit."""
+    gen = torch.Generator().manual_seed(14)
+    T, N, H, D = 700, 4, 3, 128
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q, k, v, g, h0 = gla_inputs(1 if varlen else 2, T, H, D, D, seed=65, N=N if varlen else None, h0_std=1.0)
+    do = torch.randn(q.shape[0], T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    print(f"chunk_gla reproducibility varlen={varlen}", flush=True)
+    first = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+    for _ in range(3):
+        again = _grads_dev(device, q, k, v, g, h0, do, dht, offsets=offs)
+        for name, a, b in zip(("dq", "dk", "dv", "dg", "dh0"), first, again):
+            assert torch.equal(a, b), name
