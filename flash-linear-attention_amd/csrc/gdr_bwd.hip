@@ -831,9 +831,15 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA (masked) -> dM
   __shared__ float sBeta[BT], sGam[BT];
   // Partial sums of dbeta and dgamma, one slot per contributing wave and step, added in a fixed order at the
-  // end (no atomics: the gradients are bit-reproducible from run to run).  dbeta: value side / key side x the
-  // two column halves; dgamma: row sums from the two column blocks, column sums from the two row blocks.
-  __shared__ float sDbP[4][BT], sDgRow[2][BT], sDgCol[2][BT];
+  // end (no atomics: the gradients are bit-reproducible from run to run).  Slots 0-3: dbeta from the value
+  // side / key side x the two column halves; 4-5: dgamma row sums from the two column blocks; 6-7: dgamma
+  // column sums from the two row blocks.  They live in the 16 bytes of padding behind every row of the
+  // transposed tile (and of the Aw tile where that one has only 64 rows), which no tile access touches, so
+  // that two workgroups still fit a CU.
+  auto slot = [&](int s_, int r) -> float& {
+    T* base = s_ < 4 ? &sTr1[r * LDT + BT] : (D >= 128 ? &sTr1[(r + BT) * LDT + BT] : &sAw[r * LDT + BT]);
+    return ((float*)base)[s_ & 3];
+  };
   // X1^T, then dM^T diag(beta): lives in the du/dw tile, which is dead once dA has been formed
   // (two workgroups then fit a CU)
   T* sS2 = sRow1;
@@ -856,8 +862,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
     sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
     sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
     // the quadrant above the diagonal contributes nothing: its slots stay zero
-    sDgRow[1][tid] = 0.f;
-    sDgCol[0][tid] = 0.f;
+    slot(5, tid) = 0.f;
+    slot(6, tid) = 0.f;
   }
   {
     // rows beyond L: identity
@@ -935,7 +941,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
         dvst[t][r4] = o;
       }
     part += __shfl_xor(part, 32, 64);
-    if (lane < 32) sDbP[cw][jrow] = part;
+    if (lane < 32) slot(cw, jrow) = part;
   }
   __syncthreads();  // the value tiles and Au^T are consumed
   // ================= key side: d(kb)_1 = Aw^T dw ; dAw_1 = (dw k^T) diag(beta)
@@ -989,12 +995,12 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
         float rs = x;
 #pragma unroll
         for (int off = 16; off > 0; off >>= 1) rs += __shfl_xor(rs, off, 64);
-        if ((lane & 31) == 0) sDgRow[jb][i] = rs;
+        if ((lane & 31) == 0) slot(4 + jb, i) = rs;
         colsum += x;
       }
     }
     colsum += __shfl_xor(colsum, 32, 64);
-    if (lane < 32) sDgCol[ib][j] = -colsum;
+    if (lane < 32) slot(6 + ib, j) = -colsum;
   } else {
     // quadrant (0,1) lies strictly above the diagonal
     for (int e = lane; e < 32 * 32; e += 64) sS1[(e >> 5) * LDT + 32 + (e & 31)] = (T)0.f;
@@ -1075,12 +1081,12 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
         *(v4*)&sRow2[jrow * LDD + col] = o;
       }
     part += __shfl_xor(part, 32, 64);
-    if (lane < 32) sDbP[2 + cw][jrow] = part;
+    if (lane < 32) slot(2 + cw, jrow) = part;
   }
   __syncthreads();  // every wave is past its last read of X1^T / dM^T, which share storage with the dv tile
   if (tid < L) {
-    p.dbeta[(row0 + tid) * H + hh] = (sDbP[0][tid] + sDbP[1][tid]) + (sDbP[2][tid] + sDbP[3][tid]);
-    p.dgam2[(row0 + tid) * H + hh] = (sDgRow[0][tid] + sDgRow[1][tid]) + (sDgCol[0][tid] + sDgCol[1][tid]);
+    p.dbeta[(row0 + tid) * H + hh] = (slot(0, tid) + slot(1, tid)) + (slot(2, tid) + slot(3, tid));
+    p.dgam2[(row0 + tid) * H + hh] = (slot(4, tid) + slot(5, tid)) + (slot(6, tid) + slot(7, tid));
   }
 #pragma unroll
   for (int t = 0; t < TV; ++t)
