@@ -131,6 +131,66 @@ inline int copy_or_zero(const float* src, float* dst, int64_t n, hipStream_t st)
   return FLA_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Operand fragments of the 16x16x32 MFMA for the one-pass forward kernels, whose accumulators go
+// straight back into MFMA operands.
+// ---------------------------------------------------------------------------
+// Measured on gfx950 (one wave per SIMD): LDS reads peak at
+// 256 B/clk per CU, writes near 80 B/clk.  For the access shape of an MFMA operand
+// fragment (16 consecutive rows x 4 column groups per wave) the full read rate is reached
+// by 8-byte reads whose groups are 8 bytes apart and whose row pitch is 16 bytes past a
+// multiple of 256 (or 144 bytes); the same bytes fetched as one 16-byte read, or as a
+// paired two-address read, run at half that rate.  A fragment is therefore two separate
+// 8-byte reads (volatile, so that they are not fused into a paired read): accumulator rows
+// {4g..4g+3} and {16+4g..16+4g+3} of a 32-slice, the order in which stacked 16x16
+// accumulators fed straight back as the other operand enumerate their rows.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag16(const T* tile, int ld, int row0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + (row0 + (lane & 15)) * ld + k0 + 4 * (lane >> 4);
+  v4 lo = *(lds_v4*)p;
+  v4 hi = *(lds_v4*)(p + 16);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Time-contiguous tiles ([row][t], pitch LDT = 144 bytes) are written by lanes that own
+// four adjacent rows each, i.e. with a row stride of four between neighbouring lanes
+// (64 bytes modulo 256: unswizzled, such writes run 5x slower); XOR-ing row bits 4-5
+// into the 16-byte slot index spreads them over all banks.  A fragment read covers the 16
+// rows of one 16-row tile and sees a lane-uniform term.
+FLA_DEVICE int swz_t(int row, int t) { return t ^ ((row >> 1) & 24); }
+
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag16_t(const T* tile, int row0, int t0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  const int row = row0 + (lane & 15), t = t0 + 4 * (lane >> 4);
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + row * LDT;
+  v4 lo = *(lds_v4*)(p + swz_t(row, t));
+  v4 hi = *(lds_v4*)(p + swz_t(row, t + 16));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// A lower-triangular 64x64 tile stored as its ten 16x16 blocks on and below the diagonal, block (i, j) at
+// index i (i + 1) / 2 + j, each block row-major.
+constexpr int kTriElems = 10 * 256;
+
+// A operand (16 rows x 32 contraction indices in accumulator-row order) of row tile tt, column pair s,
+// from a packed triangular tile: block (tt, 2s) gives the first four indices of each group, block
+// (tt, 2s + 1) the second four; above the diagonal that block is not stored and reads as zero.  A
+// block is 512 contiguous bytes and the 64 lanes read each of its 8-byte pieces once.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag_tri(const T* tile, int tt, int s, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef __attribute__((address_space(3))) const volatile v4 lds_v4;
+  const T* p = tile + (tt * (tt + 1) / 2 + 2 * s) * 256 + (lane & 15) * 16 + 4 * (lane >> 4);
+  v4 lo = *(lds_v4*)p;
+  v4 hi = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  if (2 * s + 1 <= tt) hi = *(lds_v4*)(p + 256);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 // Largest exponent handed to exp() where a decay is inverted (e^{-G}); keeps the operand finite in
 // 16-bit storage.  bf16 has fp32's exponent range; fp16 ends at 65504 (e^{11}), so fp16 chunks leave the
 // single-reference arithmetic much earlier (e^{8} |k| stays representable for |k| up to 20).

@@ -329,8 +329,6 @@ struct PrepParams {
 };
 
 constexpr int kPrepWorkgroups = 3 * 256;        // three resident workgroups (register budget) on each of the 256 CUs
-constexpr int kTriBlocks = 10;                   // 16x16 blocks on and below the diagonal of a 64x64 tile
-constexpr int kTriElems = kTriBlocks * 256;      // elements of one packed triangular tile
 FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 
 // A workgroup walks several (chunk, head) items (grid-stride) and loads the q, k rows, beta and the gate

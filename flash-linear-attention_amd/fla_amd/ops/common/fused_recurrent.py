@@ -144,17 +144,21 @@ class FusedRecurrentFunction(torch.autograd.Function):
     @autocast_custom_fwd
     def forward(ctx, q, k, v, g=None, gk=None, gv=None, scale=None, initial_state=None,
                 output_final_state=False, reverse=False, offsets=None, head_first=True, inplace_state=False):
-        needs_grad = any(t is not None and t.requires_grad for t in (q, k, v, g, gk, gv, initial_state))
+        # ctx.needs_input_grad, not the tensors' own flags: the wrapper above may have handed over contiguous
+        # copies made under no_grad
+        nig = ctx.needs_input_grad
+        needs_grad = any(nig[:6]) or nig[7]
         if needs_grad and inplace_state:
             raise ValueError("inplace_state=True overwrites the initial state the backward needs")
-        gates_grad = any(t is not None and t.requires_grad for t in (g, gk, gv))
+        gates_grad = any(nig[3:6])
+        gv_grad = gv is not None and nig[5]
         # the gate gradients read the unrounded output (gv) and the final state (a gradient of the final state)
         o, ht = fused_recurrent_fwd(q, k, v, g, gk, gv, scale, initial_state, output_final_state or gates_grad,
                                     reverse, offsets, head_first, inplace_state,
-                                    o_dtype=torch.float32 if (gv is not None and gv.requires_grad) else None)
+                                    o_dtype=torch.float32 if gv_grad else None)
         if needs_grad:
             ctx.save_for_backward(q, k, v, g, gk, gv, initial_state, offsets,
-                                  o if gv is not None and gv.requires_grad else None, ht if gates_grad else None)
+                                  o if gv_grad else None, ht if gates_grad else None)
             ctx.scale, ctx.reverse, ctx.head_first = scale, reverse, head_first
         return o.to(q.dtype), (ht if output_final_state else None)
 

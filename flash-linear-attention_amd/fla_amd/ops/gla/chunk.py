@@ -385,10 +385,8 @@ class ChunkGLAFunction(torch.autograd.Function):
         in_dtypes = (q.dtype, k.dtype, v.dtype, g.dtype)
         if head_first:
             q, k, v, g = (x.transpose(1, 2).contiguous() for x in (q, k, v, g))
-        if q.dtype == torch.float32:
-            warnings.warn("fla_amd chunk_gla: fp32 q/k/v are rounded to bf16 for the MFMA kernels "
-                          "(state and gates stay fp32)", stacklevel=3)
-            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        if q.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"fla_amd chunk_gla kernels: q must be bf16 or fp16, got {q.dtype}")
         k, v = k.to(q.dtype), v.to(q.dtype)
         if g.dtype not in (torch.float32, q.dtype):
             g = g.float()
@@ -448,6 +446,36 @@ class ChunkGLAFunction(torch.autograd.Function):
         return dq.to(qd), dk.to(kd), dv.to(vd), dg.to(gd), None, dh0, None, None, None
 
 
+def _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first):
+    """fp32 q/k/v (the reference runs and tests the operator in fp32, ``tests/ops/test_gla.py:29-87``): the
+    chunk kernels multiply 16-bit operands, so fp32 callers are served by the token-by-token kernels, which
+    evaluate the same recurrence in fp32 forward and backward (slower - serial in time - but to fp32
+    accuracy).  Key dims above 256 and value dims that are not multiples of 4 are split / padded."""
+    from ..common.fused_recurrent import fused_recurrent
+    K, V = q.shape[-1], v.shape[-1]
+    if K > 256:
+        o_sum, states = None, []
+        for k0 in range(0, K, 256):
+            ks = slice(k0, k0 + 256)
+            h0 = None if initial_state is None else initial_state[..., ks, :]
+            o, ht = _chunk_gla_fp32(q[..., ks], k[..., ks], v, g[..., ks], scale, h0, output_final_state, offsets,
+                                    head_first)
+            o_sum = o if o_sum is None else o_sum + o
+            states.append(ht)
+        return o_sum, (torch.cat(states, dim=-2) if output_final_state else None)
+    Vp = -(-V // 4) * 4
+    h0 = initial_state
+    if Vp != V:
+        v = F.pad(v, (0, Vp - V))
+        h0 = None if h0 is None else F.pad(h0, (0, Vp - V))
+    o, ht = fused_recurrent(q, k.float(), v.float(), gk=g.float(), scale=scale, initial_state=h0,
+                            output_final_state=output_final_state, offsets=offsets, head_first=head_first)
+    if Vp != V:
+        o = o[..., :V]
+        ht = None if ht is None else ht[..., :V]
+    return o, ht
+
+
 def chunk_gla(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -480,6 +508,8 @@ def chunk_gla(
         scale = q.shape[-1] ** -0.5
     if q.numel() == 0:
         return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
+    if q.dtype == torch.float32:
+        return _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
     K, V = q.shape[-1], v.shape[-1]
     if K > 128:
         # every key channel carries its own row of the state and o sums over them: wider key heads

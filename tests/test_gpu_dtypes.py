@@ -127,3 +127,45 @@ def test_chunk_gla_fp16_strong_gates(device):
     assert_close("ht", rht, ht, 5e-3)
     for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
         assert_close(name, a.grad, b.grad, 2e-2)
+
+
+@pytest.mark.parametrize("T,D,head_first,varlen", [(130, 64, False, False), (300, 100, True, False), (200, 128, False, True),
+                                                   (64, 300, False, False)])
+def test_chunk_gla_fp32_inputs(device, T, D, head_first, varlen):
+    """fp32 q, k, v (tests/ops/test_gla.py:29-87 and :149-201 run the operator in fp32): forward and backward
+    to fp32 accuracy, rel-L2 <= 1e-4, against the fp32 naive recurrence - no rounding of the inputs to 16 bits."""
+    import torch.nn.functional as F
+    from fla_amd.ops.gla import chunk_gla
+    from helpers import assert_close
+    from oracle.recurrent import naive_recurrent_gla
+    B, H = (1, 2) if varlen else (2, 2)
+    N = 3 if varlen else B
+    gen = torch.Generator().manual_seed(T + D)
+    q, k, v = (torch.randn(B, T, H, D, generator=gen) for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, T, H, D, generator=gen)) / 4
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    do = torch.randn(B, T, H, D, generator=gen)
+    dht = torch.randn(N, H, D, D, generator=gen) * 0.1
+    offs = torch.tensor([0, 17, 90, T]) if varlen else None
+    print(f"chunk_gla fp32 T={T} D={D} head_first={head_first} varlen={varlen}", flush=True)
+    tr = (lambda x: x.transpose(1, 2).contiguous()) if head_first else (lambda x: x)
+    leaves = [tr(x).to(device).requires_grad_() for x in (q, k, v, g)]
+    h0l = h0.to(device).requires_grad_()
+    import warnings
+    with warnings.catch_warnings(record=True) as record:
+        warnings.simplefilter("always")
+        o, ht = chunk_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=head_first,
+                          offsets=None if offs is None else offs.to(device))
+    assert not [w for w in record if "rounded" in str(w.message)]
+    assert o.dtype == torch.float32 and ht.dtype == torch.float32
+    ((o * tr(do).to(device)).sum() + (ht * dht.to(device)).sum()).backward()
+    rl = [x.clone().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gla(*rl, initial_state=rh0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    ((ro * do).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, tr(o) if head_first else o, 1e-4)
+    assert_close("ht", rht, ht, 1e-4)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
+        assert_close(name, a.grad, tr(b.grad) if head_first else b.grad, 2e-4)
+    assert_close("dh0", rh0.grad, h0l.grad, 1e-4)

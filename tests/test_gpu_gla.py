@@ -214,6 +214,37 @@ def test_chunk_gla_extreme_gates_mixed_varlen(device):
     assert_close("ht", rht, ht, TOL_HT)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_gla_many_heads(device, dtype, varlen):
+    """More than 128 (sequence, head) pairs at K = V = 128: the forward without kept states runs one
+    workgroup per head over all 128 value columns.  Ragged lengths, an initial state, and a stretch of
+    gates strong enough to send some chunks through the exact pairwise path."""
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(73)
+    if varlen:
+        T, N, H = 1100, 9, 16
+        offs = random_offsets(T, N, gen, min_len=1)
+        q, k, v, g, h0 = gla_inputs(1, T, H, 128, 128, seed=73, N=N, normalizer=16.0)
+    else:
+        T, N, H = 203, 5, 32
+        offs = None
+        q, k, v, g, h0 = gla_inputs(N, T, H, 128, 128, seed=74, normalizer=16.0)
+    g[:, 70:140, 3:7, :9] *= 40.0 if dtype == torch.float16 else 400.0
+    q, k, v = (x.to(dtype).float() for x in (q, k, v))
+    print(f"chunk_gla {N * H} heads {dtype} offs={None if offs is None else offs.tolist()}", flush=True)
+    from fla_amd.ops.gla import chunk_gla
+    dev = lambda x: None if x is None else x.to(device)
+    o, ht = chunk_gla(dev(q).to(dtype), dev(k).to(dtype), dev(v).to(dtype), dev(g), initial_state=dev(h0),
+                      output_final_state=True, offsets=dev(offs), head_first=False)
+    torch.cuda.synchronize()
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    assert o.dtype == dtype
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+
+
 @pytest.mark.parametrize("normalizer", [0.05, 0.3])
 def test_chunk_gla_backward_extreme_gates(device, normalizer):
     """Backward with gates far outside the single-reference range (the reference sweeps
