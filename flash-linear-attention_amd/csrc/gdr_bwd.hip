@@ -1109,6 +1109,61 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   }
 }
 
+#define FLA_KV(STMT)                                   \
+  if (K == 64 && V == 64) { STMT(64, 64) }             \
+  else if (K == 128 && V == 128) { STMT(128, 128) }    \
+  else if (K == 64 && V == 128) { STMT(64, 128) }      \
+  else if (K == 128 && V == 64) { STMT(128, 64) }      \
+  else if (K == 256 && V == 64) { STMT(256, 64) }      \
+  else if (K == 256 && V == 128) { STMT(256, 128) }    \
+  else return FLA_E_UNSUPPORTED;
+
+template <typename T>
+int launch_dv_local(const DvlParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
+#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+  FLA_KV(L1)
+#undef L1
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+// reverse state scan: one workgroup per (sequence, head, 32 value columns)
+template <typename T>
+int launch_dhu(const DhuParams& p, int64_t K, hipStream_t st) {
+  const int64_t total = (int64_t)(p.V / 32) * p.N * p.H;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  if (total == 0) return FLA_OK;
+  if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(256), 0, st, p);
+  else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(256), 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(256), 0, st, p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+// one workgroup per (chunk, head, 64 key channels)
+template <typename T>
+int launch_dqkwg(const DqkwgParams& p, int64_t V, dim3 grid, hipStream_t st) {
+  const int64_t nwg = (int64_t)grid.x * grid.y * (p.K / 64);
+  FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  dim3 g3((unsigned)nwg);
+  if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p);
+  else if (V == 128) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+template <typename T>
+int launch_wy_bwd(const WyBwdParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
+#define L4(KK, VV) hipLaunchKernelGGL((gdr_bwd_wy_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+  FLA_KV(L4)
+#undef L4
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+#undef FLA_KV
+
 template <typename T>
 int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, const void* vnew, const float* beta,
                    const float* gam, const void* Aw, const void* dout, const float* dht, const void* hT, void* dvl,
@@ -1121,67 +1176,15 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
-#define FLA_KV(STMT)                                   \
-  if (K == 64 && V == 64) { STMT(64, 64) }             \
-  else if (K == 128 && V == 128) { STMT(128, 128) }    \
-  else if (K == 64 && V == 128) { STMT(64, 128) }      \
-  else if (K == 128 && V == 64) { STMT(128, 64) }      \
-  else if (K == 256 && V == 64) { STMT(256, 64) }      \
-  else if (K == 256 && V == 128) { STMT(256, 128) }    \
-  else return FLA_E_UNSUPPORTED;
-  {
-    DvlParams p{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
-#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
-    FLA_KV(L1)
-#undef L1
-    FLA_CHECK_LAUNCH();
-  }
-  {
-    DhuParams p{q, k, w, dout, dvl, gam, dht, dv2, dhtf, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N, scale};
-    int64_t total = (V / 32) * N * H;
-    FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
-    if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(256), 0, st, p);
-    else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(256), 0, st, p);
-    FLA_CHECK_LAUNCH();
-  }
-  {
-    DqkwgParams p{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
-                  B * T_, (int)H, (int)K, ntfix, scale};
-    const int64_t nwg = (int64_t)grid.x * grid.y * (K / 64);
-    FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
-    dim3 g3((unsigned)nwg);
-    if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p);
-    FLA_CHECK_LAUNCH();
-  }
-  {
-    WyBwdParams p{k, v, beta, gam, Aw, dw, dv2, dkp, dk, dv, dbeta, dgam2, offsets, indices, T_, (int)H, ntfix};
-#define L4(KK, VV) hipLaunchKernelGGL((gdr_bwd_wy_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
-    FLA_KV(L4)
-#undef L4
-    FLA_CHECK_LAUNCH();
-  }
-#undef FLA_KV
-  return FLA_OK;
-}
-
-template <typename T>
-int launch_dv_local(const DvlParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
-#define FLA_KV(STMT)                                   \
-  if (K == 64 && V == 64) { STMT(64, 64) }             \
-  else if (K == 128 && V == 128) { STMT(128, 128) }    \
-  else if (K == 64 && V == 128) { STMT(64, 128) }      \
-  else if (K == 128 && V == 64) { STMT(128, 64) }      \
-  else if (K == 256 && V == 64) { STMT(256, 64) }      \
-  else if (K == 256 && V == 128) { STMT(256, 128) }    \
-  else return FLA_E_UNSUPPORTED;
-#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
-  FLA_KV(L1)
-#undef L1
-#undef FLA_KV
-  FLA_CHECK_LAUNCH();
-  return FLA_OK;
+  DvlParams p1{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
+  if ((rc = launch_dv_local<T>(p1, K, V, grid, st))) return rc;
+  DhuParams p2{q, k, w, dout, dvl, gam, dht, dv2, dhtf, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N, scale};
+  if ((rc = launch_dhu<T>(p2, K, st))) return rc;
+  DqkwgParams p3{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
+                 B * T_, (int)H, (int)K, ntfix, scale};
+  if ((rc = launch_dqkwg<T>(p3, V, grid, st))) return rc;
+  WyBwdParams p4{k, v, beta, gam, Aw, dw, dv2, dkp, dk, dv, dbeta, dgam2, offsets, indices, T_, (int)H, ntfix};
+  return launch_wy_bwd<T>(p4, K, V, grid, st);
 }
 
 }  // namespace
@@ -1227,5 +1230,70 @@ extern "C" int fla_chunk_gated_delta_rule_bwd(
     return launch_gdr_bwd<f16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, ws_dv_local, ws_dv2,
                                ws_dh_frag_t, ws_dw, ws_dk_partial, ws_dgam_partial, dq, dk, dv, dbeta, dgam2, dh0,
                                offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gated_delta_rule_bwd_dhu(const void* q, const void* k, const void* w, const float* g_cumsum,
+                                                  const float* dht, const void* dout, const void* dv, void* dh_frag_t,
+                                                  void* dv2, float* dh0, const int64_t* offsets,
+                                                  const int64_t* chunk_offsets, int qkv_dtype, int64_t B, int64_t T,
+                                                  int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                                  fla_stream_t stream) {
+  FLA_REQUIRE(q && k && w && dout && dv && dh_frag_t && dv2, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
+  FLA_REQUIRE((K == 64 || K == 128 || K == 256) && V % 32 == 0, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)w | (uintptr_t)dout | (uintptr_t)dv | (uintptr_t)dh_frag_t |
+               (uintptr_t)dv2) % 16 == 0, FLA_E_ALIGNMENT);
+  hipStream_t st = (hipStream_t)stream;
+  if (N == 0 || T == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);
+  DhuParams p{q, k, w, dout, dv, g_cumsum, dht, dv2, dh_frag_t, dh0, offsets, chunk_offsets, T, (int)H, (int)V, (int)N,
+              scale};
+  if (qkv_dtype == FLA_BF16) return launch_dhu<bf16>(p, K, st);
+  if (qkv_dtype == FLA_F16) return launch_dhu<f16>(p, K, st);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_bwd_dqkwg(const void* q, const void* k, const void* v_new, const void* w,
+                                   const float* g_cumsum, const void* h_frag_t, const void* dh_frag_t, const void* dout,
+                                   const void* dv, void* dq, void* dk, void* dw, float* dg_partial,
+                                   const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B,
+                                   int64_t T, int64_t H, int64_t K, int64_t V, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q && k && v_new && w && h_frag_t && dh_frag_t && dout && dv && dq && dk && dw && dg_partial,
+              FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 64 == 0 && (V == 64 || V == 128), FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v_new | (uintptr_t)w | (uintptr_t)h_frag_t |
+               (uintptr_t)dh_frag_t | (uintptr_t)dout | (uintptr_t)dv | (uintptr_t)dq | (uintptr_t)dk |
+               (uintptr_t)dw) % 16 == 0, FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  DqkwgParams p{q, k, v_new, w, dout, dv, g_cumsum, h_frag_t, dh_frag_t, dq, dk, dw, dg_partial, offsets, indices, T,
+                B * T, (int)H, (int)K, ntfix, scale};
+  if (qkv_dtype == FLA_BF16) return launch_dqkwg<bf16>(p, V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_dqkwg<f16>(p, V, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_bwd_prepare_wy_repr(const void* k, const void* v, const float* beta, const float* g_cumsum,
+                                       const void* Aw, const void* dw, const void* du, const void* dk_in, void* dk,
+                                       void* dv, float* dbeta, float* dg, const int64_t* offsets,
+                                       const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T,
+                                       int64_t H, int64_t K, int64_t V, fla_stream_t stream) {
+  FLA_REQUIRE(k && v && beta && Aw && dw && du && dk && dv && dbeta && dg, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)Aw | (uintptr_t)dw | (uintptr_t)du | (uintptr_t)dk_in |
+               (uintptr_t)dk | (uintptr_t)dv) % 16 == 0, FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  WyBwdParams p{k, v, beta, g_cumsum, Aw, dw, du, dk_in, dk, dv, dbeta, dg, offsets, indices, T, (int)H, ntfix};
+  if (qkv_dtype == FLA_BF16) return launch_wy_bwd<bf16>(p, K, V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_wy_bwd<f16>(p, K, V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
 }

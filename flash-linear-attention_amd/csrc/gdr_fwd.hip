@@ -40,6 +40,8 @@ struct WyParams {
   const int64_t* indices;
   int64_t T;
   int H, NTfix;
+  const void* Aw_in;   // both given: w = Aw_in (beta k), u = Au_in (beta v) on these matrices, nothing is inverted
+  const void* Au_in;
 };
 
 // out^T tile = X^T-tile A^T for a lower-triangular 16-bit A [64 x 64] in LDS and
@@ -223,6 +225,24 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
     sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
     sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
   }
+  if (p.Aw_in) {
+    // the two matrices as the caller kept them ([rows, H, 64], lower triangular): masked copies to LDS
+    const int i = tid >> 2, j0 = (tid & 3) * 16;
+    v8 aw[2], au[2];
+#pragma unroll
+    for (int h8 = 0; h8 < 2; ++h8) {
+      const int64_t off = ((row0 + (i < L ? i : L - 1)) * H + hh) * (int64_t)BT + j0 + 8 * h8;
+      aw[h8] = *(const v8*)((const T*)p.Aw_in + off);
+      au[h8] = *(const v8*)((const T*)p.Au_in + off);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (i >= L || j0 + 8 * h8 + e > i) aw[h8][e] = au[h8][e] = (T)0.f;
+    }
+    *(v8*)&sAw[i * LDT + j0] = aw[0];
+    *(v8*)&sAw[i * LDT + j0 + 8] = aw[1];
+    *(v8*)&sAu[i * LDT + j0] = au[0];
+    *(v8*)&sAu[i * LDT + j0 + 8] = au[1];
+  } else {
 #pragma unroll
   for (int i = 0; i < RPT; ++i) *(v4*)&sK[(rg * RPT + i) * LDK + c4] = kreg[i];
   __syncthreads();
@@ -282,6 +302,7 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
         *(v8*)((T*)p.Au + off + 8) = au[1];
       }
     }
+  }
   }
   __syncthreads();  // X fully consumed: its storage becomes (beta k)^T
   f32x16 accw[K / 64], accu[V / 64];
@@ -1136,7 +1157,26 @@ extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, c
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, offsets, indices, T, (int)H, ntfix};
+  WyParams p{k, v, beta, g_cumsum, w, u, Aw, Au, offsets, indices, T, (int)H, ntfix, nullptr, nullptr};
+  if (qkv_dtype == FLA_BF16) return launch_wy<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  if (qkv_dtype == FLA_F16) return launch_wy<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
+  return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_fwd_recompute_w_u(const void* k, const void* v, const float* beta, const void* Aw, const void* Au,
+                                     void* w, void* u, const int64_t* offsets, const int64_t* indices, int64_t NT,
+                                     int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                     fla_stream_t stream) {
+  FLA_REQUIRE(k && v && beta && Aw && Au && w && u, FLA_E_INVALID);
+  FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  dim3 grid;
+  int ntfix;
+  int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
+  if (rc) return rc;
+  if (grid.x == 0) return FLA_OK;
+  WyParams p{k, v, beta, nullptr, w, u, nullptr, nullptr, offsets, indices, T, (int)H, ntfix, Aw, Au};
   if (qkv_dtype == FLA_BF16) return launch_wy<bf16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_wy<f16>(p, (int)K, (int)V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

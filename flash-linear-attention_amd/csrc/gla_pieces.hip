@@ -392,6 +392,31 @@ __global__ __launch_bounds__(256) void states_to_fragments_kernel(const void* sr
   *(v8*)(d + 8) = hi;
 }
 
+// The inverse: fragment order (16-bit) back to row-major, 16-bit or fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void fragments_to_states_kernel(const T* src, void* dst, int dst_is_f32, int K, int V,
+                                                                  int transposed, int64_t total_tiles) {
+  typedef typename Elem<T>::v8 v8;
+  const int lane = threadIdx.x & 63;
+  const int64_t tile = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile >= total_tiles) return;
+  const int nkt = K / 32, nvt = V / 32;
+  const int64_t state = tile / (nkt * nvt);
+  const int t = (int)(tile % (nkt * nvt)), kt = t / nvt, vt = t % nvt;
+  const int64_t blk = state * (int64_t)K * V;
+  const T* s = src + blk + ((transposed ? (int64_t)vt * nkt + kt : (int64_t)kt * nvt + vt) * 64 + lane) * 16;
+  const v8 lo = *(const v8*)s, hi = *(const v8*)(s + 8);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int kk = kt * 32 + (transposed ? (lane & 31) : c32_row(r, lane));
+    const int vv = vt * 32 + (transposed ? c32_row(r, lane) : (lane & 31));
+    const int64_t idx = blk + (int64_t)kk * V + vv;
+    const T x = r < 8 ? lo[r] : hi[r - 8];
+    if (dst_is_f32) ((float*)dst)[idx] = (float)x;
+    else ((T*)dst)[idx] = x;
+  }
+}
+
 
 template <typename T, bool DV>
 int launch_piece(const PieceParams& p, int K, dim3 grid, hipStream_t stream) {
@@ -527,6 +552,30 @@ extern "C" int fla_states_to_fragments(const void* h_row_major, void* h_frag, in
   else if (dst_dtype == FLA_F16)
     states_to_fragments_kernel<f16><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
         h_row_major, src_is_f32, (f16*)h_frag, (int)K, (int)V, transposed, tiles);
+  else return FLA_E_UNSUPPORTED;
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+extern "C" int fla_fragments_to_states(const void* h_frag, void* h_row_major, int src_dtype, int dst_dtype,
+                                       int transposed, int64_t n_states, int64_t K, int64_t V, fla_stream_t stream) {
+  FLA_REQUIRE(h_row_major && h_frag && h_row_major != h_frag, FLA_E_INVALID);
+  FLA_REQUIRE(n_states >= 0 && K > 0 && V > 0, FLA_E_INVALID);
+  FLA_REQUIRE(K % 32 == 0 && V % 32 == 0, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE((uintptr_t)h_frag % 16 == 0, FLA_E_ALIGNMENT);
+  int dst_is_f32;
+  int rc = is_f32_code(dst_dtype, src_dtype, &dst_is_f32);
+  if (rc) return rc;
+  const int64_t tiles = n_states * (K / 32) * (V / 32);
+  if (tiles == 0) return FLA_OK;
+  const int64_t blocks = (tiles + 3) / 4;
+  FLA_REQUIRE(blocks <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  if (src_dtype == FLA_BF16)
+    fragments_to_states_kernel<bf16><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
+        (const bf16*)h_frag, h_row_major, dst_is_f32, (int)K, (int)V, transposed, tiles);
+  else if (src_dtype == FLA_F16)
+    fragments_to_states_kernel<f16><<<dim3((unsigned)blocks), 256, 0, (hipStream_t)stream>>>(
+        (const f16*)h_frag, h_row_major, dst_is_f32, (int)K, (int)V, transposed, tiles);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;

@@ -60,6 +60,11 @@ SIGNATURES = {
     "fla_states_to_fragments": (c_int, [P, P, I, I, I, I64, I64, I64, P]),
     "fla_chunk_bwd_dv_local": (c_int, [P] * 7 + [I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 26 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gated_delta_rule_bwd_dhu": (c_int, [P] * 12 + [I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_bwd_dqkwg": (c_int, [P] * 15 + [I64, I, I64, I64, I64, I64, I64, F, P]),
+    "fla_bwd_prepare_wy_repr": (c_int, [P] * 14 + [I64, I, I64, I64, I64, I64, I64, P]),
+    "fla_fwd_recompute_w_u": (c_int, [P] * 9 + [I64, I, I64, I64, I64, I64, I64, P]),
+    "fla_fragments_to_states": (c_int, [P, P, I, I, I, I64, I64, I64, P]),
     "fla_l2norm_fwd": (c_int, [P, P, I64, I64, F, I, I, P]),
     "fla_l2norm_bwd": (c_int, [P, P, P, I64, I64, F, I, I, P]),
     "fla_norm_swish_gate_workgroups": (c_int, [I64, I64]),

@@ -1,5 +1,6 @@
 """``chunk_gated_delta_rule_fwd_h`` (``fla/ops/common/chunk_delta_h.py:248-320``),
-served by ``fla_chunk_gated_delta_rule_fwd_h``."""
+served by ``fla_chunk_gated_delta_rule_fwd_h``, and ``chunk_gated_delta_rule_bwd_dhu`` (``:323-391``),
+served by ``fla_chunk_gated_delta_rule_bwd_dhu``."""
 from typing import Optional, Tuple
 
 import torch
@@ -142,3 +143,61 @@ def chunk_gated_delta_rule_fwd_scan(
         be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale),
         be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan")
     return o, ht
+
+
+def chunk_gated_delta_rule_bwd_dhu(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    w: torch.Tensor,
+    g: Optional[torch.Tensor],
+    h0: Optional[torch.Tensor],
+    dht: Optional[torch.Tensor],
+    do: torch.Tensor,
+    dv: torch.Tensor,
+    scale: float,
+    offsets: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+    chunk_size: int = 64,
+    *,
+    fragment_layout: bool = False,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
+    """Reverse state scan of the delta rule's backward (``fla/ops/common/chunk_delta_h.py:323-391``):
+    returns ``(dh, dh0, dv2)`` with ``dh`` ``[B, NT, H, K, V]`` (``[B, H, NT, K, V]`` if ``head_first``) in the
+    q/k dtype, the gradient w.r.t. the state leaving every chunk; ``g`` is the chunk-local cumsum ``[B,T,H]``.
+    ``fragment_layout=True`` leaves ``dh`` in the transposed-fragment order the next stage reads."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_bwd_dhu: chunk size is fixed to 64")
+    if head_first:
+        q, k, w, do, dv = (x.transpose(1, 2) for x in (q, k, w, do, dv))
+        g = None if g is None else g.transpose(1, 2)
+    be.require_gpu(q, k, w, do, dv)
+    q, k, w, do, dv = (x.contiguous() for x in (q, k, w, do, dv))
+    B, T, H, K = q.shape
+    V = do.shape[-1]
+    if K not in (64, 128, 256) or V % 32:
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_bwd_dhu: K in {64,128,256}, V a multiple of 32")
+    if any(x.dtype != q.dtype for x in (k, w, do, dv)) or q.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_bwd_dhu: q, k, w, do, dv all bf16 or all fp16")
+    g = None if g is None else g.float().contiguous()
+    co, N, NT = None, B, -(-T // BT)
+    if offsets is not None:
+        offsets = offsets.to(torch.int64).contiguous()
+        co = prepare_chunk_offsets(offsets, BT).to(torch.int64).contiguous()
+        N = offsets.numel() - 1
+        NT = int(co[-1])
+    dh = q.new_empty(B, NT, H, K, V)
+    dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if h0 is not None else None
+    dv2 = torch.empty_like(dv)
+    dht = None if dht is None else dht.float().contiguous()
+    be.check(be.lib().fla_chunk_gated_delta_rule_bwd_dhu(
+        be.ptr(q), be.ptr(k), be.ptr(w), be.ptr(g), be.ptr(dht), be.ptr(do), be.ptr(dv), be.ptr(dh), be.ptr(dv2),
+        be.ptr(dh0), be.ptr(offsets), be.ptr(co), be.dt(q), B, T, H, K, V, N, float(scale), be.stream_of(q)),
+        "fla_chunk_gated_delta_rule_bwd_dhu")
+    if not fragment_layout:
+        from .chunk_o import fragments_to_states
+        dh = fragments_to_states(dh, q.dtype, transposed=True)
+        if head_first:
+            dh = dh.transpose(1, 2).contiguous()
+    if head_first:
+        dv2 = dv2.transpose(1, 2).contiguous()
+    return dh, dh0, dv2

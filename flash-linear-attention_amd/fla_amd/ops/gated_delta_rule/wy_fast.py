@@ -1,5 +1,6 @@
-"""WY representation of the gated delta rule
-(``fla/ops/gated_delta_rule/wy_fast.py:320-426``), served by ``fla_gdr_fwd_wy``."""
+"""WY representation of the gated delta rule (``fla/ops/gated_delta_rule/wy_fast.py:320-426``), served by
+``fla_gdr_fwd_wy``; ``fwd_recompute_w_u`` (``:320-371``) and ``bwd_prepare_wy_repr`` (``:565-625``) on the
+reference's operands, served by ``fla_fwd_recompute_w_u`` and ``fla_bwd_prepare_wy_repr``."""
 from typing import Optional, Tuple
 
 import torch
@@ -95,3 +96,97 @@ def unpack_triangular_tiles(AT: torch.Tensor) -> torch.Tensor:
         for j in range(i + 1):
             out[..., 16 * i:16 * i + 16, 16 * j:16 * j + 16] = AT[..., i * (i + 1) // 2 + j, :, :]
     return out
+
+
+def _chunk_tables(offsets, indices):
+    if offsets is None:
+        return None, None, 0
+    if indices is None:
+        from ...utils import VarlenPlan
+        indices = VarlenPlan(offsets, BT).indices
+    indices = indices.to(torch.int64).contiguous()
+    return offsets.to(torch.int64).contiguous(), indices, indices.shape[0]
+
+
+def fwd_recompute_w_u(
+    k: torch.Tensor,
+    v: torch.Tensor,
+    beta: torch.Tensor,
+    Aw: torch.Tensor,
+    Au: torch.Tensor,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+    chunk_size: int = 64,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``w = Aw (beta k)``, ``u = Au (beta v)`` per chunk on matrices the caller kept
+    (``fla/ops/gated_delta_rule/wy_fast.py:320-371``); ``Aw`` / ``Au`` ``[B,T,H,64]`` lower triangular."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd fwd_recompute_w_u: chunk size is fixed to 64")
+    if head_first:
+        k, v, beta, Aw, Au = (x.transpose(1, 2) for x in (k, v, beta, Aw, Au))
+    be.require_gpu(k, v, beta, Aw, Au)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    if K not in (64, 128, 256) or V not in (64, 128):
+        raise NotImplementedError("fla_amd fwd_recompute_w_u: K in {64,128,256}, V in {64,128}")
+    if k.dtype not in (torch.bfloat16, torch.float16) or v.dtype != k.dtype:
+        raise NotImplementedError("fla_amd fwd_recompute_w_u: k and v both bf16 or both fp16")
+    k, v = k.contiguous(), v.contiguous()
+    Aw, Au = Aw.to(k.dtype).contiguous(), Au.to(k.dtype).contiguous()
+    beta = beta.float().contiguous()
+    offsets, indices, NT = _chunk_tables(offsets, indices)
+    w, u = torch.empty_like(k), torch.empty_like(v)
+    be.check(be.lib().fla_fwd_recompute_w_u(
+        be.ptr(k), be.ptr(v), be.ptr(beta), be.ptr(Aw), be.ptr(Au), be.ptr(w), be.ptr(u), be.ptr(offsets),
+        be.ptr(indices), NT, be.dt(k), B, T, H, K, V, be.stream_of(k)), "fla_fwd_recompute_w_u")
+    if head_first:
+        w, u = w.transpose(1, 2).contiguous(), u.transpose(1, 2).contiguous()
+    return w, u
+
+
+def bwd_prepare_wy_repr(
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: Optional[torch.Tensor],
+    beta: torch.Tensor,
+    Aw: torch.Tensor,
+    Au: Optional[torch.Tensor],
+    dw: torch.Tensor,
+    du: torch.Tensor,
+    offsets: Optional[torch.Tensor] = None,
+    indices: Optional[torch.Tensor] = None,
+    head_first: bool = True,
+    chunk_size: int = 64,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(dk, dv, dbeta, dg)`` through ``w = Aw (beta k)``, ``u = Au (beta v)``
+    (``fla/ops/gated_delta_rule/wy_fast.py:565-625``); ``g`` the chunk-local cumsum, ``dbeta`` / ``dg`` fp32.
+    ``Au`` is not read: it equals ``Aw * exp(g_i - g_j)`` and is rebuilt from ``Aw`` and ``g``."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd bwd_prepare_wy_repr: chunk size is fixed to 64")
+    if head_first:
+        k, v, beta, Aw, dw, du = (x.transpose(1, 2) for x in (k, v, beta, Aw, dw, du))
+        g = None if g is None else g.transpose(1, 2)
+    be.require_gpu(k, v, beta, Aw, dw, du)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    if K not in (64, 128, 256) or V not in (64, 128):
+        raise NotImplementedError("fla_amd bwd_prepare_wy_repr: K in {64,128,256}, V in {64,128}")
+    if k.dtype not in (torch.bfloat16, torch.float16) or v.dtype != k.dtype:
+        raise NotImplementedError("fla_amd bwd_prepare_wy_repr: k and v both bf16 or both fp16")
+    k, v = k.contiguous(), v.contiguous()
+    Aw, dw, du = Aw.to(k.dtype).contiguous(), dw.to(k.dtype).contiguous(), du.to(k.dtype).contiguous()
+    beta = beta.float().contiguous()
+    g = None if g is None else g.float().contiguous()
+    offsets, indices, NT = _chunk_tables(offsets, indices)
+    dk, dv = torch.empty_like(k), torch.empty_like(v)
+    dbeta = k.new_empty(B, T, H, dtype=torch.float32)
+    dg = k.new_empty(B, T, H, dtype=torch.float32)
+    be.check(be.lib().fla_bwd_prepare_wy_repr(
+        be.ptr(k), be.ptr(v), be.ptr(beta), be.ptr(g), be.ptr(Aw), be.ptr(dw), be.ptr(du), None, be.ptr(dk),
+        be.ptr(dv), be.ptr(dbeta), be.ptr(dg), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, V,
+        be.stream_of(k)), "fla_bwd_prepare_wy_repr")
+    if head_first:
+        dk, dv = dk.transpose(1, 2).contiguous(), dv.transpose(1, 2).contiguous()
+        dbeta, dg = dbeta.transpose(1, 2).contiguous(), dg.transpose(1, 2).contiguous()
+    return dk, dv, dbeta, dg

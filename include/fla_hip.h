@@ -424,6 +424,54 @@ int fla_chunk_gated_delta_rule_bwd(
     const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
+/* The launches of fla_chunk_gated_delta_rule_bwd one by one, for callers that hold the reference's own
+ * intermediates (the sibling operators that call these stages directly).  States cross this boundary in
+ * FLA_H_FRAGMENT_T order; fla_states_to_fragments / fla_fragments_to_states convert from and to the
+ * reference's row-major [.., K, V].  16-bit q/k/v dtype throughout, g_cumsum fp32 [B,T,H] or NULL.
+ *
+ * fla_chunk_gated_delta_rule_bwd_dhu replaces chunk_gated_delta_rule_bwd_dhu
+ * (fla/ops/common/chunk_delta_h.py:323-391, kernel :136-237): reverse scan over the chunks of a sequence,
+ *   dh[c] = dH;  dv2 = dv + (k e^{g_last-g}) dH;  dH <- e^{g_last} dH + (scale q e^g)^T do - (w e^g)^T dv2,
+ * from dH = dht.  dv is the intra-chunk part (fla_chunk_bwd_dv_local), dv2 [B,T,H,V] the sum, dh_frag_t the
+ * gradient w.r.t. the state leaving every chunk, dh0 fp32 [N,H,K,V] or NULL.  K in {64,128,256}, V % 32 == 0.
+ *
+ * fla_chunk_bwd_dqkwg replaces chunk_bwd_dqkwg (fla/ops/common/chunk_o.py:602-661, kernel :118-265) in the
+ * form the delta rule calls it (w and dv given): dq, dk (without the WY path), dw in the q/k dtype and
+ * dg_partial fp32 [K/64, B*T, H], whose sum over the first dim is the reference's dg (before the reverse
+ * cumulative sum).  v_new is the delta rule's corrected value, dv the dv2 of the scan above.  K % 64 == 0,
+ * V in {64,128}.
+ *
+ * fla_bwd_prepare_wy_repr replaces bwd_prepare_wy_repr (fla/ops/gated_delta_rule/wy_fast.py:565-625, kernel
+ * :440-562): the gradient through w = Aw (beta k), u = Au (beta v) with Au = Aw * e^{g_i-g_j}.  Aw
+ * [B,T,H,64]; dw like k, du like v.  Outputs dk (+ dk_in, a partial dk in the k dtype that is added before the
+ * single rounding; may be NULL), dv, dbeta and dg fp32 [B,T,H].  K in {64,128,256}, V in {64,128}.
+ *
+ * fla_fwd_recompute_w_u replaces fwd_recompute_w_u (fla/ops/gated_delta_rule/wy_fast.py:320-371, kernel
+ * :250-317): w = Aw (beta k), u = Au (beta v) on matrices the caller kept ([B,T,H,64], lower triangular).
+ *
+ * fla_fragments_to_states: the inverse of fla_states_to_fragments (16-bit fragments to 16-bit or fp32
+ * row-major states). */
+int fla_chunk_gated_delta_rule_bwd_dhu(const void* q, const void* k, const void* w, const float* g_cumsum,
+                                       const float* dht, const void* dout, const void* dv, void* dh_frag_t,
+                                       void* dv2, float* dh0, const int64_t* offsets,
+                                       const int64_t* chunk_offsets, int qkv_dtype, int64_t B, int64_t T,
+                                       int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                       fla_stream_t stream);
+int fla_chunk_bwd_dqkwg(const void* q, const void* k, const void* v_new, const void* w, const float* g_cumsum,
+                        const void* h_frag_t, const void* dh_frag_t, const void* dout, const void* dv, void* dq,
+                        void* dk, void* dw, float* dg_partial, const int64_t* offsets, const int64_t* indices,
+                        int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                        float scale, fla_stream_t stream);
+int fla_bwd_prepare_wy_repr(const void* k, const void* v, const float* beta, const float* g_cumsum, const void* Aw,
+                            const void* dw, const void* du, const void* dk_in, void* dk, void* dv, float* dbeta,
+                            float* dg, const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                            int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, fla_stream_t stream);
+int fla_fwd_recompute_w_u(const void* k, const void* v, const float* beta, const void* Aw, const void* Au, void* w,
+                          void* u, const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                          int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, fla_stream_t stream);
+int fla_fragments_to_states(const void* h_frag, void* h_row_major, int src_dtype, int dst_dtype, int transposed,
+                            int64_t n_states, int64_t K, int64_t V, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Row-wise steps either side of the chunk operators inside the layers
  * (fla/layers/gated_deltanet.py:234-235, fla/layers/gla.py:203-218).

@@ -33,6 +33,12 @@ per-head-gate operators (``fla/ops/common/chunk_o.py:379-441``).  They are pinne
 by the recurrence (output stage on ``chunked_gla``'s intermediates) and by autograd through the
 chunk step (dA, dv, dh) in ``tests/test_oracle_pins.py``.
 
+The ``gdr_*`` / ``chunk_bwd_dqkwg`` / ``chunk_bwd_dv`` / ``*_wy_repr`` functions after them restate the stages of
+the delta rule's backward on the reference's operands (``fla/ops/gated_delta_rule/chunk.py:76-177`` for the
+order; ``fla/ops/common/chunk_delta_h.py:136-237``, ``chunk_o.py:118-265,294-375``,
+``gated_delta_rule/wy_fast.py:250-317,440-562`` for the stages).  Pinned by autograd through one chunk step and
+through the WY map, and by their composition against autograd through the naive recurrence.
+
 Test infrastructure only.
 """
 from typing import Dict, Optional, Sequence
@@ -259,3 +265,135 @@ def chunk_bwd_dv_local(q, k, g_cumsum, do, scale, chunk_size=64, offsets=None, d
             A = A * torch.where(x <= 0, x.exp(), torch.zeros_like(x))                 # safe_exp (fla/ops/utils/exp.py:9-10)
         dv[b, s:e] = torch.einsum('hji,ihv->jhv', torch.triu(A), do[b, s:e])
     return dv
+
+
+def _gates_of(g_cumsum, b, s, e, H, dtype):
+    """(gamma [L,H], Gamma [H,L,L] lower triangular) of one chunk; zeros / ones without a gate."""
+    L = e - s
+    gc = torch.zeros(L, H, dtype=dtype) if g_cumsum is None else g_cumsum[b, s:e].to(dtype)
+    lower = torch.tril(torch.ones(L, L, dtype=dtype))
+    Gam = ((gc[:, None] - gc[None, :]).permute(2, 0, 1) * lower).exp() * lower
+    return gc, Gam
+
+
+def fwd_recompute_w_u(k, v, beta, Aw, Au, chunk_size=64, offsets=None, dtype=torch.float32):
+    """w = Aw (beta k), u = Au (beta v) per chunk; Aw, Au [B,T,H,BT]
+    (fla/ops/gated_delta_rule/wy_fast.py:250-317)."""
+    k, v, beta, Aw, Au = (x.to(dtype) for x in (k, v, beta, Aw, Au))
+    B, T, H, _ = k.shape
+    w, u = torch.zeros_like(k), torch.zeros_like(v)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        L = e - s
+        w[b, s:e] = torch.einsum('ihj,jhk->ihk', Aw[b, s:e, :, :L], k[b, s:e] * beta[b, s:e, :, None])
+        u[b, s:e] = torch.einsum('ihj,jhv->ihv', Au[b, s:e, :, :L], v[b, s:e] * beta[b, s:e, :, None])
+    return w, u
+
+
+def chunk_bwd_dv(q, k, g_cumsum, do, dh, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """dv_j = sum_{i>=j} s (k_j . q_i) e^{g_i-g_j} do_i + (k_j e^{g_last-g_j})^T dh_c
+    (fla/ops/common/chunk_o.py:294-375)."""
+    dv = chunk_bwd_dv_local(q, k, g_cumsum, do, scale, chunk_size, offsets, dtype)
+    k, dh = k.to(dtype), dh.to(dtype)
+    B, T, H, _ = k.shape
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        gc, _ = _gates_of(g_cumsum, b, s, e, H, dtype)
+        kd = k[b, s:e] * (gc[-1][None] - gc).exp()[..., None]
+        dv[b, s:e] += torch.einsum('jhk,hkv->jhv', kd, _state_of(dh, c, B, offsets))
+    return dv
+
+
+def gdr_bwd_dhu(q, k, w, g_cumsum, dht, do, dv, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """For c = last .. 0:  dh[c] = dH;  dv2 = dv + (k e^{g_last-g}) dH;
+    dH = e^{g_last} dH + (s q e^g)^T do - (w e^g)^T dv2, from dH = dht.  Returns (dh, dh0, dv2)
+    (fla/ops/common/chunk_delta_h.py:136-237)."""
+    q, k, w, do, dv = (x.to(dtype) for x in (q, k, w, do, dv))
+    B, T, H, K = q.shape
+    V = do.shape[-1]
+    dv2 = torch.zeros_like(dv)
+    out, dh0 = [], []
+    for n, (b, bos, eos) in enumerate(_spans(B, T, offsets)):
+        dH = torch.zeros(H, K, V, dtype=dtype) if dht is None else dht[n].to(dtype).clone()
+        seq = []
+        for s, e in reversed(_chunks(bos, eos, chunk_size)):
+            seq.append(dH)
+            gc, _ = _gates_of(g_cumsum, b, s, e, H, dtype)
+            eg = gc.exp()[..., None]
+            kd = k[b, s:e] * (gc[-1][None] - gc).exp()[..., None]
+            d2 = dv[b, s:e] + torch.einsum('jhk,hkv->jhv', kd, dH)
+            dv2[b, s:e] = d2
+            dH = (dH * gc[-1].exp()[:, None, None]
+                  + torch.einsum('thk,thv->hkv', scale * q[b, s:e] * eg, do[b, s:e])
+                  - torch.einsum('thk,thv->hkv', w[b, s:e] * eg, d2))
+        out.extend(reversed(seq))
+        dh0.append(dH)
+    if offsets is None:
+        NT = -(-T // chunk_size)
+        dh = torch.stack(out, 0).reshape(B, NT, H, K, V) if out else torch.zeros(B, 0, H, K, V, dtype=dtype)
+    else:
+        dh = torch.stack(out, 0)[None]
+    return dh, torch.stack(dh0, 0), dv2
+
+
+def chunk_bwd_dqkwg(q, k, v, g_cumsum, do, h, dh, dv, w, scale, chunk_size=64, offsets=None, dtype=torch.float32):
+    """Per chunk, with ds = s tril((do v^T) * Gamma):
+      dq = s e^g (do h^T) + ds k;   dk = e^{g_last-g} (v dh^T) + ds^T q;   dw = -e^g (dv h^T);
+      dg_i = sum_k (q dq - k dk + w dw)_ik + [i last] (sum_jk (k * dk_inter)_jk + e^{g_last} <h, dh>)
+    (fla/ops/common/chunk_o.py:118-265; the reference forms the intra-chunk part of dg from ds * (q k^T), whose
+    row minus column sums equal sum_k q dq_intra - k dk_intra).  v is v_new for the delta rule; dv / w None
+    for the operators without a correction term.  Returns (dq, dk, dw, dg), dg w.r.t. the cumulative gate."""
+    q, k, v, do, h, dh = (x.to(dtype) for x in (q, k, v, do, h, dh))
+    B, T, H, K = k.shape
+    dq, dk = torch.zeros_like(q), torch.zeros_like(k)
+    dw = None if w is None else torch.zeros_like(k)
+    dg = torch.zeros(B, T, H, dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        gc, Gam = _gates_of(g_cumsum, b, s, e, H, dtype)
+        eg = gc.exp()[..., None]
+        ed = (gc[-1][None] - gc).exp()[..., None]
+        hc, dhc = _state_of(h, c, B, offsets), _state_of(dh, c, B, offsets)
+        qc, kc, vc, doc = q[b, s:e], k[b, s:e], v[b, s:e], do[b, s:e]
+        ds = scale * torch.einsum('ihv,jhv->hij', doc, vc) * Gam
+        dqc = scale * eg * torch.einsum('ihv,hkv->ihk', doc, hc) + torch.einsum('hij,jhk->ihk', ds, kc)
+        dk_inter = ed * torch.einsum('jhv,hkv->jhk', vc, dhc)
+        dkc = dk_inter + torch.einsum('hij,ihk->jhk', ds, qc)
+        row = (qc * dqc - kc * dkc).sum(-1)
+        if w is not None:
+            dwc = -eg * torch.einsum('ihv,hkv->ihk', dv[b, s:e].to(dtype), hc)
+            dw[b, s:e] = dwc
+            row = row + (w[b, s:e].to(dtype) * dwc).sum(-1)
+        row[-1] += (kc * dk_inter).sum((0, 2)) + gc[-1].exp() * (hc * dhc).sum((1, 2))
+        dq[b, s:e], dk[b, s:e], dg[b, s:e] = dqc, dkc, row
+    return dq, dk, dw, (None if g_cumsum is None else dg)
+
+
+def bwd_prepare_wy_repr(k, v, g_cumsum, beta, Aw, dw, du, chunk_size=64, offsets=None, dtype=torch.float32):
+    """Gradient through w = Aw kb, u = Au vb with kb = beta k, vb = beta v, M = strict_lower(kb k^T),
+    Aw = (I + M)^-1, Au = Aw * Gamma:
+      d(kb) = Aw^T dw, d(vb) = Au^T du, dAw = strict_lower(dw kb^T) + strict_lower(du vb^T) * Gamma,
+      dM = -strict_lower(Aw^T dAw Aw^T), d(kb) += dM k, dk = beta d(kb) + dM^T kb, dv = beta d(vb),
+      dbeta = sum d(kb) k + sum d(vb) v, dg_i = rowsum_i(X) - colsum_i(X), X = strict_lower(du vb^T) * Au
+    (fla/ops/gated_delta_rule/wy_fast.py:440-562, there with both inverses as inputs).  Returns (dk, dv, dbeta, dg)."""
+    k, v, beta, Aw, dw, du = (x.to(dtype) for x in (k, v, beta, Aw, dw, du))
+    B, T, H, _ = k.shape
+    dk, dv = torch.zeros_like(k), torch.zeros_like(v)
+    dbeta, dg = torch.zeros(B, T, H, dtype=dtype), torch.zeros(B, T, H, dtype=dtype)
+    for c, b, s, e in _chunk_list(B, T, chunk_size, offsets):
+        L = e - s
+        gc, Gam = _gates_of(g_cumsum, b, s, e, H, dtype)
+        strict = torch.tril(torch.ones(L, L, dtype=dtype), -1)
+        aw = torch.tril(Aw[b, s:e, :, :L].permute(1, 0, 2))                    # [H, i, j]
+        au = aw * Gam
+        kc, vc, bc = k[b, s:e], v[b, s:e], beta[b, s:e]
+        kb, vb = kc * bc[..., None], vc * bc[..., None]
+        dkb = torch.einsum('hij,ihk->jhk', aw, dw[b, s:e])
+        dvb = torch.einsum('hij,ihv->jhv', au, du[b, s:e])
+        X0 = torch.einsum('ihv,jhv->hij', du[b, s:e], vb) * strict
+        dAw = torch.einsum('ihk,jhk->hij', dw[b, s:e], kb) * strict + X0 * Gam
+        dM = -(aw.transpose(1, 2) @ dAw @ aw.transpose(1, 2)) * strict
+        dkb = dkb + torch.einsum('hij,jhk->ihk', dM, kc)
+        dk[b, s:e] = bc[..., None] * dkb + torch.einsum('hij,ihk->jhk', dM, kb)
+        dv[b, s:e] = bc[..., None] * dvb
+        dbeta[b, s:e] = (dkb * kc).sum(-1) + (dvb * vc).sum(-1)
+        X = X0 * au
+        dg[b, s:e] = (X.sum(2) - X.sum(1)).t()
+    return dk, dv, dbeta, dg

@@ -394,3 +394,189 @@ def test_chunk_bwd_dv_local_matches_autograd_of_the_intra_chunk_output(offsets, 
     gv, = torch.autograd.grad(loss, [v])
     got = chunked.chunk_bwd_dv_local(q, k, g, do, scale, offsets=offsets, dtype=D)
     torch.testing.assert_close(got, gv, rtol=1e-10, atol=1e-10)
+
+
+# ---------------------------------------------------------------- stages of the delta rule's backward
+def _gdr_chunks(B, T, offsets):
+    return [(n, b, s, min(s + 64, eos)) for n, (b, bos, eos) in enumerate(recurrent._spans(B, T, offsets))
+            for s in range(bos, eos, 64)]
+
+
+def _local_cumsum64(x, B, T, offsets, reverse=False):
+    out = torch.zeros_like(x)
+    for _, b, s, e in _gdr_chunks(B, T, offsets):
+        blk = x[b, s:e]
+        out[b, s:e] = blk.flip(0).cumsum(0).flip(0) if reverse else blk.cumsum(0)
+    return out
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+@pytest.mark.parametrize("gated", [True, False])
+def test_gdr_backward_stages_match_autograd_through_the_chunk_step(offsets, gated):
+    """With q, k, w, u and the cumulative gate as independent leaves, the chunk step
+      v_new = u - (w e^g) h,  o = s (e^g (q h) + tril(q k^T * Gamma) v_new),  h_next = e^{g_last} h + (k e^{g_last-g})^T v_new
+    chained over the chunks has, for  sum(do * o) + sum(dht * ht):  d/du = dv2 and d/d(state leaving a chunk) = dh
+    (reverse scan), d/dq, d/dk, d/dw, d/dg = the outputs of chunk_bwd_dqkwg, d/dh0 = dh0."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q, k, w = (_rand(B, T, H, K, seed=s).requires_grad_() for s in (51, 52, 53))
+    u = _rand(B, T, H, V, seed=54).requires_grad_()
+    G = None
+    if gated:
+        G = _local_cumsum64(F.logsigmoid(_rand(B, T, H, seed=55)), B, T, offsets).requires_grad_()
+    do, dht = _rand(B, T, H, V, seed=56), _rand(N, H, K, V, seed=57)
+    h0 = (0.3 * _rand(N, H, K, V, seed=58)).requires_grad_()
+    scale = 0.33
+    taps, hs, vns, loss = [], [], torch.zeros(B, T, H, V, dtype=D), 0.
+    h, last_n = None, -1
+    for n, b, s, e in _gdr_chunks(B, T, offsets):
+        if n != last_n:
+            if last_n >= 0:
+                loss = loss + (dht[last_n] * h).sum()
+            h, last_n = h0[n], n
+        L = e - s
+        gc = torch.zeros(L, H, dtype=D) if G is None else G[b, s:e]
+        lower = torch.tril(torch.ones(L, L, dtype=D))
+        Gam = ((gc[:, None] - gc[None, :]).permute(2, 0, 1) * lower).exp() * lower
+        eg = gc.exp()[..., None]
+        hs.append(h.detach())
+        vn = u[b, s:e] - torch.einsum('ihk,hkv->ihv', w[b, s:e] * eg, h)
+        vns[b, s:e] = vn.detach()
+        P = torch.einsum('ihk,jhk->hij', q[b, s:e], k[b, s:e]) * Gam
+        o = scale * (eg * torch.einsum('ihk,hkv->ihv', q[b, s:e], h) + torch.einsum('hij,jhv->ihv', P, vn))
+        loss = loss + (do[b, s:e] * o).sum()
+        tap = torch.zeros(H, K, V, dtype=D, requires_grad=True)
+        taps.append(tap)
+        kd = k[b, s:e] * (gc[-1][None] - gc).exp()[..., None]
+        h = h * gc[-1].exp()[:, None, None] + torch.einsum('jhk,jhv->hkv', kd, vn) + tap
+    loss = loss + (dht[last_n] * h).sum()
+    leaves = [q, k, w, u, h0] + ([G] if gated else [])
+    grads = torch.autograd.grad(loss, leaves + taps)
+    gq, gk, gw, gu, gh0 = grads[:5]
+    gtaps = torch.stack(grads[len(leaves):], 0)
+    states = torch.stack(hs, 0)
+    states = states.reshape(B, -1, H, K, V) if offsets is None else states[None]
+    Gd = None if G is None else G.detach()
+    qd, kd_, wd = q.detach(), k.detach(), w.detach()
+    dvl = chunked.chunk_bwd_dv_local(qd, kd_, Gd, do, scale, offsets=offsets, dtype=D)
+    dh, dh0, dv2 = chunked.gdr_bwd_dhu(qd, kd_, wd, Gd, dht, do, dvl, scale, offsets=offsets, dtype=D)
+    dq, dk, dw, dg = chunked.chunk_bwd_dqkwg(qd, kd_, vns, Gd, do, states, dh, dv2, wd, scale, offsets=offsets, dtype=D)
+    tol = dict(rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(dv2, gu, **tol)
+    torch.testing.assert_close(dh.reshape(-1, H, K, V), gtaps, **tol)
+    torch.testing.assert_close(dh0, gh0, **tol)
+    torch.testing.assert_close(dq, gq, **tol)
+    torch.testing.assert_close(dk, gk, **tol)
+    torch.testing.assert_close(dw, gw, **tol)
+    if gated:
+        torch.testing.assert_close(dg, grads[5], **tol)
+    else:
+        assert dg is None
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_bwd_prepare_wy_repr_matches_autograd_through_the_wy_map(offsets):
+    """(dk, dv, dbeta, dg) are the gradients of  sum(dw * w) + sum(du * u)  with w = (I + M)^-1 (beta k),
+    u = (I + M * Gamma)^-1 (beta v), M = strict_lower(diag(beta) k k^T), both inverses by triangular solves."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    k = F.normalize(_rand(B, T, H, K, seed=61), dim=-1).requires_grad_()
+    v = _rand(B, T, H, V, seed=62).requires_grad_()
+    beta = torch.rand(B, T, H, dtype=D, generator=torch.Generator().manual_seed(63)).requires_grad_()
+    G = _local_cumsum64(F.logsigmoid(_rand(B, T, H, seed=64)), B, T, offsets).requires_grad_()
+    dw, du = _rand(B, T, H, K, seed=65), _rand(B, T, H, V, seed=66)
+    Aw = torch.zeros(B, T, H, 64, dtype=D)
+    Au = torch.zeros(B, T, H, 64, dtype=D)
+    loss = 0.
+    for _, b, s, e in _gdr_chunks(B, T, offsets):
+        L = e - s
+        gc = G[b, s:e]
+        eye = torch.eye(L, dtype=D)
+        strict, lower = torch.tril(torch.ones(L, L, dtype=D), -1), torch.tril(torch.ones(L, L, dtype=D))
+        kb, vb = k[b, s:e] * beta[b, s:e, :, None], v[b, s:e] * beta[b, s:e, :, None]
+        M = torch.einsum('ihk,jhk->hij', kb, k[b, s:e]) * strict
+        Gam = ((gc[:, None] - gc[None, :]).permute(2, 0, 1) * lower).exp() * lower
+        aw = torch.linalg.solve_triangular(eye + M, eye.expand(H, L, L), upper=False)
+        au = torch.linalg.solve_triangular(eye + M * Gam, eye.expand(H, L, L), upper=False)
+        Aw[b, s:e, :, :L], Au[b, s:e, :, :L] = aw.detach().permute(1, 0, 2), au.detach().permute(1, 0, 2)
+        loss = loss + (dw[b, s:e] * torch.einsum('hij,jhk->ihk', aw, kb)).sum()
+        loss = loss + (du[b, s:e] * torch.einsum('hij,jhv->ihv', au, vb)).sum()
+    gk, gv, gb, gG = torch.autograd.grad(loss, [k, v, beta, G])
+    dk, dv, dbeta, dg = chunked.bwd_prepare_wy_repr(k.detach(), v.detach(), G.detach(), beta.detach(), Aw, dw, du,
+                                                    offsets=offsets, dtype=D)
+    tol = dict(rtol=1e-9, atol=1e-9)
+    torch.testing.assert_close(dk, gk, **tol)
+    torch.testing.assert_close(dv, gv, **tol)
+    torch.testing.assert_close(dbeta, gb, **tol)
+    torch.testing.assert_close(dg, gG, **tol)
+    # the second inverse is the first one rescaled: what lets the stage take Aw alone
+    torch.testing.assert_close(Au, Aw * _gamma_rows(G.detach(), B, T, offsets), **tol)
+
+
+def _gamma_rows(G, B, T, offsets):
+    """e^{g_i - g_j} for j <= i laid out like Aw: [B, T, H, 64], zero elsewhere."""
+    out = torch.zeros(B, T, G.shape[-1], 64, dtype=D)
+    for _, b, s, e in _gdr_chunks(B, T, offsets):
+        L = e - s
+        gc = G[b, s:e]
+        lower = torch.tril(torch.ones(L, L, dtype=D))
+        out[b, s:e, :, :L] = (((gc[:, None] - gc[None, :]) * lower[..., None]).exp() * lower[..., None]).permute(0, 2, 1)
+    return out
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+def test_gdr_backward_stages_compose_to_autograd_through_the_recurrence(offsets):
+    """The reference's order (fla/ops/gated_delta_rule/chunk.py:76-177) on the oracle's stages: recompute w, u and
+    the states, dv_local, reverse scan, dq/dk/dw/dg, WY gradient, dk and dg summed, reverse chunk-local cumsum of dg;
+    against autograd through the token-by-token recurrence."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q = _rand(B, T, H, K, seed=71).requires_grad_()
+    k = F.normalize(_rand(B, T, H, K, seed=72), dim=-1).requires_grad_()
+    v = _rand(B, T, H, V, seed=73).requires_grad_()
+    g = F.logsigmoid(_rand(B, T, H, seed=74)).requires_grad_()
+    beta = torch.rand(B, T, H, dtype=D, generator=torch.Generator().manual_seed(75)).requires_grad_()
+    h0 = (0.3 * _rand(N, H, K, V, seed=76)).requires_grad_()
+    do, dht = _rand(B, T, H, V, seed=77), _rand(N, H, K, V, seed=78)
+    scale = K ** -0.5
+    o, ht = recurrent.naive_recurrent_gated_delta_rule(q, k, v, g, beta, scale=scale, initial_state=h0,
+                                                       output_final_state=True, offsets=offsets, dtype=D)
+    want = torch.autograd.grad((do * o).sum() + (dht * ht).sum(), [q, k, v, g, beta, h0])
+    qd, kd, vd, gd, bd = (x.detach() for x in (q, k, v, g, beta))
+    r = chunked.chunked_gated_delta_rule(qd, kd, vd, gd, bd, scale=scale, initial_state=h0.detach(), offsets=offsets, dtype=D)
+    G = r['g_cumsum']
+    w, u = chunked.fwd_recompute_w_u(kd, vd, bd, r['Aw'], r['Au'], offsets=offsets, dtype=D)
+    torch.testing.assert_close(w, r['w'], rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(u, r['u'], rtol=1e-10, atol=1e-10)
+    dvl = chunked.chunk_bwd_dv_local(qd, kd, G, do, scale, offsets=offsets, dtype=D)
+    dh, dh0, dv2 = chunked.gdr_bwd_dhu(qd, kd, w, G, dht, do, dvl, scale, offsets=offsets, dtype=D)
+    dq, dk, dw, dg = chunked.chunk_bwd_dqkwg(qd, kd, r['v_new'], G, do, r['h'], dh, dv2, w, scale, offsets=offsets, dtype=D)
+    dk2, dv, db, dg2 = chunked.bwd_prepare_wy_repr(kd, vd, G, bd, r['Aw'], dw, dv2, offsets=offsets, dtype=D)
+    dg = _local_cumsum64(dg + dg2, B, T, offsets, reverse=True)
+    tol = dict(rtol=1e-8, atol=1e-8)
+    for name, got, ref in zip("dq dk dv dg dbeta dh0".split(), (dq, dk + dk2, dv, dg, db, dh0), want):
+        torch.testing.assert_close(got, ref, msg=lambda m, name=name: f"{name}: {m}", **tol)
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+@pytest.mark.parametrize("gated", [True, False])
+def test_chunk_bwd_dv_matches_autograd_of_the_scalar_gated_chunk_step(offsets, gated):
+    """dv is the gradient w.r.t. v of  sum(do * o) + sum(dh * h_next)  for  o_i = s sum_{j<=i} (q_i . k_j) e^{g_i-g_j} v_j
+    (+ a term without v)  and  h_next = e^{g_last} h + (k e^{g_last-g})^T v."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    q, k = _rand(B, T, H, K, seed=81), _rand(B, T, H, K, seed=82)
+    v = _rand(B, T, H, V, seed=83).requires_grad_()
+    do = _rand(B, T, H, V, seed=84)
+    g = _local_cumsum64(F.logsigmoid(_rand(B, T, H, seed=85)), B, T, offsets) if gated else None
+    chunks = _gdr_chunks(B, T, offsets)
+    dh = _rand(len(chunks), H, K, V, seed=86)
+    scale, loss = 0.29, 0.
+    for c, (_, b, s, e) in enumerate(chunks):
+        gc = torch.zeros(e - s, H, dtype=D) if g is None else g[b, s:e]
+        A = scale * torch.einsum('ihk,jhk->hij', q[b, s:e], k[b, s:e]) * (gc.t()[:, :, None] - gc.t()[:, None, :]).exp()
+        loss = loss + (do[b, s:e] * torch.einsum('hij,jhv->ihv', torch.tril(A), v[b, s:e])).sum()
+        kd = k[b, s:e] * (gc[-1][None] - gc).exp()[..., None]
+        loss = loss + (dh[c] * torch.einsum('jhk,jhv->hkv', kd, v[b, s:e])).sum()
+    gv, = torch.autograd.grad(loss, [v])
+    states = dh.reshape(B, -1, H, K, V) if offsets is None else dh[None]
+    got = chunked.chunk_bwd_dv(q, k, g, do, states, scale, offsets=offsets, dtype=D)
+    torch.testing.assert_close(got, gv, rtol=1e-10, atol=1e-10)
