@@ -142,11 +142,21 @@ def bench_gla(device, steps, warmup):
     # gla_fwd_fused_kernel followed by the range guard's short second launch; the dominant kernel is
     # timed on its own in the form the operator runs it (guard workspaces given).  The two-kernel
     # pipeline it replaces (state scan + per-chunk output) is timed as well for comparison.
-    from fla_amd.ops.gla.chunk import chunk_gla_fwd_fused
     scale = K ** -0.5
 
+    # pointers and workspaces bound once: the host side of a launch is then a few microseconds, the launches
+    # queue up behind each other and an event interval holds device time only
+    from fla_amd import _backend as be
+    from fla_amd.ops.gla.chunk import _guard_workspaces
+    o_buf, ht_buf = torch.empty_like(v), q.new_empty(B, H, K, V, dtype=torch.float32)
+    wide, hwide = _guard_workspaces(q, B * (T // 64), H, K * V, keep=False)
+    fused_args = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o_buf), be.ptr(ht_buf), be.ptr(wide),
+                  be.ptr(hwide), None, None, None, None, 0, be.dt(q), be.dt(g), B, T, H, K, V, B, float(scale),
+                  be.stream_of(q))
+    first_launch = be.lib().fla_chunk_gla_fwd_fused_first_launch
+
     def run_fused():
-        chunk_gla_fwd_fused(q, k, v, g, scale, h0, True, first_launch_only=True)
+        be.check(first_launch(*fused_args), "fla_chunk_gla_fwd_fused_first_launch")
 
     h_hold = {}
 
