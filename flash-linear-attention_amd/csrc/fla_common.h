@@ -53,6 +53,14 @@ struct Elem<bf16> {
   static FLA_DEVICE f32x4 mfma16(v8 a, v8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
+  // c + sum of the eight products, on the packed dot-product instruction (no unpacked temporaries)
+  static FLA_DEVICE float dot8(v8 a, v8 b, float c) {
+    typedef bf16 v2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c = __builtin_amdgcn_fdot2_f32_bf16(v2{a[2 * i], a[2 * i + 1]}, v2{b[2 * i], b[2 * i + 1]}, c, false);
+    return c;
+  }
 };
 
 template <>
@@ -64,6 +72,13 @@ struct Elem<f16> {
   }
   static FLA_DEVICE f32x4 mfma16(v8 a, v8 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static FLA_DEVICE float dot8(v8 a, v8 b, float c) {
+    typedef f16 v2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c = __builtin_amdgcn_fdot2(v2{a[2 * i], a[2 * i + 1]}, v2{b[2 * i], b[2 * i + 1]}, c, false);
+    return c;
   }
 };
 

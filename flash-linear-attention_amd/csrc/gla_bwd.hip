@@ -5,16 +5,18 @@
 // LEAVING chunk c (fla/ops/gla/chunk.py:1217-1320, fla/ops/common/chunk_h.py:156-271):
 //
 //   gla_bwd_dh_kernel    reverse state scan:  store dH_c;  dH <- diag(e^{G_last}) dH + q~^T do.
-//                        The tile is kept in both orientations ([K,V] and [V,K]) and both are
-//                        stored in MFMA-fragment order, because dv contracts dH over K and dk
-//                        over V.  Also emits sum_v h_c * dH_c per key channel (for dg) from the
-//                        recomputed forward states, and dh0.
-//   gla_bwd_dv_kernel    per (chunk, head):  dv = A^T do + k^ dH_c.
+//                        The tile is kept and stored transposed ([V,K], MFMA-fragment order), the
+//                        orientation dk contracts it in; also emits dh0.
+//   gla_bwd_dv_kernel    per (chunk, head):  dv = A^T do + k^ dH_c.  dv contracts dH over K: the
+//                        stored [V,K] fragments are turned round on the matrix pipe (a product with a
+//                        permuted identity is a transposition of the accumulator layout, exact for
+//                        16-bit values).
 //   gla_bwd_dqkg_kernel  per (chunk, head, 64-wide half of K):
 //                          dA = tril(do v^T)
 //                          dq = s e^{G}  * (dA (k e^{-G}) + do h_c^T)
 //                          dk = s e^{-G} * (dA^T (q e^{G})) + e^{G_last-G} * (v dH_c^T)
 //                          dg = reverse-cumsum(q*dq - k*dk) + sum_t k*dk_inter + e^{G_last} sum_v h_c*dH_c
+//                          (the last sum from the h_c and dH_c fragments the kernel holds anyway)
 //                        (fla/ops/gla/chunk.py:409-567 intra, :726-837 inter incl. the dg formula
 //                        :818-823).  As in the forward, one reference point per chunk replaces
 //                        the 16x16 sub-block scheme.
@@ -29,10 +31,7 @@ struct BDhParams {
   const void* g;
   const void* dout;
   const float* dht;
-  const void* hT;     // forward states, FLA_H_FRAGMENT_T
-  void* dhf;          // out: dH, FLA_H_FRAGMENT
   void* dhtf;         // out: dH, FLA_H_FRAGMENT_T
-  float* hdh;         // out: [V/32][chunks][H][K] partial sums of h*dH over 32 value columns
   float* dh0;         // out: fp32 [N,H,K,V] or null
   const int64_t* offsets;
   const int64_t* chunk_offsets;
@@ -72,22 +71,17 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
   const int kq = wave & 1, vq = wave >> 1;
   const int kt32 = kbase / 32 + kq, vt32 = vbase / 32 + vq;
   const int vcol = vbase + vq * 32 + (lane & 31), kcol = kbase + kq * 32 + (lane & 31);
-  f32x16 acc1 = zero16();  // rows k, cols v
   f32x16 acc2 = zero16();  // rows v, cols k
   if (p.dht) {
     const float* dp0 = p.dht + (int64_t)nh * K * V;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      acc1[r] = dp0[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol];
-      acc2[r] = dp0[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)];
-    }
+    for (int r = 0; r < 16; ++r) acc2[r] = dp0[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)];
   }
 
   struct Regs {
     g2 g[8];
     t2 q[8];
     t2 d[8];
-    v8 h[2];
   };
   auto chunk_len = [&](int64_t c) {
     int64_t rem = sp.len - c * BT;
@@ -111,10 +105,6 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       R.q[i] = *(const t2*)(qb + (ok < limk ? ok : limk));
       R.d[i] = *(const t2*)(db + (ov < limv ? ov : limv));
     }
-    const T* hp = (const T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V +
-                  (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
-    R.h[0] = *(const v8*)hp;
-    R.h[1] = *(const v8*)(hp + 8);
   };
 
   // One barrier per chunk, operand tiles double-buffered in LDS.  Two register sets, each
@@ -123,18 +113,10 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
   auto step = [&](int64_t c, Regs& R, auto more) {
     const int buf = (int)(c & 1);
     const int L = chunk_len(c);
-    // ---- gradient w.r.t. the state leaving chunk c, both orientations, fragment order
+    // ---- gradient w.r.t. the state leaving chunk c, transposed fragment order
     {
       int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
       v8 lo, hi;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        lo[r] = (T)acc1[r];
-        hi[r] = (T)acc1[r + 8];
-      }
-      T* o1 = (T*)p.dhf + blk + (((int64_t)kt32 * (V / 32) + vt32) * 64 + lane) * 16;
-      *(v8*)o1 = lo;
-      *(v8*)(o1 + 8) = hi;
 #pragma unroll
       for (int r = 0; r < 8; ++r) {
         lo[r] = (T)acc2[r];
@@ -143,12 +125,6 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       T* o2 = (T*)p.dhtf + blk + (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
       *(v8*)o2 = lo;
       *(v8*)(o2 + 8) = hi;
-      // sum over this wave's 32 value columns of h_c * dH_c, one key channel per lane
-      float part = 0.f;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) part += (float)R.h[0][r] * acc2[r] + (float)R.h[1][r] * acc2[r + 8];
-      part += __shfl_xor(part, 32, 64);
-      if (lane < 32) p.hdh[(((int64_t)vt32 * p.total_chunks + chunk0 + c) * H + hh) * K + kcol] = part;
     }
     // ---- chunk-local prefix sums of the gates
     float G[8][2], glast0, glast1;
@@ -201,12 +177,6 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
       asm volatile("" ::: "memory");  // the loads stay here, ahead of the barrier
     }
     lds_barrier();
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      f32x4 d = *(const f32x4*)&sDecay[buf][kq * 32 + 8 * a + 4 * (lane >> 5)];
-#pragma unroll
-      for (int b = 0; b < 4; ++b) acc1[4 * a + b] *= d[b];
-    }
     {
       const float d = sDecay[buf][kq * 32 + (lane & 31)];
 #pragma unroll
@@ -216,7 +186,6 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
     for (int s = 0; s < BT; s += 16) {
       v8 fq = lds_frag32<T>(sQt[buf], LDT, kq * 32, s, lane);
       v8 fd = lds_frag32<T>(sDt[buf], LDT, vq * 32, s, lane);
-      acc1 = Elem<T>::mfma32(fq, fd, acc1);
       acc2 = Elem<T>::mfma32(fd, fq, acc2);
     }
   };
@@ -244,7 +213,9 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
   if (p.dh0) {
     float* o = p.dh0 + (int64_t)nh * K * V;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[(int64_t)(kbase + kq * 32 + c32_row(r, lane)) * V + vcol] = acc1[r];
+    for (int r4 = 0; r4 < 4; ++r4)
+      *(f32x4*)&o[(int64_t)kcol * V + vbase + vq * 32 + 8 * r4 + 4 * (lane >> 5)] =
+          f32x4{acc2[4 * r4], acc2[4 * r4 + 1], acc2[4 * r4 + 2], acc2[4 * r4 + 3]};
   }
 }
 
@@ -254,7 +225,7 @@ struct BDvParams {
   const void* k;
   const void* g;
   const void* dout;
-  const void* dhf;
+  const void* dhtf;  // dH, FLA_H_FRAGMENT_T
   const int* wide;   // [chunks, H] or null: chunks whose intra-chunk part is left to the exact kernel
   void* dv;
   const int64_t* offsets;
@@ -313,14 +284,15 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     else dreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
   }
   const int rw = wave >> 1, cw = wave & 1;
+  // dH tiles as stored: rows v, columns k (a lane holds one key column)
   v8 hf[KT32][TV][2];
   {
-    const T* hp = (const T*)p.dhf + (cl.cglob * H + hh) * (int64_t)K * V;
+    const T* hp = (const T*)p.dhtf + (cl.cglob * H + hh) * (int64_t)K * V;
 #pragma unroll
     for (int kt = 0; kt < KT32; ++kt)
 #pragma unroll
       for (int tv = 0; tv < TV; ++tv) {
-        const T* f = hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16;
+        const T* f = hp + (((int64_t)(cw * TV + tv) * KT32 + kt) * 64 + lane) * 16;
         hf[kt][tv][0] = *(const v8*)f;
         hf[kt][tv][1] = *(const v8*)(f + 8);
       }
@@ -406,14 +378,36 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     for (int tv = 0; tv < TV; ++tv)
       acc[tv] = Elem<T>::mfma32(lds_frag32<T>(sDt, LDT, (cw * TV + tv) * 32, is, lane), a, acc[tv]);
   }
+  // The state term contracts over k, so the tiles are needed with a lane per value column.  A tile in
+  // accumulator order is, read as the first operand, its own transpose (lane = row index of the product,
+  // registers = contraction index in accumulator-row order); multiplied by the identity in the same
+  // permuted order the product comes out in accumulator order with lanes and registers exchanged.
+  v8 eye[2];
 #pragma unroll
-  for (int kt = 0; kt < KT32; ++kt)
+  for (int half = 0; half < 2; ++half)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      eye[half][e] = (T)(((lane & 31) == 16 * half + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) ? 1.f : 0.f);
+#pragma unroll
+  for (int kt = 0; kt < KT32; ++kt) {
+    v8 ht[TV][2];
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv) {
+      f32x16 t = Elem<T>::mfma32(hf[kt][tv][0], eye[0], zero16());
+      t = Elem<T>::mfma32(hf[kt][tv][1], eye[1], t);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ht[tv][0][e] = (T)t[e];
+        ht[tv][1][e] = (T)t[8 + e];
+      }
+    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       v8 a = lds_frag32_perm<T>(sKh, LDK, rw * 32, kt * 32 + half * 16, lane);
 #pragma unroll
-      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(hf[kt][tv][half], a, acc[tv]);
+      for (int tv = 0; tv < TV; ++tv) acc[tv] = Elem<T>::mfma32(ht[tv][half], a, acc[tv]);
     }
+  }
   // the q tile is dead since the score phase: the dv tile goes through it and leaves as whole rows
   T* sO = sQ;
   {
@@ -447,7 +441,6 @@ struct BDqkgParams {
   const void* dout;
   const void* hT;     // forward states, FLA_H_FRAGMENT_T
   const void* dhtf;   // dH, FLA_H_FRAGMENT_T
-  const float* hdh;   // [V/32][chunks][H][K]
   const int* wide;    // [chunks, H] or null: chunks whose intra-chunk part is left to the exact kernel
   void* dq;
   void* dk;
@@ -479,6 +472,7 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   __shared__ __attribute__((aligned(16))) T sdAT[BT * LDT];  // dA^T [j][i]
   __shared__ __attribute__((aligned(16))) float sPart[16 * 64];
   __shared__ __attribute__((aligned(16))) float sPart2[16 * 64];
+  __shared__ float sHd[64];                                   // sum_v h_c * dH_c per key channel of the slice
   T* sDo = (T*)sRA;
   T* sV = (T*)sRB;
   T* sKtT = (T*)sRC;
@@ -645,13 +639,21 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     aq = Elem<T>::mfma32(lds_frag32<T>(sdA, LDT, rw * 32, js, lane), lds_frag32<T>(sKtT, LDT, cw * 32, js, lane), aq);
   for (int is = rw * 32; is < BT; is += 16)
     ak1 = Elem<T>::mfma32(lds_frag32<T>(sdAT, LDT, rw * 32, is, lane), lds_frag32<T>(sQtT, LDT, cw * 32, is, lane), ak1);
+  // sum over the value columns of h_c * dH_c on the way: both sets of fragments hold one key column per
+  // lane, and each pair is dead once its products are issued (the two row-block waves of a column block
+  // hold the same fragments; one of them reports)
+  float hd = 0.f;
 #pragma unroll
   for (int vt = 0; vt < VT32; ++vt)
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       aq = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aq);
       ak2 = Elem<T>::mfma32(lds_frag32_perm<T>(sV, LDV, rw * 32, vt * 32 + half * 16, lane), dhf[vt][half], ak2);
+      hd = Elem<T>::dot8(hf[vt][half], dhf[vt][half], hd);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  hd += __shfl_xor(hd, 32, 64);
+  if (rw == 0 && lane < 32) sHd[cw * 32 + lane] = hd;
   __syncthreads();  // every MFMA operand read is done: the tiles become fp32 staging
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -721,12 +723,7 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     }
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    float hd = 0.f;
-    for (int vt = 0; vt < VT32; ++vt)
-      hd += p.hdh[(((int64_t)vt * p.total_chunks + cl.cglob) * H + hh) * K + kb + c4 + j];
-    add[j] += __expf(glast[j]) * hd;
-  }
+  for (int j = 0; j < 4; ++j) add[j] += __expf(glast[j]) * sHd[c4 + j];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     int row = rg * 4 + i;
@@ -913,7 +910,7 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
 
 template <typename T, typename GT>
 int launch_bwd(const void* q, const void* k, const void* v, const void* g, const void* dout, const float* dht,
-               const void* hT, void* dhf, void* dhtf, float* hdh, void* dq, void* dk, void* dv, float* dg, float* dh0,
+               const void* hT, void* dhtf, void* dq, void* dk, void* dv, float* dg, float* dh0,
                const int* wide,
                const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
                int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
@@ -924,7 +921,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
   const int64_t total_chunks = grid.x;
   {
-    BDhParams p{q, g, dout, dht, hT, dhf, dhtf, hdh, dh0, offsets, chunk_offsets, T_, total_chunks,
+    BDhParams p{q, g, dout, dht, dhtf, dh0, offsets, chunk_offsets, T_, total_chunks,
                 (int)H, (int)K, (int)V, (int)N, scale};
     int64_t total = (K / 64) * (V / 64) * N * H;
     FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
@@ -932,7 +929,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   {
-    BDvParams p{q, k, g, dout, dhf, wide, dv, offsets, indices, T_, (int)H, ntfix, scale};
+    BDvParams p{q, k, g, dout, dhtf, wide, dv, offsets, indices, T_, (int)H, ntfix, scale};
 #define FLA_CASE(KK, VV)                                                                            \
   if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_dv_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
     FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
@@ -940,7 +937,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   {
-    BDqkgParams p{q, k, v, g, dout, hT, dhtf, hdh, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
+    BDqkgParams p{q, k, v, g, dout, hT, dhtf, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
                   (int)H, (int)K, ntfix, scale};
     const int64_t nwg = (int64_t)grid.x * grid.y * (K / 64);
     FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
@@ -966,25 +963,25 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
 }  // namespace
 
 extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
-                                 const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
+                                 const float* dht, const void* hT, void* dh_frag_t,
                                  void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
                                  const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
                                  int64_t NT, int qkv_dtype,
                                  int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                  float scale, fla_stream_t stream) {
-  FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag && dh_frag_t && hdh && dq && dk && dv && dg,
+  FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag_t && dq && dk && dv && dg,
               FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)dout | (uintptr_t)hT |
-               (uintptr_t)dh_frag | (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
+               (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
                (uintptr_t)dg) % 16 == 0,
               FLA_E_ALIGNMENT);
   hipStream_t st = (hipStream_t)stream;
 #define FLA_BWD(TT, GG)                                                                                           \
-  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag, dh_frag_t, hdh, dq, dk, dv, dg, dh0, wide,   \
+  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag_t, dq, dk, dv, dg, dh0, wide,   \
                             offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_BWD(bf16, float);
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_BWD(bf16, bf16);

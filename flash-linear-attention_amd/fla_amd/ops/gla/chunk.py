@@ -332,17 +332,15 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
         hT, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=False,
                             offsets=offs, indices=idx, head_first=False, chunk_size=BT, gates_are_cumsum=False,
                             fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
-    total_chunks = hT.shape[0] * hT.shape[1]
-    dhf, dhtf = torch.empty_like(hT), torch.empty_like(hT)
-    hdh = q.new_empty(V // 32, total_chunks, H, K, dtype=torch.float32)
+    dhtf = torch.empty_like(hT)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dg = q.new_empty(B, T, H, K, dtype=torch.float32)
     dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
     if dht is not None:
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
     be.check(be.lib().fla_chunk_gla_bwd(
-        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(dhf), be.ptr(dhtf),
-        be.ptr(hdh), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(dhtf),
+        be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
         be.ptr(idx), be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_bwd")
     return dq, dk, dv, dg, dh0
 

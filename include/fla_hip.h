@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 2
+#define FLA_ABI_VERSION 3
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -320,10 +320,10 @@ int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void
  * Three launches on `stream`: reverse state scan, dv, dq/dk/dg.
  *   gates   raw log-gates [B,T,H,K] (fp32 or the q/k/v dtype)
  *   dout    gradient of o, [B,T,H,V] in the q/k/v dtype; dht fp32 [N,H,K,V] or NULL
- *   hT      forward states recomputed by fla_chunk_gla_fwd_h with FLA_H_FRAGMENT_T
- *   dh_frag, dh_frag_t   workspaces, each the size of hT (gradient of the
- *           per-chunk states in the two fragment orientations)
- *   hdh     workspace fp32 [V/32, chunks, H, K]
+ *   hT      forward states in FLA_H_FRAGMENT_T order (kept by fla_chunk_gla_fwd_fused_states
+ *           or recomputed by fla_chunk_gla_fwd_h)
+ *   dh_frag_t   workspace the size of hT: the gradient of the per-chunk states,
+ *           FLA_H_FRAGMENT_T order
  *   dq, dk [B,T,H,K] and dv [B,T,H,V] in the q/k/v dtype; dg fp32 [B,T,H,K]
  *   (gradient w.r.t. the raw gates); dh0 fp32 [N,H,K,V] or NULL.
  *   wide    int32 [chunks, H] flags written by fla_chunk_gla_fwd_fused (ws_wide), or
@@ -334,7 +334,7 @@ int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void
  *           fla/ops/gla/chunk.py:409-567).
  * ---------------------------------------------------------------------- */
 int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
-                      const float* dht, const void* hT, void* dh_frag, void* dh_frag_t, float* hdh,
+                      const float* dht, const void* hT, void* dh_frag_t,
                       void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
                       const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                       int qkv_dtype, int gate_dtype,
