@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
 #pragma unroll
     for (int i = 0; i < RPTV; ++i) {
       int row = rgv * RPTV + i;
-      vreg[i] = row < L ? *(const v4*)(vp + (int64_t)row * H * V) : z;
+      vreg[i] = (row < L && p.u) ? *(const v4*)(vp + (int64_t)row * H * V) : z;
     }
   }
   if (tid < BT) {
@@ -310,17 +310,19 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
   __syncthreads();
   wy_apply<T, K>(sAw, sXbT, accw, wave, lane);
   __syncthreads();  // (beta k)^T fully consumed: its storage becomes (beta v)^T
-  wy_stage_t<T, RPTV>(sXbT, vreg, sBeta, rgv * RPTV, cv4);
-  __syncthreads();
-  wy_apply<T, V>(sAu, sXbT, accu, wave, lane);
-  __syncthreads();  // both operand regions are free: they carry the output tiles to whole-row stores
+  if (p.u) {        // u is optional: a forward that forms v_new from the triangular tiles needs w alone
+    wy_stage_t<T, RPTV>(sXbT, vreg, sBeta, rgv * RPTV, cv4);
+    __syncthreads();
+    wy_apply<T, V>(sAu, sXbT, accu, wave, lane);
+    __syncthreads();  // both operand regions are free: they carry the output tiles to whole-row stores
+  }
   T* sWo = (T*)sRA;
   T* sUo = (T*)sRB;
   wy_acc_to_lds<T, K>(sWo, accw, wave, lane);
-  wy_acc_to_lds<T, V>(sUo, accu, wave, lane);
+  if (p.u) wy_acc_to_lds<T, V>(sUo, accu, wave, lane);
   __syncthreads();
   wy_store<T, K>(sWo, (T*)p.w + (row0 * H + hh) * (int64_t)K, (int64_t)H * K, L, tid);
-  wy_store<T, V>(sUo, (T*)p.u + (row0 * H + hh) * (int64_t)V, (int64_t)H * V, L, tid);
+  if (p.u) wy_store<T, V>(sUo, (T*)p.u + (row0 * H + hh) * (int64_t)V, (int64_t)H * V, L, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -1148,7 +1150,7 @@ extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, c
                               void* Aw, void* Au, const int64_t* offsets, const int64_t* indices, int64_t NT,
                               int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                               fla_stream_t stream) {
-  FLA_REQUIRE(k && v && beta && w && u, FLA_E_INVALID);
+  FLA_REQUIRE(k && v && beta && w, FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)k | (uintptr_t)v | (uintptr_t)w | (uintptr_t)u | (uintptr_t)Aw | (uintptr_t)Au) % 16 == 0,
               FLA_E_ALIGNMENT);

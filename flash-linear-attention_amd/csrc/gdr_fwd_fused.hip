@@ -22,6 +22,14 @@
 // Operand tiles are double-buffered and the two groups meet at one barrier per chunk.  The o tile
 // takes the place of the v tile it was computed from (same lanes, same addresses), so it needs no
 // storage of its own.
+// The KEEP instantiation serves a forward pass that will be differentiated: the matrix waves also write
+// v_new and the state entering every chunk (FLA_H_FRAGMENT_T order, what the backward kernels read).  Both
+// sit in registers as MFMA operands with a lane per value column, four consecutive time rows / key rows
+// per register quad; a product with a permuted identity turns them round on the matrix pipe (exact for
+// 16-bit values), after which a lane holds four consecutive value columns of one row; a lane-swap between
+// the halves (state) or neighbouring rows of 16 lanes (v_new) pairs them up into 16-byte stores (a store
+// instruction costs the CU's memory pipeline the same whatever its width, and that pipeline is what bounds
+// the scan).
 #include "chunk_common.h"
 
 namespace {
@@ -38,6 +46,8 @@ struct GdrScanParams {
   const float* h0;
   void* o;
   float* ht;
+  void* v_new;      // KEEP: [rows, H, V]
+  void* h_frag_t;   // KEEP: [chunks, H, K*V], FLA_H_FRAGMENT_T
   const int64_t* offsets;
   const int64_t* chunk_offsets;
   const int64_t* seq_order;  // sequence ids, longest first (or NULL)
@@ -46,7 +56,37 @@ struct GdrScanParams {
   float scale;
 };
 
-template <typename T, int K>
+// Two 4-element results per lane (16-bit after conversion) -> one 8-element vector per lane: lanes 0-31 keep
+// their own a and receive a of lane + 32, lanes 32-63 receive b of lane - 32 and keep their own b.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 pair_halves(f32x4 a, f32x4 b) {
+  typedef typename Elem<T>::v4 v4;
+  typedef typename Elem<T>::v8 v8;
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const u2 ua = __builtin_bit_cast(u2, v4{(T)a[0], (T)a[1], (T)a[2], (T)a[3]});
+  const u2 ub = __builtin_bit_cast(u2, v4{(T)b[0], (T)b[1], (T)b[2], (T)b[3]});
+  const auto lo = __builtin_amdgcn_permlane32_swap(ua[0], ub[0], false, false);
+  const auto hi = __builtin_amdgcn_permlane32_swap(ua[1], ub[1], false, false);
+  return __builtin_bit_cast(v8, u4{lo[0], hi[0], lo[1], hi[1]});
+}
+
+// The same between neighbouring rows of 16 lanes: even rows keep their own a and receive a of lane + 16,
+// odd rows receive b of lane - 16 and keep their own b.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
+  typedef typename Elem<T>::v4 v4;
+  typedef typename Elem<T>::v8 v8;
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const u2 ua = __builtin_bit_cast(u2, v4{(T)a[0], (T)a[1], (T)a[2], (T)a[3]});
+  const u2 ub = __builtin_bit_cast(u2, v4{(T)b[0], (T)b[1], (T)b[2], (T)b[3]});
+  const auto lo = __builtin_amdgcn_permlane16_swap(ua[0], ub[0], false, false);
+  const auto hi = __builtin_amdgcn_permlane16_swap(ua[1], ub[1], false, false);
+  return __builtin_bit_cast(v8, u4{lo[0], hi[0], lo[1], hi[1]});
+}
+
+template <typename T, int K, bool KEEP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
   typedef typename Elem<T>::v8 v8;
@@ -274,6 +314,26 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int r = 0; r < 4; ++r) acc[kt][r] = h0p[(int64_t)(16 * kt + 4 * g + r) * V];
       }
     }
+    // KEEP: the identity in the contraction order of an accumulator pair, one operand per 16-wide half of
+    // a 32-slice, and this lane's places in the two outputs
+    v8 eye[2];
+    // wave-uniform bases (advanced chunk by chunk) and one 32-bit byte offset per lane for each output
+    char* hT_base = nullptr;
+    char* vn_base = nullptr;
+    uint32_t hT_lane = 0, vn_lane = 0;
+    if constexpr (KEEP) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) eye[half][e] = (T)(((e >> 2) == half && 4 * g + (e & 3) == c) ? 1.f : 0.f);
+      // state tile (value block of 32, key block ks): lane (g & 1) * 32 + 16 half + c, slots 4 (2 (wave & 1) + g / 2) ..
+      hT_base = (char*)p.h_frag_t +
+                ((chunk0 * H + hh) * (int64_t)K * V + (int64_t)((vbase + cb) / 32) * (K / 32) * 64 * 16) * (int64_t)sizeof(T);
+      hT_lane = (uint32_t)((((g & 1) * 32 + 16 * (g >> 1) + c) * 16 + 8 * (wave & 1)) * sizeof(T));
+      vn_base = (char*)p.v_new + ((sp.bos * H + hh) * (int64_t)V + vbase + cb) * (int64_t)sizeof(T);
+      vn_lane = (uint32_t)(((16 * (g & 1) + c) * H * V + 8 * (g >> 1)) * sizeof(T));
+    }
+    const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
     if (nchunks > 0) {
       lds_barrier();
       for (int ci = 0; ci < nchunks; ++ci) {
@@ -313,6 +373,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             hb[ks][e] = (T)acc[2 * ks][e];
             hb[ks][4 + e] = (T)acc[2 * ks + 1][e];
           }
+        if constexpr (KEEP) {
+          // the state entering this chunk, transposed tile by tile
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            // lanes 0-31 end up with key row 32 ks + c, lanes 32-63 with 32 ks + 16 + c, eight value columns each
+            const f32x4 t0 = Elem<T>::mfma16(hb[ks], eye[0], zero4());
+            const f32x4 t1 = Elem<T>::mfma16(hb[ks], eye[1], zero4());
+            *(v8*)(hT_base + hT_lane + ks * 64 * 16 * sizeof(T)) = pair_halves<T>(t0, t1);
+          }
+          hT_base += (int64_t)H * K * V * (int64_t)sizeof(T);
+        }
         f32x4 d[4], oq[4];
         auto mm_kq = [&](int tt, const v8* f) {
           d[tt] = zero4();
@@ -413,6 +484,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < KT / 2; ++i)
 #pragma unroll
           for (int s = 0; s < 2; ++s) acc[KT / 2 + i] = Elem<T>::mfma16(fb[2 * i + s], vsb[s], acc[KT / 2 + i]);
+        if constexpr (KEEP) {
+          // v_new of this chunk, turned round the same way (here, where few registers are live)
+          const int Lc = ci == nchunks - 1 ? Llast : BT;
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            // even rows of 16 lanes end up with time row 32 s2 + c, odd ones with 32 s2 + 16 + c
+            const f32x4 t0 = Elem<T>::mfma16(vnb[s2], eye[0], zero4());
+            const f32x4 t1 = Elem<T>::mfma16(vnb[s2], eye[1], zero4());
+            const v8 x = pair_rows<T>(t0, t1);
+            if (32 * s2 + 16 * (g & 1) + c < Lc) *(v8*)(vn_base + vn_lane + (int64_t)(32 * s2) * H * V * (int64_t)sizeof(T)) = x;
+          }
+          vn_base += (int64_t)BT * H * V * (int64_t)sizeof(T);
+        }
         lds_barrier();
       }
     }
@@ -432,8 +516,11 @@ int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
   FLA_REQUIRE(nblk <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   if (nblk == 0) return FLA_OK;
   dim3 grid((unsigned)nblk), block(512);
-  if (K == 64) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64>), grid, block, 0, st, p);
-  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128>), grid, block, 0, st, p);
+  const bool keep = p.v_new != nullptr;
+  if (K == 64 && keep) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64, true>), grid, block, 0, st, p);
+  else if (K == 64) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64, false>), grid, block, 0, st, p);
+  else if (K == 128 && keep) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128, true>), grid, block, 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128, false>), grid, block, 0, st, p);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;
@@ -443,7 +530,7 @@ int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
 
 extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
                                                    const float* g_cumsum, const float* h0, void* o, float* ht,
-                                                   const int64_t* offsets, const int64_t* chunk_offsets,
+                                                   void* v_new, void* h_frag_t, const int64_t* offsets, const int64_t* chunk_offsets,
                                                    const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
                                                    int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                                    fla_stream_t stream) {
@@ -451,8 +538,10 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k,
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
   FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o) % 16 == 0, FLA_E_ALIGNMENT);
-  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
+  FLA_REQUIRE((v_new == nullptr) == (h_frag_t == nullptr), FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o | (uintptr_t)v_new |
+               (uintptr_t)h_frag_t) % 16 == 0, FLA_E_ALIGNMENT);
+  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
   if (qkv_dtype == FLA_BF16) return launch_scan<bf16>(p, (int)K, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_scan<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

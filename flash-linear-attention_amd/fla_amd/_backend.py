@@ -50,7 +50,7 @@ SIGNATURES = {
                                                  I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h_both": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, P]),
     "fla_gdr_fwd_prep": (c_int, [P, P, P, P, I, P, P, F, P, P, I64, I, I64, I64, I64, I64, P]),
-    "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 13 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 17 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_o_gk": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, F, P]),

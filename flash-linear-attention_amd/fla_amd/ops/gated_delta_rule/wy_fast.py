@@ -22,10 +22,12 @@ def fwd_prepare_wy_repr(
     *,
     store_A: bool = True,
     store_Au: bool = True,
+    store_u: bool = True,
 ):
     """Returns ``(w, u, Aw, Au)`` with ``Aw = (I + strict_lower(diag(beta) K K^T))^-1``,
     ``Au = Aw * exp(g_i - g_j)``, ``w = Aw (beta K)``, ``u = Au (beta V)``; ``g`` is the
-    fp32 chunk-local cumsum of the log-gate (or ``None``)."""
+    fp32 chunk-local cumsum of the log-gate (or ``None``).  ``store_u=False`` skips ``u`` (returned as ``None``)
+    for a forward that forms ``v_new`` from the triangular tiles instead."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd fwd_prepare_wy_repr: seq-first, chunk size 64 only")
     be.require_gpu(k, v, beta)
@@ -38,7 +40,7 @@ def fwd_prepare_wy_repr(
     beta = beta.float().contiguous()
     if g is not None:
         g = g.float().contiguous()
-    w, u = torch.empty_like(k), torch.empty_like(v)
+    w, u = torch.empty_like(k), (torch.empty_like(v) if store_u else None)
     Aw = k.new_empty(B, T, H, BT) if store_A else None
     Au = k.new_empty(B, T, H, BT) if (store_A and store_Au) else None
     be.check(be.lib().fla_gdr_fwd_wy(

@@ -247,7 +247,8 @@ int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, 
  * :111-236; :379-426 kernel :250-317): Aw = (I + strict_lower(diag(beta) K K^T))^-1,
  * Au = Aw * exp(g_i - g_j), w = Aw (beta K) [B,T,H,K], u = Au (beta V) [B,T,H,V].
  * Aw, Au (optional outputs, [B,T,H,64] in the q/k/v dtype) are what the
- * reference saves for backward.
+ * reference saves for backward; u may be NULL as well (a forward that forms v_new from
+ * the triangular tiles of fla_gdr_fwd_prep keeps w and Aw alone).
  *
  * fla_chunk_gated_delta_rule_fwd_h: state scan, replaces
  * chunk_gated_delta_rule_fwd_h (fla/ops/common/chunk_delta_h.py:248-320,
@@ -302,6 +303,9 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * a chunk,  v_new = Tu (v - e^{gamma} (k h)),  o = scale e^{gamma} (q h) + Aqk v_new,
  * h <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} v_new).  g_cumsum fp32 [B,T,H] or NULL; h0, ht fp32
  * [N,H,K,V] or NULL; packed batches need chunk_offsets [N+1]; seq_order as for fla_chunk_gla_fwd_fused.
+ * v_new [B,T,H,V] and h_frag_t (the state entering every chunk, FLA_H_FRAGMENT_T, [chunks,H,K*V]), both in
+ * the q/k/v dtype and both given or both NULL: what a forward that will be differentiated keeps for
+ * fla_chunk_gated_delta_rule_bwd.
  * K in {64, 128}, V a multiple of 64. */
 int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
                      float* g_cumsum_out, void* AT, float scale, const int64_t* offsets, const int64_t* indices,
@@ -309,7 +313,8 @@ int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const floa
 
 int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
                                         const float* g_cumsum, const float* h0, void* o, float* ht,
-                                        const int64_t* offsets, const int64_t* chunk_offsets,
+                                        void* v_new, void* h_frag_t, const int64_t* offsets,
+                                        const int64_t* chunk_offsets,
                                         const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                         int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 

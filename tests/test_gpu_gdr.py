@@ -304,8 +304,11 @@ def test_chunk_gdr_reference_ladder(device, D, T, scale, normalizer, head_first)
 
 @pytest.mark.parametrize("varlen", [False, True])
 def test_chunk_gdr_keep_vs_recompute(device, varlen, monkeypatch):
-    """The backward from kept forward states and the reference-style backward that recomputes them
-    run the same kernels on the same operands: identical gradients; both forwards within tolerance."""
+    """The backward from what the forward kept (w, Aw and the v_new / states the scan wrote) and the
+    reference-style backward that recomputes them (WY launch + state scan on w, u) run the same backward
+    kernels on operands that differ by one 16-bit rounding (v_new = Tu (v - e^g (k h)) against u - e^g (w h)):
+    the two sets of gradients carry independent rounding errors and stay within the operator's tolerances of each
+    other; the forward within tolerance."""
     import fla_amd.ops.gated_delta_rule.chunk as mod
     from oracle.recurrent import naive_recurrent_gated_delta_rule
     gen = torch.Generator().manual_seed(12)
@@ -321,8 +324,8 @@ def test_chunk_gdr_keep_vs_recompute(device, varlen, monkeypatch):
                            offsets=offs)
     monkeypatch.setattr(mod, "KEEP_STATES_FOR_BACKWARD", False)
     rec = _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs)
-    for name, a, b in zip(NAMES, kept, rec):
-        assert torch.equal(a, b), name
+    for name, a, b, tol in zip(NAMES, kept, rec, TOLS):
+        assert_close(name + " kept vs recomputed", b.float().cpu(), a, tol)
     ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
                                                offsets=None if offs is None else offs.tolist())
     assert_close("o (two launches, states kept)", ro, o_keep, TOL_O)
