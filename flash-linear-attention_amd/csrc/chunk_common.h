@@ -49,7 +49,11 @@ FLA_DEVICE int64_t xcd_remap(int64_t id, int64_t total) {
 // Workgroups are dispatched in blockIdx order and dealt round-robin to the 8 XCDs; the slabs
 // of one (sequence, head) are placed on the same XCD (they read the same q/k/gate rows, which
 // then hit in that XCD's L2), and (sequence, head) items are taken in dispatch order, so that
-// with `seq_order` (sequence ids, longest first) the longest sequences start first.
+// with `seq_order` (sequence ids, longest first) the longest sequences start first.  A launch that fits
+// the chip in one wave of workgroups (at most one per CU, all start together) instead gives each XCD a
+// contiguous run of items, i.e. whole sequences where the batch allows: an XCD then walks an eighth of the
+// pages instead of all of them (189 against 191 us on 8 sequences x 16 heads x 4096 tokens).
+constexpr int64_t kNumCUs = 256;
 struct ScanItem {
   int slab;       // value-column slab
   int64_t item;   // (position in seq_order) * H + head
@@ -59,7 +63,8 @@ FLA_DEVICE ScanItem scan_item(int nslab) {
   ScanItem s;
   if (tot % (8 * nslab) == 0) {
     s.slab = (int)((p / 8) % nslab);
-    s.item = (p / (8 * nslab)) * 8 + p % 8;
+    if (tot <= kNumCUs) s.item = (p % 8) * (tot / (8 * nslab)) + p / (8 * nslab);
+    else s.item = (p / (8 * nslab)) * 8 + p % 8;
   } else {
     s.slab = (int)(p % nslab);
     s.item = p / nslab;

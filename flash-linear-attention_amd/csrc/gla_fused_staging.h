@@ -303,7 +303,7 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
       const int ls = min(ldo[i], (Lc - 1) * LDT + ocol);
       const uint32_t os = min(offo[i], (uint32_t)(Lc - 1) * opitch + (uint32_t)ocol * (uint32_t)sizeof(T));
       const v8 x = *(const v8*)&L.o[ls];
-      *(v8*)(po + os) = x;
+      __builtin_nontemporal_store(x, (v8*)(po + os));   // written once, never read here: keep it out of the L2's way
     }
     po += stro;
     ++oc;

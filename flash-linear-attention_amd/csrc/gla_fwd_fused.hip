@@ -160,7 +160,8 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     auto load_v = [&]() __attribute__((always_inline)) {
       const uint32_t lim = (lvc >= nchunks - 1 ? vlim_last : vlim_full) + (uint32_t)vc * (uint32_t)sizeof(T);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) vreg[i] = *(const t2*)(lv + (offv[i] < lim ? offv[i] : lim));
+      for (int i = 0; i < 8; ++i)   // read once by this workgroup only (q, k, g are read by both slabs of a head)
+        vreg[i] = __builtin_nontemporal_load((const t2*)(lv + (offv[i] < lim ? offv[i] : lim)));
       if (lvc + 1 < nchunks) lv += strv;
       ++lvc;
     };
