@@ -423,7 +423,7 @@ def bench_layer_steps(device, steps=20):
     rec("l2norm_fwd", lambda: l2norm_fwd(x), 2 * nb)
     rec("l2norm_bwd", lambda: l2norm_bwd(x, dy), 3 * nb)
     rec("rmsnorm_swish_gate_fwd", lambda: norm_gate_fwd(x, o, w, None, 1e-5, True), 3 * nb)
-    y, mean, rstd = norm_gate_fwd(x, o, w, None, 1e-5, True)
+    y, mean, rstd, _ = norm_gate_fwd(x, o, w, None, 1e-5, True)
     rec("rmsnorm_swish_gate_bwd", lambda: norm_gate_bwd(dy, x, o, w, None, 1e-5, mean, rstd, True), 5 * nb)
     Dc = 2048
     xc = torch.randn(B, T, Dc, device=device, generator=gen).bfloat16()

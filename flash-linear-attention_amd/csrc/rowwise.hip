@@ -183,7 +183,28 @@ struct NormGateParams {
   int64_t M;
   int N;
   float eps;
+  // residual / prenorm variants (fla/modules/fused_norm_gate.py:68-74, :265-271).  Forward: the row that is
+  // normalised is x + res, and that sum is kept in res_out; backward: `x` is that kept sum, dres the gradient that
+  // arrives for it (prenorm), dres_in a copy of dx in the kept sum's type.  *_f32: fp32 instead of the type T.
+  const void* res;
+  void* res_out;
+  const void* dres;
+  void* dres_in;
+  int res_f32, res_out_f32;   // forward
+  int x_f32;                  // backward: type of x, dres and dres_in
 };
+
+// 8 elements of a row whose storage type is T or, when f32 is set (workgroup-uniform), fp32
+template <typename T>
+FLA_DEVICE void load8_as(const void* base, int f32, int64_t idx, float* o) {
+  if (f32) Row8<float>::load((const float*)base + idx, o);
+  else Row8<T>::load((const T*)base + idx, o);
+}
+template <typename T>
+FLA_DEVICE void store8_as(void* base, int f32, int64_t idx, const float* v) {
+  if (f32) Row8<float>::store((float*)base + idx, v);
+  else Row8<T>::store((T*)base + idx, v);
+}
 
 template <typename T, bool RMS, int LPR, int NP>
 __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(NormGateParams p) {
@@ -227,6 +248,13 @@ __global__ __launch_bounds__(256) void norm_gate_fwd_kernel(NormGateParams p) {
       Row8<T>::unpack(nx[pss], v[pss]);
       Row8<T>::unpack(ng[pss], g[pss]);
       if (col < N) {
+        if (p.res) {
+          float r8[VEC];
+          load8_as<T>(p.res, p.res_f32, row * N + col, r8);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) v[pss][i] += r8[i];
+        }
+        if (p.res_out) store8_as<T>(p.res_out, p.res_out_f32, row * N + col, v[pss]);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) s1 += v[pss][i];
       } else {
@@ -297,7 +325,7 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(NormGateParams p) {
     for (int pss = 0; pss < NP; ++pss) {
       const int col = (pss * LPR + sub) * VEC;
       if (col < N) {
-        Row8<T>::load((const T*)p.x + row * N + col, xh[pss]);
+        load8_as<T>(p.x, p.x_f32, row * N + col, xh[pss]);
         Row8<T>::load((const T*)p.gate + row * N + col, g[pss]);
         Row8<T>::load((const T*)p.dy + row * N + col, d[pss]);
 #pragma unroll
@@ -327,6 +355,13 @@ __global__ __launch_bounds__(256) void norm_gate_bwd_kernel(NormGateParams p) {
       if (col < N) {
 #pragma unroll
         for (int i = 0; i < VEC; ++i) d[pss][i] = (d[pss][i] - (xh[pss][i] * c1 + c2)) * rstd;
+        if (p.dres) {
+          float r8[VEC];
+          load8_as<T>(p.dres, p.x_f32, row * N + col, r8);
+#pragma unroll
+          for (int i = 0; i < VEC; ++i) d[pss][i] += r8[i];
+        }
+        if (p.dres_in) store8_as<T>(p.dres_in, p.x_f32, row * N + col, d[pss]);
         Row8<T>::store((T*)p.dx + row * N + col, d[pss]);
         Row8<T>::store((T*)p.dgate + row * N + col, g[pss]);
       }
@@ -451,15 +486,21 @@ extern "C" int fla_norm_swish_gate_workgroups(int64_t M, int64_t N) {
   return rows_grid(M, rpw_of((int)N), 2048);
 }
 
-extern "C" int fla_norm_swish_gate_fwd(const void* x, const void* gate, const float* weight, const float* bias, void* y,
-                                       float* mean, float* rstd, int64_t M, int64_t N, float eps, int is_rms_norm,
-                                       int dtype, fla_stream_t stream) {
+extern "C" int fla_norm_swish_gate_residual_fwd(const void* x, const void* gate, const float* weight, const float* bias,
+                                                const void* residual, int residual_dtype, void* y, void* residual_out,
+                                                int residual_out_dtype, float* mean, float* rstd, int64_t M, int64_t N,
+                                                float eps, int is_rms_norm, int dtype, fla_stream_t stream) {
   FLA_REQUIRE(x && gate && y && rstd && M >= 0 && N > 0, FLA_E_INVALID);
   FLA_REQUIRE(is_rms_norm || mean, FLA_E_INVALID);
   FLA_REQUIRE(N % 8 == 0 && N <= 2048, FLA_E_UNSUPPORTED);
-  FLA_REQUIRE((((uintptr_t)x) | ((uintptr_t)gate) | ((uintptr_t)y)) % 16 == 0, FLA_E_ALIGNMENT);
+  FLA_REQUIRE((((uintptr_t)x) | ((uintptr_t)gate) | ((uintptr_t)y) | ((uintptr_t)residual) | ((uintptr_t)residual_out)) % 16 == 0,
+              FLA_E_ALIGNMENT);
+  if (residual) FLA_REQUIRE(residual_dtype == dtype || residual_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  if (residual_out) FLA_REQUIRE(residual_out_dtype == dtype || residual_out_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   if (M == 0) return FLA_OK;
-  NormGateParams p{x, gate, weight, bias, y, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr, M, (int)N, eps};
+  NormGateParams p{x, gate, weight, bias, y, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr, M, (int)N, eps,
+                   residual, residual_out, nullptr, nullptr,
+                   residual && residual_dtype == FLA_F32, residual_out && residual_out_dtype == FLA_F32, 0};
   const int grid = rows_grid(M, rpw_of((int)N), 4096);   // grid-stride: weights are loaded once per lane
   hipStream_t st = (hipStream_t)stream;
 #define D(E, TT)                                                         \
@@ -474,18 +515,28 @@ extern "C" int fla_norm_swish_gate_fwd(const void* x, const void* gate, const fl
   return FLA_E_UNSUPPORTED;
 }
 
-extern "C" int fla_norm_swish_gate_bwd(const void* dy, const void* x, const void* gate, const float* weight,
-                                       const float* bias, const float* mean, const float* rstd, void* dx, void* dgate,
-                                       float* dw_partial, float* db_partial, int64_t M, int64_t N, float eps,
-                                       int is_rms_norm, int dtype, fla_stream_t stream) {
+extern "C" int fla_norm_swish_gate_fwd(const void* x, const void* gate, const float* weight, const float* bias, void* y,
+                                       float* mean, float* rstd, int64_t M, int64_t N, float eps, int is_rms_norm,
+                                       int dtype, fla_stream_t stream) {
+  return fla_norm_swish_gate_residual_fwd(x, gate, weight, bias, nullptr, dtype, y, nullptr, dtype, mean, rstd, M, N, eps,
+                                          is_rms_norm, dtype, stream);
+}
+
+extern "C" int fla_norm_swish_gate_residual_bwd(const void* dy, const void* x, int x_dtype, const void* gate,
+                                                const float* weight, const float* bias, const float* mean,
+                                                const float* rstd, const void* dresidual, void* dx, void* dgate,
+                                                void* dresidual_in, float* dw_partial, float* db_partial, int64_t M,
+                                                int64_t N, float eps, int is_rms_norm, int dtype, fla_stream_t stream) {
   FLA_REQUIRE(dy && x && gate && rstd && dx && dgate && M >= 0 && N > 0, FLA_E_INVALID);
   FLA_REQUIRE(is_rms_norm || mean, FLA_E_INVALID);
   FLA_REQUIRE(N % 8 == 0 && N <= 2048, FLA_E_UNSUPPORTED);
-  FLA_REQUIRE((((uintptr_t)x) | ((uintptr_t)gate) | ((uintptr_t)dy) | ((uintptr_t)dx) | ((uintptr_t)dgate)) % 16 == 0,
+  FLA_REQUIRE(x_dtype == dtype || x_dtype == FLA_F32, FLA_E_UNSUPPORTED);
+  FLA_REQUIRE((((uintptr_t)x) | ((uintptr_t)gate) | ((uintptr_t)dy) | ((uintptr_t)dx) | ((uintptr_t)dgate) |
+               ((uintptr_t)dresidual) | ((uintptr_t)dresidual_in)) % 16 == 0,
               FLA_E_ALIGNMENT);
   if (M == 0) return FLA_OK;
   NormGateParams p{x, gate, weight, bias, nullptr, (float*)mean, (float*)rstd, dy, dx, dgate, dw_partial, db_partial,
-                   M, (int)N, eps};
+                   M, (int)N, eps, nullptr, nullptr, dresidual, dresidual_in, 0, 0, x_dtype == FLA_F32};
   const int grid = fla_norm_swish_gate_workgroups(M, N);
   hipStream_t st = (hipStream_t)stream;
 #define D(E, TT)                                                        \
@@ -498,4 +549,12 @@ extern "C" int fla_norm_swish_gate_bwd(const void* dy, const void* x, const void
   D(FLA_F32, float)
 #undef D
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_norm_swish_gate_bwd(const void* dy, const void* x, const void* gate, const float* weight,
+                                       const float* bias, const float* mean, const float* rstd, void* dx, void* dgate,
+                                       float* dw_partial, float* db_partial, int64_t M, int64_t N, float eps,
+                                       int is_rms_norm, int dtype, fla_stream_t stream) {
+  return fla_norm_swish_gate_residual_bwd(dy, x, dtype, gate, weight, bias, mean, rstd, nullptr, dx, dgate, nullptr,
+                                          dw_partial, db_partial, M, N, eps, is_rms_norm, dtype, stream);
 }

@@ -70,6 +70,8 @@ SIGNATURES = {
     "fla_norm_swish_gate_workgroups": (c_int, [I64, I64]),
     "fla_norm_swish_gate_fwd": (c_int, [P, P, P, P, P, P, P, I64, I64, F, I, I, P]),
     "fla_norm_swish_gate_bwd": (c_int, [P] * 11 + [I64, I64, F, I, I, P]),
+    "fla_norm_swish_gate_residual_fwd": (c_int, [P, P, P, P, P, I, P, P, I, P, P, I64, I64, F, I, I, P]),
+    "fla_norm_swish_gate_residual_bwd": (c_int, [P, P, I] + [P] * 11 + [I64, I64, F, I, I, P]),
     "fla_causal_conv1d_fwd": (c_int, [P, P, P, P, I64, I64, I64, I64, I, I, P]),
     "fla_causal_conv1d_bwd_partials": (c_int, [I64, I64]),
     "fla_causal_conv1d_bwd": (c_int, [P] * 7 + [I64, I64, I64, I64, I, I, P]),

@@ -17,66 +17,95 @@ def _f32(t):
     return None if t is None else t.detach().float().contiguous()
 
 
-def norm_gate_fwd(x, o, weight, bias, eps, is_rms_norm):
-    """Rows of ``x``/``o`` [M,N] -> ``(y, mean, rstd)`` (fla/modules/fused_norm_gate.py:186-256)."""
+def norm_gate_fwd(x, o, weight, bias, eps, is_rms_norm, residual=None, residual_dtype=None):
+    """Rows of ``x``/``o`` [M,N] -> ``(y, mean, rstd, residual_out)`` (fla/modules/fused_norm_gate.py:103-180).
+
+    With ``residual`` the normalised row is ``x + residual``; that sum is returned as ``residual_out`` (in the
+    residual's dtype), as it is when ``residual_dtype`` differs from ``x.dtype``; otherwise ``residual_out`` is ``x``."""
     be.require_gpu(x, o)
     M, N = x.shape
     if N % 8 or N > 2048:
         raise NotImplementedError(f"fla_amd norm gate: last dimension {N} must be a multiple of 8 and at most 2048")
     o = o.to(x.dtype)
+    if residual is not None:
+        assert residual.shape == (M, N)
+        residual_dtype = residual.dtype
+        if residual_dtype not in (x.dtype, torch.float32):
+            raise NotImplementedError("fla_amd norm gate: the residual is in x's dtype or in fp32")
+        residual = residual.contiguous()
     y = torch.empty_like(x)
+    keep = residual is not None or (residual_dtype is not None and residual_dtype != x.dtype)
+    residual_out = torch.empty(M, N, dtype=residual_dtype, device=x.device) if keep else None
     mean = None if is_rms_norm else torch.empty(M, dtype=torch.float32, device=x.device)
     rstd = torch.empty(M, dtype=torch.float32, device=x.device)
     if M == 0:
-        return y, mean, rstd
-    be.check(be.lib().fla_norm_swish_gate_fwd(be.ptr(x), be.ptr(o), be.ptr(_f32(weight)), be.ptr(_f32(bias)), be.ptr(y),
-                                              be.ptr(mean), be.ptr(rstd), M, N, float(eps), int(is_rms_norm), be.dt(x),
-                                              be.stream_of(x)), "fla_norm_swish_gate_fwd")
-    return y, mean, rstd
+        return y, mean, rstd, residual_out if keep else x
+    be.check(be.lib().fla_norm_swish_gate_residual_fwd(
+        be.ptr(x), be.ptr(o), be.ptr(_f32(weight)), be.ptr(_f32(bias)), be.ptr(residual),
+        be.dt(residual) if residual is not None else be.dt(x), be.ptr(y), be.ptr(residual_out),
+        be.dt(residual_out) if keep else be.dt(x), be.ptr(mean), be.ptr(rstd), M, N, float(eps), int(is_rms_norm),
+        be.dt(x), be.stream_of(x)), "fla_norm_swish_gate_residual_fwd")
+    return y, mean, rstd, residual_out if keep else x
 
 
-def norm_gate_bwd(dy, x, o, weight, bias, eps, mean, rstd, is_rms_norm):
-    """``(dx, do, dw, db)`` (fla/modules/fused_norm_gate.py:333-397)."""
+def norm_gate_bwd(dy, x, o, weight, bias, eps, mean, rstd, is_rms_norm, dresidual=None, has_residual=False,
+                  x_dtype=None):
+    """``(dx, do, dw, db, dresidual_in)`` (fla/modules/fused_norm_gate.py:301-400); ``x`` is what the forward
+    normalised (its ``residual_out``), ``x_dtype`` the dtype of the forward's ``x`` (and of ``dx``, ``do``)."""
     M, N = x.shape
-    dy = dy.to(x.dtype).contiguous()
-    dx, do = torch.empty_like(x), torch.empty_like(x)
+    x_dtype = x.dtype if x_dtype is None else x_dtype
+    dy = dy.to(x_dtype).contiguous()
+    dx = torch.empty(M, N, dtype=x_dtype, device=x.device)
+    do = torch.empty(M, N, dtype=x_dtype, device=x.device)
+    dresidual_in = torch.empty_like(x) if has_residual and dx.dtype != x.dtype else None
+    if dresidual is not None:
+        dresidual = dresidual.to(x.dtype).contiguous()
     if M == 0:
         zw = None if weight is None else torch.zeros_like(weight)
         zb = None if bias is None else torch.zeros_like(bias)
-        return dx, do, zw, zb
+        return dx, do, zw, zb, (dx if has_residual and dresidual_in is None else dresidual_in)
     nwg = be.lib().fla_norm_swish_gate_workgroups(M, N)
     dwp = torch.empty(nwg, N, dtype=torch.float32, device=x.device) if weight is not None else None
     dbp = torch.empty(nwg, N, dtype=torch.float32, device=x.device) if bias is not None else None
-    be.check(be.lib().fla_norm_swish_gate_bwd(be.ptr(dy), be.ptr(x), be.ptr(o), be.ptr(_f32(weight)), be.ptr(_f32(bias)),
-                                              be.ptr(mean), be.ptr(rstd), be.ptr(dx), be.ptr(do), be.ptr(dwp), be.ptr(dbp),
-                                              M, N, float(eps), int(is_rms_norm), be.dt(x), be.stream_of(x)),
-             "fla_norm_swish_gate_bwd")
+    be.check(be.lib().fla_norm_swish_gate_residual_bwd(
+        be.ptr(dy), be.ptr(x), be.dt(x), be.ptr(o), be.ptr(_f32(weight)), be.ptr(_f32(bias)), be.ptr(mean),
+        be.ptr(rstd), be.ptr(dresidual), be.ptr(dx), be.ptr(do), be.ptr(dresidual_in), be.ptr(dwp), be.ptr(dbp), M, N,
+        float(eps), int(is_rms_norm), be.dt(dx), be.stream_of(x)), "fla_norm_swish_gate_residual_bwd")
     dw = None if dwp is None else dwp.sum(0).to(weight.dtype)
     db = None if dbp is None else dbp.sum(0).to(bias.dtype)
-    return dx, do, dw, db
+    if has_residual and dresidual_in is None:
+        dresidual_in = dx
+    return dx, do, dw, db, dresidual_in
 
 
 class LayerNormSwishGateFn(torch.autograd.Function):
-    """Same argument list as the reference's function (fla/modules/fused_norm_gate.py:400-480).
-    The residual / prenorm variants are not covered."""
+    """Same argument list and return values as the reference's function (fla/modules/fused_norm_gate.py:402-481),
+    residual / prenorm variants included."""
 
     @staticmethod
     def forward(ctx, x, o, weight, bias, residual=None, eps=1e-6, prenorm=False, residual_in_fp32=False,
                 is_rms_norm=False):
-        if residual is not None or prenorm or residual_in_fp32:
-            raise NotImplementedError("fla_amd norm gate: residual / prenorm variants are not covered")
         shape = x.shape
         x2, o2 = _rows(x), _rows(o).to(x.dtype)
-        y, mean, rstd = norm_gate_fwd(x2, o2, weight, bias, eps, is_rms_norm)
-        ctx.save_for_backward(x2, o2, weight, bias, mean, rstd)
+        if residual is not None:
+            assert residual.shape == shape
+            residual = _rows(residual)
+        residual_dtype = residual.dtype if residual is not None else (torch.float32 if residual_in_fp32 else None)
+        y, mean, rstd, residual_out = norm_gate_fwd(x2, o2, weight, bias, eps, is_rms_norm, residual, residual_dtype)
+        ctx.save_for_backward(residual_out, o2, weight, bias, mean, rstd)
         ctx.shape, ctx.o_shape, ctx.o_dtype, ctx.eps, ctx.is_rms_norm = shape, o.shape, o.dtype, eps, is_rms_norm
-        return y.reshape(shape)
+        ctx.has_residual, ctx.prenorm, ctx.x_dtype = residual is not None, prenorm, x.dtype
+        y = y.reshape(shape)
+        return y if not prenorm else (y, residual_out.reshape(shape))
 
     @staticmethod
     def backward(ctx, dy, *args):
         x, o, weight, bias, mean, rstd = ctx.saved_tensors
-        dx, do, dw, db = norm_gate_bwd(_rows(dy), x, o, weight, bias, ctx.eps, mean, rstd, ctx.is_rms_norm)
-        return (dx.reshape(ctx.shape), do.reshape(ctx.o_shape).to(ctx.o_dtype), dw, db, None, None, None, None, None)
+        dresidual = _rows(args[0]) if ctx.prenorm else None
+        dx, do, dw, db, dres_in = norm_gate_bwd(_rows(dy), x, o, weight, bias, ctx.eps, mean, rstd, ctx.is_rms_norm,
+                                                dresidual, ctx.has_residual, ctx.x_dtype)
+        return (dx.reshape(ctx.shape), do.reshape(ctx.o_shape).to(ctx.o_dtype), dw, db,
+                dres_in.reshape(ctx.shape) if ctx.has_residual else None, None, None, None, None)
 
 
 def layer_norm_swish_gate_fn(x, o, weight, bias, residual=None, prenorm=False, residual_in_fp32=False, eps=1e-6):

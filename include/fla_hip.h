@@ -509,6 +509,23 @@ int fla_norm_swish_gate_bwd(const void* dy, const void* x, const void* gate, con
                             float* dw_partial, float* db_partial, int64_t M, int64_t N, float eps,
                             int is_rms_norm, int dtype, fla_stream_t stream);
 
+/* The same pair with the residual / prenorm arguments of layer_norm_fwd / layer_norm_bwd
+ * (fla/modules/fused_norm_gate.py:68-74, :103-180; :265-271, :301-400).
+ * Forward: the row that is normalised is x + residual (fp32 sum; residual [M,N] in `dtype` or fp32, or NULL);
+ * residual_out, if given, receives that sum in `dtype` or fp32 (what the reference returns under prenorm and
+ * keeps for its backward).  Backward: x is the tensor the forward normalised (x itself, or residual_out) in
+ * x_dtype (`dtype` or fp32); dresidual (same type, or NULL) is the gradient that arrived for residual_out and is
+ * added to dx; dresidual_in (same type, or NULL) receives a copy of dx, for a residual whose type differs from x's. */
+int fla_norm_swish_gate_residual_fwd(const void* x, const void* gate, const float* weight, const float* bias,
+                                     const void* residual, int residual_dtype, void* y, void* residual_out,
+                                     int residual_out_dtype, float* mean, float* rstd, int64_t M, int64_t N,
+                                     float eps, int is_rms_norm, int dtype, fla_stream_t stream);
+int fla_norm_swish_gate_residual_bwd(const void* dy, const void* x, int x_dtype, const void* gate,
+                                     const float* weight, const float* bias, const float* mean, const float* rstd,
+                                     const void* dresidual, void* dx, void* dgate, void* dresidual_in,
+                                     float* dw_partial, float* db_partial, int64_t M, int64_t N, float eps,
+                                     int is_rms_norm, int dtype, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Depthwise causal convolution over time, channels last, replaces the external
  * causal_conv1d_fn / causal_conv1d_update calls of ShortConvolution

@@ -30,8 +30,14 @@ def l2norm(x: torch.Tensor, eps: float = 1e-6, dtype=torch.float32) -> torch.Ten
     return x / torch.sqrt((x * x).sum(-1, keepdim=True) + eps)
 
 
-def norm_swish_gate(x, o, weight=None, bias=None, eps: float = 1e-5, is_rms_norm: bool = True, dtype=torch.float32):
+def norm_swish_gate(x, o, weight=None, bias=None, eps: float = 1e-5, is_rms_norm: bool = True, dtype=torch.float32,
+                    residual=None, prenorm: bool = False):
+    """``norm(x + residual) * weight + bias`` times ``o * sigmoid(o)``; with ``prenorm`` also the sum that was
+    normalised (fla/modules/fused_norm_gate.py:68-74, :446)."""
     x, o = x.to(dtype), o.to(dtype)
+    if residual is not None:
+        x = x + residual.to(dtype)
+    pre = x
     if not is_rms_norm:
         x = x - x.mean(-1, keepdim=True)
     rstd = 1.0 / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
@@ -40,7 +46,8 @@ def norm_swish_gate(x, o, weight=None, bias=None, eps: float = 1e-5, is_rms_norm
         y = y * weight.to(dtype)
     if bias is not None:
         y = y + bias.to(dtype)
-    return y * o * torch.sigmoid(o)
+    y = y * o * torch.sigmoid(o)
+    return (y, pre) if prenorm else y
 
 
 def causal_conv1d(x, weight, bias=None, activation: Optional[str] = None, dtype=torch.float32):

@@ -94,8 +94,54 @@ def test_norm_swish_gate_with_bias_function(device):
     assert_close("y", yr, y, 1e-5)
     for name, r, d in zip(("dx", "do", "dw", "db"), refs, leaves):
         assert_close(name, r.grad, d.grad, 1e-5)
-    with pytest.raises(NotImplementedError):
-        layer_norm_swish_gate_fn(leaves[0], leaves[1], leaves[2], leaves[3], residual=leaves[0])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("is_rms", [True, False])
+@pytest.mark.parametrize("res_kind,prenorm,in_fp32", [("same", False, False), ("same", True, False), ("fp32", True, False),
+                                                     (None, True, True), (None, True, False), ("fp32", False, False)])
+def test_norm_swish_gate_residual_prenorm(device, dtype, is_rms, res_kind, prenorm, in_fp32):
+    """The residual / prenorm forms of the reference's function (fla/modules/fused_norm_gate.py:402-481): the sum
+    x + residual is normalised, prenorm returns it, and gradients reach x, o, the weight and the residual."""
+    from fla_amd.modules import layer_norm_swish_gate_fn, rms_norm_swish_gate_fn
+    from oracle.modules import norm_swish_gate
+    gen = torch.Generator().manual_seed(11)
+    N, shape = 128, (3, 70, 2, 128)
+    x = (torch.randn(*shape, generator=gen) * 2 + 0.3).to(dtype)
+    o = torch.randn(*shape, generator=gen).to(dtype)
+    dy = torch.randn(*shape, generator=gen).to(dtype)
+    dpre = torch.randn(*shape, generator=gen)
+    w = torch.randn(N, generator=gen) * 0.5 + 1.0
+    res = None if res_kind is None else torch.randn(*shape, generator=gen).to(dtype if res_kind == "same" else torch.float32)
+    print(f"norm gate residual {dtype} rms={is_rms} res={res_kind} prenorm={prenorm} fp32={in_fp32}", flush=True)
+    fn = rms_norm_swish_gate_fn if is_rms else layer_norm_swish_gate_fn
+    xd, od, wd = x.to(device).requires_grad_(), o.to(device).requires_grad_(), w.to(device).requires_grad_()
+    rd = None if res is None else res.to(device).requires_grad_()
+    out = fn(xd, od, wd, None, residual=rd, prenorm=prenorm, residual_in_fp32=in_fp32, eps=1e-5)
+    xr, orr, wr = x.float().requires_grad_(), o.float().requires_grad_(), w.clone().requires_grad_()
+    rr = None if res is None else res.float().requires_grad_()
+    ref = norm_swish_gate(xr, orr, wr, None, eps=1e-5, is_rms_norm=is_rms, residual=rr, prenorm=prenorm)
+    ft, bt = _tols(dtype)
+    if prenorm:
+        y, pre = out
+        yr, prer = ref
+        want = res.dtype if res is not None else (torch.float32 if in_fp32 else dtype)
+        assert pre.dtype == want and pre.shape == x.shape
+        assert_close("residual_out", prer, pre, ft)
+        (y.float() * dy.to(device).float()).sum().add((pre.float() * dpre.to(device)).sum()).backward()
+        ((yr * dy.float()).sum() + (prer * dpre).sum()).backward()
+    else:
+        y, yr = out, ref
+        y.backward(dy.to(device))
+        yr.backward(dy.float())
+    assert y.dtype == dtype
+    assert_close("y", yr, y, ft)
+    assert_close("dx", xr.grad, xd.grad, bt)
+    assert_close("do", orr.grad, od.grad, bt)
+    assert_close("dw", wr.grad, wd.grad, 2e-3 if dtype != torch.float32 else 1e-5)
+    if res is not None:
+        assert rd.grad.dtype == res.dtype
+        assert_close("dresidual", rr.grad, rd.grad, bt)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

@@ -37,6 +37,11 @@ def test_norm_swish_gate_against_library(is_rms, affine):
     else:
         ref = F.layer_norm(x, (N,), w, b, eps=1e-5)
     torch.testing.assert_close(got, ref * F.silu(o))
+    # residual: the row that is normalised is the sum, and prenorm hands that sum back
+    r = torch.randn(6, N, generator=gen, dtype=torch.float64)
+    y2, pre = norm_swish_gate(x - r, o, w, b, eps=1e-5, is_rms_norm=is_rms, dtype=torch.float64, residual=r, prenorm=True)
+    torch.testing.assert_close(y2, got)
+    torch.testing.assert_close(pre, x)
 
 
 @pytest.mark.parametrize("W", [2, 3, 4])
