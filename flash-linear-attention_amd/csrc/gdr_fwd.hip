@@ -349,6 +349,8 @@ struct PrepParams {
   const int64_t* indices;
   int64_t T;
   int H, NTfix;
+  void* w;             // KEEP: w = Aw (beta k) [rows, H, K] and Aw [rows, H, 64], what the backward reads
+  void* Aw;
 };
 
 constexpr int kPrepWorkgroups = 3 * 256;        // three resident workgroups (register budget) on each of the 256 CUs
@@ -359,8 +361,25 @@ FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 // accumulators: the loads land while the inversion runs (measured: worth about 4 %; the launch is a chain
 // of short dependent phases - removing the inversion, the stores or the loads each saves 15-20 % - rather
 // than bound by one resource).
-template <typename T, int K>
-__global__ __launch_bounds__(256, 3) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
+// 32x32x16 operand whose 32 rows are contiguous in LDS and whose contraction index is the tile's row
+// (tile[kk][m], pitch ld): the transposing LDS read hands lane j of a 16-lane group element j of the four
+// rows whose 8-byte pieces the group's lanes 4i .. 4i+3 address.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag32_tr(const T* tile, int ld, int m0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef short s4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const int s = lane & 15, g = lane >> 4;
+  const T* p0 = tile + (k0 + 8 * (g >> 1) + (s >> 2)) * ld + m0 + 16 * (g & 1) + 4 * (s & 3);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 4 * ld));
+  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// KEEP: the forward of a pass that will be differentiated also leaves w = Aw (beta k) and Aw in memory (the WY
+// launch of the reference's decomposition, without a second inversion and a second pass over k).
+template <typename T, int K, bool KEEP>
+__global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
@@ -375,6 +394,8 @@ __global__ __launch_bounds__(256, 3) void gdr_fwd_prep_kernel(PrepParams p, int6
   float* sM = (float*)sRA;
   T* sQ = (T*)sRB;
   T* sTu = (T*)sRA;
+  T* sAb = (T*)sRA + kTriElems;   // KEEP: Aw diag(beta), row-major [64][LDT], behind the packed tile
+  static_assert((kTriElems + BT * LDT) * 2 <= R_BYTES, "region A holds the packed tile and Aw diag(beta)");
   float* sX = (float*)sRB;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -524,6 +545,11 @@ __global__ __launch_bounds__(256, 3) void gdr_fwd_prep_kernel(PrepParams p, int6
     lds_barrier();  // M complete; region B becomes X
     // the next item's rows start their way to the registers now: the matrix products above no longer
     // hold their accumulators, and the inversion below needs few registers and no memory
+    v8 kkeep[KEEP ? NPL : 1];
+    if constexpr (KEEP) {
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) kkeep[i] = cur.k[i];
+    }
     if (more) {
       advance();
       fetch(cur);
@@ -552,14 +578,74 @@ __global__ __launch_bounds__(256, 3) void gdr_fwd_prep_kernel(PrepParams p, int6
         *(v8*)dst = tu[0];
         *(v8*)(dst + 8) = tu[1];
       }
+      if constexpr (KEEP) {
+        // Aw row piece to memory; Aw diag(beta) as a row-major 16-bit tile behind the packed tile
+        v8 aw[2], ab[2];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4 xv = *(const f32x4*)&sX[i * LDM + 16 * jb + 4 * q4];
+          const f32x4 bj = *(const f32x4*)&sBeta[16 * jb + 4 * q4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int jj = 4 * q4 + e, j = 16 * jb + jj;
+            const float x = j <= i ? xv[e] : 0.f;
+            aw[jj >> 3][jj & 7] = (T)x;
+            ab[jj >> 3][jj & 7] = (T)(x * bj[e]);
+          }
+        }
+        *(v8*)&sAb[i * LDT + 16 * jb] = ab[0];
+        *(v8*)&sAb[i * LDT + 16 * jb + 8] = ab[1];
+        if (i < L) {
+          T* ap = (T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + 16 * jb;
+          *(v8*)ap = aw[0];
+          *(v8*)(ap + 8) = aw[1];
+        }
+      }
     }
     lds_barrier();
+    if constexpr (KEEP) {
+      // X is dead: its storage takes k row-major again (rows past the end of the chunk zero)
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int row = r0 + RPP * i;
+        *(v8*)&sQ[row * LDK + c8] = row < L ? kkeep[i] : z;
+      }
+    }
     // both tiles leave as one contiguous 10 KB block, 16 bytes per lane
     {
       T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)(2 * kTriElems);
       constexpr int NP = kTriElems / 8;   // 16-byte pieces per tile
       for (int e = tid; e < 2 * NP; e += 256)
         *(v8*)(at + e * 8) = e < NP ? *(const v8*)&sTu[e * 8] : *(const v8*)&sPo[(e - NP) * 8];
+    }
+    if constexpr (KEEP) {
+      lds_barrier();   // k row-major complete
+      // w^T = k^T (Aw diag(beta))^T: a lane ends up with one time row and four consecutive key channels per quad
+      const int rw = wave & 1, cb = wave >> 1;   // rows 32 rw .., key channels (K / 2) cb ..
+      constexpr int TN = K / 64;
+      f32x16 acc[TN];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) acc[t] = zero16();
+      const int jsteps = (rw + 1) * 2;           // Aw is lower triangular
+      for (int js = 0; js < jsteps; ++js) {
+        const v8 a = lds_frag32<T>(sAb, LDT, rw * 32, js * 16, lane);
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+          acc[t] = Elem<T>::mfma32(frag32_tr<T>(sQ, LDK, (cb * TN + t) * 32, js * 16, lane), a, acc[t]);
+      }
+      const int i = rw * 32 + (lane & 31);
+      if (i < L) {
+        T* wp = (T*)p.w + ((row0 + i) * H + hh) * (int64_t)K + 4 * (lane >> 5);
+#pragma unroll
+        for (int t = 0; t < TN; ++t)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            v4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = (T)acc[t][4 * r4 + e];
+            *(v4*)(wp + (cb * TN + t) * 32 + 8 * r4) = o;
+          }
+      }
     }
     if (!more) break;
     lin = next;
@@ -1118,10 +1204,17 @@ template <typename T>
 int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
   // (chunk, head) items, head-fastest; as many workgroups as are resident at once, each walking its share of the items
   const int64_t total = (int64_t)chunk_grid_.x * chunk_grid_.y;
-  dim3 grid((unsigned)(total < kPrepWorkgroups ? total : kPrepWorkgroups));
-  if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64>), grid, dim3(256), 0, st, p, total);
-  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128>), grid, dim3(256), 0, st, p, total);
-  else return FLA_E_UNSUPPORTED;
+  const int64_t resident = p.w ? 2 * 256 : kPrepWorkgroups;   // the w-writing variant runs two workgroups per CU
+  dim3 grid((unsigned)(total < resident ? total : resident));
+  if (p.w) {
+    if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64, true>), grid, dim3(256), 0, st, p, total);
+    else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128, true>), grid, dim3(256), 0, st, p, total);
+    else return FLA_E_UNSUPPORTED;
+  } else {
+    if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64, false>), grid, dim3(256), 0, st, p, total);
+    else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128, false>), grid, dim3(256), 0, st, p, total);
+    else return FLA_E_UNSUPPORTED;
+  }
   FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
@@ -1129,18 +1222,19 @@ int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
 }  // namespace
 
 extern "C" int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
-                                float* g_cumsum_out, void* AT, float scale, const int64_t* offsets,
+                                float* g_cumsum_out, void* AT, void* w, void* Aw, float scale, const int64_t* offsets,
                                 const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                 int64_t K, fla_stream_t stream) {
   FLA_REQUIRE(q && k && beta && AT, FLA_E_INVALID);
+  FLA_REQUIRE((w == nullptr) == (Aw == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && NT >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)AT) % 16 == 0, FLA_E_ALIGNMENT);
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)AT | (uintptr_t)w | (uintptr_t)Aw) % 16 == 0, FLA_E_ALIGNMENT);
   dim3 grid;
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  PrepParams p{q, k, beta, g, g_is_cumsum, g_cumsum_out, AT, scale, offsets, indices, T, (int)H, ntfix};
+  PrepParams p{q, k, beta, g, g_is_cumsum, g_cumsum_out, AT, scale, offsets, indices, T, (int)H, ntfix, w, Aw};
   if (qkv_dtype == FLA_BF16) return launch_prep<bf16>(p, (int)K, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_prep<f16>(p, (int)K, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

@@ -82,17 +82,15 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
 def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, output_final_state, offsets=None):
     """Forward of a pass that will be differentiated.  Returns ``(g_cumsum, o, final_state, kept)``
     with ``kept = (w, Aw, v_new, hT)`` for :func:`chunk_gated_delta_rule_bwd`.  Key dims up to 128: the
-    two-launch forward, whose scan also writes ``v_new`` and the state entering every chunk, plus the WY launch
-    for ``w`` and ``Aw``.  K = 256: the reference's decomposition (WY launch, state scan, output stage)."""
+    two-launch forward, whose first launch also writes ``w`` and ``Aw`` and whose scan also writes ``v_new`` and
+    the state entering every chunk.  K = 256: the reference's decomposition (WY launch, state scan, output stage)."""
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
     co = None if plan is None else plan.chunk_offsets
     beta = beta.float().contiguous()
     if q.shape[-1] <= _FUSED_MAX_K:
-        AT, g = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=offs, indices=idx)
-        w, _, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
-                                          store_A=True, store_Au=False, store_u=False)
+        AT, g, w, Aw = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=offs, indices=idx, keep_w=True)
         o, final_state, v_new, hT = chunk_gated_delta_rule_fwd_scan(
             q, k, v, AT, g, scale, initial_state, output_final_state, offsets=offs, chunk_offsets=co,
             seq_order=None if plan is None else plan.seq_order, keep=True)

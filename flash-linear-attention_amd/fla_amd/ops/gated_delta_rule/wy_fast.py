@@ -61,14 +61,17 @@ def fwd_prepare_scan_operands(
     offsets: Optional[torch.Tensor] = None,
     indices: Optional[torch.Tensor] = None,
     g_is_cumsum: bool = False,
-) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    keep_w: bool = False,
+):
     """Chunk-parallel half of the one-pass forward (``fla_gdr_fwd_prep``): the work of ``chunk_local_cumsum``,
     ``fwd_prepare_wy_repr`` (``fla/ops/gated_delta_rule/wy_fast.py:320-376``) and the score product of
     ``chunk_fwd_o`` (``fla/ops/common/chunk_o.py:86-97``), leaving per (chunk, head) the lower-triangular
     ``Tu = (Aw * Gamma) diag(beta)`` and ``Aqk = scale tril(q k^T * Gamma)`` as packed 16x16 blocks:
     ``AT`` is ``[chunks, H, 2, 10, 16, 16]`` in the q/k/v dtype.  ``g`` is the raw per-head log-gate
     ``[B, T, H]`` (or its chunk-local cumsum with ``g_is_cumsum``; ``None`` for the un-gated rule).
-    Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``."""
+    Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``; with ``keep_w`` the launch also writes
+    ``w = Aw (beta k)`` and ``Aw`` (what ``fwd_prepare_wy_repr`` leaves for the backward) and the return value
+    is ``(AT, g_cumsum, w, Aw)``."""
     be.require_gpu(q, k, beta)
     B, T, H, K = k.shape
     NT = 0
@@ -82,11 +85,13 @@ def fwd_prepare_scan_operands(
         g = g.float().contiguous()
         gc = g if g_is_cumsum else torch.empty_like(g)
     AT = k.new_empty(chunks, H, 2, TRI_BLOCKS, 16, 16)
+    w = torch.empty_like(k) if keep_w else None
+    Aw = k.new_empty(B, T, H, BT) if keep_w else None
     be.check(be.lib().fla_gdr_fwd_prep(
         be.ptr(q), be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
-        be.ptr(AT), float(scale), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, be.stream_of(k)),
-        "fla_gdr_fwd_prep")
-    return AT, gc
+        be.ptr(AT), be.ptr(w), be.ptr(Aw), float(scale), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K,
+        be.stream_of(k)), "fla_gdr_fwd_prep")
+    return (AT, gc, w, Aw) if keep_w else (AT, gc)
 
 
 def unpack_triangular_tiles(AT: torch.Tensor) -> torch.Tensor:

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 3
+#define FLA_ABI_VERSION 4
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -297,6 +297,9 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * inside a block): AT is [chunks, H, 2, 10, 16, 16] (chunk index as in `indices`, or b * ceil(T/64) + c).
  * g is the raw per-head log-gate [B,T,H] (g_is_cumsum == 0; its chunk-local prefix sum is formed in the kernel and
  * written to g_cumsum_out, fp32 [B,T,H], if that is given), or already the prefix sum (== 1), or NULL (no gate).
+ * w [B,T,H,K] and Aw [B,T,H,64] in the q/k/v dtype, both given or both NULL: w = Aw (beta k) and Aw = (I + M)^-1 as
+ * fwd_prepare_wy_repr leaves them (fla/ops/gated_delta_rule/wy_fast.py:320-376), for a forward that will be
+ * differentiated (fla_chunk_gated_delta_rule_bwd reads them).
  * K in {64, 128}.
  * fla_chunk_gated_delta_rule_fwd_scan is the serial part (state scan + output, replaces
  * chunk_gated_delta_rule_fwd_h + chunk_fwd_o, fla/ops/gated_delta_rule/chunk.py:47-72): with h the state entering
@@ -308,7 +311,8 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * fla_chunk_gated_delta_rule_bwd.
  * K in {64, 128}, V a multiple of 64. */
 int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
-                     float* g_cumsum_out, void* AT, float scale, const int64_t* offsets, const int64_t* indices,
+                     float* g_cumsum_out, void* AT, void* w, void* Aw, float scale, const int64_t* offsets,
+                     const int64_t* indices,
                      int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, fla_stream_t stream);
 
 int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,

@@ -99,6 +99,12 @@ def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
     # the same tiles from gates that are already cumulative
     AT2, gc2 = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), gc, K ** -0.5, g_is_cumsum=True)
     assert gc2 is gc and torch.equal(AT, AT2)
+    # the variant a differentiated forward runs: the same tiles, plus w = Aw (beta k) and Aw for the backward
+    AT3, gc3, w, Aw = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), K ** -0.5, keep_w=True)
+    torch.cuda.synchronize()
+    assert torch.equal(AT, AT3) and torch.equal(gc, gc3)
+    assert_close("Aw", ref['Aw'], Aw, 5e-3)
+    assert_close("w", ref['w'], w, 8e-3)
     o, ht = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, K ** -0.5, dev(h0), True)
     torch.cuda.synchronize()
     ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
@@ -126,6 +132,12 @@ def test_gdr_two_launch_forward_pieces_packed(device):
     tu_ref, aqk_ref = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
     assert_close("Tu", tu_ref, dense[:, :, 0], 5e-3)
     assert_close("Aqk", aqk_ref, dense[:, :, 1], 5e-3)
+    AT3, _, w, Aw = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), 128 ** -0.5, offsets=plan.offsets,
+                                              indices=plan.indices, keep_w=True)
+    torch.cuda.synchronize()
+    assert torch.equal(AT, AT3)
+    assert_close("Aw", ref['Aw'], Aw, 5e-3)
+    assert_close("w", ref['w'], w, 8e-3)
     o, ht = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, 128 ** -0.5, dev(h0), True,
                                             offsets=plan.offsets, chunk_offsets=plan.chunk_offsets,
                                             seq_order=plan.seq_order)
