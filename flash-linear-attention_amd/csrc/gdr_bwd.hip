@@ -496,7 +496,7 @@ struct DqkwgParams {
 };
 
 template <typename T, int V>
-__global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
+__global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, int64_t pairs) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDV = V + 8;
@@ -522,63 +522,120 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
   float* stC = (float*)sRC;
   float* stD = (float*)sRD;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x;
   const int H = p.H, K = p.K;
-  // The key slices of one (chunk, head) share do, v_new and dv2: they get consecutive logical
-  // ids on the same XCD, so the second slice finds those tiles in that XCD's L2.
+  // A workgroup walks items (chunk, head, key slice) with a stride of the grid size.  The key slices of one
+  // (chunk, head) share do, v_new and dv2: where the counts allow, they are items 8 apart, i.e. they run at the
+  // same time on the same XCD, and the second slice finds those tiles in that XCD's L2.
   const int nz = K / 64;
-  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int kb = (int)(lid % nz) * 64;
-  int hh;
-  ChunkLoc cl = locate_chunk_at(lid / nz, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  const int64_t nitems = pairs * nz;
+  const bool paired = nitems % (8 * nz) == 0 && gridDim.x % (8 * nz) == 0;
+  struct Item {
+    ChunkLoc cl;
+    int hh, kb;
+  };
+  auto locate = [&](int64_t it) {
+    Item r;
+    const int64_t pair = paired ? (it / (8 * nz)) * 8 + it % 8 : it / nz;
+    r.kb = (int)(paired ? (it / 8) % nz : it % nz) * 64;
+    r.cl = locate_chunk_at(pair, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    return r;
+  };
+  // The rows an item starts with (q, k, w slice: 4 rows x 4 columns per lane; do, v_new: whole rows in 16-byte
+  // pieces) are requested while the item before it is in its epilogue; rows past the end of a short chunk
+  // re-read its last row (masked at use), so no load sits under a branch.
+  const int rg0 = tid0 >> 4, c40 = (tid0 & 15) * 4;
+  struct Raw {
+    v4 q[4], k[4], w[4];
+    v8 d[NP], v[NP];
+  };
+  // byte offsets of this lane's pieces from the first row of a chunk (32-bit, off wave-uniform base pointers)
+  const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
+  uint32_t offk[4], offv[NP];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) offk[i] = (uint32_t)(rg0 * 4 + i) * pitchk + (uint32_t)c40 * (uint32_t)sizeof(T);
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int e = tid0 + 256 * i;
+    offv[i] = (uint32_t)(e / C8) * pitchv + (uint32_t)((e % C8) * 8) * (uint32_t)sizeof(T);
+  }
+  const uint32_t colk = (uint32_t)c40 * (uint32_t)sizeof(T), colv = (uint32_t)((tid0 % C8) * 8) * (uint32_t)sizeof(T);
+  auto request = [&](const Item& im, Raw& R) __attribute__((always_inline)) {
+    const uint32_t last = (uint32_t)(im.cl.L - 1);
+    const int64_t r0h = im.cl.row0 * H + im.hh;
+    const char* qb = (const char*)p.q + (r0h * K + im.kb) * (int64_t)sizeof(T);
+    const char* kb_ = (const char*)p.k + (r0h * K + im.kb) * (int64_t)sizeof(T);
+    const char* wb = (const char*)p.w + (r0h * K + im.kb) * (int64_t)sizeof(T);
+    const char* db = (const char*)p.dout + r0h * V * (int64_t)sizeof(T);
+    const char* vb = (const char*)p.vnew + r0h * V * (int64_t)sizeof(T);
+    const uint32_t limk = last * pitchk + colk, limv = last * pitchv + colv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o = offk[i] < limk ? offk[i] : limk;
+      R.q[i] = *(const v4*)(qb + o);
+      R.k[i] = *(const v4*)(kb_ + o);
+      R.w[i] = *(const v4*)(wb + o);
+    }
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const uint32_t o = offv[i] < limv ? offv[i] : limv;
+      R.d[i] = *(const v8*)(db + o);
+      R.v[i] = *(const v8*)(vb + o);
+    }
+  };
+  int64_t it = blockIdx.x;
+  if (it >= nitems) return;
+  Item im = locate(it);
+  Raw R;
+  request(im, R);
+  const v8 z8 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  for (;;) {
+  // The lane id goes through an opaque copy once per item: the LDS addresses of the body are then formed where
+  // they are used instead of being hoisted out of the loop into a hundred long-lived registers.
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rg = tid >> 4, c4 = (tid & 15) * 4;
+  const int hh = im.hh, kb = im.kb;
+  const ChunkLoc cl = im.cl;
   const int L = cl.L;
   const int64_t row0 = cl.row0;
-
-  // ---- loads
-  const int rg = tid >> 4, c4 = (tid & 15) * 4;
-  float qq[4][4], kk[4][4], ww[4][4], gam4[4];
+  // this item's q, k, w slice stays in storage precision until the epilogue (rows past the end zero)
+  v4 cq[4], ck[4], cww[4];
+  {
+    const v4 z4 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int row = rg * 4 + i;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
-      Load<T>::x4((const T*)p.q + off, qq[i]);
-      Load<T>::x4((const T*)p.k + off, kk[i]);
-      Load<T>::x4((const T*)p.w + off, ww[i]);
-      gam4[i] = p.gam ? p.gam[(row0 + row) * H + hh] : 0.f;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) qq[i][j] = kk[i][j] = ww[i][j] = 0.f;
-      gam4[i] = 0.f;
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = rg * 4 + i < L;
+      cq[i] = ok ? R.q[i] : z4;
+      ck[i] = ok ? R.k[i] : z4;
+      cww[i] = ok ? R.w[i] : z4;
     }
   }
   const float glast = p.gam ? p.gam[(row0 + L - 1) * H + hh] : 0.f;
   v8 dreg[NP], vreg[NP], d2reg[NP];
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)V + c8;
-      dreg[i] = *(const v8*)((const T*)p.dout + off);
-      vreg[i] = *(const v8*)((const T*)p.vnew + off);
-      d2reg[i] = *(const v8*)((const T*)p.dv2 + off);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) dreg[i][j] = vreg[i][j] = d2reg[i][j] = (T)0.f;
-    }
+    const int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    dreg[i] = row < L ? R.d[i] : z8;
+    vreg[i] = row < L ? R.v[i] : z8;
+    const uint32_t limv = (uint32_t)(L - 1) * pitchv + colv;
+    d2reg[i] = *(const v8*)((const char*)p.dv2 + (row0 * H + hh) * (int64_t)V * (int64_t)sizeof(T) + (offv[i] < limv ? offv[i] : limv));
   }
   const int rw = wave >> 1, cw = wave & 1;
   const int kt32 = kb / 32 + cw;
   v8 hf[VT32][2], dhf[VT32][2];
   {
-    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
+    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V * (int64_t)sizeof(T);
+    const char* hb = (const char*)p.hT + blk;
+    const char* dhb = (const char*)p.dhtf + blk;
 #pragma unroll
     for (int vt = 0; vt < VT32; ++vt) {
-      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
-      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
-      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
-      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
-      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
+      const uint32_t o = (uint32_t)(((vt * (K / 32) + kt32) * 64 + lane) * 16) * (uint32_t)sizeof(T);
+      hf[vt][0] = *(const v8*)(hb + o);
+      hf[vt][1] = *(const v8*)(hb + o + 16);
+      dhf[vt][0] = *(const v8*)(dhb + o);
+      dhf[vt][1] = *(const v8*)(dhb + o + 16);
     }
   }
   if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
@@ -593,8 +650,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
     v4 kt, qt;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      kt[i] = (T)kk[i][j];
-      qt[i] = (T)qq[i][j];
+      kt[i] = ck[i][j];
+      qt[i] = cq[i][j];
     }
     *(v4*)&sKT[(c4 + j) * LDT + rg * 4] = kt;
     *(v4*)&sQT[(c4 + j) * LDT + rg * 4] = qt;
@@ -604,9 +661,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
 #pragma unroll
   for (int vt = 0; vt < VT32; ++vt)
 #pragma unroll
-    for (int half = 0; half < 2; ++half)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) hd += (float)hf[vt][half][e] * (float)dhf[vt][half][e];
+    for (int half = 0; half < 2; ++half) hd = Elem<T>::dot8(hf[vt][half], dhf[vt][half], hd);
   __syncthreads();
   // ---- ds = s tril((do v_new^T) * Gamma), both orientations
   {
@@ -662,7 +717,7 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
     int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
-    *(v8*)&sDo[row * LDV + c8] = d2reg[i];
+    *(v8*)&sDo[row * LDV + c8] = row < L ? d2reg[i] : z8;
   }
   __syncthreads();
   // ---- dw = -e^gamma (dv2 h^T)
@@ -681,6 +736,14 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
     stB[o] = ak1[r];
     stC[o] = ak2[r];
     stD[o] = aw[r];
+  }
+  // the next item's first rows are requested now: the accumulators are in LDS, the epilogue needs few registers
+  const int64_t nit = it + gridDim.x;
+  const bool more = nit < nitems;   // workgroup-uniform
+  Item nim = im;
+  if (more) {
+    nim = locate(nit);
+    request(nim, R);
   }
   // <h, dH> of the whole key slice: reduce over the 4 waves through LDS
   __shared__ float sHd[4];
@@ -707,8 +770,8 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
       dqv[j] = (T)a[j];
       dkv[j] = (T)dk;
       dwv[j] = (T)d[j];
-      rs += qq[i][j] * a[j] - kk[i][j] * dk + ww[i][j] * d[j];
-      kin += kk[i][j] * c[j];
+      rs += (float)cq[i][j] * a[j] - (float)ck[i][j] * dk + (float)cww[i][j] * d[j];
+      kin += (float)ck[i][j] * c[j];
     }
     rowsum[i] = rs;
     if (row < L) {
@@ -740,6 +803,11 @@ __global__ __launch_bounds__(256) void gdr_bwd_dqkwg_kernel(DqkwgParams p) {
         p.dgam[((int64_t)(kb / 64) * p.total_rows + row0 + row) * H + hh] = val;
       }
     }
+  }
+  if (!more) break;
+  __syncthreads();  // the staging tiles are consumed: the next item's operand tiles may be written
+  it = nit;
+  im = nim;
   }
 }
 
@@ -1144,11 +1212,11 @@ int launch_dhu(const DhuParams& p, int64_t K, hipStream_t st) {
 // one workgroup per (chunk, head, 64 key channels)
 template <typename T>
 int launch_dqkwg(const DqkwgParams& p, int64_t V, dim3 grid, hipStream_t st) {
-  const int64_t nwg = (int64_t)grid.x * grid.y * (p.K / 64);
-  FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
-  dim3 g3((unsigned)nwg);
-  if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p);
-  else if (V == 128) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p);
+  // as many workgroups as are resident at once (two per CU), each walking its share of the items
+  const int64_t pairs = (int64_t)grid.x * grid.y, nwg = pairs * (p.K / 64);
+  dim3 g3((unsigned)(nwg < 2 * kNumCUs ? nwg : 2 * kNumCUs));
+  if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p, pairs);
+  else if (V == 128) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p, pairs);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;
