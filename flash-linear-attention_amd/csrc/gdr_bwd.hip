@@ -528,17 +528,18 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   // (chunk, head) share do, v_new and dv2: where the counts allow, they are items 8 apart, i.e. they run at the
   // same time on the same XCD, and the second slice finds those tiles in that XCD's L2.
   const int nz = K / 64;
-  const int64_t nitems = pairs * nz;
+  const uint32_t nitems = (uint32_t)pairs * (uint32_t)nz;   // < 2^31, checked by the launcher
   const bool paired = nitems % (8 * nz) == 0 && gridDim.x % (8 * nz) == 0;
   struct Item {
     ChunkLoc cl;
     int hh, kb;
   };
-  auto locate = [&](int64_t it) {
+  auto locate = [&](uint32_t it) {
     Item r;
-    const int64_t pair = paired ? (it / (8 * nz)) * 8 + it % 8 : it / nz;
-    r.kb = (int)(paired ? (it / 8) % nz : it % nz) * 64;
-    r.cl = locate_chunk_at(pair, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    const uint32_t unz = (uint32_t)nz;
+    const uint32_t pair = paired ? (it / (8 * unz)) * 8 + it % 8 : it / unz;
+    r.kb = (int)(paired ? (it / 8) % unz : it % unz) * 64;
+    r.cl = locate_chunk_at32(pair, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
     return r;
   };
   // The rows an item starts with (q, k, w slice: 4 rows x 4 columns per lane; do, v_new: whole rows in 16-byte
@@ -583,7 +584,7 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
       R.v[i] = *(const v8*)(vb + o);
     }
   };
-  int64_t it = blockIdx.x;
+  uint32_t it = blockIdx.x;
   if (it >= nitems) return;
   Item im = locate(it);
   Raw R;
@@ -738,13 +739,10 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
     stD[o] = aw[r];
   }
   // the next item's first rows are requested now: the accumulators are in LDS, the epilogue needs few registers
-  const int64_t nit = it + gridDim.x;
+  const uint32_t nit = it + gridDim.x;
   const bool more = nit < nitems;   // workgroup-uniform
-  Item nim = im;
-  if (more) {
-    nim = locate(nit);
-    request(nim, R);
-  }
+  const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it: no load under a branch)
+  request(nim, R);
   // <h, dH> of the whole key slice: reduce over the 4 waves through LDS
   __shared__ float sHd[4];
 #pragma unroll
@@ -1214,6 +1212,7 @@ template <typename T>
 int launch_dqkwg(const DqkwgParams& p, int64_t V, dim3 grid, hipStream_t st) {
   // as many workgroups as are resident at once (two per CU), each walking its share of the items
   const int64_t pairs = (int64_t)grid.x * grid.y, nwg = pairs * (p.K / 64);
+  FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   dim3 g3((unsigned)(nwg < 2 * kNumCUs ? nwg : 2 * kNumCUs));
   if (V == 64) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 64>), g3, dim3(256), 0, st, p, pairs);
   else if (V == 128) hipLaunchKernelGGL((gdr_bwd_dqkwg_kernel<T, 128>), g3, dim3(256), 0, st, p, pairs);

@@ -455,7 +455,7 @@ struct BDqkgParams {
 
 // grid (chunks, H, K/64): one workgroup per 64-wide slice of the key dim.
 template <typename T, typename GT, int V>
-__global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
+__global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int64_t pairs) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDV = V + 8;
@@ -481,120 +481,123 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   float* stB = (float*)sRB;
   float* stC = (float*)sRC;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x;
   const int H = p.H, K = p.K;
-  // The key slices of one (chunk, head) share v and do: they get consecutive logical ids on the
-  // same XCD, so the second slice finds those tiles in that XCD's L2.
+  // A workgroup walks items (chunk, head, key slice) with a stride of the grid size.  The key slices of one
+  // (chunk, head) share v and do: where the counts allow, they are items 8 apart, i.e. they run at the same
+  // time on the same XCD, and the second slice finds those tiles in that XCD's L2.
   const int nz = K / 64;
-  const int64_t lid = xcd_remap(blockIdx.x, gridDim.x);
-  const int kb = (int)(lid % nz) * 64;
-  int hh;
-  ChunkLoc cl = locate_chunk_at(lid / nz, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  const uint32_t nitems = (uint32_t)pairs * (uint32_t)nz;   // < 2^31, checked by the launcher
+  const bool paired = nitems % (8 * nz) == 0 && gridDim.x % (8 * nz) == 0;
+  struct Item {
+    ChunkLoc cl;
+    int hh, kb;
+  };
+  auto locate = [&](uint32_t it) {
+    Item r;
+    const uint32_t unz = (uint32_t)nz;
+    const uint32_t pair = paired ? (it / (8 * unz)) * 8 + it % 8 : it / unz;
+    r.kb = (int)(paired ? (it / 8) % unz : it % unz) * 64;
+    r.cl = locate_chunk_at32(pair, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    return r;
+  };
+  // The rows an item starts with (do, v: whole rows in 16-byte pieces) are requested while the item before it
+  // is in its epilogue; its q, k, g slice (4 rows x 4 columns per lane) and its state fragments are requested at
+  // its top and arrive behind the dA products, which need do and v only.  All of it at 32-bit offsets from
+  // wave-uniform base pointers; rows past the end of a short chunk re-read its last row (masked at use), so no
+  // load sits under a branch.
+  typedef GT g4 __attribute__((ext_vector_type(4)));
+  struct Raw {
+    v8 d[NP], v[NP];
+  };
+  const int rg0 = tid0 >> 4, c40 = (tid0 & 15) * 4;
+  const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
+  constexpr int GSH = sizeof(GT) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
+  uint32_t offk[4], offv[NP];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) offk[i] = (uint32_t)(rg0 * 4 + i) * pitchk + (uint32_t)c40 * (uint32_t)sizeof(T);
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int e = tid0 + 256 * i;
+    offv[i] = (uint32_t)(e / C8) * pitchv + (uint32_t)((e % C8) * 8) * (uint32_t)sizeof(T);
+  }
+  const uint32_t colk = (uint32_t)c40 * (uint32_t)sizeof(T), colv = (uint32_t)((tid0 % C8) * 8) * (uint32_t)sizeof(T);
+  auto request = [&](const Item& im, Raw& R) __attribute__((always_inline)) {
+    const uint32_t last = (uint32_t)(im.cl.L - 1);
+    const int64_t r0h = im.cl.row0 * H + im.hh;
+    const char* db = (const char*)p.dout + r0h * V * (int64_t)sizeof(T);
+    const char* vb = (const char*)p.v + r0h * V * (int64_t)sizeof(T);
+    const uint32_t limv = last * pitchv + colv;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const uint32_t o = offv[i] < limv ? offv[i] : limv;
+      R.d[i] = *(const v8*)(db + o);
+      R.v[i] = *(const v8*)(vb + o);
+    }
+  };
+  uint32_t it = blockIdx.x;
+  if (it >= nitems) return;
+  Item im = locate(it);
+  Raw R;
+  request(im, R);
+  const v8 z8 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  for (;;) {
+  // The lane id goes through an opaque copy once per item: the LDS addresses of the body are then formed where
+  // they are used instead of being hoisted out of the loop into long-lived registers.
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int rg = tid >> 4, c4 = (tid & 15) * 4;
+  const int hh = im.hh, kb = im.kb;
+  const ChunkLoc cl = im.cl;
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
   // gates beyond the single-reference range: dA is left out here and the intra-chunk terms are
   // added by gla_bwd_intra_exact_kernel
   const bool flagged = p.wide && p.wide[cl.cglob * H + hh];
-  // ---- loads: q,k,g slice as 4 rows x 4 cols per lane; do, v whole rows in 16-byte pieces
-  const int rg = tid >> 4, c4 = (tid & 15) * 4;
-  float gq[4][4], qq[4][4], kk[4][4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int row = rg * 4 + i;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
-      Load<GT>::x4((const GT*)p.g + off, gq[i]);
-      Load<T>::x4((const T*)p.q + off, qq[i]);
-      Load<T>::x4((const T*)p.k + off, kk[i]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) gq[i][j] = qq[i][j] = kk[i][j] = 0.f;
-    }
-  }
-  v8 dreg[NP], vreg[NP];
+  // ---- do, v row-major (rows past the end zero)
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)V + c8;
-      dreg[i] = *(const v8*)((const T*)p.dout + off);
-      vreg[i] = *(const v8*)((const T*)p.v + off);
-    } else {
+    const int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sDo[row * LDV + c8] = row < L ? R.d[i] : z8;
+    *(v8*)&sV[row * LDV + c8] = row < L ? R.v[i] : z8;
+  }
+  // ---- this item's q, k, g slice and state fragments: on their way during the dA products
+  g4 cg[4];
+  v4 cq[4], ck[4];
+  {
+    const int64_t r0h = row0 * H + hh;
+    const char* qb = (const char*)p.q + (r0h * K + kb) * (int64_t)sizeof(T);
+    const char* kb_ = (const char*)p.k + (r0h * K + kb) * (int64_t)sizeof(T);
+    const char* gb = (const char*)p.g + (r0h * K + kb) * (int64_t)sizeof(GT);
+    const uint32_t limk = (uint32_t)(L - 1) * pitchk + colk;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dreg[i][j] = vreg[i][j] = (T)0.f;
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t o = offk[i] < limk ? offk[i] : limk;
+      cg[i] = *(const g4*)(gb + (o << GSH));
+      cq[i] = *(const v4*)(qb + o);
+      ck[i] = *(const v4*)(kb_ + o);
     }
   }
   // operand fragments: wave (rw, cw) produces rows 32rw.., key columns kb + 32cw..
   const int rw = wave >> 1, cw = wave & 1;
   const int kt32 = kb / 32 + cw;
-  // ---- prefix sums of the gates over the 16 row groups
-  float G[4][4], glast[4];
-  {
-    float run[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        run[j] += gq[i][j];
-        G[i][j] = run[j];
-      }
-    *(f32x4*)&sPart[rg * 64 + c4] = f32x4{run[0], run[1], run[2], run[3]};
-    __syncthreads();
-    float off[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) glast[j] = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      f32x4 pr = *(const f32x4*)&sPart[r * 64 + c4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if (r < rg) off[j] += pr[j];
-        glast[j] += pr[j];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) G[i][j] += off[j];
-  }
-  // ---- operand tiles
-#pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
-    *(v8*)&sDo[row * LDV + c8] = dreg[i];
-    *(v8*)&sV[row * LDV + c8] = vreg[i];
-  }
-  float einv[4][4];  // e^{-G}, clamped
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) einv[i][j] = __expf(fminf(-G[i][j], InvDecayLimit<T>::value));
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    v4 kt, qt;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      kt[i] = (T)(kk[i][j] * einv[i][j]);
-      qt[i] = (T)(qq[i][j] * __expf(G[i][j]));
-    }
-    *(v4*)&sKtT[(c4 + j) * LDT + rg * 4] = kt;
-    *(v4*)&sQtT[(c4 + j) * LDT + rg * 4] = qt;
-  }
-  __syncthreads();
-  // state fragments for the inter-chunk terms: issued here, consumed after the score phase
   v8 hf[VT32][2], dhf[VT32][2];
   {
-    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V;
+    const int64_t blk = (cl.cglob * H + hh) * (int64_t)K * V * (int64_t)sizeof(T);
+    const char* hb = (const char*)p.hT + blk;
+    const char* dhb = (const char*)p.dhtf + blk;
 #pragma unroll
     for (int vt = 0; vt < VT32; ++vt) {
-      int64_t o = blk + (((int64_t)vt * (K / 32) + kt32) * 64 + lane) * 16;
-      hf[vt][0] = *(const v8*)((const T*)p.hT + o);
-      hf[vt][1] = *(const v8*)((const T*)p.hT + o + 8);
-      dhf[vt][0] = *(const v8*)((const T*)p.dhtf + o);
-      dhf[vt][1] = *(const v8*)((const T*)p.dhtf + o + 8);
+      const uint32_t o = (uint32_t)(((vt * (K / 32) + kt32) * 64 + lane) * 16) * (uint32_t)sizeof(T);
+      hf[vt][0] = *(const v8*)(hb + o);
+      hf[vt][1] = *(const v8*)(hb + o + 16);
+      dhf[vt][0] = *(const v8*)(dhb + o);
+      dhf[vt][1] = *(const v8*)(dhb + o + 16);
     }
   }
+  __syncthreads();
   // ---- dA = tril(do v^T) in both orientations (each gives 8-byte LDS writes)
   {
     const int ib = wave >> 1, jb = wave & 1;
@@ -631,6 +634,54 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
       }
     }
   }
+  // ---- prefix sums of the gates over the 16 row groups (q, k of the slice stay in storage precision until
+  // the epilogue; rows past the end zero)
+  float G[4][4], glast[4];
+  {
+    const v4 z4 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = rg * 4 + i < L;
+      cq[i] = ok ? cq[i] : z4;
+      ck[i] = ok ? ck[i] : z4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        run[j] += ok ? (float)cg[i][j] : 0.f;
+        G[i][j] = run[j];
+      }
+    }
+    *(f32x4*)&sPart[rg * 64 + c4] = f32x4{run[0], run[1], run[2], run[3]};
+    __syncthreads();   // also publishes dA
+    float off[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) glast[j] = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      f32x4 pr = *(const f32x4*)&sPart[r * 64 + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (r < rg) off[j] += pr[j];
+        glast[j] += pr[j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) G[i][j] += off[j];
+  }
+  // ---- gated operand tiles
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v4 kt, qt;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      kt[i] = (T)((float)ck[i][j] * __expf(fminf(-G[i][j], InvDecayLimit<T>::value)));   // e^{-G}, clamped
+      qt[i] = (T)((float)cq[i][j] * __expf(G[i][j]));
+    }
+    *(v4*)&sKtT[(c4 + j) * LDT + rg * 4] = kt;
+    *(v4*)&sQtT[(c4 + j) * LDT + rg * 4] = qt;
+  }
   __syncthreads();
   // ---- accumulate: dq (intra + inter), dk intra, dk inter
   f32x16 aq = zero16(), ak1 = zero16(), ak2 = zero16();
@@ -662,6 +713,11 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     stB[o] = ak1[r];
     stC[o] = ak2[r];
   }
+  // the next item's first rows are requested now: the accumulators are in LDS, the epilogue needs few registers
+  const uint32_t nit = it + gridDim.x;
+  const bool more = nit < nitems;   // workgroup-uniform
+  const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it: no load under a branch)
+  request(nim, R);
   __syncthreads();
   // ---- epilogue in the load mapping (4 rows x 4 key channels per lane)
   float x[4][4], ksum[4] = {0.f, 0.f, 0.f, 0.f};
@@ -676,9 +732,10 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
     for (int j = 0; j < 4; ++j) {
       // (the gate factors go through an opaque copy: the rounded operands below are recomputed
       // here instead of being kept in registers from the staging step to this point)
-      float gij = G[i][j], ei = einv[i][j];
-      asm volatile("" : "+v"(gij), "+v"(ei));
-      const float eg = __expf(gij);
+      float gij = G[i][j];
+      asm volatile("" : "+v"(gij));
+      const float eg = __expf(gij), ei = __expf(fminf(-gij, InvDecayLimit<T>::value));
+      const float qf = (float)cq[i][j], kf = (float)ck[i][j];
       float dq = p.scale * eg * a[j];
       float dki = __expf(glast[j] - gij) * c[j];
       float dk = p.scale * ei * b[j] + dki;
@@ -688,10 +745,10 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
       // k*dk at row j and cancels unless it straddles the row.  Formed with the rounded operands
       // the matrix products used, the two copies are equal and cancel exactly; with strong gates,
       // where dg is small against either sum, this is what keeps its error at rounding level.
-      const float qr = (float)(T)(qq[i][j] * eg);
-      const float kr = (float)(T)(kk[i][j] * ei);
-      x[i][j] = p.scale * (qr * a[j] - kr * b[j]) - kk[i][j] * dki;
-      ksum[j] += kk[i][j] * dki;
+      const float qr = (float)(T)(qf * eg);
+      const float kr = (float)(T)(kf * ei);
+      x[i][j] = p.scale * (qr * a[j] - kr * b[j]) - kf * dki;
+      ksum[j] += kf * dki;
     }
     if (row < L) {
       int64_t off = ((row0 + row) * H + hh) * (int64_t)K + kb + c4;
@@ -712,15 +769,21 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
   *(f32x4*)&sPart2[rg * 64 + c4] = f32x4{ksum[0], ksum[1], ksum[2], ksum[3]};
   __syncthreads();
   float add[4] = {0.f, 0.f, 0.f, 0.f};
+  // (four row groups at a time: all 32 reads in flight at once would take 128 registers from the rows that
+  // are on their way for the next item)
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    f32x4 s1 = *(const f32x4*)&sPart[r * 64 + c4];
-    f32x4 s2 = *(const f32x4*)&sPart2[r * 64 + c4];
+  for (int r0 = 0; r0 < 16; r0 += 4) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      if (r > rg) add[j] += s1[j];
-      add[j] += s2[j];
+    for (int r = r0; r < r0 + 4; ++r) {
+      f32x4 s1 = *(const f32x4*)&sPart[r * 64 + c4];
+      f32x4 s2 = *(const f32x4*)&sPart2[r * 64 + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (r > rg) add[j] += s1[j];
+        add[j] += s2[j];
+      }
     }
+    __builtin_amdgcn_sched_barrier(0);
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) add[j] += __expf(glast[j]) * sHd[c4 + j];
@@ -731,6 +794,11 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p) {
       f32x4 o = {x[i][0] + add[0], x[i][1] + add[1], x[i][2] + add[2], x[i][3] + add[3]};
       *(f32x4*)(p.dg + ((row0 + row) * H + hh) * (int64_t)K + kb + c4) = o;
     }
+  }
+  if (!more) break;
+  __syncthreads();  // the staging tiles are consumed: the next item's operand tiles may be written
+  it = nit;
+  im = nim;
   }
 }
 
@@ -939,11 +1007,12 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   {
     BDqkgParams p{q, k, v, g, dout, hT, dhtf, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
                   (int)H, (int)K, ntfix, scale};
-    const int64_t nwg = (int64_t)grid.x * grid.y * (K / 64);
+    // as many workgroups as are resident at once (two per CU), each walking its share of the items
+    const int64_t pairs = (int64_t)grid.x * grid.y, nwg = pairs * (K / 64);
     FLA_REQUIRE(nwg <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
-    dim3 g3((unsigned)nwg);
-    if (V == 64) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 64>), g3, dim3(256), 0, st, p);
-    else if (V == 128) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 128>), g3, dim3(256), 0, st, p);
+    dim3 g3((unsigned)(nwg < 2 * kNumCUs ? nwg : 2 * kNumCUs));
+    if (V == 64) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 64>), g3, dim3(256), 0, st, p, pairs);
+    else if (V == 128) hipLaunchKernelGGL((gla_bwd_dqkg_kernel<T, GT, 128>), g3, dim3(256), 0, st, p, pairs);
     else return FLA_E_UNSUPPORTED;
     FLA_CHECK_LAUNCH();
   }
