@@ -147,6 +147,21 @@ inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B,
   return FLA_OK;
 }
 
+// Workgroups of `kernel` (256 threads, no dynamic LDS) that the chip holds at once: the grid of a kernel whose
+// workgroups walk many items each.  Asked of the runtime once per kernel.
+template <typename Kern>
+inline int64_t resident_workgroups(Kern kernel) {
+  static int per_cu = 0;   // one instance per kernel type and address: callers pass distinct instantiations
+  static const void* cached = nullptr;
+  if (cached != (const void*)kernel) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) n = 1;
+    per_cu = n;
+    cached = (const void*)kernel;
+  }
+  return (int64_t)per_cu * kNumCUs;
+}
+
 // dst = src (or zeros when src is NULL), n floats: what the state gradient of a batch without any
 // chunk is (d initial_state = d final_state).  A kernel rather than a memset / memcpy call, so that
 // the launch can sit in a captured graph like the rest.

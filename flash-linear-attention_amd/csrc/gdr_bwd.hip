@@ -49,7 +49,7 @@ struct DvlParams {
 };
 
 template <typename T, int K, int V>
-__global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
+__global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p, uint32_t nitems) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
@@ -62,42 +62,87 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   __shared__ __attribute__((aligned(16))) T sDt[V * LDT];
   __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];
   __shared__ float sGam[BT];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x;
   const int H = p.H;
-  int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
-  const int L = cl.L;
-  const int64_t row0 = cl.row0;
+  // A workgroup walks (chunk, head) items with a stride of the grid size; the rows of the next item are
+  // requested as soon as those of the current one are in LDS (32-bit offsets off wave-uniform bases; rows past
+  // the end of a short chunk re-read its last row and are masked at use, so no load sits under a branch).
+  struct Item {
+    ChunkLoc cl;
+    int hh;
+  };
+  auto locate = [&](uint32_t it) {
+    Item r;
+    r.cl = locate_chunk_at32(it, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    return r;
+  };
+  struct Raw {
+    v8 q[NP], k[NP];
+    v4 d[RPTV];
+    float gam;
+  };
+  const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
+  uint32_t offk[NP], offv[RPTV];
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
-    v8 qv, kv;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c8;
-      qv = *(const v8*)((const T*)p.q + off);
-      kv = *(const v8*)((const T*)p.k + off);
-    } else {
+    const int e = tid0 + 256 * i;
+    offk[i] = (uint32_t)(e / C8) * pitchk + (uint32_t)((e % C8) * 8) * (uint32_t)sizeof(T);
+  }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qv[j] = kv[j] = (T)0.f;
+  for (int i = 0; i < RPTV; ++i)
+    offv[i] = (uint32_t)((tid0 / CGV) * RPTV + i) * pitchv + (uint32_t)((tid0 % CGV) * 4) * (uint32_t)sizeof(T);
+  const uint32_t colk = (uint32_t)((tid0 % C8) * 8) * (uint32_t)sizeof(T), colv = (uint32_t)((tid0 % CGV) * 4) * (uint32_t)sizeof(T);
+  auto request = [&](const Item& im, Raw& R) __attribute__((always_inline)) {
+    const uint32_t last = (uint32_t)(im.cl.L - 1);
+    const int64_t r0h = im.cl.row0 * H + im.hh;
+    const char* qb = (const char*)p.q + r0h * K * (int64_t)sizeof(T);
+    const char* kb = (const char*)p.k + r0h * K * (int64_t)sizeof(T);
+    const char* db = (const char*)p.dout + r0h * V * (int64_t)sizeof(T);
+    const uint32_t limk = last * pitchk + colk, limv = last * pitchv + colv;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const uint32_t o = offk[i] < limk ? offk[i] : limk;
+      R.q[i] = *(const v8*)(qb + o);
+      R.k[i] = *(const v8*)(kb + o);
     }
-    *(v8*)&sQ[row * LDK + c8] = qv;
-    *(v8*)&sK[row * LDK + c8] = kv;
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) R.d[i] = *(const v4*)(db + (offv[i] < limv ? offv[i] : limv));
+    const uint32_t grow = (uint32_t)(tid0 & (BT - 1)) < last ? (uint32_t)(tid0 & (BT - 1)) : last;
+    R.gam = p.gam ? p.gam[(im.cl.row0 + grow) * H + im.hh] : 0.f;
+  };
+  uint32_t it = blockIdx.x;
+  if (it >= nitems) return;
+  Item im = locate(it);
+  Raw R;
+  request(im, R);
+  const v8 z8 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+  for (;;) {
+  // (the lane id goes through an opaque copy once per item, so that the LDS addresses of the body are formed
+  // where they are used instead of being hoisted out of the loop into long-lived registers)
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hh = im.hh;
+  const int L = im.cl.L;
+  const int64_t row0 = im.cl.row0;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
+    *(v8*)&sQ[row * LDK + c8] = row < L ? R.q[i] : z8;
+    *(v8*)&sK[row * LDK + c8] = row < L ? R.k[i] : z8;
   }
   const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
-  v4 dreg[RPTV];
-#pragma unroll
-  for (int i = 0; i < RPTV; ++i) {
-    int row = rgv * RPTV + i;
-    if (row < L) dreg[i] = *(const v4*)((const T*)p.dout + ((row0 + row) * H + hh) * (int64_t)V + cv4);
-    else dreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     T* dst = &sDt[(cv4 + j) * LDT + rgv * RPTV];
 #pragma unroll
-    for (int i = 0; i < RPTV; ++i) dst[i] = dreg[i][j];
+    for (int i = 0; i < RPTV; ++i) dst[i] = rgv * RPTV + i < L ? R.d[i][j] : (T)0.f;
   }
-  if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
+  if (tid < BT) sGam[tid] = R.gam;
+  const uint32_t nit = it + gridDim.x;
+  const bool more = nit < nitems;   // workgroup-uniform
+  const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it)
+  request(nim, R);
   __syncthreads();
   {
     const int qi = wave >> 1, qj = wave & 1;
@@ -152,6 +197,11 @@ __global__ __launch_bounds__(256) void gdr_bwd_dvlocal_kernel(DvlParams p) {
   for (int i = 0; i < BT * C8V / 256; ++i) {
     const int e = tid + 256 * i, row = e / C8V, c8 = (e % C8V) * 8;
     if (row < L) *(v8*)(op + (int64_t)row * H * V + c8) = *(const v8*)&sO[row * LDV + c8];
+  }
+  if (!more) break;
+  __syncthreads();  // the dv tile is on its way: the next item's tiles may be written
+  it = nit;
+  im = nim;
   }
 }
 
@@ -1186,7 +1236,15 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
 
 template <typename T>
 int launch_dv_local(const DvlParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
-#define L1(KK, VV) hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+  // as many workgroups as are resident at once, each walking its share of the (chunk, head) items
+  const int64_t total = (int64_t)grid.x * grid.y;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+#define L1(KK, VV)                                                                                        \
+  {                                                                                                       \
+    const int64_t res = resident_workgroups(gdr_bwd_dvlocal_kernel<T, KK, VV>);                           \
+    hipLaunchKernelGGL((gdr_bwd_dvlocal_kernel<T, KK, VV>), dim3((unsigned)(total < res ? total : res)), dim3(256), 0, st, \
+                       p, (uint32_t)total);                                                               \
+  }
   FLA_KV(L1)
 #undef L1
   FLA_CHECK_LAUNCH();
