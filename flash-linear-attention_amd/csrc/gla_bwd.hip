@@ -236,7 +236,7 @@ struct BDvParams {
 };
 
 template <typename T, typename GT, int K, int V>
-__global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
+__global__ __launch_bounds__(256, 2) void gla_bwd_dv_kernel(BDvParams p, uint32_t nitems) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
@@ -250,10 +250,65 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   __shared__ __attribute__((aligned(16))) T sPT[BT * LDT];   // A^T [j][i]
   __shared__ __attribute__((aligned(16))) float sPart[RG * K];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x;
   const int H = p.H;
-  int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  // A workgroup walks (chunk, head) items with a stride of the grid size; the q, k, g and do rows of the next
+  // item are requested as soon as those of the current one are in LDS (32-bit offsets off wave-uniform bases;
+  // rows past the end of a short chunk re-read its last row and are masked at use, so no load sits under a
+  // branch).
+  struct Item {
+    ChunkLoc cl;
+    int hh;
+  };
+  auto locate = [&](uint32_t it) {
+    Item r;
+    r.cl = locate_chunk_at32(it, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    return r;
+  };
+  typedef GT g4 __attribute__((ext_vector_type(4)));
+  struct Raw {
+    g4 g[RPT];
+    v4 q[RPT], k[RPT], d[RPTV];
+  };
+  constexpr int GSH = sizeof(GT) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
+  const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
+  const uint32_t colk = (uint32_t)((tid0 % CG) * 4) * (uint32_t)sizeof(T), colv = (uint32_t)((tid0 % CGV) * 4) * (uint32_t)sizeof(T);
+  uint32_t offk[RPT], offv[RPTV];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) offk[i] = (uint32_t)((tid0 / CG) * RPT + i) * pitchk + colk;
+#pragma unroll
+  for (int i = 0; i < RPTV; ++i) offv[i] = (uint32_t)((tid0 / CGV) * RPTV + i) * pitchv + colv;
+  auto request = [&](const Item& im, Raw& R) __attribute__((always_inline)) {
+    const uint32_t last = (uint32_t)(im.cl.L - 1);
+    const int64_t r0h = im.cl.row0 * H + im.hh;
+    const char* qb = (const char*)p.q + r0h * K * (int64_t)sizeof(T);
+    const char* kb = (const char*)p.k + r0h * K * (int64_t)sizeof(T);
+    const char* gb = (const char*)p.g + r0h * K * (int64_t)sizeof(GT);
+    const char* db = (const char*)p.dout + r0h * V * (int64_t)sizeof(T);
+    const uint32_t limk = last * pitchk + colk, limv = last * pitchv + colv;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const uint32_t o = offk[i] < limk ? offk[i] : limk;
+      R.g[i] = *(const g4*)(gb + (o << GSH));
+      R.q[i] = *(const v4*)(qb + o);
+      R.k[i] = *(const v4*)(kb + o);
+    }
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) R.d[i] = *(const v4*)(db + (offv[i] < limv ? offv[i] : limv));
+  };
+  uint32_t it = blockIdx.x;
+  if (it >= nitems) return;
+  Item im = locate(it);
+  Raw R;
+  request(im, R);
+  for (;;) {
+  // (the lane id goes through an opaque copy once per item, so that the LDS addresses of the body are formed
+  // where they are used instead of being hoisted out of the loop into long-lived registers)
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hh = im.hh;
+  const ChunkLoc cl = im.cl;
   const int L = cl.L;
   const int64_t row0 = cl.row0;
 
@@ -264,39 +319,19 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   float gq[RPT][4], qq[RPT][4], kk[RPT][4];
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
-    int row = rg * RPT + i;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
-      Load<GT>::x4((const GT*)p.g + off, gq[i]);
-      Load<T>::x4((const T*)p.q + off, qq[i]);
-      Load<T>::x4((const T*)p.k + off, kk[i]);
-    } else {
+    const bool ok = rg * RPT + i < L;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) gq[i][j] = qq[i][j] = kk[i][j] = 0.f;
+    for (int j = 0; j < 4; ++j) {
+      gq[i][j] = ok ? (float)R.g[i][j] : 0.f;
+      qq[i][j] = ok ? (float)R.q[i][j] : 0.f;
+      kk[i][j] = ok ? (float)R.k[i][j] : 0.f;
     }
   }
   const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
   v4 dreg[RPTV];
 #pragma unroll
-  for (int i = 0; i < RPTV; ++i) {
-    int row = rgv * RPTV + i;
-    if (row < L) dreg[i] = *(const v4*)((const T*)p.dout + ((row0 + row) * H + hh) * (int64_t)V + cv4);
-    else dreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-  }
+  for (int i = 0; i < RPTV; ++i) dreg[i] = rgv * RPTV + i < L ? R.d[i] : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
   const int rw = wave >> 1, cw = wave & 1;
-  // dH tiles as stored: rows v, columns k (a lane holds one key column)
-  v8 hf[KT32][TV][2];
-  {
-    const T* hp = (const T*)p.dhtf + (cl.cglob * H + hh) * (int64_t)K * V;
-#pragma unroll
-    for (int kt = 0; kt < KT32; ++kt)
-#pragma unroll
-      for (int tv = 0; tv < TV; ++tv) {
-        const T* f = hp + (((int64_t)(cw * TV + tv) * KT32 + kt) * 64 + lane) * 16;
-        hf[kt][tv][0] = *(const v8*)f;
-        hf[kt][tv][1] = *(const v8*)(f + 8);
-      }
-  }
   // ---- prefix sums and G_last
   float G[RPT][4], glast[4];
   {
@@ -345,6 +380,23 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
     T* dst = &sDt[(cv4 + j) * LDT + rgv * RPTV];
 #pragma unroll
     for (int i = 0; i < RPTV; ++i) dst[i] = dreg[i][j];
+  }
+  const uint32_t nit = it + gridDim.x;
+  const bool more = nit < nitems;   // workgroup-uniform
+  const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it)
+  request(nim, R);
+  // dH tiles as stored: rows v, columns k (a lane holds one key column); on their way during the score phase
+  v8 hf[KT32][TV][2];
+  {
+    const char* hp = (const char*)p.dhtf + (cl.cglob * H + hh) * (int64_t)K * V * (int64_t)sizeof(T);
+#pragma unroll
+    for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv) {
+        const uint32_t o = (uint32_t)((((cw * TV + tv) * KT32 + kt) * 64 + lane) * 16) * (uint32_t)sizeof(T);
+        hf[kt][tv][0] = *(const v8*)(hp + o);
+        hf[kt][tv][1] = *(const v8*)(hp + o + 16);
+      }
   }
   __syncthreads();
   // ---- A^T on the lower-triangular quadrants
@@ -429,6 +481,11 @@ __global__ __launch_bounds__(256) void gla_bwd_dv_kernel(BDvParams p) {
   for (int i = 0; i < BT * C8V / 256; ++i) {
     const int e = tid + 256 * i, row = e / C8V, c8 = (e % C8V) * 8;
     if (row < L) *(v8*)(op + (int64_t)row * H * V + c8) = *(const v8*)&sO[row * LDV + c8];
+  }
+  if (!more) break;
+  __syncthreads();  // the dv tile is on its way: the next item's tiles may be written
+  it = nit;
+  im = nim;
   }
 }
 
@@ -998,8 +1055,15 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   }
   {
     BDvParams p{q, k, g, dout, dhtf, wide, dv, offsets, indices, T_, (int)H, ntfix, scale};
+    // as many workgroups as are resident at once, each walking its share of the (chunk, head) items
+    const int64_t total = (int64_t)grid.x * grid.y;
+    FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
 #define FLA_CASE(KK, VV)                                                                            \
-  if (K == KK && V == VV) hipLaunchKernelGGL((gla_bwd_dv_kernel<T, GT, KK, VV>), grid, dim3(256), 0, st, p);
+  if (K == KK && V == VV) {                                                                         \
+    const int64_t res = resident_workgroups(gla_bwd_dv_kernel<T, GT, KK, VV>);                      \
+    hipLaunchKernelGGL((gla_bwd_dv_kernel<T, GT, KK, VV>), dim3((unsigned)(total < res ? total : res)), dim3(256), 0, st, p, \
+                       (uint32_t)total);                                                            \
+  }
     FLA_CASE(64, 64) else FLA_CASE(128, 128) else FLA_CASE(64, 128) else FLA_CASE(128, 64) else return FLA_E_UNSUPPORTED;
 #undef FLA_CASE
     FLA_CHECK_LAUNCH();
