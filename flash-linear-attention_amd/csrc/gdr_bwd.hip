@@ -930,7 +930,7 @@ struct TileIO {
 };
 
 template <typename T, int K, int V>
-__global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
+__global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwdParams p, uint32_t nitems) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int D = K > V ? K : V;
@@ -960,23 +960,84 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   // (two workgroups then fit a CU)
   T* sS2 = sRow1;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid0 = threadIdx.x;
   const int H = p.H;
-  int hh;
-  ChunkLoc cl = locate_chunk(p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+  // A workgroup walks (chunk, head) items with a stride of the grid size; the rows an item starts with (du, v,
+  // Aw, beta, gamma) are requested as soon as those of the item before it are in LDS (32-bit offsets off
+  // wave-uniform bases; rows past the end of a short chunk re-read its last row and are masked at use, so no
+  // load sits under a branch).
+  struct Item {
+    ChunkLoc cl;
+    int hh;
+  };
+  auto locate = [&](uint32_t it) {
+    Item r;
+    r.cl = locate_chunk_at32(it, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
+    return r;
+  };
+  struct Raw {
+    v4 du[IOV::RPT], v[IOV::RPT], a[IOA::RPT];
+    float beta, gam;
+  };
+  const uint32_t pitchv = (uint32_t)H * V * (uint32_t)sizeof(T), pitcha = (uint32_t)H * BT * (uint32_t)sizeof(T);
+  const uint32_t colv = (uint32_t)((tid0 % IOV::CG) * 4) * (uint32_t)sizeof(T), cola = (uint32_t)((tid0 % IOA::CG) * 4) * (uint32_t)sizeof(T);
+  uint32_t offv[IOV::RPT], offa[IOA::RPT];
+#pragma unroll
+  for (int i = 0; i < IOV::RPT; ++i) offv[i] = (uint32_t)((tid0 / IOV::CG) * IOV::RPT + i) * pitchv + colv;
+#pragma unroll
+  for (int i = 0; i < IOA::RPT; ++i) offa[i] = (uint32_t)((tid0 / IOA::CG) * IOA::RPT + i) * pitcha + cola;
+  auto request = [&](const Item& im, Raw& R) __attribute__((always_inline)) {
+    const uint32_t last = (uint32_t)(im.cl.L - 1);
+    const int64_t r0h = im.cl.row0 * H + im.hh;
+    const char* dub = (const char*)p.du + r0h * V * (int64_t)sizeof(T);
+    const char* vb = (const char*)p.v + r0h * V * (int64_t)sizeof(T);
+    const char* ab = (const char*)p.Aw + r0h * BT * (int64_t)sizeof(T);
+    const uint32_t limv = last * pitchv + colv, lima = last * pitcha + cola;
+#pragma unroll
+    for (int i = 0; i < IOV::RPT; ++i) {
+      const uint32_t o = offv[i] < limv ? offv[i] : limv;
+      R.du[i] = *(const v4*)(dub + o);
+      R.v[i] = *(const v4*)(vb + o);
+    }
+#pragma unroll
+    for (int i = 0; i < IOA::RPT; ++i) R.a[i] = *(const v4*)(ab + (offa[i] < lima ? offa[i] : lima));
+    const uint32_t row = (uint32_t)(tid0 & (BT - 1)) < last ? (uint32_t)(tid0 & (BT - 1)) : last;
+    R.beta = p.beta[(im.cl.row0 + row) * H + im.hh];
+    R.gam = p.gam ? p.gam[(im.cl.row0 + row) * H + im.hh] : 0.f;
+  };
+  uint32_t it = blockIdx.x;
+  if (it >= nitems) return;
+  Item im = locate(it);
+  Raw R;
+  request(im, R);
+  for (;;) {
+  // (the lane id goes through an opaque copy once per item, so that the LDS addresses of the body are formed
+  // where they are used instead of being hoisted out of the loop into long-lived registers)
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int hh = im.hh;
+  const ChunkLoc cl = im.cl;
   const int L = cl.L;
   const int64_t row0 = cl.row0;
   const int rw = wave >> 1, cw = wave & 1;
 
-  // ---- issue the loads of the value side and of Aw
+  // ---- the value side and Aw, rows past the end of the chunk zero (Aw: identity, below)
   v4 rdu[IOV::RPT], rv[IOV::RPT], ra[IOA::RPT];
-  IOV::load(p.du, row0, L, H, hh, tid, rdu);
-  IOV::load(p.v, row0, L, H, hh, tid, rv);
-  IOA::load(p.Aw, row0, L, H, hh, tid, ra);
+  {
+    const v4 z4 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+#pragma unroll
+    for (int i = 0; i < IOV::RPT; ++i) {
+      const bool ok = (tid / IOV::CG) * IOV::RPT + i < L;
+      rdu[i] = ok ? R.du[i] : z4;
+      rv[i] = ok ? R.v[i] : z4;
+    }
+#pragma unroll
+    for (int i = 0; i < IOA::RPT; ++i) ra[i] = R.a[i];
+  }
   if (tid < BT) {
-    bool ok = tid < L;
-    sBeta[tid] = ok ? p.beta[(row0 + tid) * H + hh] : 0.f;
-    sGam[tid] = p.gam ? p.gam[(row0 + (ok ? tid : L - 1)) * H + hh] : 0.f;
+    sBeta[tid] = tid < L ? R.beta : 0.f;
+    sGam[tid] = R.gam;
     // the quadrant above the diagonal contributes nothing: its slots stay zero
     slot(5, tid) = 0.f;
     slot(6, tid) = 0.f;
@@ -1001,6 +1062,10 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
   v4 rdw[IOK::RPT], rk[IOK::RPT];
   IOK::load(p.dw, row0, L, H, hh, tid, rdw);
   IOK::load(p.k, row0, L, H, hh, tid, rk);
+  const uint32_t nit = it + gridDim.x;
+  const bool more = nit < nitems;   // workgroup-uniform
+  const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it)
+  request(nim, R);
   __syncthreads();
   {
     // Au^T[j][i] = Aw^T[j][i] * e^{gamma_i - gamma_j}, i >= j
@@ -1223,6 +1288,11 @@ __global__ __launch_bounds__(256) void gdr_bwd_wy_kernel(WyBwdParams p) {
       if (row < L) *(v8*)((T*)p.dv + ((row0 + row) * H + hh) * (int64_t)V + c8) = *(const v8*)&sRow1[row * LDD + c8];
     }
   }
+  if (!more) break;
+  __syncthreads();  // dk and dv are on their way: the next item's tiles may be written
+  it = nit;
+  im = nim;
+  }
 }
 
 #define FLA_KV(STMT)                                   \
@@ -1281,7 +1351,15 @@ int launch_dqkwg(const DqkwgParams& p, int64_t V, dim3 grid, hipStream_t st) {
 
 template <typename T>
 int launch_wy_bwd(const WyBwdParams& p, int64_t K, int64_t V, dim3 grid, hipStream_t st) {
-#define L4(KK, VV) hipLaunchKernelGGL((gdr_bwd_wy_kernel<T, KK, VV>), grid, dim3(256), 0, st, p);
+  // as many workgroups as are resident at once, each walking its share of the (chunk, head) items
+  const int64_t total = (int64_t)grid.x * grid.y;
+  FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+#define L4(KK, VV)                                                                                   \
+  {                                                                                                  \
+    const int64_t res = resident_workgroups(gdr_bwd_wy_kernel<T, KK, VV>);                           \
+    hipLaunchKernelGGL((gdr_bwd_wy_kernel<T, KK, VV>), dim3((unsigned)(total < res ? total : res)), dim3(256), 0, st, p, \
+                       (uint32_t)total);                                                             \
+  }
   FLA_KV(L4)
 #undef L4
   FLA_CHECK_LAUNCH();
