@@ -877,6 +877,12 @@ struct WyBwdParams {
   const int64_t* indices;
   int64_t T;
   int H, NTfix;
+  // With dgam_part (fp32 [nparts, total_rows, H], the gate-gradient partial sums of the dq/dk/dw launch) dgam2
+  // receives the gradient of the raw gate itself: the reverse chunk-local cumulative sum of (sum of the parts +
+  // this launch's own terms), as chunk_local_cumsum(reverse=True) leaves it (fla/ops/gated_delta_rule/chunk.py:170-171).
+  const float* dgam_part;
+  int nparts;
+  int64_t total_rows;
 };
 
 // Transposed 64 x N product: acc[t] (+)= X^T-tile A^T, i.e. C[column][time row] with
@@ -1265,9 +1271,22 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
     if (lane < 32) slot(2 + cw, jrow) = part;
   }
   __syncthreads();  // every wave is past its last read of X1^T / dM^T, which share storage with the dv tile
-  if (tid < L) {
-    p.dbeta[(row0 + tid) * H + hh] = (slot(0, tid) + slot(1, tid)) + (slot(2, tid) + slot(3, tid));
-    p.dgam2[(row0 + tid) * H + hh] = (slot(4, tid) + slot(5, tid)) + (slot(6, tid) + slot(7, tid));
+  if (tid < BT) {   // wave 0: one row per lane
+    const bool ok = tid < L;
+    if (ok) p.dbeta[(row0 + tid) * H + hh] = (slot(0, tid) + slot(1, tid)) + (slot(2, tid) + slot(3, tid));
+    float dgm = ok ? (slot(4, tid) + slot(5, tid)) + (slot(6, tid) + slot(7, tid)) : 0.f;
+    if (p.dgam_part) {
+      for (int z = 0; z < p.nparts; ++z)
+        dgm += ok ? p.dgam_part[((int64_t)z * p.total_rows + row0 + tid) * H + hh] : 0.f;
+      // inclusive suffix sum over the 64 rows: DPP row scans plus the totals of the later rows of 16
+      float x = row_suffix16(dgm);
+      const float t1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 16));
+      const float t2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 32));
+      const float t3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 48));
+      const int r = lane >> 4;
+      dgm = x + (r < 1 ? t1 : 0.f) + (r < 2 ? t2 : 0.f) + (r < 3 ? t3 : 0.f);
+    }
+    if (ok) p.dgam2[(row0 + tid) * H + hh] = dgm;
   }
 #pragma unroll
   for (int t = 0; t < TV; ++t)
@@ -1386,7 +1405,8 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   DqkwgParams p3{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
                  B * T_, (int)H, (int)K, ntfix, scale};
   if ((rc = launch_dqkwg<T>(p3, V, grid, st))) return rc;
-  WyBwdParams p4{k, v, beta, gam, Aw, dw, dv2, dkp, dk, dv, dbeta, dgam2, offsets, indices, T_, (int)H, ntfix};
+  WyBwdParams p4{k, v, beta, gam, Aw, dw, dv2, dkp, dk, dv, dbeta, dgam2, offsets, indices, T_, (int)H, ntfix,
+                 gam ? dgam_part : nullptr, (int)(K / 64), B * T_};
   return launch_wy_bwd<T>(p4, K, V, grid, st);
 }
 
@@ -1495,7 +1515,7 @@ extern "C" int fla_bwd_prepare_wy_repr(const void* k, const void* v, const float
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  WyBwdParams p{k, v, beta, g_cumsum, Aw, dw, du, dk_in, dk, dv, dbeta, dg, offsets, indices, T, (int)H, ntfix};
+  WyBwdParams p{k, v, beta, g_cumsum, Aw, dw, du, dk_in, dk, dv, dbeta, dg, offsets, indices, T, (int)H, ntfix, nullptr, 0, 0};
   if (qkv_dtype == FLA_BF16) return launch_wy_bwd<bf16>(p, K, V, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_wy_bwd<f16>(p, K, V, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

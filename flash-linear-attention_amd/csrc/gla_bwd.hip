@@ -896,7 +896,14 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
   constexpr int VD_BYTES = 2 * BT * LDVV * 2;
   constexpr int X_BYTES = BT * LDG * 4;
   const int H = p.H;
-  // a few hundred workgroups walk the (chunk, head) flags (almost always none is set)
+  // A few hundred workgroups walk the (chunk, head) flags (almost always none is set).  The lanes first read
+  // all flags of the workgroup side by side (one memory latency instead of one per flag) and leave if none is set.
+  {
+    int any = 0;
+    for (int64_t lin = blockIdx.x + (int64_t)threadIdx.x * gridDim.x; lin < p.total; lin += (int64_t)256 * gridDim.x)
+      any |= p.wide[lin];
+    if (!__syncthreads_or(any)) return;
+  }
   for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
   if (p.wide[lin] == 0) continue;  // workgroup-uniform
   __syncthreads();                 // the tiles of the previous flagged chunk are free

@@ -134,21 +134,17 @@ def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do
     ws_dgam = q.new_empty(K // 64, B * T, H, dtype=torch.float32)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dbeta = q.new_empty(B, T, H, dtype=torch.float32)
-    dgam2 = q.new_empty(B, T, H, dtype=torch.float32)
+    dg = q.new_empty(B, T, H, dtype=torch.float32)   # the last launch sums the partials and takes the reverse cumsum
     dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
     if dht is not None:
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
     be.check(be.lib().fla_chunk_gated_delta_rule_bwd(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(w), be.ptr(v_new), be.ptr(beta), be.ptr(g_cumsum), be.ptr(Aw),
         be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(ws_dvl), be.ptr(ws_dv2), be.ptr(ws_dh), be.ptr(ws_dw),
-        be.ptr(ws_dkp), be.ptr(ws_dgam), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dbeta), be.ptr(dgam2),
+        be.ptr(ws_dkp), be.ptr(ws_dgam), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dbeta), be.ptr(dg),
         be.ptr(dh0), be.ptr(offs), be.ptr(idx), be.ptr(co), NT, be.dt(q), B, T, H, K, V, N, float(scale),
         be.stream_of(q)), "fla_chunk_gated_delta_rule_bwd")
-    dg = None
-    if g_cumsum is not None:
-        dgam = ws_dgam.sum(0).view(B, T, H) + dgam2
-        dg = chunk_local_cumsum(dgam, BT, reverse=True, offsets=offs, indices=idx, head_first=False)
-    return dq, dk, dv, dbeta, dg, dh0
+    return dq, dk, dv, dbeta, (dg if g_cumsum is not None else None), dh0
 
 
 class ChunkGatedDeltaRuleFunction(torch.autograd.Function):

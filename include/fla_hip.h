@@ -420,16 +420,18 @@ int fla_chunk_bwd_dv_local(const void* q, const void* k, const float* g_cumsum, 
  * states in FLA_H_FRAGMENT_T order).  g_cumsum fp32 [B,T,H] or NULL.
  * Workspaces: ws_dv_local, ws_dv2 like v; ws_dh_frag_t like hT; ws_dw,
  * ws_dk_partial like k; ws_dgam_partial fp32 [K/64, B*T, H].
- * Outputs: dq, dk [B,T,H,K], dv [B,T,H,V] (q/k/v dtype); dbeta and dgam2 fp32
- * [B,T,H]; dh0 fp32 [N,H,K,V] or NULL.  The gradient w.r.t. the raw gate is the
- * reverse chunk-local cumsum of (sum over slices of ws_dgam_partial) + dgam2.
+ * Outputs: dq, dk [B,T,H,K], dv [B,T,H,V] (q/k/v dtype); dbeta and dg fp32
+ * [B,T,H]; dh0 fp32 [N,H,K,V] or NULL.  dg is the gradient w.r.t. the raw gate: the last launch
+ * adds the slices of ws_dgam_partial to its own gate terms and takes the reverse chunk-local
+ * cumulative sum (the reference's chunk_local_cumsum(dg, reverse=True), chunk.py:170-171);
+ * without a gate (g_cumsum NULL) it holds nothing meaningful.
  * K in {64,128,256}, V in {64,128}.
  * ---------------------------------------------------------------------- */
 int fla_chunk_gated_delta_rule_bwd(
     const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,
     const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT,
     void* ws_dv_local, void* ws_dv2, void* ws_dh_frag_t, void* ws_dw, void* ws_dk_partial, float* ws_dgam_partial,
-    void* dq, void* dk, void* dv, float* dbeta, float* dgam2, float* dh0,
+    void* dq, void* dk, void* dv, float* dbeta, float* dg, float* dh0,
     const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
