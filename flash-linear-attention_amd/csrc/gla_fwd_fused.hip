@@ -26,9 +26,9 @@
 namespace {
 
 // NSTG: number of staging waves (4 or 8); the workgroup has 4 + NSTG waves.
-// HT: the matrix waves keep a transposed copy of their state tiles as well and write the state
-// entering every chunk to p.hT (what the backward kernels contract over v with), for a forward pass
-// whose states are kept instead of being recomputed by the backward pass.
+// HT: the matrix waves also write the state entering every chunk to p.hT, transposed (what the backward
+// kernels contract over v with), for a forward pass whose states are kept instead of being recomputed by
+// the backward pass.
 // SG: one log-gate per (token, head), p.g is fp32 [B*T, H] (the simple-GLA / RetNet-style decay): a lane loads one
 // word per row and uses it for all its key channels, so the prefix sums and exponentials of a row are formed once.
 template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false>
@@ -82,24 +82,33 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     // =========================== matrix waves ===========================
     const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
     f32x16 acc[NKT][2];                         // state tiles kt = wave + 4a, value tiles 0/1
-    f32x16 acct[HT ? NKT : 1][2];               // HT: the same tiles transposed (rows v, columns k)
 #pragma unroll
     for (int a = 0; a < NKT; ++a)
 #pragma unroll
       for (int vt = 0; vt < 2; ++vt) {
         acc[a][vt] = zero16();
-        if (HT) acct[a][vt] = zero16();
         int kt = wave + 4 * a;
         if (p.h0 && kt < KT32) {
           const float* h0p = p.h0 + (int64_t)nh * K * V;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
+          for (int r = 0; r < 16; ++r)
             acc[a][vt][r] = h0p[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + vt * 32 + (lane & 31)];
-            if (HT) acct[a][vt][r] = h0p[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + vt * 32 + c32_row(r, lane)];
-          }
         }
       }
-    // HT: state entering chunk c, transposed fragment order, straight from the accumulators
+    // HT: the state entering chunk c in transposed fragment order (rows v, columns k: what the backward kernels
+    // contract over v with).  A tile in accumulator order, converted to 16 bits and read as the first operand, is
+    // its own transpose (lane = row index of the product, registers = contraction index in accumulator-row
+    // order); multiplied by the identity in the same permuted order the product comes out in accumulator order
+    // with lanes and registers exchanged: two matrix instructions per tile instead of a second set of
+    // accumulators that is updated alongside the first.
+    v8 eye[2];
+    if constexpr (HT) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          eye[half][e] = (T)(((lane & 31) == 16 * half + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) ? 1.f : 0.f);
+    }
     auto store_ht = [&](int64_t c) {
       if constexpr (HT) {
         T* hb = (T*)p.hT + ((chunk0 + c) * H + hh) * (int64_t)K * V;
@@ -112,8 +121,15 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
               v8 lo, hi;
 #pragma unroll
               for (int r = 0; r < 8; ++r) {
-                lo[r] = (T)acct[a][vt][r];
-                hi[r] = (T)acct[a][vt][r + 8];
+                lo[r] = (T)acc[a][vt][r];
+                hi[r] = (T)acc[a][vt][r + 8];
+              }
+              f32x16 t = Elem<T>::mfma32(lo, eye[0], zero16());
+              t = Elem<T>::mfma32(hi, eye[1], t);
+#pragma unroll
+              for (int r = 0; r < 8; ++r) {
+                lo[r] = (T)t[r];
+                hi[r] = (T)t[r + 8];
               }
               T* dst = hb + (((int64_t)(vbase / 32 + vt) * (K / 32) + kt) * 64 + lane) * 16;
               *(v8*)dst = lo;
@@ -290,24 +306,12 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
               acc[a][1][4 * q4 + b] *= d[b];
             }
           }
-          if (HT) {
-            const float dcol = sDecay[buf][kt * 32 + (lane & 31)];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              acct[a][0][r] *= dcol;
-              acct[a][1][r] *= dcol;
-            }
-          }
 #pragma unroll
           for (int ts = 0; ts < BT; ts += 16) {
             v8 fk = lds_frag32<T>(sKh[buf], LDT, kt * 32, ts, lane);
             v8 fv0 = lds_frag32<T>(sVt[buf], LDT, 0, ts, lane), fv1 = lds_frag32<T>(sVt[buf], LDT, 32, ts, lane);
             acc[a][0] = Elem<T>::mfma32(fk, fv0, acc[a][0]);
             acc[a][1] = Elem<T>::mfma32(fk, fv1, acc[a][1]);
-            if (HT) {
-              acct[a][0] = Elem<T>::mfma32(fv0, fk, acct[a][0]);
-              acct[a][1] = Elem<T>::mfma32(fv1, fk, acct[a][1]);
-            }
           }
         }
       }
