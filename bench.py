@@ -34,7 +34,8 @@ for _p in (ROOT, os.path.join(ROOT, "flash-linear-attention_amd")):
 MFMA_PEAK_FLOPS = 2.5e15   # dense bf16 MFMA, FLOP/s
 HBM_PEAK_GBS = 8000.0
 MIB = 1 << 20
-RAMP_SECONDS = 0.5         # untimed load ahead of the warm-up steps (clock ramp)
+RAMP_SECONDS = 0.5         # untimed load ahead of the warm-up steps (clock ramp): at least this long ...
+RAMP_MAX_SECONDS = 4.0     # ... and at most this long, until the step time has settled
 
 
 def _events(n):
@@ -42,13 +43,25 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
-def event_stats(fn, steps, warmup=3):
+ROW_RAMP_SECONDS = 0.2     # untimed load ahead of every timed row other than the headline step
+
+
+def event_stats(fn, steps, warmup=3, ramp=None):
     """Device time of one call from HIP events recorded on the launch stream around every call:
     median, min, max and mean in microseconds, the number of intervals longer than twice the median
     (a stalled launch: clock ramp, an allocation, something else on the box) and the wall time of the
-    whole timed loop, which is bracketed by synchronize on both sides."""
+    whole timed loop, which is bracketed by synchronize on both sides.  The setup of a row (allocations,
+    first calls) leaves the device idle for milliseconds and its clocks drop; `ramp` seconds of the call
+    itself run untimed first, so that a 20-launch row and a 200-launch row report the same figure."""
     import statistics
     import torch
+    if ramp is None:
+        ramp = ROW_RAMP_SECONDS
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < ramp:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     ev = _events(2 * steps)
@@ -72,9 +85,9 @@ def spread(st):
             "n_over_2x_median": st["n_over_2x_median"]}
 
 
-def event_avg_us(fn, steps, warmup=3):
+def event_avg_us(fn, steps, warmup=3, ramp=None):
     """Median device time of one call (see event_stats)."""
-    return event_stats(fn, steps, warmup)["median_us"]
+    return event_stats(fn, steps, warmup, ramp)["median_us"]
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
@@ -122,19 +135,30 @@ def bench_gla(device, steps, warmup):
     def step():
         return chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
 
-    # The clocks of an idle GPU need a few hundred milliseconds of load to reach their steady state (the
-    # first launches after idle run about 25 % slower): keep the device busy with the step itself for
-    # RAMP_SECONDS before the warm-up steps, whatever --warmup says.
-    t_ramp = time.perf_counter()
-    while time.perf_counter() - t_ramp < RAMP_SECONDS:
-        for _ in range(20):
-            step()
-        torch.cuda.synchronize()
+    # The clocks of an idle GPU need load to reach their steady state (the first launches after idle run about
+    # 25 % slower, and on a box whose first GPU process this is the ramp takes longer than on a warm one): keep
+    # the device busy with the step itself for at least RAMP_SECONDS before the warm-up steps, whatever --warmup
+    # says, and on until two consecutive batches of 50 steps take the same time within 1 % (at most
+    # RAMP_MAX_SECONDS).
+    if RAMP_SECONDS > 0:
+        t_ramp = time.perf_counter()
+        prev = None
+        while True:
+            t_b = time.perf_counter()
+            for _ in range(50):
+                step()
+            torch.cuda.synchronize()
+            now = time.perf_counter()
+            cur = now - t_b
+            steady = prev is not None and abs(cur - prev) <= 0.01 * prev
+            if now - t_ramp >= RAMP_MAX_SECONDS or (steady and now - t_ramp >= RAMP_SECONDS):
+                break
+            prev = cur
 
     # `warmup` untimed steps, then exactly `steps` steps between two synchronisations, each step between
     # two HIP events on the launch stream.  value = tokens / median step time; the wall time of the same
     # loop and the spread of the intervals are reported beside it.
-    st = event_stats(step, steps, warmup)
+    st = event_stats(step, steps, warmup, ramp=0.0)   # ramped above
     ms = st["median_us"] * 1e-3
     tokens_per_s = B * T / (st["median_us"] * 1e-6)
 
@@ -554,6 +578,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--no-ramp", action="store_true",
+                    help="skip the untimed clock-ramp load (for counter-collection runs, whose timings are not used)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic, used to scale the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -567,6 +593,9 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     device = torch.device("cuda:0")
+    if a.no_ramp:
+        global RAMP_SECONDS, ROW_RAMP_SECONDS
+        RAMP_SECONDS = ROW_RAMP_SECONDS = 0.0
     ms, tps, roofline, op, cfg = bench_gla(device, a.steps, a.warmup)
     extra = {"chunk_gla_fwd": op}
     if not a.no_extra:
