@@ -34,8 +34,8 @@ for _p in (ROOT, os.path.join(ROOT, "flash-linear-attention_amd")):
 MFMA_PEAK_FLOPS = 2.5e15   # dense bf16 MFMA, FLOP/s
 HBM_PEAK_GBS = 8000.0
 MIB = 1 << 20
-RAMP_SECONDS = 0.5         # untimed load ahead of the warm-up steps (clock ramp): at least this long ...
-RAMP_MAX_SECONDS = 4.0     # ... and at most this long, until the step time has settled
+RAMP_SECONDS = 1.0         # untimed load ahead of the warm-up steps (clock ramp): at least this long ...
+RAMP_MAX_SECONDS = 5.0     # ... and at most this long, until the step time has settled
 
 
 def _events(n):
@@ -138,22 +138,22 @@ def bench_gla(device, steps, warmup):
     # The clocks of an idle GPU need load to reach their steady state (the first launches after idle run about
     # 25 % slower, and on a box whose first GPU process this is the ramp takes longer than on a warm one): keep
     # the device busy with the step itself for at least RAMP_SECONDS before the warm-up steps, whatever --warmup
-    # says, and on until two consecutive batches of 50 steps take the same time within 1 % (at most
+    # says, and on until three consecutive batches of 50 steps take the same time within 0.5 % (at most
     # RAMP_MAX_SECONDS).
     if RAMP_SECONDS > 0:
         t_ramp = time.perf_counter()
-        prev = None
+        hist = []
         while True:
             t_b = time.perf_counter()
             for _ in range(50):
                 step()
             torch.cuda.synchronize()
             now = time.perf_counter()
-            cur = now - t_b
-            steady = prev is not None and abs(cur - prev) <= 0.01 * prev
+            hist.append(now - t_b)
+            last = hist[-3:]
+            steady = len(last) == 3 and max(last) - min(last) <= 0.005 * min(last)
             if now - t_ramp >= RAMP_MAX_SECONDS or (steady and now - t_ramp >= RAMP_SECONDS):
                 break
-            prev = cur
 
     # `warmup` untimed steps, then exactly `steps` steps between two synchronisations, each step between
     # two HIP events on the launch stream.  value = tokens / median step time; the wall time of the same
