@@ -5,9 +5,10 @@
 // per (chunk, head) that fla_gdr_fwd_prep leaves: Tu = (Aw * Gamma) diag(beta) and the gated causal
 // scores Aqk.  One workgroup of 8 waves owns one (sequence, head, 64 value columns) and walks the
 // chunks serially:
-//   waves 4-7 ("staging")  copy k, q and the triangular tiles of chunk c+1 to LDS, transpose k and v
-//                          into time-contiguous tiles, and write the finished o tile of chunk c-1 to
-//                          global memory;
+//   waves 4-7 ("staging")  copy k, q and the triangular tiles of chunk c+1 to LDS, transpose v into a
+//                          time-contiguous tile, and write the finished o tile of chunk c-1 to global
+//                          memory (k is staged row-major only: the state update reads its transposed
+//                          operand from that tile with the transposing LDS load);
 //   waves 0-3 ("matrix")   each own 16 value columns of the fp32 state (all K rows, in 16x16
 //                          accumulator tiles).  The delta rule is independent per value column, so a
 //                          matrix wave never exchanges data with another:
@@ -86,6 +87,21 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
   return __builtin_bit_cast(v8, u4{lo[0], hi[0], lo[1], hi[1]});
 }
 
+// A operand of the state update (16 key rows x 32 time steps in accumulator-row order) read from the row-major
+// k tile [t][k]: the transposing LDS read hands lane j of a 16-lane group the four time rows whose 8-byte pieces
+// the group's lanes 4i .. 4i+3 address, so no transposed copy of k is staged.
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag16_tr(const T* tile, int ld, int k0, int t0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef short s4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const int j = lane & 15, g = lane >> 4;
+  const T* p0 = tile + (t0 + 4 * g + (j >> 2)) * ld + k0 + 4 * (j & 3);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 16 * ld));
+  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 template <typename T, int K, bool KEEP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
@@ -97,7 +113,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
   __shared__ __attribute__((aligned(16))) T sK[2][BT * LDR];     // k    [t][k]
   __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDR];     // q    [t][k]
-  __shared__ __attribute__((aligned(16))) T sKt[2][K * LDT];     // k^T  [k][t]
   __shared__ __attribute__((aligned(16))) T sVt[2][BV * LDT];    // v^T  [v][t], later o^T
   __shared__ __attribute__((aligned(16))) T sAT[2][2 * kTriElems];  // Tu, Aqk (packed triangular tiles)
   __shared__ __attribute__((aligned(16))) float sEg[2][BT];      // e^{gamma_t}
@@ -124,28 +139,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (nchunks == 0) return;
     const int st = tid - 256;
     constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (q)
-    constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;  // k: a lane owns RPT rows x 4 columns
     constexpr int NPA = 2 * kTriElems / 4 / 256;             // 8-byte pieces of the triangular tiles per lane
     static_assert(NPA * 256 * 4 == 2 * kTriElems, "the triangular tiles split evenly over the staging lanes");
-    const int rg = st / CG, c4 = (st % CG) * 4;
     const int urg = st >> 4, uc4 = (st & 15) * 4;            // v, o: a lane owns 4 rows x 4 columns
     const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
     auto q_row = [&](int e) { return e / C8; };
     auto q_col = [&](int e) { return (e % C8) * 8; };
     struct Regs {
-      v8 q[NPW];
+      v8 q[NPW], k[NPW];
       v4 a[NPA];
-      v4 k[RPT], v[4];
+      v4 v[4];
       uint32_t gam;  // fp32 bits
     };
     // The steady state carries no address arithmetic: byte offsets of this lane's pieces from the
-    // chunk's first row are computed once, the chunk base pointers advance by constant strides, and
-    // only a sequence's last, short chunk takes the masked path.
-    uint32_t offq[NPW], offk[RPT], offv[4];
+    // chunk's first row are computed once and the chunk base pointers advance by constant strides.
+    uint32_t offq[NPW], offv[4];
 #pragma unroll
     for (int i = 0; i < NPW; ++i) offq[i] = 2 * ((uint32_t)q_row(st + 256 * i) * HK + q_col(st + 256 * i));
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) offk[i] = 2 * ((uint32_t)(rg * RPT + i) * HK + c4);
 #pragma unroll
     for (int i = 0; i < 4; ++i) offv[i] = 2 * ((uint32_t)(urg * 4 + i) * HV + uc4);
     const uint32_t offg = 4 * (uint32_t)lane * H;
@@ -163,89 +173,71 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int64_t stra = (int64_t)H * (2 * kTriElems) * 2;
     const int64_t strg = p.gam ? (int64_t)BT * H * 4 : 0;
     const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
-    int lc = 0;  // next chunk to load
+    // Every memory operation of the steady state is unconditional: the wait counts the compiler places
+    // in front of a register's first use then count the loads of the other register sets and the output
+    // stores issued since as still in flight.  (With a load or store under a branch it has to assume the
+    // path that skipped it, and the wave waits for everything it issued, the stores of a moment ago
+    // included.)  Rows past the end of a sequence's last chunk are redirected to its last row by one
+    // unsigned minimum per load (zeroed before use), and past the last chunk the pointers stay on it.
+    const uint32_t limq_full = 2 * ((uint32_t)(BT - 1) * HK), limq_last = 2 * ((uint32_t)(Llast - 1) * HK);
+    const uint32_t limv_full = 2 * ((uint32_t)(BT - 1) * HV), limv_last = 2 * ((uint32_t)(Llast - 1) * HV);
+    const uint32_t colq = 2 * (uint32_t)q_col(st), colv = 2 * (uint32_t)uc4;
+    int lc = 0;  // chunk the load pointers are on
     auto load = [&](Regs& R) __attribute__((always_inline)) {
+      const bool last = lc >= nchunks - 1;
+      const uint32_t limq = (last ? limq_last : limq_full) + colq, limv = (last ? limv_last : limv_full) + colv;
+      const uint32_t limg = 4 * (uint32_t)((last ? Llast : BT) - 1) * H;
 #pragma unroll
       for (int i = 0; i < NPA; ++i) R.a[i] = *(const v4*)(la + 2048 * i);   // full tiles whatever the chunk length
-      if (lc != nchunks - 1 || Llast == BT) {
 #pragma unroll
-        for (int i = 0; i < NPW; ++i) R.q[i] = *(const v8*)(lq + offq[i]);
-#pragma unroll
-        for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + offk[i]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + offv[i]);
-        R.gam = *(const uint32_t*)(lg + offg);
-      } else {
-        // rows past the end of the sequence are redirected to its last row (zeroed in write())
-        const uint32_t last = (uint32_t)Llast - 1;
-        auto cl = [&](uint32_t row) { return row < last ? row : last; };
-#pragma unroll
-        for (int i = 0; i < NPW; ++i) {
-          uint32_t e = st + 256 * i;
-          R.q[i] = *(const v8*)(lq + 2 * (cl(q_row(e)) * HK + q_col(e)));
-        }
-#pragma unroll
-        for (int i = 0; i < RPT; ++i) R.k[i] = *(const v4*)(lk + 2 * (cl(rg * RPT + i) * HK + c4));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + 2 * (cl(urg * 4 + i) * HV + uc4));
-        R.gam = *(const uint32_t*)(lg + 4 * cl(lane) * H);
+      for (int i = 0; i < NPW; ++i) {
+        const uint32_t o = offq[i] < limq ? offq[i] : limq;
+        R.q[i] = *(const v8*)(lq + o);
+        R.k[i] = *(const v8*)(lk + o);
       }
-      lq += strk;
-      lk += strk;
-      lv += strv;
-      la += stra;
-      lg += strg;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
+      R.gam = *(const uint32_t*)(lg + (offg < limg ? offg : limg));
+      if (lc + 1 < nchunks) {
+        lq += strk;
+        lk += strk;
+        lv += strv;
+        la += stra;
+        lg += strg;
+      }
       ++lc;
     };
     // LDS destinations of this lane (element offsets inside a tile)
-    constexpr int KV = RPT == 8 ? 8 : 4;  // elements per k^T write
-    int dq[NPW], dkr[RPT], dk[4][RPT / KV], dv[4];
+    int dq[NPW], dv[4];
 #pragma unroll
     for (int i = 0; i < NPW; ++i) dq[i] = q_row(st + 256 * i) * LDR + q_col(st + 256 * i);
 #pragma unroll
-    for (int i = 0; i < RPT; ++i) dkr[i] = (rg * RPT + i) * LDR + c4;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int i0 = 0; i0 < RPT / KV; ++i0) dk[j][i0] = (c4 + j) * LDT + swz_t(c4 + j, rg * RPT + KV * i0);
-      dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
-    }
+    for (int j = 0; j < 4; ++j) dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
     int wc = 0;  // next chunk to write to LDS
-    auto write = [&](Regs& R) __attribute__((always_inline)) {
+    // maybe_last: the chunk may be the sequence's last, short one (rows past its end are zeroed)
+    auto write = [&](Regs& R, auto maybe_last) __attribute__((always_inline)) {
       const int b = wc & 1;
-      if (wc == nchunks - 1 && Llast < BT) {  // zero the rows past the end of the sequence
-        const int L = Llast;
+      if constexpr (decltype(maybe_last)::value) {
+        if (wc == nchunks - 1 && Llast < BT) {
+          const int L = Llast;
 #pragma unroll
-        for (int i = 0; i < NPW; ++i)
-          if (q_row(st + 256 * i) >= L)
+          for (int i = 0; i < NPW; ++i)
+            if (q_row(st + 256 * i) >= L)
 #pragma unroll
-            for (int j = 0; j < 8; ++j) R.q[i][j] = (T)0.f;
+              for (int j = 0; j < 8; ++j) R.q[i][j] = R.k[i][j] = (T)0.f;
 #pragma unroll
-        for (int i = 0; i < RPT; ++i)
-          if (rg * RPT + i >= L) R.k[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          for (int i = 0; i < 4; ++i)
+            if (urg * 4 + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        }
       }
 #pragma unroll
       for (int i = 0; i < NPW; ++i) *(v8*)&sQ[b][dq[i]] = R.q[i];
 #pragma unroll
       for (int i = 0; i < NPA; ++i) *(v4*)&sAT[b][st * 4 + 1024 * i] = R.a[i];
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) *(v4*)&sK[b][dkr[i]] = R.k[i];
+      for (int i = 0; i < NPW; ++i) *(v8*)&sK[b][dq[i]] = R.k[i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int i0 = 0; i0 < RPT / KV; ++i0) {
-          if constexpr (KV == 8) {
-            v4 lo = {R.k[0][j], R.k[1][j], R.k[2][j], R.k[3][j]};
-            v4 hi = {R.k[4][j], R.k[5][j], R.k[6][j], R.k[7][j]};
-            *(v8*)&sKt[b][dk[j][i0]] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          } else {
-            v4 kc = {R.k[4 * i0][j], R.k[4 * i0 + 1][j], R.k[4 * i0 + 2][j], R.k[4 * i0 + 3][j]};
-            *(v4*)&sKt[b][dk[j][i0]] = kc;
-          }
-        }
         v4 vc = {R.v[0][j], R.v[1][j], R.v[2][j], R.v[3][j]};
         *(v4*)&sVt[b][dv[j]] = vc;
       }
@@ -262,12 +254,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // The matrix waves left o^T of a chunk where v^T of that chunk was; each lane reads back
     // exactly the addresses it writes in write(), so the tile can be refilled right after.
     int oc = 0;  // next chunk whose output is stored
-    auto store_o = [&]() __attribute__((always_inline)) {
+    auto store_o = [&](auto maybe_last) __attribute__((always_inline)) {
       const int b = oc & 1;
       v4 x[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) x[j] = *(const v4*)&sVt[b][dv[j]];
-      if (oc != nchunks - 1 || Llast == BT) {
+      bool full = true;
+      if constexpr (decltype(maybe_last)::value) full = oc != nchunks - 1 || Llast == BT;
+      if (full) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
       } else {
@@ -278,28 +272,50 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       so += strv;
       ++oc;
     };
-    // Two register sets: a chunk is loaded three iterations before the matrix waves use it
-    // (two before it is written to LDS), so the loads have a whole chunk period to land.
-    Regs R0, R1;
+    // Three register sets: a chunk is loaded four iterations before the matrix waves use it (three before it
+    // is written to LDS), so its loads have two chunk periods to land.  Iteration c (the matrix waves work on
+    // chunk c) stores the output of chunk c-1, writes the tiles of chunk c+1 and loads chunk c+4 into the set
+    // just emptied; sets rotate R1, R2, R0.  The steady-state loop runs whole rotations over the iterations
+    // that touch neither the first nor the last chunk and leaves only at its latch.
+    constexpr std::true_type any_chunk{};
+    constexpr std::false_type inner_chunk{};
+    Regs R0, R1, R2;
     load(R0);
-    if (nchunks > 1) load(R1);
-    write(R0);
-    if (nchunks > 2) load(R0);
+    load(R1);
+    load(R2);
+    write(R0, any_chunk);
+    load(R0);
     lds_barrier();
-    // iteration c (the matrix waves work on chunk c): R holds chunk c+1
-    auto iter = [&](int c, Regs& R) __attribute__((always_inline)) {
-      if (c >= 1) store_o();
-      if (c + 1 < nchunks) {
-        write(R);
-        if (c + 3 < nchunks) load(R);
-      }
+    if (nchunks > 1) {
+      write(R1, any_chunk);   // iteration 0
+      load(R1);
       lds_barrier();
-    };
-    for (int c = 0; c < nchunks; c += 2) {
-      iter(c, R1);
-      if (c + 1 < nchunks) iter(c + 1, R0);
+      auto iter = [&](Regs& R) __attribute__((always_inline)) {
+        store_o(inner_chunk);
+        write(R, inner_chunk);
+        load(R);
+        lds_barrier();
+      };
+      const int inner = nchunks > 3 ? nchunks - 3 : 0;   // iterations 1 .. nchunks - 3
+      for (int trips = inner / 3; trips > 0; --trips) {
+        iter(R2);
+        iter(R0);
+        iter(R1);
+      }
+      const int rem = inner % 3;
+      if (rem >= 1) iter(R2);
+      if (rem >= 2) iter(R0);
+      if (nchunks > 2) {      // iteration nchunks - 2 writes the last chunk
+        store_o(inner_chunk);
+        if (rem == 0) write(R2, any_chunk);
+        else if (rem == 1) write(R0, any_chunk);
+        else write(R1, any_chunk);
+        lds_barrier();
+      }
+      store_o(inner_chunk);   // iteration nchunks - 1: the output of chunk nchunks - 2
     }
-    store_o();
+    lds_barrier();
+    store_o(any_chunk);
   } else {
     // =========================== matrix waves ===========================
     const int cb = 16 * wave;  // first of this wave's 16 columns within the slab
@@ -340,7 +356,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int b = ci & 1;
         const T* Kr = sK[b];
         const T* Q = sQ[b];
-        const T* Kt = sKt[b];
         const T* Tu = sAT[b];
         const T* P = sAT[b] + kTriElems;
         const int vrow = cb + c;
@@ -359,7 +374,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
           for (int i = 0; i < KT / 2; ++i)
 #pragma unroll
-            for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16_t<T>(Kt, 16 * (half * (KT / 2) + i), 32 * s, lane);
+            for (int s = 0; s < 2; ++s) f[2 * i + s] = frag16_tr<T>(Kr, LDR, 16 * (half * (KT / 2) + i), 32 * s, lane);
         };
         load_kq(0, fa);
         load_kq(1, fb);
