@@ -229,24 +229,40 @@ struct DhuParams {
 //   phase B: update dH; stage (k^, dv_loc^T) and publish dH for the next (earlier) chunk
 // X = (q, w, do, gamma) and Y = (k, dv_loc, gamma) are prefetched one full iteration ahead.
 template <typename T, int K>
-__global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
+__global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   typedef T t2 __attribute__((ext_vector_type(2)));
   constexpr int BV = 32;
   constexpr int LDK = K + 8;
-  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;   // q, w, k: a lane owns RPT rows x 4 columns
+  constexpr int C8 = K / 8, NP = BT * C8 / 256;   // q, w, k: 16-byte pieces per row / per staging lane
   constexpr int KT32 = K / 32;
   constexpr int NKT = (KT32 + 3) / 4;
   __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];    // k e^{gamma_last-gamma}, row-major
-  __shared__ __attribute__((aligned(16))) T sQt[K * LDT];     // (s q e^gamma)^T, swz16
-  __shared__ __attribute__((aligned(16))) T sWt[K * LDT];     // -(w e^gamma)^T, swz16
+  __shared__ __attribute__((aligned(16))) T sQr[BT * LDK];    // s q e^gamma, row-major
+  __shared__ __attribute__((aligned(16))) T sWr[BT * LDK];    // -w e^gamma, row-major
   __shared__ __attribute__((aligned(16))) T sDoT[BV * LDT];   // do^T
   __shared__ __attribute__((aligned(16))) T sDvl[BV * LDT];   // dv_loc^T
   __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];   // dH^T in 16-bit
   __shared__ __attribute__((aligned(16))) T sDv2T[BV * LDT];  // dv2^T
+  __shared__ float sDec[2];                                    // e^{gamma_last} of chunk c at [c & 1]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // Waves 0-3 ("matrix") carry the state gradient and do the two products of a chunk; waves 4-7 ("staging")
+  // load the next chunk's rows, gate them and write the operand tiles, and store dv2.  With one four-wave
+  // workgroup per CU every SIMD held a single wave that alternated between the two kinds of work (55 % of a
+  // chunk period went into staging while the matrix pipe idled); two workgroups per CU overlapped perfectly, so
+  // the second wave per SIMD is brought along instead.  Per chunk c (walking backwards) the groups meet twice:
+  //   B1(c)  k^ / dv_loc tiles of chunk c and the 16-bit dH are in LDS
+  //          matrix: dv2 = dv_loc + k^ dH -> LDS          staging: q~^T, w~^T, do^T of chunk c -> LDS
+  //   B2(c)  matrix: dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, publishes dH for chunk c-1
+  //          staging: dv2 of chunk c -> memory; k^ / dv_loc tiles of chunk c-1 -> LDS
+  // Each tile is written in the half of the period in which the matrix waves read the other kind, so nothing is
+  // double-buffered.  The staging waves are bound by the number of memory instructions they issue (about 70
+  // cycles each once the CU's memory pipeline is full), so q, w and k move as 16-byte pieces into row-major
+  // tiles and the matrix waves, which have the time, read the transposed operands of the state update with the
+  // transposing LDS load.
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int H = p.H, V = p.V;
   const int nvt = V / BV;
   int64_t id = xcd_remap(blockIdx.x, gridDim.x);
@@ -257,266 +273,300 @@ __global__ __launch_bounds__(256) void gdr_bwd_dhu_kernel(DhuParams p) {
   SeqSpan sp = seq_span(p.offsets, n, p.T);
   const int64_t nchunks = (sp.len + BT - 1) / BT;
   const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
-
-  f32x16 acc[NKT], acct[NKT];
-#pragma unroll
-  for (int a = 0; a < NKT; ++a) {
-    acc[a] = zero16();
-    acct[a] = zero16();
-    int kt = wave + 4 * a;
-    if (p.dht && kt < KT32) {
-      const float* d0 = p.dht + (int64_t)nh * K * V;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        acc[a][r] = d0[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
-        acct[a][r] = d0[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + c32_row(r, lane)];
-      }
-    }
-  }
-
-  const int rg = tid / CG, c4 = (tid % CG) * 4;
-  const int urg = tid >> 4, uc2 = (tid & 15) * 2;
-  struct XRegs {
-    v4 q[RPT];
-    v4 w[RPT];
-    t2 d[4];
-  };
-  struct YRegs {
-    v4 k[RPT];
-    float gam[RPT];
-    t2 dvl[4];
-    float glast;
-  };
   auto chunk_len = [&](int64_t c) {
     int64_t rem = sp.len - c * BT;
     return (int)(rem < BT ? rem : BT);
   };
-  // Loads are unconditional (a load under a branch makes the wave drain its whole load queue at the
-  // join): byte offsets of this lane's rows from the first row of a chunk are computed once, rows past
-  // the end of a short chunk are redirected to its last row, chunks before the first one to chunk 0;
-  // the staging functions zero what must not count.
-  const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
-  const uint32_t pitchG = (uint32_t)H * 4u;
-  uint32_t offk[RPT], offg[RPT], offv[4];
-#pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    offk[i] = (uint32_t)(rg * RPT + i) * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
-    offg[i] = (uint32_t)(rg * RPT + i) * pitchG;
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) offv[i] = (uint32_t)(urg * 4 + i) * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-  const char* gq = (const char*)p.q + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
-  const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
-  const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
-  const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
-  const char* gl = (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
-  // without gates every gate load reads one zero word (no select on the loaded value: it would
-  // make the wave wait for the load where it is issued)
-  const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : (const char*)&kZeroWord;
-  auto load_x = [&](int64_t c, XRegs& R) __attribute__((always_inline)) {
-    c = c < 0 ? 0 : c;
-    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
-    const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV;
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      const uint32_t lk = last * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
-      const uint32_t o = offk[i] < lk ? offk[i] : lk;
-      R.q[i] = *(const v4*)(gq + ck + o);
-      R.w[i] = *(const v4*)(gw + ck + o);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-      R.d[i] = *(const t2*)(gd + cv + (offv[i] < lv ? offv[i] : lv));
-    }
-  };
-  auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
-    c = c < 0 ? 0 : c;
-    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
-    const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV, cg = p.gam ? c * BT * (int64_t)pitchG : 0;
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      const uint32_t lk = last * pitchK + (uint32_t)c4 * (uint32_t)sizeof(T);
-      R.k[i] = *(const v4*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
-      const uint32_t og = offg[i] < last * pitchG ? offg[i] : last * pitchG;
-      R.gam[i] = *(const float*)(gg + cg + (p.gam ? og : 0u));
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-      R.dvl[i] = *(const t2*)(gl + cv + (offv[i] < lv ? offv[i] : lv));
-    }
-    R.glast = *(const float*)(gg + cg + (p.gam ? last * pitchG : 0u));
-  };
-  // e^{gamma} of the rows of the chunk held in X (zero past its end): formed when the same chunk is
-  // staged as Y, one iteration earlier, so that nothing loop-carried depends on a load in flight
-  float egx[RPT];
-  auto stage_x = [&](const XRegs& R) {
-    // a lane owns RPT consecutive time rows of 4 key columns: one vector write per column
-    // (in pieces of at most one 16-byte slot, the unit the swizzle permutes)
-    constexpr int PW = RPT < 8 ? RPT : 8;
-    typedef T rvec __attribute__((ext_vector_type(PW)));
-    float eg[RPT];
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) eg[i] = egx[i];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int i0 = 0; i0 < RPT; i0 += PW) {
-        rvec xq, xw;
-#pragma unroll
-        for (int i = 0; i < PW; ++i) {
-          xq[i] = (T)((float)R.q[i0 + i][j] * p.scale * eg[i0 + i]);
-          xw[i] = (T)(-(float)R.w[i0 + i][j] * eg[i0 + i]);
-        }
-        *(rvec*)&sQt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT + i0)] = xq;
-        *(rvec*)&sWt[(c4 + j) * LDT + swz16(c4 + j, rg * RPT + i0)] = xw;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      v4 dv = v4{R.d[0][j], R.d[1][j], R.d[2][j], R.d[3][j]};
-      *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
-    }
-  };
-  auto stage_y = [&](const YRegs& R, int L) {
-#pragma unroll
-    for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      egx[i] = (row < L) ? __expf(R.gam[i]) : 0.f;
-      float e = (row < L) ? __expf(R.glast - R.gam[i]) : 0.f;
-      v4 kv;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) kv[j] = (T)((float)R.k[i][j] * e);
-      *(v4*)&sKh[row * LDK + c4] = kv;
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      v4 dv = v4{R.dvl[0][j], R.dvl[1][j], R.dvl[2][j], R.dvl[3][j]};
-      if (L < BT) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i >= L) dv[i] = (T)0.f;
-      }
-      *(v4*)&sDvl[(uc2 + j) * LDT + urg * 4] = dv;
-    }
-  };
-  // gradient w.r.t. the state leaving chunk c: 16-bit transpose in LDS, FRAGMENT_T copy in HBM
-  auto publish = [&](int64_t c) {
-#pragma unroll
-    for (int a = 0; a < NKT; ++a) {
-      int kt = wave + 4 * a;
-      if (kt < KT32) {
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          v4 x;
-#pragma unroll
-          for (int b = 0; b < 4; ++b) x[b] = (T)acc[a][4 * q4 + b];
-          *(v4*)&sDHt[(lane & 31) * LDK + kt * 32 + 8 * q4 + 4 * (lane >> 5)] = x;
-        }
-        v8 lo, hi;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          lo[r] = (T)acct[a][r];
-          hi[r] = (T)acct[a][r + 8];
-        }
-        T* hp = (T*)p.dhtf + ((chunk0 + c) * H + hh) * (int64_t)K * V + (((int64_t)vt * (K / 32) + kt) * 64 + lane) * 16;
-        *(v8*)hp = lo;
-        *(v8*)(hp + 8) = hi;
-      }
-    }
-  };
 
-  XRegs X;
-  YRegs Y;
-  float dec = 1.f;
-  if (nchunks > 0) {
-    load_x(nchunks - 1, X);
-    load_y(nchunks - 1, Y);
-    stage_y(Y, chunk_len(nchunks - 1));
-    dec = __expf(Y.glast);
-    publish(nchunks - 1);
-    load_y(nchunks - 2, Y);
-  }
-  // One chunk of the reverse scan.  The first chunk of the sequence (processed last) is peeled off
-  // so that the steady-state loop has no memory operation under a branch.
-  auto step = [&](int64_t c, auto more) __attribute__((always_inline)) {
-    const int L = chunk_len(c);
-    const int64_t rbase = sp.bos + c * BT;
-    lds_barrier();  // (1)
-    // ---- dv2 = dv_loc + k^ dH : wave w owns rows 16w..16w+15, two 16-column tiles
-    {
-      f32x4 d[2] = {zero4(), zero4()};
+  if (wave >= 4) {
+    // =========================== staging waves ===========================
+    if (nchunks == 0) return;
+    const int st = tid - 256;
+    const int prow = st / C8, c8 = (st % C8) * 8;   // piece i of a lane: row prow + (256 / C8) i, columns c8 ..
+    constexpr int PR = 256 / C8;
+    const int urg = st >> 4, uc2 = (st & 15) * 2;
+    struct XRegs {
+      v8 q[NP];
+      v8 w[NP];
+      t2 d[4];
+    };
+    struct YRegs {
+      v8 k[NP];
+      float gam[NP];
+      t2 dvl[4];
+      float glast;
+    };
+    // Loads are unconditional (a load under a branch makes the wave drain its whole load queue at the
+    // join): byte offsets of this lane's rows from the first row of a chunk are computed once, rows past
+    // the end of a short chunk are redirected to its last row, chunks before the first one to chunk 0;
+    // the staging functions zero what must not count.
+    const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
+    const uint32_t pitchG = (uint32_t)H * 4u;
+    uint32_t offk[NP], offg[NP], offv[4];
 #pragma unroll
-      for (int ks = 0; ks < K; ks += 32) {
-        v8 a = lds_frag16<T>(sKh, LDK, wave * 16, ks, lane);
+    for (int i = 0; i < NP; ++i) {
+      offk[i] = (uint32_t)(prow + PR * i) * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+      offg[i] = (uint32_t)(prow + PR * i) * pitchG;
+    }
 #pragma unroll
-        for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, lds_frag16<T>(sDHt, LDK, j * 16, ks, lane), d[j]);
+    for (int i = 0; i < 4; ++i) offv[i] = (uint32_t)(urg * 4 + i) * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+    const char* gq = (const char*)p.q + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+    const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+    const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+    const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const char* gl = (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    // without gates every gate load reads one zero word (no select on the loaded value: it would
+    // make the wave wait for the load where it is issued)
+    const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : (const char*)&kZeroWord;
+    auto load_x = [&](int64_t c, XRegs& R) __attribute__((always_inline)) {
+      c = c < 0 ? 0 : c;
+      const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+      const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+        const uint32_t o = offk[i] < lk ? offk[i] : lk;
+        R.q[i] = *(const v8*)(gq + ck + o);
+        R.w[i] = *(const v8*)(gw + ck + o);
       }
-      const int tr = wave * 16 + 4 * (lane >> 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+        R.d[i] = *(const t2*)(gd + cv + (offv[i] < lv ? offv[i] : lv));
+      }
+    };
+    auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
+      c = c < 0 ? 0 : c;
+      const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+      const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV, cg = p.gam ? c * BT * (int64_t)pitchG : 0;
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+        R.k[i] = *(const v8*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
+        const uint32_t og = offg[i] < last * pitchG ? offg[i] : last * pitchG;
+        R.gam[i] = *(const float*)(gg + cg + (p.gam ? og : 0u));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+        R.dvl[i] = *(const t2*)(gl + cv + (offv[i] < lv ? offv[i] : lv));
+      }
+      R.glast = *(const float*)(gg + cg + (p.gam ? last * pitchG : 0u));
+    };
+    // e^{gamma} of the rows of the chunk held in X (zero past its end): formed when the same chunk is
+    // staged as Y, half a period earlier, so that nothing loop-carried depends on a load in flight
+    float egx[NP];
+    auto stage_x = [&](const XRegs& R) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < NP; ++i) {
+        const float eq = p.scale * egx[i], ew = -egx[i];
+        v8 xq, xw;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          xq[j] = (T)((float)R.q[i][j] * eq);
+          xw[j] = (T)((float)R.w[i][j] * ew);
+        }
+        *(v8*)&sQr[(prow + PR * i) * LDK + c8] = xq;
+        *(v8*)&sWr[(prow + PR * i) * LDK + c8] = xw;
+      }
+      // (the loaded pairs go through an opaque copy where they are consumed: otherwise the compiler carries a
+      // rearranged copy round the loop and waits for the load at the latch, right after issuing it)
+      t2 rd[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t u = __builtin_bit_cast(uint32_t, R.d[i]);
+        asm volatile("" : "+v"(u));
+        rd[i] = __builtin_bit_cast(t2, u);
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        int vc = j * 16 + (lane & 15);
-        v4 dl = *(const v4*)&sDvl[vc * LDT + tr];
-        v4 o;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[r] = (T)((float)dl[r] + d[j][r]);
-        *(v4*)&sDv2T[vc * LDT + tr] = o;
+        v4 dv = v4{rd[0][j], rd[1][j], rd[2][j], rd[3][j]};
+        *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
       }
-      // The wave reads its own 16 rows back in row-major order (its writes only: no barrier) and
-      // stores each row's 32 columns as four 16-byte pieces.
-      {
-        const int row = wave * 16 + (lane >> 2), v0 = (lane & 3) * 8;
-        v8 x;
+    };
+    auto stage_y = [&](const YRegs& R, int64_t c) __attribute__((always_inline)) {
+      const int L = chunk_len(c);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) x[e] = sDv2T[(v0 + e) * LDT + row];
-        if (row < L) *(v8*)((T*)p.dv2 + ((rbase + row) * H + hh) * (int64_t)V + vbase + v0) = x;
+      for (int i = 0; i < NP; ++i) {
+        int row = prow + PR * i;
+        egx[i] = (row < L) ? __expf(R.gam[i]) : 0.f;
+        float e = (row < L) ? __expf(R.glast - R.gam[i]) : 0.f;
+        v8 kv;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) kv[j] = (T)((float)R.k[i][j] * e);
+        *(v8*)&sKh[row * LDK + c8] = kv;
+      }
+      t2 rl[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t u = __builtin_bit_cast(uint32_t, R.dvl[i]);
+        asm volatile("" : "+v"(u));
+        rl[i] = __builtin_bit_cast(t2, u);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        v4 dv = v4{rl[0][j], rl[1][j], rl[2][j], rl[3][j]};
+        if (L < BT) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (urg * 4 + i >= L) dv[i] = (T)0.f;
+        }
+        *(v4*)&sDvl[(uc2 + j) * LDT + urg * 4] = dv;
+      }
+      if (st == 0) sDec[c & 1] = __expf(R.glast);
+    };
+    // dv2 of chunk c leaves as whole rows, 16 bytes per lane: a 16-lane group turns a block of 8 value columns x
+    // 16 time rows of the transposed tile round with two transposing LDS loads (lane j ends up with time row
+    // 16 tb + j, columns 8 vb ..).  Only a sequence's last chunk (the first one processed) can be short: it takes
+    // the variant with the masked store, the steady state stores unconditionally.
+    const int dgrp = st >> 4, dtb = dgrp >> 2, dvb = dgrp & 3, dj = st & 15;
+    const int dsrc = (8 * dvb + (dj >> 2)) * LDT + 16 * dtb + 4 * (dj & 3);
+    auto store_dv2 = [&](int64_t c, auto maybe_short) __attribute__((always_inline)) {
+      typedef short s4 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) s4 lds_s4;
+      s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sDv2T[dsrc]);
+      s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sDv2T[dsrc + 4 * LDT]);
+      const v8 x = __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+      const int row = 16 * dtb + dj;
+      T* dst = (T*)p.dv2 + ((sp.bos + c * BT + row) * H + hh) * (int64_t)V + vbase + 8 * dvb;
+      if constexpr (decltype(maybe_short)::value) {
+        if (row < chunk_len(c)) *(v8*)dst = x;
+      } else {
+        *(v8*)dst = x;
+      }
+    };
+    XRegs X;
+    YRegs Y;
+    load_x(nchunks - 1, X);
+    load_y(nchunks - 1, Y);
+    stage_y(Y, nchunks - 1);
+    load_y(nchunks - 2, Y);
+    // The first chunk of the sequence (processed last) is peeled off so that the steady-state loop has no
+    // memory operation under a branch.
+    if (nchunks > 1) {
+      // the sequence's last chunk, possibly short
+      lds_barrier();  // B1(nchunks - 1)
+      stage_x(X);
+      load_x(nchunks - 2, X);
+      lds_barrier();  // B2(nchunks - 1)
+      store_dv2(nchunks - 1, std::true_type{});
+      stage_y(Y, nchunks - 2);
+      load_y(nchunks - 3, Y);
+      for (int64_t c = nchunks - 2; c >= 1; --c) {
+        lds_barrier();  // B1(c)
+        stage_x(X);
+        load_x(c - 1, X);
+        lds_barrier();  // B2(c)
+        store_dv2(c, std::false_type{});
+        stage_y(Y, c - 1);
+        load_y(c - 2, Y);
       }
     }
+    lds_barrier();  // B1(0)
     stage_x(X);
-    const float dec_c = dec;
-    load_x(c - 1, X);
-    lds_barrier();  // (2)
-    // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
+    lds_barrier();  // B2(0)
+    store_dv2(0, std::true_type{});
+  } else {
+    // =========================== matrix waves ===========================
+    f32x16 acc[NKT], acct[NKT];
 #pragma unroll
     for (int a = 0; a < NKT; ++a) {
+      acc[a] = zero16();
+      acct[a] = zero16();
       int kt = wave + 4 * a;
-      if (kt < KT32) {
+      if (p.dht && kt < KT32) {
+        const float* d0 = p.dht + (int64_t)nh * K * V;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          acc[a][r] *= dec_c;
-          acct[a][r] *= dec_c;
-        }
-#pragma unroll
-        for (int s = 0; s < BT; s += 16) {
-          v8 fq = lds_frag32_swz<T>(sQt, LDT, kt * 32, s, lane);
-          v8 fd = lds_frag32<T>(sDoT, LDT, 0, s, lane);
-          v8 fw = lds_frag32_swz<T>(sWt, LDT, kt * 32, s, lane);
-          v8 f2 = lds_frag32<T>(sDv2T, LDT, 0, s, lane);
-          acc[a] = Elem<T>::mfma32(fq, fd, acc[a]);
-          acc[a] = Elem<T>::mfma32(fw, f2, acc[a]);
-          acct[a] = Elem<T>::mfma32(fd, fq, acct[a]);
-          acct[a] = Elem<T>::mfma32(f2, fw, acct[a]);
+          acc[a][r] = d0[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)];
+          acct[a][r] = d0[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + c32_row(r, lane)];
         }
       }
     }
-    if constexpr (decltype(more)::value) {
-      stage_y(Y, chunk_len(c - 1));
-      dec = __expf(Y.glast);
-      publish(c - 1);
-      load_y(c - 2, Y);
+    // gradient w.r.t. the state leaving chunk c: 16-bit transpose in LDS, FRAGMENT_T copy in HBM
+    auto publish = [&](int64_t c) __attribute__((always_inline)) {
+#pragma unroll
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            v4 x;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) x[b] = (T)acc[a][4 * q4 + b];
+            *(v4*)&sDHt[(lane & 31) * LDK + kt * 32 + 8 * q4 + 4 * (lane >> 5)] = x;
+          }
+          v8 lo, hi;
+#pragma unroll
+          for (int r = 0; r < 8; ++r) {
+            lo[r] = (T)acct[a][r];
+            hi[r] = (T)acct[a][r + 8];
+          }
+          T* hp = (T*)p.dhtf + ((chunk0 + c) * H + hh) * (int64_t)K * V + (((int64_t)vt * (K / 32) + kt) * 64 + lane) * 16;
+          *(v8*)hp = lo;
+          *(v8*)(hp + 8) = hi;
+        }
+      }
+    };
+    if (nchunks > 0) publish(nchunks - 1);
+    for (int64_t c = nchunks - 1; c >= 0; --c) {
+      lds_barrier();  // B1(c)
+      // ---- dv2 = dv_loc + k^ dH : wave w owns rows 16w..16w+15, two 16-column tiles
+      {
+        f32x4 d[2] = {zero4(), zero4()};
+#pragma unroll
+        for (int ks = 0; ks < K; ks += 32) {
+          v8 a = lds_frag16<T>(sKh, LDK, wave * 16, ks, lane);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, lds_frag16<T>(sDHt, LDK, j * 16, ks, lane), d[j]);
+        }
+        const int tr = wave * 16 + 4 * (lane >> 4);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          int vc = j * 16 + (lane & 15);
+          v4 dl = *(const v4*)&sDvl[vc * LDT + tr];
+          v4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = (T)((float)dl[r] + d[j][r]);
+          *(v4*)&sDv2T[vc * LDT + tr] = o;
+        }
+      }
+      lds_barrier();  // B2(c)
+      // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
+      const float dec_c = sDec[c & 1];
+#pragma unroll
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            acc[a][r] *= dec_c;
+            acct[a][r] *= dec_c;
+          }
+#pragma unroll
+          for (int s = 0; s < BT; s += 16) {
+            v8 fq = frag32_tr<T>(sQr, LDK, kt * 32, s, lane);
+            v8 fd = lds_frag32<T>(sDoT, LDT, 0, s, lane);
+            v8 fw = frag32_tr<T>(sWr, LDK, kt * 32, s, lane);
+            v8 f2 = lds_frag32<T>(sDv2T, LDT, 0, s, lane);
+            acc[a] = Elem<T>::mfma32(fq, fd, acc[a]);
+            acc[a] = Elem<T>::mfma32(fw, f2, acc[a]);
+            acct[a] = Elem<T>::mfma32(fd, fq, acct[a]);
+            acct[a] = Elem<T>::mfma32(f2, fw, acct[a]);
+          }
+        }
+      }
+      if (c > 0) publish(c - 1);
     }
-  };
-  for (int64_t c = nchunks - 1; c >= 1; --c) step(c, std::true_type{});
-  if (nchunks > 0) step(0, std::false_type{});
-  if (p.dh0) {
-    float* o = p.dh0 + (int64_t)nh * K * V;
+    if (p.dh0) {
+      float* o = p.dh0 + (int64_t)nh * K * V;
 #pragma unroll
-    for (int a = 0; a < NKT; ++a) {
-      int kt = wave + 4 * a;
-      if (kt < KT32) {
+      for (int a = 0; a < NKT; ++a) {
+        int kt = wave + 4 * a;
+        if (kt < KT32) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[a][r];
+          for (int r = 0; r < 16; ++r) o[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[a][r];
+        }
       }
     }
   }
@@ -1346,9 +1396,9 @@ int launch_dhu(const DhuParams& p, int64_t K, hipStream_t st) {
   const int64_t total = (int64_t)(p.V / 32) * p.N * p.H;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   if (total == 0) return FLA_OK;
-  if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(256), 0, st, p);
-  else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(256), 0, st, p);
-  else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(256), 0, st, p);
+  if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(512), 0, st, p);
+  else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(512), 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(512), 0, st, p);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;

@@ -361,21 +361,6 @@ FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 // accumulators: the loads land while the inversion runs (measured: worth about 4 %; the launch is a chain
 // of short dependent phases - removing the inversion, the stores or the loads each saves 15-20 % - rather
 // than bound by one resource).
-// 32x32x16 operand whose 32 rows are contiguous in LDS and whose contraction index is the tile's row
-// (tile[kk][m], pitch ld): the transposing LDS read hands lane j of a 16-lane group element j of the four
-// rows whose 8-byte pieces the group's lanes 4i .. 4i+3 address.
-template <typename T>
-FLA_DEVICE typename Elem<T>::v8 frag32_tr(const T* tile, int ld, int m0, int k0, int lane) {
-  typedef typename Elem<T>::v4 v4;
-  typedef short s4 __attribute__((ext_vector_type(4)));
-  typedef __attribute__((address_space(3))) s4 lds_s4;
-  const int s = lane & 15, g = lane >> 4;
-  const T* p0 = tile + (k0 + 8 * (g >> 1) + (s >> 2)) * ld + m0 + 16 * (g & 1) + 4 * (s & 3);
-  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
-  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 4 * ld));
-  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 // KEEP: the forward of a pass that will be differentiated also leaves w = Aw (beta k) and Aw in memory (the WY
 // launch of the reference's decomposition, without a second inversion and a second pass over k).
 template <typename T, int K, bool KEEP>

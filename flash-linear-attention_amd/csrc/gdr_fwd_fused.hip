@@ -87,21 +87,6 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
   return __builtin_bit_cast(v8, u4{lo[0], hi[0], lo[1], hi[1]});
 }
 
-// A operand of the state update (16 key rows x 32 time steps in accumulator-row order) read from the row-major
-// k tile [t][k]: the transposing LDS read hands lane j of a 16-lane group the four time rows whose 8-byte pieces
-// the group's lanes 4i .. 4i+3 address, so no transposed copy of k is staged.
-template <typename T>
-FLA_DEVICE typename Elem<T>::v8 frag16_tr(const T* tile, int ld, int k0, int t0, int lane) {
-  typedef typename Elem<T>::v4 v4;
-  typedef short s4 __attribute__((ext_vector_type(4)));
-  typedef __attribute__((address_space(3))) s4 lds_s4;
-  const int j = lane & 15, g = lane >> 4;
-  const T* p0 = tile + (t0 + 4 * g + (j >> 2)) * ld + k0 + 4 * (j & 3);
-  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
-  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 16 * ld));
-  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
-}
-
 template <typename T, int K, bool KEEP>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {

@@ -80,3 +80,33 @@ FLA_DEVICE f32x4 zero4() {
   f32x4 z = {0.f, 0.f, 0.f, 0.f};
   return z;
 }
+
+// Operands whose contraction index is the tile's ROW (tile[kk][m], pitch ld) come out of LDS through the
+// transposing load ds_read_b64_tr_b16: it hands lane j of a 16-lane group element j of each of the four rows whose
+// 8-byte pieces the group's lanes 4i .. 4i+3 address.
+// 32x32x16 operand: 32 operand rows m0 .. m0+31 (contiguous in LDS), contraction slice [k0, k0+16) (tile rows).
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag32_tr(const T* tile, int ld, int m0, int k0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef short s4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const int s = lane & 15, g = lane >> 4;
+  const T* p0 = tile + (k0 + 8 * (g >> 1) + (s >> 2)) * ld + m0 + 16 * (g & 1) + 4 * (s & 3);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 4 * ld));
+  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// 16x16x32 operand: 16 operand rows k0 .. k0+15, contraction slice [t0, t0+32) in accumulator-row order (slot
+// (g = lane/16, e) holds t0 + 16*(e/4) + 4*g + e%4, as frag16_t of chunk_common.h delivers it from a transposed copy).
+template <typename T>
+FLA_DEVICE typename Elem<T>::v8 frag16_tr(const T* tile, int ld, int k0, int t0, int lane) {
+  typedef typename Elem<T>::v4 v4;
+  typedef short s4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s4 lds_s4;
+  const int j = lane & 15, g = lane >> 4;
+  const T* p0 = tile + (t0 + 4 * g + (j >> 2)) * ld + k0 + 4 * (j & 3);
+  s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)p0);
+  s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)(p0 + 16 * ld));
+  return __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+}
