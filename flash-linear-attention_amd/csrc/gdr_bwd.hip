@@ -224,43 +224,46 @@ struct DhuParams {
   float scale;
 };
 
-// One workgroup: all K rows x 32 value columns.  Two barriers per chunk:
-//   phase A: dv2 from (k^, dH^T, dv_loc^T); stage (q~^T, -w~^T, do^T) of the same chunk
-//   phase B: update dH; stage (k^, dv_loc^T) and publish dH for the next (earlier) chunk
-// X = (q, w, do, gamma) and Y = (k, dv_loc, gamma) are prefetched one full iteration ahead.
+// One workgroup of eight waves: all K rows x 32 value columns of one (sequence, head).
+// Waves 0-3 ("matrix") carry the state gradient and do the two products of a chunk; waves 4-7 ("staging") load
+// the next chunk's rows, write the operand tiles and store dv2.  (With one four-wave workgroup per CU every SIMD
+// held a single wave that alternated between the two kinds of work: 55 % of a chunk period went into staging
+// while the matrix pipe idled, and two workgroups per CU overlapped perfectly - so the second wave per SIMD is
+// brought along instead.)  Per chunk c (walking backwards) the groups meet twice:
+//   B1(c)  k, dv_loc and the gates of chunk c and the 16-bit dH are in LDS
+//          matrix:  dv2 = dv_loc + e^{gamma_last-gamma} * (k dH) -> LDS, and -e^{gamma} * dv2 beside it
+//          staging: q, w and s e^{gamma} * do of chunk c -> LDS
+//   B2(c)  matrix:  dH <- e^{gamma_last} dH + q^T (s e^{gamma} * do) + w^T (-e^{gamma} * dv2); publishes dH
+//          staging: dv2 of chunk c -> memory; k, dv_loc, gates of chunk c-1 -> LDS
+// Each tile is written in the half of the period in which the matrix waves read the other kind, so nothing is
+// double-buffered.  The gates are per (token, head): as row scalings they commute out of the K-wide operands
+// onto the 32-column ones (do, dv2) and onto the product k dH, so q, w and k are staged as plain 16-byte copies -
+// the staging waves are bound by the instructions they issue (a memory instruction costs the issuing wave about
+// 70 cycles once the CU's memory pipeline is full), the matrix waves have time to spare - and every transposed
+// operand is read from a row-major tile with the transposing LDS load.
 template <typename T, int K>
 __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
-  typedef T t2 __attribute__((ext_vector_type(2)));
   constexpr int BV = 32;
   constexpr int LDK = K + 8;
+  constexpr int LDV = BV + 8;
   constexpr int C8 = K / 8, NP = BT * C8 / 256;   // q, w, k: 16-byte pieces per row / per staging lane
+  constexpr int PR = 256 / C8;                    // rows between two pieces of a lane
   constexpr int KT32 = K / 32;
   constexpr int NKT = (KT32 + 3) / 4;
-  __shared__ __attribute__((aligned(16))) T sKh[BT * LDK];    // k e^{gamma_last-gamma}, row-major
-  __shared__ __attribute__((aligned(16))) T sQr[BT * LDK];    // s q e^gamma, row-major
-  __shared__ __attribute__((aligned(16))) T sWr[BT * LDK];    // -w e^gamma, row-major
-  __shared__ __attribute__((aligned(16))) T sDoT[BV * LDT];   // do^T
-  __shared__ __attribute__((aligned(16))) T sDvl[BV * LDT];   // dv_loc^T
-  __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];   // dH^T in 16-bit
-  __shared__ __attribute__((aligned(16))) T sDv2T[BV * LDT];  // dv2^T
-  __shared__ float sDec[2];                                    // e^{gamma_last} of chunk c at [c & 1]
+  __shared__ __attribute__((aligned(16))) T sK[BT * LDK];      // k, row-major
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];      // q, row-major
+  __shared__ __attribute__((aligned(16))) T sW[BT * LDK];      // w, row-major
+  __shared__ __attribute__((aligned(16))) T sDo[BT * LDV];     // s e^{gamma} * do, row-major [t][v]
+  __shared__ __attribute__((aligned(16))) T sDvl[BT * LDV];    // dv_loc, row-major [t][v]
+  __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];    // dH^T in 16-bit
+  __shared__ __attribute__((aligned(16))) T sDv2T[BV * LDT];   // dv2^T
+  __shared__ __attribute__((aligned(16))) T sDv2s[BV * LDT];   // (-e^{gamma} * dv2)^T
+  __shared__ __attribute__((aligned(16))) float sEg[BT];       // e^{gamma_t} (0 past the end of a short chunk)
+  __shared__ __attribute__((aligned(16))) float sEd[BT];       // e^{gamma_last - gamma_t} (0 past the end)
+  __shared__ float sDec[2];                                     // e^{gamma_last} of chunk c at [c & 1]
 
-  // Waves 0-3 ("matrix") carry the state gradient and do the two products of a chunk; waves 4-7 ("staging")
-  // load the next chunk's rows, gate them and write the operand tiles, and store dv2.  With one four-wave
-  // workgroup per CU every SIMD held a single wave that alternated between the two kinds of work (55 % of a
-  // chunk period went into staging while the matrix pipe idled); two workgroups per CU overlapped perfectly, so
-  // the second wave per SIMD is brought along instead.  Per chunk c (walking backwards) the groups meet twice:
-  //   B1(c)  k^ / dv_loc tiles of chunk c and the 16-bit dH are in LDS
-  //          matrix: dv2 = dv_loc + k^ dH -> LDS          staging: q~^T, w~^T, do^T of chunk c -> LDS
-  //   B2(c)  matrix: dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, publishes dH for chunk c-1
-  //          staging: dv2 of chunk c -> memory; k^ / dv_loc tiles of chunk c-1 -> LDS
-  // Each tile is written in the half of the period in which the matrix waves read the other kind, so nothing is
-  // double-buffered.  The staging waves are bound by the number of memory instructions they issue (about 70
-  // cycles each once the CU's memory pipeline is full), so q, w and k move as 16-byte pieces into row-major
-  // tiles and the matrix waves, which have the time, read the transposed operands of the state update with the
-  // transposing LDS load.
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int H = p.H, V = p.V;
@@ -282,34 +285,29 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     // =========================== staging waves ===========================
     if (nchunks == 0) return;
     const int st = tid - 256;
-    const int prow = st / C8, c8 = (st % C8) * 8;   // piece i of a lane: row prow + (256 / C8) i, columns c8 ..
-    constexpr int PR = 256 / C8;
-    const int urg = st >> 4, uc2 = (st & 15) * 2;
+    const int prow = st / C8, c8 = (st % C8) * 8;   // piece i of a lane: row prow + PR i, columns c8 ..
+    const int vrow = st >> 2, vc8 = (st & 3) * 8;   // do, dv_loc, dv2: one row, 8 of the 32 columns
     struct XRegs {
       v8 q[NP];
       v8 w[NP];
-      t2 d[4];
+      v8 d;
     };
     struct YRegs {
       v8 k[NP];
-      float gam[NP];
-      t2 dvl[4];
-      float glast;
+      v8 dvl;
+      float gam, glast;
     };
     // Loads are unconditional (a load under a branch makes the wave drain its whole load queue at the
     // join): byte offsets of this lane's rows from the first row of a chunk are computed once, rows past
-    // the end of a short chunk are redirected to its last row, chunks before the first one to chunk 0;
-    // the staging functions zero what must not count.
+    // the end of a short chunk are redirected to its last row, chunks before the first one to chunk 0.
+    // What a redirected row holds never counts: its gate factors are zero.
     const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
     const uint32_t pitchG = (uint32_t)H * 4u;
-    uint32_t offk[NP], offg[NP], offv[4];
+    uint32_t offk[NP];
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      offk[i] = (uint32_t)(prow + PR * i) * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
-      offg[i] = (uint32_t)(prow + PR * i) * pitchG;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) offv[i] = (uint32_t)(urg * 4 + i) * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
+    for (int i = 0; i < NP; ++i) offk[i] = (uint32_t)(prow + PR * i) * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+    const uint32_t offv = (uint32_t)vrow * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+    const uint32_t offg = (uint32_t)vrow * pitchG;
     const char* gq = (const char*)p.q + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
     const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
     const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
@@ -322,96 +320,53 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
       c = c < 0 ? 0 : c;
       const uint32_t last = (uint32_t)(chunk_len(c) - 1);
       const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV;
+      const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
 #pragma unroll
       for (int i = 0; i < NP; ++i) {
-        const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
         const uint32_t o = offk[i] < lk ? offk[i] : lk;
         R.q[i] = *(const v8*)(gq + ck + o);
         R.w[i] = *(const v8*)(gw + ck + o);
       }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-        R.d[i] = *(const t2*)(gd + cv + (offv[i] < lv ? offv[i] : lv));
-      }
+      const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+      R.d = *(const v8*)(gd + cv + (offv < lv ? offv : lv));
     };
     auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
       c = c < 0 ? 0 : c;
       const uint32_t last = (uint32_t)(chunk_len(c) - 1);
       const int64_t ck = c * BT * (int64_t)pitchK, cv = c * BT * (int64_t)pitchV, cg = p.gam ? c * BT * (int64_t)pitchG : 0;
+      const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
 #pragma unroll
-      for (int i = 0; i < NP; ++i) {
-        const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
-        R.k[i] = *(const v8*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
-        const uint32_t og = offg[i] < last * pitchG ? offg[i] : last * pitchG;
-        R.gam[i] = *(const float*)(gg + cg + (p.gam ? og : 0u));
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t lv = last * pitchV + (uint32_t)uc2 * (uint32_t)sizeof(T);
-        R.dvl[i] = *(const t2*)(gl + cv + (offv[i] < lv ? offv[i] : lv));
-      }
+      for (int i = 0; i < NP; ++i) R.k[i] = *(const v8*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
+      const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+      R.dvl = *(const v8*)(gl + cv + (offv < lv ? offv : lv));
+      const uint32_t og = offg < last * pitchG ? offg : last * pitchG;
+      R.gam = *(const float*)(gg + cg + (p.gam ? og : 0u));
       R.glast = *(const float*)(gg + cg + (p.gam ? last * pitchG : 0u));
     };
-    // e^{gamma} of the rows of the chunk held in X (zero past its end): formed when the same chunk is
-    // staged as Y, half a period earlier, so that nothing loop-carried depends on a load in flight
-    float egx[NP];
+    // s e^{gamma} of this lane's do row in the chunk held in X (zero past its end): formed when the same chunk
+    // is staged as Y, half a period earlier, so that nothing loop-carried depends on a load in flight
+    float egx = 0.f;
     auto stage_x = [&](const XRegs& R) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < NP; ++i) {
-        const float eq = p.scale * egx[i], ew = -egx[i];
-        v8 xq, xw;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          xq[j] = (T)((float)R.q[i][j] * eq);
-          xw[j] = (T)((float)R.w[i][j] * ew);
-        }
-        *(v8*)&sQr[(prow + PR * i) * LDK + c8] = xq;
-        *(v8*)&sWr[(prow + PR * i) * LDK + c8] = xw;
+        *(v8*)&sQ[(prow + PR * i) * LDK + c8] = R.q[i];
+        *(v8*)&sW[(prow + PR * i) * LDK + c8] = R.w[i];
       }
-      // (the loaded pairs go through an opaque copy where they are consumed: otherwise the compiler carries a
-      // rearranged copy round the loop and waits for the load at the latch, right after issuing it)
-      t2 rd[4];
+      v8 x;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t u = __builtin_bit_cast(uint32_t, R.d[i]);
-        asm volatile("" : "+v"(u));
-        rd[i] = __builtin_bit_cast(t2, u);
-      }
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        v4 dv = v4{rd[0][j], rd[1][j], rd[2][j], rd[3][j]};
-        *(v4*)&sDoT[(uc2 + j) * LDT + urg * 4] = dv;
-      }
+      for (int j = 0; j < 8; ++j) x[j] = (T)((float)R.d[j] * egx);
+      *(v8*)&sDo[vrow * LDV + vc8] = x;
     };
     auto stage_y = [&](const YRegs& R, int64_t c) __attribute__((always_inline)) {
       const int L = chunk_len(c);
 #pragma unroll
-      for (int i = 0; i < NP; ++i) {
-        int row = prow + PR * i;
-        egx[i] = (row < L) ? __expf(R.gam[i]) : 0.f;
-        float e = (row < L) ? __expf(R.glast - R.gam[i]) : 0.f;
-        v8 kv;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) kv[j] = (T)((float)R.k[i][j] * e);
-        *(v8*)&sKh[row * LDK + c8] = kv;
-      }
-      t2 rl[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        uint32_t u = __builtin_bit_cast(uint32_t, R.dvl[i]);
-        asm volatile("" : "+v"(u));
-        rl[i] = __builtin_bit_cast(t2, u);
-      }
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        v4 dv = v4{rl[0][j], rl[1][j], rl[2][j], rl[3][j]};
-        if (L < BT) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (urg * 4 + i >= L) dv[i] = (T)0.f;
-        }
-        *(v4*)&sDvl[(uc2 + j) * LDT + urg * 4] = dv;
+      for (int i = 0; i < NP; ++i) *(v8*)&sK[(prow + PR * i) * LDK + c8] = R.k[i];
+      *(v8*)&sDvl[vrow * LDV + vc8] = R.dvl;
+      const float eg = vrow < L ? __expf(R.gam) : 0.f;
+      egx = p.scale * eg;
+      if ((st & 3) == 0) {
+        sEg[vrow] = eg;
+        sEd[vrow] = vrow < L ? __expf(R.glast - R.gam) : 0.f;
       }
       if (st == 0) sDec[c & 1] = __expf(R.glast);
     };
@@ -441,10 +396,9 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     load_y(nchunks - 1, Y);
     stage_y(Y, nchunks - 1);
     load_y(nchunks - 2, Y);
-    // The first chunk of the sequence (processed last) is peeled off so that the steady-state loop has no
-    // memory operation under a branch.
+    // The first chunk of the sequence (processed last) and its last one (processed first, possibly short) are
+    // peeled off so that the steady-state loop has no memory operation under a branch.
     if (nchunks > 1) {
-      // the sequence's last chunk, possibly short
       lds_barrier();  // B1(nchunks - 1)
       stage_x(X);
       load_x(nchunks - 2, X);
@@ -511,28 +465,33 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     if (nchunks > 0) publish(nchunks - 1);
     for (int64_t c = nchunks - 1; c >= 0; --c) {
       lds_barrier();  // B1(c)
-      // ---- dv2 = dv_loc + k^ dH : wave w owns rows 16w..16w+15, two 16-column tiles
+      // ---- dv2 = dv_loc + e^{gamma_last-gamma} * (k dH): wave w owns rows 16w..16w+15, two 16-column tiles
       {
         f32x4 d[2] = {zero4(), zero4()};
 #pragma unroll
         for (int ks = 0; ks < K; ks += 32) {
-          v8 a = lds_frag16<T>(sKh, LDK, wave * 16, ks, lane);
+          v8 a = lds_frag16<T>(sK, LDK, wave * 16, ks, lane);
 #pragma unroll
           for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, lds_frag16<T>(sDHt, LDK, j * 16, ks, lane), d[j]);
         }
         const int tr = wave * 16 + 4 * (lane >> 4);
+        const f32x4 ed = *(const f32x4*)&sEd[tr], eg = *(const f32x4*)&sEg[tr];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           int vc = j * 16 + (lane & 15);
-          v4 dl = *(const v4*)&sDvl[vc * LDT + tr];
-          v4 o;
+          v4 o, os;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[r] = (T)((float)dl[r] + d[j][r]);
+          for (int r = 0; r < 4; ++r) {
+            const float x = (float)sDvl[(tr + r) * LDV + vc] + ed[r] * d[j][r];
+            o[r] = (T)x;
+            os[r] = (T)(-eg[r] * x);
+          }
           *(v4*)&sDv2T[vc * LDT + tr] = o;
+          *(v4*)&sDv2s[vc * LDT + tr] = os;
         }
       }
       lds_barrier();  // B2(c)
-      // ---- dH <- e^{gamma_last} dH + q~^T do - w~^T dv2, in both orientations
+      // ---- dH <- e^{gamma_last} dH + q^T (s e^gamma * do) + w^T (-e^gamma * dv2), in both orientations
       const float dec_c = sDec[c & 1];
 #pragma unroll
       for (int a = 0; a < NKT; ++a) {
@@ -545,10 +504,10 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
           }
 #pragma unroll
           for (int s = 0; s < BT; s += 16) {
-            v8 fq = frag32_tr<T>(sQr, LDK, kt * 32, s, lane);
-            v8 fd = lds_frag32<T>(sDoT, LDT, 0, s, lane);
-            v8 fw = frag32_tr<T>(sWr, LDK, kt * 32, s, lane);
-            v8 f2 = lds_frag32<T>(sDv2T, LDT, 0, s, lane);
+            v8 fq = frag32_tr<T>(sQ, LDK, kt * 32, s, lane);
+            v8 fd = frag32_tr<T>(sDo, LDV, 0, s, lane);
+            v8 fw = frag32_tr<T>(sW, LDK, kt * 32, s, lane);
+            v8 f2 = lds_frag32<T>(sDv2s, LDT, 0, s, lane);
             acc[a] = Elem<T>::mfma32(fq, fd, acc[a]);
             acc[a] = Elem<T>::mfma32(fw, f2, acc[a]);
             acct[a] = Elem<T>::mfma32(fd, fq, acct[a]);
