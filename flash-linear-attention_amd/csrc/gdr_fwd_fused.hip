@@ -87,12 +87,18 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
   return __builtin_bit_cast(v8, u4{lo[0], hi[0], lo[1], hi[1]});
 }
 
-template <typename T, int K, bool KEEP>
+// NMW: matrix waves that carry state, 16 value columns each; the workgroup's slab is 16 NMW columns wide.  Four
+// (64 columns) is the form described above; two (32 columns, waves 2-3 only keep the barriers) doubles the number of
+// workgroups where 64-column slabs would leave half the CUs without one - a CU is fed at a fixed rate, and a
+// 32-column workgroup needs three quarters of the bytes of a 64-column one per chunk.
+template <typename T, int K, bool KEEP, int NMW = 4>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
-  constexpr int BV = 64;
+  constexpr int BV = 16 * NMW;
+  constexpr int RV = BV / 16;   // v, o: rows of a staging lane's 4-column piece
+  typedef T rvv __attribute__((ext_vector_type(RV)));
   constexpr int LDR = K + 8;  // pitch of the row-major k and q tiles
   constexpr int KS = K / 32;  // 32-wide contraction slices of the state
   constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
@@ -126,23 +132,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (q)
     constexpr int NPA = 2 * kTriElems / 4 / 256;             // 8-byte pieces of the triangular tiles per lane
     static_assert(NPA * 256 * 4 == 2 * kTriElems, "the triangular tiles split evenly over the staging lanes");
-    const int urg = st >> 4, uc4 = (st & 15) * 4;            // v, o: a lane owns 4 rows x 4 columns
+    const int urg = st / (BV / 4), uc4 = (st % (BV / 4)) * 4;   // v, o: a lane owns RV rows x 4 columns
     const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
     auto q_row = [&](int e) { return e / C8; };
     auto q_col = [&](int e) { return (e % C8) * 8; };
     struct Regs {
       v8 q[NPW], k[NPW];
       v4 a[NPA];
-      v4 v[4];
+      v4 v[RV];
       uint32_t gam;  // fp32 bits
     };
     // The steady state carries no address arithmetic: byte offsets of this lane's pieces from the
     // chunk's first row are computed once and the chunk base pointers advance by constant strides.
-    uint32_t offq[NPW], offv[4];
+    uint32_t offq[NPW], offv[RV];
 #pragma unroll
     for (int i = 0; i < NPW; ++i) offq[i] = 2 * ((uint32_t)q_row(st + 256 * i) * HK + q_col(st + 256 * i));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) offv[i] = 2 * ((uint32_t)(urg * 4 + i) * HV + uc4);
+    for (int i = 0; i < RV; ++i) offv[i] = 2 * ((uint32_t)(urg * RV + i) * HV + uc4);
     const uint32_t offg = 4 * (uint32_t)lane * H;
     const int64_t row00 = sp.bos * H + hh;
     const char* lq = (const char*)p.q + row00 * K * 2;
@@ -166,6 +172,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // unsigned minimum per load (zeroed before use), and past the last chunk the pointers stay on it.
     const uint32_t limq_full = 2 * ((uint32_t)(BT - 1) * HK), limq_last = 2 * ((uint32_t)(Llast - 1) * HK);
     const uint32_t limv_full = 2 * ((uint32_t)(BT - 1) * HV), limv_last = 2 * ((uint32_t)(Llast - 1) * HV);
+    static_assert(RV == 4 || RV == 2, "slab of 64 or 32 value columns");
     const uint32_t colq = 2 * (uint32_t)q_col(st), colv = 2 * (uint32_t)uc4;
     int lc = 0;  // chunk the load pointers are on
     auto load = [&](Regs& R) __attribute__((always_inline)) {
@@ -181,7 +188,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         R.k[i] = *(const v8*)(lk + o);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
+      for (int i = 0; i < RV; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
       R.gam = *(const uint32_t*)(lg + (offg < limg ? offg : limg));
       if (lc + 1 < nchunks) {
         lq += strk;
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int i = 0; i < NPW; ++i) dq[i] = q_row(st + 256 * i) * LDR + q_col(st + 256 * i);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * 4);
+    for (int j = 0; j < 4; ++j) dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * RV);
     int wc = 0;  // next chunk to write to LDS
     // maybe_last: the chunk may be the sequence's last, short one (rows past its end are zeroed)
     auto write = [&](Regs& R, auto maybe_last) __attribute__((always_inline)) {
@@ -211,8 +218,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
               for (int j = 0; j < 8; ++j) R.q[i][j] = R.k[i][j] = (T)0.f;
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (urg * 4 + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+          for (int i = 0; i < RV; ++i)
+            if (urg * RV + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
         }
       }
 #pragma unroll
@@ -223,8 +230,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = 0; i < NPW; ++i) *(v8*)&sK[b][dq[i]] = R.k[i];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        v4 vc = {R.v[0][j], R.v[1][j], R.v[2][j], R.v[3][j]};
-        *(v4*)&sVt[b][dv[j]] = vc;
+        rvv vc;
+#pragma unroll
+        for (int i = 0; i < RV; ++i) vc[i] = R.v[i][j];
+        *(rvv*)&sVt[b][dv[j]] = vc;
       }
       if (wave == 4) {
         // lanes past the end of a short chunk carry the last row's gate
@@ -241,18 +250,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int oc = 0;  // next chunk whose output is stored
     auto store_o = [&](auto maybe_last) __attribute__((always_inline)) {
       const int b = oc & 1;
-      v4 x[4];
+      rvv x[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x[j] = *(const v4*)&sVt[b][dv[j]];
+      for (int j = 0; j < 4; ++j) x[j] = *(const rvv*)&sVt[b][dv[j]];
       bool full = true;
       if constexpr (decltype(maybe_last)::value) full = oc != nchunks - 1 || Llast == BT;
       if (full) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+        for (int i = 0; i < RV; ++i) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
       } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (urg * 4 + i < Llast) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
+        for (int i = 0; i < RV; ++i)
+          if (urg * RV + i < Llast) *(v4*)(so + offv[i]) = v4{x[0][i], x[1][i], x[2][i], x[3][i]};
       }
       so += strv;
       ++oc;
@@ -301,6 +310,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     lds_barrier();
     store_o(any_chunk);
+  } else if (wave >= NMW) {
+    // waves without a share of the state keep the barrier count
+    if (nchunks > 0) {
+      lds_barrier();
+      for (int ci = 0; ci < nchunks; ++ci) lds_barrier();
+    }
   } else {
     // =========================== matrix waves ===========================
     const int cb = 16 * wave;  // first of this wave's 16 columns within the slab
@@ -512,16 +527,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 template <typename T>
 int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
-  const int64_t nblk = (int64_t)p.N * p.H * (p.V / 64);
-  FLA_REQUIRE(nblk <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  int64_t nblk = (int64_t)p.N * p.H * (p.V / 64);
+  FLA_REQUIRE(nblk <= 0x7fffffffLL / 2, FLA_E_UNSUPPORTED);
   if (nblk == 0) return FLA_OK;
+  // 32-column slabs while they still give every workgroup a CU of its own
+  const bool narrow = 2 * nblk <= kNumCUs;
+  if (narrow) nblk *= 2;
   dim3 grid((unsigned)nblk), block(512);
   const bool keep = p.v_new != nullptr;
-  if (K == 64 && keep) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64, true>), grid, block, 0, st, p);
-  else if (K == 64) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 64, false>), grid, block, 0, st, p);
-  else if (K == 128 && keep) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128, true>), grid, block, 0, st, p);
-  else if (K == 128) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, 128, false>), grid, block, 0, st, p);
+#define FLA_SCAN(KK, KEEPV)                                                                              \
+  if (narrow) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 2>), grid, block, 0, st, p);          \
+  else hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 4>), grid, block, 0, st, p);
+  if (K == 64 && keep) { FLA_SCAN(64, true) }
+  else if (K == 64) { FLA_SCAN(64, false) }
+  else if (K == 128 && keep) { FLA_SCAN(128, true) }
+  else if (K == 128) { FLA_SCAN(128, false) }
   else return FLA_E_UNSUPPORTED;
+#undef FLA_SCAN
   FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
