@@ -67,11 +67,10 @@ struct StageLds {
 // (left in L.o by the matrix waves) to memory as whole rows, and one more barrier + store follows the last chunk.
 // SG: one log-gate per (token, head), p.g is fp32 [B*T, H]: a lane loads one word per row and uses it for all
 // its key channels, so the prefix sums and exponentials of a row are formed once.
-template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O>
+template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O, int BV = 64>
 FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, const SeqSpan& sp, int64_t nchunks,
                                 int hh, int vbase, int wave, int lane, int tid) {
   typedef typename Elem<T>::v8 v8;
-  constexpr int BV = 64;
   constexpr int LDK = K + 8;
   constexpr int CPW = K / NSTG;                // key columns per staging wave
   constexpr int CPL = CPW / 4;                 // key columns per staging lane (8 for K=128, 4 for K=64)
@@ -277,15 +276,16 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
   };
 
   // The matrix waves leave each finished output tile in LDS; the staging waves write it to
-  // memory one chunk period later as whole 128-byte rows (8 lanes x 16 bytes per row).
+  // memory one chunk period later as whole rows of the slab (BV / 8 lanes x 16 bytes per row).
   constexpr int NPO = BT * (BV / 8) / (64 * NSTG);
+  static_assert(NPO >= 1, "output pieces per staging lane");
   const uint32_t opitch = (uint32_t)H * V * (uint32_t)sizeof(T);
   uint32_t offo[NPO];
   int ldo[NPO];
-  const int ocol = (tid & 7) * 8;   // element offset inside a row: the same for every piece of a lane
+  const int ocol = (tid & (BV / 8 - 1)) * 8;   // element offset inside a row: the same for every piece of a lane
 #pragma unroll
   for (int i = 0; i < NPO; ++i) {
-    const int orow = ((tid - 256) + 64 * NSTG * i) >> 3;
+    const int orow = ((tid - 256) + 64 * NSTG * i) / (BV / 8);
     ldo[i] = orow * LDT + ocol;
     offo[i] = (uint32_t)orow * opitch + (uint32_t)ocol * (uint32_t)sizeof(T);
   }

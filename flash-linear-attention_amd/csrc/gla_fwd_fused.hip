@@ -31,13 +31,17 @@ namespace {
 // the backward pass.
 // SG: one log-gate per (token, head), p.g is fp32 [B*T, H] (the simple-GLA / RetNet-style decay): a lane loads one
 // word per row and uses it for all its key channels, so the prefix sums and exponentials of a row are formed once.
-template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false>
+// NVT: 32-column value tiles of the workgroup's slab.  Two (64 columns) is the form described above; one (32 columns,
+// the matrix waves with cw = 1 only form their score quadrant) doubles the number of workgroups where 64-column slabs
+// would leave half the CUs without one: a CU is fed at a fixed rate, and a 32-column workgroup needs five sixths of
+// the bytes of a 64-column one per chunk (three quarters when it also writes the states).
+template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false, int NVT = 2>
 __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
   static_assert(!SG || sizeof(GT) == 4, "per-head gates are fp32");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   typedef T t2 __attribute__((ext_vector_type(2)));
-  constexpr int BV = 64;
+  constexpr int BV = 32 * NVT;
   constexpr int LDK = K + 8;
   constexpr int KT32 = K / 32;                 // 32-row state tiles
   constexpr int NKT = (KT32 + 3) / 4;          // state tiles per matrix wave (x2 value tiles)
@@ -51,7 +55,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   __shared__ __attribute__((aligned(16))) T sVt[2][BV * LDT];    // v   [v][t]
   __shared__ __attribute__((aligned(16))) float sDecay[2][K];
   __shared__ __attribute__((aligned(16))) T sP[BT * LDT];        // tril(S) [i][j]
-  __shared__ __attribute__((aligned(16))) T sHf[KT32 * 2 * 64 * 16];  // state, fragment order [kt][vt][lane][16]
+  __shared__ __attribute__((aligned(16))) T sHf[KT32 * NVT * 64 * 16];  // state, fragment order [kt][vt][lane][16]
   __shared__ __attribute__((aligned(16))) T sO[BT * LDT];        // finished output tile [t][v]
   __shared__ int sWide[2][NSTG];                                   // per staging wave: gates out of range
 
@@ -77,15 +81,15 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   if (wave >= 4) {
     // staging waves: see gla_fused_staging.h
     StageLds<T> L{{sQ[0], sQ[1]}, {sK[0], sK[1]}, {sKh[0], sKh[1]}, {sDecay[0], sDecay[1]}, {sWide[0], sWide[1]}, sO};
-    gla_stage_waves<T, GT, K, NSTG, SG, true>(p, L, sp, nchunks, hh, vbase, wave, lane, tid);
+    gla_stage_waves<T, GT, K, NSTG, SG, true, BV>(p, L, sp, nchunks, hh, vbase, wave, lane, tid);
   } else {
     // =========================== matrix waves ===========================
     const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
-    f32x16 acc[NKT][2];                         // state tiles kt = wave + 4a, value tiles 0/1
+    f32x16 acc[NKT][NVT];                       // state tiles kt = wave + 4a, value tiles 0 .. NVT-1
 #pragma unroll
     for (int a = 0; a < NKT; ++a)
 #pragma unroll
-      for (int vt = 0; vt < 2; ++vt) {
+      for (int vt = 0; vt < NVT; ++vt) {
         acc[a][vt] = zero16();
         int kt = wave + 4 * a;
         if (p.h0 && kt < KT32) {
@@ -117,7 +121,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           int kt = wave + 4 * a;
           if (kt < KT32) {
 #pragma unroll
-            for (int vt = 0; vt < 2; ++vt) {
+            for (int vt = 0; vt < NVT; ++vt) {
               v8 lo, hi;
 #pragma unroll
               for (int r = 0; r < 8; ++r) {
@@ -145,14 +149,14 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         int kt = wave + 4 * a;
         if (kt < KT32) {
 #pragma unroll
-          for (int vt = 0; vt < 2; ++vt) {
+          for (int vt = 0; vt < NVT; ++vt) {
             v8 lo, hi;
 #pragma unroll
             for (int r = 0; r < 8; ++r) {
               lo[r] = (T)acc[a][vt][r];
               hi[r] = (T)acc[a][vt][r + 8];
             }
-            T* dst = &sHf[((kt * 2 + vt) * 64 + lane) * 16];
+            T* dst = &sHf[((kt * NVT + vt) * 64 + lane) * 16];
             *(v8*)dst = lo;
             *(v8*)(dst + 8) = hi;
           }
@@ -160,43 +164,45 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     };
     publish_state();
-    // The matrix waves also stage the value tile (time-contiguous) of the next chunk: 8 rows x
+    // The matrix waves also stage the value tile (time-contiguous) of the next chunk: RPV rows x
     // 2 columns per lane, loaded one chunk period ahead.
-    const int vrg = tid >> 5, vc = (tid & 31) * 2;
+    constexpr int RPV = BV / 8;   // 8 rows of 64 columns, 4 rows of 32
+    typedef T rpv __attribute__((ext_vector_type(RPV)));
+    const int vrg = tid / (BV / 2), vc = (tid % (BV / 2)) * 2;
     const uint32_t vpitch = (uint32_t)H * V * (uint32_t)sizeof(T);
     const char* lv = (const char*)p.v + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
     const int64_t strv = (int64_t)BT * vpitch;
     const int Llast = (int)(sp.len - (nchunks - 1) * BT);
-    uint32_t offv[8];
+    uint32_t offv[RPV];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) offv[i] = (uint32_t)(vrg * 8 + i) * vpitch + (uint32_t)vc * (uint32_t)sizeof(T);
+    for (int i = 0; i < RPV; ++i) offv[i] = (uint32_t)(vrg * RPV + i) * vpitch + (uint32_t)vc * (uint32_t)sizeof(T);
     const uint32_t vlim_full = (uint32_t)(BT - 1) * vpitch, vlim_last = (uint32_t)(Llast - 1) * vpitch;
     int64_t lvc = 0;  // chunk the value pointer is on (stays on the last one)
-    t2 vreg[8];
+    t2 vreg[RPV];
     auto load_v = [&]() __attribute__((always_inline)) {
       const uint32_t lim = (lvc >= nchunks - 1 ? vlim_last : vlim_full) + (uint32_t)vc * (uint32_t)sizeof(T);
 #pragma unroll
-      for (int i = 0; i < 8; ++i)   // read once by this workgroup only (q, k, g are read by both slabs of a head)
+      for (int i = 0; i < RPV; ++i)   // read once by this workgroup only (q, k, g are read by every slab of a head)
         vreg[i] = __builtin_nontemporal_load((const t2*)(lv + (offv[i] < lim ? offv[i] : lim)));
       if (lvc + 1 < nchunks) lv += strv;
       ++lvc;
     };
-    const int dv0 = (vc + 0) * LDT + vrg * 8, dv1 = (vc + 1) * LDT + vrg * 8;
+    const int dv0 = (vc + 0) * LDT + vrg * RPV, dv1 = (vc + 1) * LDT + vrg * RPV;
     auto stage_v = [&](int buf, int64_t c) __attribute__((always_inline)) {
       const int L = chunk_len(c);
-      v8 a, b;
+      rpv a, b;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < RPV; ++i) {
         a[i] = vreg[i][0];
         b[i] = vreg[i][1];
       }
       if (L < BT) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (vrg * 8 + i >= L) a[i] = b[i] = (T)0.f;
+        for (int i = 0; i < RPV; ++i)
+          if (vrg * RPV + i >= L) a[i] = b[i] = (T)0.f;
       }
-      *(v8*)&sVt[buf][dv0] = a;
-      *(v8*)&sVt[buf][dv1] = b;
+      *(rpv*)&sVt[buf][dv0] = a;
+      *(rpv*)&sVt[buf][dv1] = b;
     };
     if (nchunks > 0) {
       load_v();
@@ -220,9 +226,9 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         if (wide) {
           // hand the state entering this chunk to the exact kernel (fragment order, this slab's columns)
           T* hw = (T*)p.hwide + ((chunk0 + c) * H + hh) * (int64_t)K * V;
-          for (int e = tid; e < KT32 * 2 * 64 * 2; e += 256) {
-            int piece = e & 1, ln = (e >> 1) & 63, tile = e >> 7;  // tile = kt*2 + vt
-            int kt = tile >> 1, vt = tile & 1;
+          for (int e = tid; e < KT32 * NVT * 64 * 2; e += 256) {
+            int piece = e & 1, ln = (e >> 1) & 63, tile = e >> 7;  // tile = kt*NVT + vt
+            int kt = tile / NVT, vt = tile % NVT;
             v8 x = *(const v8*)&sHf[(tile * 64 + ln) * 16 + piece * 8];
             *(v8*)(hw + (((int64_t)kt * (V / 32) + (vbase / 32 + vt)) * 64 + ln) * 16 + piece * 8) = x;
           }
@@ -240,13 +246,15 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
                               frag32_swz<T>(sQ[buf], LDK, qi * 32, ks, lane), s);
       }
       f32x16 o = zero16();
+      if (cw < NVT) {
 #pragma unroll
       for (int kt = 0; kt < KT32; ++kt) {
-        const T* hf = &sHf[((kt * 2 + cw) * 64 + lane) * 16];
+        const T* hf = &sHf[((kt * NVT + cw) * 64 + lane) * 16];
         v8 h0v = *(const v8*)hf, h1v = *(const v8*)(hf + 8);
         // transposed product (h^T q~^T): a lane ends up with four consecutive value columns of one row
         o = Elem<T>::mfma32(h0v, frag32_perm_swz<T>(sQ[buf], LDK, rw * 32, kt * 32, lane), o);
         o = Elem<T>::mfma32(h1v, frag32_perm_swz<T>(sQ[buf], LDK, rw * 32, kt * 32 + 16, lane), o);
+      }
       }
       {
         const int i = qi * 32 + (lane & 31);
@@ -271,6 +279,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
       lds_barrier();  // B2(c): P visible; nobody reads the state fragments any more
+      if (cw < NVT) {
       if (rw == 0) {
 #pragma unroll
         for (int js = 0; js < 32; js += 16)
@@ -292,6 +301,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           *(v4*)(orow_ + 8 * r4) = ov;
         }
       }
+      }
       // ---- state update
 #pragma unroll
       for (int a = 0; a < NKT; ++a) {
@@ -302,16 +312,16 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
             f32x4 d = *(const f32x4*)&sDecay[buf][kt * 32 + 8 * q4 + 4 * (lane >> 5)];
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
-              acc[a][0][4 * q4 + b] *= d[b];
-              acc[a][1][4 * q4 + b] *= d[b];
+#pragma unroll
+              for (int vt = 0; vt < NVT; ++vt) acc[a][vt][4 * q4 + b] *= d[b];
             }
           }
 #pragma unroll
           for (int ts = 0; ts < BT; ts += 16) {
             v8 fk = lds_frag32<T>(sKh[buf], LDT, kt * 32, ts, lane);
-            v8 fv0 = lds_frag32<T>(sVt[buf], LDT, 0, ts, lane), fv1 = lds_frag32<T>(sVt[buf], LDT, 32, ts, lane);
-            acc[a][0] = Elem<T>::mfma32(fk, fv0, acc[a][0]);
-            acc[a][1] = Elem<T>::mfma32(fk, fv1, acc[a][1]);
+#pragma unroll
+            for (int vt = 0; vt < NVT; ++vt)
+              acc[a][vt] = Elem<T>::mfma32(fk, lds_frag32<T>(sVt[buf], LDT, 32 * vt, ts, lane), acc[a][vt]);
           }
         }
       }
@@ -325,7 +335,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         int kt = wave + 4 * a;
         if (kt < KT32) {
 #pragma unroll
-          for (int vt = 0; vt < 2; ++vt)
+          for (int vt = 0; vt < NVT; ++vt)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
               htp[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + vt * 32 + (lane & 31)] = acc[a][vt][r];
@@ -557,16 +567,25 @@ int launch_fused(const FusedParams& p, int K, hipStream_t st) {
     FLA_CHECK_LAUNCH();
     return FLA_OK;
   }
+  // 32-column slabs for a forward that keeps the states, while they still give every workgroup a CU of its own
+  // (205 -> 187 us at B=4, H=16, T=4096; without the state stores the chunk period is set by the gating work of
+  // the staging waves, which does not shrink with the slab: 157 against 158 us)
+  const bool narrow = p.hT != nullptr && 2 * total <= kNumCUs;
+  if (narrow) total *= 2;
   dim3 grid((unsigned)total);
+#define FLA_FUSED(KK, HTV)                                                                                     \
+  if (narrow) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, KK, 4, HTV, SG, 1>), grid, dim3(512), 0, st, p);  \
+  else hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, KK, 4, HTV, SG, 2>), grid, dim3(512), 0, st, p);
   if (p.hT) {
-    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, true, SG>), grid, dim3(512), 0, st, p);
-    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, true, SG>), grid, dim3(512), 0, st, p);
+    if (K == 128) { FLA_FUSED(128, true) }
+    else if (K == 64) { FLA_FUSED(64, true) }
     else return FLA_E_UNSUPPORTED;
   } else {
-    if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, false, SG>), grid, dim3(512), 0, st, p);
-    else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, false, SG>), grid, dim3(512), 0, st, p);
+    if (K == 128) { FLA_FUSED(128, false) }
+    else if (K == 64) { FLA_FUSED(64, false) }
     else return FLA_E_UNSUPPORTED;
   }
+#undef FLA_FUSED
   FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
