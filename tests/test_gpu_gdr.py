@@ -359,3 +359,41 @@ def test_chunk_gdr_gradients_are_reproducible(device, varlen):
         again = _grads_dev(device, q, k, v, g, beta, h0, do, dht, offsets=offs)
         for name, a, b in zip(NAMES, first, again):
             assert torch.equal(a, b), name
+
+
+def test_chunk_gdr_slab_width_independence(device):
+    """B=4 x H=16 puts the scan on 32-column slabs (128 workgroups of 64 columns would leave half the CUs idle),
+    the same batch stacked twice on 64-column slabs; the delta rule is independent per value column, so outputs
+    and final states of the first four sequences agree bit for bit.  Also against the recurrence on one pair."""
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    B, T, H, D = 4, 1024, 16, 128
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, D, D, seed=71)
+    print("chunk_gdr slab-width independence B=4 vs B=8", flush=True)
+    o4, ht4 = _run(device, q, k, v, g, beta, h0)
+    twice = lambda x: torch.cat([x, x], 0)
+    o8, ht8 = _run(device, twice(q), twice(k), twice(v), twice(g), twice(beta), twice(h0))
+    assert torch.equal(o8[:B], o4) and torch.equal(o8[B:], o4)
+    assert torch.equal(ht8[:B], ht4) and torch.equal(ht8[B:], ht4)
+    b, h = 3, 11
+    sl = lambda x: x[b:b + 1, :, h:h + 1]
+    ro, rht = naive_recurrent_gated_delta_rule(sl(q), sl(k), sl(v), sl(g), sl(beta), initial_state=h0[b:b + 1, h:h + 1],
+                                               output_final_state=True)
+    assert_close("o[3,11]", ro, o4[b:b + 1, :, h:h + 1], TOL_O)
+    assert_close("ht[3,11]", rht, ht4[b:b + 1, h:h + 1], TOL_HT)
+
+
+def test_chunk_gdr_slab_width_independence_backward(device):
+    """The same for a forward that keeps its intermediates and the backward that reads them: gradients of the
+    batch stacked twice (64-column slabs) equal those of the batch alone (32-column slabs) bit for bit, except the
+    gradients shared by nothing (all of them are per sequence)."""
+    B, T, H, D = 4, 512, 16, 128
+    gen = torch.Generator().manual_seed(72)
+    q, k, v, g, beta, h0 = gdr_inputs(B, T, H, D, D, seed=72)
+    do = torch.randn(B, T, H, D, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    print("chunk_gdr slab-width independence (backward) B=4 vs B=8", flush=True)
+    twice = lambda x: torch.cat([x, x], 0)
+    g4 = _grads_dev(device, q, k, v, g, beta, h0, do, dht)
+    g8 = _grads_dev(device, twice(q), twice(k), twice(v), twice(g), twice(beta), twice(h0), twice(do), twice(dht))
+    for name, a, b in zip(NAMES, g4, g8):
+        assert torch.equal(b[:B], a) and torch.equal(b[B:], a), name
