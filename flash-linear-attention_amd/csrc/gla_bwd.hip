@@ -39,7 +39,147 @@ struct BDhParams {
   int64_t total_chunks;
   int H, K, V, N;
   float scale;
+  const void* qg;      // optional: the gated queries q e^{G} the forward staged, [rows, H, K] in the q dtype
+  const float* decay;  //   and e^{G_last} per chunk, [chunks, H, K]
 };
+
+// The same scan from what a states-keeping forward left behind: dH_c = e^{G_last} dH_{c+1} + s (q e^{G})^T do with
+// the gated queries and the decay factors read back instead of being formed from q and g again - no prefix sums,
+// no exponentials, 16-byte loads (5 memory instructions per lane and chunk instead of 24) and half the bytes.  The
+// tiles are plain row-major copies; both operands of the update contract over time, i.e. over the tiles' rows,
+// and come out of LDS through the transposing load.  The scale is kept out of the operands: the accumulators
+// carry dH / s (the incoming d ht is divided by s, every copy that leaves is multiplied by it).
+template <typename T>
+__global__ __launch_bounds__(256) void gla_bwd_dh_qg_kernel(BDhParams p) {
+  typedef typename Elem<T>::v8 v8;
+  __shared__ __attribute__((aligned(16))) T sQ[2][64 * LDT];  // [t][k] q e^{G}
+  __shared__ __attribute__((aligned(16))) T sD[2][64 * LDT];  // [t][v] do
+  __shared__ __attribute__((aligned(16))) float sDecay[2][64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int H = p.H, K = p.K, V = p.V;
+  const int nkt = K / 64, nvt = V / 64, ntile = nkt * nvt;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile = (int)(id % ntile);
+  const int nh = (int)(id / ntile);
+  const int n = nh / H, hh = nh % H;
+  const int kbase = (tile % nkt) * 64, vbase = (tile / nkt) * 64;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+
+  // a lane owns two 16-byte pieces of each tile: rows prow and prow + 32, columns c8 ..
+  const int prow = tid >> 3, c8 = (tid & 7) * 8;
+  const char* qp = (const char*)((const T*)p.qg + (sp.bos * H + hh) * (int64_t)K + kbase + c8);
+  const char* dp = (const char*)((const T*)p.dout + (sp.bos * H + hh) * (int64_t)V + vbase + c8);
+  const float* cp = p.decay + (chunk0 * H + hh) * (int64_t)K + kbase + (tid & 63);
+  const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
+  const int64_t strideC = (int64_t)H * K;
+
+  const int kq = wave & 1, vq = wave >> 1;
+  const int kt32 = kbase / 32 + kq, vt32 = vbase / 32 + vq;
+  const int kcol = kbase + kq * 32 + (lane & 31);
+  // An empty sequence hands d ht through to d h0 bit for bit: no factor goes on and off it.
+  const float scale = nchunks > 0 ? p.scale : 1.f, inv_scale = 1.f / scale;
+  f32x16 acc2 = zero16();  // rows v, cols k: dH / s
+  if (p.dht) {
+    const float* dp0 = p.dht + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc2[r] = dp0[(int64_t)kcol * V + vbase + vq * 32 + c32_row(r, lane)] * inv_scale;
+  }
+  struct Regs {
+    v8 q[2], d[2];
+    float dec;
+  };
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+  // Every load is unconditional: rows past the end of a short (last) chunk are redirected to its last row and
+  // their do rows zeroed where they are staged (the forward did not write gated queries there).
+  auto load_chunk = [&](int64_t c, Regs& R) {
+    const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+    const char* qb = qp + c * BT * (int64_t)pitchK;
+    const char* db = dp + c * BT * (int64_t)pitchV;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t row = (uint32_t)(prow + 32 * i) < last ? (uint32_t)(prow + 32 * i) : last;
+      R.q[i] = *(const v8*)(qb + row * pitchK);
+      R.d[i] = *(const v8*)(db + row * pitchV);
+    }
+    R.dec = cp[c * strideC];
+  };
+  // One barrier per chunk, tiles double-buffered in LDS; two register sets, each refilled right after the
+  // staging step that consumed it.
+  auto step = [&](int64_t c, Regs& R, auto more) {
+    const int buf = (int)(c & 1);
+    const int L = chunk_len(c);
+    // ---- gradient w.r.t. the state leaving chunk c, transposed fragment order
+    {
+      int64_t blk = ((chunk0 + c) * H + hh) * (int64_t)K * V;
+      v8 lo, hi;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        lo[r] = (T)(acc2[r] * scale);
+        hi[r] = (T)(acc2[r + 8] * scale);
+      }
+      T* o2 = (T*)p.dhtf + blk + (((int64_t)vt32 * (K / 32) + kt32) * 64 + lane) * 16;
+      *(v8*)o2 = lo;
+      *(v8*)(o2 + 8) = hi;
+    }
+    const v8 z8 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = prow + 32 * i;
+      *(v8*)&sQ[buf][row * LDT + c8] = R.q[i];
+      *(v8*)&sD[buf][row * LDT + c8] = row < L ? R.d[i] : z8;
+    }
+    if (tid < 64) sDecay[buf][tid] = R.dec;
+    if constexpr (decltype(more)::value) {
+      load_chunk(c >= 2 ? c - 2 : 0, R);
+      asm volatile("" ::: "memory");  // the loads stay here, ahead of the barrier
+    }
+    lds_barrier();
+    {
+      const float d = sDecay[buf][kq * 32 + (lane & 31)];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc2[r] *= d;
+    }
+#pragma unroll
+    for (int s = 0; s < BT; s += 16) {
+      v8 fq = frag32_tr<T>(sQ[buf], LDT, kq * 32, s, lane);
+      v8 fd = frag32_tr<T>(sD[buf], LDT, vq * 32, s, lane);
+      acc2 = Elem<T>::mfma32(fd, fq, acc2);
+    }
+  };
+  Regs R0, R1;
+  if (nchunks > 0) {
+    load_chunk(nchunks - 1, R0);
+    asm volatile("" ::: "memory");
+    load_chunk(nchunks > 1 ? nchunks - 2 : 0, R1);
+    asm volatile("" ::: "memory");
+    int64_t c = nchunks - 1;
+    for (; c >= 3; c -= 2) {
+      step(c, R0, std::true_type{});
+      step(c - 1, R1, std::true_type{});
+    }
+    if (c == 2) {
+      step(2, R0, std::true_type{});
+      step(1, R1, std::false_type{});
+      step(0, R0, std::false_type{});
+    } else {
+      step(c, R0, std::false_type{});
+      if (c == 1) step(0, R1, std::false_type{});
+    }
+  }
+  if (p.dh0) {
+    float* o = p.dh0 + (int64_t)nh * K * V;
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4)
+      *(f32x4*)&o[(int64_t)kcol * V + vbase + vq * 32 + 8 * r4 + 4 * (lane >> 5)] =
+          f32x4{acc2[4 * r4] * scale, acc2[4 * r4 + 1] * scale, acc2[4 * r4 + 2] * scale, acc2[4 * r4 + 3] * scale};
+  }
+}
 
 template <typename T, typename GT>
 __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
@@ -1042,8 +1182,8 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
 
 template <typename T, typename GT>
 int launch_bwd(const void* q, const void* k, const void* v, const void* g, const void* dout, const float* dht,
-               const void* hT, void* dhtf, void* dq, void* dk, void* dv, float* dg, float* dh0,
-               const int* wide,
+               const void* hT, const void* qg, const float* decay, void* dhtf, void* dq, void* dk, void* dv, float* dg,
+               float* dh0, const int* wide,
                const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
                int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
   dim3 grid;
@@ -1054,10 +1194,11 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
   const int64_t total_chunks = grid.x;
   {
     BDhParams p{q, g, dout, dht, dhtf, dh0, offsets, chunk_offsets, T_, total_chunks,
-                (int)H, (int)K, (int)V, (int)N, scale};
+                (int)H, (int)K, (int)V, (int)N, scale, qg, decay};
     int64_t total = (K / 64) * (V / 64) * N * H;
     FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
-    hipLaunchKernelGGL((gla_bwd_dh_kernel<T, GT>), dim3((unsigned)total), dim3(256), 0, st, p);
+    if (qg) hipLaunchKernelGGL((gla_bwd_dh_qg_kernel<T>), dim3((unsigned)total), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((gla_bwd_dh_kernel<T, GT>), dim3((unsigned)total), dim3(256), 0, st, p);
     FLA_CHECK_LAUNCH();
   }
   {
@@ -1102,26 +1243,27 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
 
 }  // namespace
 
-extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
-                                 const float* dht, const void* hT, void* dh_frag_t,
-                                 void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
-                                 const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
-                                 int64_t NT, int qkv_dtype,
-                                 int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
-                                 float scale, fla_stream_t stream) {
+static int gla_bwd_impl(const void* q, const void* k, const void* v, const void* gates, const void* dout,
+                        const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
+                        void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                        const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                        int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                        int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag_t && dq && dk && dv && dg,
               FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
+  FLA_REQUIRE((q_gated == nullptr) == (chunk_decay == nullptr), FLA_E_INVALID);
+  if (q_gated) FLA_REQUIRE(scale != 0.f, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)dout | (uintptr_t)hT |
                (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
-               (uintptr_t)dg) % 16 == 0,
+               (uintptr_t)dg | (uintptr_t)q_gated) % 16 == 0,
               FLA_E_ALIGNMENT);
   hipStream_t st = (hipStream_t)stream;
 #define FLA_BWD(TT, GG)                                                                                           \
-  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, dh_frag_t, dq, dk, dv, dg, dh0, wide,   \
+  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dh0, wide,   \
                             offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_BWD(bf16, float);
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_BWD(bf16, bf16);
@@ -1129,4 +1271,27 @@ extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, co
   if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F16) FLA_BWD(f16, f16);
 #undef FLA_BWD
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* gates, const void* dout,
+                                 const float* dht, const void* hT, void* dh_frag_t,
+                                 void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                                 const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
+                                 int64_t NT, int qkv_dtype,
+                                 int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                 float scale, fla_stream_t stream) {
+  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, nullptr, nullptr, dh_frag_t, dq, dk, dv, dg, dh0, wide, offsets,
+                      indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const void* gates,
+                                      const void* dout, const float* dht, const void* hT, const void* q_gated,
+                                      const float* chunk_decay, void* dh_frag_t, void* dq, void* dk, void* dv,
+                                      float* dg, float* dh0, const int* wide, const int64_t* offsets,
+                                      const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                                      int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
+                                      int64_t V, int64_t N, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q_gated && chunk_decay, FLA_E_INVALID);
+  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dh0, wide,
+                      offsets, indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
 }

@@ -22,6 +22,8 @@ struct FusedParams {
   int H, V, N;
   float scale;
   void* hT;         // HT variant: the state entering every chunk, FLA_H_FRAGMENT_T order, [chunks, H, K*V]
+  void* qg;         // HT variant, optional: the gated queries q e^{G} as staged, [rows, H, K] in the q dtype
+  float* decay;     //   and e^{G_last} of every chunk, [chunks, H, K] (both or neither)
 };
 
 // The row-major q~ / k~ tiles are written by lanes that own four adjacent rows each, i.e.

@@ -143,6 +143,24 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
     };
+    // HT: the gated queries of a chunk and its decay factors, as the staging waves left them in LDS, for a
+    // backward pass whose reverse state scan then streams them instead of forming prefix sums and exponentials
+    // of its own.  The slabs of a head share the rows out; rows past the end of a short chunk are not written.
+    auto store_qg = [&](int buf, int64_t c) {
+      if constexpr (HT) {
+        if (p.qg) {
+          constexpr int C8 = K / 8;
+          const int nrow = BT / nvb > 0 ? BT / nvb : 0, r0 = vb * nrow;
+          const int L = chunk_len(c);
+          T* qb = (T*)p.qg + ((sp.bos + c * BT) * H + hh) * (int64_t)K;
+          for (int e = tid; e < nrow * C8; e += 256) {
+            const int row = r0 + e / C8, c8 = (e % C8) * 8;
+            if (row < L) *(v8*)(qb + (int64_t)row * H * K + c8) = *(const v8*)&sQ[buf][row * LDK + swz_rm(row, c8)];
+          }
+          if (vb == 0 && tid < K) p.decay[((chunk0 + c) * H + hh) * (int64_t)K + tid] = sDecay[buf][tid];
+        }
+      }
+    };
     auto publish_state = [&]() {
 #pragma unroll
       for (int a = 0; a < NKT; ++a) {
@@ -218,6 +236,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         load_v();
       }
       store_ht(c);  // unconditional and a whole chunk period ahead of the next wait for the value loads
+      store_qg(buf, c);
       if (p.wide) {
         int wide = 0;
 #pragma unroll
@@ -593,7 +612,8 @@ int launch_fused(const FusedParams& p, int K, hipStream_t st) {
 }  // namespace
 
 static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const void* gates, const float* h0,
-                              void* o, float* ht, int* ws_wide, void* ws_hwide, void* h_frag_t, const int64_t* offsets,
+                              void* o, float* ht, int* ws_wide, void* ws_hwide, void* h_frag_t, void* qg,
+                              float* decay, const int64_t* offsets,
                               const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                               int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false,
@@ -612,8 +632,10 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     FLA_REQUIRE((uintptr_t)h_frag_t % 16 == 0, FLA_E_ALIGNMENT);
     if (offsets) FLA_REQUIRE(chunk_offsets != nullptr, FLA_E_INVALID);
   }
+  FLA_REQUIRE((qg == nullptr) == (decay == nullptr), FLA_E_INVALID);
+  if (qg) FLA_REQUIRE(h_frag_t != nullptr && (uintptr_t)qg % 16 == 0 && V <= 256, FLA_E_INVALID);
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
-                T, (int)H, (int)V, (int)N, scale, h_frag_t};
+                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;
@@ -656,7 +678,7 @@ extern "C" int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void*
                                        const int64_t* seq_order, int64_t NT,
                                        int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                                        int64_t V, int64_t N, float scale, fla_stream_t stream) {
-  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, offsets, indices, chunk_offsets,
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, nullptr, nullptr, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
 }
 
@@ -666,7 +688,7 @@ extern "C" int fla_chunk_gla_fwd_fused_first_launch(const void* q, const void* k
                                                     const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                                                     int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
                                                     int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
-  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, offsets, indices, chunk_offsets,
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, nullptr, nullptr, nullptr, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream, false, false);
 }
 
@@ -677,8 +699,20 @@ extern "C" int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, cons
                                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
                                               int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(h_frag_t, FLA_E_INVALID);
-  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, offsets, indices, chunk_offsets,
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, nullptr, nullptr, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const void* v, const void* gates,
+                                            const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                            void* h_frag_t, void* q_gated, float* chunk_decay, const int64_t* offsets,
+                                            const int64_t* indices, const int64_t* chunk_offsets,
+                                            const int64_t* seq_order, int64_t NT, int qkv_dtype, int gate_dtype,
+                                            int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                            float scale, fla_stream_t stream) {
+  FLA_REQUIRE(h_frag_t && q_gated && chunk_decay, FLA_E_INVALID);
+  return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, q_gated, chunk_decay, offsets,
+                            indices, chunk_offsets, seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
 }
 
 extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, const float* g,
@@ -687,6 +721,6 @@ extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, cons
                                               const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                                               int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                                               int64_t N, float scale, fla_stream_t stream) {
-  return gla_fwd_fused_impl(q, k, v, g, h0, o, ht, ws_wide, ws_hwide, h_frag_t, offsets, indices, chunk_offsets,
+  return gla_fwd_fused_impl(q, k, v, g, h0, o, ht, ws_wide, ws_hwide, h_frag_t, nullptr, nullptr, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true);
 }

@@ -188,7 +188,9 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     single-reference range are detected on the device and recomputed exactly; ``return_flags``
     also returns the int32 ``[chunks, H]`` flags (for the backward pass).  With a list
     ``states_out`` the launch also writes the state entering every chunk (transposed fragment
-    order, what the backward kernels read) and appends it.  ``head_gates``: ``g`` is one fp32 log-gate
+    order, what the backward kernels read) and appends it, followed (per-key gates only) by the gated queries
+    ``q e^{G}`` ``[B,T,H,K]`` and the chunk decays ``e^{G_last}`` ``[chunks,H,K]`` the backward's reverse state scan
+    streams (``fla_chunk_gla_fwd_fused_kept``).  ``head_gates``: ``g`` is one fp32 log-gate
     per (token, head), ``[B,T,H]`` (``fla_chunk_simple_gla_fwd_fused``)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
@@ -218,9 +220,17 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), *tail[:5], be.dt(q), *tail[7:]),
                  "fla_chunk_simple_gla_fwd_fused")
     elif states_out is not None:
-        hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
-        be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
-        states_out.append(hT)
+        nt = plan.NT if plan is not None else -(-T // BT)
+        hT = q.new_empty(B, nt, H, K, V)
+        if V <= 256:
+            qg = torch.empty_like(q)
+            decay = q.new_empty(B, nt, H, K, dtype=torch.float32)
+            be.check(be.lib().fla_chunk_gla_fwd_fused_kept(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), *tail),
+                     "fla_chunk_gla_fwd_fused_kept")
+            states_out.extend((hT, qg, decay))
+        else:
+            be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
+            states_out.append(hT)
     elif first_launch_only:   # benchmark hook: the scan without the guard's second launch
         be.check(be.lib().fla_chunk_gla_fwd_fused_first_launch(*head, *tail), "fla_chunk_gla_fwd_fused_first_launch")
     else:
@@ -313,10 +323,12 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
     return g_cumsum, A, h, ht, o
 
 
-def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None, hT=None):
+def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None, hT=None, qg=None,
+                         decay=None):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
     Returns ``(dq, dk, dv, dg, dh0)``; without ``hT`` (the states a forward pass kept) it
-    recomputes the per-chunk states as the reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``wide``: the forward's
+    recomputes the per-chunk states as the reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``qg``, ``decay``:
+    the gated queries and chunk decays of ``fla_chunk_gla_fwd_fused_kept``, if the forward kept them.  ``wide``: the forward's
     gate-range flags (int32 ``[chunks, H]``); flagged chunks get their intra-chunk terms
     from the exact kernel.  Without it the result is exact only while the chunk-cumulative
     log-gate stays within +-80."""
@@ -338,10 +350,13 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
     if dht is not None:
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
-    be.check(be.lib().fla_chunk_gla_bwd(
-        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(dhtf),
-        be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
-        be.ptr(idx), be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q)), "fla_chunk_gla_bwd")
+    tail = (be.ptr(dhtf), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
+            be.ptr(idx), be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q))
+    head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT))
+    if qg is not None and decay is not None and float(scale) != 0.0:
+        be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), *tail), "fla_chunk_gla_bwd_kept")
+    else:
+        be.check(be.lib().fla_chunk_gla_bwd(*head, *tail), "fla_chunk_gla_bwd")
     return dq, dk, dv, dg, dh0
 
 
@@ -368,7 +383,9 @@ def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
     _, _, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, False, offsets, return_flags=True,
                                      states_out=states)
     dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht,
-                                               offsets, wide, hT=states[0])
+                                               offsets, wide, hT=states[0],
+                                               qg=states[1] if len(states) > 1 else None,
+                                               decay=states[2] if len(states) > 2 else None)
     if head_first:
         dq, dk, dv, dg = (x.transpose(1, 2) for x in (dq, dk, dv, dg))
     return dq, dk, dv, dg, dh0
@@ -406,7 +423,8 @@ class ChunkGLAFunction(torch.autograd.Function):
                                 states_out=states)
         # the inputs, the small table of chunks whose gates need the exact intra-chunk arithmetic, and
         # (unless recomputation is asked for) the per-chunk states the fused launch wrote on its way
-        ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None, states[0] if states else None)
+        kept = tuple(states) + (None,) * (3 - len(states)) if states else (None, None, None)
+        ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None, *kept)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         if (KP, VP) != (K, V):
@@ -421,7 +439,7 @@ class ChunkGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        q, k, v, g, h0, offsets, wide, hT = ctx.saved_tensors
+        q, k, v, g, h0, offsets, wide, hT, qg, decay = ctx.saved_tensors
         K, V, KP, VP = ctx.dims
         if ctx.head_first:
             do = do.transpose(1, 2)
@@ -431,7 +449,8 @@ class ChunkGLAFunction(torch.autograd.Function):
         do = do.contiguous()
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
-        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide, hT=hT)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide, hT=hT, qg=qg,
+                                                   decay=decay)
         if (KP, VP) != (K, V):
             dq, dk, dg, dv = dq[..., :K], dk[..., :K], dg[..., :K], dv[..., :V]
             if dh0 is not None:

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 4
+#define FLA_ABI_VERSION 5
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -224,6 +224,18 @@ int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, const void* v, 
                                    int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                                    int64_t V, int64_t N, float scale, fla_stream_t stream);
 
+/* fla_chunk_gla_fwd_fused_states that also leaves what the backward's reverse state scan would otherwise form
+ * from q and the gates again (the reference's chunk_bwd_dh does, fla/ops/common/chunk_h.py:156-271): the gated
+ * queries q_gated = q e^{G} ([B,T,H,K] in the q/k/v dtype, G the chunk-local prefix sum of the log-gates; rows
+ * past the end of a short chunk are not written) and chunk_decay = e^{G_last} (fp32 [chunks, H, K]).  Hand both
+ * to fla_chunk_gla_bwd_kept. */
+int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const void* v, const void* gates,
+                                 const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                 void* h_frag_t, void* q_gated, float* chunk_decay, const int64_t* offsets,
+                                 const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order,
+                                 int64_t NT, int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
+                                 int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
+
 /* The fused forward for one log-gate per (token, head), g fp32 [B,T,H]: chunk_simple_gla
  * (fla/ops/simple_gla/chunk.py:16-131: h_t = e^{g_t} h_{t-1} + k_t v_t^T, o_t = scale q_t^T h_t) without
  * the [B,T,H,K] gate tensor a call through fla_chunk_gla_fwd_fused would need.  Same kernel, the staging
@@ -349,6 +361,16 @@ int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* g
                       int qkv_dtype, int gate_dtype,
                       int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                       float scale, fla_stream_t stream);
+
+/* The same with q_gated and chunk_decay from fla_chunk_gla_fwd_fused_kept: the reverse state scan
+ * (chunk_bwd_dh, fla/ops/common/chunk_h.py:338-402) streams them and do instead of re-forming prefix sums and
+ * exponentials from q and the gates; results equal fla_chunk_gla_bwd's to rounding.  scale must not be 0. */
+int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const void* gates, const void* dout,
+                           const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
+                           void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                           const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                           int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                           int64_t N, float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * The chunk-parallel stages of GLA under the operand layouts of the reference's internal
