@@ -319,10 +319,10 @@ def bench_gdr(device, steps=50, warmup=20):
         st_p = event_stats(prep, steps, 5)
         st_s = event_stats(scan, steps, 5)
         state_bytes = n_states * H * K * V * 4
-        tri = chunks * H * 2 * 10 * 256 * 2                     # the packed triangular tiles
+        tri = chunks * H * 10 * 256 * 2                         # the packed triangular tile
         # algorithmic bytes of each launch: every operand read once, every result written once
-        bytes_prep = 2 * T * H * K * 2 + 2 * T * H * 4 + T * H * 4 + tri          # q, k, g, beta in; gamma, tiles out
-        bytes_scan = 4 * T * H * K * 2 + T * H * 4 + tri + state_bytes            # q, k, v, gamma, tiles in; o, ht out
+        bytes_prep = T * H * K * 2 + 2 * T * H * 4 + T * H * 4 + tri              # k, g, beta in; gamma, tile out
+        bytes_scan = 4 * T * H * K * 2 + T * H * 4 + tri + state_bytes            # q, k, v, gamma, tile in; o, ht out
         ach = bytes_scan / (st_s["median_us"] * 1e-6) / 1e9
         out[name] = {
             "us": round(us, 1), **spread(st), "tokens_per_s": round(tokens / (us * 1e-6), 1),
@@ -340,10 +340,10 @@ def bench_gdr(device, steps=50, warmup=20):
             "launches_bytes_total": bytes_prep + bytes_scan}
 
     plan = VarlenPlan(offs, 64)
-    AT, gc = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=plan.offsets, indices=plan.indices)
+    AT, gc = fwd_prepare_scan_operands(k, beta, g, offsets=plan.offsets, indices=plan.indices)
     row("config2_varlen",
         lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, offsets=offs, head_first=False),
-        lambda: fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=plan.offsets, indices=plan.indices),
+        lambda: fwd_prepare_scan_operands(k, beta, g, offsets=plan.offsets, indices=plan.indices),
         lambda: chunk_gated_delta_rule_fwd_scan(q, k, v, AT, gc, scale, None, True, offsets=plan.offsets,
                                                 chunk_offsets=plan.chunk_offsets, seq_order=plan.seq_order),
         N, plan.NT, T)
@@ -351,10 +351,10 @@ def bench_gdr(device, steps=50, warmup=20):
     B, T2 = 8, 4096
     q, k, v = (x.view(B, T2, H, -1) for x in (q, k, v))
     g, beta = g.view(B, T2, H), beta.view(B, T2, H)
-    AT, gc = fwd_prepare_scan_operands(q, k, beta, g, scale)
+    AT, gc = fwd_prepare_scan_operands(k, beta, g)
     row("B8_T4096",
         lambda: chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False),
-        lambda: fwd_prepare_scan_operands(q, k, beta, g, scale),
+        lambda: fwd_prepare_scan_operands(k, beta, g),
         lambda: chunk_gated_delta_rule_fwd_scan(q, k, v, AT, gc, scale, None, True),
         B, B * T2 // 64, B * T2)
     return out

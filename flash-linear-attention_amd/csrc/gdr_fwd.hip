@@ -327,24 +327,22 @@ __global__ __launch_bounds__(256, K <= 128 ? 4 : 2) void gdr_fwd_wy_kernel(WyPar
 
 // ---------------------------------------------------------------------------
 // Chunk-parallel preparation for the one-pass forward (fla_chunk_gated_delta_rule_fwd_scan): per
-// (chunk, head) the two lower-triangular 64x64 matrices the scan applies to value-column slabs,
+// (chunk, head) the lower-triangular 64x64 matrix the scan applies to value-column slabs,
 //   Tu  = (Aw * Gamma) diag(beta)        Tu_ij  = Aw_ij e^{gamma_i - gamma_j} beta_j   (j <= i)
-//   Aqk = scale tril(q k^T * Gamma)      Aqk_ij = scale (q_i . k_j) e^{gamma_i - gamma_j}
-// With them  v_new = u - e^{gamma} (w h) = Tu (v - e^{gamma} (k h))  (u = Tu v and
+// With it  v_new = u - e^{gamma} (w h) = Tu (v - e^{gamma} (k h))  (u = Tu v and
 // e^{gamma} w = Tu diag(e^{gamma}) k, since Aw Gamma-scaling is D Aw D^-1 and diagonal matrices
-// commute), so neither w nor u is formed and the scan reads k, q, v and these 10 KB instead of
-// k, q, w, u and a 8 KB score tile.  Only the ten 16x16 blocks on and below the diagonal are stored,
-// block (tt, jb) at index tt (tt + 1) / 2 + jb, each block row-major: at [chunk, head, {Tu, Aqk}, 10, 16, 16].
-// Rows past the end of a short chunk come out as zeros (beta and q are zero there).
+// commute), so neither w nor u is formed and the scan reads k, q, v and these 5 KB instead of
+// k, q, w, u and a 8 KB score tile (the gated scores q k^T are formed inside the scan, which holds q and k
+// anyway; this launch reads k alone).  Only the ten 16x16 blocks on and below the diagonal are stored,
+// block (tt, jb) at index tt (tt + 1) / 2 + jb, each block row-major: at [chunk, head, 10, 16, 16].
+// Rows past the end of a short chunk come out as zeros (beta is zero there).
 struct PrepParams {
-  const void* q;
   const void* k;
   const float* beta;
   const float* g;      // raw log-gates [rows, H] (g_is_cumsum == 0) or their chunk-local prefix sums, or NULL
   int g_is_cumsum;
   float* gam_out;      // [rows, H]: the chunk-local prefix sums (written when g is raw), or NULL
   void* AT;
-  float scale;
   const int64_t* offsets;
   const int64_t* indices;
   int64_t T;
@@ -353,10 +351,11 @@ struct PrepParams {
   void* Aw;
 };
 
-constexpr int kPrepWorkgroups = 3 * 256;        // three resident workgroups (register budget) on each of the 256 CUs
+// resident workgroups per CU (register budget): four, or three for the variant that also writes w and Aw
+constexpr int kPrepResident = 4, kPrepResidentKeep = 3;
 FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 
-// A workgroup walks several (chunk, head) items (grid-stride) and loads the q, k rows, beta and the gate
+// A workgroup walks several (chunk, head) items (grid-stride) and loads the k rows, beta and the gate
 // of its next item into registers once the matrix products of the current one have released their
 // accumulators: the loads land while the inversion runs (measured: worth about 4 %; the launch is a chain
 // of short dependent phases - removing the inversion, the stores or the loads each saves 15-20 % - rather
@@ -364,20 +363,19 @@ FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 // KEEP: the forward of a pass that will be differentiated also leaves w = Aw (beta k) and Aw in memory (the WY
 // launch of the reference's decomposition, without a second inversion and a second pass over k).
 template <typename T, int K, bool KEEP>
-__global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
+__global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
   constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
   constexpr int R_BYTES = BT * LDK * 2 > BT * LDM * 4 ? BT * LDK * 2 : BT * LDM * 4;
   __shared__ __attribute__((aligned(16))) char sRA[R_BYTES];   // k row-major -> M (fp32) -> packed Tu tile
-  __shared__ __attribute__((aligned(16))) char sRB[R_BYTES];   // q row-major -> X (fp32)
-  __shared__ __attribute__((aligned(16))) T sPo[kTriElems];    // packed score tile
+  __shared__ __attribute__((aligned(16))) char sRB[R_BYTES];   // X (fp32) -> KEEP: k row-major again
   __shared__ __attribute__((aligned(16))) float sBeta[BT];
   __shared__ __attribute__((aligned(16))) float sGam[BT];
   T* sK = (T*)sRA;
   float* sM = (float*)sRA;
-  T* sQ = (T*)sRB;
+  T* sK2 = (T*)sRB;
   T* sTu = (T*)sRA;
   T* sAb = (T*)sRA + kTriElems;   // KEEP: Aw diag(beta), row-major [64][LDT], behind the packed tile
   static_assert((kTriElems + BT * LDT) * 2 <= R_BYTES, "region A holds the packed tile and Aw diag(beta)");
@@ -397,7 +395,7 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
   struct Item {
     int L, hh;
     int64_t row0, cglob;
-    v8 q[NPL], k[NPL];
+    v8 k[NPL];
     float beta, g;   // wave 0: this lane's row
   };
   // Items are numbered head-fastest: item = chunk * H + head.  The walk keeps (chunk, head) and advances
@@ -432,13 +430,11 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
     it.hh = hh;
     it.row0 = cl.row0;
     it.cglob = cl.cglob;
-    const char* qp = (const char*)p.q + (cl.row0 * H + hh) * (int64_t)K * 2;
     const char* kp = (const char*)p.k + (cl.row0 * H + hh) * (int64_t)K * 2;
     const uint32_t lim = (uint32_t)(cl.L - 1) * pitch + c8 * 2;   // rows past the end: re-read the last one
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
       const uint32_t o = off[i] < lim ? off[i] : lim;
-      it.q[i] = *(const v8*)(qp + o);
       it.k[i] = *(const v8*)(kp + o);
     }
     if (wave == 0) {
@@ -464,11 +460,10 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
     const int L = cur.L;
     const int hh = cur.hh;
     const int64_t row0 = cur.row0, cglob = cur.cglob;
-    // ---- q, k row-major (rows past the end of the chunk zero), beta, gamma
+    // ---- k row-major (rows past the end of the chunk zero), beta, gamma
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
       const int row = r0 + RPP * i;
-      *(v8*)&sQ[row * LDK + c8] = row < L ? cur.q[i] : z;
       *(v8*)&sK[row * LDK + c8] = row < L ? cur.k[i] : z;
     }
     if (wave == 0) {
@@ -492,31 +487,17 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
     const int64_t next = lin + gridDim.x;
     const bool more = next < total;   // workgroup-uniform
 
-    // ---- S = k k^T and the transposed scores k q^T on the lower-triangular 32x32 quadrants
+    // ---- S = k k^T on the lower-triangular 32x32 quadrants
     const int qi = wave >> 1, qj = wave & 1;
-    f32x16 s = zero16(), sq = zero16();
+    f32x16 s = zero16();
     if (qj <= qi) {
 #pragma unroll
       for (int ks = 0; ks < K; ks += 16) {
-        const v8 kj = lds_frag32<T>(sK, LDK, qj * 32, ks, lane);
-        s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), kj, s);
-        sq = Elem<T>::mfma32(kj, lds_frag32<T>(sQ, LDK, qi * 32, ks, lane), sq);
+        s = Elem<T>::mfma32(lds_frag32<T>(sK, LDK, qi * 32, ks, lane), lds_frag32<T>(sK, LDK, qj * 32, ks, lane), s);
       }
     }
-    lds_barrier();  // k and q row-major fully consumed: their storage becomes M and the packed score tile
+    lds_barrier();  // k row-major fully consumed: its storage becomes M
     if (qj <= qi) {
-      // sq: lane <-> row i, registers <-> four consecutive columns j per quad
-      const int i = qi * 32 + (lane & 31), tt = i >> 4;
-      const float gi = sGam[i];
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int j0 = qj * 32 + 8 * r4 + 4 * (lane >> 5);
-        const f32x4 gj = *(const f32x4*)&sGam[j0];
-        v4 o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (T)(j0 + e <= i ? p.scale * sq[4 * r4 + e] * __expf(gi - gj[e]) : 0.f);
-        if ((j0 >> 4) <= tt) *(v4*)&sPo[tri_block(tt, j0 >> 4) * 256 + (i & 15) * 16 + (j0 & 15)] = o;
-      }
       // s: lane <-> column j, registers <-> four consecutive rows i per quad
       const int j = qj * 32 + (lane & 31);
 #pragma unroll
@@ -593,15 +574,14 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
 #pragma unroll
       for (int i = 0; i < NPL; ++i) {
         const int row = r0 + RPP * i;
-        *(v8*)&sQ[row * LDK + c8] = row < L ? kkeep[i] : z;
+        *(v8*)&sK2[row * LDK + c8] = row < L ? kkeep[i] : z;
       }
     }
-    // both tiles leave as one contiguous 10 KB block, 16 bytes per lane
+    // the tile leaves as one contiguous 5 KB block, 16 bytes per lane
     {
-      T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)(2 * kTriElems);
-      constexpr int NP = kTriElems / 8;   // 16-byte pieces per tile
-      for (int e = tid; e < 2 * NP; e += 256)
-        *(v8*)(at + e * 8) = e < NP ? *(const v8*)&sTu[e * 8] : *(const v8*)&sPo[(e - NP) * 8];
+      T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)kTriElems;
+      constexpr int NP = kTriElems / 8;   // 16-byte pieces
+      for (int e = tid; e < NP; e += 256) *(v8*)(at + e * 8) = *(const v8*)&sTu[e * 8];
     }
     if constexpr (KEEP) {
       lds_barrier();   // k row-major complete
@@ -616,7 +596,7 @@ __global__ __launch_bounds__(256, KEEP ? 2 : 3) void gdr_fwd_prep_kernel(PrepPar
         const v8 a = lds_frag32<T>(sAb, LDT, rw * 32, js * 16, lane);
 #pragma unroll
         for (int t = 0; t < TN; ++t)
-          acc[t] = Elem<T>::mfma32(frag32_tr<T>(sQ, LDK, (cb * TN + t) * 32, js * 16, lane), a, acc[t]);
+          acc[t] = Elem<T>::mfma32(frag32_tr<T>(sK2, LDK, (cb * TN + t) * 32, js * 16, lane), a, acc[t]);
       }
       const int i = rw * 32 + (lane & 31);
       if (i < L) {
@@ -1189,7 +1169,7 @@ template <typename T>
 int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
   // (chunk, head) items, head-fastest; as many workgroups as are resident at once, each walking its share of the items
   const int64_t total = (int64_t)chunk_grid_.x * chunk_grid_.y;
-  const int64_t resident = p.w ? 2 * 256 : kPrepWorkgroups;   // the w-writing variant runs two workgroups per CU
+  const int64_t resident = (p.w ? kPrepResidentKeep : kPrepResident) * kNumCUs;
   dim3 grid((unsigned)(total < resident ? total : resident));
   if (p.w) {
     if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64, true>), grid, dim3(256), 0, st, p, total);
@@ -1206,20 +1186,20 @@ int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
-                                float* g_cumsum_out, void* AT, void* w, void* Aw, float scale, const int64_t* offsets,
+extern "C" int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_cumsum,
+                                float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
                                 const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                 int64_t K, fla_stream_t stream) {
-  FLA_REQUIRE(q && k && beta && AT, FLA_E_INVALID);
+  FLA_REQUIRE(k && beta && AT, FLA_E_INVALID);
   FLA_REQUIRE((w == nullptr) == (Aw == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && NT >= 0, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)AT | (uintptr_t)w | (uintptr_t)Aw) % 16 == 0, FLA_E_ALIGNMENT);
+  FLA_REQUIRE(((uintptr_t)k | (uintptr_t)AT | (uintptr_t)w | (uintptr_t)Aw) % 16 == 0, FLA_E_ALIGNMENT);
   dim3 grid;
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  PrepParams p{q, k, beta, g, g_is_cumsum, g_cumsum_out, AT, scale, offsets, indices, T, (int)H, ntfix, w, Aw};
+  PrepParams p{k, beta, g, g_is_cumsum, g_cumsum_out, AT, offsets, indices, T, (int)H, ntfix, w, Aw};
   if (qkv_dtype == FLA_BF16) return launch_prep<bf16>(p, (int)K, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_prep<f16>(p, (int)K, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

@@ -1,17 +1,20 @@
 // One-pass gated-delta-rule forward for gfx950: state scan and output in one launch; neither w, u,
 // v_new nor the per-chunk states exist in memory.
 //
-// Inputs are q, k, v, the chunk-local gate prefix sums gamma and the two packed triangular 64x64 tiles
-// per (chunk, head) that fla_gdr_fwd_prep leaves: Tu = (Aw * Gamma) diag(beta) and the gated causal
-// scores Aqk.  One workgroup of 8 waves owns one (sequence, head, 64 value columns) and walks the
-// chunks serially:
-//   waves 4-7 ("staging")  copy k, q and the triangular tiles of chunk c+1 to LDS, transpose v into a
-//                          time-contiguous tile, and write the finished o tile of chunk c-1 to global
-//                          memory (k is staged row-major only: the state update reads its transposed
-//                          operand from that tile with the transposing LDS load);
+// Inputs are q, k, v, the chunk-local gate prefix sums gamma and the packed triangular 64x64 tile per
+// (chunk, head) that fla_gdr_fwd_prep leaves: Tu = (Aw * Gamma) diag(beta).  One workgroup of 8 waves owns
+// one (sequence, head, 64 value columns) and walks the chunks serially:
+//   waves 4-7 ("staging")  copy k, q and the gate row of chunk c+2 and the triangular tile of chunk c+1 to
+//                          LDS, transpose v of chunk c+1 into a time-contiguous tile, and write the
+//                          finished o tile of chunk c-1 to global memory (k is staged row-major only: the
+//                          state update reads its transposed operand from that tile with the transposing
+//                          LDS load);
 //   waves 0-3 ("matrix")   each own 16 value columns of the fp32 state (all K rows, in 16x16
 //                          accumulator tiles).  The delta rule is independent per value column, so a
-//                          matrix wave never exchanges data with another:
+//                          matrix wave exchanges one thing with the others: the gated causal scores
+//                          Aqk = s tril(q k^T * Gamma) of the *next* chunk, of whose ten 16x16 blocks each
+//                          wave forms two or three while it works on the current chunk (k and q are in LDS
+//                          a chunk period early for that; the barrier that ends the period publishes them):
 //                            v_new = Tu (v - e^{gamma} * (k h))
 //                            o     = s e^{gamma} * (q h) + Aqk v_new
 //                            h    <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} * v_new)
@@ -20,7 +23,8 @@
 //                          and v_new go from accumulators straight back into MFMA operands: the
 //                          contraction index of the LDS-side operand is permuted to the accumulator
 //                          row order instead.
-// Operand tiles are double-buffered and the two groups meet at one barrier per chunk.  The o tile
+// Operand tiles are double-buffered (k, q and the gate rows: three buffers) and the two groups meet at one
+// barrier per chunk.  The o tile
 // takes the place of the v tile it was computed from (same lanes, same addresses), so it needs no
 // storage of its own.
 // The KEEP instantiation serves a forward pass that will be differentiated: the matrix waves also write
@@ -36,13 +40,13 @@
 namespace {
 
 // Per chunk and workgroup the kernel reads q, k (16 KB each at K=128), its 64 value columns (8 KB) and
-// 10 KB of triangular blocks, and its time follows those bytes: the launch is bound by the rate at which
+// 5 KB of triangular blocks, and its time follows those bytes: the launch is bound by the rate at which
 // data reaches the CUs through L2, both value-column slabs of a head pulling q, k and the tiles.
 struct GdrScanParams {
   const void* q;
   const void* k;
   const void* v;
-  const void* AT;   // [chunks, H, 2, 10, 16, 16]: Tu, Aqk
+  const void* AT;   // [chunks, H, 10, 16, 16]: Tu
   const float* gam;
   const float* h0;
   void* o;
@@ -102,13 +106,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int LDR = K + 8;  // pitch of the row-major k and q tiles
   constexpr int KS = K / 32;  // 32-wide contraction slices of the state
   constexpr int KT = K / 16;  // 16-row state tiles per matrix wave
-  __shared__ __attribute__((aligned(16))) T sK[2][BT * LDR];     // k    [t][k]
-  __shared__ __attribute__((aligned(16))) T sQ[2][BT * LDR];     // q    [t][k]
+  constexpr int ATS = kTriElems;  // elements per (chunk, head) in AT
+  // k, q and the gate rows of a chunk are in LDS one chunk period before the rest of it (three buffers, chunk
+  // modulo 3): Aqk of chunk c + 1 is formed from them while chunk c is in work.
+  __shared__ __attribute__((aligned(16))) T sK[3][BT * LDR];     // k    [t][k]
+  __shared__ __attribute__((aligned(16))) T sQ[3][BT * LDR];     // q    [t][k]
   __shared__ __attribute__((aligned(16))) T sVt[2][BV * LDT];    // v^T  [v][t], later o^T
-  __shared__ __attribute__((aligned(16))) T sAT[2][2 * kTriElems];  // Tu, Aqk (packed triangular tiles)
-  __shared__ __attribute__((aligned(16))) float sEg[2][BT];      // e^{gamma_t}
-  __shared__ __attribute__((aligned(16))) float sEd[2][BT];      // e^{gamma_last - gamma_t}
-  __shared__ float sDec[2];                                      // e^{gamma_last}
+  __shared__ __attribute__((aligned(16))) T sAT[2][kTriElems];   // Tu (packed triangular tile)
+  __shared__ __attribute__((aligned(16))) T sP[2][kTriElems];    // Aqk, same packing
+  __shared__ __attribute__((aligned(16))) float sGam[3][BT];     // gamma_t
+  __shared__ __attribute__((aligned(16))) float sEg[3][BT];      // e^{gamma_t}
+  __shared__ __attribute__((aligned(16))) float sEd[3][BT];      // e^{gamma_last - gamma_t}
+  __shared__ float sDec[3];                                      // e^{gamma_last}
 
   const int tid = threadIdx.x, lane = tid & 63;
   // wave-uniform by construction: keeps the role split and the barriers on scalar branches
@@ -125,20 +134,65 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int nchunks = (int)((sp.len + BT - 1) / BT);
   const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
 
+  // Aqk = scale tril(q k^T * Gamma) of the chunk whose tiles are in buffer b, shared out over waves 0-3 by 16x16
+  // block: a block is computed transposed (k rows against q rows), which leaves every lane with four
+  // adjacent entries of one row of Aqk - an 8-byte piece of the packed tile frag_tri() reads.  Rows past the
+  // end of a short chunk are zero in the q and k tiles.
+  auto compute_p = [&](int b3, int pb) __attribute__((always_inline)) {
+    const T* Kr = sK[b3];
+    const T* Q = sQ[b3];
+    T* Po = sP[pb];
+    const int c = lane & 15, g = lane >> 4;
+    // (row block, column block) of this wave's blocks, a nibble each, first in the low bits: two or three
+    // blocks for each of the four waves, or five for each of the two waves that carry no state
+    int tis, tjs, cnt;
+    if constexpr (NMW == 4) {
+      tis = wave == 0 ? 0x33 : wave == 1 ? 0x33 : wave == 2 ? 0x222 : 0x011;
+      tjs = wave == 0 ? 0x10 : wave == 1 ? 0x32 : wave == 2 ? 0x210 : 0x010;
+      cnt = wave < 2 ? 2 : 3;
+    } else {
+      tis = wave == 2 ? 0x03333 : 0x11222;
+      tjs = wave == 2 ? 0x03210 : 0x10210;
+      cnt = wave >= 2 ? 5 : 0;
+    }
+    v8 fq[KS];
+    int cur = -1;
+#pragma unroll
+    for (int n = 0; n < (NMW == 4 ? 3 : 5); ++n) {
+      if (n < cnt) {
+        const int ti = (tis >> (4 * n)) & 15, tj = (tjs >> (4 * n)) & 15;
+        if (ti != cur) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) fq[ks] = frag16<T>(Q, LDR, 16 * ti, 32 * ks, lane);
+          cur = ti;
+        }
+        f32x4 sc = zero4();
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) sc = Elem<T>::mfma16(frag16<T>(Kr, LDR, 16 * tj, 32 * ks, lane), fq[ks], sc);
+        const float gi = sGam[b3][16 * ti + c];
+        const f32x4 gj = *(const f32x4*)&sGam[b3][16 * tj + 4 * g];
+        v4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          o[r] = (T)((ti > tj || 4 * g + r <= c) ? p.scale * sc[r] * __expf(gi - gj[r]) : 0.f);
+        *(v4*)&Po[(ti * (ti + 1) / 2 + tj) * 256 + c * 16 + 4 * g] = o;
+      }
+    }
+  };
+
   if (wave >= 4) {
     // =========================== staging waves ===========================
     if (nchunks == 0) return;
     const int st = tid - 256;
     constexpr int C8 = K / 8, NPW = BT * C8 / 256;           // 16-byte pieces per row / per lane (q)
-    constexpr int NPA = 2 * kTriElems / 4 / 256;             // 8-byte pieces of the triangular tiles per lane
-    static_assert(NPA * 256 * 4 == 2 * kTriElems, "the triangular tiles split evenly over the staging lanes");
+    static_assert(kTriElems == 8 * (256 + 64), "Tu: a 16-byte piece per staging lane and 64 more");
     const int urg = st / (BV / 4), uc4 = (st % (BV / 4)) * 4;   // v, o: a lane owns RV rows x 4 columns
     const uint32_t HK = (uint32_t)H * K, HV = (uint32_t)H * V;
     auto q_row = [&](int e) { return e / C8; };
     auto q_col = [&](int e) { return (e % C8) * 8; };
     struct Regs {
       v8 q[NPW], k[NPW];
-      v4 a[NPA];
+      v8 a0, a1;
       v4 v[RV];
       uint32_t gam;  // fp32 bits
     };
@@ -154,14 +208,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const char* lq = (const char*)p.q + row00 * K * 2;
     const char* lk = (const char*)p.k + row00 * K * 2;
     const char* lv = (const char*)p.v + (row00 * V + vbase) * 2;
-    const char* la = (const char*)p.AT + ((chunk0 * H + hh) * (int64_t)(2 * kTriElems) + st * 4) * 2;
+    const char* la = (const char*)p.AT + (chunk0 * H + hh) * (int64_t)ATS * 2;
+    const uint32_t offa0 = 16 * (uint32_t)st, offa1 = 16 * (uint32_t)(256 + lane);
     // The gate load is unconditional (a load under a branch would make the wave drain its whole load
     // queue at the join); without gates it reads a dummy address and the bits are masked to zero.
     const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
     const char* lg = p.gam ? (const char*)p.gam + row00 * 4 : lq;
     char* so = (char*)p.o + (row00 * V + vbase) * 2;
     const int64_t strk = (int64_t)BT * HK * 2, strv = (int64_t)BT * HV * 2;
-    const int64_t stra = (int64_t)H * (2 * kTriElems) * 2;
+    const int64_t stra = (int64_t)H * ATS * 2;
     const int64_t strg = p.gam ? (int64_t)BT * H * 4 : 0;
     const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
     // Every memory operation of the steady state is unconditional: the wait counts the compiler places
@@ -174,30 +229,40 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t limv_full = 2 * ((uint32_t)(BT - 1) * HV), limv_last = 2 * ((uint32_t)(Llast - 1) * HV);
     static_assert(RV == 4 || RV == 2, "slab of 64 or 32 value columns");
     const uint32_t colq = 2 * (uint32_t)q_col(st), colv = 2 * (uint32_t)uc4;
-    int lc = 0;  // chunk the load pointers are on
-    auto load = [&](Regs& R) __attribute__((always_inline)) {
-      const bool last = lc >= nchunks - 1;
-      const uint32_t limq = (last ? limq_last : limq_full) + colq, limv = (last ? limv_last : limv_full) + colv;
+    // k, q and the gate run one chunk ahead of v and Tu: register set j holds k, q, gamma of chunk j + 1 and
+    // v, Tu of chunk j.
+    int lcq = 0, lcv = 0;  // chunks the two groups of load pointers are on
+    auto load_kq = [&](Regs& R) __attribute__((always_inline)) {
+      const bool last = lcq >= nchunks - 1;
+      const uint32_t limq = (last ? limq_last : limq_full) + colq;
       const uint32_t limg = 4 * (uint32_t)((last ? Llast : BT) - 1) * H;
-#pragma unroll
-      for (int i = 0; i < NPA; ++i) R.a[i] = *(const v4*)(la + 2048 * i);   // full tiles whatever the chunk length
 #pragma unroll
       for (int i = 0; i < NPW; ++i) {
         const uint32_t o = offq[i] < limq ? offq[i] : limq;
         R.q[i] = *(const v8*)(lq + o);
         R.k[i] = *(const v8*)(lk + o);
       }
-#pragma unroll
-      for (int i = 0; i < RV; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
       R.gam = *(const uint32_t*)(lg + (offg < limg ? offg : limg));
-      if (lc + 1 < nchunks) {
+      if (lcq + 1 < nchunks) {
         lq += strk;
         lk += strk;
-        lv += strv;
-        la += stra;
         lg += strg;
       }
-      ++lc;
+      ++lcq;
+    };
+    auto load = [&](Regs& R) __attribute__((always_inline)) {
+      const bool last = lcv >= nchunks - 1;
+      const uint32_t limv = (last ? limv_last : limv_full) + colv;
+      R.a0 = *(const v8*)(la + offa0);   // a full tile whatever the chunk length
+      R.a1 = *(const v8*)(la + offa1);   // its last 64 pieces: every wave loads them, the first one writes them
+#pragma unroll
+      for (int i = 0; i < RV; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
+      if (lcv + 1 < nchunks) {
+        lv += strv;
+        la += stra;
+      }
+      ++lcv;
+      load_kq(R);
     };
     // LDS destinations of this lane (element offsets inside a tile)
     int dq[NPW], dv[4];
@@ -205,29 +270,43 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < NPW; ++i) dq[i] = q_row(st + 256 * i) * LDR + q_col(st + 256 * i);
 #pragma unroll
     for (int j = 0; j < 4; ++j) dv[j] = (uc4 + j) * LDT + swz_t(uc4 + j, urg * RV);
-    int wc = 0;  // next chunk to write to LDS
-    // maybe_last: the chunk may be the sequence's last, short one (rows past its end are zeroed)
-    auto write = [&](Regs& R, auto maybe_last) __attribute__((always_inline)) {
-      const int b = wc & 1;
-      if constexpr (decltype(maybe_last)::value) {
-        if (wc == nchunks - 1 && Llast < BT) {
-          const int L = Llast;
+    // Rows past the end of a sequence's last, short chunk are zeroed on the way to LDS.  (What a set holds
+    // beyond the last chunk is that chunk again; nothing reads the buffer it goes to.)
+    int wq = 0, wq3 = 0;  // next chunk whose k, q, gate rows are written, and its buffer
+    auto write_kq = [&](Regs& R) __attribute__((always_inline)) {
+      if (wq == nchunks - 1 && Llast < BT) {
 #pragma unroll
-          for (int i = 0; i < NPW; ++i)
-            if (q_row(st + 256 * i) >= L)
+        for (int i = 0; i < NPW; ++i)
+          if (q_row(st + 256 * i) >= Llast)
 #pragma unroll
-              for (int j = 0; j < 8; ++j) R.q[i][j] = R.k[i][j] = (T)0.f;
-#pragma unroll
-          for (int i = 0; i < RV; ++i)
-            if (urg * RV + i >= L) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        }
+            for (int j = 0; j < 8; ++j) R.q[i][j] = R.k[i][j] = (T)0.f;
       }
 #pragma unroll
-      for (int i = 0; i < NPW; ++i) *(v8*)&sQ[b][dq[i]] = R.q[i];
+      for (int i = 0; i < NPW; ++i) *(v8*)&sQ[wq3][dq[i]] = R.q[i];
 #pragma unroll
-      for (int i = 0; i < NPA; ++i) *(v4*)&sAT[b][st * 4 + 1024 * i] = R.a[i];
+      for (int i = 0; i < NPW; ++i) *(v8*)&sK[wq3][dq[i]] = R.k[i];
+      if (wave == 4) {
+        // lanes past the end of a short chunk carry the last row's gate
+        const float gam = __uint_as_float(R.gam & gmask);
+        const float glast = __uint_as_float(__builtin_amdgcn_readlane(R.gam & gmask, 63));
+        sGam[wq3][lane] = gam;
+        sEg[wq3][lane] = __expf(gam);
+        sEd[wq3][lane] = __expf(glast - gam);
+        if (lane == 0) sDec[wq3] = __expf(glast);
+      }
+      ++wq;
+      wq3 = wq3 == 2 ? 0 : wq3 + 1;
+    };
+    int wc = 0;  // next chunk whose v, Tu are written
+    auto write = [&](Regs& R) __attribute__((always_inline)) {
+      const int b = wc & 1;
+      if (wc == nchunks - 1 && Llast < BT) {
 #pragma unroll
-      for (int i = 0; i < NPW; ++i) *(v8*)&sK[b][dq[i]] = R.k[i];
+        for (int i = 0; i < RV; ++i)
+          if (urg * RV + i >= Llast) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      }
+      *(v8*)&sAT[b][st * 8] = R.a0;
+      if (wave == 4) *(v8*)&sAT[b][2048 + lane * 8] = R.a1;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         rvv vc;
@@ -235,15 +314,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < RV; ++i) vc[i] = R.v[i][j];
         *(rvv*)&sVt[b][dv[j]] = vc;
       }
-      if (wave == 4) {
-        // lanes past the end of a short chunk carry the last row's gate
-        const float gam = __uint_as_float(R.gam & gmask);
-        const float glast = __uint_as_float(__builtin_amdgcn_readlane(R.gam & gmask, 63));
-        sEg[b][lane] = __expf(gam);
-        sEd[b][lane] = __expf(glast - gam);
-        if (lane == 0) sDec[b] = __expf(glast);
-      }
       ++wc;
+      write_kq(R);
     };
     // The matrix waves left o^T of a chunk where v^T of that chunk was; each lane reads back
     // exactly the addresses it writes in write(), so the tile can be refilled right after.
@@ -266,27 +338,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       so += strv;
       ++oc;
     };
-    // Three register sets: a chunk is loaded four iterations before the matrix waves use it (three before it
-    // is written to LDS), so its loads have two chunk periods to land.  Iteration c (the matrix waves work on
-    // chunk c) stores the output of chunk c-1, writes the tiles of chunk c+1 and loads chunk c+4 into the set
-    // just emptied; sets rotate R1, R2, R0.  The steady-state loop runs whole rotations over the iterations
-    // that touch neither the first nor the last chunk and leaves only at its latch.
+    // Three register sets: a set is loaded three iterations before it is written to LDS, so its loads have two
+    // chunk periods to land.  Iteration c (the matrix waves work on chunk c and form Aqk of chunk c + 1) stores
+    // the output of chunk c-1, writes set c + 1 (k, q, gamma of chunk c + 2; v, Tu of chunk c + 1) and loads set
+    // c + 4 into the registers just emptied; sets rotate R1, R2, R0.  The steady-state loop runs whole rotations
+    // over the iterations that touch neither the first nor the last chunk and leaves only at its latch.
     constexpr std::true_type any_chunk{};
     constexpr std::false_type inner_chunk{};
     Regs R0, R1, R2;
+    load_kq(R0);              // k, q, gamma of chunk 0 on their own
+    write_kq(R0);
     load(R0);
     load(R1);
     load(R2);
-    write(R0, any_chunk);
+    lds_barrier();            // Aqk of chunk 0 can be formed
+    write(R0);
     load(R0);
     lds_barrier();
     if (nchunks > 1) {
-      write(R1, any_chunk);   // iteration 0
+        write(R1);              // iteration 0
       load(R1);
       lds_barrier();
       auto iter = [&](Regs& R) __attribute__((always_inline)) {
         store_o(inner_chunk);
-        write(R, inner_chunk);
+            write(R);
         load(R);
         lds_barrier();
       };
@@ -299,11 +374,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const int rem = inner % 3;
       if (rem >= 1) iter(R2);
       if (rem >= 2) iter(R0);
-      if (nchunks > 2) {      // iteration nchunks - 2 writes the last chunk
+      if (nchunks > 2) {      // iteration nchunks - 2 writes the last chunk's v and Tu
         store_o(inner_chunk);
-        if (rem == 0) write(R2, any_chunk);
-        else if (rem == 1) write(R0, any_chunk);
-        else write(R1, any_chunk);
+            if (rem == 0) write(R2);
+        else if (rem == 1) write(R0);
+        else write(R1);
         lds_barrier();
       }
       store_o(inner_chunk);   // iteration nchunks - 1: the output of chunk nchunks - 2
@@ -311,10 +386,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     lds_barrier();
     store_o(any_chunk);
   } else if (wave >= NMW) {
-    // waves without a share of the state keep the barrier count
+    // waves without a share of the state form their share of the scores and keep the barrier count
     if (nchunks > 0) {
       lds_barrier();
-      for (int ci = 0; ci < nchunks; ++ci) lds_barrier();
+      compute_p(0, 0);
+      lds_barrier();
+      int b3 = 0;
+      for (int ci = 0; ci < nchunks; ++ci) {
+        const int n3 = b3 == 2 ? 0 : b3 + 1;
+        if (ci + 1 < nchunks) compute_p(n3, (ci + 1) & 1);
+        lds_barrier();
+        b3 = n3;
+      }
     }
   } else {
     // =========================== matrix waves ===========================
@@ -352,12 +435,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
     if (nchunks > 0) {
       lds_barrier();
+      if constexpr (NMW == 4) compute_p(0, 0);
+      lds_barrier();
+      int b3 = 0;   // ci modulo 3
       for (int ci = 0; ci < nchunks; ++ci) {
         const int b = ci & 1;
-        const T* Kr = sK[b];
-        const T* Q = sQ[b];
+        const int n3 = b3 == 2 ? 0 : b3 + 1;
+        const T* Kr = sK[b3];
+        const T* Q = sQ[b3];
         const T* Tu = sAT[b];
-        const T* P = sAT[b] + kTriElems;
+        const T* P = sP[b];
+        if constexpr (NMW == 4) {
+          if (ci + 1 < nchunks) compute_p(n3, b ^ 1);   // with 32-column slabs the two other waves form the scores
+        }
         const int vrow = cb + c;
         T* vt = &sVt[b][vrow * LDT];
         // LDS reads are issued a group ahead of the MFMAs that consume them; the scheduling
@@ -424,11 +514,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         v8 ft[6];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-          eg[tt] = *(const f32x4*)&sEg[b][16 * tt + 4 * g];
-          ed[tt] = *(const f32x4*)&sEd[b][16 * tt + 4 * g];
+          eg[tt] = *(const f32x4*)&sEg[b3][16 * tt + 4 * g];
+          ed[tt] = *(const f32x4*)&sEd[b3][16 * tt + 4 * g];
           vv[tt] = *(const v4*)(vt + swz_t(vrow, 16 * tt + 4 * g));
         }
-        const float dec = sDec[b];
+        const float dec = sDec[b3];
         ft[0] = frag_tri<T>(Tu, 0, 0, lane);
         ft[1] = frag_tri<T>(Tu, 1, 0, lane);
         ft[2] = frag_tri<T>(Tu, 2, 0, lane);
@@ -513,6 +603,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           vn_base += (int64_t)BT * H * V * (int64_t)sizeof(T);
         }
         lds_barrier();
+        b3 = n3;
       }
     }
     if (p.ht) {

@@ -1,14 +1,13 @@
 """``chunk_gated_delta_rule`` with the reference's signature
 (``fla/ops/gated_delta_rule/chunk.py:258-363``).
 
-Forward on the device (chunk size 64), two launches: ``fla_gdr_fwd_prep`` (chunk-parallel: prefix sum of the
-gate, KK^T, block inverse, gated causal q k^T scores; leaves two packed triangular 64x64 tiles per chunk and
-head) -> ``fla_chunk_gated_delta_rule_fwd_scan`` (state scan and output in one pass over q, k, v; w, u, v_new
-and the per-chunk states are never formed).
-A forward pass that will be differentiated runs the reference's decomposition instead (cumsum, WY launch, state
-scan, output stage) and keeps w, Aw, v_new and the per-chunk states for the backward; with
-``KEEP_STATES_FOR_BACKWARD = False`` the backward recomputes them with
-``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
+Forward on the device (chunk size 64), two launches: ``fla_gdr_fwd_prep`` (chunk-parallel, reads k: prefix sum of
+the gate, KK^T, block inverse; leaves one packed triangular 64x64 tile per chunk and head) ->
+``fla_chunk_gated_delta_rule_fwd_scan`` (gated causal q k^T scores, state scan and output in one pass over q, k,
+v; w, u, v_new and the per-chunk states are never formed).
+A forward pass that will be differentiated runs the same two launches with more outputs and keeps w, Aw, v_new
+and the per-chunk states for the backward; with ``KEEP_STATES_FOR_BACKWARD = False`` the backward recomputes
+them with ``fla_chunk_gated_delta_rule_fwd_h`` like the reference.
 """
 import os
 import warnings
@@ -63,7 +62,7 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     co = None if plan is None else plan.chunk_offsets
     if fused:
         # two launches; Aw / Au are not formed on this path
-        AT, g = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=offs, indices=idx)
+        AT, g = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx)
         o, final_state = chunk_gated_delta_rule_fwd_scan(q, k, v, AT, g, scale, initial_state, output_final_state,
                                                          offsets=offs, chunk_offsets=co,
                                                          seq_order=None if plan is None else plan.seq_order)
@@ -90,7 +89,7 @@ def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, outp
     co = None if plan is None else plan.chunk_offsets
     beta = beta.float().contiguous()
     if q.shape[-1] <= _FUSED_MAX_K:
-        AT, g, w, Aw = fwd_prepare_scan_operands(q, k, beta, g, scale, offsets=offs, indices=idx, keep_w=True)
+        AT, g, w, Aw = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, keep_w=True)
         o, final_state, v_new, hT = chunk_gated_delta_rule_fwd_scan(
             q, k, v, AT, g, scale, initial_state, output_final_state, offsets=offs, chunk_offsets=co,
             seq_order=None if plan is None else plan.seq_order, keep=True)

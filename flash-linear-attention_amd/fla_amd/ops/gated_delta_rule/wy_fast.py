@@ -53,26 +53,23 @@ TRI_BLOCKS = 10   # 16x16 blocks on and below the diagonal of a 64x64 tile
 
 
 def fwd_prepare_scan_operands(
-    q: torch.Tensor,
     k: torch.Tensor,
     beta: torch.Tensor,
     g: Optional[torch.Tensor],
-    scale: float,
     offsets: Optional[torch.Tensor] = None,
     indices: Optional[torch.Tensor] = None,
     g_is_cumsum: bool = False,
     keep_w: bool = False,
 ):
-    """Chunk-parallel half of the one-pass forward (``fla_gdr_fwd_prep``): the work of ``chunk_local_cumsum``,
-    ``fwd_prepare_wy_repr`` (``fla/ops/gated_delta_rule/wy_fast.py:320-376``) and the score product of
-    ``chunk_fwd_o`` (``fla/ops/common/chunk_o.py:86-97``), leaving per (chunk, head) the lower-triangular
-    ``Tu = (Aw * Gamma) diag(beta)`` and ``Aqk = scale tril(q k^T * Gamma)`` as packed 16x16 blocks:
-    ``AT`` is ``[chunks, H, 2, 10, 16, 16]`` in the q/k/v dtype.  ``g`` is the raw per-head log-gate
+    """Chunk-parallel half of the one-pass forward (``fla_gdr_fwd_prep``): the work of ``chunk_local_cumsum``
+    and ``fwd_prepare_wy_repr`` (``fla/ops/gated_delta_rule/wy_fast.py:320-376``), leaving per (chunk, head) the
+    lower-triangular ``Tu = (Aw * Gamma) diag(beta)`` as packed 16x16 blocks: ``AT`` is
+    ``[chunks, H, 10, 16, 16]`` in the k dtype (the scan forms the gated scores ``q k^T`` itself).  ``g`` is the raw per-head log-gate
     ``[B, T, H]`` (or its chunk-local cumsum with ``g_is_cumsum``; ``None`` for the un-gated rule).
     Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``; with ``keep_w`` the launch also writes
     ``w = Aw (beta k)`` and ``Aw`` (what ``fwd_prepare_wy_repr`` leaves for the backward) and the return value
     is ``(AT, g_cumsum, w, Aw)``."""
-    be.require_gpu(q, k, beta)
+    be.require_gpu(k, beta)
     B, T, H, K = k.shape
     NT = 0
     chunks = B * (-(-T // BT))
@@ -84,21 +81,21 @@ def fwd_prepare_scan_operands(
     if g is not None:
         g = g.float().contiguous()
         gc = g if g_is_cumsum else torch.empty_like(g)
-    AT = k.new_empty(chunks, H, 2, TRI_BLOCKS, 16, 16)
+    AT = k.new_empty(chunks, H, TRI_BLOCKS, 16, 16)
     w = torch.empty_like(k) if keep_w else None
     Aw = k.new_empty(B, T, H, BT) if keep_w else None
     be.check(be.lib().fla_gdr_fwd_prep(
-        be.ptr(q), be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
-        be.ptr(AT), be.ptr(w), be.ptr(Aw), float(scale), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K,
+        be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
+        be.ptr(AT), be.ptr(w), be.ptr(Aw), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K,
         be.stream_of(k)), "fla_gdr_fwd_prep")
     return (AT, gc, w, Aw) if keep_w else (AT, gc)
 
 
 def unpack_triangular_tiles(AT: torch.Tensor) -> torch.Tensor:
-    """``[chunks, H, 2, 10, 16, 16]`` packed blocks -> dense ``[chunks, H, 2, 64, 64]`` (zeros above the diagonal
+    """``[chunks, H, 10, 16, 16]`` packed blocks -> dense ``[chunks, H, 64, 64]`` (zeros above the diagonal
     blocks); for tests and debugging."""
     chunks, H = AT.shape[:2]
-    out = AT.new_zeros(chunks, H, 2, 64, 64)
+    out = AT.new_zeros(chunks, H, 64, 64)
     for i in range(4):
         for j in range(i + 1):
             out[..., 16 * i:16 * i + 16, 16 * j:16 * j + 16] = AT[..., i * (i + 1) // 2 + j, :, :]

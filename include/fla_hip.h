@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 5
+#define FLA_ABI_VERSION 6
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -300,13 +300,11 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
 
 /* The two-launch forward that forms neither w, u, v_new nor the per-chunk states (what
  * chunk_gated_delta_rule runs when nothing is kept for a backward pass).  fla_gdr_fwd_prep is the chunk-parallel part: it replaces
- * chunk_local_cumsum of the gate, fwd_prepare_wy_repr (fla/ops/gated_delta_rule/wy_fast.py:320-376) and the
- * score product of chunk_fwd_o (fla/ops/common/chunk_o.py:86-97) and leaves, per (chunk, head), two
- * lower-triangular 64x64 matrices in the q/k/v dtype:
+ * chunk_local_cumsum of the gate and fwd_prepare_wy_repr (fla/ops/gated_delta_rule/wy_fast.py:320-376), reads k,
+ * beta and the gate, and leaves, per (chunk, head), one lower-triangular 64x64 matrix in the q/k/v dtype:
  *   Tu  = (Aw * Gamma) diag(beta),  Gamma_ij = exp(gamma_i - gamma_j)   (so that u = Tu v, e^{gamma} w = Tu e^{gamma} k)
- *   Aqk = scale tril(q k^T * Gamma)
- * stored as their ten 16x16 blocks on and below the diagonal (block (i, j) at index i (i + 1) / 2 + j, row-major
- * inside a block): AT is [chunks, H, 2, 10, 16, 16] (chunk index as in `indices`, or b * ceil(T/64) + c).
+ * stored as its ten 16x16 blocks on and below the diagonal (block (i, j) at index i (i + 1) / 2 + j, row-major
+ * inside a block): AT is [chunks, H, 10, 16, 16] (chunk index as in `indices`, or b * ceil(T/64) + c).
  * g is the raw per-head log-gate [B,T,H] (g_is_cumsum == 0; its chunk-local prefix sum is formed in the kernel and
  * written to g_cumsum_out, fp32 [B,T,H], if that is given), or already the prefix sum (== 1), or NULL (no gate).
  * w [B,T,H,K] and Aw [B,T,H,64] in the q/k/v dtype, both given or both NULL: w = Aw (beta k) and Aw = (I + M)^-1 as
@@ -315,15 +313,16 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * K in {64, 128}.
  * fla_chunk_gated_delta_rule_fwd_scan is the serial part (state scan + output, replaces
  * chunk_gated_delta_rule_fwd_h + chunk_fwd_o, fla/ops/gated_delta_rule/chunk.py:47-72): with h the state entering
- * a chunk,  v_new = Tu (v - e^{gamma} (k h)),  o = scale e^{gamma} (q h) + Aqk v_new,
+ * a chunk and Aqk = scale tril(q k^T * Gamma) (the score product of chunk_fwd_o, fla/ops/common/chunk_o.py:86-97,
+ * formed inside the scan one chunk ahead),  v_new = Tu (v - e^{gamma} (k h)),  o = scale e^{gamma} (q h) + Aqk v_new,
  * h <- e^{gamma_last} h + k^T (e^{gamma_last - gamma} v_new).  g_cumsum fp32 [B,T,H] or NULL; h0, ht fp32
  * [N,H,K,V] or NULL; packed batches need chunk_offsets [N+1]; seq_order as for fla_chunk_gla_fwd_fused.
  * v_new [B,T,H,V] and h_frag_t (the state entering every chunk, FLA_H_FRAGMENT_T, [chunks,H,K*V]), both in
  * the q/k/v dtype and both given or both NULL: what a forward that will be differentiated keeps for
  * fla_chunk_gated_delta_rule_bwd.
  * K in {64, 128}, V a multiple of 64. */
-int fla_gdr_fwd_prep(const void* q, const void* k, const float* beta, const float* g, int g_is_cumsum,
-                     float* g_cumsum_out, void* AT, void* w, void* Aw, float scale, const int64_t* offsets,
+int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_cumsum,
+                     float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
                      const int64_t* indices,
                      int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, fla_stream_t stream);
 

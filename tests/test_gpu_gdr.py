@@ -77,9 +77,8 @@ def _dense_tiles(ref, beta, B, T, H, offsets=None):
 
 @pytest.mark.parametrize("B,T,H,K,V", [(2, 200, 2, 128, 128), (2, 64, 2, 64, 64), (1, 1, 1, 128, 64), (2, 300, 3, 64, 128)])
 def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
-    """The operator's own decomposition: fla_gdr_fwd_prep (gate prefix sums, Tu = Au diag(beta) and the gated
-    scores as packed triangular tiles) against the fp32 chunked oracle, then the scan on them against the
-    naive recurrence."""
+    """The operator's own decomposition: fla_gdr_fwd_prep (gate prefix sums and Tu = Au diag(beta) as a packed
+    triangular tile) against the fp32 chunked oracle, then the scan on it against the naive recurrence."""
     from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_scan
     from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_scan_operands, unpack_triangular_tiles
     from oracle.chunked import chunked_gated_delta_rule
@@ -88,19 +87,18 @@ def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
     ref = chunked_gated_delta_rule(q, k, v, g, beta, initial_state=h0)
     dev = lambda x: x.to(device)
     print(f"gdr prep + scan B={B} T={T} H={H} K={K} V={V}", flush=True)
-    AT, gc = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), K ** -0.5)
+    AT, gc = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g))
     torch.cuda.synchronize()
     torch.testing.assert_close(gc.cpu(), ref['g_cumsum'], rtol=1e-5, atol=1e-5)
     dense = unpack_triangular_tiles(AT).float().cpu()
-    tu_ref, aqk_ref = _dense_tiles(ref, beta, B, T, H)
-    assert_close("Tu", tu_ref, dense[:, :, 0], 5e-3)
-    assert_close("Aqk", aqk_ref, dense[:, :, 1], 5e-3)
+    tu_ref, _ = _dense_tiles(ref, beta, B, T, H)
+    assert_close("Tu", tu_ref, dense, 5e-3)
     assert torch.equal(dense.triu(1), torch.zeros_like(dense))          # nothing above the diagonal
     # the same tiles from gates that are already cumulative
-    AT2, gc2 = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), gc, K ** -0.5, g_is_cumsum=True)
+    AT2, gc2 = fwd_prepare_scan_operands(dev(k), dev(beta), gc, g_is_cumsum=True)
     assert gc2 is gc and torch.equal(AT, AT2)
     # the variant a differentiated forward runs: the same tiles, plus w = Aw (beta k) and Aw for the backward
-    AT3, gc3, w, Aw = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), K ** -0.5, keep_w=True)
+    AT3, gc3, w, Aw = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g), keep_w=True)
     torch.cuda.synchronize()
     assert torch.equal(AT, AT3) and torch.equal(gc, gc3)
     assert_close("Aw", ref['Aw'], Aw, 5e-3)
@@ -125,14 +123,12 @@ def test_gdr_two_launch_forward_pieces_packed(device):
     dev = lambda x: x.to(device)
     plan = VarlenPlan(dev(offs), 64)
     print(f"gdr prep + scan packed {offs.tolist()}", flush=True)
-    AT, gc = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), 128 ** -0.5, offsets=plan.offsets,
-                                       indices=plan.indices)
+    AT, gc = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g), offsets=plan.offsets, indices=plan.indices)
     torch.cuda.synchronize()
     dense = unpack_triangular_tiles(AT).float().cpu()
-    tu_ref, aqk_ref = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
-    assert_close("Tu", tu_ref, dense[:, :, 0], 5e-3)
-    assert_close("Aqk", aqk_ref, dense[:, :, 1], 5e-3)
-    AT3, _, w, Aw = fwd_prepare_scan_operands(dev(q), dev(k), dev(beta), dev(g), 128 ** -0.5, offsets=plan.offsets,
+    tu_ref, _ = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
+    assert_close("Tu", tu_ref, dense, 5e-3)
+    AT3, _, w, Aw = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g), offsets=plan.offsets,
                                               indices=plan.indices, keep_w=True)
     torch.cuda.synchronize()
     assert torch.equal(AT, AT3)
@@ -146,6 +142,42 @@ def test_gdr_two_launch_forward_pieces_packed(device):
                                                offsets=offs.tolist())
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
+
+
+@pytest.mark.parametrize("K", [64, 128])
+@pytest.mark.parametrize("B,H", [(2, 2), (3, 48)])
+def test_gdr_scan_forms_the_gated_scores(device, K, B, H):
+    """The scan forms Aqk = scale tril(q k^T * Gamma) itself, one chunk ahead of its use.  With Tu the identity, a
+    zero initial state and v zero except in one chunk, where its rows are unit vectors, the state entering that
+    chunk is zero and the output rows of the chunk are Aqk: checked against the fp32 chunked oracle's scores for
+    the first chunk (formed before the loop), inner chunks and a short last chunk; (3, 48) runs 64-column slabs
+    of a 128-column value (four waves share the blocks), (2, 2) 32-column slabs of a 64-column one (two waves)."""
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_scan
+    from oracle.chunked import chunked_gated_delta_rule
+    T, V = 64 * 4 + 37, 64 if H == 2 else 128
+    q, k, v, g, beta, _ = gdr_inputs(B, T, H, K, V, seed=23)
+    ref = chunked_gated_delta_rule(q[:1, :, :2], k[:1, :, :2], v[:1, :, :2], g[:1, :, :2], beta[:1, :, :2])
+    _, aqk_ref = _dense_tiles(ref, beta[:1, :, :2], 1, T, 2)
+    chunks = -(-T // 64)
+    eye_tile = torch.zeros(10, 16, 16)
+    for i in range(4):
+        eye_tile[i * (i + 1) // 2 + i] = torch.eye(16)
+    AT = eye_tile.expand(B * chunks, H, 10, 16, 16).contiguous().to(device).bfloat16()
+    gc = g.view(B, T, H).clone()
+    for c0 in range(0, T, 64):
+        gc[:, c0:c0 + 64] = g[:, c0:c0 + 64].cumsum(1)
+    dev = lambda x: x.to(device)
+    for c in (0, 1, chunks - 2, chunks - 1):
+        L = min(64, T - 64 * c)
+        print(f"gdr scan scores K={K} B={B} H={H} chunk {c}", flush=True)
+        vv = torch.zeros(B, T, H, V)
+        vv[:, 64 * c:64 * c + L, :, :L] = torch.eye(L)[None, :, None, :]
+        o, ht = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(vv.bfloat16()), AT, dev(gc), K ** -0.5, None, True)
+        torch.cuda.synchronize()
+        got = o[0, 64 * c:64 * c + L, :2, :L].float().cpu().permute(1, 0, 2)     # [head, row, column]
+        assert_close(f"Aqk of chunk {c}", aqk_ref[c, :, :L, :L], got, 5e-3)
+        assert torch.equal(got.triu(1), torch.zeros_like(got))
+        assert torch.equal(o[:, :64 * c].float().cpu(), torch.zeros(B, 64 * c, H, V))   # nothing before the chunk
 
 
 @pytest.mark.parametrize("varlen", [False, True])
