@@ -633,7 +633,11 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     if (offsets) FLA_REQUIRE(chunk_offsets != nullptr, FLA_E_INVALID);
   }
   FLA_REQUIRE((qg == nullptr) == (decay == nullptr), FLA_E_INVALID);
-  if (qg) FLA_REQUIRE(h_frag_t != nullptr && (uintptr_t)qg % 16 == 0 && V <= 256, FLA_E_INVALID);
+  if (qg) {
+    FLA_REQUIRE(h_frag_t != nullptr, FLA_E_INVALID);
+    FLA_REQUIRE(V <= 256, FLA_E_UNSUPPORTED);
+    FLA_REQUIRE((uintptr_t)qg % 16 == 0, FLA_E_ALIGNMENT);
+  }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
                 T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay};
   hipStream_t st = (hipStream_t)stream;

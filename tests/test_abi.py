@@ -53,6 +53,20 @@ def test_argument_validation_without_device():
     # the allocation-free cumsum refuses what its static scratch array (4 Mi floats) cannot hold
     assert lib.fla_chunk_global_cumsum_static(p, p, 0, 0, 1, 4 * 1024 * 1024 // 64 + 1, 8, 8, 64, 0, None, None, 0, None) == -4
     assert lib.fla_chunk_global_cumsum_static(None, p, 0, 0, 1, 1, 1, 1, 64, 0, None, None, 0, None) == -1
+    # the states-keeping GLA forward that also leaves gated queries and chunk decays: all three outputs or none,
+    # at most 256 value columns; its backward divides by the scale
+    z = (None,) * 4
+    fwd = lambda hT, qg, dec, V: lib.fla_chunk_gla_fwd_fused_kept(p, p, p, p, None, p, None, None, None, hT, qg, dec, *z,
+                                                                  0, 0, 2, 1, 64, 1, 64, V, 1, 1.0, None)
+    assert fwd(p, p, None, 64) == -1 and fwd(None, p, p, 64) == -1 and fwd(p, None, None, 64) == -1
+    assert fwd(p, p, p, 320) == -2
+    bwd = lambda qg, dec, scale: lib.fla_chunk_gla_bwd_kept(p, p, p, p, p, None, p, qg, dec, p, p, p, p, p, None, None,
+                                                            None, None, None, 0, 0, 2, 1, 64, 1, 64, 64, 1, scale, None)
+    assert bwd(p, None, 1.0) == -1 and bwd(p, p, 0.0) == -1
+    # the delta rule's chunk-parallel launch: w and Aw together or not at all, K in {64, 128}
+    prep = lambda w, Aw, K: lib.fla_gdr_fwd_prep(p, p, None, 0, None, p, w, Aw, None, None, 0, 0, 1, 64, 1, K, None)
+    assert prep(p, None, 64) == -1 and prep(None, p, 64) == -1
+    assert lib.fla_gdr_fwd_prep(None, p, None, 0, None, p, None, None, None, None, 0, 0, 1, 64, 1, 64, None) == -1
 
 
 @pytest.mark.parametrize("bt", [16, 64])
