@@ -212,6 +212,7 @@ struct DhuParams {
   const void* w;
   const void* dout;
   const void* dvl;
+  const void* Aqk;   // FROMP: the packed score tiles the forward kept, [chunks, H, 10, 16, 16] (dvl unused)
   const float* gam;
   const float* dht;
   void* dv2;
@@ -241,7 +242,10 @@ struct DhuParams {
 // the staging waves are bound by the instructions they issue (a memory instruction costs the issuing wave about
 // 70 cycles once the CU's memory pipeline is full), the matrix waves have time to spare - and every transposed
 // operand is read from a row-major tile with the transposing LDS load.
-template <typename T, int K>
+// FROMP: dv_loc = Aqk^T do is not read from memory but formed here from the packed score tile Aqk the forward
+// kept (5 KB per chunk and head) and the raw do rows, which then travel with the k group: four more small
+// matrix products per wave and chunk instead of a launch that reads q, k, do and writes dv_loc.
+template <typename T, int K, bool FROMP>
 __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
@@ -256,7 +260,8 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
   __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];      // q, row-major
   __shared__ __attribute__((aligned(16))) T sW[BT * LDK];      // w, row-major
   __shared__ __attribute__((aligned(16))) T sDo[BT * LDV];     // s e^{gamma} * do, row-major [t][v]
-  __shared__ __attribute__((aligned(16))) T sDvl[BT * LDV];    // dv_loc, row-major [t][v]
+  __shared__ __attribute__((aligned(16))) T sDvl[BT * LDV];    // dv_loc (FROMP: do), row-major [t][v]
+  __shared__ __attribute__((aligned(16))) T sP[FROMP ? kTriElems : 8];   // FROMP: Aqk, packed triangular tile
   __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];    // dH^T in 16-bit
   __shared__ __attribute__((aligned(16))) T sDv2T[BV * LDT];   // dv2^T
   __shared__ __attribute__((aligned(16))) T sDv2s[BV * LDT];   // (-e^{gamma} * dv2)^T
@@ -294,7 +299,8 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     };
     struct YRegs {
       v8 k[NP];
-      v8 dvl;
+      v8 dvl;       // FROMP: do
+      v8 a0, a1;    // FROMP: pieces of the score tile
       float gam, glast;
     };
     // Loads are unconditional (a load under a branch makes the wave drain its whole load queue at the
@@ -312,7 +318,9 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     const char* gk = (const char*)p.k + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
     const char* gw = (const char*)p.w + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
     const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
-    const char* gl = (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const char* gl = FROMP ? gd : (const char*)p.dvl + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const char* ga = FROMP ? (const char*)p.Aqk + (chunk0 * H + hh) * (int64_t)kTriElems * (int64_t)sizeof(T) : nullptr;
+    const uint32_t offa0 = 16 * (uint32_t)st, offa1 = 16 * (uint32_t)(256 + (st & 63));
     // without gates every gate load reads one zero word (no select on the loaded value: it would
     // make the wave wait for the load where it is issued)
     const char* gg = p.gam ? (const char*)p.gam + (sp.bos * H + hh) * 4 : (const char*)&kZeroWord;
@@ -327,8 +335,10 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
         R.q[i] = *(const v8*)(gq + ck + o);
         R.w[i] = *(const v8*)(gw + ck + o);
       }
-      const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
-      R.d = *(const v8*)(gd + cv + (offv < lv ? offv : lv));
+      if constexpr (!FROMP) {
+        const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+        R.d = *(const v8*)(gd + cv + (offv < lv ? offv : lv));
+      }
     };
     auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
       c = c < 0 ? 0 : c;
@@ -339,6 +349,11 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
       for (int i = 0; i < NP; ++i) R.k[i] = *(const v8*)(gk + ck + (offk[i] < lk ? offk[i] : lk));
       const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
       R.dvl = *(const v8*)(gl + cv + (offv < lv ? offv : lv));
+      if constexpr (FROMP) {
+        const char* pa = ga + c * (int64_t)H * kTriElems * (int64_t)sizeof(T);
+        R.a0 = *(const v8*)(pa + offa0);
+        R.a1 = *(const v8*)(pa + offa1);   // the last 64 pieces: every wave loads them, the first one writes them
+      }
       const uint32_t og = offg < last * pitchG ? offg : last * pitchG;
       R.gam = *(const float*)(gg + cg + (p.gam ? og : 0u));
       R.glast = *(const float*)(gg + cg + (p.gam ? last * pitchG : 0u));
@@ -346,6 +361,7 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
     // s e^{gamma} of this lane's do row in the chunk held in X (zero past its end): formed when the same chunk
     // is staged as Y, half a period earlier, so that nothing loop-carried depends on a load in flight
     float egx = 0.f;
+    v8 dkeep;   // FROMP: this lane's do piece of the chunk last staged as Y
     auto stage_x = [&](const XRegs& R) __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < NP; ++i) {
@@ -354,7 +370,7 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
       }
       v8 x;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) x[j] = (T)((float)R.d[j] * egx);
+      for (int j = 0; j < 8; ++j) x[j] = (T)((float)(FROMP ? dkeep[j] : R.d[j]) * egx);
       *(v8*)&sDo[vrow * LDV + vc8] = x;
     };
     auto stage_y = [&](const YRegs& R, int64_t c) __attribute__((always_inline)) {
@@ -362,6 +378,11 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
 #pragma unroll
       for (int i = 0; i < NP; ++i) *(v8*)&sK[(prow + PR * i) * LDK + c8] = R.k[i];
       *(v8*)&sDvl[vrow * LDV + vc8] = R.dvl;
+      if constexpr (FROMP) {
+        dkeep = R.dvl;
+        *(v8*)&sP[st * 8] = R.a0;
+        if (wave == 4) *(v8*)&sP[2048 + lane * 8] = R.a1;
+      }
       const float eg = vrow < L ? __expf(R.gam) : 0.f;
       egx = p.scale * eg;
       if ((st & 3) == 0) {
@@ -476,13 +497,34 @@ __global__ __launch_bounds__(512) void gdr_bwd_dhu_kernel(DhuParams p) {
         }
         const int tr = wave * 16 + 4 * (lane >> 4);
         const f32x4 ed = *(const f32x4*)&sEd[tr], eg = *(const f32x4*)&sEg[tr];
+        f32x4 dl[2] = {zero4(), zero4()};
+        if constexpr (FROMP) {
+          // dv_loc rows 16 wave ..: sum over the time rows i of Aqk[i][t] do[i][v]; Aqk^T comes out of the
+          // row-major 16x16 blocks (row blocks 2s and 2s+1 of column block `wave`) through the transposing load,
+          // blocks above the diagonal are not stored
+          typedef short s4 __attribute__((ext_vector_type(4)));
+          typedef __attribute__((address_space(3))) s4 lds_s4;
+          const int jj = lane & 15, gg = lane >> 4;
+          const int off = (4 * gg + (jj >> 2)) * 16 + 4 * (jj & 3);
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            const int t0 = 2 * s, t1 = 2 * s + 1;
+            if (t1 < wave) continue;   // wave-uniform
+            s4 lo = {0, 0, 0, 0};
+            if (t0 >= wave) lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sP[(t0 * (t0 + 1) / 2 + wave) * 256 + off]);
+            s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sP[(t1 * (t1 + 1) / 2 + wave) * 256 + off]);
+            const v8 a = __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) dl[j] = Elem<T>::mfma16(a, frag16_tr<T>(sDvl, LDV, 16 * j, 32 * s, lane), dl[j]);
+          }
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           int vc = j * 16 + (lane & 15);
           v4 o, os;
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float x = (float)sDvl[(tr + r) * LDV + vc] + ed[r] * d[j][r];
+            const float x = (FROMP ? dl[j][r] : (float)sDvl[(tr + r) * LDV + vc]) + ed[r] * d[j][r];
             o[r] = (T)x;
             os[r] = (T)(-eg[r] * x);
           }
@@ -1355,9 +1397,13 @@ int launch_dhu(const DhuParams& p, int64_t K, hipStream_t st) {
   const int64_t total = (int64_t)(p.V / 32) * p.N * p.H;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
   if (total == 0) return FLA_OK;
-  if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64>), dim3((unsigned)total), dim3(512), 0, st, p);
-  else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256>), dim3((unsigned)total), dim3(512), 0, st, p);
-  else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128>), dim3((unsigned)total), dim3(512), 0, st, p);
+  if (p.Aqk) {
+    if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64, true>), dim3((unsigned)total), dim3(512), 0, st, p);
+    else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128, true>), dim3((unsigned)total), dim3(512), 0, st, p);
+    else return FLA_E_UNSUPPORTED;
+  } else if (K == 64) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 64, false>), dim3((unsigned)total), dim3(512), 0, st, p);
+  else if (K == 256) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 256, false>), dim3((unsigned)total), dim3(512), 0, st, p);
+  else if (K == 128) hipLaunchKernelGGL((gdr_bwd_dhu_kernel<T, 128, false>), dim3((unsigned)total), dim3(512), 0, st, p);
   else return FLA_E_UNSUPPORTED;
   FLA_CHECK_LAUNCH();
   return FLA_OK;
@@ -1397,8 +1443,8 @@ int launch_wy_bwd(const WyBwdParams& p, int64_t K, int64_t V, dim3 grid, hipStre
 
 template <typename T>
 int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, const void* vnew, const float* beta,
-                   const float* gam, const void* Aw, const void* dout, const float* dht, const void* hT, void* dvl,
-                   void* dv2, void* dhtf, void* dw, void* dkp, float* dgam_part, void* dq, void* dk, void* dv,
+                   const float* gam, const void* Aw, const void* dout, const float* dht, const void* hT,
+                   const void* Aqk, void* dvl, void* dv2, void* dhtf, void* dw, void* dkp, float* dgam_part, void* dq, void* dk, void* dv,
                    float* dbeta, float* dgam2, float* dh0, const int64_t* offsets, const int64_t* indices,
                    const int64_t* chunk_offsets, int64_t NT, int64_t B, int64_t T_, int64_t H, int64_t K, int64_t V,
                    int64_t N, float scale, hipStream_t st) {
@@ -1407,9 +1453,11 @@ int launch_gdr_bwd(const void* q, const void* k, const void* v, const void* w, c
   int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
-  DvlParams p1{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
-  if ((rc = launch_dv_local<T>(p1, K, V, grid, st))) return rc;
-  DhuParams p2{q, k, w, dout, dvl, gam, dht, dv2, dhtf, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N, scale};
+  if (!Aqk) {   // dv_loc by a launch of its own unless the forward kept its score tiles
+    DvlParams p1{q, k, dout, gam, dvl, offsets, indices, T_, (int)H, ntfix, scale};
+    if ((rc = launch_dv_local<T>(p1, K, V, grid, st))) return rc;
+  }
+  DhuParams p2{q, k, w, dout, dvl, Aqk, gam, dht, dv2, dhtf, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N, scale};
   if ((rc = launch_dhu<T>(p2, K, st))) return rc;
   DqkwgParams p3{q, k, vnew, w, dout, dv2, gam, hT, dhtf, dq, dkp, dw, dgam_part, offsets, indices, T_,
                  B * T_, (int)H, (int)K, ntfix, scale};
@@ -1441,25 +1489,26 @@ extern "C" int fla_chunk_bwd_dv_local(const void* q, const void* k, const float*
 
 extern "C" int fla_chunk_gated_delta_rule_bwd(
     const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,
-    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT,
+    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT, const void* Aqk,
     void* ws_dv_local, void* ws_dv2, void* ws_dh_frag_t, void* ws_dw, void* ws_dk_partial, float* ws_dgam_partial,
     void* dq, void* dk, void* dv, float* dbeta, float* dgam2, float* dh0,
     const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,
     int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream) {
-  FLA_REQUIRE(q && k && v && w && v_new && beta && Aw && dout && hT && ws_dv_local && ws_dv2 && ws_dh_frag_t &&
+  FLA_REQUIRE(q && k && v && w && v_new && beta && Aw && dout && hT && (ws_dv_local || Aqk) && ws_dv2 && ws_dh_frag_t &&
                   ws_dw && ws_dk_partial && ws_dgam_partial && dq && dk && dv && dbeta && dgam2,
               FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE((K == 64 || K == 128 || K == 256) && (V == 64 || V == 128), FLA_E_UNSUPPORTED);
+  if (Aqk) FLA_REQUIRE(K <= 128 && (uintptr_t)Aqk % 16 == 0, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
   hipStream_t st = (hipStream_t)stream;
   if (qkv_dtype == FLA_BF16)
-    return launch_gdr_bwd<bf16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, ws_dv_local, ws_dv2,
+    return launch_gdr_bwd<bf16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, Aqk, ws_dv_local, ws_dv2,
                                 ws_dh_frag_t, ws_dw, ws_dk_partial, ws_dgam_partial, dq, dk, dv, dbeta, dgam2, dh0,
                                 offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st);
   if (qkv_dtype == FLA_F16)
-    return launch_gdr_bwd<f16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, ws_dv_local, ws_dv2,
+    return launch_gdr_bwd<f16>(q, k, v, w, v_new, beta, g_cumsum, Aw, dout, dht, hT, Aqk, ws_dv_local, ws_dv2,
                                ws_dh_frag_t, ws_dw, ws_dk_partial, ws_dgam_partial, dq, dk, dv, dbeta, dgam2, dh0,
                                offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st);
   return FLA_E_UNSUPPORTED;
@@ -1479,7 +1528,7 @@ extern "C" int fla_chunk_gated_delta_rule_bwd_dhu(const void* q, const void* k, 
                (uintptr_t)dv2) % 16 == 0, FLA_E_ALIGNMENT);
   hipStream_t st = (hipStream_t)stream;
   if (N == 0 || T == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);
-  DhuParams p{q, k, w, dout, dv, g_cumsum, dht, dv2, dh_frag_t, dh0, offsets, chunk_offsets, T, (int)H, (int)V, (int)N,
+  DhuParams p{q, k, w, dout, dv, nullptr, g_cumsum, dht, dv2, dh_frag_t, dh0, offsets, chunk_offsets, T, (int)H, (int)V, (int)N,
               scale};
   if (qkv_dtype == FLA_BF16) return launch_dhu<bf16>(p, K, st);
   if (qkv_dtype == FLA_F16) return launch_dhu<f16>(p, K, st);

@@ -53,6 +53,7 @@ struct GdrScanParams {
   float* ht;
   void* v_new;      // KEEP: [rows, H, V]
   void* h_frag_t;   // KEEP: [chunks, H, K*V], FLA_H_FRAGMENT_T
+  void* Aqk_out;    // KEEP: [chunks, H, 10, 16, 16], the gated scores (or NULL)
   const int64_t* offsets;
   const int64_t* chunk_offsets;
   const int64_t* seq_order;  // sequence ids, longest first (or NULL)
@@ -138,10 +139,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // block: a block is computed transposed (k rows against q rows), which leaves every lane with four
   // adjacent entries of one row of Aqk - an 8-byte piece of the packed tile frag_tri() reads.  Rows past the
   // end of a short chunk are zero in the q and k tiles.
-  auto compute_p = [&](int b3, int pb) __attribute__((always_inline)) {
+  auto compute_p = [&](int b3, int pb, int chunk) __attribute__((always_inline)) {
     const T* Kr = sK[b3];
     const T* Q = sQ[b3];
     T* Po = sP[pb];
+    // KEEP: the first value slab of a head also leaves the tile in memory for the backward pass
+    T* Pg = nullptr;
+    if constexpr (KEEP) {
+      if (vb == 0 && p.Aqk_out) Pg = (T*)p.Aqk_out + ((chunk0 + chunk) * H + hh) * (int64_t)kTriElems;
+    }
     const int c = lane & 15, g = lane >> 4;
     // (row block, column block) of this wave's blocks, a nibble each, first in the low bits: two or three
     // blocks for each of the four waves, or five for each of the two waves that carry no state
@@ -176,6 +182,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int r = 0; r < 4; ++r)
           o[r] = (T)((ti > tj || 4 * g + r <= c) ? p.scale * sc[r] * __expf(gi - gj[r]) : 0.f);
         *(v4*)&Po[(ti * (ti + 1) / 2 + tj) * 256 + c * 16 + 4 * g] = o;
+        if constexpr (KEEP) {
+          if (Pg) *(v4*)&Pg[(ti * (ti + 1) / 2 + tj) * 256 + c * 16 + 4 * g] = o;
+        }
       }
     }
   };
@@ -389,12 +398,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // waves without a share of the state form their share of the scores and keep the barrier count
     if (nchunks > 0) {
       lds_barrier();
-      compute_p(0, 0);
+      compute_p(0, 0, 0);
       lds_barrier();
       int b3 = 0;
       for (int ci = 0; ci < nchunks; ++ci) {
         const int n3 = b3 == 2 ? 0 : b3 + 1;
-        if (ci + 1 < nchunks) compute_p(n3, (ci + 1) & 1);
+        if (ci + 1 < nchunks) compute_p(n3, (ci + 1) & 1, ci + 1);
         lds_barrier();
         b3 = n3;
       }
@@ -435,7 +444,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int Llast = (int)(sp.len - (int64_t)(nchunks - 1) * BT);
     if (nchunks > 0) {
       lds_barrier();
-      if constexpr (NMW == 4) compute_p(0, 0);
+      if constexpr (NMW == 4) compute_p(0, 0, 0);
       lds_barrier();
       int b3 = 0;   // ci modulo 3
       for (int ci = 0; ci < nchunks; ++ci) {
@@ -446,7 +455,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const T* Tu = sAT[b];
         const T* P = sP[b];
         if constexpr (NMW == 4) {
-          if (ci + 1 < nchunks) compute_p(n3, b ^ 1);   // with 32-column slabs the two other waves form the scores
+          if (ci + 1 < nchunks) compute_p(n3, b ^ 1, ci + 1);   // with 32-column slabs the two other waves form the scores
         }
         const int vrow = cb + c;
         T* vt = &sVt[b][vrow * LDT];
@@ -643,7 +652,7 @@ int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
 
 extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
                                                    const float* g_cumsum, const float* h0, void* o, float* ht,
-                                                   void* v_new, void* h_frag_t, const int64_t* offsets, const int64_t* chunk_offsets,
+                                                   void* v_new, void* h_frag_t, void* Aqk_out, const int64_t* offsets, const int64_t* chunk_offsets,
                                                    const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
                                                    int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                                    fla_stream_t stream) {
@@ -652,9 +661,10 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k,
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
   FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
   FLA_REQUIRE((v_new == nullptr) == (h_frag_t == nullptr), FLA_E_INVALID);
+  FLA_REQUIRE(Aqk_out == nullptr || v_new != nullptr, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o | (uintptr_t)v_new |
-               (uintptr_t)h_frag_t) % 16 == 0, FLA_E_ALIGNMENT);
-  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
+               (uintptr_t)h_frag_t | (uintptr_t)Aqk_out) % 16 == 0, FLA_E_ALIGNMENT);
+  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
   if (qkv_dtype == FLA_BF16) return launch_scan<bf16>(p, (int)K, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_scan<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;

@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -51,7 +51,7 @@ SIGNATURES = {
                                                  I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h_both": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, P]),
     "fla_gdr_fwd_prep": (c_int, [P, P, P, I, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, P]),
-    "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 13 + [I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 14 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 17 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_kept": (c_int, [P] * 19 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
@@ -61,7 +61,7 @@ SIGNATURES = {
     "fla_chunk_bwd_dh": (c_int, [P] * 9 + [I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_states_to_fragments": (c_int, [P, P, I, I, I, I64, I64, I64, P]),
     "fla_chunk_bwd_dv_local": (c_int, [P] * 7 + [I64, I, I64, I64, I64, I64, I64, F, P]),
-    "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 26 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gated_delta_rule_bwd": (c_int, [P] * 27 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_bwd_dhu": (c_int, [P] * 12 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_bwd_dqkwg": (c_int, [P] * 15 + [I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_bwd_prepare_wy_repr": (c_int, [P] * 14 + [I64, I, I64, I64, I64, I64, I64, P]),

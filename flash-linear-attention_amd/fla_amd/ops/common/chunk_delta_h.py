@@ -125,8 +125,9 @@ def chunk_gated_delta_rule_fwd_scan(
     ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o`` (``fla/ops/gated_delta_rule/chunk.py:47-72``)
     on ``q, k, v`` and the packed triangular tiles ``AT`` of ``fwd_prepare_scan_operands``; neither w, u,
     v_new nor the per-chunk states are materialised.  ``g`` is the fp32 chunk-local cumsum.  Seq-first.
-    Returns ``(o, final_state)``; with ``keep`` also ``v_new`` and the state entering every chunk in
-    transposed-fragment order (``[B, NT, H, K, V]``), what the backward reads: ``(o, final_state, v_new, hT)``."""
+    Returns ``(o, final_state)``; with ``keep`` also ``v_new``, the state entering every chunk in
+    transposed-fragment order (``[B, NT, H, K, V]``) and the packed score tiles ``Aqk``
+    (``[chunks, H, 10, 16, 16]``), what the backward reads: ``(o, final_state, v_new, hT, Aqk)``."""
     be.require_gpu(q, k, v, AT)
     B, T, H, K = k.shape
     V = v.shape[-1]
@@ -141,16 +142,17 @@ def chunk_gated_delta_rule_fwd_scan(
         h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
     if g is not None and g.dtype != torch.float32:
         g = g.float()
-    v_new = hT = None
+    v_new = hT = Aqk = None
     if keep:
         v_new = torch.empty_like(v)
         hT = k.new_empty(B, AT.shape[0] // B if offsets is None else AT.shape[0], H, K, V)
+        Aqk = torch.empty_like(AT)
     be.check(be.lib().fla_chunk_gated_delta_rule_fwd_scan(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(v_new),
-        be.ptr(hT), be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale),
-        be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan")
+        be.ptr(hT), be.ptr(Aqk), be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N,
+        float(scale), be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan")
     if keep:
-        return o, ht, v_new, hT
+        return o, ht, v_new, hT, Aqk
     return o, ht
 
 

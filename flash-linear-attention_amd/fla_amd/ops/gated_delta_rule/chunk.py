@@ -80,7 +80,7 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
 
 def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, output_final_state, offsets=None):
     """Forward of a pass that will be differentiated.  Returns ``(g_cumsum, o, final_state, kept)``
-    with ``kept = (w, Aw, v_new, hT)`` for :func:`chunk_gated_delta_rule_bwd`.  Key dims up to 128: the
+    with ``kept = (w, Aw, v_new, hT[, Aqk])`` for :func:`chunk_gated_delta_rule_bwd`.  Key dims up to 128: the
     two-launch forward, whose first launch also writes ``w`` and ``Aw`` and whose scan also writes ``v_new`` and
     the state entering every chunk.  K = 256: the reference's decomposition (WY launch, state scan, output stage)."""
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
@@ -90,10 +90,10 @@ def chunk_gated_delta_rule_fwd_keep(q, k, v, g, beta, scale, initial_state, outp
     beta = beta.float().contiguous()
     if q.shape[-1] <= _FUSED_MAX_K:
         AT, g, w, Aw = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, keep_w=True)
-        o, final_state, v_new, hT = chunk_gated_delta_rule_fwd_scan(
+        o, final_state, v_new, hT, Aqk = chunk_gated_delta_rule_fwd_scan(
             q, k, v, AT, g, scale, initial_state, output_final_state, offsets=offs, chunk_offsets=co,
             seq_order=None if plan is None else plan.seq_order, keep=True)
-        return g, o, final_state, (w, Aw, v_new, hT)
+        return g, o, final_state, (w, Aw, v_new, hT, Aqk)
     g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
     w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
                                       store_A=True, store_Au=False)
@@ -118,8 +118,10 @@ def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do
     N = B if plan is None else plan.N
     NT = 0 if plan is None else plan.NT
     beta = beta.float().contiguous()
+    Aqk = None
     if kept is not None:
-        w, Aw, v_new, hT = kept
+        w, Aw, v_new, hT = kept[:4]
+        Aqk = kept[4] if len(kept) > 4 else None   # the score tiles of the two-launch forward (K <= 128)
     else:
         w, u, Aw, _ = fwd_prepare_wy_repr(k, v, beta, g_cumsum, offsets=offs, indices=idx, head_first=False,
                                           chunk_size=BT, store_A=True, store_Au=False)
@@ -127,7 +129,7 @@ def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do
             k=k, w=w, u=u, g=g_cumsum, initial_state=initial_state, output_final_state=False, offsets=offs,
             indices=idx, head_first=False, chunk_size=BT, fragment_layout=True, transposed_fragments=True,
             chunk_offsets=co)
-    ws_dvl, ws_dv2 = torch.empty_like(v), torch.empty_like(v)
+    ws_dvl, ws_dv2 = (torch.empty_like(v) if Aqk is None else None), torch.empty_like(v)
     ws_dh = torch.empty_like(hT)
     ws_dw, ws_dkp = torch.empty_like(k), torch.empty_like(k)
     ws_dgam = q.new_empty(K // 64, B * T, H, dtype=torch.float32)
@@ -139,7 +141,7 @@ def chunk_gated_delta_rule_bwd(q, k, v, g_cumsum, beta, scale, initial_state, do
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
     be.check(be.lib().fla_chunk_gated_delta_rule_bwd(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(w), be.ptr(v_new), be.ptr(beta), be.ptr(g_cumsum), be.ptr(Aw),
-        be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(ws_dvl), be.ptr(ws_dv2), be.ptr(ws_dh), be.ptr(ws_dw),
+        be.ptr(do), be.ptr(dht), be.ptr(hT), be.ptr(Aqk), be.ptr(ws_dvl), be.ptr(ws_dv2), be.ptr(ws_dh), be.ptr(ws_dw),
         be.ptr(ws_dkp), be.ptr(ws_dgam), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dbeta), be.ptr(dg),
         be.ptr(dh0), be.ptr(offs), be.ptr(idx), be.ptr(co), NT, be.dt(q), B, T, H, K, V, N, float(scale),
         be.stream_of(q)), "fla_chunk_gated_delta_rule_bwd")

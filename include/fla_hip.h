@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 6
+#define FLA_ABI_VERSION 7
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -319,7 +319,8 @@ int fla_chunk_fwd_o(const void* q, const void* k, const void* v, const float* g_
  * [N,H,K,V] or NULL; packed batches need chunk_offsets [N+1]; seq_order as for fla_chunk_gla_fwd_fused.
  * v_new [B,T,H,V] and h_frag_t (the state entering every chunk, FLA_H_FRAGMENT_T, [chunks,H,K*V]), both in
  * the q/k/v dtype and both given or both NULL: what a forward that will be differentiated keeps for
- * fla_chunk_gated_delta_rule_bwd.
+ * fla_chunk_gated_delta_rule_bwd.  Aqk_out (only with those two, or NULL): the score tiles, packed like AT,
+ * [chunks,H,10,16,16], for the same backward.
  * K in {64, 128}, V a multiple of 64. */
 int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_cumsum,
                      float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
@@ -328,7 +329,7 @@ int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_
 
 int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
                                         const float* g_cumsum, const float* h0, void* o, float* ht,
-                                        void* v_new, void* h_frag_t, const int64_t* offsets,
+                                        void* v_new, void* h_frag_t, void* Aqk_out, const int64_t* offsets,
                                         const int64_t* chunk_offsets,
                                         const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                         int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
@@ -435,10 +436,13 @@ int fla_chunk_bwd_dv_local(const void* q, const void* k, const float* g_cumsum, 
  * chunk_gated_delta_rule_bwd (fla/ops/gated_delta_rule/chunk.py:76-177):
  * chunk_bwd_dv_local (common/chunk_o.py:551), chunk_gated_delta_rule_bwd_dhu
  * (common/chunk_delta_h.py:323), chunk_bwd_dqkwg (common/chunk_o.py:602) and
- * bwd_prepare_wy_repr (gated_delta_rule/wy_fast.py:565).  Four launches.
+ * bwd_prepare_wy_repr (gated_delta_rule/wy_fast.py:565).  Four launches, or three with Aqk.
  * Inputs recomputed by the caller with the forward entry points: w, v_new, Aw
  * (fla_gdr_fwd_wy, fla_chunk_gated_delta_rule_fwd_h) and hT (the per-chunk
  * states in FLA_H_FRAGMENT_T order).  g_cumsum fp32 [B,T,H] or NULL.
+ * Aqk: the packed score tiles [chunks,H,10,16,16] that fla_chunk_gated_delta_rule_fwd_scan leaves on request, or
+ * NULL.  With them (K <= 128) the reverse state scan forms dv_local = Aqk^T do itself: the chunk_bwd_dv_local
+ * launch is skipped and ws_dv_local may be NULL.
  * Workspaces: ws_dv_local, ws_dv2 like v; ws_dh_frag_t like hT; ws_dw,
  * ws_dk_partial like k; ws_dgam_partial fp32 [K/64, B*T, H].
  * Outputs: dq, dk [B,T,H,K], dv [B,T,H,V] (q/k/v dtype); dbeta and dg fp32
@@ -450,7 +454,7 @@ int fla_chunk_bwd_dv_local(const void* q, const void* k, const float* g_cumsum, 
  * ---------------------------------------------------------------------- */
 int fla_chunk_gated_delta_rule_bwd(
     const void* q, const void* k, const void* v, const void* w, const void* v_new, const float* beta,
-    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT,
+    const float* g_cumsum, const void* Aw, const void* dout, const float* dht, const void* hT, const void* Aqk,
     void* ws_dv_local, void* ws_dv2, void* ws_dh_frag_t, void* ws_dw, void* ws_dk_partial, float* ws_dgam_partial,
     void* dq, void* dk, void* dv, float* dbeta, float* dg, float* dh0,
     const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int qkv_dtype,

@@ -67,6 +67,10 @@ def test_argument_validation_without_device():
     prep = lambda w, Aw, K: lib.fla_gdr_fwd_prep(p, p, None, 0, None, p, w, Aw, None, None, 0, 0, 1, 64, 1, K, None)
     assert prep(p, None, 64) == -1 and prep(None, p, 64) == -1
     assert lib.fla_gdr_fwd_prep(None, p, None, 0, None, p, None, None, None, None, 0, 0, 1, 64, 1, 64, None) == -1
+    # its scan: v_new and the states together or not at all, the score tiles only with them
+    scan = lambda vn, hT, aqk: lib.fla_chunk_gated_delta_rule_fwd_scan(p, p, p, p, None, None, p, None, vn, hT, aqk, None, None,
+                                                                       None, 0, 1, 64, 1, 64, 64, 1, 1.0, None)
+    assert scan(p, None, None) == -1 and scan(None, None, p) == -1
 
 
 @pytest.mark.parametrize("bt", [16, 64])

@@ -91,7 +91,7 @@ def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
     torch.cuda.synchronize()
     torch.testing.assert_close(gc.cpu(), ref['g_cumsum'], rtol=1e-5, atol=1e-5)
     dense = unpack_triangular_tiles(AT).float().cpu()
-    tu_ref, _ = _dense_tiles(ref, beta, B, T, H)
+    tu_ref, aqk_ref = _dense_tiles(ref, beta, B, T, H)
     assert_close("Tu", tu_ref, dense, 5e-3)
     assert torch.equal(dense.triu(1), torch.zeros_like(dense))          # nothing above the diagonal
     # the same tiles from gates that are already cumulative
@@ -108,6 +108,15 @@ def test_gdr_two_launch_forward_pieces(device, B, T, H, K, V):
     ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True)
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
+    # the scan of a differentiated forward: same outputs, plus v_new, the states and the score tiles it formed
+    o2, ht2, v_new, hT, Aqk = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, K ** -0.5, dev(h0), True,
+                                                              keep=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)
+    assert_close("v_new", ref['v_new'], v_new, 8e-3)
+    dense_p = unpack_triangular_tiles(Aqk).float().cpu()
+    assert_close("Aqk", aqk_ref, dense_p, 5e-3)
+    assert torch.equal(dense_p.triu(1), torch.zeros_like(dense_p))
 
 
 def test_gdr_two_launch_forward_pieces_packed(device):
@@ -126,7 +135,7 @@ def test_gdr_two_launch_forward_pieces_packed(device):
     AT, gc = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g), offsets=plan.offsets, indices=plan.indices)
     torch.cuda.synchronize()
     dense = unpack_triangular_tiles(AT).float().cpu()
-    tu_ref, _ = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
+    tu_ref, aqk_ref = _dense_tiles(ref, beta, 1, T, H, offs.tolist())
     assert_close("Tu", tu_ref, dense, 5e-3)
     AT3, _, w, Aw = fwd_prepare_scan_operands(dev(k), dev(beta), dev(g), offsets=plan.offsets,
                                               indices=plan.indices, keep_w=True)
@@ -142,6 +151,12 @@ def test_gdr_two_launch_forward_pieces_packed(device):
                                                offsets=offs.tolist())
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
+    o2, ht2, _, _, Aqk = chunk_gated_delta_rule_fwd_scan(dev(q), dev(k), dev(v), AT, gc, 128 ** -0.5, dev(h0), True,
+                                                         offsets=plan.offsets, chunk_offsets=plan.chunk_offsets,
+                                                         seq_order=plan.seq_order, keep=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2) and torch.equal(ht, ht2)
+    assert_close("Aqk", aqk_ref, unpack_triangular_tiles(Aqk).float().cpu(), 5e-3)
 
 
 @pytest.mark.parametrize("K", [64, 128])
