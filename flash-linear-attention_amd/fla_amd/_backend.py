@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -45,7 +45,7 @@ SIGNATURES = {
     "fla_chunk_gla_fwd_fused_first_launch": (c_int, [P] * 13 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_states": (c_int, [P] * 14 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_kept": (c_int, [P] * 16 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
-    "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 14 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 16 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_gdr_fwd_wy": (c_int, [P, P, P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                                  I64, I64, I64, I64, I64, I64, P]),

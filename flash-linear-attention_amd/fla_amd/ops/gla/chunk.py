@@ -213,12 +213,17 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     if head_gates:
         if g.dtype != torch.float32 or g.shape != q.shape[:3]:
             raise ValueError("head gates must be fp32 [B, T, H]")
-        hT = None
+        hT = qg = decay = None
         if states_out is not None:
-            hT = q.new_empty(B, plan.NT if plan is not None else -(-T // BT), H, K, V)
+            nt = plan.NT if plan is not None else -(-T // BT)
+            hT = q.new_empty(B, nt, H, K, V)
             states_out.append(hT)
-        be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), *tail[:5], be.dt(q), *tail[7:]),
-                 "fla_chunk_simple_gla_fwd_fused")
+            if V <= 256:
+                qg = torch.empty_like(q)
+                decay = q.new_empty(B, nt, H, K, dtype=torch.float32)
+                states_out.extend((qg, decay))
+        be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), *tail[:5],
+                                                         be.dt(q), *tail[7:]), "fla_chunk_simple_gla_fwd_fused")
     elif states_out is not None:
         nt = plan.NT if plan is not None else -(-T // BT)
         hT = q.new_empty(B, nt, H, K, V)

@@ -19,7 +19,7 @@ from ..gla.chunk import chunk_gla, chunk_gla_bwd_device, chunk_gla_fwd_fused
 class ChunkSimpleGLAFunction(torch.autograd.Function):
     """Seq-first, K and V in {64, 128}, 16-bit q/k/v: the forward reads the per-head gates as they are
     (``fla_chunk_simple_gla_fwd_fused``, which also keeps the per-chunk states for the backward pass unless
-    recomputation is asked for); only the backward pass, which runs on the GLA kernels, forms the
+    recomputation is asked for, and the gated queries and chunk decays its reverse state scan streams); only the backward pass, which runs on the GLA kernels, forms the
     ``[B,T,H,K]`` gate tensor, and reduces the gate gradient over the key channels
     (the reference: ``fla/ops/simple_gla/chunk.py:134-210``)."""
 
@@ -32,7 +32,7 @@ class ChunkSimpleGLAFunction(torch.autograd.Function):
         flags_states = [] if gla_chunk.KEEP_STATES_FOR_BACKWARD and any(ctx.needs_input_grad) else None
         o, ht, wide = chunk_gla_fwd_fused(q, k, v, gf, scale, h0, output_final_state, offsets=offsets,
                                           return_flags=True, states_out=flags_states, head_gates=True)
-        ctx.save_for_backward(q, k, v, gf, h0, offsets, wide, flags_states[0] if flags_states else None)
+        ctx.save_for_backward(q, k, v, gf, h0, offsets, wide, *(flags_states or ()))
         ctx.scale, ctx.g_dtype = scale, g.dtype
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
         return o, ht
@@ -40,12 +40,14 @@ class ChunkSimpleGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        q, k, v, gf, h0, offsets, wide, hT = ctx.saved_tensors
+        q, k, v, gf, h0, offsets, wide, *kept = ctx.saved_tensors
+        hT = kept[0] if kept else None
+        qg, decay = (kept[1], kept[2]) if len(kept) > 2 else (None, None)
         K = q.shape[-1]
         gk = gf.unsqueeze(-1).expand(*gf.shape, K).contiguous()
         h0f = None if h0 is None else h0.float().contiguous()
         dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, gk, ctx.scale, h0f, do.to(q.dtype).contiguous(), dht,
-                                                   offsets, wide, hT=hT)
+                                                   offsets, wide, hT=hT, qg=qg, decay=decay)
         if dh0 is not None:
             dh0 = dh0.to(ctx.h0_dtype)
         return dq, dk, dv, dg.sum(-1).to(ctx.g_dtype), None, dh0, None, None
