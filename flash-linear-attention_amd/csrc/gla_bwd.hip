@@ -26,6 +26,13 @@
 
 namespace {
 
+// Gate operand of the chunk-parallel kernels: GT is the element type of per-key log-gates [rows, H, K], or
+// HeadGate for one fp32 log-gate per (token, head), [rows, H], which a lane broadcasts over its key channels.
+struct HeadGate {};
+template <typename GT> struct GateOf { typedef GT elem; static constexpr bool per_head = false; };
+template <> struct GateOf<HeadGate> { typedef float elem; static constexpr bool per_head = true; };
+
+
 struct BDhParams {
   const void* q;
   const void* g;
@@ -405,12 +412,14 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dv_kernel(BDvParams p, uint32_
     r.cl = locate_chunk_at32(it, p.offsets, p.indices, p.T, p.NTfix, H, &r.hh);
     return r;
   };
-  typedef GT g4 __attribute__((ext_vector_type(4)));
+  typedef typename GateOf<GT>::elem GE;
+  constexpr bool PER_HEAD = GateOf<GT>::per_head;
+  typedef GE g4 __attribute__((ext_vector_type(4)));
   struct Raw {
     g4 g[RPT];
     v4 q[RPT], k[RPT], d[RPTV];
   };
-  constexpr int GSH = sizeof(GT) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
+  constexpr int GSH = sizeof(GE) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
   const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
   const uint32_t colk = (uint32_t)((tid0 % CG) * 4) * (uint32_t)sizeof(T), colv = (uint32_t)((tid0 % CGV) * 4) * (uint32_t)sizeof(T);
   uint32_t offk[RPT], offv[RPTV];
@@ -423,13 +432,19 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dv_kernel(BDvParams p, uint32_
     const int64_t r0h = im.cl.row0 * H + im.hh;
     const char* qb = (const char*)p.q + r0h * K * (int64_t)sizeof(T);
     const char* kb = (const char*)p.k + r0h * K * (int64_t)sizeof(T);
-    const char* gb = (const char*)p.g + r0h * K * (int64_t)sizeof(GT);
+    const char* gb = (const char*)p.g + r0h * (PER_HEAD ? 1 : K) * (int64_t)sizeof(GE);
     const char* db = (const char*)p.dout + r0h * V * (int64_t)sizeof(T);
     const uint32_t limk = last * pitchk + colk, limv = last * pitchv + colv;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       const uint32_t o = offk[i] < limk ? offk[i] : limk;
-      R.g[i] = *(const g4*)(gb + (o << GSH));
+      if constexpr (PER_HEAD) {
+        const uint32_t row = (uint32_t)((tid0 / CG) * RPT + i);
+        const float x = *(const float*)(gb + (row < last ? row : last) * (uint32_t)H * 4u);
+        R.g[i] = g4{x, x, x, x};
+      } else {
+        R.g[i] = *(const g4*)(gb + (o << GSH));
+      }
       R.q[i] = *(const v4*)(qb + o);
       R.k[i] = *(const v4*)(kb + o);
     }
@@ -642,6 +657,7 @@ struct BDqkgParams {
   void* dq;
   void* dk;
   float* dg;
+  float* dg_head;   // or: fp32 [rows, H], zeroed by the caller, receives the sums of dg over the key channels (dg unused)
   const int64_t* offsets;
   const int64_t* indices;
   int64_t T;
@@ -703,13 +719,15 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
   // its top and arrive behind the dA products, which need do and v only.  All of it at 32-bit offsets from
   // wave-uniform base pointers; rows past the end of a short chunk re-read its last row (masked at use), so no
   // load sits under a branch.
-  typedef GT g4 __attribute__((ext_vector_type(4)));
+  typedef typename GateOf<GT>::elem GE;
+  constexpr bool PER_HEAD = GateOf<GT>::per_head;
+  typedef GE g4 __attribute__((ext_vector_type(4)));
   struct Raw {
     v8 d[NP], v[NP];
   };
   const int rg0 = tid0 >> 4, c40 = (tid0 & 15) * 4;
   const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
-  constexpr int GSH = sizeof(GT) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
+  constexpr int GSH = sizeof(GE) == 4 ? 1 : 0;   // gate bytes = q/k bytes << GSH
   uint32_t offk[4], offv[NP];
 #pragma unroll
   for (int i = 0; i < 4; ++i) offk[i] = (uint32_t)(rg0 * 4 + i) * pitchk + (uint32_t)c40 * (uint32_t)sizeof(T);
@@ -767,12 +785,18 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
     const int64_t r0h = row0 * H + hh;
     const char* qb = (const char*)p.q + (r0h * K + kb) * (int64_t)sizeof(T);
     const char* kb_ = (const char*)p.k + (r0h * K + kb) * (int64_t)sizeof(T);
-    const char* gb = (const char*)p.g + (r0h * K + kb) * (int64_t)sizeof(GT);
+    const char* gb = PER_HEAD ? (const char*)p.g + r0h * 4 : (const char*)p.g + (r0h * K + kb) * (int64_t)sizeof(GE);
     const uint32_t limk = (uint32_t)(L - 1) * pitchk + colk;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t o = offk[i] < limk ? offk[i] : limk;
-      cg[i] = *(const g4*)(gb + (o << GSH));
+      if constexpr (PER_HEAD) {
+        const uint32_t row = (uint32_t)(rg0 * 4 + i), last = (uint32_t)(L - 1);
+        const float x = *(const float*)(gb + (row < last ? row : last) * (uint32_t)H * 4u);
+        cg[i] = g4{x, x, x, x};
+      } else {
+        cg[i] = *(const g4*)(gb + (o << GSH));
+      }
       cq[i] = *(const v4*)(qb + o);
       ck[i] = *(const v4*)(kb_ + o);
     }
@@ -987,8 +1011,13 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     int row = rg * 4 + i;
-    if (row < L) {
-      f32x4 o = {x[i][0] + add[0], x[i][1] + add[1], x[i][2] + add[2], x[i][3] + add[3]};
+    f32x4 o = {x[i][0] + add[0], x[i][1] + add[1], x[i][2] + add[2], x[i][3] + add[3]};
+    if (p.dg_head) {
+      // one gate per (token, head): the sum over this slice's 64 key channels, which sit in the 16 lanes of a DPP
+      // row; the slices of a head (and the exact kernel, a launch later) add up in a fixed order
+      const float tot = row_prefix16((o[0] + o[1]) + (o[2] + o[3]));
+      if ((tid & 15) == 15 && row < L) atomicAdd(p.dg_head + (row0 + row) * H + hh, tot);
+    } else if (row < L) {
       *(f32x4*)(p.dg + ((row0 + row) * H + hh) * (int64_t)K + kb + c4) = o;
     }
   }
@@ -1021,6 +1050,7 @@ struct BExactParams {
   void* dk;
   void* dv;
   float* dg;
+  float* dg_head;
   const int64_t* offsets;
   const int64_t* indices;
   int64_t T;
@@ -1070,7 +1100,11 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
     v4 qv = {(T)0.f, (T)0.f, (T)0.f, (T)0.f}, kv = qv;
     if (row < L) {
       int64_t off = baseK + row * strideK + c4;
-      Load<GT>::x4((const GT*)p.g + off, gv);
+      if constexpr (GateOf<GT>::per_head) {
+        gv[0] = gv[1] = gv[2] = gv[3] = ((const float*)p.g)[(row0 + row) * H + hh];
+      } else {
+        Load<GT>::x4((const GT*)p.g + off, gv);
+      }
       qv = *(const v4*)((const T*)p.q + off);
       kv = *(const v4*)((const T*)p.k + off);
     }
@@ -1174,7 +1208,17 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
     float run = 0.f;
     for (int t = L - 1; t >= 0; --t) {
       run += sX[t * LDG + c];
-      p.dg[baseK + t * strideK + c] += run;
+      if (p.dg_head) sX[t * LDG + c] = run;
+      else p.dg[baseK + t * strideK + c] += run;
+    }
+  }
+  if (p.dg_head) {
+    // one gate per (token, head): a row's channels are summed in a fixed order, one addition per row
+    __syncthreads();
+    for (int t = tid; t < L; t += 256) {
+      float sum = 0.f;
+      for (int c = 0; c < K; ++c) sum += sX[t * LDG + c];
+      atomicAdd(p.dg_head + (cl.row0 + t) * H + hh, sum);
     }
   }
   }
@@ -1183,7 +1227,7 @@ __global__ __launch_bounds__(256) void gla_bwd_intra_exact_kernel(BExactParams p
 template <typename T, typename GT>
 int launch_bwd(const void* q, const void* k, const void* v, const void* g, const void* dout, const float* dht,
                const void* hT, const void* qg, const float* decay, void* dhtf, void* dq, void* dk, void* dv, float* dg,
-               float* dh0, const int* wide,
+               float* dg_head, float* dh0, const int* wide,
                const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
                int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
   dim3 grid;
@@ -1198,6 +1242,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     int64_t total = (K / 64) * (V / 64) * N * H;
     FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
     if (qg) hipLaunchKernelGGL((gla_bwd_dh_qg_kernel<T>), dim3((unsigned)total), dim3(256), 0, st, p);
+    else if constexpr (GateOf<GT>::per_head) return FLA_E_INVALID;   // per-head gates come with kept gated queries
     else hipLaunchKernelGGL((gla_bwd_dh_kernel<T, GT>), dim3((unsigned)total), dim3(256), 0, st, p);
     FLA_CHECK_LAUNCH();
   }
@@ -1217,7 +1262,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   {
-    BDqkgParams p{q, k, v, g, dout, hT, dhtf, wide, dq, dk, dg, offsets, indices, T_, total_chunks,
+    BDqkgParams p{q, k, v, g, dout, hT, dhtf, wide, dq, dk, dg, dg_head, offsets, indices, T_, total_chunks,
                   (int)H, (int)K, ntfix, scale};
     // as many workgroups as are resident at once (two per CU), each walking its share of the items
     const int64_t pairs = (int64_t)grid.x * grid.y, nwg = pairs * (K / 64);
@@ -1229,7 +1274,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     FLA_CHECK_LAUNCH();
   }
   if (wide) {
-    BExactParams p{q, k, v, g, dout, wide, dq, dk, dv, dg, offsets, indices, T_, (int)H, ntfix, scale,
+    BExactParams p{q, k, v, g, dout, wide, dq, dk, dv, dg, dg_head, offsets, indices, T_, (int)H, ntfix, scale,
                    (int64_t)grid.x * grid.y};
     const dim3 gx((unsigned)(p.total < 512 ? p.total : 512));
 #define FLA_CASE(KK, VV)                                                                                      \
@@ -1245,26 +1290,31 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
 
 static int gla_bwd_impl(const void* q, const void* k, const void* v, const void* gates, const void* dout,
                         const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
-                        void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                        void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dg_head, float* dh0,
+                        const int* wide,
                         const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                         int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
-                        int64_t N, float scale, fla_stream_t stream) {
-  FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag_t && dq && dk && dv && dg,
+                        int64_t N, float scale, fla_stream_t stream, bool head_gates = false) {
+  FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag_t && dq && dk && dv && (dg || dg_head),
               FLA_E_INVALID);
+  if (head_gates) FLA_REQUIRE(q_gated && dg_head, FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
   else FLA_REQUIRE(N == B, FLA_E_INVALID);
   FLA_REQUIRE((q_gated == nullptr) == (chunk_decay == nullptr), FLA_E_INVALID);
   if (q_gated) FLA_REQUIRE(scale != 0.f, FLA_E_INVALID);
-  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)gates | (uintptr_t)dout | (uintptr_t)hT |
-               (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
+  FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (head_gates ? 0 : (uintptr_t)gates) | (uintptr_t)dout |
+               (uintptr_t)hT | (uintptr_t)dh_frag_t | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv |
                (uintptr_t)dg | (uintptr_t)q_gated) % 16 == 0,
               FLA_E_ALIGNMENT);
   hipStream_t st = (hipStream_t)stream;
 #define FLA_BWD(TT, GG)                                                                                           \
-  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dh0, wide,   \
+  return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dg_head, dh0, wide,   \
                             offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
+  if (head_gates && qkv_dtype == FLA_BF16) FLA_BWD(bf16, HeadGate);
+  if (head_gates && qkv_dtype == FLA_F16) FLA_BWD(f16, HeadGate);
+  if (head_gates) return FLA_E_UNSUPPORTED;
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_F32) FLA_BWD(bf16, float);
   if (qkv_dtype == FLA_BF16 && gate_dtype == FLA_BF16) FLA_BWD(bf16, bf16);
   if (qkv_dtype == FLA_F16 && gate_dtype == FLA_F32) FLA_BWD(f16, float);
@@ -1280,7 +1330,7 @@ extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, co
                                  int64_t NT, int qkv_dtype,
                                  int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                  float scale, fla_stream_t stream) {
-  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, nullptr, nullptr, dh_frag_t, dq, dk, dv, dg, dh0, wide, offsets,
+  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, nullptr, nullptr, dh_frag_t, dq, dk, dv, dg, nullptr, dh0, wide, offsets,
                       indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
 }
 
@@ -1292,6 +1342,18 @@ extern "C" int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* 
                                       int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                                       int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q_gated && chunk_decay, FLA_E_INVALID);
-  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dh0, wide,
+  return gla_bwd_impl(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, nullptr, dh0, wide,
                       offsets, indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+}
+
+extern "C" int fla_chunk_simple_gla_bwd(const void* q, const void* k, const void* v, const float* g, const void* dout,
+                                        const float* dht, const void* hT, const void* q_gated,
+                                        const float* chunk_decay, void* dh_frag_t, void* dq, void* dk, void* dv,
+                                        float* dg, float* dh0, const int* wide, const int64_t* offsets,
+                                        const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                                        int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                        int64_t N, float scale, fla_stream_t stream) {
+  FLA_REQUIRE(q_gated && chunk_decay && dg, FLA_E_INVALID);
+  return gla_bwd_impl(q, k, v, g, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, nullptr, dg, dh0, wide,
+                      offsets, indices, chunk_offsets, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true);
 }

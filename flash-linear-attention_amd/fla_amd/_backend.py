@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -55,6 +55,7 @@ SIGNATURES = {
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 17 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_kept": (c_int, [P] * 19 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_bwd": (c_int, [P] * 19 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_o_gk": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_dA": (c_int, [P] * 5 + [I64, I, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_dv": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, P]),

@@ -329,14 +329,16 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
 
 
 def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None, hT=None, qg=None,
-                         decay=None):
+                         decay=None, head_gates=False):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
     Returns ``(dq, dk, dv, dg, dh0)``; without ``hT`` (the states a forward pass kept) it
     recomputes the per-chunk states as the reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``qg``, ``decay``:
     the gated queries and chunk decays of ``fla_chunk_gla_fwd_fused_kept``, if the forward kept them.  ``wide``: the forward's
     gate-range flags (int32 ``[chunks, H]``); flagged chunks get their intra-chunk terms
     from the exact kernel.  Without it the result is exact only while the chunk-cumulative
-    log-gate stays within +-80."""
+    log-gate stays within +-80.  ``head_gates``: ``g`` is one fp32 log-gate per (token, head), ``[B, T, H]``, and
+    ``dg`` comes back in that shape (``fla_chunk_simple_gla_bwd`` when the forward kept its gated queries; otherwise
+    the gates are broadcast over the key channels and the per-key gradient is summed afterwards)."""
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
@@ -345,23 +347,36 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     V = v.shape[-1]
     N = B if plan is None else plan.N
     NT = 0 if plan is None else plan.NT
+    kept = qg is not None and decay is not None and float(scale) != 0.0 and hT is not None
+    g_head = None
+    if head_gates and not kept:
+        g_head, g = g, g.unsqueeze(-1).expand(*g.shape, K).contiguous()
     if hT is None:
         hT, _ = chunk_fwd_h(k=k, v=v, g=None, gk=g, gv=None, h0=initial_state, output_final_state=False,
                             offsets=offs, indices=idx, head_first=False, chunk_size=BT, gates_are_cumsum=False,
                             fragment_layout=True, transposed_fragments=True, chunk_offsets=co)
     dhtf = torch.empty_like(hT)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    dg = q.new_empty(B, T, H, K, dtype=torch.float32)
+    if kept and head_gates:
+        dg = q.new_zeros(B, T, H, dtype=torch.float32)   # the kernels add their slices' sums to it
+    else:
+        dg = q.new_empty(B, T, H, K, dtype=torch.float32)
     dh0 = q.new_empty(N, H, K, V, dtype=torch.float32) if initial_state is not None else None
     if dht is not None:
         dht = (dht if dht.dtype == torch.float32 else dht.float()).contiguous()
-    tail = (be.ptr(dhtf), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg), be.ptr(dh0), be.ptr(wide), be.ptr(offs),
+    tail = (be.ptr(dh0), be.ptr(wide), be.ptr(offs),
             be.ptr(idx), be.ptr(co), NT, be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q))
+    outs = (be.ptr(dhtf), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg))
     head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT))
-    if qg is not None and decay is not None and float(scale) != 0.0:
-        be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), *tail), "fla_chunk_gla_bwd_kept")
+    if kept and head_gates:
+        be.check(be.lib().fla_chunk_simple_gla_bwd(*head, be.ptr(qg), be.ptr(decay), *outs, *tail[:7], *tail[8:]),
+                 "fla_chunk_simple_gla_bwd")
+    elif kept:
+        be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), *outs, *tail), "fla_chunk_gla_bwd_kept")
     else:
-        be.check(be.lib().fla_chunk_gla_bwd(*head, *tail), "fla_chunk_gla_bwd")
+        be.check(be.lib().fla_chunk_gla_bwd(*head, *outs, *tail), "fla_chunk_gla_bwd")
+    if g_head is not None:
+        dg = dg.sum(-1)
     return dq, dk, dv, dg, dh0
 
 

@@ -19,8 +19,10 @@ from ..gla.chunk import chunk_gla, chunk_gla_bwd_device, chunk_gla_fwd_fused
 class ChunkSimpleGLAFunction(torch.autograd.Function):
     """Seq-first, K and V in {64, 128}, 16-bit q/k/v: the forward reads the per-head gates as they are
     (``fla_chunk_simple_gla_fwd_fused``, which also keeps the per-chunk states for the backward pass unless
-    recomputation is asked for, and the gated queries and chunk decays its reverse state scan streams); only the backward pass, which runs on the GLA kernels, forms the
-    ``[B,T,H,K]`` gate tensor, and reduces the gate gradient over the key channels
+    recomputation is asked for, and the gated queries and chunk decays its reverse state scan streams); the backward
+    pass runs on the GLA kernels' per-head-gate instantiations (``fla_chunk_simple_gla_bwd``) - only when it
+    recomputes the states does it form the ``[B,T,H,K]`` gate tensor and reduce the gate gradient over the key
+    channels afterwards
     (the reference: ``fla/ops/simple_gla/chunk.py:134-210``)."""
 
     @staticmethod
@@ -43,14 +45,12 @@ class ChunkSimpleGLAFunction(torch.autograd.Function):
         q, k, v, gf, h0, offsets, wide, *kept = ctx.saved_tensors
         hT = kept[0] if kept else None
         qg, decay = (kept[1], kept[2]) if len(kept) > 2 else (None, None)
-        K = q.shape[-1]
-        gk = gf.unsqueeze(-1).expand(*gf.shape, K).contiguous()
         h0f = None if h0 is None else h0.float().contiguous()
-        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, gk, ctx.scale, h0f, do.to(q.dtype).contiguous(), dht,
-                                                   offsets, wide, hT=hT, qg=qg, decay=decay)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, gf, ctx.scale, h0f, do.to(q.dtype).contiguous(), dht,
+                                                   offsets, wide, hT=hT, qg=qg, decay=decay, head_gates=True)
         if dh0 is not None:
             dh0 = dh0.to(ctx.h0_dtype)
-        return dq, dk, dv, dg.sum(-1).to(ctx.g_dtype), None, dh0, None, None
+        return dq, dk, dv, dg.to(ctx.g_dtype), None, dh0, None, None
 
 
 def chunk_simple_gla(

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 8
+#define FLA_ABI_VERSION 9
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -373,6 +373,19 @@ int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const vo
                            const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                            int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                            int64_t N, float scale, fla_stream_t stream);
+
+/* The backward of chunk_simple_gla (fla/ops/simple_gla/chunk.py:134-210: chunk_bwd_dh, chunk_bwd_dqkwg,
+ * chunk_bwd_dv with one gate per (token, head)) on the same three launches: g fp32 [B,T,H] is read as it is (a lane
+ * broadcasts its row's gate over its key channels) and dg, fp32 [B,T,H], which the caller zeroes, receives the
+ * gate gradient summed over the key channels (each 64-channel slice of a head adds its share; the additions of
+ * one entry happen in a fixed order).  hT, q_gated and chunk_decay as fla_chunk_simple_gla_fwd_fused left them;
+ * everything else as for fla_chunk_gla_bwd_kept. */
+int fla_chunk_simple_gla_bwd(const void* q, const void* k, const void* v, const float* g, const void* dout,
+                             const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
+                             void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                             const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
+                             int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                             float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * The chunk-parallel stages of GLA under the operand layouts of the reference's internal

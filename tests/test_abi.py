@@ -63,6 +63,10 @@ def test_argument_validation_without_device():
     bwd = lambda qg, dec, scale: lib.fla_chunk_gla_bwd_kept(p, p, p, p, p, None, p, qg, dec, p, p, p, p, p, None, None,
                                                             None, None, None, 0, 0, 2, 1, 64, 1, 64, 64, 1, scale, None)
     assert bwd(p, None, 1.0) == -1 and bwd(p, p, 0.0) == -1
+    # the per-head-gate backward needs the kept gated queries and a gate-gradient buffer
+    sgb = lambda qg, dg: lib.fla_chunk_simple_gla_bwd(p, p, p, p, p, None, p, qg, p, p, p, p, p, dg, None, None, None, None,
+                                                      None, 0, 2, 1, 64, 1, 64, 64, 1, 1.0, None)
+    assert sgb(None, p) == -1 and sgb(p, None) == -1
     # the delta rule's chunk-parallel launch: w and Aw together or not at all, K in {64, 128}
     prep = lambda w, Aw, K: lib.fla_gdr_fwd_prep(p, p, None, 0, None, p, w, Aw, None, None, 0, 0, 1, 64, 1, K, None)
     assert prep(p, None, 64) == -1 and prep(None, p, 64) == -1

@@ -305,3 +305,51 @@ def test_chunk_simple_gla_per_head_gate_kernel_fp16_and_gradients(device):
     for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
         assert_close(name, a.grad, b.grad, TOL_G)
     assert_close("dh0", rh0.grad, h0l.grad, TOL_G)
+
+
+@pytest.mark.parametrize("varlen", [False, True])
+def test_chunk_simple_gla_strong_gates_backward_reproducible(device, varlen, monkeypatch):
+    """Gates strong enough that chunks leave the single-reference range (their intra-chunk terms come from the
+    exact kernel): the per-head gate gradient, which the backward kernels accumulate from their key slices, is
+    the same bit for bit on a second run, agrees with the form that writes per-key gradients and sums them
+    afterwards (the backward that recomputes the states), and both meet the fp32 recurrence."""
+    import fla_amd.ops.gla.chunk as gla_mod
+    from fla_amd.ops.simple_gla import chunk_simple_gla
+    from oracle.recurrent import naive_recurrent_gla
+    N, H, K, V, T = 3, 2, 128, 128, 333
+    B = 1 if varlen else 2
+    gen = torch.Generator().manual_seed(91)
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    q = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    g = -2.5 * torch.rand(B, T, H, generator=gen)       # about -80 per chunk: most chunks are flagged
+    h0 = torch.randn(N if varlen else B, H, K, V, generator=gen) * 0.1
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(h0.shape, generator=gen) * 0.1
+    dev = _dev(device)
+    print(f"chunk_simple_gla strong gates varlen={varlen}", flush=True)
+
+    def run():
+        leaves = [dev(x).detach().requires_grad_() for x in (q, k, v, g)]
+        h0l = dev(h0).detach().requires_grad_()
+        o, ht = chunk_simple_gla(*leaves, initial_state=h0l, output_final_state=True, cu_seqlens=dev(offs),
+                                 head_first=False)
+        torch.autograd.backward((o, ht), (dev(do), dev(dht)))
+        torch.cuda.synchronize()
+        return [x.grad for x in leaves] + [h0l.grad]
+
+    first, second = run(), run()
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    monkeypatch.setattr(gla_mod, "KEEP_STATES_FOR_BACKWARD", False)
+    rec = run()
+    rl = [x.detach().float().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.detach().float().requires_grad_()
+    ro, rht = naive_recurrent_gla(rl[0], rl[1], rl[2], None, g=rl[3], initial_state=rh0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    ((ro * do.float()).sum() + (rht * dht).sum()).backward()
+    refs = [x.grad for x in rl] + [rh0.grad]
+    for name, r, a, b, tol in zip(("dq", "dk", "dv", "dg", "dh0"), refs, first, rec, (TOL_G, TOL_G, TOL_G, 4e-2, TOL_G)):
+        assert_close(f"{name} (kept)", r, a, tol)
+        assert_close(f"{name} (recomputed)", r, b, tol)
