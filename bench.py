@@ -521,7 +521,7 @@ def bench_simple_gla(device, steps=20):
                                                    head_first=False), steps)
         us_b = event_avg_us(lambda: chunk_gla(q, k, v, g[..., None].expand(B, T, H, D), initial_state=h0,
                                               output_final_state=True, head_first=False), steps)
-    # forward + backward at config 4's batch (B=4): per-head-gate forward that keeps the states, GLA backward kernels
+    # forward + backward at config 4's batch (B=4): per-head-gate forward that keeps the states, per-head-gate backward
     Bb = 4
     leaves = [x[:Bb].clone().requires_grad_() for x in (q, k, v, g)]
     h0b = h0[:Bb].clone().requires_grad_()
