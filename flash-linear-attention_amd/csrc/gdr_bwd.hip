@@ -960,14 +960,23 @@ struct TileIO {
   typedef typename Elem<T>::v4 v4;
   static constexpr int CG = DIM / 4, RG = 256 / CG, RPT = BT / RG;
   typedef T tvec __attribute__((ext_vector_type(RPT)));
+  // Unconditional: rows past the end of a short chunk re-read its last row (a load under a branch makes the
+  // compiler wait for it, and for everything issued before it, at the join); zero_tail() clears them before use.
   static FLA_DEVICE void load(const void* src, int64_t row0, int L, int H, int hh, int tid, v4* reg) {
     const int rg = tid / CG, c4 = (tid % CG) * 4;
-    const T* p = (const T*)src + (row0 * H + hh) * (int64_t)DIM + c4;
+    const char* p = (const char*)((const T*)src + (row0 * H + hh) * (int64_t)DIM + c4);
+    const uint32_t pitch = (uint32_t)H * DIM * (uint32_t)sizeof(T), lim = (uint32_t)(L - 1) * pitch;
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
-      int row = rg * RPT + i;
-      reg[i] = row < L ? *(const v4*)(p + (int64_t)row * H * DIM) : v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      const uint32_t o = (uint32_t)(rg * RPT + i) * pitch;
+      reg[i] = *(const v4*)(p + (o < lim ? o : lim));
     }
+  }
+  static FLA_DEVICE void zero_tail(int L, int tid, v4* reg) {
+    const int rg = tid / CG;
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+      if (rg * RPT + i >= L) reg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
   }
   static FLA_DEVICE void put_rows(T* dst, int ld, int tid, const v4* reg) {
     const int rg = tid / CG, c4 = (tid % CG) * 4;
@@ -1060,7 +1069,8 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
     for (int i = 0; i < IOA::RPT; ++i) R.a[i] = *(const v4*)(ab + (offa[i] < lima ? offa[i] : lima));
     const uint32_t row = (uint32_t)(tid0 & (BT - 1)) < last ? (uint32_t)(tid0 & (BT - 1)) : last;
     R.beta = p.beta[(im.cl.row0 + row) * H + im.hh];
-    R.gam = p.gam ? p.gam[(im.cl.row0 + row) * H + im.hh] : 0.f;
+    // without gates the load reads one zero word (no branch round a load)
+    R.gam = *(p.gam ? p.gam + (im.cl.row0 + row) * H + im.hh : &kZeroWord);
   };
   uint32_t it = blockIdx.x;
   if (it >= nitems) return;
@@ -1183,6 +1193,8 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
   }
   __syncthreads();  // the value tiles and Au^T are consumed
   // ================= key side: d(kb)_1 = Aw^T dw ; dAw_1 = (dw k^T) diag(beta)
+  IOK::zero_tail(L, tid, rdw);
+  IOK::zero_tail(L, tid, rk);
   IOK::put_rows(sRow1, LDD, tid, rdw);
   IOK::put_tr(sTr1, tid, rdw);
   IOK::put_rows(sRow2, LDD, tid, rk);
