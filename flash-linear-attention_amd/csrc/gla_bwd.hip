@@ -7,6 +7,8 @@
 //   gla_bwd_dh_kernel    reverse state scan:  store dH_c;  dH <- diag(e^{G_last}) dH + q~^T do.
 //                        The tile is kept and stored transposed ([V,K], MFMA-fragment order), the
 //                        orientation dk contracts it in; also emits dh0.
+//   gla_bwd_dh_qg_kernel the same scan on the gated queries q e^{G} and the chunk decays e^{G_last} a
+//                        states-keeping forward left: no prefix sums, no exponentials, 16-byte row pieces.
 //   gla_bwd_dv_kernel    per (chunk, head):  dv = A^T do + k^ dH_c.  dv contracts dH over K: the
 //                        stored [V,K] fragments are turned round on the matrix pipe (a product with a
 //                        permuted identity is a transposition of the accumulator layout, exact for
@@ -20,6 +22,9 @@
 //                        (fla/ops/gla/chunk.py:409-567 intra, :726-837 inter incl. the dg formula
 //                        :818-823).  As in the forward, one reference point per chunk replaces
 //                        the 16x16 sub-block scheme.
+// The chunk-parallel kernels also exist for one gate per (token, head) (chunk_simple_gla's backward,
+// fla/ops/simple_gla/chunk.py:134-210): the gate word of a row is broadcast over the lane's key channels and dg
+// leaves as its sum over the key channels.
 #include <type_traits>
 
 #include "chunk_common.h"
@@ -31,7 +36,6 @@ namespace {
 struct HeadGate {};
 template <typename GT> struct GateOf { typedef GT elem; static constexpr bool per_head = false; };
 template <> struct GateOf<HeadGate> { typedef float elem; static constexpr bool per_head = true; };
-
 
 struct BDhParams {
   const void* q;
