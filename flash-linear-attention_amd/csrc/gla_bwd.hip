@@ -192,6 +192,291 @@ __global__ __launch_bounds__(256) void gla_bwd_dh_qg_kernel(BDhParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Reverse state scan and dv in one pass, from what a states-keeping forward left: the gated queries q e^{G}, the
+// chunk decays e^{G_last}, k^ = k e^{G_last-G} (key-major tiles) and the causal score tile P = tril(q~ k~^T):
+//   dv_c = s P_c^T do_c + k^_c dH_c          dH_{c-1} = e^{G_last} dH_c + s (q e^{G})_c^T do_c
+// (fla/ops/gla/chunk.py:1037-1061 with fla/ops/common/chunk_h.py:338-402).  dH never comes back from memory for dv,
+// and neither q, k nor the gates are read.  One workgroup of eight waves per (sequence, head, 32 value columns):
+// waves 4-7 ("staging") load the next chunk's tiles, write them to LDS and store dv; waves 0-3 ("matrix") carry
+// dH / s in accumulators (both orientations: the fragment-order copy for the dq/dk launch is the transposed one)
+// and do the products.  Per chunk c (walking backwards) the groups meet twice:
+//   B1(c)  k^, P, do of chunk c and the 16-bit dH_c are in LDS
+//          matrix:  dv = s P^T do + k^ dH -> LDS (transposed)           staging: q e^{G}, decay, do of chunk c -> LDS
+//   B2(c)  matrix:  dH <- decay * dH + (q e^{G})^T do; publishes dH     staging: dv of chunk c -> memory; chunk c-1 -> LDS
+// Chunks whose cumulative log-gate left the single-reference range (flagged) get their intra-chunk term from the exact
+// kernel: P is skipped for them (k^ and q e^{G} are exact for any gate).
+struct BDhvParams {
+  const void* qg;       // [rows, H, K]
+  const void* kh_t;     // [chunks, H, K, 64]
+  const void* scores;   // [chunks, H, 64, 64]
+  const float* decay;   // [chunks, H, K]
+  const void* dout;     // [rows, H, V]
+  const float* dht;     // [N, H, K, V] or null
+  const int* wide;      // [chunks, H] or null
+  void* dhtf;           // out: dH, FLA_H_FRAGMENT_T
+  void* dv;             // out: [rows, H, V]
+  float* dh0;           // out: [N, H, K, V] or null
+  const int64_t* offsets;
+  const int64_t* chunk_offsets;
+  int64_t T;
+  int H, V, N;
+  float scale;
+};
+
+template <typename T, int K>
+__global__ __launch_bounds__(512) void gla_bwd_dhv_kernel(BDhvParams p) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int BV = 32;
+  constexpr int LDK = K + 8;
+  constexpr int LDV = BV + 8;
+  constexpr int C8 = K / 8, NP = BT * C8 / 256;   // q e^{G}: 16-byte pieces per row / per staging lane
+  constexpr int PR = 256 / C8;                    // rows between two pieces of a lane
+  constexpr int NKH = K * (BT / 8) / 256;         // k^ tile: pieces per staging lane (the tile is contiguous in memory)
+  constexpr int NPP = BT * (BT / 8) / 256;        // score tile: pieces per staging lane
+  constexpr int KT32 = K / 32;
+  static_assert(KT32 <= 4, "one 32-row block of the state per matrix wave");
+  __shared__ __attribute__((aligned(16))) T sKh[K * LDT];      // k^, key-major [k][t]
+  __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];      // q e^{G}, row-major [t][k]
+  __shared__ __attribute__((aligned(16))) T sP[BT * LDT];      // P [i][j]
+  __shared__ __attribute__((aligned(16))) T sDoY[BT * LDV];    // do [t][v], for the dv products
+  __shared__ __attribute__((aligned(16))) T sDoX[BT * LDV];    // do [t][v], for the update
+  __shared__ __attribute__((aligned(16))) T sDHt[BV * LDK];    // dH^T in 16-bit [v][k]
+  __shared__ __attribute__((aligned(16))) T sDvT[BV * LDT];    // dv^T [v][t]
+  __shared__ __attribute__((aligned(16))) float sDec[K];       // e^{G_last} of the chunk being folded in
+  __shared__ int sFlag;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int H = p.H, V = p.V;
+  const int nvt = V / BV;
+  int64_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int vt = (int)(id % nvt);
+  const int nh = (int)(id / nvt);
+  const int n = nh / H, hh = nh % H;
+  const int vbase = vt * BV;
+  SeqSpan sp = seq_span(p.offsets, n, p.T);
+  const int64_t nchunks = (sp.len + BT - 1) / BT;
+  const int64_t chunk0 = p.chunk_offsets ? p.chunk_offsets[n] : (int64_t)n * ((p.T + BT - 1) / BT);
+  auto chunk_len = [&](int64_t c) {
+    int64_t rem = sp.len - c * BT;
+    return (int)(rem < BT ? rem : BT);
+  };
+  // An empty sequence hands d ht through to d h0 bit for bit: no factor goes on and off it.
+  const float scale = nchunks > 0 ? p.scale : 1.f, inv_scale = 1.f / scale;
+
+  if (wave >= 4) {
+    // =========================== staging waves ===========================
+    if (nchunks == 0) return;
+    const int st = tid - 256;
+    const int prow = st / C8, c8 = (st % C8) * 8;   // q e^{G}: piece i of a lane is row prow + PR i, columns c8 ..
+    const int vrow = st >> 2, vc8 = (st & 3) * 8;   // do, dv: one row, 8 of the 32 columns
+    struct XRegs {
+      v8 q[NP];
+      float dec;
+    };
+    struct YRegs {
+      v8 kh[NKH];
+      v8 pp[NPP];
+      v8 d;
+      int flag;
+    };
+    // Every load is unconditional: rows past the end of a short chunk are redirected to its last row (their do rows
+    // are zeroed where they are staged), chunks before the first one to chunk 0.
+    const uint32_t pitchK = (uint32_t)H * K * (uint32_t)sizeof(T), pitchV = (uint32_t)H * V * (uint32_t)sizeof(T);
+    uint32_t offk[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) offk[i] = (uint32_t)(prow + PR * i) * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+    const uint32_t offv = (uint32_t)vrow * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+    const char* gq = (const char*)p.qg + (sp.bos * H + hh) * (int64_t)K * (int64_t)sizeof(T);
+    const char* gd = (const char*)p.dout + ((sp.bos * H + hh) * (int64_t)V + vbase) * (int64_t)sizeof(T);
+    const char* gk = (const char*)p.kh_t + (chunk0 * H + hh) * (int64_t)K * BT * (int64_t)sizeof(T) + 16 * st;
+    const char* gp = (const char*)p.scores + (chunk0 * H + hh) * (int64_t)BT * BT * (int64_t)sizeof(T) + 16 * st;
+    const float* gdec = p.decay + (chunk0 * H + hh) * (int64_t)K + (st & (K - 1));
+    const int* gf = p.wide ? p.wide + chunk0 * H + hh : (const int*)&kZeroWord;
+    const int64_t strKh = (int64_t)H * K * BT * (int64_t)sizeof(T), strP = (int64_t)H * BT * BT * (int64_t)sizeof(T);
+    auto load_x = [&](int64_t c, XRegs& R) __attribute__((always_inline)) {
+      c = c < 0 ? 0 : c;
+      const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+      const int64_t ck = c * BT * (int64_t)pitchK;
+      const uint32_t lk = last * pitchK + (uint32_t)c8 * (uint32_t)sizeof(T);
+#pragma unroll
+      for (int i = 0; i < NP; ++i) R.q[i] = *(const v8*)(gq + ck + (offk[i] < lk ? offk[i] : lk));
+      R.dec = gdec[c * (int64_t)H * K];
+    };
+    auto load_y = [&](int64_t c, YRegs& R) __attribute__((always_inline)) {
+      c = c < 0 ? 0 : c;
+      const uint32_t last = (uint32_t)(chunk_len(c) - 1);
+#pragma unroll
+      for (int i = 0; i < NKH; ++i) R.kh[i] = *(const v8*)(gk + c * strKh + 4096 * i);
+#pragma unroll
+      for (int i = 0; i < NPP; ++i) R.pp[i] = *(const v8*)(gp + c * strP + 4096 * i);
+      const uint32_t lv = last * pitchV + (uint32_t)vc8 * (uint32_t)sizeof(T);
+      R.d = *(const v8*)(gd + c * BT * (int64_t)pitchV + (offv < lv ? offv : lv));
+      R.flag = gf[p.wide ? c * H : 0];
+    };
+    v8 dkeep;   // this lane's do piece of the chunk last staged as Y (zero past the end of the chunk)
+    auto stage_x = [&](const XRegs& R) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < NP; ++i) *(v8*)&sQ[(prow + PR * i) * LDK + c8] = R.q[i];
+      *(v8*)&sDoX[vrow * LDV + vc8] = dkeep;
+      if (st < K) sDec[st] = R.dec;
+    };
+    auto stage_y = [&](const YRegs& R, int64_t c) __attribute__((always_inline)) {
+      const int L = chunk_len(c);
+#pragma unroll
+      for (int i = 0; i < NKH; ++i) {
+        const int e = st + 256 * i;
+        *(v8*)&sKh[(e >> 3) * LDT + (e & 7) * 8] = R.kh[i];
+      }
+#pragma unroll
+      for (int i = 0; i < NPP; ++i) {
+        const int e = st + 256 * i;
+        *(v8*)&sP[(e >> 3) * LDT + (e & 7) * 8] = R.pp[i];
+      }
+      const v8 z8 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      dkeep = vrow < L ? R.d : z8;
+      *(v8*)&sDoY[vrow * LDV + vc8] = dkeep;
+      if (st == 0) sFlag = R.flag;
+    };
+    // dv of chunk c leaves as whole rows, 16 bytes per lane: a 16-lane group turns a block of 8 value columns x
+    // 16 time rows of the transposed tile round with two transposing LDS loads.  Only a sequence's last chunk (the
+    // first one processed) can be short: it takes the variant with the masked store.
+    const int dgrp = st >> 4, dtb = dgrp >> 2, dvb = dgrp & 3, dj = st & 15;
+    const int dsrc = (8 * dvb + (dj >> 2)) * LDT + 16 * dtb + 4 * (dj & 3);
+    auto store_dv = [&](int64_t c, auto maybe_short) __attribute__((always_inline)) {
+      typedef short s4 __attribute__((ext_vector_type(4)));
+      typedef __attribute__((address_space(3))) s4 lds_s4;
+      s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sDvT[dsrc]);
+      s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4*)&sDvT[dsrc + 4 * LDT]);
+      const v8 x = __builtin_shufflevector(__builtin_bit_cast(v4, lo), __builtin_bit_cast(v4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+      const int row = 16 * dtb + dj;
+      T* dst = (T*)p.dv + ((sp.bos + c * BT + row) * H + hh) * (int64_t)V + vbase + 8 * dvb;
+      if constexpr (decltype(maybe_short)::value) {
+        if (row < chunk_len(c)) *(v8*)dst = x;
+      } else {
+        *(v8*)dst = x;
+      }
+    };
+    XRegs X;
+    YRegs Y;
+    load_x(nchunks - 1, X);
+    load_y(nchunks - 1, Y);
+    stage_y(Y, nchunks - 1);
+    load_y(nchunks - 2, Y);
+    if (nchunks > 1) {
+      lds_barrier();  // B1(nchunks - 1)
+      stage_x(X);
+      load_x(nchunks - 2, X);
+      lds_barrier();  // B2(nchunks - 1)
+      store_dv(nchunks - 1, std::true_type{});
+      stage_y(Y, nchunks - 2);
+      load_y(nchunks - 3, Y);
+      for (int64_t c = nchunks - 2; c >= 1; --c) {
+        lds_barrier();  // B1(c)
+        stage_x(X);
+        load_x(c - 1, X);
+        lds_barrier();  // B2(c)
+        store_dv(c, std::false_type{});
+        stage_y(Y, c - 1);
+        load_y(c - 2, Y);
+      }
+    }
+    lds_barrier();  // B1(0)
+    stage_x(X);
+    lds_barrier();  // B2(0)
+    store_dv(0, std::true_type{});
+  } else {
+    // =========================== matrix waves ===========================
+    const int kt = wave;   // this wave's 32 key rows of the state gradient
+    f32x16 acc = zero16(), acct = zero16();   // dH / s: rows k x columns v, and transposed
+    if (p.dht && kt < KT32) {
+      const float* d0 = p.dht + (int64_t)nh * K * V;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[r] = d0[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] * inv_scale;
+        acct[r] = d0[(int64_t)(kt * 32 + (lane & 31)) * V + vbase + c32_row(r, lane)] * inv_scale;
+      }
+    }
+    // gradient w.r.t. the state leaving chunk c: 16-bit transpose in LDS, FRAGMENT_T copy in memory
+    auto publish = [&](int64_t c) __attribute__((always_inline)) {
+      if (kt < KT32) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          v4 x;
+#pragma unroll
+          for (int b = 0; b < 4; ++b) x[b] = (T)(acc[4 * q4 + b] * scale);
+          *(v4*)&sDHt[(lane & 31) * LDK + kt * 32 + 8 * q4 + 4 * (lane >> 5)] = x;
+        }
+        v8 lo, hi;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          lo[r] = (T)(acct[r] * scale);
+          hi[r] = (T)(acct[r + 8] * scale);
+        }
+        T* hp = (T*)p.dhtf + ((chunk0 + c) * H + hh) * (int64_t)K * V + (((int64_t)vt * (K / 32) + kt) * 64 + lane) * 16;
+        *(v8*)hp = lo;
+        *(v8*)(hp + 8) = hi;
+      }
+    };
+    if (nchunks > 0) publish(nchunks - 1);
+    for (int64_t c = nchunks - 1; c >= 0; --c) {
+      lds_barrier();  // B1(c)
+      // ---- dv = s P^T do + k^ dH: wave w owns time rows 16w .. 16w+15, two 16-column tiles
+      {
+        f32x4 d[2] = {zero4(), zero4()}, dl[2] = {zero4(), zero4()};
+#pragma unroll
+        for (int ks = 0; ks < K; ks += 32) {
+          const v8 a = frag16_tr<T>(sKh, LDT, wave * 16, ks, lane);
+#pragma unroll
+          for (int j = 0; j < 2; ++j) d[j] = Elem<T>::mfma16(a, frag16<T>(sDHt, LDK, j * 16, ks, lane), d[j]);
+        }
+        if (!sFlag) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            if (32 * s + 31 < 16 * wave) continue;   // P is lower triangular (wave-uniform)
+            const v8 a = frag16_tr<T>(sP, LDT, wave * 16, 32 * s, lane);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) dl[j] = Elem<T>::mfma16(a, frag16_tr<T>(sDoY, LDV, 16 * j, 32 * s, lane), dl[j]);
+          }
+        }
+        const int tr = wave * 16 + 4 * (lane >> 4);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int vc = j * 16 + (lane & 15);
+          v4 o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[r] = (T)(scale * dl[j][r] + d[j][r]);
+          *(v4*)&sDvT[vc * LDT + tr] = o;
+        }
+      }
+      lds_barrier();  // B2(c)
+      // ---- dH / s <- decay * dH / s + (q e^{G})^T do, in both orientations
+      if (kt < KT32) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] *= sDec[kt * 32 + c32_row(r, lane)];
+        const float dt = sDec[kt * 32 + (lane & 31)];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acct[r] *= dt;
+#pragma unroll
+        for (int s = 0; s < BT; s += 16) {
+          const v8 fq = frag32_tr<T>(sQ, LDK, kt * 32, s, lane);
+          const v8 fd = frag32_tr<T>(sDoX, LDV, 0, s, lane);
+          acc = Elem<T>::mfma32(fq, fd, acc);
+          acct = Elem<T>::mfma32(fd, fq, acct);
+        }
+      }
+      if (c > 0) publish(c - 1);
+    }
+    if (p.dh0 && kt < KT32) {
+      float* o = p.dh0 + (int64_t)nh * K * V;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[(int64_t)(kt * 32 + c32_row(r, lane)) * V + vbase + (lane & 31)] = acc[r] * scale;
+    }
+  }
+}
+
 template <typename T, typename GT>
 __global__ __launch_bounds__(256) void gla_bwd_dh_kernel(BDhParams p) {
   typedef typename Elem<T>::v8 v8;
@@ -1233,14 +1518,25 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
                const void* hT, const void* qg, const float* decay, void* dhtf, void* dq, void* dk, void* dv, float* dg,
                float* dg_head, float* dh0, const int* wide,
                const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT, int64_t B,
-               int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st) {
+               int64_t T_, int64_t H, int64_t K, int64_t V, int64_t N, float scale, hipStream_t st,
+               const void* kh_t = nullptr, const void* scores = nullptr) {
   dim3 grid;
   int ntfix;
   int rc = chunk_grid(offsets, indices, B, T_, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return copy_or_zero(dht, dh0, N * H * K * V, st);   // no chunk at all: d h0 = d ht
   const int64_t total_chunks = grid.x;
-  {
+  const bool fused_dv = qg && kh_t && scores;   // the reverse state scan also forms dv
+  if (fused_dv) {
+    BDhvParams p{qg, kh_t, scores, decay, dout, dht, wide, dhtf, dv, dh0, offsets, chunk_offsets, T_, (int)H, (int)V, (int)N,
+                 scale};
+    const int64_t total = (V / 32) * N * H;
+    FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+    if (K == 64) hipLaunchKernelGGL((gla_bwd_dhv_kernel<T, 64>), dim3((unsigned)total), dim3(512), 0, st, p);
+    else if (K == 128) hipLaunchKernelGGL((gla_bwd_dhv_kernel<T, 128>), dim3((unsigned)total), dim3(512), 0, st, p);
+    else return FLA_E_UNSUPPORTED;
+    FLA_CHECK_LAUNCH();
+  } else {
     BDhParams p{q, g, dout, dht, dhtf, dh0, offsets, chunk_offsets, T_, total_chunks,
                 (int)H, (int)K, (int)V, (int)N, scale, qg, decay};
     int64_t total = (K / 64) * (V / 64) * N * H;
@@ -1250,7 +1546,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* g, const
     else hipLaunchKernelGGL((gla_bwd_dh_kernel<T, GT>), dim3((unsigned)total), dim3(256), 0, st, p);
     FLA_CHECK_LAUNCH();
   }
-  {
+  if (!fused_dv) {
     BDvParams p{q, k, g, dout, dhtf, wide, dv, offsets, indices, T_, (int)H, ntfix, scale};
     // as many workgroups as are resident at once, each walking its share of the (chunk, head) items
     const int64_t total = (int64_t)grid.x * grid.y;
@@ -1298,10 +1594,13 @@ static int gla_bwd_impl(const void* q, const void* k, const void* v, const void*
                         const int* wide,
                         const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                         int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
-                        int64_t N, float scale, fla_stream_t stream, bool head_gates = false) {
+                        int64_t N, float scale, fla_stream_t stream, bool head_gates = false,
+                        const void* kh_t = nullptr, const void* scores = nullptr) {
   FLA_REQUIRE(q && k && v && gates && dout && hT && dh_frag_t && dq && dk && dv && (dg || dg_head),
               FLA_E_INVALID);
   if (head_gates) FLA_REQUIRE(q_gated && dg_head, FLA_E_INVALID);
+  FLA_REQUIRE((kh_t == nullptr) == (scores == nullptr) && (kh_t == nullptr || q_gated != nullptr), FLA_E_INVALID);
+  FLA_REQUIRE(((uintptr_t)kh_t | (uintptr_t)scores) % 16 == 0, FLA_E_ALIGNMENT);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(K % 64 == 0 && V % 64 == 0 && K <= 128 && V <= 128, FLA_E_UNSUPPORTED);
   if (offsets) FLA_REQUIRE(indices && chunk_offsets && B == 1, FLA_E_INVALID);
@@ -1315,7 +1614,7 @@ static int gla_bwd_impl(const void* q, const void* k, const void* v, const void*
   hipStream_t st = (hipStream_t)stream;
 #define FLA_BWD(TT, GG)                                                                                           \
   return launch_bwd<TT, GG>(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, dg_head, dh0, wide,   \
-                            offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st)
+                            offsets, indices, chunk_offsets, NT, B, T, H, K, V, N, scale, st, kh_t, scores)
   if (head_gates && qkv_dtype == FLA_BF16) FLA_BWD(bf16, HeadGate);
   if (head_gates && qkv_dtype == FLA_F16) FLA_BWD(f16, HeadGate);
   if (head_gates) return FLA_E_UNSUPPORTED;
@@ -1340,14 +1639,16 @@ extern "C" int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, co
 
 extern "C" int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const void* gates,
                                       const void* dout, const float* dht, const void* hT, const void* q_gated,
-                                      const float* chunk_decay, void* dh_frag_t, void* dq, void* dk, void* dv,
+                                      const float* chunk_decay, const void* khat_t, const void* scores,
+                                      void* dh_frag_t, void* dq, void* dk, void* dv,
                                       float* dg, float* dh0, const int* wide, const int64_t* offsets,
                                       const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                                       int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                                       int64_t V, int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q_gated && chunk_decay, FLA_E_INVALID);
   return gla_bwd_impl(q, k, v, gates, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, dg, nullptr, dh0, wide,
-                      offsets, indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+                      offsets, indices, chunk_offsets, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream, false,
+                      khat_t, scores);
 }
 
 extern "C" int fla_chunk_simple_gla_bwd(const void* q, const void* k, const void* v, const float* g, const void* dout,

@@ -24,6 +24,8 @@ struct FusedParams {
   void* hT;         // HT variant: the state entering every chunk, FLA_H_FRAGMENT_T order, [chunks, H, K*V]
   void* qg;         // HT variant, optional: the gated queries q e^{G} as staged, [rows, H, K] in the q dtype
   float* decay;     //   and e^{G_last} of every chunk, [chunks, H, K] (both or neither)
+  void* kh_t;       // with qg, optional: k^ = k e^{G_last - G} per chunk as staged, [chunks, H, K, 64] (key-major) ...
+  void* scores;     //   ... and the chunk's causal score tile tril(q~ k~^T), [chunks, H, 64, 64] (both or neither)
 };
 
 // The row-major q~ / k~ tiles are written by lanes that own four adjacent rows each, i.e.

@@ -159,6 +159,29 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
           }
           if (vb == 0 && tid < K) p.decay[((chunk0 + c) * H + hh) * (int64_t)K + tid] = sDecay[buf][tid];
         }
+        if (p.kh_t) {
+          // k^ of the chunk, key-major as staged (rows of 64 time steps; zero past the end of a short chunk): the
+          // slabs share the key rows out
+          const int nrow = K / nvb, r0 = vb * nrow;
+          T* kb = (T*)p.kh_t + ((chunk0 + c) * H + hh) * (int64_t)K * BT;
+          for (int e = tid; e < nrow * (BT / 8); e += 256) {
+            const int row = r0 + e / (BT / 8), c8 = (e % (BT / 8)) * 8;
+            *(v8*)(kb + row * BT + c8) = *(const v8*)&sKh[buf][row * LDT + c8];
+          }
+        }
+      }
+    };
+    // the score tile of chunk c, once every wave has written its quadrant (rows shared out over the slabs)
+    auto store_scores = [&](int64_t c) {
+      if constexpr (HT) {
+        if (p.scores) {
+          const int nrow = BT / nvb, r0 = vb * nrow;
+          T* pb = (T*)p.scores + ((chunk0 + c) * H + hh) * (int64_t)BT * BT;
+          for (int e = tid; e < nrow * (BT / 8); e += 256) {
+            const int row = r0 + e / (BT / 8), c8 = (e % (BT / 8)) * 8;
+            *(v8*)(pb + row * BT + c8) = *(const v8*)&sP[row * LDT + c8];
+          }
+        }
       }
     };
     auto publish_state = [&]() {
@@ -298,6 +321,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         }
       }
       lds_barrier();  // B2(c): P visible; nobody reads the state fragments any more
+      store_scores(c);
       if (cw < NVT) {
       if (rw == 0) {
 #pragma unroll
@@ -617,7 +641,7 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
                               const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                               int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false,
-                              bool exact_pass = true) {
+                              bool exact_pass = true, void* kh_t = nullptr, void* scores = nullptr) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
   if (head_gates) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
@@ -638,8 +662,13 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     FLA_REQUIRE(V <= 256, FLA_E_UNSUPPORTED);
     FLA_REQUIRE((uintptr_t)qg % 16 == 0, FLA_E_ALIGNMENT);
   }
+  FLA_REQUIRE((kh_t == nullptr) == (scores == nullptr), FLA_E_INVALID);
+  if (kh_t) {
+    FLA_REQUIRE(qg != nullptr, FLA_E_INVALID);
+    FLA_REQUIRE(((uintptr_t)kh_t | (uintptr_t)scores) % 16 == 0, FLA_E_ALIGNMENT);
+  }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
-                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay};
+                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay, kh_t, scores};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;
@@ -709,14 +738,16 @@ extern "C" int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, cons
 
 extern "C" int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const void* v, const void* gates,
                                             const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
-                                            void* h_frag_t, void* q_gated, float* chunk_decay, const int64_t* offsets,
+                                            void* h_frag_t, void* q_gated, float* chunk_decay, void* khat_t,
+                                            void* scores, const int64_t* offsets,
                                             const int64_t* indices, const int64_t* chunk_offsets,
                                             const int64_t* seq_order, int64_t NT, int qkv_dtype, int gate_dtype,
                                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                             float scale, fla_stream_t stream) {
   FLA_REQUIRE(h_frag_t && q_gated && chunk_decay, FLA_E_INVALID);
   return gla_fwd_fused_impl(q, k, v, gates, h0, o, ht, ws_wide, ws_hwide, h_frag_t, q_gated, chunk_decay, offsets,
-                            indices, chunk_offsets, seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream);
+                            indices, chunk_offsets, seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale, stream,
+                            false, true, khat_t, scores);
 }
 
 extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, const float* g,

@@ -27,6 +27,9 @@ _SUPPORTED_KV = {(64, 64), (128, 128), (64, 128), (128, 64)}
 # pass, which the reference starts by recomputing those states (fla/ops/gla/chunk.py:1239-1253).
 # FLA_AMD_RECOMPUTE_STATES=1 (or setting this flag to False) restores the reference's behaviour.
 KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("", "0")
+# With the states, a differentiated forward (per-key gates, V <= 128) also keeps k^ = k e^{G_last - G} and the score tile
+# of every chunk (1.5 more tensors of k's size), from which the backward's reverse state scan forms dv on its way.
+KEEP_KHAT_AND_SCORES = os.environ.get("FLA_AMD_GLA_FUSED_DV", "1") not in ("", "0")
 
 
 def _pad_dim(x: Optional[torch.Tensor], size: int) -> Optional[torch.Tensor]:
@@ -230,9 +233,13 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         if V <= 256:
             qg = torch.empty_like(q)
             decay = q.new_empty(B, nt, H, K, dtype=torch.float32)
-            be.check(be.lib().fla_chunk_gla_fwd_fused_kept(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), *tail),
-                     "fla_chunk_gla_fwd_fused_kept")
-            states_out.extend((hT, qg, decay))
+            kh = sc = None
+            if KEEP_KHAT_AND_SCORES and V <= 128:
+                kh = q.new_empty(B, nt, H, K, BT)
+                sc = q.new_empty(B, nt, H, BT, BT)
+            be.check(be.lib().fla_chunk_gla_fwd_fused_kept(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), be.ptr(kh),
+                                                           be.ptr(sc), *tail), "fla_chunk_gla_fwd_fused_kept")
+            states_out.extend((hT, qg, decay) if kh is None else (hT, qg, decay, kh, sc))
         else:
             be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
             states_out.append(hT)
@@ -329,7 +336,7 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
 
 
 def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide=None, hT=None, qg=None,
-                         decay=None, head_gates=False):
+                         decay=None, head_gates=False, kh=None, scores=None):
     """Backward on prepared tensors (seq-first, 16-bit, 64-aligned head dims).
     Returns ``(dq, dk, dv, dg, dh0)``; without ``hT`` (the states a forward pass kept) it
     recomputes the per-chunk states as the reference does (``fla/ops/gla/chunk.py:1239-1253``).  ``qg``, ``decay``:
@@ -372,7 +379,8 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
         be.check(be.lib().fla_chunk_simple_gla_bwd(*head, be.ptr(qg), be.ptr(decay), *outs, *tail[:7], *tail[8:]),
                  "fla_chunk_simple_gla_bwd")
     elif kept:
-        be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), *outs, *tail), "fla_chunk_gla_bwd_kept")
+        be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), be.ptr(kh), be.ptr(scores), *outs,
+                                                 *tail), "fla_chunk_gla_bwd_kept")
     else:
         be.check(be.lib().fla_chunk_gla_bwd(*head, *outs, *tail), "fla_chunk_gla_bwd")
     if g_head is not None:
@@ -405,7 +413,9 @@ def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
     dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht,
                                                offsets, wide, hT=states[0],
                                                qg=states[1] if len(states) > 1 else None,
-                                               decay=states[2] if len(states) > 2 else None)
+                                               decay=states[2] if len(states) > 2 else None,
+                                               kh=states[3] if len(states) > 4 else None,
+                                               scores=states[4] if len(states) > 4 else None)
     if head_first:
         dq, dk, dv, dg = (x.transpose(1, 2) for x in (dq, dk, dv, dg))
     return dq, dk, dv, dg, dh0
@@ -443,7 +453,7 @@ class ChunkGLAFunction(torch.autograd.Function):
                                 states_out=states)
         # the inputs, the small table of chunks whose gates need the exact intra-chunk arithmetic, and
         # (unless recomputation is asked for) the per-chunk states the fused launch wrote on its way
-        kept = tuple(states) + (None,) * (3 - len(states)) if states else (None, None, None)
+        kept = tuple(states) + (None,) * (5 - len(states)) if states else (None,) * 5
         ctx.save_for_backward(q, k, v, g, h0, offsets, flags[0] if flags else None, *kept)
         ctx.scale, ctx.head_first, ctx.dims, ctx.in_dtypes = scale, head_first, (K, V, KP, VP), in_dtypes
         ctx.h0_dtype = None if initial_state is None else initial_state.dtype
@@ -459,7 +469,7 @@ class ChunkGLAFunction(torch.autograd.Function):
     @staticmethod
     @contiguous
     def backward(ctx, do, dht):
-        q, k, v, g, h0, offsets, wide, hT, qg, decay = ctx.saved_tensors
+        q, k, v, g, h0, offsets, wide, hT, qg, decay, kh, scores = ctx.saved_tensors
         K, V, KP, VP = ctx.dims
         if ctx.head_first:
             do = do.transpose(1, 2)
@@ -470,7 +480,7 @@ class ChunkGLAFunction(torch.autograd.Function):
         if dht is not None and (KP, VP) != (K, V):
             dht = F.pad(dht, (0, VP - V, 0, KP - K))
         dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, ctx.scale, h0, do, dht, offsets, wide, hT=hT, qg=qg,
-                                                   decay=decay)
+                                                   decay=decay, kh=kh, scores=scores)
         if (KP, VP) != (K, V):
             dq, dk, dg, dv = dq[..., :K], dk[..., :K], dg[..., :K], dv[..., :V]
             if dh0 is not None:

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 9
+#define FLA_ABI_VERSION 10
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -228,10 +228,13 @@ int fla_chunk_gla_fwd_fused_states(const void* q, const void* k, const void* v, 
  * from q and the gates again (the reference's chunk_bwd_dh does, fla/ops/common/chunk_h.py:156-271): the gated
  * queries q_gated = q e^{G} ([B,T,H,K] in the q/k/v dtype, G the chunk-local prefix sum of the log-gates; rows
  * past the end of a short chunk are not written) and chunk_decay = e^{G_last} (fp32 [chunks, H, K]).  Hand both
- * to fla_chunk_gla_bwd_kept. */
+ * to fla_chunk_gla_bwd_kept.  khat_t and scores (both or neither, q/k/v dtype): k^ = k e^{G_last - G} per chunk,
+ * key-major [chunks, H, K, 64], and the chunk's causal score tile tril(q~ k~^T) (unscaled), [chunks, H, 64, 64]; with
+ * them fla_chunk_gla_bwd_kept forms dv inside its reverse state scan. */
 int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const void* v, const void* gates,
                                  const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
-                                 void* h_frag_t, void* q_gated, float* chunk_decay, const int64_t* offsets,
+                                 void* h_frag_t, void* q_gated, float* chunk_decay, void* khat_t, void* scores,
+                                 const int64_t* offsets,
                                  const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order,
                                  int64_t NT, int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
                                  int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
@@ -366,10 +369,12 @@ int fla_chunk_gla_bwd(const void* q, const void* k, const void* v, const void* g
 
 /* The same with q_gated and chunk_decay from fla_chunk_gla_fwd_fused_kept: the reverse state scan
  * (chunk_bwd_dh, fla/ops/common/chunk_h.py:338-402) streams them and do instead of re-forming prefix sums and
- * exponentials from q and the gates; results equal fla_chunk_gla_bwd's to rounding.  scale must not be 0. */
+ * exponentials from q and the gates; results equal fla_chunk_gla_bwd's to rounding.  scale must not be 0.
+ * khat_t and scores (both or NULL) as the forward left them: the scan then also forms dv = s P^T do + k^ dH
+ * (chunk_gla_bwd_dv, fla/ops/gla/chunk.py:1037-1061) and the launch of its own for dv is skipped: two launches. */
 int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const void* gates, const void* dout,
                            const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
-                           void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                           const void* khat_t, const void* scores, void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
                            const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                            int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                            int64_t N, float scale, fla_stream_t stream);

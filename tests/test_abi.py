@@ -56,11 +56,11 @@ def test_argument_validation_without_device():
     # the states-keeping GLA forward that also leaves gated queries and chunk decays: all three outputs or none,
     # at most 256 value columns; its backward divides by the scale
     z = (None,) * 4
-    fwd = lambda hT, qg, dec, V: lib.fla_chunk_gla_fwd_fused_kept(p, p, p, p, None, p, None, None, None, hT, qg, dec, *z,
+    fwd = lambda hT, qg, dec, V: lib.fla_chunk_gla_fwd_fused_kept(p, p, p, p, None, p, None, None, None, hT, qg, dec, None, None, *z,
                                                                   0, 0, 2, 1, 64, 1, 64, V, 1, 1.0, None)
     assert fwd(p, p, None, 64) == -1 and fwd(None, p, p, 64) == -1 and fwd(p, None, None, 64) == -1
     assert fwd(p, p, p, 320) == -2
-    bwd = lambda qg, dec, scale: lib.fla_chunk_gla_bwd_kept(p, p, p, p, p, None, p, qg, dec, p, p, p, p, p, None, None,
+    bwd = lambda qg, dec, scale: lib.fla_chunk_gla_bwd_kept(p, p, p, p, p, None, p, qg, dec, None, None, p, p, p, p, p, None, None,
                                                             None, None, None, 0, 0, 2, 1, 64, 1, 64, 64, 1, scale, None)
     assert bwd(p, None, 1.0) == -1 and bwd(p, p, 0.0) == -1
     # the per-head-gate backward needs the kept gated queries and a gate-gradient buffer
