@@ -1653,12 +1653,13 @@ extern "C" int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* 
 
 extern "C" int fla_chunk_simple_gla_bwd(const void* q, const void* k, const void* v, const float* g, const void* dout,
                                         const float* dht, const void* hT, const void* q_gated,
-                                        const float* chunk_decay, void* dh_frag_t, void* dq, void* dk, void* dv,
-                                        float* dg, float* dh0, const int* wide, const int64_t* offsets,
+                                        const float* chunk_decay, const void* khat_t, const void* scores,
+                                        void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide, const int64_t* offsets,
                                         const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                                         int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                                         int64_t N, float scale, fla_stream_t stream) {
   FLA_REQUIRE(q_gated && chunk_decay && dg, FLA_E_INVALID);
   return gla_bwd_impl(q, k, v, g, dout, dht, hT, q_gated, chunk_decay, dh_frag_t, dq, dk, dv, nullptr, dg, dh0, wide,
-                      offsets, indices, chunk_offsets, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true);
+                      offsets, indices, chunk_offsets, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true,
+                      khat_t, scores);
 }

@@ -752,11 +752,11 @@ extern "C" int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const 
 
 extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, const float* g,
                                               const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
-                                              void* h_frag_t, void* q_gated, float* chunk_decay,
-                                              const int64_t* offsets, const int64_t* indices,
+                                              void* h_frag_t, void* q_gated, float* chunk_decay, void* khat_t,
+                                              void* scores, const int64_t* offsets, const int64_t* indices,
                                               const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                                               int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                                               int64_t N, float scale, fla_stream_t stream) {
   return gla_fwd_fused_impl(q, k, v, g, h0, o, ht, ws_wide, ws_hwide, h_frag_t, q_gated, chunk_decay, offsets, indices, chunk_offsets,
-                            seq_order, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true);
+                            seq_order, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true, true, khat_t, scores);
 }

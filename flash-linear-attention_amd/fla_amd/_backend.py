@@ -45,7 +45,7 @@ SIGNATURES = {
     "fla_chunk_gla_fwd_fused_first_launch": (c_int, [P] * 13 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_states": (c_int, [P] * 14 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_fused_kept": (c_int, [P] * 18 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
-    "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 16 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_fwd_fused": (c_int, [P] * 18 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_gdr_fwd_wy": (c_int, [P, P, P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_h": (c_int, [P, P, P, P, P, P, P, P, P, P, I, I, I,
                                                  I64, I64, I64, I64, I64, I64, P]),
@@ -55,7 +55,7 @@ SIGNATURES = {
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 17 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_kept": (c_int, [P] * 21 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),
-    "fla_chunk_simple_gla_bwd": (c_int, [P] * 19 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_bwd": (c_int, [P] * 21 + [I64, I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_fwd_o_gk": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_dA": (c_int, [P] * 5 + [I64, I, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd_dv": (c_int, [P] * 8 + [I64, I, I, I, I64, I64, I64, I64, I64, P]),

@@ -216,7 +216,7 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     if head_gates:
         if g.dtype != torch.float32 or g.shape != q.shape[:3]:
             raise ValueError("head gates must be fp32 [B, T, H]")
-        hT = qg = decay = None
+        hT = qg = decay = kh = sc = None
         if states_out is not None:
             nt = plan.NT if plan is not None else -(-T // BT)
             hT = q.new_empty(B, nt, H, K, V)
@@ -225,7 +225,11 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
                 qg = torch.empty_like(q)
                 decay = q.new_empty(B, nt, H, K, dtype=torch.float32)
                 states_out.extend((qg, decay))
-        be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), *tail[:5],
+                if KEEP_KHAT_AND_SCORES and V <= 128:
+                    kh = q.new_empty(B, nt, H, K, BT)
+                    sc = q.new_empty(B, nt, H, BT, BT)
+                    states_out.extend((kh, sc))
+        be.check(be.lib().fla_chunk_simple_gla_fwd_fused(*head, be.ptr(hT), be.ptr(qg), be.ptr(decay), be.ptr(kh), be.ptr(sc), *tail[:5],
                                                          be.dt(q), *tail[7:]), "fla_chunk_simple_gla_fwd_fused")
     elif states_out is not None:
         nt = plan.NT if plan is not None else -(-T // BT)
@@ -376,7 +380,8 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     outs = (be.ptr(dhtf), be.ptr(dq), be.ptr(dk), be.ptr(dv), be.ptr(dg))
     head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(do), be.ptr(dht), be.ptr(hT))
     if kept and head_gates:
-        be.check(be.lib().fla_chunk_simple_gla_bwd(*head, be.ptr(qg), be.ptr(decay), *outs, *tail[:7], *tail[8:]),
+        be.check(be.lib().fla_chunk_simple_gla_bwd(*head, be.ptr(qg), be.ptr(decay), be.ptr(kh), be.ptr(scores), *outs,
+                                                   *tail[:7], *tail[8:]),
                  "fla_chunk_simple_gla_bwd")
     elif kept:
         be.check(be.lib().fla_chunk_gla_bwd_kept(*head, be.ptr(qg), be.ptr(decay), be.ptr(kh), be.ptr(scores), *outs,

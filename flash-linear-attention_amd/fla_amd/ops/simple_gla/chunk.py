@@ -45,9 +45,11 @@ class ChunkSimpleGLAFunction(torch.autograd.Function):
         q, k, v, gf, h0, offsets, wide, *kept = ctx.saved_tensors
         hT = kept[0] if kept else None
         qg, decay = (kept[1], kept[2]) if len(kept) > 2 else (None, None)
+        kh, scores = (kept[3], kept[4]) if len(kept) > 4 else (None, None)
         h0f = None if h0 is None else h0.float().contiguous()
         dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, gf, ctx.scale, h0f, do.to(q.dtype).contiguous(), dht,
-                                                   offsets, wide, hT=hT, qg=qg, decay=decay, head_gates=True)
+                                                   offsets, wide, hT=hT, qg=qg, decay=decay, head_gates=True, kh=kh,
+                                                   scores=scores)
         if dh0 is not None:
             dh0 = dh0.to(ctx.h0_dtype)
         return dq, dk, dv, dg.to(ctx.g_dtype), None, dh0, None, None

@@ -243,11 +243,11 @@ int fla_chunk_gla_fwd_fused_kept(const void* q, const void* k, const void* v, co
  * (fla/ops/simple_gla/chunk.py:16-131: h_t = e^{g_t} h_{t-1} + k_t v_t^T, o_t = scale q_t^T h_t) without
  * the [B,T,H,K] gate tensor a call through fla_chunk_gla_fwd_fused would need.  Same kernel, the staging
  * waves load one gate word per row; everything else (workspaces of the range guard, h_frag_t as in
- * fla_chunk_gla_fwd_fused_states or NULL, q_gated and chunk_decay as in fla_chunk_gla_fwd_fused_kept or both
- * NULL, packed batches) as for the entry points above. */
+ * fla_chunk_gla_fwd_fused_states or NULL, q_gated and chunk_decay, khat_t and scores as in
+ * fla_chunk_gla_fwd_fused_kept or NULL in pairs, packed batches) as for the entry points above. */
 int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, const float* g,
                                    const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
-                                   void* h_frag_t, void* q_gated, float* chunk_decay,
+                                   void* h_frag_t, void* q_gated, float* chunk_decay, void* khat_t, void* scores,
                                    const int64_t* offsets, const int64_t* indices,
                                    const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                                    int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
@@ -387,7 +387,7 @@ int fla_chunk_gla_bwd_kept(const void* q, const void* k, const void* v, const vo
  * everything else as for fla_chunk_gla_bwd_kept. */
 int fla_chunk_simple_gla_bwd(const void* q, const void* k, const void* v, const float* g, const void* dout,
                              const float* dht, const void* hT, const void* q_gated, const float* chunk_decay,
-                             void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
+                             const void* khat_t, const void* scores, void* dh_frag_t, void* dq, void* dk, void* dv, float* dg, float* dh0, const int* wide,
                              const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets, int64_t NT,
                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                              float scale, fla_stream_t stream);

@@ -64,7 +64,7 @@ def test_argument_validation_without_device():
                                                             None, None, None, 0, 0, 2, 1, 64, 1, 64, 64, 1, scale, None)
     assert bwd(p, None, 1.0) == -1 and bwd(p, p, 0.0) == -1
     # the per-head-gate backward needs the kept gated queries and a gate-gradient buffer
-    sgb = lambda qg, dg: lib.fla_chunk_simple_gla_bwd(p, p, p, p, p, None, p, qg, p, p, p, p, p, dg, None, None, None, None,
+    sgb = lambda qg, dg: lib.fla_chunk_simple_gla_bwd(p, p, p, p, p, None, p, qg, p, None, None, p, p, p, p, dg, None, None, None, None,
                                                       None, 0, 2, 1, 64, 1, 64, 64, 1, 1.0, None)
     assert sgb(None, p) == -1 and sgb(p, None) == -1
     # the delta rule's chunk-parallel launch: w and Aw together or not at all, K in {64, 128}
