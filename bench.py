@@ -46,13 +46,15 @@ def _events(n):
 ROW_RAMP_SECONDS = 0.2     # untimed load ahead of every timed row other than the headline step
 
 
-def event_stats(fn, steps, warmup=3, ramp=None):
+def event_stats(fn, steps, warmup=3, ramp=None, between=None):
     """Device time of one call from HIP events recorded on the launch stream around every call:
     median, min, max and mean in microseconds, the number of intervals longer than twice the median
     (a stalled launch: clock ramp, an allocation, something else on the box) and the wall time of the
     whole timed loop, which is bracketed by synchronize on both sides.  The setup of a row (allocations,
     first calls) leaves the device idle for milliseconds and its clocks drop; `ramp` seconds of the call
-    itself run untimed first, so that a 20-launch row and a 200-launch row report the same figure."""
+    itself run untimed first, so that a 20-launch row and a 200-launch row report the same figure.
+    `between`, if given, runs on the same stream ahead of every timed call, outside its pair of events
+    (a write over a large buffer that pushes the previous call's tensors out of the last-level cache)."""
     import statistics
     import torch
     if ramp is None:
@@ -68,6 +70,8 @@ def event_stats(fn, steps, warmup=3, ramp=None):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
+        if between is not None:
+            between()
         ev[2 * i].record()
         fn()
         ev[2 * i + 1].record()
@@ -85,9 +89,9 @@ def spread(st):
             "n_over_2x_median": st["n_over_2x_median"]}
 
 
-def event_avg_us(fn, steps, warmup=3, ramp=None):
+def event_avg_us(fn, steps, warmup=3, ramp=None, between=None):
     """Median device time of one call (see event_stats)."""
-    return event_stats(fn, steps, warmup, ramp)["median_us"]
+    return event_stats(fn, steps, warmup, ramp, between)["median_us"]
 
 
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
@@ -439,9 +443,19 @@ def bench_layer_steps(device, steps=20):
     nb = x.numel() * 2
     out = {}
 
+    # These rows move 134 MB tensors, which a 256 MB last-level cache partly keeps from one launch to the
+    # next: `us` is timed with 1 GiB read between the launches (every operand then comes from HBM, as it
+    # does behind the operators inside a layer; a read, because the dirty lines of a 1 GiB write would still
+    # be draining under the timed launch), `us_back_to_back` without.  Either way part of a launch's own
+    # output can still sit in that cache when its end event fires, so a row above the device-copy rate is
+    # not an HBM rate.
+    flush = torch.zeros(1 << 28, dtype=torch.int32, device=device)
+
     def rec(name, fn, nbytes):
-        us = event_avg_us(fn, steps)
-        out[name] = {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1),
+        warm = event_avg_us(fn, steps)
+        us = event_avg_us(fn, steps, ramp=0.0, between=flush.max)
+        out[name] = {"us": round(us, 1), "us_back_to_back": round(warm, 1), "algorithmic_bytes": nbytes,
+                     "GBs": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
     rec("l2norm_fwd", lambda: l2norm_fwd(x), 2 * nb)
@@ -486,9 +500,15 @@ def bench_gla_stages(device, steps=20):
     b_qk, b_v, b_g, b_a, b_h = tok * K * 2, tok * V * 2, tok * K * 4, tok * 64 * 4, h.numel() * 4
     out = {}
 
+    # timed like the layer steps: 1 GiB read between the launches, so that no operand is still in the
+    # 256 MB last-level cache (`us`); `us_back_to_back` is the same launch without that read
+    flush = torch.zeros(1 << 28, dtype=torch.int32, device=device)
+
     def rec(name, fn, nbytes):
-        us = event_avg_us(fn, steps)
-        out[name] = {"us": round(us, 1), "algorithmic_bytes": nbytes, "GBs": round(nbytes / us / 1e3, 1),
+        warm = event_avg_us(fn, steps)
+        us = event_avg_us(fn, steps, ramp=0.0, between=flush.max)
+        out[name] = {"us": round(us, 1), "us_back_to_back": round(warm, 1), "algorithmic_bytes": nbytes,
+                     "GBs": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
     rec("chunk_gla_fwd_o_gk", lambda: chunk_gla_fwd_o_gk(q, v, G, A, h, K ** -0.5, head_first=False),
