@@ -7,9 +7,9 @@ A step is one chunk_gla forward on the headline workload (B=8, T=4096, H=16,
 K=V=128, bf16 q/k/v, fp32 log-gates and state, initial state given, final state
 returned), inputs resident in HBM.  Prints ONE JSON line:
 
-* value            tokens/s of the whole forward: B*T / the median step time (every step sits between
-                   two HIP events on the launch stream; min, max, the number of stalled intervals and
-                   the wall time of the same loop are reported in extra.chunk_gla_fwd)
+* value            tokens/s of the whole forward: tokens of the K timed steps / the wall time between the two
+                   synchronisations that bracket them (ms_per_step = that wall time / K; the host time of a
+                   call with the launches stubbed out is in extra.chunk_gla_fwd.host_us_per_call)
 * roofline         the dominant kernel of that forward against the HBM roofline:
                    algorithmic bytes per launch / its median duration measured
                    here with HIP events on the launch stream; traffic = HBM bytes per launch from
@@ -94,6 +94,38 @@ def event_avg_us(fn, steps, warmup=3, ramp=None, between=None):
     return event_stats(fn, steps, warmup, ramp, between)["median_us"]
 
 
+class _StubLib:
+    """Stands in for the loaded library: the named entry points return 0 without launching anything."""
+
+    def __init__(self, real, names):
+        self._real, self._names = real, set(names)
+
+    def __getattr__(self, name):
+        if name in self._names:
+            return lambda *a: 0
+        return getattr(self._real, name)
+
+
+def host_time_us(fn, entry_points, n=2000):
+    """Host time of one call of `fn` with the kernel launches of `entry_points` stubbed out (argument
+    marshalling, allocations and Python included; the device stays idle)."""
+    import torch
+    from fla_amd import _backend as be
+    real = be.lib()
+    be._lib = _StubLib(real, entry_points)
+    try:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        dt = time.perf_counter() - t0
+    finally:
+        be._lib = real
+    return dt / n * 1e6
+
+
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_counters.txt")
 
 
@@ -159,12 +191,22 @@ def bench_gla(device, steps, warmup):
             if now - t_ramp >= RAMP_MAX_SECONDS or (steady and now - t_ramp >= RAMP_SECONDS):
                 break
 
-    # `warmup` untimed steps, then exactly `steps` steps between two synchronisations, each step between
-    # two HIP events on the launch stream.  value = tokens / median step time; the wall time of the same
-    # loop and the spread of the intervals are reported beside it.
-    st = event_stats(step, steps, warmup, ramp=0.0)   # ramped above
-    ms = st["median_us"] * 1e-3
-    tokens_per_s = B * T / (st["median_us"] * 1e-6)
+    # `warmup` untimed steps, then exactly `steps` steps between two synchronisations: value = tokens of those
+    # steps / the wall time between the two synchronisations (host side of every step included; the host
+    # needs a fraction of a step per call, so the launches queue up and the device sets the pace).
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) / steps * 1e6
+    ms = wall_us * 1e-3
+    tokens_per_s = B * T / (wall_us * 1e-6)
+
+    # host side of one step: the same call with the two launches replaced by stubs that return at once
+    host_us = host_time_us(step, ("fla_chunk_gla_fwd_fused",))
 
     # device time of the kernels of the forward, HIP events on the launch stream.  The operator is
     # gla_fwd_fused_kernel followed by the range guard's short second launch; the dominant kernel is
@@ -222,8 +264,10 @@ def bench_gla(device, steps, warmup):
     op = {"algorithmic_bytes": floor_bytes, "achieved_GBs": round(floor_bytes / (ms * 1e-3) / 1e9, 1),
           "frac_of_hbm_peak": round(floor_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
           "algorithmic_flops": flops, "frac_of_mfma_peak": round(flops / (ms * 1e-3) / MFMA_PEAK_FLOPS, 4),
-          "step_us": round(st["median_us"], 1), **spread(st),
-          "wall_us_per_step": round(st["wall_us_per_call"], 1),
+          "wall_us_per_step": round(wall_us, 1), "host_us_per_call": round(host_us, 1),
+          # the step is the dominant kernel plus the range guard's short second launch: host-bound would show as
+          # a wall time per step well above the device time of the two
+          "host_bound": bool(host_us > 0.5 * wall_us or wall_us > 1.08 * us_f),
           "two_kernel_pipeline_us": {"gla_fwd_h_kernel": round(us_h, 1), "gla_fwd_o_kernel": round(us_o, 1)},
           "two_kernel_pipeline_GBs": {"gla_fwd_h_kernel": round(bytes_h / (us_h * 1e-6) / 1e9, 1),
                                       "gla_fwd_o_kernel": round(bytes_o / (us_o * 1e-6) / 1e9, 1)}}

@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -79,6 +79,11 @@ SIGNATURES = {
     "fla_causal_conv1d_bwd_partials": (c_int, [I64, I64]),
     "fla_causal_conv1d_bwd": (c_int, [P] * 7 + [I64, I64, I64, I64, I, I, P]),
     "fla_causal_conv1d_update": (c_int, [P] * 5 + [I64, I64, I64, I, I, P]),
+    "fla_gate_logsigmoid_fwd": (c_int, [P, P, I64, F, I, F, I, I, P]),
+    "fla_gate_logsigmoid_bwd": (c_int, [P, P, P, I64, F, I, F, I, I, P]),
+    "fla_gdn_gate_workgroups": (c_int, [I64, I64]),
+    "fla_gdn_gate_fwd": (c_int, [P, P, P, P, P, P, I64, I64, I, I, P]),
+    "fla_gdn_gate_bwd": (c_int, [P] * 9 + [I64, I64, I, I, P]),
     "fla_selftest_mfma": (c_int, [P, P, P, I64, I64, I64, I, P]),
 }
 

@@ -226,6 +226,26 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
                 None, None, None)
 
 
+def _direct_launch_ok(q, k, v, g, beta, initial_state, head_first) -> bool:
+    """True when a call can go straight to the two forward launches: no operand takes part in autograd and every
+    operand already has the layout, dtype and head dims the kernels read.  Anything else takes the autograd
+    function, which converts and pads."""
+    if head_first or q.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    K, V = q.shape[-1], v.shape[-1]
+    if K > _FUSED_MAX_K or (K, V) not in _SUPPORTED_KV:
+        return False
+    if torch.is_autocast_enabled():
+        return False
+    ts = (q, k, v, beta) if g is None else (q, k, v, beta, g)
+    if torch.is_grad_enabled() and (any(t.requires_grad for t in ts) or
+                                    (initial_state is not None and initial_state.requires_grad)):
+        return False
+    if not all(t.is_cuda and t.is_contiguous() for t in ts):
+        return False
+    return initial_state is None or (initial_state.dtype == torch.float32 and initial_state.is_contiguous())
+
+
 def apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first):
     """The autograd function on heads of any supported width (``g`` may be None: un-gated rule)."""
     K, V = k.shape[-1], v.shape[-1]
@@ -283,4 +303,9 @@ def chunk_gated_delta_rule(
         assert scale > 0, "Scale must be positive."
     if q.numel() == 0:
         return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
+    if _direct_launch_ok(q, k, v, g, beta, initial_state, head_first):
+        # nothing to differentiate and nothing to convert: no autograd node, no copies
+        _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
+                                                    offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+        return o, ht
     return apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first)

@@ -498,6 +498,26 @@ class ChunkGLAFunction(torch.autograd.Function):
         return dq.to(qd), dk.to(kd), dv.to(vd), dg.to(gd), None, dh0, None, None, None
 
 
+def _direct_launch_ok(q, k, v, g, initial_state, head_first) -> bool:
+    """True when a call can go straight to the fused launch: no operand takes part in autograd, and every
+    operand already has the layout, dtype and head dims the kernel reads (seq-first, contiguous, one 16-bit
+    dtype, fp32 or 16-bit gates, fp32 state, built tile sizes).  Anything else takes the autograd function,
+    which converts and pads."""
+    if head_first or q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        return False
+    if g.dtype != torch.float32 and g.dtype != q.dtype:
+        return False
+    if (q.shape[-1], v.shape[-1]) not in _SUPPORTED_KV:
+        return False
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad or g.requires_grad or
+                                    (initial_state is not None and initial_state.requires_grad)):
+        return False
+    if not (q.is_cuda and k.is_cuda and v.is_cuda and g.is_cuda and q.is_contiguous() and k.is_contiguous()
+            and v.is_contiguous() and g.is_contiguous()):
+        return False
+    return initial_state is None or (initial_state.dtype == torch.float32 and initial_state.is_contiguous())
+
+
 def _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first):
     """fp32 q/k/v (the reference runs and tests the operator in fp32, ``tests/ops/test_gla.py:29-87``): the
     chunk kernels multiply 16-bit operands, so fp32 callers are served by the token-by-token kernels, which
@@ -586,5 +606,8 @@ def chunk_gla(
             outs.append(o)
             states.append(ht)
         return torch.cat(outs, dim=-1), (torch.cat(states, dim=-1) if output_final_state else None)
+    if _direct_launch_ok(q, k, v, g, initial_state, head_first):
+        # nothing to differentiate and nothing to convert: no autograd node, no copies
+        return chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets)
     o, final_state = ChunkGLAFunction.apply(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
     return o, final_state

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 10
+#define FLA_ABI_VERSION 11
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -597,6 +597,33 @@ int fla_causal_conv1d_bwd(const void* x, const float* weight, const float* bias,
                           int dtype, fla_stream_t stream);
 int fla_causal_conv1d_update(const void* x, void* cache, const float* weight, const float* bias, void* y,
                              int64_t B, int64_t D, int64_t W, int silu, int dtype, fla_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Gate pre-activations of the layers that call the chunk operators.
+ *
+ * fla_gate_logsigmoid_fwd / _bwd replace the elementwise torch ops in front of chunk_gla
+ * (fla/layers/gla.py:214-217): y = logsigmoid(x) / normalizer, then max(y, clamp_min) when has_clamp;
+ * dx = dy * sigmoid(-x) / normalizer where the clamp did not bind, 0 elsewhere.  n elements
+ * (n % 8 == 0); x/dx in x_dtype, y in y_dtype (fp32, or x_dtype), dy in dy_dtype (fp32, or x_dtype).
+ *
+ * fla_gdn_gate_fwd / _bwd replace the two lines in front of chunk_gated_delta_rule
+ * (fla/layers/gated_deltanet.py:236-237): g[m,h] = -exp(A_log[h]) * softplus(a[m,h] + dt_bias[h]) in
+ * fp32 (softplus as torch.nn.functional.softplus, threshold 20) and beta = sigmoid(b) in b_dtype;
+ * a, b [M,H] in a_dtype / b_dtype (both fp32 or the same 16-bit type), A_log, dt_bias fp32 [H] (dt_bias
+ * may be NULL), H <= 256; b / beta (and dbeta / db) may be NULL together.  The backward writes da, db and
+ * per-workgroup partial sums partials fp32 [P,2,H], P = fla_gdn_gate_workgroups(M, H): their sums over P
+ * are the gradients of A_log (index 0) and dt_bias (index 1); fixed order, no atomics.
+ * ---------------------------------------------------------------------- */
+int fla_gate_logsigmoid_fwd(const void* x, void* y, int64_t n, float normalizer, int has_clamp, float clamp_min,
+                            int x_dtype, int y_dtype, fla_stream_t stream);
+int fla_gate_logsigmoid_bwd(const void* x, const void* dy, void* dx, int64_t n, float normalizer, int has_clamp,
+                            float clamp_min, int x_dtype, int dy_dtype, fla_stream_t stream);
+int fla_gdn_gate_workgroups(int64_t M, int64_t H);
+int fla_gdn_gate_fwd(const void* a, const void* b, const float* A_log, const float* dt_bias, float* g, void* beta,
+                     int64_t M, int64_t H, int a_dtype, int b_dtype, fla_stream_t stream);
+int fla_gdn_gate_bwd(const void* a, const void* b, const float* A_log, const float* dt_bias, const float* dg,
+                     const void* dbeta, void* da, void* db, float* partials, int64_t M, int64_t H, int a_dtype,
+                     int b_dtype, fla_stream_t stream);
 
 /* Diagnostics: C[M,N] (fp32) = A[M,Kd] * B[N,Kd]^T with bf16 operands, computed
  * with the same MFMA fragment helpers the kernels use (mode 0: 32x32x16 tiles,

@@ -12,6 +12,12 @@
   ``W - 1``, cropped to ``T``, then SiLU; ``causal_conv1d_step`` follows ``step``
   (``:203-210``): roll the cache left, write ``x`` last, ``sum(cache * w) + b``, SiLU.
 
+* ``gla_gate`` follows ``fla/layers/gla.py:214-217`` (``logsigmoid(x) / normalizer``, then an optional
+  ``clamp_min``); ``gdn_gate`` follows ``fla/layers/gated_deltanet.py:236-237``
+  (``g = -exp(A_log) * softplus(a + dt_bias)`` in fp32, ``beta = sigmoid(b)``).  Both are written from
+  the defining formulas (``log(1 / (1 + e^{-x}))``, ``log(1 + e^{x})``) in a numerically stable form and
+  pinned against ``torch.nn.functional.logsigmoid`` / ``softplus`` / ``sigmoid``.
+
 Pinned by tests/test_oracle_modules.py: unit norm and scale invariance of ``l2norm``;
 ``norm_swish_gate`` against ``torch.nn.functional.layer_norm`` / ``rms_norm`` times
 ``silu``; ``causal_conv1d`` against ``torch.nn.functional.conv1d``, causality, and the
@@ -73,3 +79,24 @@ def causal_conv1d_step(x, cache, weight, bias=None, activation: Optional[str] = 
     if activation in ("silu", "swish"):
         y = y * torch.sigmoid(y)
     return y, cache
+
+
+def gla_gate(x, normalizer: float = 16.0, clamp_min: Optional[float] = None, dtype=torch.float32):
+    """``log sigmoid(x) / normalizer`` with ``log sigmoid(x) = min(x, 0) - log(1 + e^{-|x|})``, clamped from below."""
+    x = x.to(dtype)
+    y = (torch.minimum(x, torch.zeros_like(x)) - torch.log1p(torch.exp(-x.abs()))) / normalizer
+    if clamp_min is not None:
+        y = torch.clamp(y, min=clamp_min)
+    return y
+
+
+def gdn_gate(a, b, A_log, dt_bias=None, dtype=torch.float32):
+    """``(g, beta)``: ``g = -e^{A_log} * log(1 + e^{a + dt_bias})`` (the argument itself above 20, where the two
+    agree to fp32 precision), ``beta = 1 / (1 + e^{-b})``."""
+    x = a.to(dtype)
+    if dt_bias is not None:
+        x = x + dt_bias.to(dtype)
+    sp = torch.where(x > 20, x, torch.log1p(torch.exp(torch.clamp(x, max=20))))
+    g = -torch.exp(A_log.to(dtype)) * sp
+    beta = None if b is None else 1.0 / (1.0 + torch.exp(-b.to(dtype)))
+    return g, beta

@@ -201,3 +201,81 @@ def test_short_convolution_step(device, dtype, W):
     got = torch.cat(outs, dim=1)
     assert_close("y", full, got, 1e-6 if dtype == torch.float32 else 4e-3)
     assert torch.equal(cache, x[:, -W:].transpose(1, 2))
+
+
+@pytest.mark.parametrize("dtype,out_dtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+                                             (torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16)])
+@pytest.mark.parametrize("normalizer,clamp_min", [(16.0, None), (1.0, None), (0.05, None), (16.0, -0.05)])
+def test_gla_gate(device, dtype, out_dtype, normalizer, clamp_min):
+    """logsigmoid(x) / normalizer (+ clamp) of fla/layers/gla.py:214-217, forward and backward."""
+    from fla_amd.modules import gla_gate
+    from oracle.modules import gla_gate as ref_gate
+    gen = torch.Generator().manual_seed(11)
+    x = (torch.randn(2, 129, 4, 64, generator=gen) * 3).to(dtype)
+    x[0, 0, 0, :8] = torch.tensor([-90.0, -30.0, -12.0, 0.0, 12.0, 30.0, 90.0, 1e-3]).to(dtype)
+    dy = torch.randn(2, 129, 4, 64, generator=gen)
+    print(f"gla_gate {dtype}->{out_dtype} normalizer={normalizer} clamp={clamp_min}", flush=True)
+    xd = x.to(device).requires_grad_()
+    y = gla_gate(xd, normalizer, clamp_min, output_dtype=out_dtype)
+    y.backward(dy.to(device).to(out_dtype))
+    xr = x.double().requires_grad_()
+    yr = ref_gate(xr, normalizer, clamp_min, dtype=torch.float64)
+    yr.backward(dy.to(out_dtype).double())
+    assert y.dtype == out_dtype and xd.grad.dtype == dtype
+    assert_close("y", yr, y, 1e-5 if out_dtype == torch.float32 else 4e-3)
+    # tiny values far on the positive side must keep their relative accuracy too (they are e^{-x}, not 0)
+    if out_dtype == torch.float32 and clamp_min is None:
+        big = x.double() > 10
+        assert_close("y(x > 10)", yr[big], y.detach().cpu()[big], 1e-5)
+    assert_close("dx", xr.grad, xd.grad, 1e-5 if dtype == torch.float32 else 4e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("H,with_b,with_bias", [(16, True, True), (6, True, True), (32, False, True), (7, True, False)])
+def test_gdn_gate(device, dtype, H, with_b, with_bias):
+    """g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b) of fla/layers/gated_deltanet.py:236-237,
+    forward and backward incl. the per-head parameter gradients; run twice for bit-equal gradients."""
+    from fla_amd.modules import gdn_gate
+    from oracle.modules import gdn_gate as ref_gate
+    gen = torch.Generator().manual_seed(H)
+    a = (torch.randn(3, 211, H, generator=gen) * 4).to(dtype)
+    a[0, 0, 0], a[0, 0, 1] = 35.0, -60.0
+    b = (torch.randn(3, 211, H, generator=gen) * 2).to(dtype) if with_b else None
+    A_log = torch.randn(H, generator=gen)
+    dt_bias = torch.randn(H, generator=gen) if with_bias else None
+    dg = torch.randn(3, 211, H, generator=gen)
+    dbeta = torch.randn(3, 211, H, generator=gen).to(dtype) if with_b else None
+    print(f"gdn_gate {dtype} H={H} b={with_b} bias={with_bias}", flush=True)
+
+    def run():
+        leaves = [t.to(device).requires_grad_() if t is not None else None for t in (a, b, A_log, dt_bias)]
+        g, beta = gdn_gate(*leaves)
+        outs, grads = [g], [dg.to(device)]
+        if with_b:
+            outs.append(beta)
+            grads.append(dbeta.to(device))
+        torch.autograd.backward(outs, grads)
+        return g, beta, [None if t is None else t.grad for t in leaves]
+
+    g, beta, grads = run()
+    _, _, grads2 = run()
+    for x, y in zip(grads, grads2):
+        assert (x is None and y is None) or torch.equal(x, y)
+    leaves = [t.double().requires_grad_() if t is not None else None for t in (a, b, A_log, dt_bias)]
+    gr, br = ref_gate(*leaves, dtype=torch.float64)
+    outs, gs = [gr], [dg.double()]
+    if with_b:
+        outs.append(br)
+        gs.append(dbeta.double())
+    torch.autograd.backward(outs, gs)
+    ft, bt = _tols(dtype)
+    assert g.dtype == torch.float32
+    assert_close("g", gr, g, 1e-5)
+    if with_b:
+        assert beta.dtype == dtype
+        assert_close("beta", br, beta, ft)
+        assert_close("db", leaves[1].grad, grads[1], bt)
+    assert_close("da", leaves[0].grad, grads[0], bt)
+    assert_close("dA_log", leaves[2].grad, grads[2], 1e-4)
+    if with_bias:
+        assert_close("ddt_bias", leaves[3].grad, grads[3], 1e-4)

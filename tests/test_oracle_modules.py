@@ -4,7 +4,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from oracle.modules import causal_conv1d, causal_conv1d_step, l2norm, norm_swish_gate
+from oracle.modules import causal_conv1d, causal_conv1d_step, gdn_gate, gla_gate, l2norm, norm_swish_gate
 
 
 def test_l2norm_unit_norm_and_scale_invariance():
@@ -82,3 +82,39 @@ def test_causal_conv1d_step_matches_full_convolution():
         y, cache = causal_conv1d_step(x[:, t], cache, w, b, "silu", dtype=torch.float64)
         torch.testing.assert_close(y, full[:, t])
     torch.testing.assert_close(cache, x[:, -W:].transpose(1, 2))
+
+
+@pytest.mark.parametrize("normalizer", [16.0, 1.0, 0.05])
+def test_gla_gate_against_library(normalizer):
+    gen = torch.Generator().manual_seed(7)
+    x = torch.cat([torch.randn(4, 33, generator=gen, dtype=torch.float64) * 3,
+                   torch.tensor([[-800.0, -40.0, 0.0, 40.0, 800.0] + [0.5] * 28], dtype=torch.float64)])
+    ref = F.logsigmoid(x) / normalizer
+    torch.testing.assert_close(gla_gate(x, normalizer, dtype=torch.float64), ref)
+    # a gate is a log-probability: never positive, 0 only in the limit, log(1/2)/normalizer at 0
+    assert gla_gate(x, normalizer, dtype=torch.float64).max() <= 0
+    torch.testing.assert_close(gla_gate(torch.zeros(1, dtype=torch.float64), normalizer, dtype=torch.float64),
+                               torch.tensor([-0.6931471805599453 / normalizer], dtype=torch.float64))
+    torch.testing.assert_close(gla_gate(x, normalizer, clamp_min=-0.3, dtype=torch.float64), ref.clamp_min(-0.3))
+    # and its derivative: sigmoid(-x) / normalizer where the clamp is open, 0 where it binds
+    xg = x.clone().requires_grad_()
+    gla_gate(xg, normalizer, clamp_min=-0.3, dtype=torch.float64).sum().backward()
+    want = torch.sigmoid(-x) / normalizer * (ref >= -0.3)
+    torch.testing.assert_close(xg.grad, want)
+
+
+def test_gdn_gate_against_library():
+    gen = torch.Generator().manual_seed(8)
+    H = 6
+    a = torch.randn(3, 17, H, generator=gen, dtype=torch.float64) * 4
+    a[0, 0, 0], a[0, 0, 1] = 35.0, -60.0          # either side of softplus' linear switch
+    b = torch.randn(3, 17, H, generator=gen, dtype=torch.float64) * 3
+    A_log = torch.randn(H, generator=gen, dtype=torch.float64)
+    dt_bias = torch.randn(H, generator=gen, dtype=torch.float64)
+    g, beta = gdn_gate(a, b, A_log, dt_bias, dtype=torch.float64)
+    torch.testing.assert_close(g, -A_log.exp() * F.softplus(a + dt_bias))
+    torch.testing.assert_close(beta, torch.sigmoid(b))
+    assert g.max() <= 0 and 0 <= beta.min() and beta.max() <= 1
+    g2, none = gdn_gate(a, None, A_log, None, dtype=torch.float64)
+    assert none is None
+    torch.testing.assert_close(g2, -A_log.exp() * F.softplus(a))
