@@ -607,6 +607,58 @@ def bench_simple_gla(device, steps=20):
             "fwd_bwd_B4_us": round(us_fb, 1), "fwd_bwd_B4_through_per_key_gate_kernels_us": round(us_fb_b, 1)}
 
 
+def bench_layer_fusion(device, steps=20):
+    """What folding the steps in front of the operators into their forward launches saves inside a layer, at the
+    headline shape (B=8, T=4096, H=16, D=128, nothing differentiated): the gate pre-activation of a GLA layer
+    (logsigmoid(x)/16 on the bf16 output of the gate projection, fla/layers/gla.py:214) and the l2 norm of q and k of
+    a gated DeltaNet layer (fla/layers/gated_deltanet.py:234-235), as separate launches in front of the operator
+    against the opt-in forms in which the operator's own launches do that work."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.modules import gla_gate_fwd, l2norm_fwd
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from fla_amd.ops.gla import chunk_gla
+    B, T, H, D = 8, 4096, 16, 128
+    gen = torch.Generator(device=device).manual_seed(7)
+    q, k, v = (torch.randn(B, T, H, D, device=device, generator=gen).bfloat16() for _ in range(3))
+    x = torch.randn(B, T, H, D, device=device, generator=gen).bfloat16()
+    h0 = torch.randn(B, H, D, D, device=device, generator=gen) * 0.1
+    g = F.logsigmoid(torch.randn(B, T, H, device=device, generator=gen))
+    beta = torch.randn(B, T, H, device=device, generator=gen).sigmoid()
+    nb = q.numel() * 2
+    out = {}
+
+    def gla_two_step():
+        return chunk_gla(q, k, v, gla_gate_fwd(x, 16.0), initial_state=h0, output_final_state=True, head_first=False)
+
+    def gla_fused():
+        return chunk_gla(q, k, v, x, initial_state=h0, output_final_state=True, head_first=False,
+                         gate_logit_normalizer=16.0)
+
+    def gdr_two_step():
+        return chunk_gated_delta_rule(l2norm_fwd(q), l2norm_fwd(k), v, g, beta, initial_state=h0,
+                                      output_final_state=True, head_first=False)
+
+    def gdr_fused():
+        return chunk_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True, head_first=False,
+                                      use_qk_l2norm_in_kernel=True)
+
+    with torch.no_grad():
+        a, b = event_avg_us(gla_two_step, steps), event_avg_us(gla_fused, steps)
+        gate = event_avg_us(lambda: gla_gate_fwd(x, 16.0), steps)
+        out["gla_gate_logsigmoid"] = {
+            "separate_launches_us": round(a, 1), "gate_launch_alone_us": round(gate, 1), "in_kernel_us": round(b, 1),
+            "saved_us": round(a - b, 1),
+            # logits in (bf16) + fp32 gates out, then the operator on fp32 gates / the operator on the bf16 logits
+            "bytes_separate": 7 * nb + 2 * nb + 2 * h0.numel() * 4, "bytes_in_kernel": 5 * nb + 2 * h0.numel() * 4}
+        a, b = event_avg_us(gdr_two_step, steps), event_avg_us(gdr_fused, steps)
+        out["gdr_qk_l2norm"] = {
+            "separate_launches_us": round(a, 1), "in_kernel_us": round(b, 1), "saved_us": round(a - b, 1),
+            # two norms (read + write each), then the operator / the operator alone
+            "bytes_separate": 8 * nb + 2 * h0.numel() * 4, "bytes_in_kernel": 4 * nb + 2 * h0.numel() * 4}
+    return out
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -667,6 +719,7 @@ def main():
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
         extra["layer_steps"] = bench_layer_steps(device)
+        extra["layer_fusion"] = bench_layer_fusion(device)
         extra["chunk_simple_gla_fwd"] = bench_simple_gla(device)
         extra["gla_stages_reference_operands"] = bench_gla_stages(device)
         extra["device_copy_1GiB"] = bench_copy(device)

@@ -123,6 +123,35 @@ FLA_DEVICE float row_suffix16(float x) {
   return x;
 }
 
+// Sum over an aligned group of N (8 or 16) consecutive lanes, result in every lane of the group: two
+// exchanges inside the quads, then the mirror images of the half row and the row (VALU only).
+template <int N>
+FLA_DEVICE float group_allsum(float x) {
+  static_assert(N == 8 || N == 16, "lanes per group");
+  x += dpp_f32<0xB1>(x);    // quad_perm [1,0,3,2]
+  x += dpp_f32<0x4E>(x);    // quad_perm [2,3,0,1]
+  x += dpp_f32<0x141>(x);   // row_half_mirror
+  if (N == 16) x += dpp_f32<0x140>(x);   // row_mirror
+  return x;
+}
+
+// A row of 8 * N elements is held by N adjacent lanes, 8 elements each: x / sqrt(sum x^2 + eps) of this lane's
+// piece, rounded to T (fla/modules/l2norm.py:18-40: eps inside the square root).
+template <typename T, int N>
+FLA_DEVICE typename Elem<T>::v8 l2norm_piece(typename Elem<T>::v8 x, float eps) {
+  float f[8], ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    f[i] = (float)x[i];
+    ss = fmaf(f[i], f[i], ss);
+  }
+  const float rstd = __builtin_amdgcn_rsqf(group_allsum<N>(ss) + eps);
+  typename Elem<T>::v8 y;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) y[i] = (T)(f[i] * rstd);
+  return y;
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a fence over
 // global memory as well: a wave with global stores in flight then drains its whole vector
 // memory queue (loads included) at every barrier, which exposes the full memory latency of

@@ -349,6 +349,7 @@ struct PrepParams {
   int H, NTfix;
   void* w;             // KEEP: w = Aw (beta k) [rows, H, K] and Aw [rows, H, 64], what the backward reads
   void* Aw;
+  float l2_eps;        // L2N: every k row is replaced by k / sqrt(sum k^2 + l2_eps) on its way in
 };
 
 // resident workgroups per CU (register budget): four, or three for the variant that also writes w and Aw
@@ -362,8 +363,11 @@ FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 // than bound by one resource).
 // KEEP: the forward of a pass that will be differentiated also leaves w = Aw (beta k) and Aw in memory (the WY
 // launch of the reference's decomposition, without a second inversion and a second pass over k).
-template <typename T, int K, bool KEEP>
+// L2N: k arrives un-normalised and is l2-normalised row by row as it is staged (what l2_norm(k) in front of the
+// operator does, fla/layers/gated_deltanet.py:235); a row of K elements sits in K / 8 adjacent lanes.
+template <typename T, int K, bool KEEP, bool L2N = false>
 __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
+  static_assert(!(KEEP && L2N), "a forward that keeps w and Aw takes normalised keys");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
@@ -464,7 +468,9 @@ __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
       const int row = r0 + RPP * i;
-      *(v8*)&sK[row * LDK + c8] = row < L ? cur.k[i] : z;
+      v8 kr = cur.k[i];
+      if constexpr (L2N) kr = l2norm_piece<T, K / 8>(kr, p.l2_eps);
+      *(v8*)&sK[row * LDK + c8] = row < L ? kr : z;
     }
     if (wave == 0) {
       const bool ok = lane < L;
@@ -1171,7 +1177,12 @@ int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
   const int64_t total = (int64_t)chunk_grid_.x * chunk_grid_.y;
   const int64_t resident = (p.w ? kPrepResidentKeep : kPrepResident) * kNumCUs;
   dim3 grid((unsigned)(total < resident ? total : resident));
-  if (p.w) {
+  if (p.l2_eps >= 0.f) {
+    if (p.w) return FLA_E_UNSUPPORTED;
+    if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64, false, true>), grid, dim3(256), 0, st, p, total);
+    else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128, false, true>), grid, dim3(256), 0, st, p, total);
+    else return FLA_E_UNSUPPORTED;
+  } else if (p.w) {
     if (K == 64) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 64, true>), grid, dim3(256), 0, st, p, total);
     else if (K == 128) hipLaunchKernelGGL((gdr_fwd_prep_kernel<T, 128, true>), grid, dim3(256), 0, st, p, total);
     else return FLA_E_UNSUPPORTED;
@@ -1186,10 +1197,10 @@ int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_cumsum,
-                                float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
-                                const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
-                                int64_t K, fla_stream_t stream) {
+static int gdr_fwd_prep_impl(const void* k, const float* beta, const float* g, int g_is_cumsum,
+                             float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
+                             const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                             int64_t K, float l2_eps, fla_stream_t stream) {
   FLA_REQUIRE(k && beta && AT, FLA_E_INVALID);
   FLA_REQUIRE((w == nullptr) == (Aw == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && NT >= 0, FLA_E_INVALID);
@@ -1199,10 +1210,27 @@ extern "C" int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  PrepParams p{k, beta, g, g_is_cumsum, g_cumsum_out, AT, offsets, indices, T, (int)H, ntfix, w, Aw};
+  PrepParams p{k, beta, g, g_is_cumsum, g_cumsum_out, AT, offsets, indices, T, (int)H, ntfix, w, Aw, l2_eps};
   if (qkv_dtype == FLA_BF16) return launch_prep<bf16>(p, (int)K, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_prep<f16>(p, (int)K, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g, int g_is_cumsum,
+                                float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
+                                const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                                int64_t K, fla_stream_t stream) {
+  return gdr_fwd_prep_impl(k, beta, g, g_is_cumsum, g_cumsum_out, AT, w, Aw, offsets, indices, NT, qkv_dtype, B, T,
+                           H, K, -1.f, stream);
+}
+
+extern "C" int fla_gdr_fwd_prep_l2norm(const void* k, const float* beta, const float* g, int g_is_cumsum,
+                                       float* g_cumsum_out, void* AT, const int64_t* offsets,
+                                       const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T,
+                                       int64_t H, int64_t K, float eps, fla_stream_t stream) {
+  FLA_REQUIRE(eps >= 0.f, FLA_E_INVALID);
+  return gdr_fwd_prep_impl(k, beta, g, g_is_cumsum, g_cumsum_out, AT, nullptr, nullptr, offsets, indices, NT,
+                           qkv_dtype, B, T, H, K, eps, stream);
 }
 
 extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum, void* w, void* u,

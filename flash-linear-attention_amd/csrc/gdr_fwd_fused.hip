@@ -60,6 +60,7 @@ struct GdrScanParams {
   int64_t T;
   int H, V, N;
   float scale;
+  float l2_eps;     // L2N: q and k rows are l2-normalised (x / sqrt(sum x^2 + l2_eps)) as they are staged
 };
 
 // Two 4-element results per lane (16-bit after conversion) -> one 8-element vector per lane: lanes 0-31 keep
@@ -96,9 +97,13 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
 // (64 columns) is the form described above; two (32 columns, waves 2-3 only keep the barriers) doubles the number of
 // workgroups where 64-column slabs would leave half the CUs without one - a CU is fed at a fixed rate, and a
 // 32-column workgroup needs three quarters of the bytes of a 64-column one per chunk.
-template <typename T, int K, bool KEEP, int NMW = 4>
+// L2N: q and k arrive un-normalised and the staging waves l2-normalise every row on its way to LDS (the two
+// l2_norm launches in front of the operator, fla/layers/gated_deltanet.py:234-235): a row is held by K / 8
+// adjacent lanes, so its sum of squares is four lane exchanges.
+template <typename T, int K, bool KEEP, int NMW = 4, bool L2N = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
+  static_assert(!(KEEP && L2N), "a forward that keeps its intermediates takes normalised q and k");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int BV = 16 * NMW;
@@ -289,6 +294,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           if (q_row(st + 256 * i) >= Llast)
 #pragma unroll
             for (int j = 0; j < 8; ++j) R.q[i][j] = R.k[i][j] = (T)0.f;
+      }
+      if constexpr (L2N) {
+#pragma unroll
+        for (int i = 0; i < NPW; ++i) {
+          R.q[i] = l2norm_piece<T, K / 8>(R.q[i], p.l2_eps);
+          R.k[i] = l2norm_piece<T, K / 8>(R.k[i], p.l2_eps);
+        }
       }
 #pragma unroll
       for (int i = 0; i < NPW; ++i) *(v8*)&sQ[wq3][dq[i]] = R.q[i];
@@ -638,24 +650,33 @@ int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
 #define FLA_SCAN(KK, KEEPV)                                                                              \
   if (narrow) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 2>), grid, block, 0, st, p);          \
   else hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 4>), grid, block, 0, st, p);
+#define FLA_SCAN_L2N(KK)                                                                                 \
+  if (narrow) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, false, 2, true>), grid, block, 0, st, p);    \
+  else hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, false, 4, true>), grid, block, 0, st, p);
+  if (p.l2_eps >= 0.f) {
+    if (keep) return FLA_E_UNSUPPORTED;
+    if (K == 64) { FLA_SCAN_L2N(64) }
+    else if (K == 128) { FLA_SCAN_L2N(128) }
+    else return FLA_E_UNSUPPORTED;
+  } else
   if (K == 64 && keep) { FLA_SCAN(64, true) }
   else if (K == 64) { FLA_SCAN(64, false) }
   else if (K == 128 && keep) { FLA_SCAN(128, true) }
   else if (K == 128) { FLA_SCAN(128, false) }
   else return FLA_E_UNSUPPORTED;
 #undef FLA_SCAN
+#undef FLA_SCAN_L2N
   FLA_CHECK_LAUNCH();
   return FLA_OK;
 }
 
 }  // namespace
 
-extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
-                                                   const float* g_cumsum, const float* h0, void* o, float* ht,
-                                                   void* v_new, void* h_frag_t, void* Aqk_out, const int64_t* offsets, const int64_t* chunk_offsets,
-                                                   const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
-                                                   int64_t H, int64_t K, int64_t V, int64_t N, float scale,
-                                                   fla_stream_t stream) {
+static int gdr_fwd_scan_impl(const void* q, const void* k, const void* v, const void* AT, const float* g_cumsum,
+                             const float* h0, void* o, float* ht, void* v_new, void* h_frag_t, void* Aqk_out,
+                             const int64_t* offsets, const int64_t* chunk_offsets, const int64_t* seq_order,
+                             int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                             float scale, float l2_eps, fla_stream_t stream) {
   FLA_REQUIRE(q && k && v && AT && o, FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
@@ -664,8 +685,30 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k,
   FLA_REQUIRE(Aqk_out == nullptr || v_new != nullptr, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o | (uintptr_t)v_new |
                (uintptr_t)h_frag_t | (uintptr_t)Aqk_out) % 16 == 0, FLA_E_ALIGNMENT);
-  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets, seq_order, T, (int)H, (int)V, (int)N, scale};
+  GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets, seq_order, T,
+                  (int)H, (int)V, (int)N, scale, l2_eps};
   if (qkv_dtype == FLA_BF16) return launch_scan<bf16>(p, (int)K, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_scan<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
+}
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void* v, const void* AT,
+                                                   const float* g_cumsum, const float* h0, void* o, float* ht,
+                                                   void* v_new, void* h_frag_t, void* Aqk_out, const int64_t* offsets, const int64_t* chunk_offsets,
+                                                   const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
+                                                   int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                                   fla_stream_t stream) {
+  return gdr_fwd_scan_impl(q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets,
+                           seq_order, qkv_dtype, B, T, H, K, V, N, scale, -1.f, stream);
+}
+
+extern "C" int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const void* k, const void* v, const void* AT,
+                                                          const float* g_cumsum, const float* h0, void* o, float* ht,
+                                                          const int64_t* offsets, const int64_t* chunk_offsets,
+                                                          const int64_t* seq_order, int qkv_dtype, int64_t B,
+                                                          int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                                          float scale, float eps, fla_stream_t stream) {
+  FLA_REQUIRE(eps >= 0.f, FLA_E_INVALID);
+  return gdr_fwd_scan_impl(q, k, v, AT, g_cumsum, h0, o, ht, nullptr, nullptr, nullptr, offsets, chunk_offsets,
+                           seq_order, qkv_dtype, B, T, H, K, V, N, scale, eps, stream);
 }

@@ -26,7 +26,22 @@ struct FusedParams {
   float* decay;     //   and e^{G_last} of every chunk, [chunks, H, K] (both or neither)
   void* kh_t;       // with qg, optional: k^ = k e^{G_last - G} per chunk as staged, [chunks, H, K, 64] (key-major) ...
   void* scores;     //   ... and the chunk's causal score tile tril(q~ k~^T), [chunks, H, 64, 64] (both or neither)
+  // LOGITS form: p.g holds the gate projection's output x and the log-gate is max(logsigmoid(x) * gate_inv_norm,
+  // gate_clamp_min) (fla/layers/gla.py:214-217), formed by the staging waves on the way to the prefix sums
+  float gate_inv_norm;
+  float gate_clamp_min;   // -inf: no clamp
 };
+
+// log2(sigmoid(x)) * inv_norm, clamped from below at clamp2 (both in the log2 domain): two transcendental
+// instructions per element.  log2(1 + e) keeps an absolute error of 1e-7, far below what a log-gate needs;
+// x = +inf gives exactly 0 (the value rows past the end of a short chunk are set to).
+FLA_DEVICE float log2_sigmoid_gate(float x, float inv_norm, float clamp2) {
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float t = x * LOG2E;
+  const float e = __builtin_amdgcn_exp2f(-fabsf(t));
+  const float l = __builtin_amdgcn_logf(1.f + e);
+  return fmaxf((fminf(t, 0.f) - l) * inv_norm, clamp2);
+}
 
 // The row-major q~ / k~ tiles are written by lanes that own four adjacent rows each, i.e.
 // with a row stride of four between neighbouring lanes (64 bytes modulo 256: measured 2.5x
@@ -71,7 +86,7 @@ struct StageLds {
 // (left in L.o by the matrix waves) to memory as whole rows, and one more barrier + store follows the last chunk.
 // SG: one log-gate per (token, head), p.g is fp32 [B*T, H]: a lane loads one word per row and uses it for all
 // its key channels, so the prefix sums and exponentials of a row are formed once.
-template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O, int BV = 64>
+template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O, int BV = 64, bool LOGITS = false>
 FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, const SeqSpan& sp, int64_t nchunks,
                                 int hh, int vbase, int wave, int lane, int tid) {
   typedef typename Elem<T>::v8 v8;
@@ -160,7 +175,7 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
         if (rg * RPT + i >= L) {
 #pragma unroll
           for (int j = 0; j < CPL; ++j) {
-            R.g[i][j] = (GT)0.f;
+            R.g[i][j] = LOGITS ? (GT)INFINITY : (GT)0.f;   // a log-gate of exactly zero either way
             R.q[i][j] = (T)0.f;
             R.k[i][j] = (T)0.f;
           }
@@ -183,6 +198,7 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
     begin_loads();
     float G[RPT][CPL], glast[CPL];
     float gabs = 0.f;
+    [[maybe_unused]] const float clamp2 = p.gate_clamp_min * LOG2E;
     if constexpr (SG) {
       // one gate per row: a single prefix sum, shared by all key channels of the lane (the
       // exponentials below then collapse to one pair per row)
@@ -212,7 +228,8 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
       float run = 0.f;
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
-        run = fmaf((float)R.g[i][j], LOG2E, run);   // prefix sums in the log2 domain
+        if constexpr (LOGITS) run += log2_sigmoid_gate((float)R.g[i][j], p.gate_inv_norm, clamp2);
+        else run = fmaf((float)R.g[i][j], LOG2E, run);   // prefix sums in the log2 domain
         G[i][j] = run;
       }
       const float pre = row_prefix16(run);

@@ -35,9 +35,11 @@ namespace {
 // the matrix waves with cw = 1 only form their score quadrant) doubles the number of workgroups where 64-column slabs
 // would leave half the CUs without one: a CU is fed at a fixed rate, and a 32-column workgroup needs five sixths of
 // the bytes of a 64-column one per chunk (three quarters when it also writes the states).
-template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false, int NVT = 2>
+// LOGITS: p.g holds gate logits; the staging waves apply logsigmoid / normalizer (and the clamp) themselves.
+template <typename T, typename GT, int K, int NSTG, bool HT, bool SG = false, int NVT = 2, bool LOGITS = false>
 __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedParams p) {
   static_assert(!SG || sizeof(GT) == 4, "per-head gates are fp32");
+  static_assert(!LOGITS || (!SG && !HT), "gate logits: per-key gates, forward without kept states");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   typedef T t2 __attribute__((ext_vector_type(2)));
@@ -81,7 +83,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
   if (wave >= 4) {
     // staging waves: see gla_fused_staging.h
     StageLds<T> L{{sQ[0], sQ[1]}, {sK[0], sK[1]}, {sKh[0], sKh[1]}, {sDecay[0], sDecay[1]}, {sWide[0], sWide[1]}, sO};
-    gla_stage_waves<T, GT, K, NSTG, SG, true, BV>(p, L, sp, nchunks, hh, vbase, wave, lane, tid);
+    gla_stage_waves<T, GT, K, NSTG, SG, true, BV, LOGITS>(p, L, sp, nchunks, hh, vbase, wave, lane, tid);
   } else {
     // =========================== matrix waves ===========================
     const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
@@ -408,6 +410,8 @@ struct ExactParams {
   int64_t total;   // (chunk, head) pairs
   int head_gates;  // g is fp32 [B*T, H]: one log-gate per (token, head)
   int hwide_vk;    // hwide holds [V][K] tiles (the 128-column kernel) instead of fragment-order ones
+  int gate_logits; // g holds gate logits: the log-gate is max(logsigmoid(g) * gate_inv_norm, gate_clamp_min)
+  float gate_inv_norm, gate_clamp_min;
 };
 
 template <typename T, typename GT, int K, int V>
@@ -457,6 +461,12 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
         for (int j = 0; j < 4; ++j) gq[i][j] = x;
       } else {
         Load<GT>::x4((const GT*)p.g + off, gq[i]);
+        if (p.gate_logits) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            gq[i][j] = log2_sigmoid_gate(gq[i][j], p.gate_inv_norm, p.gate_clamp_min * 1.4426950408889634f) *
+                       0.6931471805599453f;
+        }
       }
       qreg[i] = *(const v4*)((const T*)p.q + off);
       kreg[i] = *(const v4*)((const T*)p.k + off);
@@ -601,10 +611,21 @@ inline bool use_wide_kernel(const FusedParams& p, int K) {
 }
 
 template <typename T, typename GT, bool SG = false>
-int launch_fused(const FusedParams& p, int K, hipStream_t st) {
+int launch_fused(const FusedParams& p, int K, hipStream_t st, bool logits = false) {
   int64_t total = (int64_t)(p.V / 64) * p.N * p.H;
   if (total == 0) return FLA_OK;
   FLA_REQUIRE(total <= 0x7fffffffLL, FLA_E_UNSUPPORTED);
+  if constexpr (!SG) {
+    if (logits) {
+      FLA_REQUIRE(!p.hT, FLA_E_UNSUPPORTED);
+      dim3 grid((unsigned)total);
+      if (K == 128) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 128, 4, false, false, 2, true>), grid, dim3(512), 0, st, p);
+      else if (K == 64) hipLaunchKernelGGL((gla_fwd_fused_kernel<T, GT, 64, 4, false, false, 2, true>), grid, dim3(512), 0, st, p);
+      else return FLA_E_UNSUPPORTED;
+      FLA_CHECK_LAUNCH();
+      return FLA_OK;
+    }
+  }
   if (use_wide_kernel(p, K)) {
     hipLaunchKernelGGL((gla_fwd_fused_wide_kernel<T, GT, SG>), dim3((unsigned)(p.N * p.H)), dim3(512), 0, st, p);
     FLA_CHECK_LAUNCH();
@@ -641,8 +662,10 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
                               const int64_t* indices, const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                               int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H, int64_t K,
                               int64_t V, int64_t N, float scale, fla_stream_t stream, bool head_gates = false,
-                              bool exact_pass = true, void* kh_t = nullptr, void* scores = nullptr) {
+                              bool exact_pass = true, void* kh_t = nullptr, void* scores = nullptr,
+                              bool logits = false, float gate_inv_norm = 1.f, float gate_clamp_min = -INFINITY) {
   FLA_REQUIRE(q && k && v && gates && o, FLA_E_INVALID);
+  if (logits) FLA_REQUIRE(!head_gates && !h_frag_t, FLA_E_UNSUPPORTED);
   if (head_gates) FLA_REQUIRE(gate_dtype == FLA_F32, FLA_E_UNSUPPORTED);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE((K == 64 || K == 128) && V % 64 == 0 && V <= 1024, FLA_E_UNSUPPORTED);
@@ -668,7 +691,7 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     FLA_REQUIRE(((uintptr_t)kh_t | (uintptr_t)scores) % 16 == 0, FLA_E_ALIGNMENT);
   }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
-                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay, kh_t, scores};
+                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay, kh_t, scores, gate_inv_norm, gate_clamp_min};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;
@@ -677,11 +700,12 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     if (rc) return rc;
   }
   ExactParams e{q, k, v, gates, ws_wide, ws_hwide, o, offsets, indices, T, (int)H, ntfix, scale,
-                (int64_t)grid.x * grid.y, head_gates ? 1 : 0, use_wide_kernel(p, (int)K) ? 1 : 0};
+                (int64_t)grid.x * grid.y, head_gates ? 1 : 0, (!logits && use_wide_kernel(p, (int)K)) ? 1 : 0,
+                logits ? 1 : 0, gate_inv_norm, gate_clamp_min};
   if (ws_wide) grid = dim3((unsigned)(e.total < 512 ? e.total : 512));
 #define FLA_FUSED(TT, GG)                                                \
   {                                                                      \
-    int rc = launch_fused<TT, GG>(p, (int)K, st);                        \
+    int rc = launch_fused<TT, GG>(p, (int)K, st, logits);                \
     if (rc || !ws_wide || grid.x == 0 || !exact_pass) return rc;         \
     return launch_exact<TT, GG>(e, (int)K, (int)V, grid, st);            \
   }
@@ -759,4 +783,18 @@ extern "C" int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, cons
                                               int64_t N, float scale, fla_stream_t stream) {
   return gla_fwd_fused_impl(q, k, v, g, h0, o, ht, ws_wide, ws_hwide, h_frag_t, q_gated, chunk_decay, offsets, indices, chunk_offsets,
                             seq_order, NT, qkv_dtype, FLA_F32, B, T, H, K, V, N, scale, stream, true, true, khat_t, scores);
+}
+
+extern "C" int fla_chunk_gla_fwd_fused_logits(const void* q, const void* k, const void* v, const void* gate_logits,
+                                              const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                              const int64_t* offsets, const int64_t* indices,
+                                              const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
+                                              int qkv_dtype, int gate_dtype, int64_t B, int64_t T, int64_t H,
+                                              int64_t K, int64_t V, int64_t N, float scale, float normalizer,
+                                              int has_clamp, float clamp_min, fla_stream_t stream) {
+  FLA_REQUIRE(normalizer != 0.f, FLA_E_INVALID);
+  return gla_fwd_fused_impl(q, k, v, gate_logits, h0, o, ht, ws_wide, ws_hwide, nullptr, nullptr, nullptr, offsets,
+                            indices, chunk_offsets, seq_order, NT, qkv_dtype, gate_dtype, B, T, H, K, V, N, scale,
+                            stream, false, true, nullptr, nullptr, true, 1.f / normalizer,
+                            has_clamp ? clamp_min : -INFINITY);
 }

@@ -120,6 +120,7 @@ def chunk_gated_delta_rule_fwd_scan(
     seq_order: Optional[torch.Tensor] = None,
     *,
     keep: bool = False,
+    l2norm_eps: Optional[float] = None,
 ):
     """Serial half of the one-pass forward (``fla_chunk_gated_delta_rule_fwd_scan``): the work of
     ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o`` (``fla/ops/gated_delta_rule/chunk.py:47-72``)
@@ -127,7 +128,9 @@ def chunk_gated_delta_rule_fwd_scan(
     v_new nor the per-chunk states are materialised.  ``g`` is the fp32 chunk-local cumsum.  Seq-first.
     Returns ``(o, final_state)``; with ``keep`` also ``v_new``, the state entering every chunk in
     transposed-fragment order (``[B, NT, H, K, V]``) and the packed score tiles ``Aqk``
-    (``[chunks, H, 10, 16, 16]``), what the backward reads: ``(o, final_state, v_new, hT, Aqk)``."""
+    (``[chunks, H, 10, 16, 16]``), what the backward reads: ``(o, final_state, v_new, hT, Aqk)``.
+    ``l2norm_eps``: ``q`` and ``k`` are un-normalised and the launch l2-normalises their rows as it stages them
+    (``fla_chunk_gated_delta_rule_fwd_scan_l2norm``; not with ``keep``)."""
     be.require_gpu(q, k, v, AT)
     B, T, H, K = k.shape
     V = v.shape[-1]
@@ -147,6 +150,14 @@ def chunk_gated_delta_rule_fwd_scan(
         v_new = torch.empty_like(v)
         hT = k.new_empty(B, AT.shape[0] // B if offsets is None else AT.shape[0], H, K, V)
         Aqk = torch.empty_like(AT)
+    if l2norm_eps is not None:
+        if keep:
+            raise ValueError("l2norm_eps: forward without kept intermediates only")
+        be.check(be.lib().fla_chunk_gated_delta_rule_fwd_scan_l2norm(
+            be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht),
+            be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale),
+            float(l2norm_eps), be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan_l2norm")
+        return o, ht
     be.check(be.lib().fla_chunk_gated_delta_rule_fwd_scan(
         be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(v_new),
         be.ptr(hT), be.ptr(Aqk), be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N,

@@ -48,11 +48,13 @@ def _round_k(d: int) -> int:
 
 def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
                                offsets=None, indices=None, head_first=True, chunk_size=64,
-                               *, plan: Optional[VarlenPlan] = None, store_A: bool = True, fused: bool = True):
+                               *, plan: Optional[VarlenPlan] = None, store_A: bool = True, fused: bool = True,
+                               l2norm_eps: Optional[float] = None):
     """Reference-shaped forward (``fla/ops/gated_delta_rule/chunk.py:20-73``): returns
     ``(g_cumsum, o, Aw, Au, final_state)``.  ``fused=False`` runs the reference's steps one by one
     (cumsum, WY representation, state scan, output stage); the default two-launch form does not form
-    ``Aw`` / ``Au`` and returns ``None`` for them."""
+    ``Aw`` / ``Au`` and returns ``None`` for them.  ``l2norm_eps`` (two-launch form only): ``q`` and ``k`` are
+    un-normalised and both launches l2-normalise the rows as they stage them."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd: seq-first, chunk size 64 only")
     if offsets is not None and plan is None:
@@ -62,11 +64,14 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     co = None if plan is None else plan.chunk_offsets
     if fused:
         # two launches; Aw / Au are not formed on this path
-        AT, g = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx)
+        AT, g = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, l2norm_eps=l2norm_eps)
         o, final_state = chunk_gated_delta_rule_fwd_scan(q, k, v, AT, g, scale, initial_state, output_final_state,
                                                          offsets=offs, chunk_offsets=co,
-                                                         seq_order=None if plan is None else plan.seq_order)
+                                                         seq_order=None if plan is None else plan.seq_order,
+                                                         l2norm_eps=l2norm_eps)
         return g, o, None, None, final_state
+    if l2norm_eps is not None:
+        raise ValueError("l2norm_eps needs the two-launch form")
     g = None if g is None else chunk_local_cumsum(g, BT, offsets=offs, indices=idx, head_first=False)
     w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, g, offsets=offs, indices=idx, head_first=False, chunk_size=BT,
                                        store_A=store_A)
@@ -279,6 +284,7 @@ def chunk_gated_delta_rule(
     offsets: Optional[torch.LongTensor] = None,
     head_first: bool = True,
     cu_seqlens: Optional[torch.LongTensor] = None,
+    use_qk_l2norm_in_kernel: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     r"""
     Args:
@@ -289,6 +295,10 @@ def chunk_gated_delta_rule(
         scale: default ``K ** -0.5``; must be positive.
         initial_state: ``[N, H, K, V]`` or ``None``; output_final_state: return the fp32 final state.
         offsets (synonym ``cu_seqlens``): int64 ``[N+1]`` boundaries of a packed batch (batch 1, seq-first).
+        use_qk_l2norm_in_kernel (extension, default off): ``q`` and ``k`` are un-normalised and the operator
+            applies ``l2_norm`` (eps 1e-6, ``fla/modules/l2norm.py``) to both, as the layer does in front of it
+            (``fla/layers/gated_deltanet.py:234-235``).  A forward that is not differentiated normalises the rows
+            inside its two launches; otherwise the stand-alone ``l2_norm`` runs first, with its backward.
 
     Returns ``(o, final_state)``.
     """
@@ -303,9 +313,14 @@ def chunk_gated_delta_rule(
         assert scale > 0, "Scale must be positive."
     if q.numel() == 0:
         return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
-    if _direct_launch_ok(q, k, v, g, beta, initial_state, head_first):
+    direct = _direct_launch_ok(q, k, v, g, beta, initial_state, head_first)
+    if use_qk_l2norm_in_kernel and not direct:
+        from ...modules.l2norm import l2_norm
+        q, k = l2_norm(q), l2_norm(k)
+    if direct:
         # nothing to differentiate and nothing to convert: no autograd node, no copies
         _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
-                                                    offsets=offsets, head_first=False, chunk_size=BT, store_A=False)
+                                                    offsets=offsets, head_first=False, chunk_size=BT, store_A=False,
+                                                    l2norm_eps=1e-6 if use_qk_l2norm_in_kernel else None)
         return o, ht
     return apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first)

@@ -60,6 +60,7 @@ def fwd_prepare_scan_operands(
     indices: Optional[torch.Tensor] = None,
     g_is_cumsum: bool = False,
     keep_w: bool = False,
+    l2norm_eps: Optional[float] = None,
 ):
     """Chunk-parallel half of the one-pass forward (``fla_gdr_fwd_prep``): the work of ``chunk_local_cumsum``
     and ``fwd_prepare_wy_repr`` (``fla/ops/gated_delta_rule/wy_fast.py:320-376``), leaving per (chunk, head) the
@@ -68,7 +69,8 @@ def fwd_prepare_scan_operands(
     ``[B, T, H]`` (or its chunk-local cumsum with ``g_is_cumsum``; ``None`` for the un-gated rule).
     Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``; with ``keep_w`` the launch also writes
     ``w = Aw (beta k)`` and ``Aw`` (what ``fwd_prepare_wy_repr`` leaves for the backward) and the return value
-    is ``(AT, g_cumsum, w, Aw)``."""
+    is ``(AT, g_cumsum, w, Aw)``.  ``l2norm_eps``: ``k`` is un-normalised and the launch l2-normalises its rows
+    as it stages them (``fla_gdr_fwd_prep_l2norm``; not with ``keep_w``)."""
     be.require_gpu(k, beta)
     B, T, H, K = k.shape
     NT = 0
@@ -84,6 +86,14 @@ def fwd_prepare_scan_operands(
     AT = k.new_empty(chunks, H, TRI_BLOCKS, 16, 16)
     w = torch.empty_like(k) if keep_w else None
     Aw = k.new_empty(B, T, H, BT) if keep_w else None
+    if l2norm_eps is not None:
+        if keep_w:
+            raise ValueError("l2norm_eps: forward without kept intermediates only")
+        be.check(be.lib().fla_gdr_fwd_prep_l2norm(
+            be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc), be.ptr(AT),
+            be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, float(l2norm_eps), be.stream_of(k)),
+            "fla_gdr_fwd_prep_l2norm")
+        return AT, gc
     be.check(be.lib().fla_gdr_fwd_prep(
         be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
         be.ptr(AT), be.ptr(w), be.ptr(Aw), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K,

@@ -185,7 +185,8 @@ def _guard_workspaces(q, chunks, H, KV, keep):
 
 
 def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, offsets=None, exact_guard=True,
-                        return_flags=False, states_out=None, head_gates=False, first_launch_only=False):
+                        return_flags=False, states_out=None, head_gates=False, first_launch_only=False,
+                        gate_logits=None):
     """Forward through ``fla_chunk_gla_fwd_fused``: seq-first, K in {64,128}, V % 64 == 0.
     With ``exact_guard`` (needs V <= 128) chunks whose cumulative log-gate leaves the
     single-reference range are detected on the device and recomputed exactly; ``return_flags``
@@ -194,7 +195,9 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
     order, what the backward kernels read) and appends it, followed (per-key gates only) by the gated queries
     ``q e^{G}`` ``[B,T,H,K]`` and the chunk decays ``e^{G_last}`` ``[chunks,H,K]`` the backward's reverse state scan
     streams (``fla_chunk_gla_fwd_fused_kept``).  ``head_gates``: ``g`` is one fp32 log-gate
-    per (token, head), ``[B,T,H]`` (``fla_chunk_simple_gla_fwd_fused``)."""
+    per (token, head), ``[B,T,H]`` (``fla_chunk_simple_gla_fwd_fused``).  ``gate_logits = (normalizer, clamp_min)``:
+    ``g`` is the gate projection's output and the kernel forms ``logsigmoid(g) / normalizer`` (clamped from below
+    unless ``clamp_min`` is None) itself (``fla_chunk_gla_fwd_fused_logits``; no kept states, per-key gates)."""
     B, T, H, K = q.shape
     V = v.shape[-1]
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
@@ -213,7 +216,14 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
             0 if plan is None else plan.NT,
             be.dt(q), be.dt(g), B, T, H, K, V, N, float(scale), be.stream_of(q))
     head = (be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(wide), be.ptr(hwide))
-    if head_gates:
+    if gate_logits is not None:
+        if head_gates or states_out is not None or first_launch_only:
+            raise ValueError("gate logits: per-key gates, forward without kept states")
+        normalizer, clamp_min = gate_logits
+        be.check(be.lib().fla_chunk_gla_fwd_fused_logits(*head, *tail[:-1], float(normalizer), int(clamp_min is not None),
+                                                         float(clamp_min or 0.0), tail[-1]),
+                 "fla_chunk_gla_fwd_fused_logits")
+    elif head_gates:
         if g.dtype != torch.float32 or g.shape != q.shape[:3]:
             raise ValueError("head gates must be fp32 [B, T, H]")
         hT = qg = decay = kh = sc = None
@@ -559,6 +569,8 @@ def chunk_gla(
     offsets: Optional[torch.LongTensor] = None,
     head_first: bool = True,
     cu_seqlens: Optional[torch.LongTensor] = None,
+    gate_logit_normalizer: Optional[float] = None,
+    gate_clamp_min: Optional[float] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     r"""
     Args:
@@ -571,10 +583,25 @@ def chunk_gla(
         offsets (synonym ``cu_seqlens``): int64 ``[N+1]`` sequence boundaries of a
             packed batch (batch size 1, seq-first only).
         head_first: layout switch; seq-first is the native layout.
+        gate_logit_normalizer (extension, default off): when given, ``g`` is the output of the layer's gate
+            projection and the log-gates are ``logsigmoid(g) / gate_logit_normalizer``, clamped from below at
+            ``gate_clamp_min`` if that is given (``fla/layers/gla.py:214-217``).  A forward that is not
+            differentiated applies that inside the fused launch (no fp32 gate tensor is written or read);
+            otherwise it is one elementwise launch in front of the operator, with its backward.
 
     Returns ``(o, final_state)``.
     """
     offsets = resolve_offsets(offsets, cu_seqlens)
+    if gate_logit_normalizer is not None:
+        from ...modules.gate_activations import gla_gate
+        if (q.numel() and q.dtype != torch.float32 and q.shape[-1] in (64, 128) and v.shape[-1] <= 128
+                and _direct_launch_ok(q, k, v, g, initial_state, head_first)):
+            check_varlen_args(q, offsets, head_first, initial_state)
+            return chunk_gla_fwd_fused(q, k, v, g, q.shape[-1] ** -0.5 if scale is None else scale, initial_state,
+                                       output_final_state, offsets,
+                                       gate_logits=(gate_logit_normalizer, gate_clamp_min))
+        g = gla_gate(g, gate_logit_normalizer, gate_clamp_min,
+                     output_dtype=torch.float32 if q.dtype != torch.float32 else None)
     check_varlen_args(q, offsets, head_first, initial_state)
     if scale is None:
         scale = q.shape[-1] ** -0.5

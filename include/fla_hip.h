@@ -202,6 +202,19 @@ int fla_chunk_gla_fwd_fused(const void* q, const void* k, const void* v, const v
                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                             float scale, fla_stream_t stream);
 
+/* fla_chunk_gla_fwd_fused on the gate projection's output instead of the log-gates: the kernel itself forms
+ * g = logsigmoid(gate_logits) / normalizer (then max(g, clamp_min) when has_clamp), the elementwise pass a GLA
+ * layer runs in front of chunk_gla (fla/layers/gla.py:214-217), on its way to the prefix sums; the fp32
+ * [B,T,H,K] log-gate tensor is never written or read.  gate_logits [B,T,H,K] in gate_dtype (fp32, or the
+ * q/k/v dtype).  Forward without kept states; a pass that will be differentiated applies
+ * fla_gate_logsigmoid_fwd and calls the entry points above. */
+int fla_chunk_gla_fwd_fused_logits(const void* q, const void* k, const void* v, const void* gate_logits,
+                                   const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
+                                   const int64_t* offsets, const int64_t* indices, const int64_t* chunk_offsets,
+                                   const int64_t* seq_order, int64_t NT, int qkv_dtype, int gate_dtype, int64_t B,
+                                   int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
+                                   float normalizer, int has_clamp, float clamp_min, fla_stream_t stream);
+
 /* Diagnostics: only the first of the two launches of fla_chunk_gla_fwd_fused (the scan, with the flag and
  * state hand-over stores of the range guard when the workspaces are given), so that a benchmark can put
  * events round the dominant kernel in the form the operator runs.  o is incomplete for flagged chunks. */
@@ -338,6 +351,21 @@ int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void
                                         const int64_t* chunk_offsets,
                                         const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                         int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
+
+/* The same two launches on un-normalised q and k: every q and k row is replaced by x / sqrt(sum x^2 + eps) as it
+ * is staged, the two l2_norm launches a gated DeltaNet layer runs in front of the operator
+ * (fla/layers/gated_deltanet.py:234-235, fla/modules/l2norm.py:18-40), so the normalised tensors are never
+ * written or read.  Forward without kept intermediates; a pass that will be differentiated runs
+ * fla_l2norm_fwd / _bwd either side of the entry points above. */
+int fla_gdr_fwd_prep_l2norm(const void* k, const float* beta, const float* g, int g_is_cumsum, float* g_cumsum_out,
+                            void* AT, const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
+                            int64_t B, int64_t T, int64_t H, int64_t K, float eps, fla_stream_t stream);
+int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const void* k, const void* v, const void* AT,
+                                               const float* g_cumsum, const float* h0, void* o, float* ht,
+                                               const int64_t* offsets, const int64_t* chunk_offsets,
+                                               const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
+                                               int64_t H, int64_t K, int64_t V, int64_t N, float scale, float eps,
+                                               fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Chunked GLA backward (chunk size 64), replaces chunk_gla_bwd

@@ -444,3 +444,61 @@ def test_chunk_gdr_slab_width_independence_backward(device):
     g8 = _grads_dev(device, twice(q), twice(k), twice(v), twice(g), twice(beta), twice(h0), twice(do), twice(dht))
     for name, a, b in zip(NAMES, g4, g8):
         assert torch.equal(b[:B], a) and torch.equal(b[B:], a), name
+
+
+@pytest.mark.parametrize("K,V,T,varlen", [(128, 128, 300, False), (128, 128, 1000, True), (64, 128, 130, False),
+                                          (64, 64, 65, True), (128, 64, 1, False)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_chunk_gdr_qk_l2norm_in_kernel(device, dtype, K, V, T, varlen):
+    """The opt-in form on un-normalised q and k: the two forward launches l2-normalise the rows themselves
+    (fla/layers/gated_deltanet.py:234-235).  Against the recurrence on the oracle's l2norm (rounded to the
+    storage type, as the stand-alone launch leaves it), and against that two-step form of the same library."""
+    from fla_amd.modules import l2norm_fwd
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from oracle.modules import l2norm
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(T + K + V)
+    B, H, N = (1, 3, 3) if varlen else (2, 3, 2)
+    q = (torch.randn(B, T, H, K, generator=gen) * 1.7).to(dtype)
+    k = (torch.randn(B, T, H, K, generator=gen) * 0.6).to(dtype)
+    _, _, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=T, dtype=dtype, N=N)
+    offs = random_offsets(T, N, gen) if varlen else None
+    print(f"chunk_gdr in-kernel l2norm {dtype} K={K} V={V} T={T} varlen={varlen}", flush=True)
+    dev = lambda t: None if t is None else t.to(device)
+    o, ht = chunk_gated_delta_rule(dev(q), dev(k), dev(v), dev(g), dev(beta), initial_state=dev(h0),
+                                   output_final_state=True, offsets=dev(offs), head_first=False,
+                                   use_qk_l2norm_in_kernel=True)
+    qn, kn = l2norm(q).to(dtype), l2norm(k).to(dtype)
+    ro, rht = naive_recurrent_gated_delta_rule(qn, kn, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    o2, ht2 = chunk_gated_delta_rule(l2norm_fwd(dev(q)), l2norm_fwd(dev(k)), dev(v), dev(g), dev(beta),
+                                     initial_state=dev(h0), output_final_state=True, offsets=dev(offs),
+                                     head_first=False)
+    assert_close("o vs two-step", o2, o, 3e-3)
+    assert_close("ht vs two-step", ht2, ht, 2e-3)
+
+
+def test_chunk_gdr_qk_l2norm_backward(device):
+    """With gradients the l2norm form runs the stand-alone l2 norm and its backward either side of the operator:
+    gradients of the raw q and k against autograd through the oracle's l2norm and recurrence."""
+    from fla_amd.ops.gated_delta_rule import chunk_gated_delta_rule
+    from oracle.modules import l2norm
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(3)
+    B, T, H, K, V = 2, 130, 2, 64, 64
+    q = (torch.randn(B, T, H, K, generator=gen) * 1.7).bfloat16()
+    k = (torch.randn(B, T, H, K, generator=gen) * 0.6).bfloat16()
+    _, _, v, g, beta, h0 = gdr_inputs(B, T, H, K, V, seed=4)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    print("chunk_gdr l2norm backward", flush=True)
+    leaves = [t.to(device).requires_grad_() for t in (q, k, v, g, beta)]
+    o, _ = chunk_gated_delta_rule(*leaves, initial_state=h0.to(device), head_first=False, use_qk_l2norm_in_kernel=True)
+    o.backward(do.to(device))
+    ref = [t.float().requires_grad_() for t in (q, k, v, g, beta)]
+    ro, _ = naive_recurrent_gated_delta_rule(l2norm(ref[0]), l2norm(ref[1]), ref[2], ref[3], ref[4], initial_state=h0)
+    ro.backward(do.float())
+    assert_close("o", ro, o, TOL_O)
+    for name, a, b in zip(("dq", "dk", "dv", "dg", "dbeta"), ref, leaves):
+        assert_close(name, a.grad, b.grad, 2e-2)

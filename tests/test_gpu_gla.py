@@ -536,3 +536,69 @@ def test_chunk_gla_kept_gated_queries_and_decays(device, B, H, varlen):
     want_decay = torch.stack(want_decay)
     got_decay = decay.reshape(-1, H, D)[:want_decay.shape[0]].cpu()
     torch.testing.assert_close(got_decay, want_decay, rtol=2e-5, atol=1e-30)
+
+
+@pytest.mark.parametrize("logit_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("K,V,T,normalizer,clamp_min,varlen", [
+    (128, 128, 300, 16.0, None, False),
+    (128, 128, 257, 16.0, -0.02, True),
+    (64, 128, 130, 1.0, None, False),
+    (128, 64, 200, 0.05, None, True),      # strong gates: the flagged chunks go through the exact launch
+    (64, 64, 1, 16.0, None, False),
+])
+def test_chunk_gla_from_gate_logits(device, logit_dtype, K, V, T, normalizer, clamp_min, varlen):
+    """The opt-in form that takes the gate projection's output: the fused launch applies
+    logsigmoid(x) / normalizer (+ clamp) itself (fla/layers/gla.py:214-217).  Against the recurrence on the
+    oracle's gates, and against the two-step form (gate launch, then the operator) of the same library."""
+    from fla_amd.modules import gla_gate_fwd
+    from fla_amd.ops.gla import chunk_gla
+    from oracle.modules import gla_gate
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(T + K)
+    B, H = (1, 3) if varlen else (2, 3)
+    q, k, v, _, _ = gla_inputs(B, T, H, K, V, seed=T + V)
+    x = (torch.randn(B, T, H, K, generator=gen) * 2).to(logit_dtype)
+    offs = random_offsets(T, 3, gen) if varlen else None
+    h0 = torch.randn(3 if varlen else B, H, K, V, generator=gen) * 0.1
+    print(f"chunk_gla gate logits {logit_dtype} K={K} V={V} T={T} normalizer={normalizer} clamp={clamp_min} "
+          f"varlen={varlen}", flush=True)
+    dev = lambda t: None if t is None else t.to(device)
+    o, ht = chunk_gla(dev(q), dev(k), dev(v), dev(x), initial_state=dev(h0), output_final_state=True,
+                      offsets=dev(offs), head_first=False, gate_logit_normalizer=normalizer,
+                      gate_clamp_min=clamp_min)
+    g = gla_gate(x, normalizer, clamp_min)
+    ro, rht = naive_recurrent_gla(q, k, v, g, initial_state=h0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    assert o.dtype == torch.bfloat16
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    g_dev = gla_gate_fwd(dev(x), normalizer, clamp_min)
+    o2, ht2 = chunk_gla(dev(q), dev(k), dev(v), g_dev, initial_state=dev(h0), output_final_state=True,
+                        offsets=dev(offs), head_first=False)
+    assert_close("o vs two-step", o2, o, 2e-3)
+    assert_close("ht vs two-step", ht2, ht, 1e-4)
+
+
+def test_chunk_gla_from_gate_logits_backward(device):
+    """With gradients the logits form runs the gate launch and its backward either side of the operator:
+    d(logits) against autograd through the oracle's gate and recurrence."""
+    from fla_amd.ops.gla import chunk_gla
+    from oracle.modules import gla_gate
+    from oracle.recurrent import naive_recurrent_gla
+    gen = torch.Generator().manual_seed(5)
+    B, T, H, K, V = 2, 130, 2, 64, 64
+    q, k, v, _, h0 = gla_inputs(B, T, H, K, V, seed=9)
+    x = (torch.randn(B, T, H, K, generator=gen) * 2).bfloat16()
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    print("chunk_gla gate logits backward", flush=True)
+    leaves = [t.to(device).requires_grad_() for t in (q, k, v, x)]
+    o, _ = chunk_gla(*leaves, initial_state=h0.to(device), head_first=False, gate_logit_normalizer=16.0,
+                     gate_clamp_min=-0.05)
+    o.backward(do.to(device))
+    ref = [t.float().requires_grad_() for t in (q, k, v, x)]
+    ro, _ = naive_recurrent_gla(ref[0], ref[1], ref[2], gla_gate(ref[3], 16.0, -0.05), initial_state=h0)
+    ro.backward(do.float())
+    assert_close("o", ro, o, TOL_O)
+    for name, a, b in zip(("dq", "dk", "dv", "dx"), ref, leaves):
+        assert b.grad.dtype == b.dtype
+        assert_close(name, a.grad, b.grad, 1.5e-2)
