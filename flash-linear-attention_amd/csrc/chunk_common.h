@@ -1,6 +1,8 @@
 // Helpers shared by the chunk kernels: chunk geometry, vector loads with
 // conversion to fp32, the XCD-aware workgroup renumbering.
 #pragma once
+#include <mutex>
+#include <unordered_map>
 #include "fla_common.h"
 #include "mfma_tiles.h"
 
@@ -148,18 +150,23 @@ inline int chunk_grid(const int64_t* offsets, const int64_t* indices, int64_t B,
 }
 
 // Workgroups of `kernel` (256 threads, no dynamic LDS) that the chip holds at once: the grid of a kernel whose
-// workgroups walk many items each.  Asked of the runtime once per kernel.
-template <typename Kern>
-inline int64_t resident_workgroups(Kern kernel) {
-  static int per_cu = 0;   // one instance per kernel type and address: callers pass distinct instantiations
-  static const void* cached = nullptr;
-  if (cached != (const void*)kernel) {
+// workgroups walk many items each.  Asked of the runtime once per kernel address; the small table is shared by
+// every instantiation and guarded by a mutex (entry points may be called from several host threads).
+inline int64_t resident_workgroups_of(const void* kernel) {
+  static std::mutex mu;
+  static std::unordered_map<const void*, int> per_cu;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = per_cu.find(kernel);
+  if (it == per_cu.end()) {
     int n = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) n = 1;
-    per_cu = n;
-    cached = (const void*)kernel;
+    it = per_cu.emplace(kernel, n).first;
   }
-  return (int64_t)per_cu * kNumCUs;
+  return (int64_t)it->second * kNumCUs;
+}
+template <typename Kern>
+inline int64_t resident_workgroups(Kern kernel) {
+  return resident_workgroups_of((const void*)kernel);
 }
 
 // dst = src (or zeros when src is NULL), n floats: what the state gradient of a batch without any

@@ -682,12 +682,14 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
   FLA_REQUIRE((qg == nullptr) == (decay == nullptr), FLA_E_INVALID);
   if (qg) {
     FLA_REQUIRE(h_frag_t != nullptr, FLA_E_INVALID);
-    FLA_REQUIRE(V <= 256, FLA_E_UNSUPPORTED);
+    // the value slabs of a head share the rows of the kept tiles out evenly: 1, 2 or 4 slabs (8 in the narrow form)
+    FLA_REQUIRE(V == 64 || V == 128 || V == 256, FLA_E_UNSUPPORTED);
     FLA_REQUIRE((uintptr_t)qg % 16 == 0, FLA_E_ALIGNMENT);
   }
   FLA_REQUIRE((kh_t == nullptr) == (scores == nullptr), FLA_E_INVALID);
   if (kh_t) {
     FLA_REQUIRE(qg != nullptr, FLA_E_INVALID);
+    FLA_REQUIRE(V <= 128, FLA_E_UNSUPPORTED);   // what fla_chunk_gla_bwd_kept reads them for
     FLA_REQUIRE(((uintptr_t)kh_t | (uintptr_t)scores) % 16 == 0, FLA_E_ALIGNMENT);
   }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,

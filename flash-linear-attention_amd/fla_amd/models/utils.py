@@ -22,9 +22,24 @@ def _same_storage(a: torch.Tensor, b: torch.Tensor) -> bool:
     return a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.dtype == b.dtype
 
 
-class Cache:
+# The reference's Cache subclasses transformers' (fla/models/utils.py:11), whose `generate` checks
+# `isinstance(past_key_values, Cache)`; do the same wherever transformers is importable.
+try:
+    from transformers.cache_utils import Cache as _CacheBase
+except Exception:   # transformers absent or broken: a plain class serves callers that drive the operators directly
+    _CacheBase = object
+
+
+class Cache(_CacheBase):
 
     def __init__(self, seen_tokens: int = 0, persistent: bool = False):
+        # like the reference, the base class's own constructor is not run: nothing of its per-layer
+        # key/value bookkeeping applies; `layers` is left empty for the base class's helpers that walk it
+        if _CacheBase is not object:
+            try:
+                self.layers = []
+            except AttributeError:
+                pass
         self.states: List[Dict[str, Any]] = []
         self._seen_tokens = seen_tokens  # `generate` reads this to place new tokens
         self.persistent = persistent
@@ -67,14 +82,26 @@ class Cache:
             if not isinstance(attn_state, (tuple, list)) or len(attn_state) != 2:
                 raise ValueError("`attn_state` must be a tuple of two tensors for key/value states")
             # key/value states of softmax-attention layers in hybrid models (outside the linear-attention path;
-            # kept for interface parity): appended along the token axis, optionally cut to the newest
-            # `window_size` tokens
-            held = self.states[layer_idx].get('attn_state') if layer_idx < len(self.states) else None
-            if held is not None:
-                attn_state = tuple(torch.cat([h, n], -2) for h, n in zip(held, attn_state))
+            # kept for interface parity, fla/models/utils.py:75-111)
             window_size = (cache_kwargs or {}).get('window_size', None)
-            if window_size is not None and attn_state[0].shape[-2] > window_size:
-                attn_state = tuple(x[..., -window_size:, :].contiguous() for x in attn_state)
+            input_size = attn_state[0].shape[-2]
+            held = self.states[layer_idx].get('attn_state') if layer_idx < len(self.states) else None
+            if held is None:
+                # first entry of the layer: only the newest `window_size` tokens are kept (in a buffer of the
+                # cache's own: it is shifted in place later, which must not reach into the caller's tensor)
+                if window_size is not None and input_size >= window_size:
+                    attn_state = tuple(x[..., -window_size:, :].clone() for x in attn_state)
+            elif window_size is not None and held[0].shape[-2] == window_size and input_size <= window_size:
+                # a full window: shift the held buffers left by the new tokens and write those at the end,
+                # in the buffers the cache already holds (same addresses from step to step)
+                for h, n in zip(held, attn_state):
+                    if input_size < window_size:
+                        h.copy_(h.roll(-input_size, -2))
+                    h[..., -input_size:, :] = n
+                attn_state = tuple(held)
+            else:
+                # a window that is not full yet grows by the new tokens and is not cut
+                attn_state = tuple(torch.cat([h, n], -2) for h, n in zip(held, attn_state))
         if len(self.states) <= layer_idx:
             state = dict(recurrent_state=recurrent_state, attn_state=attn_state, conv_state=conv_state,
                          ffn_state=ffn_state)

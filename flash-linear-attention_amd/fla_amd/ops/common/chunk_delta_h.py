@@ -33,8 +33,17 @@ def chunk_gated_delta_rule_fwd_h(
     the log-gate ``[B,T,H]`` (or ``None``).  ``h`` is ``[B,NT,H,K,V]`` holding the
     state entering each chunk (row-major, or MFMA-fragment order for
     ``fla_chunk_fwd_o`` when ``fragment_layout``)."""
-    if head_first or chunk_size != BT:
-        raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd_h: seq-first, chunk size 64 only")
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd_h: chunk size 64 only")
+    if head_first:
+        # head-first operands ([B,H,T,*]) are transposed on the way in, h ([B,H,NT,K,V]) and v_new on the way out
+        if fragment_layout:
+            raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd_h: fragment-order states are seq-first")
+        tr = lambda x: None if x is None else x.transpose(1, 2).contiguous()
+        h, v_new, ht = chunk_gated_delta_rule_fwd_h(
+            tr(k), tr(w), tr(u), tr(g), initial_state, output_final_state, offsets, indices, False, chunk_size,
+            states_in_fp32=states_in_fp32, chunk_offsets=chunk_offsets, store_v_new=store_v_new)
+        return h.transpose(1, 2), (None if v_new is None else v_new.transpose(1, 2)), ht
     be.require_gpu(k, w, u)
     B, T, H, K = k.shape
     V = u.shape[-1]

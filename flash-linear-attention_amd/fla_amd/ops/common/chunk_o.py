@@ -28,9 +28,15 @@ def chunk_fwd_o(
     (``fla/ops/common/chunk_o.py:444-496``).  ``h`` ``[B,NT,H,K,V]`` is row-major as in the reference
     (fp32 or 16-bit; re-ordered for the kernel by one extra pass over the states), or, with
     ``fragment_layout=True``, the MFMA-fragment-order states the scan kernels of this library write;
-    ``g`` is the fp32 chunk-local cumsum ``[B,T,H]`` or ``None``."""
-    if head_first or chunk_size != BT:
-        raise NotImplementedError("fla_amd chunk_fwd_o: seq-first, chunk size 64 only")
+    ``g`` is the fp32 chunk-local cumsum ``[B,T,H]`` or ``None``.  Head-first operands (``[B,H,T,*]``, states
+    ``[B,H,NT,K,V]``) are transposed on the way in and ``o`` on the way out."""
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd chunk_fwd_o: chunk size 64 only")
+    if head_first:
+        if fragment_layout:
+            raise NotImplementedError("fla_amd chunk_fwd_o: fragment-order states are seq-first")
+        tr = lambda x: None if x is None else x.transpose(1, 2).contiguous()
+        return chunk_fwd_o(tr(q), tr(k), tr(v), tr(h), tr(g), scale, offsets, indices, False, chunk_size).transpose(1, 2)
     be.require_gpu(q, k, v, h)
     B, T, H, K = q.shape
     V = v.shape[-1]

@@ -28,8 +28,14 @@ def fwd_prepare_wy_repr(
     ``Au = Aw * exp(g_i - g_j)``, ``w = Aw (beta K)``, ``u = Au (beta V)``; ``g`` is the
     fp32 chunk-local cumsum of the log-gate (or ``None``).  ``store_u=False`` skips ``u`` (returned as ``None``)
     for a forward that forms ``v_new`` from the triangular tiles instead."""
-    if head_first or chunk_size != BT:
-        raise NotImplementedError("fla_amd fwd_prepare_wy_repr: seq-first, chunk size 64 only")
+    if chunk_size != BT:
+        raise NotImplementedError("fla_amd fwd_prepare_wy_repr: chunk size 64 only")
+    if head_first:
+        # head-first operands ([B,H,T,*]) are transposed on the way in and every result on the way out
+        tr = lambda x: None if x is None else x.transpose(1, 2).contiguous()
+        outs = fwd_prepare_wy_repr(tr(k), tr(v), tr(beta), tr(g), offsets, indices, False, chunk_size,
+                                   store_A=store_A, store_Au=store_Au, store_u=store_u)
+        return tuple(None if x is None else x.transpose(1, 2) for x in outs)
     be.require_gpu(k, v, beta)
     B, T, H, K = k.shape
     V = v.shape[-1]

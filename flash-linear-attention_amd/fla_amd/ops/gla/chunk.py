@@ -8,6 +8,7 @@ range of the single-reference-point scores.  The two-kernel form (``fla_chunk_gl
 ``chunk_fwd_h`` / ``chunk_gla_fwd_o_gk``.
 """
 import os
+import threading
 import warnings
 from typing import Optional, Tuple
 
@@ -166,21 +167,25 @@ def chunk_gla_bwd_dv(k, g, A, do, dh, offsets=None, indices=None, head_first=Tru
     return dv.transpose(1, 2) if head_first else dv
 
 
-# Workspaces of the range guard for forward passes whose flags nobody keeps: one pair per (device,
-# stream, shape, dtype), reused by every call (launches on one stream are ordered, so the next call
-# may overwrite them).  A forward that hands its flags to a backward pass gets fresh ones.
+# Workspaces of the range guard for forward passes whose flags nobody keeps: one pair per (device, stream, dtype,
+# host thread), grown to the largest call seen and reused by every later call (launches on one stream are ordered,
+# so the next call may overwrite them; two host threads never share a pair).  The state hand-over buffer holds one
+# [K, V] tile per (chunk, head) - 268 MB at B=8, T=4096, H=16, K=V=128 in 16 bits - and stays allocated; a forward
+# that hands its flags to a backward pass gets fresh ones.
 _GUARD_WS = {}
 
 
 def _guard_workspaces(q, chunks, H, KV, keep):
     if keep:
         return q.new_empty(chunks, H, dtype=torch.int32), q.new_empty(chunks, H, KV)
-    key = (q.device, torch.cuda.current_stream(q.device).cuda_stream, chunks, H, KV, q.dtype)
+    key = (q.device, torch.cuda.current_stream(q.device).cuda_stream, q.dtype, threading.get_ident())
     ws = _GUARD_WS.get(key)
-    if ws is None:
-        if len(_GUARD_WS) >= 8:
+    n_flags, n_state = chunks * H, chunks * H * KV
+    if ws is None or ws[0].numel() < n_flags or ws[1].numel() < n_state:
+        if ws is None and len(_GUARD_WS) >= 16:
             _GUARD_WS.clear()
-        ws = _GUARD_WS[key] = (q.new_empty(chunks, H, dtype=torch.int32), q.new_empty(chunks, H, KV))
+        ws = _GUARD_WS[key] = (q.new_empty(max(n_flags, 0 if ws is None else ws[0].numel()), dtype=torch.int32),
+                               q.new_empty(max(n_state, 0 if ws is None else ws[1].numel())))
     return ws
 
 
@@ -301,14 +306,20 @@ def _internal_layout(head_first, *tensors):
     return tuple(None if t is None else (t.transpose(1, 2) if head_first else t).contiguous() for t in tensors)
 
 
-def _check_internal(q, k, v, T):
-    if min(BT, max(16, 1 << (max(T, 1) - 1).bit_length())) != BT:
-        raise NotImplementedError("fla_amd chunk_gla_fwd / chunk_gla_bwd: chunk size is fixed to 64 (needs T > 32)")
+def _check_internal(q, k, v, T, offsets=None):
+    """Returns the reference's chunk length for the call, ``min(64, max(16, npow2(T)))`` (``fla/ops/gla/chunk.py:1350``).
+    The kernels walk chunks of 64; for T <= 32 a batch of equal-length sequences is one chunk either way (same
+    cumulative gates, states and outputs; the score tile has 16 or 32 columns instead of 64)."""
+    bt = min(BT, max(16, 1 << (max(T, 1) - 1).bit_length()))
+    if bt != BT and offsets is not None:
+        raise NotImplementedError("fla_amd chunk_gla_fwd / chunk_gla_bwd: packed batches of 32 tokens or fewer are "
+                                  "chunked by 16 or 32 in the reference; the kernels are built for chunks of 64")
     if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise NotImplementedError("fla_amd chunk_gla_fwd / chunk_gla_bwd: q, k, v must share one 16-bit dtype")
     if (q.shape[-1], v.shape[-1]) not in _SUPPORTED_KV:
         raise NotImplementedError(f"fla_amd chunk_gla_fwd / chunk_gla_bwd: head dims {q.shape[-1]}, {v.shape[-1]} "
                                   f"outside the built tiles {sorted(_SUPPORTED_KV)}")
+    return bt
 
 
 def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state,
@@ -321,7 +332,7 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
     log-gate stays within +-80 (bf16) / +-8 (fp16) - the backward entry below does not read it."""
     q, k, v, g, g_cumsum = _internal_layout(head_first, q, k, v, g, g_cumsum)
     B, T, H, K = q.shape
-    _check_internal(q, k, v, T)
+    bt = _check_internal(q, k, v, T, offsets)
     plan = VarlenPlan(offsets, BT) if offsets is not None else None
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
@@ -343,6 +354,8 @@ def chunk_gla_fwd(q, k, v, g, g_cumsum, scale, initial_state, output_final_state
                        chunk_size=BT, k=k, gates_are_cumsum=True, A_out=A)
     o, _ = chunk_gla_fwd_fused(q, k, v, g if g.dtype in (torch.float32, q.dtype) else g.float(), scale, initial_state,
                                False, offsets)
+    if bt != BT:
+        A = A[..., :bt]
     if head_first:
         g_cumsum, A, o = (x.transpose(1, 2) for x in (g_cumsum, A, o))
         h = h.transpose(1, 2)
@@ -403,17 +416,31 @@ def chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wid
     return dq, dk, dv, dg, dh0
 
 
+def _gate_range_flags(g_cumsum: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """int32 ``[B * NT, H]``: 1 where a chunk's cumulative log-gates leave the range in which the kernels score a
+    chunk with one reference point (|G| <= 80 for bf16 operands, 8 for fp16) - what the fused forward's staging
+    waves flag on their way - from seq-first cumulative gates ``[B, T, H, K]`` of equal-length sequences."""
+    B, T, H, K = g_cumsum.shape
+    limit = 80.0 if dtype == torch.bfloat16 else 8.0
+    peak = g_cumsum.abs().amax(-1)                                    # [B, T, H]
+    pad = -T % BT
+    if pad:
+        peak = F.pad(peak, (0, 0, 0, pad))
+    return (peak.view(B, -1, BT, H).amax(2) > limit).to(torch.int32).view(-1, H).contiguous()
+
+
 def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
                   offsets=None, indices=None, head_first=True, chunk_size=64):
     """Reference-shaped backward (``fla/ops/gla/chunk.py:1217-1320``) for internal callers (GSA:
     ``g=None, g_cumsum=..., h=..., A=...``, ``fla/ops/gsa/chunk.py:741-757``): returns ``(dq, dk, dv, dg, dh0)`` in
     the caller's layout, ``dg`` the gradient of the raw gates (the chunk-local reverse cumulative sum already
     applied, as ``chunk_gla_bwd_kernel_inter`` leaves it, ``fla/ops/gla/chunk.py:818-823``).  Either ``g`` or
-    ``g_cumsum`` may be ``None``.  The per-chunk states and the gate-range flags come from one run of the fused
-    forward launch and the scores are recomputed on chip, so ``h`` and ``A`` are accepted and not read; exact for
+    ``g_cumsum`` may be ``None``.  Row-major states ``h`` (fp32 or the q/k/v dtype) of equal-length sequences are
+    used as given, together with ``g_cumsum``; otherwise the per-chunk states and the gate-range flags come from one
+    run of the fused forward launch.  The scores are recomputed on chip (``A`` is accepted and not read); exact for
     any gate."""
     q, k, v, g, g_cumsum, do = _internal_layout(head_first, q, k, v, g, g_cumsum, do)
-    _check_internal(q, k, v, q.shape[1])
+    _check_internal(q, k, v, q.shape[1], offsets)
     if g is None:
         if g_cumsum is None:
             raise ValueError("chunk_gla_bwd needs g or g_cumsum")
@@ -422,15 +449,25 @@ def chunk_gla_bwd(q, k, v, g, g_cumsum, scale, initial_state, h, A, do, dht,
                                        indices=None if plan is None else plan.indices, head_first=False)
     elif g.dtype not in (torch.float32, q.dtype):
         g = g.float()
-    states = []
-    _, _, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, False, offsets, return_flags=True,
-                                     states_out=states)
-    dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do.to(q.dtype).contiguous(), dht,
-                                               offsets, wide, hT=states[0],
-                                               qg=states[1] if len(states) > 1 else None,
-                                               decay=states[2] if len(states) > 2 else None,
-                                               kh=states[3] if len(states) > 4 else None,
-                                               scores=states[4] if len(states) > 4 else None)
+    do = do.to(q.dtype).contiguous()
+    if h is not None and g_cumsum is not None and offsets is None and h.dtype in (torch.float32, q.dtype):
+        # the caller's states (row-major, the state entering every chunk) are re-ordered for the kernels instead of
+        # being recomputed; the chunks whose cumulative gates leave the range of the single-reference-point scores
+        # are read off the cumulative gates the caller holds
+        from ..common.chunk_o import states_to_fragments
+        hT = states_to_fragments(h.transpose(1, 2) if head_first else h, q.dtype, transposed=True)
+        wide = _gate_range_flags(g_cumsum, q.dtype)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide, hT=hT)
+    else:
+        states = []
+        _, _, wide = chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, False, offsets, return_flags=True,
+                                         states_out=states)
+        dq, dk, dv, dg, dh0 = chunk_gla_bwd_device(q, k, v, g, scale, initial_state, do, dht, offsets, wide,
+                                                   hT=states[0],
+                                                   qg=states[1] if len(states) > 1 else None,
+                                                   decay=states[2] if len(states) > 2 else None,
+                                                   kh=states[3] if len(states) > 4 else None,
+                                                   scores=states[4] if len(states) > 4 else None)
     if head_first:
         dq, dk, dv, dg = (x.transpose(1, 2) for x in (dq, dk, dv, dg))
     return dq, dk, dv, dg, dh0

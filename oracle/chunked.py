@@ -27,8 +27,10 @@ recurrences.  Chunks never straddle sequences; tail chunks are short.
 
 The three ``gla_*`` functions at the end restate single stages of the GLA pipeline on the
 operands the reference's internal callers pass (scores ``A`` and row-major per-chunk states):
-``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  ``chunk_bwd_dh`` restates the reverse
-state scan of ``fla/ops/common/chunk_h.py:146-262``, ``chunk_bwd_dv_local`` the intra-chunk dv of the
+``fla/ops/gla/chunk.py:320-393`` (output), ``:582-624`` (dA), ``:642-710`` (dv).  ``chunk_fwd_h`` restates the state
+scan of ``fla/ops/common/chunk_h.py:29-137`` for any mix of per-head, per-key and per-value gates (pinned by the
+token-by-token recurrence), ``chunk_bwd_dh`` the reverse
+state scan of ``fla/ops/common/chunk_h.py:146-262`` (same gates; pinned by autograd through the state chain), ``chunk_bwd_dv_local`` the intra-chunk dv of the
 per-head-gate operators (``fla/ops/common/chunk_o.py:379-441``).  They are pinned
 by the recurrence (output stage on ``chunked_gla``'s intermediates) and by autograd through the
 chunk step (dA, dv, dh) in ``tests/test_oracle_pins.py``.
@@ -217,9 +219,46 @@ def gla_bwd_dv(k, g_cumsum, A, do, dh, chunk_size=64, offsets=None, dtype=torch.
     return dv
 
 
-def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=torch.float32):
-    """For c = last .. 0:  dh[c] = dH;  dH = e^{g_last} diag(e^{gk_last}) dH + (s q e^{g} e^{gk})^T do, from dH = dht.
-    g [B,T,H] and gk [B,T,H,K] are chunk-cumulative log-gates, either may be None.  Returns dh in the
+def chunk_fwd_h(k, v, g=None, gk=None, gv=None, h0=None, chunk_size=64, offsets=None, dtype=torch.float32):
+    """The state entering every chunk and the final state, for any mix of chunk-cumulative log-gates g [B,T,H],
+    gk [B,T,H,K], gv [B,T,H,V]:  h_next = e^{g_last} diag(e^{gk_last}) h diag(e^{gv_last})
+    + (k e^{gk_last - gk})^T (v e^{g_last - g} e^{gv_last - gv})   (fla/ops/common/chunk_h.py:73-137).
+    Returns h in storage order ([B,NT,H,K,V] / [1,NT_total,H,K,V]) and ht [N,H,K,V]."""
+    k, v = k.to(dtype), v.to(dtype)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    out, ht = [], []
+    for n, (b, bos, eos) in enumerate(_spans(B, T, offsets)):
+        h = torch.zeros(H, K, V, dtype=dtype) if h0 is None else h0[n].to(dtype).clone()
+        for s, e in _chunks(bos, eos, chunk_size):
+            out.append(h)
+            kt, vt = k[b, s:e], v[b, s:e]
+            if g is not None:
+                gg = g[b, s:e].to(dtype)
+                vt = vt * (gg[-1][None] - gg).exp()[..., None]
+                h = h * gg[-1].exp()[:, None, None]
+            if gk is not None:
+                gg = gk[b, s:e].to(dtype)
+                kt = kt * (gg[-1][None] - gg).exp()
+                h = h * gg[-1].exp()[:, :, None]
+            if gv is not None:
+                gg = gv[b, s:e].to(dtype)
+                vt = vt * (gg[-1][None] - gg).exp()
+                h = h * gg[-1].exp()[:, None, :]
+            h = h + torch.einsum('thk,thv->hkv', kt, vt)
+        ht.append(h)
+    if offsets is None:
+        NT = -(-T // chunk_size)
+        hs = torch.stack(out, 0).reshape(B, NT, H, K, V) if out else torch.zeros(B, 0, H, K, V, dtype=dtype)
+    else:
+        hs = torch.stack(out, 0)[None]
+    return hs, torch.stack(ht, 0)
+
+
+def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=torch.float32, gv=None):
+    """For c = last .. 0:  dh[c] = dH;  dH = e^{g_last} diag(e^{gk_last}) dH diag(e^{gv_last})
+    + (s q e^{g} e^{gk})^T (do e^{gv}), from dH = dht.
+    g [B,T,H], gk [B,T,H,K] and gv [B,T,H,V] are chunk-cumulative log-gates, each may be None.  Returns dh in the
     storage order of the states ([B,NT,H,K,V] / [1,NT_total,H,K,V]) and dh0 [N,H,K,V]
     (fla/ops/common/chunk_h.py:202-262)."""
     q, do = q.to(dtype), do.to(dtype)
@@ -233,6 +272,7 @@ def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=to
         for s, e in reversed(_chunks(bos, eos, chunk_size)):
             seq.append(dH)
             qt = scale * q[b, s:e]
+            dot = do[b, s:e]
             decay = torch.ones(H, K, dtype=dtype)
             if g is not None:
                 qt = qt * g[b, s:e].to(dtype).exp()[..., None]
@@ -240,7 +280,11 @@ def chunk_bwd_dh(q, g, gk, do, dht, scale, chunk_size=64, offsets=None, dtype=to
             if gk is not None:
                 qt = qt * gk[b, s:e].to(dtype).exp()
                 decay = decay * gk[b, e - 1].to(dtype).exp()
-            dH = dH * decay[:, :, None] + torch.einsum('thk,thv->hkv', qt, do[b, s:e])
+            dH = dH * decay[:, :, None]
+            if gv is not None:
+                dot = dot * gv[b, s:e].to(dtype).exp()
+                dH = dH * gv[b, e - 1].to(dtype).exp()[:, None, :]
+            dH = dH + torch.einsum('thk,thv->hkv', qt, dot)
         out.extend(reversed(seq))
         dh0.append(dH)
     if offsets is None:

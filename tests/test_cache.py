@@ -63,3 +63,38 @@ def test_attention_window():
     d.update(attn_state=(k, v), layer_idx=0, offset=6, cache_kwargs={})
     d.update(attn_state=(nk, nv), layer_idx=0, offset=1, cache_kwargs={})
     assert d[0]['attn_state'][0].shape[-2] == 7
+
+
+def test_attention_window_follows_the_reference_lengths():
+    """The length rules of fla/models/utils.py:75-111, case by case: the first entry is cut to the window; a window
+    that is not full grows by the new tokens and is never cut (a multi-token update may overshoot it); a full
+    window is shifted in place in the buffers the cache holds."""
+    kw = dict(cache_kwargs=dict(window_size=4))
+    tok = lambda a, b: (torch.arange(a, b, dtype=torch.float32).view(1, 1, -1, 1).expand(1, 1, b - a, 2).contiguous(),
+                        -torch.arange(a, b, dtype=torch.float32).view(1, 1, -1, 1).expand(1, 1, b - a, 2).contiguous())
+    c = _cache()
+    c.update(attn_state=tok(0, 3), layer_idx=0, offset=3, **kw)          # prefill shorter than the window
+    assert c[0]['attn_state'][0].shape[-2] == 3
+    c.update(attn_state=tok(3, 5), layer_idx=0, offset=2, **kw)          # crosses the window boundary: 5, not cut
+    assert c[0]['attn_state'][0].shape[-2] == 5
+    c.update(attn_state=tok(5, 6), layer_idx=0, offset=1, **kw)          # 5 != window: keeps growing, as the reference does
+    assert c[0]['attn_state'][0].shape[-2] == 6
+    d = _cache()
+    d.update(attn_state=tok(0, 9), layer_idx=0, offset=9, **kw)          # first entry longer than the window: newest 4
+    ks, vs = d[0]['attn_state']
+    assert ks.shape[-2] == 4 and ks[0, 0, :, 0].tolist() == [5., 6., 7., 8.]
+    ptrs = (ks.data_ptr(), vs.data_ptr())
+    d.update(attn_state=tok(9, 11), layer_idx=0, offset=2, **kw)         # full window: shifted in place
+    ks2, vs2 = d[0]['attn_state']
+    assert (ks2.data_ptr(), vs2.data_ptr()) == ptrs
+    assert ks2[0, 0, :, 0].tolist() == [7., 8., 9., 10.] and vs2[0, 0, :, 1].tolist() == [-7., -8., -9., -10.]
+    d.update(attn_state=tok(11, 15), layer_idx=0, offset=4, **kw)        # a whole window of new tokens
+    assert d[0]['attn_state'][0].data_ptr() == ptrs[0] and d[0]['attn_state'][0][0, 0, :, 0].tolist() == [11., 12., 13., 14.]
+
+
+def test_is_a_transformers_cache_when_transformers_is_there():
+    try:
+        from transformers.cache_utils import Cache as HFCache
+    except Exception:
+        pytest.skip("transformers not importable")
+    assert isinstance(_cache(), HFCache)

@@ -301,3 +301,29 @@ def test_gdr_stage_argument_errors(device):
         fwd_recompute_w_u(x[..., :48], x, s, A, A, head_first=False)
     with pytest.raises(NotImplementedError):
         bwd_prepare_wy_repr(x, x[..., :48], s, s, A, A, x, x[..., :48], None, None, False, 64)
+
+
+def test_head_first_forms_of_the_forward_stages(device):
+    """fwd_prepare_wy_repr, chunk_gated_delta_rule_fwd_h and chunk_fwd_o take head-first operands as the
+    reference's do by default ([B,H,T,*], states [B,H,NT,K,V]): bit-identical to the seq-first results, transposed."""
+    from fla_amd.ops.common.chunk_delta_h import chunk_gated_delta_rule_fwd_h
+    from fla_amd.ops.common.chunk_o import chunk_fwd_o
+    from fla_amd.ops.gated_delta_rule.wy_fast import fwd_prepare_wy_repr
+    from fla_amd.ops.utils import chunk_local_cumsum
+    B, T, H, K, V = 2, 200, 3, 128, 128
+    q, k, v, g, beta, h0 = (x.to(device) for x in gdr_inputs(B, T, H, K, V, seed=77))
+    gc = chunk_local_cumsum(g, 64, head_first=False)
+    hf = lambda x: x.transpose(1, 2).contiguous()
+    print("head-first forward stages", flush=True)
+    w, u, Aw, Au = fwd_prepare_wy_repr(k, v, beta, gc, head_first=False)
+    w2, u2, Aw2, Au2 = fwd_prepare_wy_repr(hf(k), hf(v), hf(beta), hf(gc), head_first=True)
+    for a, b in ((w, w2), (u, u2), (Aw, Aw2), (Au, Au2)):
+        assert torch.equal(a, b.transpose(1, 2))
+    h, v_new, ht = chunk_gated_delta_rule_fwd_h(k, w, u, gc, h0, True, head_first=False)
+    h2, v_new2, ht2 = chunk_gated_delta_rule_fwd_h(hf(k), hf(w), hf(u), hf(gc), h0, True, head_first=True)
+    assert tuple(h2.shape) == (B, H, -(-T // 64), K, V)
+    assert torch.equal(h, h2.transpose(1, 2)) and torch.equal(v_new, v_new2.transpose(1, 2)) and torch.equal(ht, ht2)
+    o = chunk_fwd_o(q, k, v_new, h, gc, K ** -0.5, head_first=False)
+    o2 = chunk_fwd_o(hf(q), hf(k), v_new2, h2, hf(gc), K ** -0.5, head_first=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2.transpose(1, 2))

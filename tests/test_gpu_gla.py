@@ -602,3 +602,53 @@ def test_chunk_gla_from_gate_logits_backward(device):
     for name, a, b in zip(("dq", "dk", "dv", "dx"), ref, leaves):
         assert b.grad.dtype == b.dtype
         assert_close(name, a.grad, b.grad, 1.5e-2)
+
+
+def test_kept_forward_rejects_value_dims_its_row_split_does_not_cover(device):
+    """fla_chunk_gla_fwd_fused_kept shares the rows of the kept tiles out over the value slabs of a head: value
+    dims that do not divide them evenly (V = 192) are refused, as are the score tiles beyond V = 128."""
+    from fla_amd import _backend as be
+    B, T, H, K = 1, 64, 1, 128
+    for V, with_scores, want in ((192, False, -2), (256, True, -2), (256, False, 0), (128, True, 0)):
+        q, k = (torch.randn(B, T, H, K, device=device).bfloat16() for _ in range(2))
+        v = torch.randn(B, T, H, V, device=device).bfloat16()
+        g = -torch.rand(B, T, H, K, device=device)
+        o, hT, qg = torch.empty_like(v), q.new_empty(B, 1, H, K, V), torch.empty_like(q)
+        decay = q.new_empty(B, 1, H, K, dtype=torch.float32)
+        kh = q.new_empty(B, 1, H, K, 64) if with_scores else None
+        sc = q.new_empty(B, 1, H, 64, 64) if with_scores else None
+        print(f"kept forward V={V} scores={with_scores}", flush=True)
+        rc = be.lib().fla_chunk_gla_fwd_fused_kept(
+            be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), None, be.ptr(o), None, None, None, be.ptr(hT), be.ptr(qg),
+            be.ptr(decay), be.ptr(kh), be.ptr(sc), None, None, None, None, 0, be.dt(q), be.dt(g), B, T, H, K, V, B,
+            K ** -0.5, be.stream_of(q))
+        torch.cuda.synchronize()
+        assert rc == want, (V, with_scores, rc)
+
+
+@pytest.mark.parametrize("T,bt", [(7, 16), (16, 16), (20, 32), (32, 32)])
+def test_chunk_gla_internal_entries_short_sequences(device, T, bt):
+    """chunk_gla_fwd / chunk_gla_bwd for T <= 32, where the reference's chunk length is 16 or 32
+    (fla/ops/gla/chunk.py:1350): the score tile comes back with that many columns, everything else as for one
+    chunk of 64."""
+    from fla_amd.ops.gla.chunk import chunk_gla_bwd, chunk_gla_fwd
+    from oracle.chunked import chunked_gla
+    B, H, K, V = 2, 2, 64, 128
+    q, k, v, g, h0 = gla_inputs(B, T, H, K, V, seed=T, h0_std=1.0)
+    gen = torch.Generator().manual_seed(T)
+    do = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    dht = torch.randn(B, H, K, V, generator=gen) * 0.1
+    dev = lambda x: x.to(device)
+    print(f"chunk_gla_fwd / bwd T={T}", flush=True)
+    gc, A, h, ht, o = chunk_gla_fwd(dev(q), dev(k), dev(v), dev(g), None, K ** -0.5, dev(h0), True, head_first=False)
+    ref = chunked_gla(q, k, v, g, initial_state=h0)
+    assert tuple(A.shape) == (B, T, H, bt) and tuple(h.shape) == (B, 1, H, K, V)
+    assert_close("o", ref['o'], o, TOL_O)
+    assert_close("ht", ref['ht'], ht, TOL_HT)
+    assert_close("A", ref['A'][..., :bt], A, 1e-2)
+    assert_close("g_cumsum", ref['g_cumsum'], gc, 1e-5)
+    dq, dk, dv, dg, dh0 = chunk_gla_bwd(dev(q), dev(k), dev(v), dev(g), gc, K ** -0.5, dev(h0), h, A, dev(do), dev(dht),
+                                        head_first=False)
+    grads = _grads_ref(q, k, v, g, h0, do, dht)
+    for name, r, x, tol in zip(("dq", "dk", "dv", "dg", "dh0"), grads, (dq, dk, dv, dg, dh0), (8e-3, 8e-3, 8e-3, 1e-2, 5e-3)):
+        assert_close(name, r, x, tol)

@@ -271,3 +271,81 @@ def test_chunk_bwd_dv_local_reference_operands(device, B, T, H, K, V, varlen, ga
     torch.cuda.synchronize()
     assert dv.shape == do.shape and dv.dtype == do.dtype
     assert_close("dv_local", chunked.chunk_bwd_dv_local(q, k, g, do, K ** -0.5, offsets=ol), dv, 1e-2)
+
+
+# ---- the argument forms GSA and RWKV6 use beside the GLA stages (fla/ops/gsa/chunk.py:664-675, 794-820;
+# fla/ops/rwkv6/chunk.py:1134-1147): decay on the value axis, head-first layout, grouped query heads
+@pytest.mark.parametrize("head_first", [False, True])
+@pytest.mark.parametrize("B,T,H,K,V,varlen", [(2, 200, 3, 64, 128, False), (1, 300, 2, 128, 64, True),
+                                              (2, 130, 2, 100, 50, False), (2, 20, 2, 64, 64, False)])
+def test_chunk_fwd_h_value_gates(device, head_first, B, T, H, K, V, varlen):
+    """chunk_fwd_h(gv=...) as GSA calls it: row-major states and final state against the oracle's state scan with
+    per-value gates (5e-3, bf16 operands); head-first operands give the same states, transposed."""
+    from fla_amd.ops.common.chunk_h import chunk_fwd_h
+    from oracle import chunked, cumsum
+    if varlen and head_first:
+        pytest.skip("packed batches are seq-first")
+    gen = torch.Generator().manual_seed(T + K + V)
+    N = 3 if varlen else B
+    offs = random_offsets(T, N, gen, min_len=1) if varlen else None
+    ol = None if offs is None else offs.tolist()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    gv = cumsum.chunk_local_cumsum(F.logsigmoid(torch.randn(B, T, H, V, generator=gen)) / 4, 64, offsets=ol)
+    h0 = torch.randn(N, H, K, V, generator=gen) * 0.1
+    print(f"chunk_fwd_h gv head_first={head_first} B={B} T={T} H={H} K={K} V={V} varlen={varlen}", flush=True)
+    d = lambda x: None if x is None else x.to(device)
+    hf = lambda x: x.transpose(1, 2).contiguous() if head_first else x
+    indices = None
+    if varlen:
+        from fla_amd.utils import VarlenPlan
+        indices = VarlenPlan(offs.to(device), 64).indices
+    for fp32 in (True, False):
+        h, ht = chunk_fwd_h(d(hf(k)), d(hf(v)), None, None, d(hf(gv)), d(h0), True, offsets=d(offs), indices=indices,
+                            head_first=head_first, chunk_size=64, states_in_fp32=fp32)
+        torch.cuda.synchronize()
+        ref_h, ref_ht = chunked.chunk_fwd_h(k, v, None, None, gv, h0, offsets=ol)
+        if head_first:
+            h = h.transpose(1, 2)
+        assert h.dtype == (torch.float32 if fp32 else torch.bfloat16) and ht.dtype == torch.float32
+        assert_close("h", ref_h, h, 5e-3)
+        assert_close("ht", ref_ht, ht, 5e-3)
+
+
+@pytest.mark.parametrize("head_first", [False, True])
+@pytest.mark.parametrize("gates", ["gv", "gk", "g"])
+@pytest.mark.parametrize("NG", [1, 2])
+def test_chunk_bwd_dh_value_gates_grouped_heads_and_head_first(device, head_first, gates, NG):
+    """chunk_bwd_dh with decay on the value axis, with HQ = NG * H query heads (a query head decays with its
+    group's gates; dh0 sums over the group) and in head-first layout, against the oracle's reverse scan."""
+    from fla_amd.ops.common.chunk_h import chunk_bwd_dh
+    from oracle import chunked, cumsum
+    B, T, H, K, V = 2, 200, 2, 64, 128
+    HQ = NG * H
+    gen = torch.Generator().manual_seed(7 + NG)
+    q = torch.randn(B, T, HQ, K, generator=gen).bfloat16()
+    do = torch.randn(B, T, HQ, V, generator=gen).bfloat16()
+    k = torch.randn(B, T, H, K, generator=gen).bfloat16()
+    v = torch.randn(B, T, H, V, generator=gen).bfloat16()
+    raw = {"gv": F.logsigmoid(torch.randn(B, T, H, V, generator=gen)) / 4,
+           "gk": F.logsigmoid(torch.randn(B, T, H, K, generator=gen)) / 4,
+           "g": F.logsigmoid(torch.randn(B, T, H, generator=gen))}
+    gates_c = {n: (cumsum.chunk_local_cumsum(x, 64) if n == gates else None) for n, x in raw.items()}
+    dht = torch.randn(B, HQ, K, V, generator=gen) * 0.1
+    h0 = torch.zeros(B, H, K, V)
+    scale = K ** -0.5
+    print(f"chunk_bwd_dh gates={gates} NG={NG} head_first={head_first}", flush=True)
+    d = lambda x: None if x is None else x.to(device)
+    hf = lambda x: None if x is None else (x.transpose(1, 2).contiguous() if head_first else x)
+    dh, dh0 = chunk_bwd_dh(d(hf(q)), d(hf(k)), d(hf(v)), d(hf(gates_c["g"])), d(hf(gates_c["gk"])),
+                           d(hf(gates_c["gv"])), d(hf(do)), d(h0), d(dht), scale, head_first=head_first,
+                           chunk_size=64, states_in_fp32=True)
+    torch.cuda.synchronize()
+    rep = lambda x: None if x is None else x.repeat_interleave(NG, dim=2)
+    ref_dh, ref_dh0 = chunked.chunk_bwd_dh(q, rep(gates_c["g"]), rep(gates_c["gk"]), do, dht, scale,
+                                           gv=rep(gates_c["gv"]))
+    if head_first:
+        dh = dh.transpose(1, 2)
+    assert tuple(dh.shape) == (B, -(-T // 64), HQ, K, V) and tuple(dh0.shape) == (B, H, K, V)
+    assert_close("dh", ref_dh, dh, 5e-3)
+    assert_close("dh0", ref_dh0.reshape(B, H, NG, K, V).sum(2), dh0, 5e-3)

@@ -334,43 +334,93 @@ def test_gla_stage_gradients_match_autograd_through_the_chunk_step(offsets):
 
 
 @pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
-@pytest.mark.parametrize("gates", ["gk", "g", "both", "none"])
+@pytest.mark.parametrize("gates", ["gk", "g", "both", "none", "gv", "all"])
 def test_chunk_bwd_dh_matches_autograd_through_the_state_chain(offsets, gates):
     """dh[c] is the gradient of  sum(do * o) + sum(dht * ht)  w.r.t. the state leaving chunk c (taken with a
     zero tap added to every state), dh0 the one w.r.t. the initial state; only the inter-chunk part of o sees
-    the states:  o = (s q e^{g} e^{gk}) h,  h_next = e^{g_last + gk_last} h + (k e^{g_last - g + gk_last - gk})^T v."""
+    the states:  o = ((s q e^{g} e^{gk}) h) e^{gv},
+    h_next = e^{g_last} diag(e^{gk_last}) h diag(e^{gv_last}) + (k e^{gk_last - gk})^T (v e^{g_last - g} e^{gv_last - gv})."""
     B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
     N = B if offsets is None else len(offsets) - 1
     q, k, v = _rand(B, T, H, K, seed=31), _rand(B, T, H, K, seed=32), _rand(B, T, H, V, seed=33)
     gk = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, K, seed=34)), 64, offsets=offsets).to(D)
     g = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, seed=35)), 64, offsets=offsets).to(D)
-    if gates in ("g", "none"):
+    gv = cumsum.chunk_local_cumsum(F.logsigmoid(_rand(B, T, H, V, seed=39)), 64, offsets=offsets).to(D)
+    if gates not in ("gk", "both", "all"):
         gk = None
-    if gates in ("gk", "none"):
+    if gates not in ("g", "both", "all"):
         g = None
+    if gates not in ("gv", "all"):
+        gv = None
     do, dht = _rand(B, T, H, V, seed=36), _rand(N, H, K, V, seed=37)
     h0 = _rand(N, H, K, V, seed=38).requires_grad_()
     scale = 0.41
-    taps, loss = [], 0.
+    taps, loss, entering, finals = [], 0., [], []
     for n, (b, bos, eos) in enumerate(recurrent._spans(B, T, offsets)):
         h = h0[n]
         for s in range(bos, eos, 64):
             e = min(s + 64, eos)
+            entering.append(h.detach())
             lg = torch.zeros(e - s, H, K, dtype=D)
+            lv = torch.zeros(e - s, H, V, dtype=D)
             if g is not None:
                 lg = lg + g[b, s:e][..., None]
             if gk is not None:
                 lg = lg + gk[b, s:e]
-            loss = loss + (do[b, s:e] * torch.einsum('thk,hkv->thv', scale * q[b, s:e] * lg.exp(), h)).sum()
+            if gv is not None:
+                lv = lv + gv[b, s:e]
+            o = torch.einsum('thk,hkv->thv', scale * q[b, s:e] * lg.exp(), h) * lv.exp()
+            loss = loss + (do[b, s:e] * o).sum()
             kd = k[b, s:e] * (lg[-1][None] - lg).exp()
+            vd = v[b, s:e] * (lv[-1][None] - lv).exp()
             tap = torch.zeros(H, K, V, dtype=D, requires_grad=True)
             taps.append(tap)
-            h = h * lg[-1].exp()[:, :, None] + torch.einsum('thk,thv->hkv', kd, v[b, s:e]) + tap
+            h = h * lg[-1].exp()[:, :, None] * lv[-1].exp()[:, None, :] + torch.einsum('thk,thv->hkv', kd, vd) + tap
         loss = loss + (dht[n] * h).sum()
+        finals.append(h.detach())
     grads = torch.autograd.grad(loss, [h0] + taps)
-    dh, dh0 = chunked.chunk_bwd_dh(q, g, gk, do, dht, scale, offsets=offsets, dtype=D)
+    dh, dh0 = chunked.chunk_bwd_dh(q, g, gk, do, dht, scale, offsets=offsets, dtype=D, gv=gv)
     torch.testing.assert_close(dh0, grads[0], rtol=1e-10, atol=1e-10)
     torch.testing.assert_close(dh.reshape(-1, H, K, V), torch.stack(grads[1:], 0), rtol=1e-10, atol=1e-10)
+    # the forward states of the same chain, as chunk_fwd_h restates them
+    hs, ht = chunked.chunk_fwd_h(k, v, g, gk, gv, h0.detach(), offsets=offsets, dtype=D)
+    torch.testing.assert_close(hs.reshape(-1, H, K, V), torch.stack(entering, 0), rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(ht, torch.stack(finals, 0), rtol=1e-10, atol=1e-10)
+
+
+@pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
+@pytest.mark.parametrize("gates", ["gk", "gv", "g", "all"])
+def test_chunk_fwd_h_final_state_matches_the_recurrence(offsets, gates):
+    """The chunked state scan ends where the token-by-token recurrence ends, for every kind of gate (the chunk
+    form takes cumulative gates, the recurrence raw ones), and its stored states are the recurrence's states at
+    the chunk boundaries (checked through a run that stops there)."""
+    B, T, H, K, V = (2 if offsets is None else 1), 150, 2, 8, 6
+    N = B if offsets is None else len(offsets) - 1
+    q, k, v = _rand(B, T, H, K, seed=51), _rand(B, T, H, K, seed=52), _rand(B, T, H, V, seed=53)
+    raw = dict(gk=F.logsigmoid(_rand(B, T, H, K, seed=54)), g=F.logsigmoid(_rand(B, T, H, seed=55)),
+               gv=F.logsigmoid(_rand(B, T, H, V, seed=56)))
+    use = {"gk": ("gk",), "gv": ("gv",), "g": ("g",), "all": ("gk", "g", "gv")}[gates]
+    raw = {n: (x if n in use else None) for n, x in raw.items()}
+    def local_cumsum(x):   # in the test's own precision (the oracle's cumsum returns fp32, like the reference's)
+        out = torch.empty_like(x)
+        for b, bos, eos in recurrent._spans(B, T, offsets):
+            for s in range(bos, eos, 64):
+                out[b, s:min(s + 64, eos)] = torch.cumsum(x[b, s:min(s + 64, eos)], 0)
+        return out
+
+    cum = {n: (None if x is None else local_cumsum(x)) for n, x in raw.items()}
+    h0 = _rand(N, H, K, V, seed=57)
+    hs, ht = chunked.chunk_fwd_h(k, v, cum["g"], cum["gk"], cum["gv"], h0, offsets=offsets, dtype=D)
+    _, rht = recurrent.naive_recurrent_gla(q, k, v, gk=raw["gk"], g=raw["g"], gv=raw["gv"], initial_state=h0,
+                                           output_final_state=True, offsets=offsets, dtype=D)
+    torch.testing.assert_close(ht, rht, rtol=1e-10, atol=1e-10)
+    if offsets is None:
+        # the state entering chunk 1 is the final state of a run over the first 64 tokens
+        cut = lambda x: None if x is None else x[:, :64]
+        _, r64 = recurrent.naive_recurrent_gla(q[:, :64], k[:, :64], v[:, :64], gk=cut(raw["gk"]), g=cut(raw["g"]),
+                                               gv=cut(raw["gv"]), initial_state=h0, output_final_state=True, dtype=D)
+        torch.testing.assert_close(hs[:, 1], r64, rtol=1e-10, atol=1e-10)
+        torch.testing.assert_close(hs[:, 0], h0, rtol=0, atol=0)
 
 
 @pytest.mark.parametrize("offsets", [None, [0, 40, 41, 150]])
