@@ -100,6 +100,14 @@ def test_config2_chunk_gated_delta_rule_varlen_full_size(device):
                                                        beta[:, s:e, h:h + 1].cpu(), output_final_state=True)
             assert_close(f"o[seq {n}, head {h}]", ro, o[:, s:e, h:h + 1], 1e-2)
             assert_close(f"ht[seq {n}, head {h}]", rht, ht[n:n + 1, h:h + 1], 5e-3)
+    # (a2) and on the longest sequence, the one whose serial chain bounds the launch, for one head
+    n = max(range(len(lens)), key=lambda i: lens[i])
+    s, e, h = int(offs[n]), int(offs[n + 1]), 7
+    sl = lambda x: x[:, s:e, h:h + 1].float().cpu()
+    ro, rht = naive_recurrent_gated_delta_rule(sl(q), sl(k), sl(v), gl[:, s:e, h:h + 1].cpu(),
+                                               beta[:, s:e, h:h + 1].cpu(), output_final_state=True)
+    assert_close(f"o[longest seq {n} ({e - s} tokens), head {h}]", ro, o[:, s:e, h:h + 1], 1e-2)
+    assert_close(f"ht[longest seq {n}, head {h}]", rht, ht[n:n + 1, h:h + 1], 5e-3)
     # (b1) the packed batch equals its sequences run one by one
     for n in range(len(lens)):
         s, e = int(offs[n]), int(offs[n + 1])
@@ -158,6 +166,56 @@ def test_config3_decode_step_full_size(device, op):
         ro, rs = ref(sl, S0[b:b + 1, h:h + 1].cpu())
         assert_close(f"o[{b},{h}]", ro, o_all[b:b + 1, :, h:h + 1], 1e-2)
         assert_close(f"state[{b},{h}]", rs, state_in[b:b + 1, h:h + 1], 1e-5)
+
+
+@pytest.mark.parametrize("op", ["gla", "gdr"])
+def test_config3_decode_1000_steps_full_size(device, op):
+    """1000 consecutive in-place decode steps at B=256, H=32, D=128 (what bench.py times): on three (b, h) slices the
+    outputs and the final state equal one fused_recurrent call over the same 1000 tokens to fp32 round-off, and the
+    fp32 naive recurrence within the operator's tolerances."""
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from fla_amd.ops.gla import fused_recurrent_gla
+    from oracle.recurrent import naive_recurrent_gated_delta_rule, naive_recurrent_gla
+    B, H, D, steps = 256, 32, 128, 1000
+    g = torch.Generator(device=device).manual_seed(3)
+    S = torch.randn(B, H, D, D, device=device, generator=g) * 0.1
+    S0 = S.clone()
+    q, v = (torch.randn(B, steps, H, D, device=device, generator=g).bfloat16() for _ in range(2))
+    print(f"config 3: {steps} in-place decode steps, {op}", flush=True)
+    if op == "gla":
+        k = torch.randn(B, steps, H, D, device=device, generator=g).bfloat16()
+        gate = F.logsigmoid(torch.randn(B, steps, H, D, device=device, generator=g))
+        args, fn = (q, k, v, gate), fused_recurrent_gla
+        ref = lambda a, s0: naive_recurrent_gla(a[0].float(), a[1].float(), a[2].float(), a[3], initial_state=s0,
+                                                output_final_state=True)
+    else:
+        k = F.normalize(torch.randn(B, steps, H, D, device=device, generator=g), dim=-1).bfloat16()
+        gate = F.logsigmoid(torch.randn(B, steps, H, device=device, generator=g))
+        beta = torch.randn(B, steps, H, device=device, generator=g).sigmoid()
+        args, fn = (q, k, v, gate, beta), fused_recurrent_gated_delta_rule
+        ref = lambda a, s0: naive_recurrent_gated_delta_rule(a[0].float(), a[1].float(), a[2].float(), a[3], a[4],
+                                                             initial_state=s0, output_final_state=True)
+    picks = ((0, 0), (100, 17), (255, 31))
+    kept = {p: [] for p in picks}
+    with torch.no_grad():
+        for t in range(steps):
+            step = [x[:, t:t + 1].contiguous() for x in args]
+            o, ret = fn(*step, initial_state=S, output_final_state=True, head_first=False, inplace_state=True)
+            for b, h in picks:
+                kept[(b, h)].append(o[b:b + 1, :, h:h + 1])
+    assert ret.data_ptr() == S.data_ptr() and torch.isfinite(S).all()
+    for b, h in picks:
+        a = [x[b:b + 1, :, h:h + 1].contiguous() for x in args]
+        o_all, s_all = fn(*a, initial_state=S0[b:b + 1, h:h + 1].contiguous(), output_final_state=True,
+                          head_first=False)
+        o_steps = torch.cat(kept[(b, h)], 1)
+        # (the launcher picks its slab width from the batch, so the two runs may add in a different order: equal to
+        # fp32 round-off, not bit for bit; the bit-exact step-by-step check at one batch size is the 4-step test above)
+        assert_close(f"o[{b},{h}] steps vs one call", o_all, o_steps, 2e-3)
+        assert_close(f"state[{b},{h}] steps vs one call", s_all, S[b:b + 1, h:h + 1], 1e-5)
+        ro, rs = ref([x.cpu() for x in a], S0[b:b + 1, h:h + 1].cpu())
+        assert_close(f"o[{b},{h}]", ro, o_steps, 1e-2)
+        assert_close(f"state[{b},{h}]", rs, S[b:b + 1, h:h + 1], 1e-4)
 
 
 @pytest.mark.parametrize("op", ["gla", "gdr"])
