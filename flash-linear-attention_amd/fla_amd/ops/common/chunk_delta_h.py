@@ -176,6 +176,47 @@ def chunk_gated_delta_rule_fwd_scan(
     return o, ht
 
 
+def chunk_gated_delta_rule_fwd_onepass(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    g: Optional[torch.Tensor],
+    beta: torch.Tensor,
+    scale: float,
+    initial_state: Optional[torch.Tensor],
+    output_final_state: bool,
+    offsets: Optional[torch.Tensor] = None,
+    seq_order: Optional[torch.Tensor] = None,
+    *,
+    l2norm_eps: Optional[float] = None,
+):
+    """The whole forward (``fla/ops/gated_delta_rule/chunk.py:20-73``) in one launch,
+    ``fla_chunk_gated_delta_rule_fwd_onepass``: ``g`` is the raw per-head log-gate ``[B,T,H]`` (or ``None``), ``beta``
+    ``[B,T,H]``; the prefix sum of the gate, the WY blocks, the state scan and the output stage all happen inside the
+    scan's workgroups.  Seq-first, K in {64, 128}, V a multiple of 64.  Returns ``(o, final_state)``.
+    ``l2norm_eps``: ``q`` and ``k`` are un-normalised and are l2-normalised row by row as they are staged."""
+    be.require_gpu(q, k, v, beta)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    N = B
+    if offsets is not None:
+        N = len(offsets) - 1
+        offsets = offsets.to(torch.int64).contiguous()
+    o = torch.empty_like(v)
+    ht = k.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
+    h0 = None
+    if initial_state is not None:
+        h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
+    if g is not None:
+        g = g.float().contiguous()
+    beta = beta.float().contiguous()
+    be.check(be.lib().fla_chunk_gated_delta_rule_fwd_onepass(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(g), be.ptr(beta), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(offsets),
+        None, be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale), int(l2norm_eps is not None),
+        float(l2norm_eps or 0.0), be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_onepass")
+    return o, ht
+
+
 def chunk_gated_delta_rule_bwd_dhu(
     q: torch.Tensor,
     k: torch.Tensor,

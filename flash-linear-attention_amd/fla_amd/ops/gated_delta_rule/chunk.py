@@ -20,7 +20,7 @@ from ... import _backend as be
 from ...utils import (VarlenPlan, autocast_custom_bwd, autocast_custom_fwd, check_varlen_args, contiguous,
                       empty_batch_result, resolve_offsets)
 from ..common.chunk_delta_h import (chunk_gated_delta_rule_fwd_h, chunk_gated_delta_rule_fwd_h_both,
-                                    chunk_gated_delta_rule_fwd_scan)
+                                    chunk_gated_delta_rule_fwd_onepass, chunk_gated_delta_rule_fwd_scan)
 from ..common.chunk_o import chunk_fwd_o
 from ..utils.cumsum import chunk_local_cumsum
 from .wy_fast import fwd_prepare_scan_operands, fwd_prepare_wy_repr
@@ -35,6 +35,13 @@ _FUSED_MAX_K = 128  # the one-pass forward kernel holds at most 128 key channels
 # second state scan cost more than the memory.  FLA_AMD_RECOMPUTE_STATES=1 (or setting this flag to
 # False) restores the reference's behaviour.
 KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("", "0")
+# FLA_AMD_GDR_ONEPASS=1: a forward that is not differentiated runs as ONE launch (the WY blocks of a chunk are formed
+# inside the scan's workgroups, fla_chunk_gated_delta_rule_fwd_onepass) once 64-column slabs give every CU a
+# workgroup.  Off by default: the launch moves only the operator's own bytes, but the extra work lands on the
+# scan's matrix waves, which are on the critical path of a chunk period, and measured slower than the two launches
+# (212 against 190 us at B=8, T=4096, H=16, K=V=128).
+ONEPASS_FORWARD = os.environ.get("FLA_AMD_GDR_ONEPASS", "0") not in ("", "0")
+_ONEPASS_MIN_WORKGROUPS = 129
 
 
 def _round64(d: int) -> int:
@@ -49,12 +56,14 @@ def _round_k(d: int) -> int:
 def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
                                offsets=None, indices=None, head_first=True, chunk_size=64,
                                *, plan: Optional[VarlenPlan] = None, store_A: bool = True, fused: bool = True,
-                               l2norm_eps: Optional[float] = None):
+                               l2norm_eps: Optional[float] = None, want_g_cumsum: bool = True):
     """Reference-shaped forward (``fla/ops/gated_delta_rule/chunk.py:20-73``): returns
     ``(g_cumsum, o, Aw, Au, final_state)``.  ``fused=False`` runs the reference's steps one by one
     (cumsum, WY representation, state scan, output stage); the default two-launch form does not form
     ``Aw`` / ``Au`` and returns ``None`` for them.  ``l2norm_eps`` (two-launch form only): ``q`` and ``k`` are
-    un-normalised and both launches l2-normalise the rows as they stage them."""
+    un-normalised and both launches l2-normalise the rows as they stage them.  ``want_g_cumsum=False``: the caller
+    does not read the cumulative gates, which lets a large enough batch run as one launch (``g_cumsum`` is then
+    returned as ``None``)."""
     if head_first or chunk_size != BT:
         raise NotImplementedError("fla_amd chunk_gated_delta_rule_fwd: seq-first, chunk size 64 only")
     if offsets is not None and plan is None:
@@ -62,6 +71,13 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
     offs = None if plan is None else plan.offsets
     idx = None if plan is None else plan.indices
     co = None if plan is None else plan.chunk_offsets
+    if fused and ONEPASS_FORWARD and want_g_cumsum is False:
+        N = q.shape[0] if plan is None else plan.N
+        if N * q.shape[2] * (v.shape[-1] // 64) >= _ONEPASS_MIN_WORKGROUPS:
+            o, final_state = chunk_gated_delta_rule_fwd_onepass(
+                q, k, v, g, beta, scale, initial_state, output_final_state, offsets=offs,
+                seq_order=None if plan is None else plan.seq_order, l2norm_eps=l2norm_eps)
+            return None, o, None, None, final_state
     if fused:
         # two launches; Aw / Au are not formed on this path
         AT, g = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, l2norm_eps=l2norm_eps)
@@ -183,7 +199,7 @@ class ChunkGatedDeltaRuleFunction(torch.autograd.Function):
         else:
             _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, h0, output_final_state,
                                                         offsets=offsets, head_first=False, chunk_size=BT,
-                                                        store_A=False, fused=KP <= _FUSED_MAX_K)
+                                                        store_A=False, fused=KP <= _FUSED_MAX_K, want_g_cumsum=False)
             # a backward that recomputes starts from the raw gate, like the reference's
             gc = None if g is None else g.float().contiguous()
         ctx.save_for_backward(q, k, v, gc, beta, h0, offsets, *kept)
@@ -321,6 +337,7 @@ def chunk_gated_delta_rule(
         # nothing to differentiate and nothing to convert: no autograd node, no copies
         _, o, _, _, ht = chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_final_state,
                                                     offsets=offsets, head_first=False, chunk_size=BT, store_A=False,
-                                                    l2norm_eps=1e-6 if use_qk_l2norm_in_kernel else None)
+                                                    l2norm_eps=1e-6 if use_qk_l2norm_in_kernel else None,
+                                                    want_g_cumsum=False)
         return o, ht
     return apply_in_value_slabs(q, k, v, g, beta, scale, initial_state, output_final_state, offsets, head_first)

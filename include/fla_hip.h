@@ -367,6 +367,23 @@ int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const void* k, con
                                                int64_t H, int64_t K, int64_t V, int64_t N, float scale, float eps,
                                                fla_stream_t stream);
 
+/* The whole forward of chunk_gated_delta_rule in ONE launch (fla/ops/gated_delta_rule/chunk.py:20-73: cumsum,
+ * fwd_prepare_wy_repr, chunk_gated_delta_rule_fwd_h, chunk_fwd_o): q, k, v, the raw per-head log-gate g (fp32
+ * [B,T,H] or NULL) and beta (fp32 [B,T,H]) in, o and the final state out; no per-chunk tile crosses memory.  The
+ * serial scan of fla_chunk_gated_delta_rule_fwd_scan with the WY operator of the next chunk formed on its matrix
+ * waves: M = strict_lower(diag(beta) K K^T * Gamma) in 16x16 blocks, the four diagonal blocks inverted in fp32, and
+ * v_new = (I + M)^-1 diag(beta) (v - e^{gamma} (k h)) by block forward substitution.  qk_l2norm: q and k are
+ * un-normalised and every row is replaced by x / sqrt(sum x^2 + l2norm_eps) as it is staged
+ * (fla/layers/gated_deltanet.py:234-235).  Forward without kept intermediates.  K in {64, 128}, V a multiple of 64;
+ * packed batches pass offsets [N+1] (and optionally seq_order, as for fla_chunk_gla_fwd_fused); chunk_offsets is
+ * accepted for symmetry with the two-launch form and not read. */
+int fla_chunk_gated_delta_rule_fwd_onepass(const void* q, const void* k, const void* v, const float* g,
+                                           const float* beta, const float* h0, void* o, float* ht,
+                                           const int64_t* offsets, const int64_t* chunk_offsets,
+                                           const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                                           int64_t K, int64_t V, int64_t N, float scale, int qk_l2norm,
+                                           float l2norm_eps, fla_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Chunked GLA backward (chunk size 64), replaces chunk_gla_bwd
  * (fla/ops/gla/chunk.py:1217-1320: chunk_bwd_dh common/chunk_h.py:338-402,

@@ -502,3 +502,42 @@ def test_chunk_gdr_qk_l2norm_backward(device):
     assert_close("o", ro, o, TOL_O)
     for name, a, b in zip(("dq", "dk", "dv", "dg", "dbeta"), ref, leaves):
         assert_close(name, a.grad, b.grad, 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K,V,T,varlen,gated,h0", [
+    (128, 128, 300, False, True, True), (128, 128, 1000, True, True, True), (64, 128, 130, False, True, False),
+    (128, 64, 65, True, True, True), (64, 64, 1, False, True, True), (128, 128, 63, False, False, True),
+    (128, 128, 257, True, False, False), (128, 256, 200, False, True, True)])
+def test_chunk_gdr_onepass_forward(device, monkeypatch, dtype, K, V, T, varlen, gated, h0):
+    """The one-launch forward (the WY blocks formed inside the scan, block forward substitution instead of the
+    64x64 inverse), forced at these small shapes: against the fp32 recurrence, and against the two-launch form."""
+    import fla_amd.ops.gated_delta_rule.chunk as mod
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    gen = torch.Generator().manual_seed(T + K + V)
+    B, H, N = (1, 3, 4) if varlen else (2, 3, 2)
+    q, k, v, g, beta, s0 = gdr_inputs(B, T, H, K, V, seed=T + 1, dtype=dtype, N=N)
+    if not gated:
+        g = None
+    if not h0:
+        s0 = None
+    offs = random_offsets(T, N, gen) if varlen else None
+    print(f"chunk_gdr one-pass {dtype} K={K} V={V} T={T} varlen={varlen} gated={gated} h0={h0}", flush=True)
+    dev = lambda t: None if t is None else t.to(device)
+    args = (dev(q), dev(k), dev(v), dev(g), dev(beta))
+    kw = dict(initial_state=dev(s0), output_final_state=True, offsets=dev(offs), head_first=False)
+    monkeypatch.setattr(mod, "_ONEPASS_MIN_WORKGROUPS", 1)
+    monkeypatch.setattr(mod, "ONEPASS_FORWARD", True)
+    calls = []
+    real = mod.chunk_gated_delta_rule_fwd_onepass
+    monkeypatch.setattr(mod, "chunk_gated_delta_rule_fwd_onepass", lambda *a, **k2: (calls.append(1), real(*a, **k2))[1])
+    o, ht = mod.chunk_gated_delta_rule(*args, **kw)
+    assert calls, "the one-launch form was not taken"
+    monkeypatch.setattr(mod, "ONEPASS_FORWARD", False)
+    o2, ht2 = mod.chunk_gated_delta_rule(*args, **kw)
+    ro, rht = naive_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=s0, output_final_state=True,
+                                               offsets=None if offs is None else offs.tolist())
+    assert_close("o", ro, o, TOL_O)
+    assert_close("ht", rht, ht, TOL_HT)
+    assert_close("o vs two-launch", o2, o, 6e-3)
+    assert_close("ht vs two-launch", ht2, ht, 6e-3)
