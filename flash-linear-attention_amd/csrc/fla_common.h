@@ -152,6 +152,13 @@ FLA_DEVICE typename Elem<T>::v8 l2norm_piece(typename Elem<T>::v8 x, float eps) 
   return y;
 }
 
+// 1 / sqrt(sum x^2 + eps) of the row this lane's 8-element piece belongs to (N adjacent lanes hold the row): the
+// squares on the packed dot-product instruction, the sum over the lanes as in group_allsum.
+template <typename T, int N>
+FLA_DEVICE float l2norm_rstd(typename Elem<T>::v8 x, float eps) {
+  return __builtin_amdgcn_rsqf(group_allsum<N>(Elem<T>::dot8(x, x, 0.f)) + eps);
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a fence over
 // global memory as well: a wave with global stores in flight then drains its whole vector
 // memory queue (loads included) at every barrier, which exposes the full memory latency of

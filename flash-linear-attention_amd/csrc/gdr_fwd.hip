@@ -349,7 +349,8 @@ struct PrepParams {
   int H, NTfix;
   void* w;             // KEEP: w = Aw (beta k) [rows, H, K] and Aw [rows, H, 64], what the backward reads
   void* Aw;
-  float l2_eps;        // L2N: every k row is replaced by k / sqrt(sum k^2 + l2_eps) on its way in
+  float l2_eps;        // L2N: k is un-normalised; the launch works with k / sqrt(sum k^2 + l2_eps) ...
+  float* rk_out;       //      ... and leaves the factors 1 / sqrt(sum k^2 + l2_eps), fp32 [rows, H], for the scan
 };
 
 // resident workgroups per CU (register budget): four, or three for the variant that also writes w and Aw
@@ -363,8 +364,10 @@ FLA_DEVICE int tri_block(int tt, int jb) { return tt * (tt + 1) / 2 + jb; }
 // than bound by one resource).
 // KEEP: the forward of a pass that will be differentiated also leaves w = Aw (beta k) and Aw in memory (the WY
 // launch of the reference's decomposition, without a second inversion and a second pass over k).
-// L2N: k arrives un-normalised and is l2-normalised row by row as it is staged (what l2_norm(k) in front of the
-// operator does, fla/layers/gated_deltanet.py:235); a row of K elements sits in K / 8 adjacent lanes.
+// L2N: k arrives un-normalised (what l2_norm(k) in front of the operator would normalise,
+// fla/layers/gated_deltanet.py:235).  The rows are not rewritten: k^ = r k with r = 1 / sqrt(sum k^2 + eps) per row, so
+// k^ k^T = diag(r) (k k^T) diag(r) and the factors go onto the rows and columns of the product; r comes from the
+// pieces the lanes hold anyway (a row of K elements sits in K / 8 adjacent lanes) and is left in memory for the scan.
 template <typename T, int K, bool KEEP, bool L2N = false>
 __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void gdr_fwd_prep_kernel(PrepParams p, int64_t total) {
   static_assert(!(KEEP && L2N), "a forward that keeps w and Aw takes normalised keys");
@@ -377,6 +380,7 @@ __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void
   __shared__ __attribute__((aligned(16))) char sRB[R_BYTES];   // X (fp32) -> KEEP: k row-major again
   __shared__ __attribute__((aligned(16))) float sBeta[BT];
   __shared__ __attribute__((aligned(16))) float sGam[BT];
+  __shared__ __attribute__((aligned(16))) float sRk[L2N ? BT : 4];   // L2N: 1 / |k_t| (zero past the end of the chunk)
   T* sK = (T*)sRA;
   float* sM = (float*)sRA;
   T* sK2 = (T*)sRB;
@@ -468,8 +472,14 @@ __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
       const int row = r0 + RPP * i;
-      v8 kr = cur.k[i];
-      if constexpr (L2N) kr = l2norm_piece<T, K / 8>(kr, p.l2_eps);
+      const v8 kr = cur.k[i];
+      if constexpr (L2N) {
+        const float rk = l2norm_rstd<T, K / 8>(kr, p.l2_eps);
+        if (c8 == 0) {
+          sRk[row] = row < L ? rk : 0.f;
+          if (row < L) p.rk_out[(row0 + row) * H + hh] = rk;
+        }
+      }
       *(v8*)&sK[row * LDK + c8] = row < L ? kr : z;
     }
     if (wave == 0) {
@@ -509,7 +519,13 @@ __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int ib = qi * 32 + 8 * r4 + 4 * (lane >> 5);
-        const f32x4 b = *(const f32x4*)&sBeta[ib];
+        f32x4 b = *(const f32x4*)&sBeta[ib];
+        if constexpr (L2N) {
+          const f32x4 ri = *(const f32x4*)&sRk[ib];
+          const float rj = sRk[j];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) b[e] *= ri[e] * rj;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) sM[(ib + e) * LDM + j] = (j < ib + e) ? b[e] * s[4 * r4 + e] : 0.f;
       }
@@ -1200,8 +1216,9 @@ int launch_prep(const PrepParams& p, int K, dim3 chunk_grid_, hipStream_t st) {
 static int gdr_fwd_prep_impl(const void* k, const float* beta, const float* g, int g_is_cumsum,
                              float* g_cumsum_out, void* AT, void* w, void* Aw, const int64_t* offsets,
                              const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T, int64_t H,
-                             int64_t K, float l2_eps, fla_stream_t stream) {
+                             int64_t K, float l2_eps, fla_stream_t stream, float* rk_out = nullptr) {
   FLA_REQUIRE(k && beta && AT, FLA_E_INVALID);
+  FLA_REQUIRE((l2_eps >= 0.f) == (rk_out != nullptr), FLA_E_INVALID);
   FLA_REQUIRE((w == nullptr) == (Aw == nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && NT >= 0, FLA_E_INVALID);
   FLA_REQUIRE(((uintptr_t)k | (uintptr_t)AT | (uintptr_t)w | (uintptr_t)Aw) % 16 == 0, FLA_E_ALIGNMENT);
@@ -1210,7 +1227,7 @@ static int gdr_fwd_prep_impl(const void* k, const float* beta, const float* g, i
   int rc = chunk_grid(offsets, indices, B, T, H, NT, &grid, &ntfix);
   if (rc) return rc;
   if (grid.x == 0) return FLA_OK;
-  PrepParams p{k, beta, g, g_is_cumsum, g_cumsum_out, AT, offsets, indices, T, (int)H, ntfix, w, Aw, l2_eps};
+  PrepParams p{k, beta, g, g_is_cumsum, g_cumsum_out, AT, offsets, indices, T, (int)H, ntfix, w, Aw, l2_eps, rk_out};
   if (qkv_dtype == FLA_BF16) return launch_prep<bf16>(p, (int)K, grid, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_prep<f16>(p, (int)K, grid, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
@@ -1225,12 +1242,12 @@ extern "C" int fla_gdr_fwd_prep(const void* k, const float* beta, const float* g
 }
 
 extern "C" int fla_gdr_fwd_prep_l2norm(const void* k, const float* beta, const float* g, int g_is_cumsum,
-                                       float* g_cumsum_out, void* AT, const int64_t* offsets,
+                                       float* g_cumsum_out, void* AT, float* k_rstd_out, const int64_t* offsets,
                                        const int64_t* indices, int64_t NT, int qkv_dtype, int64_t B, int64_t T,
                                        int64_t H, int64_t K, float eps, fla_stream_t stream) {
-  FLA_REQUIRE(eps >= 0.f, FLA_E_INVALID);
+  FLA_REQUIRE(eps >= 0.f && k_rstd_out, FLA_E_INVALID);
   return gdr_fwd_prep_impl(k, beta, g, g_is_cumsum, g_cumsum_out, AT, nullptr, nullptr, offsets, indices, NT,
-                           qkv_dtype, B, T, H, K, eps, stream);
+                           qkv_dtype, B, T, H, K, eps, stream, k_rstd_out);
 }
 
 extern "C" int fla_gdr_fwd_wy(const void* k, const void* v, const float* beta, const float* g_cumsum, void* w, void* u,

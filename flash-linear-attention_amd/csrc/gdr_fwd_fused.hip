@@ -60,7 +60,8 @@ struct GdrScanParams {
   int64_t T;
   int H, V, N;
   float scale;
-  float l2_eps;     // L2N: q and k rows are l2-normalised (x / sqrt(sum x^2 + l2_eps)) as they are staged
+  float l2_eps;     // L2N: q and k are un-normalised; the launch works with x / sqrt(sum x^2 + l2_eps) ...
+  const float* rk;  //      ... the factors of k, fp32 [rows, H], come from fla_gdr_fwd_prep_l2norm
 };
 
 // Two 4-element results per lane (16-bit after conversion) -> one 8-element vector per lane: lanes 0-31 keep
@@ -97,9 +98,13 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
 // (64 columns) is the form described above; two (32 columns, waves 2-3 only keep the barriers) doubles the number of
 // workgroups where 64-column slabs would leave half the CUs without one - a CU is fed at a fixed rate, and a
 // 32-column workgroup needs three quarters of the bytes of a 64-column one per chunk.
-// L2N: q and k arrive un-normalised and the staging waves l2-normalise every row on its way to LDS (the two
-// l2_norm launches in front of the operator, fla/layers/gated_deltanet.py:234-235): a row is held by K / 8
-// adjacent lanes, so its sum of squares is four lane exchanges.
+// L2N: q and k arrive un-normalised (the two l2_norm launches in front of the operator,
+// fla/layers/gated_deltanet.py:234-235, are not run).  The rows are not rewritten: with q^ = rq q and k^ = rk k per row,
+// every place the normalised rows enter is linear in them, so the factors ride on quantities that are scaled anyway -
+// rk on e^{gamma} in front of (k h) and on e^{gamma_last - gamma} in the state update, rq and rk on the rows and
+// columns of the score blocks, rq on the scale of the inter-chunk output.  rk comes from the first launch; rq is formed
+// by the staging lanes from the q pieces they hold (a row sits in K / 8 adjacent lanes: four packed dot products and
+// four lane exchanges per piece).
 template <typename T, int K, bool KEEP, int NMW = 4, bool L2N = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
@@ -124,6 +129,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   __shared__ __attribute__((aligned(16))) float sEg[3][BT];      // e^{gamma_t}
   __shared__ __attribute__((aligned(16))) float sEd[3][BT];      // e^{gamma_last - gamma_t}
   __shared__ float sDec[3];                                      // e^{gamma_last}
+  __shared__ __attribute__((aligned(16))) float sRq[L2N ? 3 : 1][L2N ? BT : 4];    // L2N: 1 / |q_t|
+  __shared__ __attribute__((aligned(16))) float sRk[L2N ? 3 : 1][L2N ? BT : 4];    // L2N: 1 / |k_t|
+  __shared__ __attribute__((aligned(16))) float sEgk[L2N ? 3 : 1][L2N ? BT : 4];   // L2N: e^{gamma_t} / |k_t|
 
   const int tid = threadIdx.x, lane = tid & 63;
   // wave-uniform by construction: keeps the role split and the barriers on scalar branches
@@ -182,6 +190,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int ks = 0; ks < KS; ++ks) sc = Elem<T>::mfma16(frag16<T>(Kr, LDR, 16 * tj, 32 * ks, lane), fq[ks], sc);
         const float gi = sGam[b3][16 * ti + c];
         const f32x4 gj = *(const f32x4*)&sGam[b3][16 * tj + 4 * g];
+        if constexpr (L2N) {
+          const float ri = sRq[b3][16 * ti + c];
+          const f32x4 rj = *(const f32x4*)&sRk[b3][16 * tj + 4 * g];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sc[r] *= ri * rj[r];
+        }
         v4 o;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
@@ -209,6 +223,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       v8 a0, a1;
       v4 v[RV];
       uint32_t gam;  // fp32 bits
+      uint32_t rk;   // L2N: fp32 bits
     };
     // The steady state carries no address arithmetic: byte offsets of this lane's pieces from the
     // chunk's first row are computed once and the chunk base pointers advance by constant strides.
@@ -228,6 +243,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // queue at the join); without gates it reads a dummy address and the bits are masked to zero.
     const uint32_t gmask = p.gam ? 0xffffffffu : 0u;
     const char* lg = p.gam ? (const char*)p.gam + row00 * 4 : lq;
+    const char* lr = L2N ? (const char*)p.rk + row00 * 4 : lq;
+    const int64_t strr = (int64_t)BT * H * 4;
     char* so = (char*)p.o + (row00 * V + vbase) * 2;
     const int64_t strk = (int64_t)BT * HK * 2, strv = (int64_t)BT * HV * 2;
     const int64_t stra = (int64_t)H * ATS * 2;
@@ -257,10 +274,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         R.k[i] = *(const v8*)(lk + o);
       }
       R.gam = *(const uint32_t*)(lg + (offg < limg ? offg : limg));
+      if constexpr (L2N) R.rk = *(const uint32_t*)(lr + (offg < limg ? offg : limg));
       if (lcq + 1 < nchunks) {
         lq += strk;
         lk += strk;
         lg += strg;
+        if constexpr (L2N) lr += strr;
       }
       ++lcq;
     };
@@ -298,8 +317,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       if constexpr (L2N) {
 #pragma unroll
         for (int i = 0; i < NPW; ++i) {
-          R.q[i] = l2norm_piece<T, K / 8>(R.q[i], p.l2_eps);
-          R.k[i] = l2norm_piece<T, K / 8>(R.k[i], p.l2_eps);
+          const float rq = l2norm_rstd<T, K / 8>(R.q[i], p.l2_eps);
+          if (st % C8 == 0) sRq[wq3][q_row(st + 256 * i)] = rq;
         }
       }
 #pragma unroll
@@ -312,7 +331,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const float glast = __uint_as_float(__builtin_amdgcn_readlane(R.gam & gmask, 63));
         sGam[wq3][lane] = gam;
         sEg[wq3][lane] = __expf(gam);
-        sEd[wq3][lane] = __expf(glast - gam);
+        if constexpr (L2N) {
+          const float rk = __uint_as_float(R.rk);
+          sRk[wq3][lane] = rk;
+          sEgk[wq3][lane] = __expf(gam) * rk;
+          sEd[wq3][lane] = __expf(glast - gam) * rk;
+        } else {
+          sEd[wq3][lane] = __expf(glast - gam);
+        }
         if (lane == 0) sDec[wq3] = __expf(glast);
       }
       ++wq;
@@ -535,7 +561,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         v8 ft[6];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-          eg[tt] = *(const f32x4*)&sEg[b3][16 * tt + 4 * g];
+          if constexpr (L2N) eg[tt] = *(const f32x4*)&sEgk[b3][16 * tt + 4 * g];   // e^{gamma} / |k|, for the (k h) term
+          else eg[tt] = *(const f32x4*)&sEg[b3][16 * tt + 4 * g];
           ed[tt] = *(const f32x4*)&sEd[b3][16 * tt + 4 * g];
           vv[tt] = *(const v4*)(vt + swz_t(vrow, 16 * tt + 4 * g));
         }
@@ -572,6 +599,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         vn[3] = Elem<T>::mfma16(ft[4], rb[0], zero4());
         vn[2] = Elem<T>::mfma16(ft[3], rb[1], vn[2]);
         vn[3] = Elem<T>::mfma16(ft[5], rb[1], vn[3]);
+        if constexpr (L2N) {
+          // the (q h) term carries e^{gamma} / |q| instead
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt) {
+            const f32x4 e = *(const f32x4*)&sEg[b3][16 * tt + 4 * g];
+            const f32x4 rq = *(const f32x4*)&sRq[b3][16 * tt + 4 * g];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) eg[tt][r] = e[r] * rq[r];
+          }
+        }
         v8 vnb[2], vsb[2];  // v_new and its decayed copy as operands contracting over time
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
@@ -676,8 +713,9 @@ static int gdr_fwd_scan_impl(const void* q, const void* k, const void* v, const 
                              const float* h0, void* o, float* ht, void* v_new, void* h_frag_t, void* Aqk_out,
                              const int64_t* offsets, const int64_t* chunk_offsets, const int64_t* seq_order,
                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
-                             float scale, float l2_eps, fla_stream_t stream) {
+                             float scale, float l2_eps, fla_stream_t stream, const float* k_rstd = nullptr) {
   FLA_REQUIRE(q && k && v && AT && o, FLA_E_INVALID);
+  FLA_REQUIRE((l2_eps >= 0.f) == (k_rstd != nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
   FLA_REQUIRE(V % 64 == 0 && H <= 0x7fffff, FLA_E_UNSUPPORTED);
@@ -686,7 +724,7 @@ static int gdr_fwd_scan_impl(const void* q, const void* k, const void* v, const 
   FLA_REQUIRE(((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)AT | (uintptr_t)o | (uintptr_t)v_new |
                (uintptr_t)h_frag_t | (uintptr_t)Aqk_out) % 16 == 0, FLA_E_ALIGNMENT);
   GdrScanParams p{q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets, seq_order, T,
-                  (int)H, (int)V, (int)N, scale, l2_eps};
+                  (int)H, (int)V, (int)N, scale, l2_eps, k_rstd};
   if (qkv_dtype == FLA_BF16) return launch_scan<bf16>(p, (int)K, (hipStream_t)stream);
   if (qkv_dtype == FLA_F16) return launch_scan<f16>(p, (int)K, (hipStream_t)stream);
   return FLA_E_UNSUPPORTED;
@@ -703,12 +741,13 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k,
 }
 
 extern "C" int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const void* k, const void* v, const void* AT,
-                                                          const float* g_cumsum, const float* h0, void* o, float* ht,
+                                                          const float* g_cumsum, const float* k_rstd, const float* h0,
+                                                          void* o, float* ht,
                                                           const int64_t* offsets, const int64_t* chunk_offsets,
                                                           const int64_t* seq_order, int qkv_dtype, int64_t B,
                                                           int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                                                           float scale, float eps, fla_stream_t stream) {
-  FLA_REQUIRE(eps >= 0.f, FLA_E_INVALID);
+  FLA_REQUIRE(eps >= 0.f && k_rstd, FLA_E_INVALID);
   return gdr_fwd_scan_impl(q, k, v, AT, g_cumsum, h0, o, ht, nullptr, nullptr, nullptr, offsets, chunk_offsets,
-                           seq_order, qkv_dtype, B, T, H, K, V, N, scale, eps, stream);
+                           seq_order, qkv_dtype, B, T, H, K, V, N, scale, eps, stream, k_rstd);
 }

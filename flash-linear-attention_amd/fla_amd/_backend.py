@@ -53,8 +53,8 @@ SIGNATURES = {
     "fla_chunk_gated_delta_rule_fwd_h_both": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, P]),
     "fla_gdr_fwd_prep": (c_int, [P, P, P, I, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 14 + [I, I64, I64, I64, I64, I64, I64, F, P]),
-    "fla_gdr_fwd_prep_l2norm": (c_int, [P, P, P, I, P, P, P, P, I64, I, I64, I64, I64, I64, F, P]),
-    "fla_chunk_gated_delta_rule_fwd_scan_l2norm": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, F, P]),
+    "fla_gdr_fwd_prep_l2norm": (c_int, [P, P, P, I, P, P, P, P, P, I64, I, I64, I64, I64, I64, F, P]),
+    "fla_chunk_gated_delta_rule_fwd_scan_l2norm": (c_int, [P] * 12 + [I, I64, I64, I64, I64, I64, I64, F, F, P]),
     "fla_chunk_gated_delta_rule_fwd_onepass": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, I, F, P]),
     "fla_chunk_fwd_o": (c_int, [P, P, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, I64, F, P]),
     "fla_chunk_gla_bwd": (c_int, [P] * 17 + [I64, I, I, I64, I64, I64, I64, I64, I64, F, P]),

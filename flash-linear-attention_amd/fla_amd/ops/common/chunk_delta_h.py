@@ -130,6 +130,7 @@ def chunk_gated_delta_rule_fwd_scan(
     *,
     keep: bool = False,
     l2norm_eps: Optional[float] = None,
+    k_rstd: Optional[torch.Tensor] = None,
 ):
     """Serial half of the one-pass forward (``fla_chunk_gated_delta_rule_fwd_scan``): the work of
     ``chunk_gated_delta_rule_fwd_h`` followed by ``chunk_fwd_o`` (``fla/ops/gated_delta_rule/chunk.py:47-72``)
@@ -138,8 +139,9 @@ def chunk_gated_delta_rule_fwd_scan(
     Returns ``(o, final_state)``; with ``keep`` also ``v_new``, the state entering every chunk in
     transposed-fragment order (``[B, NT, H, K, V]``) and the packed score tiles ``Aqk``
     (``[chunks, H, 10, 16, 16]``), what the backward reads: ``(o, final_state, v_new, hT, Aqk)``.
-    ``l2norm_eps``: ``q`` and ``k`` are un-normalised and the launch l2-normalises their rows as it stages them
-    (``fla_chunk_gated_delta_rule_fwd_scan_l2norm``; not with ``keep``)."""
+    ``l2norm_eps``: ``q`` and ``k`` are un-normalised and the launch works with their l2-normalised rows
+    (``fla_chunk_gated_delta_rule_fwd_scan_l2norm``; ``k_rstd`` are the factors of ``k`` that
+    ``fwd_prepare_scan_operands(..., l2norm_eps=...)`` returned; not with ``keep``)."""
     be.require_gpu(q, k, v, AT)
     B, T, H, K = k.shape
     V = v.shape[-1]
@@ -162,8 +164,10 @@ def chunk_gated_delta_rule_fwd_scan(
     if l2norm_eps is not None:
         if keep:
             raise ValueError("l2norm_eps: forward without kept intermediates only")
+        if k_rstd is None:
+            raise ValueError("l2norm_eps: the scan needs k_rstd from fwd_prepare_scan_operands")
         be.check(be.lib().fla_chunk_gated_delta_rule_fwd_scan_l2norm(
-            be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(h0), be.ptr(o), be.ptr(ht),
+            be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(AT), be.ptr(g), be.ptr(k_rstd), be.ptr(h0), be.ptr(o), be.ptr(ht),
             be.ptr(offsets), be.ptr(chunk_offsets), be.ptr(seq_order), be.dt(k), B, T, H, K, V, N, float(scale),
             float(l2norm_eps), be.stream_of(k)), "fla_chunk_gated_delta_rule_fwd_scan_l2norm")
         return o, ht

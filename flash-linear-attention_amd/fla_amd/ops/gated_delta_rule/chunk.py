@@ -80,11 +80,11 @@ def chunk_gated_delta_rule_fwd(q, k, v, g, beta, scale, initial_state, output_fi
             return None, o, None, None, final_state
     if fused:
         # two launches; Aw / Au are not formed on this path
-        AT, g = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, l2norm_eps=l2norm_eps)
+        AT, g, *rstd = fwd_prepare_scan_operands(k, beta, g, offsets=offs, indices=idx, l2norm_eps=l2norm_eps)
         o, final_state = chunk_gated_delta_rule_fwd_scan(q, k, v, AT, g, scale, initial_state, output_final_state,
                                                          offsets=offs, chunk_offsets=co,
                                                          seq_order=None if plan is None else plan.seq_order,
-                                                         l2norm_eps=l2norm_eps)
+                                                         l2norm_eps=l2norm_eps, k_rstd=rstd[0] if rstd else None)
         return g, o, None, None, final_state
     if l2norm_eps is not None:
         raise ValueError("l2norm_eps needs the two-launch form")

@@ -75,8 +75,9 @@ def fwd_prepare_scan_operands(
     ``[B, T, H]`` (or its chunk-local cumsum with ``g_is_cumsum``; ``None`` for the un-gated rule).
     Seq-first, K in {64, 128}.  Returns ``(AT, g_cumsum)``; with ``keep_w`` the launch also writes
     ``w = Aw (beta k)`` and ``Aw`` (what ``fwd_prepare_wy_repr`` leaves for the backward) and the return value
-    is ``(AT, g_cumsum, w, Aw)``.  ``l2norm_eps``: ``k`` is un-normalised and the launch l2-normalises its rows
-    as it stages them (``fla_gdr_fwd_prep_l2norm``; not with ``keep_w``)."""
+    is ``(AT, g_cumsum, w, Aw)``.  ``l2norm_eps``: ``k`` is un-normalised and the launch works with its
+    l2-normalised rows (``fla_gdr_fwd_prep_l2norm``; not with ``keep_w``); the return value is then
+    ``(AT, g_cumsum, k_rstd)`` with the per-row factors ``1 / sqrt(sum k^2 + eps)`` (fp32 ``[B,T,H]``) the scan reads."""
     be.require_gpu(k, beta)
     B, T, H, K = k.shape
     NT = 0
@@ -95,11 +96,12 @@ def fwd_prepare_scan_operands(
     if l2norm_eps is not None:
         if keep_w:
             raise ValueError("l2norm_eps: forward without kept intermediates only")
+        k_rstd = k.new_empty(B, T, H, dtype=torch.float32)
         be.check(be.lib().fla_gdr_fwd_prep_l2norm(
             be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc), be.ptr(AT),
-            be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, float(l2norm_eps), be.stream_of(k)),
-            "fla_gdr_fwd_prep_l2norm")
-        return AT, gc
+            be.ptr(k_rstd), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K, float(l2norm_eps),
+            be.stream_of(k)), "fla_gdr_fwd_prep_l2norm")
+        return AT, gc, k_rstd
     be.check(be.lib().fla_gdr_fwd_prep(
         be.ptr(k), be.ptr(beta), be.ptr(g), int(g_is_cumsum), be.ptr(None if g_is_cumsum else gc),
         be.ptr(AT), be.ptr(w), be.ptr(Aw), be.ptr(offsets), be.ptr(indices), NT, be.dt(k), B, T, H, K,

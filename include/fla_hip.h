@@ -352,17 +352,20 @@ int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k, const void
                                         const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
                                         int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
-/* The same two launches on un-normalised q and k: every q and k row is replaced by x / sqrt(sum x^2 + eps) as it
- * is staged, the two l2_norm launches a gated DeltaNet layer runs in front of the operator
- * (fla/layers/gated_deltanet.py:234-235, fla/modules/l2norm.py:18-40), so the normalised tensors are never
- * written or read.  Forward without kept intermediates; a pass that will be differentiated runs
- * fla_l2norm_fwd / _bwd either side of the entry points above. */
+/* The same two launches on un-normalised q and k: the operator works with x / sqrt(sum x^2 + eps) in place of every
+ * q and k row, what the two l2_norm launches a gated DeltaNet layer runs in front of it leave
+ * (fla/layers/gated_deltanet.py:234-235, fla/modules/l2norm.py:18-40), without writing or reading normalised tensors:
+ * every place a normalised row enters is linear in it, so the per-row factors ride on quantities the kernels scale
+ * anyway.  The first launch leaves the factors of k in k_rstd_out (fp32 [B,T,H]) for the second, which forms those
+ * of q itself.  Forward without kept intermediates; a pass that will be differentiated runs fla_l2norm_fwd / _bwd
+ * either side of the entry points above. */
 int fla_gdr_fwd_prep_l2norm(const void* k, const float* beta, const float* g, int g_is_cumsum, float* g_cumsum_out,
-                            void* AT, const int64_t* offsets, const int64_t* indices, int64_t NT, int qkv_dtype,
-                            int64_t B, int64_t T, int64_t H, int64_t K, float eps, fla_stream_t stream);
+                            void* AT, float* k_rstd_out, const int64_t* offsets, const int64_t* indices, int64_t NT,
+                            int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, float eps,
+                            fla_stream_t stream);
 int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const void* k, const void* v, const void* AT,
-                                               const float* g_cumsum, const float* h0, void* o, float* ht,
-                                               const int64_t* offsets, const int64_t* chunk_offsets,
+                                               const float* g_cumsum, const float* k_rstd, const float* h0, void* o,
+                                               float* ht, const int64_t* offsets, const int64_t* chunk_offsets,
                                                const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
                                                int64_t H, int64_t K, int64_t V, int64_t N, float scale, float eps,
                                                fla_stream_t stream);

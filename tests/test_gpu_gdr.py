@@ -476,8 +476,8 @@ def test_chunk_gdr_qk_l2norm_in_kernel(device, dtype, K, V, T, varlen):
     o2, ht2 = chunk_gated_delta_rule(l2norm_fwd(dev(q)), l2norm_fwd(dev(k)), dev(v), dev(g), dev(beta),
                                      initial_state=dev(h0), output_final_state=True, offsets=dev(offs),
                                      head_first=False)
-    assert_close("o vs two-step", o2, o, 3e-3)
-    assert_close("ht vs two-step", ht2, ht, 2e-3)
+    assert_close("o vs two-step", o2, o, 6e-3)
+    assert_close("ht vs two-step", ht2, ht, 6e-3)
 
 
 def test_chunk_gdr_qk_l2norm_backward(device):
