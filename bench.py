@@ -332,6 +332,51 @@ def bench_decode(device, steps=1000):
     return out
 
 
+def bench_decode_layer_step(device, steps=300):
+    """One token through what a gated DeltaNet layer runs around its state update at the decode shape (B=256, H=32,
+    D=128): short-convolution step, l2 norm of q and k, the in-place recurrent step, gated RMS norm of the output -
+    five launches - run eagerly (wall time per step, host included) and replayed from one captured HIP graph."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.modules import FusedRMSNormSwishGate, ShortConvolution, l2_norm
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    torch.manual_seed(0)
+    B, H, D, W = 256, 32, 128, 4
+    conv = ShortConvolution(H * D, W, activation="silu").to(device).bfloat16()
+    norm = FusedRMSNormSwishGate(D).to(device)
+    x = torch.randn(B, 1, H * D, device=device).bfloat16()
+    gate_in = torch.randn(B, 1, H * D, device=device).bfloat16()
+    g = F.logsigmoid(torch.randn(B, 1, H, device=device))
+    beta = torch.rand(B, 1, H, device=device)
+    state = torch.randn(B, H, D, D, device=device) * 0.1
+    cache = torch.zeros(B, H * D, W, device=device, dtype=torch.bfloat16)
+
+    def step():
+        y, _ = conv(x, cache=cache)
+        q = l2_norm(y.view(B, 1, H, D))
+        k = l2_norm(torch.roll(y, 1, dims=-1).view(B, 1, H, D))
+        o, _ = fused_recurrent_gated_delta_rule(q, k, y.view(B, 1, H, D), g, beta, initial_state=state,
+                                                output_final_state=True, head_first=False, inplace_state=True)
+        return norm(o, gate_in.view(B, 1, H, D))
+
+    with torch.no_grad():
+        st_e = event_stats(step, steps, 20)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        st_g = event_stats(graph.replay, steps, 20)
+    assert torch.isfinite(state).all()
+    return {"launches_per_step": 6, "eager_wall_us_per_step": round(st_e["wall_us_per_call"], 1),
+            "eager_event_median_us": round(st_e["median_us"], 1),
+            "hip_graph_replay_wall_us_per_step": round(st_g["wall_us_per_call"], 1),
+            "hip_graph_replay_event_median_us": round(st_g["median_us"], 1)}
+
+
 def bench_gdr(device, steps=50, warmup=20):
     """chunk_gated_delta_rule forward: the packed workload (12 sequences, 32768 tokens) and the
     fixed-length shape B=8, T=4096 of the headline metric.  Each row carries a roofline block for its
@@ -448,14 +493,46 @@ def bench_backward(device, steps=20):
 
     leaves.extend([q, k, v, gk, h0, kn, g, beta])
 
-    for name, fn in (("chunk_gla", gla_step), ("chunk_gated_delta_rule", gdr_step)):
+    import fla_amd.ops.gated_delta_rule.chunk as gdr_mod
+    import fla_amd.ops.gla.chunk as gla_mod
+
+    def saved_bytes(forward):
+        """Bytes a forward keeps for its backward: distinct storages among the tensors autograd saves (the operator's
+        inputs included; `inputs_bytes` says how much of it they are)."""
+        seen = {}
+
+        def pack(t):
+            seen[t.untyped_storage().data_ptr()] = t.untyped_storage().nbytes()
+            return t
+
+        with torch.autograd.graph.saved_tensors_hooks(pack, lambda t: t):
+            outs = forward()
+        del outs
+        return sum(seen.values())
+
+    gla_fwd = lambda: chunk_gla(q, k, v, gk, initial_state=h0, output_final_state=True, head_first=False)
+    gdr_fwd = lambda: chunk_gated_delta_rule(q, kn, v, g, beta, initial_state=h0, output_final_state=True,
+                                             head_first=False)
+    nbytes = lambda *ts: sum(t.numel() * t.element_size() for t in ts)
+    for name, fn, mod, fwd, ins in (("chunk_gla", gla_step, gla_mod, gla_fwd, (q, k, v, gk, h0)),
+                                    ("chunk_gated_delta_rule", gdr_step, gdr_mod, gdr_fwd, (q, kn, v, g, beta, h0))):
         st = event_stats(fn, steps, 5)
         us = st["median_us"]
         # forward + backward FLOPs (dense-tile counts): GLA 10KV + 4*BT*(K+V); delta rule 16KV + 2*BT*(9K+5V) + 8*BT^2
         fl = B * T * H * ((10 * K * V + 4 * 64 * (K + V)) if name == "chunk_gla"
                           else (16 * K * V + 2 * 64 * (9 * K + 5 * V) + 8 * 64 * 64))
         out[name] = {"fwd_bwd_us": round(us, 1), **spread(st), "tokens_per_s": round(B * T / (us * 1e-6), 1),
-                     "algorithmic_flops": fl, "frac_of_mfma_peak": round(fl / (us * 1e-6) / MFMA_PEAK_FLOPS, 4)}
+                     "algorithmic_flops": fl, "frac_of_mfma_peak": round(fl / (us * 1e-6) / MFMA_PEAK_FLOPS, 4),
+                     "inputs_bytes": nbytes(*ins), "saved_for_backward_bytes": saved_bytes(fwd)}
+        # the reference's trade: nothing but the inputs (and the gate-range flags) kept, states recomputed in the backward
+        mod.KEEP_STATES_FOR_BACKWARD = False
+        try:
+            st_r = event_stats(fn, steps, 5)
+            out[name]["recompute_states"] = {"fwd_bwd_us": round(st_r["median_us"], 1),
+                                             "saved_for_backward_bytes": saved_bytes(fwd)}
+        finally:
+            mod.KEEP_STATES_FOR_BACKWARD = True
+        clear()
     return out
 
 
@@ -659,6 +736,56 @@ def bench_layer_fusion(device, steps=20):
     return out
 
 
+def bench_fp32_inputs(device, steps=5):
+    """chunk_gla on fp32 q, k, v (the reference's own tests run the operator in fp32): the token-by-token fp32 kernels
+    serve it, exact to 1e-4 and serial in time; timed at B=8, T=4096, H=16, K=V=128."""
+    import torch
+    import torch.nn.functional as F
+    from fla_amd.ops.gla import chunk_gla
+    B, T, H, D = 8, 4096, 16, 128
+    gen = torch.Generator(device=device).manual_seed(8)
+    q, k, v = (torch.randn(B, T, H, D, device=device, generator=gen) for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, T, H, D, device=device, generator=gen)) / 16
+    h0 = torch.randn(B, H, D, D, device=device, generator=gen) * 0.1
+    import fla_amd.ops.gla.chunk as mod
+    fn = lambda: chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
+    with torch.no_grad():
+        us = event_avg_us(fn, steps, warmup=2, ramp=0.0)
+        # opt-in (FLA_AMD_FP32_VIA_FP16=1): q, k, v rounded to fp16 and the chunk kernels run; the casts are part of the call
+        mod.FP32_INPUTS_VIA_FP16_CHUNK = True
+        try:
+            us16 = event_avg_us(fn, 20)
+        finally:
+            mod.FP32_INPUTS_VIA_FP16_CHUNK = False
+    return {"us": round(us, 1), "tokens_per_s": round(B * T / us * 1e6, 1),
+            "via_fp16_chunk_kernels_us": round(us16, 1)}
+
+
+def bench_gdr_onepass(device, steps=30):
+    """The one-launch form of chunk_gated_delta_rule forward (opt-in, FLA_AMD_GDR_ONEPASS=1) beside the default two
+    launches at B=8, T=4096, H=16, K=V=128: fewer bytes and one launch, but the extra work sits on the scan's matrix
+    waves."""
+    import torch
+    import torch.nn.functional as F
+    import fla_amd.ops.gated_delta_rule.chunk as mod
+    B, T, H, D = 8, 4096, 16, 128
+    gen = torch.Generator(device=device).manual_seed(9)
+    q = torch.randn(B, T, H, D, device=device, generator=gen).bfloat16()
+    k = F.normalize(torch.randn(B, T, H, D, device=device, generator=gen), dim=-1).bfloat16()
+    v = torch.randn(B, T, H, D, device=device, generator=gen).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, device=device, generator=gen))
+    beta = torch.randn(B, T, H, device=device, generator=gen).sigmoid()
+    fn = lambda: mod.chunk_gated_delta_rule(q, k, v, g, beta, output_final_state=True, head_first=False)
+    out = {}
+    for flag, name in ((False, "two_launches_us"), (True, "one_launch_us")):
+        mod.ONEPASS_FORWARD = flag
+        try:
+            out[name] = round(event_avg_us(fn, steps), 1)
+        finally:
+            mod.ONEPASS_FORWARD = False
+    return out
+
+
 def cpu_baseline(c, budget_s=15.0):
     """The oracle's fp32 naive recurrence on the host cores, over as many whole
     sequences of the same workload as fit in about `budget_s` seconds."""
@@ -716,10 +843,13 @@ def main():
     extra = {"chunk_gla_fwd": op}
     if not a.no_extra:
         extra["decode_step"] = bench_decode(device)
+        extra["decode_layer_step"] = bench_decode_layer_step(device)
         extra["chunk_gated_delta_rule_fwd"] = bench_gdr(device)
         extra["fwd_bwd_config4"] = bench_backward(device)
         extra["layer_steps"] = bench_layer_steps(device)
         extra["layer_fusion"] = bench_layer_fusion(device)
+        extra["chunk_gla_fp32_inputs"] = bench_fp32_inputs(device)
+        extra["chunk_gated_delta_rule_fwd_one_launch"] = bench_gdr_onepass(device)
         extra["chunk_simple_gla_fwd"] = bench_simple_gla(device)
         extra["gla_stages_reference_operands"] = bench_gla_stages(device)
         extra["device_copy_1GiB"] = bench_copy(device)

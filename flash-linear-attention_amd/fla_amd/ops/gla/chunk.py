@@ -31,6 +31,11 @@ KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("
 # With the states, a differentiated forward (per-key gates, V <= 128) also keeps k^ = k e^{G_last - G} and the score tile
 # of every chunk (1.5 more tensors of k's size), from which the backward's reverse state scan forms dv on its way.
 KEEP_KHAT_AND_SCORES = os.environ.get("FLA_AMD_GLA_FUSED_DV", "1") not in ("", "0")
+# fp32 q/k/v: by default the fp32 token-by-token kernels (exact to 1e-4, serial in time).  FLA_AMD_FP32_VIA_FP16=1 rounds
+# q, k, v to fp16 and runs the chunk kernels instead (gates and states stay fp32): about 5e-4 relative error - inside
+# the 4e-3 the reference's own fp32 tests allow (tests/ops/test_gla.py:195-201) - and some fifty times faster, for
+# inputs whose magnitudes fit fp16 (|x| < 65504; the caller's responsibility).
+FP32_INPUTS_VIA_FP16_CHUNK = os.environ.get("FLA_AMD_FP32_VIA_FP16", "0") not in ("", "0")
 
 
 def _pad_dim(x: Optional[torch.Tensor], size: int) -> Optional[torch.Tensor]:
@@ -645,6 +650,10 @@ def chunk_gla(
     if q.numel() == 0:
         return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
     if q.dtype == torch.float32:
+        if FP32_INPUTS_VIA_FP16_CHUNK:
+            o, ht = chunk_gla(q.half(), k.half(), v.half(), g.float(), scale=scale, initial_state=initial_state,
+                              output_final_state=output_final_state, offsets=offsets, head_first=head_first)
+            return o.float(), ht
         return _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
     K, V = q.shape[-1], v.shape[-1]
     if K > 128:

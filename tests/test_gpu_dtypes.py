@@ -169,3 +169,42 @@ def test_chunk_gla_fp32_inputs(device, T, D, head_first, varlen):
     for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
         assert_close(name, a.grad, tr(b.grad) if head_first else b.grad, 2e-4)
     assert_close("dh0", rh0.grad, h0l.grad, 1e-4)
+
+
+@pytest.mark.parametrize("T,D,varlen", [(300, 128, False), (257, 100, True)])
+def test_chunk_gla_fp32_inputs_via_fp16_chunk_kernels(device, monkeypatch, T, D, varlen):
+    """The opt-in fast route for fp32 q, k, v (rounded to fp16, chunk kernels, fp32 gates and states): forward and
+    backward inside the tolerances of the reference's own fp32 tests (tests/ops/test_gla.py:195-201: 4e-3 on o,
+    5e-3 on the rest), fp32 tensors in and out."""
+    import torch.nn.functional as F
+    import fla_amd.ops.gla.chunk as mod
+    from helpers import assert_close
+    from oracle.recurrent import naive_recurrent_gla
+    B, H = (1, 2) if varlen else (2, 2)
+    N = 3 if varlen else B
+    gen = torch.Generator().manual_seed(T + D)
+    q, k, v = (torch.randn(B, T, H, D, generator=gen) for _ in range(3))
+    g = F.logsigmoid(torch.randn(B, T, H, D, generator=gen))
+    h0 = torch.randn(N, H, D, D, generator=gen)
+    do = torch.randn(B, T, H, D, generator=gen)
+    dht = torch.randn(N, H, D, D, generator=gen) * 0.1
+    offs = torch.tensor([0, 17, 90, T]) if varlen else None
+    print(f"chunk_gla fp32 via fp16 chunk kernels T={T} D={D} varlen={varlen}", flush=True)
+    monkeypatch.setattr(mod, "FP32_INPUTS_VIA_FP16_CHUNK", True)
+    leaves = [x.to(device).requires_grad_() for x in (q, k, v, g)]
+    h0l = h0.to(device).requires_grad_()
+    o, ht = mod.chunk_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=False,
+                          offsets=None if offs is None else offs.to(device))
+    assert o.dtype == torch.float32 and ht.dtype == torch.float32
+    ((o * do.to(device)).sum() + (ht * dht.to(device)).sum()).backward()
+    rl = [x.clone().requires_grad_() for x in (q, k, v, g)]
+    rh0 = h0.clone().requires_grad_()
+    ro, rht = naive_recurrent_gla(*rl, initial_state=rh0, output_final_state=True,
+                                  offsets=None if offs is None else offs.tolist())
+    ((ro * do).sum() + (rht * dht).sum()).backward()
+    assert_close("o", ro, o, 4e-3)
+    assert_close("ht", rht, ht, 5e-3)
+    for name, a, b in zip(("dq", "dk", "dv", "dg"), rl, leaves):
+        assert b.grad.dtype == torch.float32
+        assert_close(name, a.grad, b.grad, 5e-3)
+    assert_close("dh0", rh0.grad, h0l.grad, 5e-3)
