@@ -30,6 +30,9 @@ struct FusedParams {
   // gate_clamp_min) (fla/layers/gla.py:214-217), formed by the staging waves on the way to the prefix sums
   float gate_inv_norm;
   float gate_clamp_min;   // -inf: no clamp
+  // the workgroup redoes the output rows of its own flagged chunks after its last chunk (the 64- and 32-column
+  // kernels; otherwise a second launch does)
+  int exact_tail;
 };
 
 // log2(sigmoid(x)) * inv_norm, clamped from below at clamp2 (both in the log2 domain): two transcendental
@@ -243,7 +246,7 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
     }
     // The scores use one reference point per chunk (e^{G} on q, e^{-G} on k), exact while
     // |G| stays below InvDecayLimit<T>::value.  Chunks beyond that are flagged and recomputed by
-    // the exact kernel afterwards (their q~, k~ tiles may hold infinities: only the scores
+    // the exact routine afterwards (their q~, k~ tiles may hold infinities: only the scores
     // use them, and those are recomputed).
     const int out_of_range = __any(gabs > InvDecayLimit<T>::value * LOG2E);  // wave-uniform
     if (lane == 0) L.wide[buf][pw] = out_of_range;

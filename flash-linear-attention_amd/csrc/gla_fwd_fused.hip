@@ -25,6 +25,206 @@
 
 namespace {
 
+// Exact recomputation of the output rows of flagged chunks: the scores
+//   A_ij = s sum_k q_ik k_jk e^{G_ik - G_jk}   (j <= i)
+// are evaluated pair by pair in fp32 with every exponent <= 0, as the reference does on its
+// diagonal sub-blocks (fla/ops/gla/chunk.py:113-170), then o = (s q e^{G}) h_c + A v on MFMA.
+struct ExactParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* g;
+  const int* wide;
+  const void* hwide;
+  void* o;
+  const int64_t* offsets;
+  const int64_t* indices;
+  int64_t T;
+  int H, NTfix;
+  float scale;
+  int64_t total;   // (chunk, head) pairs
+  int head_gates;  // g is fp32 [B*T, H]: one log-gate per (token, head)
+  int hwide_vk;    // hwide holds [V][K] tiles (the 128-column kernel) instead of fragment-order ones
+  int gate_logits; // g holds gate logits: the log-gate is max(logsigmoid(g) * gate_inv_norm, gate_clamp_min)
+  float gate_inv_norm, gate_clamp_min;
+};
+
+// LDS tiles of one flagged chunk
+template <typename T>
+struct ExactLds {
+  float* g;      // G     [t][k], pitch K + 4
+  T* q;          // q, later s q e^{G}  [t][k], pitch K + 8
+  T* k;          // k     [t][k]
+  T* vt;         // v     [v][t], VS rows, pitch LDT
+  T* p;          // A     [i][j], pitch LDT
+  float* part;   // gate sums of the row groups, [256 / (K / 4)][K]
+};
+
+// One flagged chunk of head hh: output rows of the value columns vbase .. vbase + VS - 1 (V columns per row in
+// memory).  Called by all NTHR threads of a workgroup (NTHR = 256 or 512): the first four waves load, stage and run
+// the matrix products, every thread takes a share of the pairwise scores; the barriers are reached by all.
+template <typename T, typename GT, int K, int VS, int NTHR>
+FLA_DEVICE void gla_exact_chunk(const ExactParams& p, const ExactLds<T>& S, const ChunkLoc& cl, int hh, int V, int vbase,
+                                int tid) {
+  typedef typename Elem<T>::v8 v8;
+  typedef typename Elem<T>::v4 v4;
+  constexpr int LDK = K + 8;
+  constexpr int LDG = K + 4;
+  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
+  constexpr int CGV = VS / 4, RGV = 256 / CGV, RPTV = BT / RGV;
+  constexpr int KT32 = K / 32, TV = VS >= 64 ? VS / 64 : 1;
+  static_assert(NTHR == 256 || NTHR == 512, "threads of the calling workgroup");
+  const int H = p.H;
+  const int lane = tid & 63, wave = tid >> 6;
+  const bool worker = wave < 4;   // wave-uniform
+  const int L = cl.L;
+  const int64_t row0 = cl.row0;
+  const int rg = (tid & 255) / CG, c4 = ((tid & 255) % CG) * 4;
+  float G[RPT][4];
+  v4 qreg[RPT], kreg[RPT];
+  if (worker) {
+    float gq[RPT][4];
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      if (row < L) {
+        int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
+        if (p.head_gates) {
+          const float x = ((const float*)p.g)[(row0 + row) * H + hh];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) gq[i][j] = x;
+        } else {
+          Load<GT>::x4((const GT*)p.g + off, gq[i]);
+          if (p.gate_logits) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              gq[i][j] = log2_sigmoid_gate(gq[i][j], p.gate_inv_norm, p.gate_clamp_min * 1.4426950408889634f) *
+                         0.6931471805599453f;
+          }
+        }
+        qreg[i] = *(const v4*)((const T*)p.q + off);
+        kreg[i] = *(const v4*)((const T*)p.k + off);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gq[i][j] = 0.f;
+        qreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+        kreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      }
+    }
+    const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
+#pragma unroll
+    for (int i = 0; i < RPTV; ++i) {
+      int row = rgv * RPTV + i;
+      v4 x = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+      if (row < L) x = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + vbase + cv4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S.vt[(cv4 + j) * LDT + row] = x[j];
+    }
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < RPT; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        run[j] += gq[i][j];
+        G[i][j] = run[j];
+      }
+    *(f32x4*)&S.part[rg * K + c4] = f32x4{run[0], run[1], run[2], run[3]};
+  }
+  __syncthreads();
+  if (worker) {
+    float off[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int r = 0; r < rg; ++r) {
+      f32x4 pr = *(const f32x4*)&S.part[r * K + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) off[j] += pr[j];
+    }
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      *(f32x4*)&S.g[row * LDG + c4] = f32x4{G[i][0] + off[0], G[i][1] + off[1], G[i][2] + off[2], G[i][3] + off[3]};
+      *(v4*)&S.q[row * LDK + c4] = qreg[i];
+      *(v4*)&S.k[row * LDK + c4] = kreg[i];
+    }
+  }
+  __syncthreads();
+  // ---- exact scores: a thread handles row i and every NQ-th column j <= i
+  {
+    constexpr int NQ = NTHR / BT;
+    const int i = tid / NQ, jq = tid % NQ;
+    for (int j = jq; j < BT; j += NQ) {
+      float a = 0.f;
+      if (j <= i) {
+        for (int kk = 0; kk < K; kk += 4) {
+          f32x4 gi = *(const f32x4*)&S.g[i * LDG + kk];
+          f32x4 gj = *(const f32x4*)&S.g[j * LDG + kk];
+          v4 qv = *(const v4*)&S.q[i * LDK + kk];
+          v4 kv = *(const v4*)&S.k[j * LDK + kk];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a += (float)qv[e] * (float)kv[e] * __expf(gi[e] - gj[e]);
+        }
+      }
+      S.p[i * LDT + j] = (T)(a * p.scale);
+    }
+  }
+  __syncthreads();
+  // ---- q~ = s q e^{G} over the raw q tile (every lane rewrites exactly what it reads)
+  if (worker) {
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      int row = rg * RPT + i;
+      f32x4 gg = *(const f32x4*)&S.g[row * LDG + c4];
+      v4 qv = *(const v4*)&S.q[row * LDK + c4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qv[j] = (T)((float)qv[j] * p.scale * __expf(gg[j]));
+      *(v4*)&S.q[row * LDK + c4] = qv;
+    }
+  }
+  __syncthreads();
+  const int rw = wave >> 1, cw = wave & 1;
+  if (worker && cw * TV * 32 < VS) {
+    f32x16 acc[TV];
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
+    const T* hp = (const T*)p.hwide + (cl.cglob * H + hh) * (int64_t)K * V;
+#pragma unroll
+    for (int kt = 0; kt < KT32; ++kt)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        if (p.hwide_vk) {   // [V][K]: a lane reads 8 consecutive key channels of its value column
+          v8 a = lds_frag32<T>(S.q, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+          for (int tv = 0; tv < TV; ++tv) {
+            v8 b = *(const v8*)(hp + (int64_t)(vbase + (cw * TV + tv) * 32 + (lane & 31)) * K + kt * 32 + half * 16 + 8 * (lane >> 5));
+            acc[tv] = Elem<T>::mfma32(a, b, acc[tv]);
+          }
+        } else {
+          v8 a = lds_frag32_perm<T>(S.q, LDK, rw * 32, kt * 32 + half * 16, lane);
+#pragma unroll
+          for (int tv = 0; tv < TV; ++tv) {
+            v8 b = *(const v8*)(hp + (((int64_t)kt * (V / 32) + (vbase / 32 + cw * TV + tv)) * 64 + lane) * 16 + half * 8);
+            acc[tv] = Elem<T>::mfma32(a, b, acc[tv]);
+          }
+        }
+      }
+    const int jend = (rw + 1) * 32;
+    for (int js = 0; js < jend; js += 16) {
+      v8 a = lds_frag32<T>(S.p, LDT, rw * 32, js, lane);
+#pragma unroll
+      for (int tv = 0; tv < TV; ++tv)
+        acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(S.vt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
+    }
+    T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V + vbase;
+#pragma unroll
+    for (int tv = 0; tv < TV; ++tv)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int i = rw * 32 + c32_row(r, lane);
+        if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
+      }
+  }
+  __syncthreads();   // the tiles are free for the next flagged chunk
+}
+
 // NSTG: number of staging waves (4 or 8); the workgroup has 4 + NSTG waves.
 // HT: the matrix waves also write the state entering every chunk to p.hT, transposed (what the backward
 // kernels contract over v with), for a forward pass whose states are kept instead of being recomputed by
@@ -80,6 +280,7 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     return (int)(rem < BT ? rem : BT);
   };
 
+  int any_wide = 0;   // matrix waves: some chunk of this workgroup was flagged
   if (wave >= 4) {
     // staging waves: see gla_fused_staging.h
     StageLds<T> L{{sQ[0], sQ[1]}, {sK[0], sK[1]}, {sKh[0], sKh[1]}, {sDecay[0], sDecay[1]}, {sWide[0], sWide[1]}, sO};
@@ -267,8 +468,9 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
 #pragma unroll
         for (int w2 = 0; w2 < NSTG; ++w2) wide |= sWide[buf][w2];
         if (tid == 0) p.wide[(chunk0 + c) * H + hh] = wide;
+        any_wide |= wide;
         if (wide) {
-          // hand the state entering this chunk to the exact kernel (fragment order, this slab's columns)
+          // hand over the state entering this chunk for the exact recomputation (fragment order, this slab's columns)
           T* hw = (T*)p.hwide + ((chunk0 + c) * H + hh) * (int64_t)K * V;
           for (int e = tid; e < KT32 * NVT * 64 * 2; e += 256) {
             int piece = e & 1, ln = (e >> 1) & 63, tile = e >> 7;  // tile = kt*NVT + vt
@@ -388,41 +590,34 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
       }
     }
   }
+  // Flagged chunks (rare: chunk-cumulative log-gates beyond the single-reference range): the workgroup redoes the
+  // output rows of its own slab from the states it handed over, in the tiles the scan no longer needs, so the
+  // operator needs no second launch.  Both wave groups take part; every barrier below is reached by all waves.
+  if (p.exact_tail) {
+    if (tid == 0) sWide[0][0] = any_wide;
+    __syncthreads();   // also completes this workgroup's stores: the states handed over and the rows about to be rewritten
+    if (sWide[0][0]) {
+      const ExactParams e{p.q, p.k, p.v, p.g, p.wide, p.hwide, p.o, nullptr, nullptr, p.T, H, 0, p.scale, 0,
+                          SG ? 1 : 0, 0, LOGITS ? 1 : 0, p.gate_inv_norm, p.gate_clamp_min};
+      const ExactLds<T> S{(float*)&sQ[0][0], sK[0], sK[1], sVt[0], sP, (float*)&sKh[0][0]};
+      static_assert(sizeof(sQ) >= BT * (K + 4) * sizeof(float) && sizeof(sKh[0]) >= (256 / (K / 4)) * K * sizeof(float),
+                    "tiles of the exact recomputation fit the scan's");
+      for (int64_t c = 0; c < nchunks; ++c) {
+        // this workgroup's own flag, read past the caches other workgroups' flags of the same line may sit in
+        if (__hip_atomic_load(&p.wide[(chunk0 + c) * H + hh], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) continue;
+        const ChunkLoc cl{sp.bos + c * BT, chunk_len(c), chunk0 + c};
+        gla_exact_chunk<T, GT, K, BV, 256 + 64 * NSTG>(e, S, cl, hh, V, vbase, tid);
+      }
+    }
+  }
 }
 
-// Exact recomputation of the output rows of flagged chunks: the scores
-//   A_ij = s sum_k q_ik k_jk e^{G_ik - G_jk}   (j <= i)
-// are evaluated pair by pair in fp32 with every exponent <= 0, as the reference does on its
-// diagonal sub-blocks (fla/ops/gla/chunk.py:113-170), then o = (s q e^{G}) h_c + A v on MFMA.
-struct ExactParams {
-  const void* q;
-  const void* k;
-  const void* v;
-  const void* g;
-  const int* wide;
-  const void* hwide;
-  void* o;
-  const int64_t* offsets;
-  const int64_t* indices;
-  int64_t T;
-  int H, NTfix;
-  float scale;
-  int64_t total;   // (chunk, head) pairs
-  int head_gates;  // g is fp32 [B*T, H]: one log-gate per (token, head)
-  int hwide_vk;    // hwide holds [V][K] tiles (the 128-column kernel) instead of fragment-order ones
-  int gate_logits; // g holds gate logits: the log-gate is max(logsigmoid(g) * gate_inv_norm, gate_clamp_min)
-  float gate_inv_norm, gate_clamp_min;
-};
-
+// The second launch of the operator where the scan does not redo its flagged chunks itself (the 128-column kernel).
 template <typename T, typename GT, int K, int V>
 __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
-  typedef typename Elem<T>::v8 v8;
-  typedef typename Elem<T>::v4 v4;
   constexpr int LDK = K + 8;
   constexpr int LDG = K + 4;
-  constexpr int CG = K / 4, RG = 256 / CG, RPT = BT / RG;
-  constexpr int CGV = V / 4, RGV = 256 / CGV, RPTV = BT / RGV;
-  constexpr int KT32 = K / 32, TV = V / 64;
+  constexpr int RG = 256 / (K / 4);
   const int H = p.H;
   // A few hundred workgroups walk the (chunk, head) flags: almost always none is set, and a
   // launch of one workgroup per chunk would cost more than the scan.  The lanes first read all flags
@@ -433,155 +628,18 @@ __global__ __launch_bounds__(256) void gla_fwd_o_exact_kernel(ExactParams p) {
       any |= p.wide[lin];
     if (!__syncthreads_or(any)) return;
   }
-  for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
-  if (p.wide[lin] == 0) continue;  // workgroup-uniform
-  __syncthreads();                 // the tiles of the previous flagged chunk are free
-  int hh;
-  ChunkLoc cl = locate_chunk_at(lin, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
   __shared__ __attribute__((aligned(16))) float sG[BT * LDG];
   __shared__ __attribute__((aligned(16))) T sQ[BT * LDK];
   __shared__ __attribute__((aligned(16))) T sK[BT * LDK];
   __shared__ __attribute__((aligned(16))) T sVt[V * LDT];
   __shared__ __attribute__((aligned(16))) T sP[BT * LDT];
   __shared__ __attribute__((aligned(16))) float sPart[RG * K];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int L = cl.L;
-  const int64_t row0 = cl.row0;
-  const int rg = tid / CG, c4 = (tid % CG) * 4;
-  float gq[RPT][4];
-  v4 qreg[RPT], kreg[RPT];
-#pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    int row = rg * RPT + i;
-    if (row < L) {
-      int64_t off = ((row0 + row) * H + hh) * (int64_t)K + c4;
-      if (p.head_gates) {
-        const float x = ((const float*)p.g)[(row0 + row) * H + hh];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) gq[i][j] = x;
-      } else {
-        Load<GT>::x4((const GT*)p.g + off, gq[i]);
-        if (p.gate_logits) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            gq[i][j] = log2_sigmoid_gate(gq[i][j], p.gate_inv_norm, p.gate_clamp_min * 1.4426950408889634f) *
-                       0.6931471805599453f;
-        }
-      }
-      qreg[i] = *(const v4*)((const T*)p.q + off);
-      kreg[i] = *(const v4*)((const T*)p.k + off);
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) gq[i][j] = 0.f;
-      qreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-      kreg[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-    }
-  }
-  const int rgv = tid / CGV, cv4 = (tid % CGV) * 4;
-#pragma unroll
-  for (int i = 0; i < RPTV; ++i) {
-    int row = rgv * RPTV + i;
-    v4 x = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-    if (row < L) x = *(const v4*)((const T*)p.v + ((row0 + row) * H + hh) * (int64_t)V + cv4);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) sVt[(cv4 + j) * LDT + row] = x[j];
-  }
-  float run[4] = {0.f, 0.f, 0.f, 0.f};
-  float G[RPT][4];
-#pragma unroll
-  for (int i = 0; i < RPT; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      run[j] += gq[i][j];
-      G[i][j] = run[j];
-    }
-  *(f32x4*)&sPart[rg * K + c4] = f32x4{run[0], run[1], run[2], run[3]};
-  __syncthreads();
-  float off[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int r = 0; r < rg; ++r) {
-    f32x4 pr = *(const f32x4*)&sPart[r * K + c4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) off[j] += pr[j];
-  }
-#pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    int row = rg * RPT + i;
-    *(f32x4*)&sG[row * LDG + c4] = f32x4{G[i][0] + off[0], G[i][1] + off[1], G[i][2] + off[2], G[i][3] + off[3]};
-    *(v4*)&sQ[row * LDK + c4] = qreg[i];
-    *(v4*)&sK[row * LDK + c4] = kreg[i];
-  }
-  __syncthreads();
-  // ---- exact scores: lane handles row i and every fourth column j <= i
-  {
-    const int i = tid >> 2, jq = tid & 3;
-    for (int j = 0; j < BT; ++j) {
-      if ((j & 3) != jq) continue;
-      float a = 0.f;
-      if (j <= i) {
-        for (int kk = 0; kk < K; kk += 4) {
-          f32x4 gi = *(const f32x4*)&sG[i * LDG + kk];
-          f32x4 gj = *(const f32x4*)&sG[j * LDG + kk];
-          v4 qv = *(const v4*)&sQ[i * LDK + kk];
-          v4 kv = *(const v4*)&sK[j * LDK + kk];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) a += (float)qv[e] * (float)kv[e] * __expf(gi[e] - gj[e]);
-        }
-      }
-      sP[i * LDT + j] = (T)(a * p.scale);
-    }
-  }
-  __syncthreads();
-  // ---- q~ = s q e^{G} over the raw q tile (every lane rewrites exactly what it reads)
-#pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    int row = rg * RPT + i;
-    f32x4 gg = *(const f32x4*)&sG[row * LDG + c4];
-    v4 qv = *(const v4*)&sQ[row * LDK + c4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) qv[j] = (T)((float)qv[j] * p.scale * __expf(gg[j]));
-    *(v4*)&sQ[row * LDK + c4] = qv;
-  }
-  __syncthreads();
-  const int rw = wave >> 1, cw = wave & 1;
-  f32x16 acc[TV];
-#pragma unroll
-  for (int tv = 0; tv < TV; ++tv) acc[tv] = zero16();
-  const T* hp = (const T*)p.hwide + (cl.cglob * H + hh) * (int64_t)K * V;
-#pragma unroll
-  for (int kt = 0; kt < KT32; ++kt)
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      if (p.hwide_vk) {   // [V][K]: a lane reads 8 consecutive key channels of its value column
-        v8 a = lds_frag32<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
-#pragma unroll
-        for (int tv = 0; tv < TV; ++tv) {
-          v8 b = *(const v8*)(hp + (int64_t)((cw * TV + tv) * 32 + (lane & 31)) * K + kt * 32 + half * 16 + 8 * (lane >> 5));
-          acc[tv] = Elem<T>::mfma32(a, b, acc[tv]);
-        }
-      } else {
-        v8 a = lds_frag32_perm<T>(sQ, LDK, rw * 32, kt * 32 + half * 16, lane);
-#pragma unroll
-        for (int tv = 0; tv < TV; ++tv) {
-          v8 b = *(const v8*)(hp + (((int64_t)kt * (V / 32) + (cw * TV + tv)) * 64 + lane) * 16 + half * 8);
-          acc[tv] = Elem<T>::mfma32(a, b, acc[tv]);
-        }
-      }
-    }
-  const int jend = (rw + 1) * 32;
-  for (int js = 0; js < jend; js += 16) {
-    v8 a = lds_frag32<T>(sP, LDT, rw * 32, js, lane);
-#pragma unroll
-    for (int tv = 0; tv < TV; ++tv)
-      acc[tv] = Elem<T>::mfma32(a, lds_frag32<T>(sVt, LDT, (cw * TV + tv) * 32, js, lane), acc[tv]);
-  }
-  T* op = (T*)p.o + (row0 * H + hh) * (int64_t)V;
-#pragma unroll
-  for (int tv = 0; tv < TV; ++tv)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      int i = rw * 32 + c32_row(r, lane);
-      if (i < L) op[(int64_t)i * H * V + (cw * TV + tv) * 32 + (lane & 31)] = (T)acc[tv][r];
-    }
+  const ExactLds<T> S{sG, sQ, sK, sVt, sP, sPart};
+  for (int64_t lin = blockIdx.x; lin < p.total; lin += gridDim.x) {
+    if (p.wide[lin] == 0) continue;  // workgroup-uniform
+    int hh;
+    ChunkLoc cl = locate_chunk_at(lin, p.offsets, p.indices, p.T, p.NTfix, H, &hh);
+    gla_exact_chunk<T, GT, K, V, 256>(p, S, cl, hh, V, 0, (int)threadIdx.x);
   }
 }
 
@@ -693,7 +751,7 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
     FLA_REQUIRE(((uintptr_t)kh_t | (uintptr_t)scores) % 16 == 0, FLA_E_ALIGNMENT);
   }
   FusedParams p{q, k, v, gates, h0, o, ht, offsets, chunk_offsets, seq_order, ws_wide, ws_hwide,
-                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay, kh_t, scores, gate_inv_norm, gate_clamp_min};
+                T, (int)H, (int)V, (int)N, scale, h_frag_t, qg, decay, kh_t, scores, gate_inv_norm, gate_clamp_min, 0};
   hipStream_t st = (hipStream_t)stream;
   dim3 grid;
   int ntfix = 0;
@@ -705,6 +763,9 @@ static int gla_fwd_fused_impl(const void* q, const void* k, const void* v, const
                 (int64_t)grid.x * grid.y, head_gates ? 1 : 0, (!logits && use_wide_kernel(p, (int)K)) ? 1 : 0,
                 logits ? 1 : 0, gate_inv_norm, gate_clamp_min};
   if (ws_wide) grid = dim3((unsigned)(e.total < 512 ? e.total : 512));
+  // the 64- and 32-column kernels redo flagged chunks themselves; the 128-column kernel leaves them to a second launch
+  p.exact_tail = ws_wide && exact_pass && !(!logits && use_wide_kernel(p, (int)K)) ? 1 : 0;
+  if (p.exact_tail) exact_pass = false;
 #define FLA_FUSED(TT, GG)                                                \
   {                                                                      \
     int rc = launch_fused<TT, GG>(p, (int)K, st, logits);                \

@@ -1,9 +1,9 @@
 """``chunk_gla`` with the reference's signature (``fla/ops/gla/chunk.py:1409-1495``).
 
 Forward on the device (chunk size 64): one launch, ``fla_chunk_gla_fwd_fused`` (prefix sums of the
-gates, gated scores, output and state scan in one pass; the per-chunk states stay on the chip),
-followed by a short second launch that recomputes the output rows of chunks whose gates left the
-range of the single-reference-point scores.  The two-kernel form (``fla_chunk_gla_fwd_h`` ->
+gates, gated scores, output and state scan in one pass; the per-chunk states stay on the chip;
+chunks whose gates left the range of the single-reference-point scores are flagged and their
+output rows recomputed exactly by the same launch after its last chunk).  The two-kernel form (``fla_chunk_gla_fwd_h`` ->
 ``fla_chunk_gla_fwd_o``) serves the reference-shaped internal entry points ``chunk_gla_fwd`` /
 ``chunk_fwd_h`` / ``chunk_gla_fwd_o_gk``.
 """
@@ -267,7 +267,7 @@ def chunk_gla_fwd_fused(q, k, v, g, scale, initial_state, output_final_state, of
         else:
             be.check(be.lib().fla_chunk_gla_fwd_fused_states(*head, be.ptr(hT), *tail), "fla_chunk_gla_fwd_fused_states")
             states_out.append(hT)
-    elif first_launch_only:   # benchmark hook: the scan without the guard's second launch
+    elif first_launch_only:   # benchmark hook: the scan without the recomputation of flagged chunks
         be.check(be.lib().fla_chunk_gla_fwd_fused_first_launch(*head, *tail), "fla_chunk_gla_fwd_fused_first_launch")
     else:
         be.check(be.lib().fla_chunk_gla_fwd_fused(*head, *tail), "fla_chunk_gla_fwd_fused")

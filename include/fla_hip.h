@@ -189,8 +189,11 @@ int fla_chunk_gla_fwd_o(const void* q, const void* k, const void* v, const void*
  * range ends at 65504).  With the workspaces
  * ws_wide (int32 [chunks, H]) and ws_hwide (q/k/v dtype, [chunks, H, K*V]) given
  * (V <= 128), chunks outside that range are flagged on the device and their
- * output rows recomputed by a second launch with exact pairwise exponents
- * (the reference's diagonal sub-block arithmetic, fla/ops/gla/chunk.py:113-170);
+ * output rows recomputed with exact pairwise exponents (the reference's diagonal
+ * sub-block arithmetic, fla/ops/gla/chunk.py:113-170) by the workgroup that owns
+ * them, after its last chunk (one launch in all; the 128-column kernel used for
+ * more than 128 (sequence, head) pairs at K = V = 128 leaves them to a short
+ * second launch);
  * packed batches then also need indices [NT,2] and chunk_offsets [N+1].
  * seq_order (int64 [N], a permutation of the sequence ids, or NULL) is the order
  * in which sequences are handed to the hardware; longest first balances a
@@ -215,9 +218,9 @@ int fla_chunk_gla_fwd_fused_logits(const void* q, const void* k, const void* v, 
                                    int64_t T, int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                    float normalizer, int has_clamp, float clamp_min, fla_stream_t stream);
 
-/* Diagnostics: only the first of the two launches of fla_chunk_gla_fwd_fused (the scan, with the flag and
+/* Diagnostics: the scan of fla_chunk_gla_fwd_fused without the recomputation of flagged chunks (with the flag and
  * state hand-over stores of the range guard when the workspaces are given), so that a benchmark can put
- * events round the dominant kernel in the form the operator runs.  o is incomplete for flagged chunks. */
+ * events round the dominant kernel alone.  o is incomplete for flagged chunks. */
 int fla_chunk_gla_fwd_fused_first_launch(const void* q, const void* k, const void* v, const void* gates,
                                          const float* h0, void* o, float* ht, int* ws_wide, void* ws_hwide,
                                          const int64_t* offsets, const int64_t* indices,
