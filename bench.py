@@ -334,7 +334,7 @@ def bench_decode(device, steps=1000):
 def bench_decode_layer_step(device, steps=300):
     """One token through what a gated DeltaNet layer runs around its state update at the decode shape (B=256, H=32,
     D=128): short-convolution step, l2 norm of q and k, the in-place recurrent step, gated RMS norm of the output -
-    five launches - run eagerly (wall time per step, host included) and replayed from one captured HIP graph."""
+    six launches with the shift that derives k - run eagerly (wall time per step, host included) and replayed from one captured HIP graph."""
     import torch
     import torch.nn.functional as F
     from fla_amd.modules import FusedRMSNormSwishGate, ShortConvolution, l2_norm
@@ -358,22 +358,35 @@ def bench_decode_layer_step(device, steps=300):
                                                 output_final_state=True, head_first=False, inplace_state=True)
         return norm(o, gate_in.view(B, 1, H, D))
 
-    with torch.no_grad():
-        st_e = event_stats(step, steps, 20)
+    def step_fused_norms():   # the two l2 norms inside the recurrent step's launch: four launches
+        y, _ = conv(x, cache=cache)
+        o, _ = fused_recurrent_gated_delta_rule(y.view(B, 1, H, D), torch.roll(y, 1, dims=-1).view(B, 1, H, D),
+                                                y.view(B, 1, H, D), g, beta, initial_state=state,
+                                                output_final_state=True, head_first=False, inplace_state=True,
+                                                use_qk_l2norm_in_kernel=True)
+        return norm(o, gate_in.view(B, 1, H, D))
+
+    def eager_and_graph(fn):
+        st_e = event_stats(fn, steps, 20)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            step()
+            fn()
         torch.cuda.current_stream().wait_stream(side)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            step()
+            fn()
         st_g = event_stats(graph.replay, steps, 20)
+        return {"eager_wall_us_per_step": round(st_e["wall_us_per_call"], 1),
+                "eager_event_median_us": round(st_e["median_us"], 1),
+                "hip_graph_replay_wall_us_per_step": round(st_g["wall_us_per_call"], 1),
+                "hip_graph_replay_event_median_us": round(st_g["median_us"], 1)}
+
+    with torch.no_grad():
+        out = {"launches_per_step": 6, **eager_and_graph(step)}
+        out["l2norm_in_step"] = {"launches_per_step": 4, **eager_and_graph(step_fused_norms)}
     assert torch.isfinite(state).all()
-    return {"launches_per_step": 6, "eager_wall_us_per_step": round(st_e["wall_us_per_call"], 1),
-            "eager_event_median_us": round(st_e["median_us"], 1),
-            "hip_graph_replay_wall_us_per_step": round(st_g["wall_us_per_call"], 1),
-            "hip_graph_replay_event_median_us": round(st_g["median_us"], 1)}
+    return out
 
 
 def bench_gdr(device, steps=50, warmup=20):

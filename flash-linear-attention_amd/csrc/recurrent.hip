@@ -38,6 +38,7 @@ struct RParams {
   float scale;
   int reverse;
   int beta_per_value;
+  float l2_eps;   // GDR, >= 0: q and k enter as x / sqrt(sum x^2 + l2_eps) (the l2 norm the layer applies in front of the step)
 };
 
 template <typename X>
@@ -59,7 +60,7 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
   __shared__ __attribute__((aligned(16))) float sv[2][BV];
   __shared__ __attribute__((aligned(16))) float sdv[2][BV];  // e^{gv} (GLA) or beta (GDR)
   __shared__ __attribute__((aligned(16))) float sred[2][2][RG][BV];
-  __shared__ float sscal[2][2];  // e^{g}, q.k
+  __shared__ float sscal[2][4];  // e^{g}, q.k, 1/|q|, 1/|k| (the last two 1 unless the rows are normalised here)
 
   const int tid = threadIdx.x;
   const int H = p.H, K = p.K, V = p.V;
@@ -111,12 +112,27 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
     }
     if (tid == 0) sscal[buf][0] = p.g ? __expf(ld<GT>(p.g, row * H + hh)) : 1.f;
     if (GDR && tid < 64) {
-      // q.k over the whole key dim, reduced inside wave 0
-      float acc = 0.f;
-      for (int i = tid; i < K; i += 64) acc += ld<T>(p.q, qk + i) * p.scale * ld<T>(p.k, qk + i);
+      // q.k (and, where the rows are normalised here, q.q and k.k) over the whole key dim, reduced inside wave 0
+      float acc = 0.f, aq = 0.f, ak = 0.f;
+      for (int i = tid; i < K; i += 64) {
+        const float qx = ld<T>(p.q, qk + i), kx = ld<T>(p.k, qk + i);
+        acc += qx * p.scale * kx;
+        aq += qx * qx;
+        ak += kx * kx;
+      }
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
-      if (tid == 0) sscal[buf][1] = acc;
+      for (int off = 32; off > 0; off >>= 1) {
+        acc += __shfl_down(acc, off, 64);
+        aq += __shfl_down(aq, off, 64);
+        ak += __shfl_down(ak, off, 64);
+      }
+      if (tid == 0) {
+        const bool l2 = p.l2_eps >= 0.f;
+        const float rq = l2 ? rsqrtf(aq + p.l2_eps) : 1.f, rk = l2 ? rsqrtf(ak + p.l2_eps) : 1.f;
+        sscal[buf][1] = acc * rq * rk;
+        sscal[buf][2] = rq;
+        sscal[buf][3] = rk;
+      }
     }
   };
 
@@ -133,6 +149,7 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
     // Everything read from the staging buffers is taken before the barrier:
     // the next step restages this buffer before its own barrier.
     const float qk = GDR ? sscal[buf][1] : 0.f;
+    const float rq = GDR ? sscal[buf][2] : 1.f, rk = GDR ? sscal[buf][3] : 1.f;
     float krow[NR];
     if (!GDR) {
 #pragma unroll
@@ -150,7 +167,7 @@ __global__ __launch_bounds__(256) void recurrent_fwd_kernel(RParams p) {
 #pragma unroll
       for (int i = 0; i < NR; ++i) {
         int row = rg + RG * i;
-        float kr = sk[buf][row], qr = sq[buf][row];
+        float kr = sk[buf][row] * rk, qr = sq[buf][row] * rq;
         krow[i] = kr;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -280,9 +297,22 @@ extern "C" int fla_fused_recurrent_fwd(const void* q, const void* k, const void*
   int rc = check_common(q, k, v, o, offsets, B, T, H, K, V, N);
   if (rc) return rc;
   FLA_REQUIRE((((uintptr_t)h0) | ((uintptr_t)ht)) % 16 == 0, FLA_E_ALIGNMENT);
-  RParams p{q, k, v, g, gk, gv, nullptr, o, h0, ht, offsets, T, (int)H, (int)K, (int)V, scale, reverse, 0};
+  RParams p{q, k, v, g, gk, gv, nullptr, o, h0, ht, offsets, T, (int)H, (int)K, (int)V, scale, reverse, 0, -1.f};
   if (!g && !gk && !gv) gate_dtype = FLA_F32;
   return dispatch_r<false>(p, qkv_dtype, gate_dtype, o_dtype, N * H, (hipStream_t)stream);
+}
+
+static int recurrent_gdr_impl(const void* q, const void* k, const void* v, const void* g, const void* beta, void* o,
+                              const float* h0, float* ht, const int64_t* offsets, int qkv_dtype, int gate_dtype,
+                              int o_dtype, int beta_per_value, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                              int64_t N, float scale, float l2_eps, fla_stream_t stream) {
+  int rc = check_common(q, k, v, o, offsets, B, T, H, K, V, N);
+  if (rc) return rc;
+  FLA_REQUIRE((((uintptr_t)h0) | ((uintptr_t)ht)) % 16 == 0, FLA_E_ALIGNMENT);
+  RParams p{q, k, v, g, nullptr, nullptr, beta, o, h0, ht, offsets, T, (int)H, (int)K, (int)V, scale, 0, beta_per_value,
+            l2_eps};
+  if (!g && !beta) gate_dtype = FLA_F32;
+  return dispatch_r<true>(p, qkv_dtype, gate_dtype, o_dtype, N * H, (hipStream_t)stream);
 }
 
 extern "C" int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const void* k, const void* v, const void* g,
@@ -291,10 +321,18 @@ extern "C" int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const voi
                                                         int o_dtype, int beta_per_value, int64_t B, int64_t T,
                                                         int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                                         fla_stream_t stream) {
-  int rc = check_common(q, k, v, o, offsets, B, T, H, K, V, N);
-  if (rc) return rc;
-  FLA_REQUIRE((((uintptr_t)h0) | ((uintptr_t)ht)) % 16 == 0, FLA_E_ALIGNMENT);
-  RParams p{q, k, v, g, nullptr, nullptr, beta, o, h0, ht, offsets, T, (int)H, (int)K, (int)V, scale, 0, beta_per_value};
-  if (!g && !beta) gate_dtype = FLA_F32;
-  return dispatch_r<true>(p, qkv_dtype, gate_dtype, o_dtype, N * H, (hipStream_t)stream);
+  return recurrent_gdr_impl(q, k, v, g, beta, o, h0, ht, offsets, qkv_dtype, gate_dtype, o_dtype, beta_per_value, B, T, H,
+                            K, V, N, scale, -1.f, stream);
+}
+
+extern "C" int fla_fused_recurrent_gated_delta_rule_fwd_l2norm(const void* q, const void* k, const void* v,
+                                                               const void* g, const void* beta, void* o,
+                                                               const float* h0, float* ht, const int64_t* offsets,
+                                                               int qkv_dtype, int gate_dtype, int o_dtype,
+                                                               int beta_per_value, int64_t B, int64_t T, int64_t H,
+                                                               int64_t K, int64_t V, int64_t N, float scale,
+                                                               float l2norm_eps, fla_stream_t stream) {
+  FLA_REQUIRE(l2norm_eps >= 0.f, FLA_E_INVALID);
+  return recurrent_gdr_impl(q, k, v, g, beta, o, h0, ht, offsets, qkv_dtype, gate_dtype, o_dtype, beta_per_value, B, T, H,
+                            K, V, N, scale, l2norm_eps, stream);
 }

@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -37,6 +37,8 @@ SIGNATURES = {
     "fla_fused_recurrent_bwd": (c_int, [P] * 14 + [I, I, I64, I64, I64, I64, I64, I64, F, I, P]),
     "fla_fused_recurrent_gated_delta_rule_fwd": (c_int, [P, P, P, P, P, P, P, P, P, I, I, I, I,
                                                          I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_fused_recurrent_gated_delta_rule_fwd_l2norm": (c_int, [P, P, P, P, P, P, P, P, P, I, I, I, I,
+                                                                I64, I64, I64, I64, I64, I64, F, F, P]),
     "fla_chunk_gla_fwd_h": (c_int, [P, P, P, I, P, P, P, P, P, I, I, I, I,
                                     I64, I64, I64, I64, I64, I64, P]),
     "fla_chunk_gla_fwd_o": (c_int, [P, P, P, P, I, P, P, P, P, P, I64, I, I,

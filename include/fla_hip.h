@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 11
+#define FLA_ABI_VERSION 12
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -140,6 +140,19 @@ int fla_fused_recurrent_gated_delta_rule_fwd(const void* q, const void* k, const
                                              int beta_per_value,
                                              int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                                              int64_t N, float scale, fla_stream_t stream);
+
+/* The same step on un-normalised q and k: every row enters as x / sqrt(sum x^2 + l2norm_eps), the l2 norm the
+ * layer applies in front of the operator (fla/layers/gated_deltanet.py:234-237, fla/modules/l2norm.py), formed from
+ * the rows the step loads anyway: two launches fewer per decode step. */
+int fla_fused_recurrent_gated_delta_rule_fwd_l2norm(const void* q, const void* k, const void* v,
+                                                    const void* g, const void* beta,
+                                                    void* o, const float* h0, float* ht,
+                                                    const int64_t* offsets,
+                                                    int qkv_dtype, int gate_dtype, int o_dtype,
+                                                    int beta_per_value,
+                                                    int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
+                                                    int64_t N, float scale, float l2norm_eps,
+                                                    fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Chunked GLA forward (chunk size 64).

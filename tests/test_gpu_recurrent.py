@@ -4,7 +4,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import assert_close, gdr_inputs, gla_inputs, random_offsets
+from helpers import assert_close, gdr_inputs, gla_inputs, random_offsets, rel_l2
 
 pytestmark = pytest.mark.gpu
 
@@ -103,6 +103,42 @@ def test_fused_recurrent_gated_delta_rule_variants(device):
                                                    output_final_state=True, offsets=offs.tolist())
         assert_close("o", ro, o, 1e-5)
         assert_close("ht", rht, ht, 1e-5)
+
+
+@pytest.mark.parametrize("T,D,varlen", [(1, 128, False), (37, 128, False), (5, 64, False), (3, 100, False), (40, 128, True)])
+def test_fused_recurrent_gated_delta_rule_l2norm_in_kernel(device, T, D, varlen):
+    """use_qk_l2norm_in_kernel on raw q, k == l2_norm in front of the operator (the layer's form,
+    fla/layers/gated_deltanet.py:234-237), and both match the oracle on normalised rows."""
+    from fla_amd.modules import l2_norm
+    from fla_amd.ops.gated_delta_rule import fused_recurrent_gated_delta_rule
+    from oracle.recurrent import naive_recurrent_gated_delta_rule
+    torch.manual_seed(5)
+    B, H = (1, 3) if varlen else (2, 3)
+    offsets = torch.tensor([0, 7, 8, T], device=device) if varlen else None
+    N = 3 if varlen else B
+    q = (torch.randn(B, T, H, D, device=device) * 3).bfloat16()
+    k = (torch.randn(B, T, H, D, device=device) * 0.2).bfloat16()
+    v = torch.randn(B, T, H, D, device=device).bfloat16()
+    g = F.logsigmoid(torch.randn(B, T, H, device=device))
+    beta = torch.rand(B, T, H, device=device)
+    h0 = torch.randn(N, H, D, D, device=device) * 0.1
+    o1, ht1 = fused_recurrent_gated_delta_rule(q, k, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=offsets, head_first=False, use_qk_l2norm_in_kernel=True)
+    # (the stand-alone kernel takes rows that are multiples of 8 elements)
+    nrm = l2_norm if D % 8 == 0 else (lambda x: F.normalize(x.float(), dim=-1, eps=1e-6).to(x.dtype))
+    qn, kn = nrm(q), nrm(k)
+    o2, ht2 = fused_recurrent_gated_delta_rule(qn, kn, v, g, beta, initial_state=h0, output_final_state=True,
+                                               offsets=offsets, head_first=False)
+    # the separate launches round the normalised rows to bf16, the fused step keeps them in fp32
+    assert rel_l2(o1, o2) < 6e-3 and rel_l2(ht1, ht2) < 6e-3
+    qf, kf = q.float(), k.float()
+    qr = (qf / torch.sqrt((qf * qf).sum(-1, keepdim=True) + 1e-6)).cpu()
+    kr = (kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + 1e-6)).cpu()
+    o_ref, ht_ref = naive_recurrent_gated_delta_rule(qr, kr, v.float().cpu(), g.cpu(), beta.cpu(), initial_state=h0.cpu(),
+                                                     output_final_state=True,
+                                                     offsets=None if offsets is None else offsets.cpu())
+    assert rel_l2(o1.float().cpu(), o_ref) < 5e-3
+    assert rel_l2(ht1.cpu(), ht_ref) < 1e-4
 
 
 @pytest.mark.parametrize("op", ["gla", "gdr"])
