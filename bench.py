@@ -749,8 +749,9 @@ def bench_layer_fusion(device, steps=20):
 
 
 def bench_fp32_inputs(device, steps=5):
-    """chunk_gla on fp32 q, k, v (the reference's own tests run the operator in fp32): the token-by-token fp32 kernels
-    serve it, exact to 1e-4 and serial in time; timed at B=8, T=4096, H=16, K=V=128."""
+    """chunk_gla on fp32 q, k, v (the reference's own tests run the operator in fp32) at B=8, T=4096, H=16, K=V=128:
+    the default route (scaled to fp16, chunk kernels, fp32 gates and states; the scaling and casts are part of the
+    call) and the exact one (FLA_AMD_FP32_EXACT=1: fp32 token-by-token kernels, 1e-4, serial in time)."""
     import torch
     import torch.nn.functional as F
     from fla_amd.ops.gla import chunk_gla
@@ -762,15 +763,14 @@ def bench_fp32_inputs(device, steps=5):
     import fla_amd.ops.gla.chunk as mod
     fn = lambda: chunk_gla(q, k, v, g, initial_state=h0, output_final_state=True, head_first=False)
     with torch.no_grad():
-        us = event_avg_us(fn, steps, warmup=2, ramp=0.0)
-        # opt-in (FLA_AMD_FP32_VIA_FP16=1): q, k, v rounded to fp16 and the chunk kernels run; the casts are part of the call
-        mod.FP32_INPUTS_VIA_FP16_CHUNK = True
+        us16 = event_avg_us(fn, 20)
+        mod.FP32_INPUTS_EXACT = True
         try:
-            us16 = event_avg_us(fn, 20)
+            us = event_avg_us(fn, steps, warmup=2, ramp=0.0)
         finally:
-            mod.FP32_INPUTS_VIA_FP16_CHUNK = False
-    return {"us": round(us, 1), "tokens_per_s": round(B * T / us * 1e6, 1),
-            "via_fp16_chunk_kernels_us": round(us16, 1)}
+            mod.FP32_INPUTS_EXACT = False
+    return {"us": round(us16, 1), "tokens_per_s": round(B * T / us16 * 1e6, 1),
+            "exact_fp32_route_us": round(us, 1)}
 
 
 def bench_gdr_onepass(device, steps=30):

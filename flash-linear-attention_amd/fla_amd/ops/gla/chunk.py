@@ -31,11 +31,93 @@ KEEP_STATES_FOR_BACKWARD = os.environ.get("FLA_AMD_RECOMPUTE_STATES", "0") in ("
 # With the states, a differentiated forward (per-key gates, V <= 128) also keeps k^ = k e^{G_last - G} and the score tile
 # of every chunk (1.5 more tensors of k's size), from which the backward's reverse state scan forms dv on its way.
 KEEP_KHAT_AND_SCORES = os.environ.get("FLA_AMD_GLA_FUSED_DV", "1") not in ("", "0")
-# fp32 q/k/v: by default the fp32 token-by-token kernels (exact to 1e-4, serial in time).  FLA_AMD_FP32_VIA_FP16=1 rounds
-# q, k, v to fp16 and runs the chunk kernels instead (gates and states stay fp32): about 5e-4 relative error - inside
-# the 4e-3 the reference's own fp32 tests allow (tests/ops/test_gla.py:195-201) - and some fifty times faster, for
-# inputs whose magnitudes fit fp16 (|x| < 65504; the caller's responsibility).
-FP32_INPUTS_VIA_FP16_CHUNK = os.environ.get("FLA_AMD_FP32_VIA_FP16", "0") not in ("", "0")
+# fp32 q/k/v run through the fp16 chunk kernels, as the reference runs them through its chunk kernels with fp32 operands
+# on the matrix pipe at reduced precision (tests/ops/test_gla.py:149-201): q, k and v are divided by a power of two >= their
+# largest magnitude (exact; found on the device, no synchronisation) and rounded to fp16, gates and states stay fp32, and
+# the results are scaled back.  About 5e-4 relative error - the reference's own fp32 tests allow 4e-3 (:195-201).
+# FLA_AMD_FP32_EXACT=1 takes the fp32 token-by-token kernels instead: exact to 1e-4, serial in time (10.5 ms against
+# 1.0 ms at B=8, T=4096, H=16, D=128).
+FP32_INPUTS_EXACT = os.environ.get("FLA_AMD_FP32_EXACT", "0") not in ("", "0")
+
+
+def _pow2_scale(x: torch.Tensor) -> torch.Tensor:
+    """A power of two >= max|x| as a tensor of one element on x's device (1 for an all-zero tensor); one pass over x."""
+    lo, hi = torch.aminmax(x.detach())
+    amax = torch.maximum(-lo, hi).float().reshape(1)
+    return torch.where(amax > 0, torch.exp2(torch.ceil(torch.log2(amax.clamp_min(1e-37)))), torch.ones_like(amax))
+
+
+def _scaled_half(x: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+    """x / s rounded to fp16 in one pass (s a power of two: the division is exact)."""
+    return torch.mul(x.detach(), 1.0 / s, out=torch.empty_like(x, dtype=torch.float16))
+
+
+class _ScaledFp16ChunkGla(torch.autograd.Function):
+    """fp32 q, k, v through the fp16 chunk kernels with every fp16 tensor - inputs, and in the backward pass the
+    cotangent of o - divided by a power of two that brings it to at most 1 (the operator is linear in each of q, k,
+    v, and its gradients are linear in the cotangents, so the scales factor out exactly)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g, initial_state, scale, output_final_state, offsets, head_first):
+        sq, sk, sv = _pow2_scale(q), _pow2_scale(k), _pow2_scale(v)
+        skv = sk * sv
+        need = ctx.needs_input_grad
+        with torch.enable_grad():
+            leaves = [_scaled_half(q, sq).requires_grad_(need[0]), _scaled_half(k, sk).requires_grad_(need[1]),
+                      _scaled_half(v, sv).requires_grad_(need[2]), g.detach().float().requires_grad_(need[3]),
+                      None if initial_state is None else (initial_state.detach().float() / skv).requires_grad_(need[4])]
+            o_h, ht_h = chunk_gla(leaves[0], leaves[1], leaves[2], leaves[3], scale=scale, initial_state=leaves[4],
+                                  output_final_state=output_final_state, offsets=offsets, head_first=head_first)
+        ctx.inner = (leaves, o_h, ht_h)
+        ctx.scales = (sq, sk, sv)
+        ctx.in_dtypes = (g.dtype, None if initial_state is None else initial_state.dtype)
+        o = o_h.detach() * (sq * skv)      # (a one-element fp32 tensor promotes the product to fp32)
+        ht = None if ht_h is None else ht_h.detach() * skv
+        return o, ht
+
+    @staticmethod
+    def backward(ctx, do, dht):
+        leaves, o_h, ht_h = ctx.inner
+        sq, sk, sv = ctx.scales
+        skv = sk * sv
+        co = do.float() * (sq * skv)
+        ch = None if (dht is None or ht_h is None) else dht.float() * skv
+        wanted = [i for i, x in enumerate(leaves) if x is not None and x.requires_grad]
+        targets = [leaves[i] for i in wanted]
+        res = [None] * 5
+
+        def accumulate(grads, c):
+            back = (c / sq, c / sk, c / sv, c, c / skv)
+            for i, gr in zip(wanted, grads):
+                if gr is not None:
+                    term = gr.float() * back[i]
+                    res[i] = term if res[i] is None else res[i] + term
+
+        # The two cotangents live on unrelated scales (that of o carries q's scale, that of the final state does not),
+        # and the gradients are linear in them: one pass each, every pass with its cotangent brought to at most 1.
+        c = _pow2_scale(co)
+        cots = [(co / c).half()] + ([torch.zeros_like(ht_h)] if ht_h is not None else [])
+        outs = [o_h] + ([ht_h] if ht_h is not None else [])
+        accumulate(torch.autograd.grad(outs, targets, cots, allow_unused=True, retain_graph=ch is not None), c)
+        if ch is not None:
+            c = _pow2_scale(ch)
+            accumulate(torch.autograd.grad([o_h, ht_h], targets, [torch.zeros_like(o_h), ch / c], allow_unused=True), c)
+        if res[3] is not None:
+            res[3] = res[3].to(ctx.in_dtypes[0])
+        if res[4] is not None:
+            res[4] = res[4].to(ctx.in_dtypes[1])
+        return res[0], res[1], res[2], res[3], res[4], None, None, None, None
+
+
+def _chunk_gla_fp32_via_fp16(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first):
+    if torch.is_grad_enabled() and any(x is not None and x.requires_grad for x in (q, k, v, g, initial_state)):
+        return _ScaledFp16ChunkGla.apply(q, k, v, g, initial_state, scale, output_final_state, offsets, head_first)
+    sq, sk, sv = _pow2_scale(q), _pow2_scale(k), _pow2_scale(v)
+    skv = sk * sv
+    h0 = None if initial_state is None else initial_state.float() / skv
+    o, ht = chunk_gla(_scaled_half(q, sq), _scaled_half(k, sk), _scaled_half(v, sv), g.float(), scale=scale,
+                      initial_state=h0, output_final_state=output_final_state, offsets=offsets, head_first=head_first)
+    return o * (sq * skv), None if ht is None else ht * skv
 
 
 def _pad_dim(x: Optional[torch.Tensor], size: int) -> Optional[torch.Tensor]:
@@ -650,11 +732,9 @@ def chunk_gla(
     if q.numel() == 0:
         return empty_batch_result(q.transpose(1, 2) if head_first else q, v, offsets, initial_state, output_final_state)
     if q.dtype == torch.float32:
-        if FP32_INPUTS_VIA_FP16_CHUNK:
-            o, ht = chunk_gla(q.half(), k.half(), v.half(), g.float(), scale=scale, initial_state=initial_state,
-                              output_final_state=output_final_state, offsets=offsets, head_first=head_first)
-            return o.float(), ht
-        return _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
+        if FP32_INPUTS_EXACT:
+            return _chunk_gla_fp32(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
+        return _chunk_gla_fp32_via_fp16(q, k, v, g, scale, initial_state, output_final_state, offsets, head_first)
     K, V = q.shape[-1], v.shape[-1]
     if K > 128:
         # every key channel carries its own row of the state and o sums over them: wider key heads

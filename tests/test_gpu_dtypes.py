@@ -131,11 +131,14 @@ def test_chunk_gla_fp16_strong_gates(device):
 
 @pytest.mark.parametrize("T,D,head_first,varlen", [(130, 64, False, False), (300, 100, True, False), (200, 128, False, True),
                                                    (64, 300, False, False)])
-def test_chunk_gla_fp32_inputs(device, T, D, head_first, varlen):
-    """fp32 q, k, v (tests/ops/test_gla.py:29-87 and :149-201 run the operator in fp32): forward and backward
-    to fp32 accuracy, rel-L2 <= 1e-4, against the fp32 naive recurrence - no rounding of the inputs to 16 bits."""
+def test_chunk_gla_fp32_inputs(device, monkeypatch, T, D, head_first, varlen):
+    """fp32 q, k, v on the exact route (FLA_AMD_FP32_EXACT=1; tests/ops/test_gla.py:29-87 and :149-201 run the operator in
+    fp32): forward and backward to fp32 accuracy, rel-L2 <= 1e-4, against the fp32 naive recurrence - no rounding of
+    the inputs to 16 bits."""
     import torch.nn.functional as F
+    import fla_amd.ops.gla.chunk as mod
     from fla_amd.ops.gla import chunk_gla
+    monkeypatch.setattr(mod, "FP32_INPUTS_EXACT", True)
     from helpers import assert_close
     from oracle.recurrent import naive_recurrent_gla
     B, H = (1, 2) if varlen else (2, 2)
@@ -171,11 +174,12 @@ def test_chunk_gla_fp32_inputs(device, T, D, head_first, varlen):
     assert_close("dh0", rh0.grad, h0l.grad, 1e-4)
 
 
-@pytest.mark.parametrize("T,D,varlen", [(300, 128, False), (257, 100, True)])
-def test_chunk_gla_fp32_inputs_via_fp16_chunk_kernels(device, monkeypatch, T, D, varlen):
-    """The opt-in fast route for fp32 q, k, v (rounded to fp16, chunk kernels, fp32 gates and states): forward and
-    backward inside the tolerances of the reference's own fp32 tests (tests/ops/test_gla.py:195-201: 4e-3 on o,
-    5e-3 on the rest), fp32 tensors in and out."""
+@pytest.mark.parametrize("T,D,varlen,magnitude", [(300, 128, False, 1.0), (257, 100, True, 1.0), (130, 64, False, 3e5),
+                                                   (130, 64, False, 1e-6)])
+def test_chunk_gla_fp32_inputs_default_route(device, T, D, varlen, magnitude):
+    """The default route for fp32 q, k, v (scaled by powers of two into fp16's range, chunk kernels, fp32 gates and
+    states): forward and backward inside the tolerances of the reference's own fp32 tests (tests/ops/test_gla.py:195-201:
+    4e-3 on o, 5e-3 on the rest), fp32 tensors in and out - also for magnitudes far outside what fp16 holds."""
     import torch.nn.functional as F
     import fla_amd.ops.gla.chunk as mod
     from helpers import assert_close
@@ -183,14 +187,13 @@ def test_chunk_gla_fp32_inputs_via_fp16_chunk_kernels(device, monkeypatch, T, D,
     B, H = (1, 2) if varlen else (2, 2)
     N = 3 if varlen else B
     gen = torch.Generator().manual_seed(T + D)
-    q, k, v = (torch.randn(B, T, H, D, generator=gen) for _ in range(3))
+    q, k, v = (torch.randn(B, T, H, D, generator=gen) * magnitude for _ in range(3))
     g = F.logsigmoid(torch.randn(B, T, H, D, generator=gen))
-    h0 = torch.randn(N, H, D, D, generator=gen)
+    h0 = torch.randn(N, H, D, D, generator=gen) * magnitude ** 2
     do = torch.randn(B, T, H, D, generator=gen)
     dht = torch.randn(N, H, D, D, generator=gen) * 0.1
     offs = torch.tensor([0, 17, 90, T]) if varlen else None
-    print(f"chunk_gla fp32 via fp16 chunk kernels T={T} D={D} varlen={varlen}", flush=True)
-    monkeypatch.setattr(mod, "FP32_INPUTS_VIA_FP16_CHUNK", True)
+    print(f"chunk_gla fp32 default route T={T} D={D} varlen={varlen} magnitude={magnitude}", flush=True)
     leaves = [x.to(device).requires_grad_() for x in (q, k, v, g)]
     h0l = h0.to(device).requires_grad_()
     o, ht = mod.chunk_gla(*leaves, initial_state=h0l, output_final_state=True, head_first=False,
