@@ -135,6 +135,21 @@ FLA_DEVICE float group_allsum(float x) {
   return x;
 }
 
+// Sum over the 32 lanes of a half wave (lanes 0-31 or 32-63); the result is valid in the second DPP row of the half
+// (lanes 16-31 and 48-63): group sums of 16, then row_bcast:15 hands the first row's total to the second.
+FLA_DEVICE float half_wave_sum_hi(float x) {
+  x = group_allsum<16>(x);
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x142, 0xA, 0xF, true));   // row_bcast:15 into rows 1, 3
+  return x;
+}
+// Sum over the 64 lanes of a wave, valid in the last DPP row (lanes 48-63): as above, then row_bcast:31 hands the
+// first half's total to the last row.
+FLA_DEVICE float wave_sum_lane63(float x) {
+  x = half_wave_sum_hi(x);
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x143, 0xC, 0xF, true));   // row_bcast:31 into rows 2, 3
+  return x;
+}
+
 // A row of 8 * N elements is held by N adjacent lanes, 8 elements each: x / sqrt(sum x^2 + eps) of this lane's
 // piece, rounded to T (fla/modules/l2norm.py:18-40: eps inside the square root).
 template <typename T, int N>

@@ -846,9 +846,8 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   request(nim, R);
   // <h, dH> of the whole key slice: reduce over the 4 waves through LDS
   __shared__ float sHd[4];
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) hd += __shfl_xor(hd, off, 64);
-  if (lane == 0) sHd[wave] = hd;
+  hd = wave_sum_lane63(hd);
+  if (lane == 63) sHd[wave] = hd;
   __syncthreads();
   // waves (rw=0,cw) and (rw=1,cw) loaded the same fragments: count each key tile once
   const float hd_all = sHd[0] + sHd[1];
@@ -882,14 +881,10 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   }
   // row sums over the 16 lanes that share a row group; total of k*dk_inter over the workgroup
 #pragma unroll
-  for (int off = 8; off > 0; off >>= 1) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rowsum[i] += __shfl_xor(rowsum[i], off, 64);
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) kin += __shfl_xor(kin, off, 64);
+  for (int i = 0; i < 4; ++i) rowsum[i] = group_allsum<16>(rowsum[i]);
+  kin = wave_sum_lane63(kin);
   __shared__ float sKin[4];
-  if (lane == 0) sKin[wave] = kin;
+  if (lane == 63) sKin[wave] = kin;
   __syncthreads();
   const float kin_all = sKin[0] + sKin[1] + sKin[2] + sKin[3];
   if ((tid & 15) == 0) {
@@ -1241,11 +1236,11 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
         float x = low ? dAu[r] * au : 0.f;                  // dAu * Au
         float tot = low ? dA[r] + dAu[r] * gamma : 0.f;     // dAw total
         sS1[i * LDT + j] = (T)tot;                          // dA (masked) [i][j]
-        // row sums: reduce over the 32 lanes holding the same row
-        float rs = x;
-#pragma unroll
-        for (int off = 16; off > 0; off >>= 1) rs += __shfl_xor(rs, off, 64);
-        if ((lane & 31) == 0) slot(4 + jb, i) = rs;
+        // row sums over the 32 lanes holding the same row: inside each row of 16 lanes on the data-parallel path,
+        // then the first row's total handed to the second (sixteen butterflies through the LDS crossbar per lane
+        // were a third of this kernel's time)
+        const float rs = half_wave_sum_hi(x);
+        if ((lane & 31) == 16) slot(4 + jb, i) = rs;
         colsum += x;
       }
     }
