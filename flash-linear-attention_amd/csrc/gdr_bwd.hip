@@ -914,7 +914,7 @@ struct WyBwdParams {
   const void* Aw;
   const void* dw;
   const void* du;
-  const void* dk_in;   // partial dk from the dq/dk/dw kernel, added before the single rounding
+  const void* dk_in;   // partial dk from the dq/dk/dw kernel, added to this launch's (rounded) part on the way out
   void* dk;
   void* dv;
   float* dbeta;
@@ -1005,7 +1005,7 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
   __shared__ __attribute__((aligned(16))) T sTr1[D * LDT];     // du^T, dw^T, k^T      [d][t]
   __shared__ __attribute__((aligned(16))) T sAw[BT * LDT];     // Aw [i][j]
   __shared__ __attribute__((aligned(16))) T sAwT[BT * LDT];    // Aw^T
-  __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA (masked) -> dM
+  __shared__ __attribute__((aligned(16))) T sS1[BT * LDT];     // Au^T -> dA^T (masked) -> dM
   __shared__ float sBeta[BT], sGam[BT];
   // Partial sums of dbeta and dgamma, one slot per contributing wave and step, added in a fixed order at the
   // end (no atomics: the gradients are bit-reproducible from run to run).  Slots 0-3: dbeta from the value
@@ -1127,7 +1127,6 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
   const uint32_t nit = it + gridDim.x;
   const bool more = nit < nitems;   // workgroup-uniform
   const Item nim = locate(more ? nit : it);   // (past the last item the request repeats it)
-  request(nim, R);
   __syncthreads();
   {
     // Au^T[j][i] = Aw^T[j][i] * e^{gamma_i - gamma_j}, i >= j
@@ -1194,18 +1193,30 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
   IOK::put_tr(sTr1, tid, rdw);
   IOK::put_rows(sRow2, LDD, tid, rk);
   __syncthreads();
+  request(nim, R);  // the next item's first rows
   // the partial dk of the previous launch is needed only in the last step: fetched now, so that its
   // latency hides behind the products
-  v4 dinr[TK][4];
+  // In the mapping of the final stores (whole rows, 16 bytes per lane: a lane per accumulator row would touch 32
+  // cache lines per instruction).  Unconditional, at a row inside the chunk, masked where they are used: a load under
+  // a branch is waited for at the join; without a partial dk the rows of k are read.
+  constexpr int CKs = K / 8, NDI = BT * CKs / 256;
+  v8 dinr[NDI];
   {
-    const T* dip = p.dk_in ? (const T*)p.dk_in + ((row0 + jrow) * H + hh) * (int64_t)K : nullptr;
+    const T* dip = (p.dk_in ? (const T*)p.dk_in : (const T*)p.k) + (row0 * H + hh) * (int64_t)K;
 #pragma unroll
-    for (int t = 0; t < TK; ++t)
+    for (int i = 0; i < NDI; ++i) {
+      const int e = tid + 256 * i, row = e / CKs, c8 = (e % CKs) * 8;
+      dinr[i] = *(const v8*)(dip + (int64_t)(row < L ? row : L - 1) * H * K + c8);
+    }
+  }
+  // the gate-gradient partial sums of the launch before, for the last step as well (wave 0, one row per lane)
+  float dgpv[4];   // (at most four key slices of 64 channels; no branch round the loads)
+  {
+    const int rl = (tid & (BT - 1)) < L ? (tid & (BT - 1)) : L - 1;
+    const float* gp0 = p.dgam_part ? p.dgam_part + (row0 + rl) * H + hh : &kZeroWord;
+    const int64_t zs = p.dgam_part ? p.total_rows * H : 0;
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        dinr[t][r4] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
-        if (dip && jrow < L) dinr[t][r4] = *(const v4*)(dip + (cw * TK + t) * 32 + 8 * r4 + 4 * (lane >> 5));
-      }
+    for (int z = 0; z < 4; ++z) dgpv[z] = gp0[(z < p.nparts ? z : 0) * zs];
   }
   f32x16 dkb[TK];   // d(kb)^T: columns (cw*TK+t)*32.., time row jrow
 #pragma unroll
@@ -1227,15 +1238,20 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       int i0 = ib * 32 + 8 * a + 4 * (lane >> 5);
+      // this lane's four rows of column j are adjacent in the transposed tiles: one 8-byte access each for Aw and
+      // for dA, which is left transposed (dA^T[j][i]; the product below reads it through the transposing load)
+      const f32x4 gi4 = *(const f32x4*)&sGam[i0];
+      const v4 aw4 = *(const v4*)&sAwT[j * LDT + i0];
+      v4 tot4;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         int i = i0 + b, r = 4 * a + b;
         bool low = j < i;
-        float gamma = low ? __expf(sGam[i] - gj) : 0.f;
-        float au = (float)sAw[i * LDT + j] * gamma;         // Au_ij
+        float gamma = low ? __expf(gi4[b] - gj) : 0.f;
+        float au = (float)aw4[b] * gamma;                   // Au_ij
         float x = low ? dAu[r] * au : 0.f;                  // dAu * Au
         float tot = low ? dA[r] + dAu[r] * gamma : 0.f;     // dAw total
-        sS1[i * LDT + j] = (T)tot;                          // dA (masked) [i][j]
+        tot4[b] = (T)tot;
         // row sums over the 32 lanes holding the same row: inside each row of 16 lanes on the data-parallel path,
         // then the first row's total handed to the second (sixteen butterflies through the LDS crossbar per lane
         // were a third of this kernel's time)
@@ -1243,12 +1259,13 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
         if ((lane & 31) == 16) slot(4 + jb, i) = rs;
         colsum += x;
       }
+      *(v4*)&sS1[j * LDT + i0] = tot4;                       // dA^T (masked) [j][i]
     }
     colsum += __shfl_xor(colsum, 32, 64);
     if (lane < 32) slot(6 + ib, j) = -colsum;
   } else {
-    // quadrant (0,1) lies strictly above the diagonal
-    for (int e = lane; e < 32 * 32; e += 64) sS1[(e >> 5) * LDT + 32 + (e & 31)] = (T)0.f;
+    // quadrant (0,1) lies strictly above the diagonal (rows 32.. of the transposed tile, columns 0..31)
+    for (int e = lane; e < 32 * 32; e += 64) sS1[(32 + (e >> 5)) * LDT + (e & 31)] = (T)0.f;
   }
   __syncthreads();  // dA complete; dw^T consumed
   IOK::put_tr(sTr1, tid, rk);   // k^T
@@ -1257,7 +1274,7 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
     // wave (rw, cw): rows a = 32rw.., cols j = 32cw..  ; contraction over b
     f32x16 x1 = zero16();
     for (int bs = 0; bs < BT; bs += 16)
-      x1 = Elem<T>::mfma32(lds_frag32<T>(sS1, LDT, rw * 32, bs, lane), lds_frag32<T>(sAw, LDT, cw * 32, bs, lane), x1);
+      x1 = Elem<T>::mfma32(frag32_tr<T>(sS1, LDT, rw * 32, bs, lane), lds_frag32<T>(sAw, LDT, cw * 32, bs, lane), x1);
     const int j = cw * 32 + (lane & 31);
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
@@ -1315,12 +1332,11 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
       for (int r4 = 0; r4 < 4; ++r4) {
         const int col = (cw * TK + t) * 32 + 8 * r4 + 4 * (lane >> 5);
         v4 kk = *(const v4*)&sRow2[jrow * LDD + col], o;
-        const v4 din = dinr[t][r4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float d = dkb[t][4 * r4 + e];
           part += d * (float)kk[e];
-          o[e] = (T)(d * bj + dk2[t][4 * r4 + e] + (float)din[e]);
+          o[e] = (T)(d * bj + dk2[t][4 * r4 + e]);
         }
         // dk takes the place of the k element this lane has just read (nobody else reads the tile any more)
         *(v4*)&sRow2[jrow * LDD + col] = o;
@@ -1334,8 +1350,10 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
     if (ok) p.dbeta[(row0 + tid) * H + hh] = (slot(0, tid) + slot(1, tid)) + (slot(2, tid) + slot(3, tid));
     float dgm = ok ? (slot(4, tid) + slot(5, tid)) + (slot(6, tid) + slot(7, tid)) : 0.f;
     if (p.dgam_part) {
-      for (int z = 0; z < p.nparts; ++z)
-        dgm += ok ? p.dgam_part[((int64_t)z * p.total_rows + row0 + tid) * H + hh] : 0.f;
+      float dgp = 0.f;
+#pragma unroll
+      for (int z = 0; z < 4; ++z) dgp += z < p.nparts ? dgpv[z] : 0.f;
+      dgm += ok ? dgp : 0.f;
       // inclusive suffix sum over the 64 rows: DPP row scans plus the totals of the later rows of 16
       float x = row_suffix16(dgm);
       const float t1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 16));
@@ -1356,9 +1374,16 @@ __global__ __launch_bounds__(256, K <= 128 ? 2 : 1) void gdr_bwd_wy_kernel(WyBwd
   // several times their bytes)
   {
     constexpr int CK = K / 8, CV = V / 8;
-    for (int e = tid; e < BT * CK; e += 256) {
-      const int row = e / CK, c8 = (e % CK) * 8;
-      if (row < L) *(v8*)((T*)p.dk + ((row0 + row) * H + hh) * (int64_t)K + c8) = *(const v8*)&sRow2[row * LDD + c8];
+    // dk = this launch's part (rounded once into the tile) + the partial dk of the launch before
+#pragma unroll
+    for (int i = 0; i < NDI; ++i) {
+      const int e = tid + 256 * i, row = e / CK, c8 = (e % CK) * 8;
+      v8 x = *(const v8*)&sRow2[row * LDD + c8];
+      if (p.dk_in) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x[j] = (T)((float)x[j] + (float)dinr[i][j]);
+      }
+      if (row < L) *(v8*)((T*)p.dk + ((row0 + row) * H + hh) * (int64_t)K + c8) = x;
     }
     for (int e = tid; e < BT * CV; e += 256) {
       const int row = e / CV, c8 = (e % CV) * 8;
