@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   __shared__ __attribute__((aligned(16))) char sRB[REG_A];  // v_new row-major -> staging (dk intra)
   __shared__ __attribute__((aligned(16))) char sRC[REG_C];  // k^T | q^T -> staging (dk inter)
   __shared__ __attribute__((aligned(16))) char sRD[REG_C];  // ds | ds^T -> staging (dw)
-  __shared__ float sGam[BT];
+  __shared__ __attribute__((aligned(16))) float sGam[BT];
   T* sDo = (T*)sRA;
   T* sVn = (T*)sRB;
   T* sKT = (T*)sRC;
@@ -650,6 +650,7 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   struct Raw {
     v4 q[4], k[4], w[4];
     v8 d[NP], v[NP];
+    float gam;   // the gate row of lane % 64
   };
   // byte offsets of this lane's pieces from the first row of a chunk (32-bit, off wave-uniform base pointers)
   const uint32_t pitchk = (uint32_t)H * K * (uint32_t)sizeof(T), pitchv = (uint32_t)H * V * (uint32_t)sizeof(T);
@@ -684,6 +685,10 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
       R.d[i] = *(const v8*)(db + o);
       R.v[i] = *(const v8*)(vb + o);
     }
+    // with the rows, not behind the state fragments the item itself asks for: a value that goes to LDS right away
+    // would otherwise wait for every load queued in front of it (without gates: one zero word, no branch)
+    const uint32_t grow = (uint32_t)(tid0 & (BT - 1)) < last ? (uint32_t)(tid0 & (BT - 1)) : last;
+    R.gam = *(p.gam ? p.gam + (im.cl.row0 + grow) * H + im.hh : &kZeroWord);
   };
   uint32_t it = blockIdx.x;
   if (it >= nitems) return;
@@ -714,7 +719,6 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
       cww[i] = ok ? R.w[i] : z4;
     }
   }
-  const float glast = p.gam ? p.gam[(row0 + L - 1) * H + hh] : 0.f;
   v8 dreg[NP], vreg[NP], d2reg[NP];
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
@@ -740,7 +744,7 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
       dhf[vt][1] = *(const v8*)(dhb + o + 16);
     }
   }
-  if (tid < BT) sGam[tid] = p.gam ? p.gam[(row0 + (tid < L ? tid : L - 1)) * H + hh] : 0.f;
+  if (tid < BT) sGam[tid] = R.gam;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
     int e = tid + 256 * i, row = e / C8, c8 = (e % C8) * 8;
@@ -758,12 +762,6 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
     *(v4*)&sKT[(c4 + j) * LDT + rg * 4] = kt;
     *(v4*)&sQT[(c4 + j) * LDT + rg * 4] = qt;
   }
-  // <h_c, dH_c> over this wave's tiles (same fragment order on both sides)
-  float hd = 0.f;
-#pragma unroll
-  for (int vt = 0; vt < VT32; ++vt)
-#pragma unroll
-    for (int half = 0; half < 2; ++half) hd = Elem<T>::dot8(hf[vt][half], dhf[vt][half], hd);
   __syncthreads();
   // ---- ds = s tril((do v_new^T) * Gamma), both orientations
   {
@@ -778,16 +776,18 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
         s2 = Elem<T>::mfma32(fv, fd, s2);  // rows j, cols i
       }
       const int c = lane & 31;
+      const float gj1 = sGam[jb * 32 + c], gi2 = sGam[ib * 32 + c];
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
         int r0 = 8 * a + 4 * (lane >> 5);
+        const f32x4 gi1 = *(const f32x4*)&sGam[ib * 32 + r0], gj2 = *(const f32x4*)&sGam[jb * 32 + r0];
         v4 x1, x2;
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
           int i1 = ib * 32 + r0 + b, j1 = jb * 32 + c;
-          x1[b] = (T)((j1 <= i1) ? s1[4 * a + b] * p.scale * __expf(sGam[i1] - sGam[j1]) : 0.f);
+          x1[b] = (T)((j1 <= i1) ? s1[4 * a + b] * p.scale * __expf(gi1[b] - gj1) : 0.f);
           int j2 = jb * 32 + r0 + b, i2 = ib * 32 + c;
-          x2[b] = (T)((j2 <= i2) ? s2[4 * a + b] * p.scale * __expf(sGam[i2] - sGam[j2]) : 0.f);
+          x2[b] = (T)((j2 <= i2) ? s2[4 * a + b] * p.scale * __expf(gi2 - gj2[b]) : 0.f);
         }
         *(v4*)&sDsT[(jb * 32 + c) * LDT + ib * 32 + r0] = x1;
         *(v4*)&sDs[(ib * 32 + c) * LDT + jb * 32 + r0] = x2;
@@ -797,24 +797,38 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   __syncthreads();
   // ---- dq = s e^gamma (do h^T) + ds k ; dk_intra = ds^T q ; dk_inter = v_new dH^T
   f32x16 aq = zero16(), ak1 = zero16(), ak2 = zero16(), aw = zero16();
+  const float glast = sGam[L - 1];
+  // <h_c, dH_c> over this wave's tiles (same fragment order on both sides); here, where the fragments are first
+  // needed, and not at the top of the item, where they have just been asked for
+  float hd = 0.f;
+#pragma unroll
+  for (int vt = 0; vt < VT32; ++vt)
+#pragma unroll
+    for (int half = 0; half < 2; ++half) hd = Elem<T>::dot8(hf[vt][half], dhf[vt][half], hd);
 #pragma unroll
   for (int vt = 0; vt < VT32; ++vt)
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      aq = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aq);
-      ak2 = Elem<T>::mfma32(lds_frag32_perm<T>(sVn, LDV, rw * 32, vt * 32 + half * 16, lane), dhf[vt][half], ak2);
+      // transposed products (the state fragment as the first operand): a lane ends up with one time row and, per
+      // register quad, four adjacent key channels - the per-row factors are one exponential per lane, and the
+      // accumulators leave as 16-byte pieces
+      aq = Elem<T>::mfma32(hf[vt][half], lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), aq);
+      ak2 = Elem<T>::mfma32(dhf[vt][half], lds_frag32_perm<T>(sVn, LDV, rw * 32, vt * 32 + half * 16, lane), ak2);
     }
+  const float gm = sGam[rw * 32 + (lane & 31)];   // this lane's time row
+  {
+    const float eq = p.scale * __expf(gm), ek = __expf(glast - gm);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float g = sGam[rw * 32 + c32_row(r, lane)];
-    aq[r] *= p.scale * __expf(g);
-    ak2[r] *= __expf(glast - g);
+    for (int r = 0; r < 16; ++r) {
+      aq[r] *= eq;
+      ak2[r] *= ek;
+    }
   }
   const int jend = (rw + 1) * 32;
   for (int js = 0; js < jend; js += 16)
-    aq = Elem<T>::mfma32(lds_frag32<T>(sDs, LDT, rw * 32, js, lane), lds_frag32<T>(sKT, LDT, cw * 32, js, lane), aq);
+    aq = Elem<T>::mfma32(lds_frag32<T>(sKT, LDT, cw * 32, js, lane), lds_frag32<T>(sDs, LDT, rw * 32, js, lane), aq);
   for (int is = rw * 32; is < BT; is += 16)
-    ak1 = Elem<T>::mfma32(lds_frag32<T>(sDsT, LDT, rw * 32, is, lane), lds_frag32<T>(sQT, LDT, cw * 32, is, lane), ak1);
+    ak1 = Elem<T>::mfma32(lds_frag32<T>(sQT, LDT, cw * 32, is, lane), lds_frag32<T>(sDsT, LDT, rw * 32, is, lane), ak1);
   __syncthreads();  // do is consumed: its tile takes dv2
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
@@ -827,17 +841,20 @@ __global__ __launch_bounds__(256, 2) void gdr_bwd_dqkwg_kernel(DqkwgParams p, in
   for (int vt = 0; vt < VT32; ++vt)
 #pragma unroll
     for (int half = 0; half < 2; ++half)
-      aw = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aw);
+      aw = Elem<T>::mfma32(hf[vt][half], lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), aw);
+  {
+    const float ew = -__expf(gm);
 #pragma unroll
-  for (int r = 0; r < 16; ++r) aw[r] *= -__expf(sGam[rw * 32 + c32_row(r, lane)]);
+    for (int r = 0; r < 16; ++r) aw[r] *= ew;
+  }
   __syncthreads();  // all operand reads done: tiles become fp32 staging
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    int o = (rw * 32 + c32_row(r, lane)) * LDM + cw * 32 + (lane & 31);
-    stA[o] = aq[r];
-    stB[o] = ak1[r];
-    stC[o] = ak2[r];
-    stD[o] = aw[r];
+  for (int a4 = 0; a4 < 4; ++a4) {
+    const int o = (rw * 32 + (lane & 31)) * LDM + cw * 32 + 8 * a4 + 4 * (lane >> 5);
+    *(f32x4*)&stA[o] = f32x4{aq[4 * a4], aq[4 * a4 + 1], aq[4 * a4 + 2], aq[4 * a4 + 3]};
+    *(f32x4*)&stB[o] = f32x4{ak1[4 * a4], ak1[4 * a4 + 1], ak1[4 * a4 + 2], ak1[4 * a4 + 3]};
+    *(f32x4*)&stC[o] = f32x4{ak2[4 * a4], ak2[4 * a4 + 1], ak2[4 * a4 + 2], ak2[4 * a4 + 3]};
+    *(f32x4*)&stD[o] = f32x4{aw[4 * a4], aw[4 * a4 + 1], aw[4 * a4 + 2], aw[4 * a4 + 3]};
   }
   // the next item's first rows are requested now: the accumulators are in LDS, the epilogue needs few registers
   const uint32_t nit = it + gridDim.x;
