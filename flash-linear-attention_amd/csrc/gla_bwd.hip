@@ -1196,10 +1196,12 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
   // ---- accumulate: dq (intra + inter), dk intra, dk inter
   f32x16 aq = zero16(), ak1 = zero16(), ak2 = zero16();
   const int jend = (rw + 1) * 32;
+  // (transposed products - the key-channel operand first: a lane ends up with one time row and, per register quad,
+  // four adjacent key channels, so the accumulators leave for the staging tiles as 16-byte pieces)
   for (int js = 0; js < jend; js += 16)
-    aq = Elem<T>::mfma32(lds_frag32<T>(sdA, LDT, rw * 32, js, lane), lds_frag32<T>(sKtT, LDT, cw * 32, js, lane), aq);
+    aq = Elem<T>::mfma32(lds_frag32<T>(sKtT, LDT, cw * 32, js, lane), lds_frag32<T>(sdA, LDT, rw * 32, js, lane), aq);
   for (int is = rw * 32; is < BT; is += 16)
-    ak1 = Elem<T>::mfma32(lds_frag32<T>(sdAT, LDT, rw * 32, is, lane), lds_frag32<T>(sQtT, LDT, cw * 32, is, lane), ak1);
+    ak1 = Elem<T>::mfma32(lds_frag32<T>(sQtT, LDT, cw * 32, is, lane), lds_frag32<T>(sdAT, LDT, rw * 32, is, lane), ak1);
   // sum over the value columns of h_c * dH_c on the way: both sets of fragments hold one key column per
   // lane, and each pair is dead once its products are issued (the two row-block waves of a column block
   // hold the same fragments; one of them reports)
@@ -1208,8 +1210,8 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
   for (int vt = 0; vt < VT32; ++vt)
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      aq = Elem<T>::mfma32(lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), hf[vt][half], aq);
-      ak2 = Elem<T>::mfma32(lds_frag32_perm<T>(sV, LDV, rw * 32, vt * 32 + half * 16, lane), dhf[vt][half], ak2);
+      aq = Elem<T>::mfma32(hf[vt][half], lds_frag32_perm<T>(sDo, LDV, rw * 32, vt * 32 + half * 16, lane), aq);
+      ak2 = Elem<T>::mfma32(dhf[vt][half], lds_frag32_perm<T>(sV, LDV, rw * 32, vt * 32 + half * 16, lane), ak2);
       hd = Elem<T>::dot8(hf[vt][half], dhf[vt][half], hd);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1217,11 +1219,11 @@ __global__ __launch_bounds__(256, 2) void gla_bwd_dqkg_kernel(BDqkgParams p, int
   if (rw == 0 && lane < 32) sHd[cw * 32 + lane] = hd;
   __syncthreads();  // every MFMA operand read is done: the tiles become fp32 staging
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    int o = (rw * 32 + c32_row(r, lane)) * LDM + cw * 32 + (lane & 31);
-    stA[o] = aq[r];
-    stB[o] = ak1[r];
-    stC[o] = ak2[r];
+  for (int a4 = 0; a4 < 4; ++a4) {
+    const int o = (rw * 32 + (lane & 31)) * LDM + cw * 32 + 8 * a4 + 4 * (lane >> 5);
+    *(f32x4*)&stA[o] = f32x4{aq[4 * a4], aq[4 * a4 + 1], aq[4 * a4 + 2], aq[4 * a4 + 3]};
+    *(f32x4*)&stB[o] = f32x4{ak1[4 * a4], ak1[4 * a4 + 1], ak1[4 * a4 + 2], ak1[4 * a4 + 3]};
+    *(f32x4*)&stC[o] = f32x4{ak2[4 * a4], ak2[4 * a4 + 1], ak2[4 * a4 + 2], ak2[4 * a4 + 3]};
   }
   // the next item's first rows are requested now: the accumulators are in LDS, the epilogue needs few registers
   const uint32_t nit = it + gridDim.x;
