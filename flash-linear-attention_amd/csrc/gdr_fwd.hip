@@ -108,6 +108,14 @@ FLA_DEVICE void wy_stage_t(T* dstT, const typename Elem<T>::v4* reg, const float
   }
 }
 
+// One step of the forward substitution of wy_invert: x[c] += nm[J] * (x[c] of lane J of this DPP row), c <= J.
+template <int J>
+FLA_DEVICE void wy_subst_step(float (&x)[16], const float (&nm)[16]) {
+#pragma unroll
+  for (int c = 0; c <= J; ++c) x[c] = fmaf(nm[J], dpp_f32<0x150 + J>(x[c]), x[c]);   // row_newbcast:J
+  if constexpr (J < 14) wy_subst_step<J + 1>(x, nm);
+}
+
 // X = (I + M)^-1 for a strictly lower triangular fp32 M [64][LDM] in LDS, into sX [64][LDM]
 // (lower triangle valid; the upper right quadrant is used as scratch and holds garbage afterwards).
 // 16x16 diagonal blocks by forward substitution, then block merges X_ba = -X_bb (M_ba X_aa) on the
@@ -121,24 +129,30 @@ FLA_DEVICE void wy_invert(const float* sM, float* sX, int tid) {
     int blk = e >> 8, i = (e >> 4) & 15, j = e & 15;
     sX[(32 * blk + i) * LDM + 32 * blk + 16 + j] = 0.f;
   }
-  // 16x16 diagonal blocks by forward substitution (one lane per column)
+  // 16x16 diagonal blocks by forward substitution, all four at once on the first wave: DPP row b is block b,
+  // a lane holds row i of its block of M (zero on and above the diagonal) and of X.  Step j subtracts
+  // M[i][j] X[j][:] from every row; X[j][:] reaches the 16 lanes of the block through row_newbcast:j, so the
+  // 120 dependent updates are register-to-register (the order of the products in every entry's sum is j
+  // ascending, as a row-by-row substitution forms them).
   if (tid < 64) {
-    const int b = tid >> 4, col = tid & 15;
-    const float* Mb = sM + (16 * b) * LDM + 16 * b;
-    float x[16];
+    const int b = tid >> 4, i = tid & 15;
+    const float* Mr = sM + (16 * b + i) * LDM + 16 * b;
+    float nm[16], x[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      float m[16];
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 m = *(const f32x4*)&Mr[4 * q];
 #pragma unroll
-      for (int q = 0; 4 * q < i; ++q) *(f32x4*)&m[4 * q] = *(const f32x4*)&Mb[i * LDM + 4 * q];
-      float s = (i == col) ? 1.f : 0.f;
-#pragma unroll
-      for (int j = 0; j < i; ++j) s -= m[j] * x[j];
-      x[i] = s;
-      if ((i & 3) == 3) __builtin_amdgcn_sched_barrier(0);   // keeps the row loads of later rows from piling up in registers
+      for (int e = 0; e < 4; ++e) nm[4 * q + e] = -m[e];
     }
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sX[(16 * b + i) * LDM + 16 * b + col] = x[i];
+    for (int c = 0; c < 16; ++c) x[c] = (c == i) ? 1.f : 0.f;
+    wy_subst_step<0>(x, nm);
+    float* Xr = sX + (16 * b + i) * LDM + 16 * b;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const f32x4 o = {x[4 * q], x[4 * q + 1], x[4 * q + 2], x[4 * q + 3]};
+      *(f32x4*)&Xr[4 * q] = o;
+    }
   }
   lds_barrier();
   // ---- 32x32 diagonal blocks: X_ba = -X_bb (M_ba X_aa) for the block pairs (1,0) and (3,2)
@@ -545,65 +559,70 @@ __global__ __launch_bounds__(256, KEEP ? kPrepResidentKeep : kPrepResident) void
 
     wy_invert(sM, sX, tid);
 
-    // ---- Tu = (X * Gamma) diag(beta), one 16-element block row per thread, straight to memory
+    // ---- Tu = (X * Gamma) diag(beta): the ten 16x16 blocks of the lower triangle are dealt to the waves; a lane
+    // holds four adjacent columns of one row, and a block leaves for memory as 512 contiguous bytes straight
+    // from the registers (the packed tile is never staged)
     {
-      const int i = tid >> 2, jb = tid & 3, tt = i >> 4;
-      if (jb <= tt) {
-        const float gi = sGam[i];
-        v8 tu[2];
+      const int wv = __builtin_amdgcn_readfirstlane(wave);
+      const int r = lane >> 2, c4 = 4 * (lane & 3);
+      T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)kTriElems;
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const f32x4 xv = *(const f32x4*)&sX[i * LDM + 16 * jb + 4 * q4];
-          const f32x4 gj = *(const f32x4*)&sGam[16 * jb + 4 * q4];
-          const f32x4 bj = *(const f32x4*)&sBeta[16 * jb + 4 * q4];
+      for (int pass = 0; pass < 3; ++pass) {
+        const int idx = wv + 4 * pass;          // tri_block(tt, jb)
+        if (idx < 10) {
+          const int tt = idx >= 6 ? 3 : idx >= 3 ? 2 : idx >= 1 ? 1 : 0;
+          const int jb = idx - tt * (tt + 1) / 2;
+          const int i = 16 * tt + r, j0 = 16 * jb + c4;
+          const f32x4 xv = *(const f32x4*)&sX[i * LDM + j0];
+          const f32x4 gj = *(const f32x4*)&sGam[j0];
+          const f32x4 bj = *(const f32x4*)&sBeta[j0];
+          const float gi = sGam[i];
+          // X is zero above the diagonal of a diagonal block; the exponent there is set to zero so that the product stays zero
+          const f32x4 x = xv;
+          v4 tu;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int jj = 4 * q4 + e, j = 16 * jb + jj;
-            tu[jj >> 3][jj & 7] = (T)(j <= i ? xv[e] * __expf(gi - gj[e]) * bj[e] : 0.f);
+            const float d = gi - gj[e];
+            tu[e] = (T)(x[e] * __expf(tt != jb || c4 + e <= r ? d : 0.f) * bj[e]);
+          }
+          *(v4*)(at + idx * 256 + 4 * lane) = tu;
+          if constexpr (KEEP) {
+            // Aw row piece to memory; Aw diag(beta) as a row-major 16-bit tile in region A (M is dead)
+            v4 aw, ab;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              aw[e] = (T)x[e];
+              ab[e] = (T)(x[e] * bj[e]);
+            }
+            *(v4*)&sAb[i * LDT + j0] = ab;
+            if (i < L) *(v4*)((T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + j0) = aw;
           }
         }
-        T* dst = sTu + tri_block(tt, jb) * 256 + (i & 15) * 16;   // M is dead: its storage takes the packed tile
-        *(v8*)dst = tu[0];
-        *(v8*)(dst + 8) = tu[1];
       }
       if constexpr (KEEP) {
-        // Aw row piece to memory; Aw diag(beta) as a row-major 16-bit tile behind the packed tile
-        v8 aw[2], ab[2];
+        // the blocks above the diagonal of Aw and of Aw diag(beta) are zero
+        const v4 z4 = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
 #pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-          const f32x4 xv = *(const f32x4*)&sX[i * LDM + 16 * jb + 4 * q4];
-          const f32x4 bj = *(const f32x4*)&sBeta[16 * jb + 4 * q4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int jj = 4 * q4 + e, j = 16 * jb + jj;
-            const float x = j <= i ? xv[e] : 0.f;
-            aw[jj >> 3][jj & 7] = (T)x;
-            ab[jj >> 3][jj & 7] = (T)(x * bj[e]);
+        for (int pass = 0; pass < 2; ++pass) {
+          const int u = wv + 4 * pass;          // the six blocks (tt, jb), jb > tt
+          if (u < 6) {
+            const int tt = u >= 5 ? 2 : u >= 3 ? 1 : 0;
+            const int jb = u - (tt == 0 ? 0 : tt == 1 ? 3 : 5) + tt + 1;
+            const int i = 16 * tt + r, j0 = 16 * jb + c4;
+            *(v4*)&sAb[i * LDT + j0] = z4;
+            if (i < L) *(v4*)((T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + j0) = z4;
           }
-        }
-        *(v8*)&sAb[i * LDT + 16 * jb] = ab[0];
-        *(v8*)&sAb[i * LDT + 16 * jb + 8] = ab[1];
-        if (i < L) {
-          T* ap = (T*)p.Aw + ((row0 + i) * H + hh) * (int64_t)BT + 16 * jb;
-          *(v8*)ap = aw[0];
-          *(v8*)(ap + 8) = aw[1];
         }
       }
     }
-    lds_barrier();
     if constexpr (KEEP) {
-      // X is dead: its storage takes k row-major again (rows past the end of the chunk zero)
+      lds_barrier();   // X fully consumed
+      // its storage takes k row-major again (rows past the end of the chunk zero)
 #pragma unroll
       for (int i = 0; i < NPL; ++i) {
         const int row = r0 + RPP * i;
         *(v8*)&sK2[row * LDK + c8] = row < L ? kkeep[i] : z;
       }
-    }
-    // the tile leaves as one contiguous 5 KB block, 16 bytes per lane
-    {
-      T* at = (T*)p.AT + (cglob * H + hh) * (int64_t)kTriElems;
-      constexpr int NP = kTriElems / 8;   // 16-byte pieces
-      for (int e = tid; e < NP; e += 256) *(v8*)(at + e * 8) = *(const v8*)&sTu[e * 8];
     }
     if constexpr (KEEP) {
       lds_barrier();   // k row-major complete
