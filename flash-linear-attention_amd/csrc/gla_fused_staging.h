@@ -89,9 +89,15 @@ struct StageLds {
 // (left in L.o by the matrix waves) to memory as whole rows, and one more barrier + store follows the last chunk.
 // SG: one log-gate per (token, head), p.g is fp32 [B*T, H]: a lane loads one word per row and uses it for all
 // its key channels, so the prefix sums and exponentials of a row are formed once.
-template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O, int BV = 64, bool LOGITS = false>
+// keep(buf, c): called right behind B1(c), while the tiles of chunk c sit complete in buffer buf (kernels that leave
+// copies of them in memory for a backward pass do it there; the tiles are next written after B1(c+1)).
+struct NoKeep {
+  FLA_DEVICE void operator()(int, int64_t) const {}
+};
+template <typename T, typename GT, int K, int NSTG, bool SG, bool STORE_O, int BV = 64, bool LOGITS = false,
+          typename KeepFn = NoKeep>
 FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, const SeqSpan& sp, int64_t nchunks,
-                                int hh, int vbase, int wave, int lane, int tid) {
+                                int hh, int vbase, int wave, int lane, int tid, KeepFn keep = KeepFn()) {
   typedef typename Elem<T>::v8 v8;
   constexpr int LDK = K + 8;
   constexpr int CPW = K / NSTG;                // key columns per staging wave
@@ -358,23 +364,28 @@ FLA_DEVICE void gla_stage_waves(const FusedParams& p, const StageLds<T>& L, cons
     // issues the same loads, so the wait counts keep the two register sets two chunk periods
     // apart instead of waiting for the set that was refilled last.
     lds_barrier();  // B1(0)
+    keep(0, 0);
     if (nchunks > 1) {
       stage(RB, 1, 1, [] { lds_barrier(); });  // contains B2(0)
       int64_t c = 1;
       for (int64_t pairs = (nchunks - 2) >> 1; pairs > 0; --pairs, c += 2) {
         lds_barrier();  // B1(c), c odd
         store_o();
+        keep(1, c);
         stage(RA, 0, c + 1, [] { lds_barrier(); });  // contains B2(c)
         lds_barrier();  // B1(c+1)
         store_o();
+        keep(0, c + 1);
         stage(RB, 1, c + 2, [] { lds_barrier(); });  // contains B2(c+1)
       }
       lds_barrier();  // B1(c)
       store_o();
+      keep(1, c);
       if (c + 1 < nchunks) {
         stage(RA, 0, c + 1, [] { lds_barrier(); });  // contains B2(c)
         lds_barrier();  // B1(c+1)
         store_o();
+        keep(0, c + 1);
       }
       lds_barrier();  // B2 of the last chunk
     } else {

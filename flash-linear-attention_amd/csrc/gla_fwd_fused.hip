@@ -280,11 +280,42 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
     return (int)(rem < BT ? rem : BT);
   };
 
+  // HT: the gated queries of a chunk and its decay factors, as the staging waves left them in LDS, for a
+  // backward pass whose reverse state scan then streams them instead of forming prefix sums and exponentials
+  // of its own.  The slabs of a head share the rows out; rows past the end of a short chunk are not written.
+  auto store_qg = [&](int buf, int64_t c) __attribute__((always_inline)) {
+    const int tid = (int)(threadIdx.x & 255);   // the staging waves run it, 256 threads like the matrix waves
+    if constexpr (HT) {
+      if (p.qg) {
+        constexpr int C8 = K / 8;
+        const int nrow = BT / nvb > 0 ? BT / nvb : 0, r0 = vb * nrow;
+        const int L = chunk_len(c);
+        T* qb = (T*)p.qg + ((sp.bos + c * BT) * H + hh) * (int64_t)K;
+        for (int e = tid; e < nrow * C8; e += 256) {
+          const int row = r0 + e / C8, c8 = (e % C8) * 8;
+          if (row < L) *(v8*)(qb + (int64_t)row * H * K + c8) = *(const v8*)&sQ[buf][row * LDK + swz_rm(row, c8)];
+        }
+        if (vb == 0 && tid < K) p.decay[((chunk0 + c) * H + hh) * (int64_t)K + tid] = sDecay[buf][tid];
+      }
+      if (p.kh_t) {
+        // k^ of the chunk, key-major as staged (rows of 64 time steps; zero past the end of a short chunk): the
+        // slabs share the key rows out
+        const int nrow = K / nvb, r0 = vb * nrow;
+        T* kb = (T*)p.kh_t + ((chunk0 + c) * H + hh) * (int64_t)K * BT;
+        for (int e = tid; e < nrow * (BT / 8); e += 256) {
+          const int row = r0 + e / (BT / 8), c8 = (e % (BT / 8)) * 8;
+          *(v8*)(kb + row * BT + c8) = *(const v8*)&sKh[buf][row * LDT + c8];
+        }
+      }
+    }
+  };
   int any_wide = 0;   // matrix waves: some chunk of this workgroup was flagged
   if (wave >= 4) {
     // staging waves: see gla_fused_staging.h
     StageLds<T> L{{sQ[0], sQ[1]}, {sK[0], sK[1]}, {sKh[0], sKh[1]}, {sDecay[0], sDecay[1]}, {sWide[0], sWide[1]}, sO};
-    gla_stage_waves<T, GT, K, NSTG, SG, true, BV, LOGITS>(p, L, sp, nchunks, hh, vbase, wave, lane, tid);
+    // (the copies of q~ and k^ a backward pass reads are theirs: the matrix waves are the critical path of a forward
+    // that keeps its activations)
+    gla_stage_waves<T, GT, K, NSTG, SG, true, BV, LOGITS>(p, L, sp, nchunks, hh, vbase, wave, lane, tid, store_qg);
   } else {
     // =========================== matrix waves ===========================
     const int rw = wave >> 1, cw = wave & 1;   // output tile: rows 32rw.., value columns 32cw..
@@ -342,34 +373,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
               *(v8*)dst = lo;
               *(v8*)(dst + 8) = hi;
             }
-          }
-        }
-      }
-    };
-    // HT: the gated queries of a chunk and its decay factors, as the staging waves left them in LDS, for a
-    // backward pass whose reverse state scan then streams them instead of forming prefix sums and exponentials
-    // of its own.  The slabs of a head share the rows out; rows past the end of a short chunk are not written.
-    auto store_qg = [&](int buf, int64_t c) {
-      if constexpr (HT) {
-        if (p.qg) {
-          constexpr int C8 = K / 8;
-          const int nrow = BT / nvb > 0 ? BT / nvb : 0, r0 = vb * nrow;
-          const int L = chunk_len(c);
-          T* qb = (T*)p.qg + ((sp.bos + c * BT) * H + hh) * (int64_t)K;
-          for (int e = tid; e < nrow * C8; e += 256) {
-            const int row = r0 + e / C8, c8 = (e % C8) * 8;
-            if (row < L) *(v8*)(qb + (int64_t)row * H * K + c8) = *(const v8*)&sQ[buf][row * LDK + swz_rm(row, c8)];
-          }
-          if (vb == 0 && tid < K) p.decay[((chunk0 + c) * H + hh) * (int64_t)K + tid] = sDecay[buf][tid];
-        }
-        if (p.kh_t) {
-          // k^ of the chunk, key-major as staged (rows of 64 time steps; zero past the end of a short chunk): the
-          // slabs share the key rows out
-          const int nrow = K / nvb, r0 = vb * nrow;
-          T* kb = (T*)p.kh_t + ((chunk0 + c) * H + hh) * (int64_t)K * BT;
-          for (int e = tid; e < nrow * (BT / 8); e += 256) {
-            const int row = r0 + e / (BT / 8), c8 = (e % (BT / 8)) * 8;
-            *(v8*)(kb + row * BT + c8) = *(const v8*)&sKh[buf][row * LDT + c8];
           }
         }
       }
@@ -462,7 +465,6 @@ __global__ __launch_bounds__(256 + 64 * NSTG) void gla_fwd_fused_kernel(FusedPar
         load_v();
       }
       store_ht(c);  // unconditional and a whole chunk period ahead of the next wait for the value loads
-      store_qg(buf, c);
       if (p.wide) {
         int wide = 0;
 #pragma unroll
