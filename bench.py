@@ -559,6 +559,34 @@ def bench_copy(device, steps=20):
             "frac_of_hbm_peak": round(2 * (1 << 30) / us / 1e3 / HBM_PEAK_GBS, 4)}
 
 
+def bench_cu_feed_rate(device, steps=20):
+    """What a CU is fed per nanosecond when it streams rows the way the staging waves of the chunk scans do
+    (fla_selftest_stream_tiles: one 256-thread workgroup per CU, 64 rows x 256 bytes per tensor and chunk at a
+    4 KiB row pitch, registers refilled as they are consumed, no arithmetic), for the sharing patterns of the
+    benchmark shapes: B=16 (every workgroup its own rows), B=8 with two and B=4 with four workgroups per
+    (sequence, head) - the value slabs of a head.  A scan's chunk period cannot be shorter than the bytes its
+    workgroup moves per chunk divided by this rate."""
+    import torch
+    from fla_amd import _backend as be
+    T, H, nt = 4096, 16, 4
+    out = {}
+    for B, share in ((16, 1), (8, 2), (4, 4)):
+        x = torch.randint(-2**31, 2**31 - 1, (nt, B, T, H, 64), dtype=torch.int32, device=device)
+        sink = torch.zeros(B * H * share, dtype=torch.int32, device=device)
+        tb = B * T * H * 256
+        fn = lambda: be.check(be.lib().fla_selftest_stream_tiles(be.ptr(x), tb, nt, be.ptr(sink), B, T, H, share,
+                                                                 be.stream_of(x)), "stream_tiles")
+        us = event_stats(fn, steps, 5)["median_us"]
+        per_wg = nt * T * 256
+        out[f"B{B}_share{share}"] = {
+            "us": round(us, 1), "workgroups": B * H * share,
+            "bytes_per_ns_per_cu": round(per_wg / us / 1e3, 1),
+            "into_cus_TBs": round(per_wg * B * H * share / us / 1e6, 2),
+            "from_hbm_TBs": round(nt * tb / us / 1e6, 2)}
+        del x
+    return out
+
+
 def bench_layer_steps(device, steps=20):
     """The row-wise steps either side of the operators at the operators' benchmark shape
     (B=8, T=4096, H=16, D=128; the convolution on 2048 channels, kernel 4): device time of each
@@ -865,6 +893,7 @@ def main():
         extra["chunk_simple_gla_fwd"] = bench_simple_gla(device)
         extra["gla_stages_reference_operands"] = bench_gla_stages(device)
         extra["device_copy_1GiB"] = bench_copy(device)
+        extra["cu_feed_rate"] = bench_cu_feed_rate(device)
     out = {
         "metric": "chunk fwd tokens/s (GLA, GatedDeltaNet, T=4K, D=128) + % of MFMA/HBM roofline",
         "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

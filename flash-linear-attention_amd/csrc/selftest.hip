@@ -1,6 +1,7 @@
 // Diagnostics: a tiny GEMM through the same MFMA fragment helpers the kernels
 // use, so that operand/accumulator lane ownership can be verified on a device
-// against a library matmul.
+// against a library matmul; and a probe of the rate at which a CU is fed when
+// it streams rows the way the chunk scans do.
 #include "fla_common.h"
 #include "mfma_tiles.h"
 
@@ -46,6 +47,57 @@ __global__ __launch_bounds__(64) void selftest_kernel(const bf16* __restrict__ A
   }
 }
 
+// One workgroup per CU (the LDS array sees to that) reads every row of one (sequence, head) of NT tensors
+// [B, T, H, 128] (16-bit elements: 256-byte row pieces at a pitch of 256 H bytes), 64 rows at a time, each register
+// refilled as soon as it is consumed - the access pattern of the staging waves of the chunk scans without their
+// arithmetic.  `share` workgroups read the same (sequence, head), as the value slabs of a head do.  The XOR of all
+// the words a workgroup read goes to sink[workgroup], which makes the result checkable.
+template <int NT>
+__global__ __launch_bounds__(256) void stream_tiles_kernel(const char* __restrict__ x, int64_t tensor_bytes,
+                                                           uint32_t* __restrict__ sink, int T, int H, int share) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  constexpr int NP = 4 * NT;   // 16-byte pieces per thread and 64-row chunk
+  __shared__ char pad[96 * 1024];
+  pad[threadIdx.x * 64] = (char)T;
+  const int tid = threadIdx.x;
+  const int pair = blockIdx.x / share;
+  const int b = pair / H, hh = pair % H;
+  const uint32_t pitch = (uint32_t)H * 256u;
+  uint32_t off[NP];
+  const char* base[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int e = tid + 256 * i;   // piece index: tensor, row, 16-byte column
+    off[i] = (uint32_t)((e % 1024) / 16) * pitch + (uint32_t)(e % 16) * 16u;
+    base[i] = x + (int64_t)(e / 1024) * tensor_bytes + ((int64_t)b * T * H + hh) * 256;
+  }
+  const int nchunks = T / 64;
+  const int64_t cstride = (int64_t)64 * pitch;
+  u4 R[NP];
+  u4 acc = {0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < NP; ++i) R[i] = *(const u4*)(base[i] + off[i]);
+  for (int c = 1; c < nchunks; ++c) {
+    const int64_t co = (int64_t)c * cstride;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      acc ^= R[i];
+      R[i] = *(const u4*)(base[i] + co + off[i]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NP; ++i) acc ^= R[i];
+  uint32_t w = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  // wave, then workgroup
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) w ^= (uint32_t)__shfl_xor((int)w, m);
+  uint32_t* red = (uint32_t*)(pad + 64 * 1024);
+  __syncthreads();
+  if ((tid & 63) == 0) red[tid >> 6] = w;
+  __syncthreads();
+  if (tid == 0) sink[blockIdx.x] = red[0] ^ red[1] ^ red[2] ^ red[3];
+}
+
 }  // namespace
 
 extern "C" int fla_selftest_mfma(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t Kd, int mode,
@@ -64,6 +116,26 @@ extern "C" int fla_selftest_mfma(const void* A, const void* B, float* C, int64_t
     hipLaunchKernelGGL(selftest_kernel<2>, dim3(M / 32, N / 32), dim3(64), 0, st, a, b, C, (int)M, (int)N, (int)Kd);
   } else {
     return FLA_E_INVALID;
+  }
+  FLA_CHECK_LAUNCH();
+  return FLA_OK;
+}
+
+extern "C" int fla_selftest_stream_tiles(const void* x, int64_t tensor_bytes, int n_tensors, uint32_t* sink, int64_t B,
+                                         int64_t T, int64_t H, int share, fla_stream_t stream) {
+  FLA_REQUIRE(x && sink, FLA_E_INVALID);
+  FLA_REQUIRE(B > 0 && H > 0 && T >= 64 && T % 64 == 0 && share >= 1 && n_tensors >= 1 && n_tensors <= 4,
+              FLA_E_UNSUPPORTED);
+  FLA_REQUIRE(tensor_bytes >= B * T * H * 256 && tensor_bytes % 16 == 0 && (uintptr_t)x % 16 == 0, FLA_E_INVALID);
+  FLA_REQUIRE(B * H * share <= 65536 && H * 256 * 64 < (1LL << 31) / 64, FLA_E_UNSUPPORTED);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)(B * H * share));
+  const char* xc = (const char*)x;
+  switch (n_tensors) {
+    case 1: hipLaunchKernelGGL(stream_tiles_kernel<1>, grid, dim3(256), 0, st, xc, tensor_bytes, sink, (int)T, (int)H, share); break;
+    case 2: hipLaunchKernelGGL(stream_tiles_kernel<2>, grid, dim3(256), 0, st, xc, tensor_bytes, sink, (int)T, (int)H, share); break;
+    case 3: hipLaunchKernelGGL(stream_tiles_kernel<3>, grid, dim3(256), 0, st, xc, tensor_bytes, sink, (int)T, (int)H, share); break;
+    default: hipLaunchKernelGGL(stream_tiles_kernel<4>, grid, dim3(256), 0, st, xc, tensor_bytes, sink, (int)T, (int)H, share); break;
   }
   FLA_CHECK_LAUNCH();
   return FLA_OK;

@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -91,6 +91,7 @@ SIGNATURES = {
     "fla_gdn_gate_fwd": (c_int, [P, P, P, P, P, P, I64, I64, I, I, P]),
     "fla_gdn_gate_bwd": (c_int, [P] * 9 + [I64, I64, I, I, P]),
     "fla_selftest_mfma": (c_int, [P, P, P, I64, I64, I64, I, P]),
+    "fla_selftest_stream_tiles": (c_int, [P, I64, I, P, I64, I64, I64, I, P]),
 }
 
 

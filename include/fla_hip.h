@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 12
+#define FLA_ABI_VERSION 13
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -695,6 +695,14 @@ int fla_gdn_gate_bwd(const void* a, const void* b, const float* A_log, const flo
  * used for fragment-layout states).  M, N multiples of 32, Kd of 32. */
 int fla_selftest_mfma(const void* A, const void* B, float* C, int64_t M, int64_t N, int64_t Kd,
                       int mode, fla_stream_t stream);
+
+/* Diagnostics: the rate at which a CU is fed when it streams rows the way the chunk scans do (no counterpart in the
+ * reference; bench.py reports it beside the scans it bounds).  x holds n_tensors (1-4) tensors [B, T, H, 128] of 16-bit
+ * elements, tensor_bytes apart; one 256-thread workgroup per CU reads every row of one (sequence, head) of all of
+ * them, 64 rows at a time, and `share` workgroups read the same (sequence, head).  sink[B*H*share] receives the XOR of
+ * all 32-bit words each workgroup read.  T a multiple of 64. */
+int fla_selftest_stream_tiles(const void* x, int64_t tensor_bytes, int n_tensors, uint32_t* sink, int64_t B,
+                              int64_t T, int64_t H, int share, fla_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -50,6 +50,8 @@ def test_argument_validation_without_device():
     assert lib.fla_chunk_local_cumsum(p, p, 7, 1, 0, 1, 1, 64, 0, None, None, 0, None) == -2     # unknown dtype
     assert lib.fla_chunk_gla_fwd_h(p, p, p, 0, None, p, None, None, None, 1, 0, 1, 1, 1, 64, 1, 100, 64, 1, None) == -2
     assert lib.fla_selftest_mfma(p, p, p, 33, 32, 32, 0, None) == -2
+    assert lib.fla_selftest_stream_tiles(p, 1 << 20, 3, p, 1, 100, 1, 1, None) == -2   # T not a multiple of 64
+    assert lib.fla_selftest_stream_tiles(p, 1 << 10, 3, p, 1, 64, 1, 1, None) == -1     # tensors overlap
     # the allocation-free cumsum refuses what its static scratch array (4 Mi floats) cannot hold
     assert lib.fla_chunk_global_cumsum_static(p, p, 0, 0, 1, 4 * 1024 * 1024 // 64 + 1, 8, 8, 64, 0, None, None, 0, None) == -4
     assert lib.fla_chunk_global_cumsum_static(None, p, 0, 0, 1, 1, 1, 1, 64, 0, None, None, 0, None) == -1

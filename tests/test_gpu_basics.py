@@ -24,6 +24,27 @@ def test_mfma_fragment_layout(device, mode):
     assert_close(f"mfma mode {mode}", ref, C, 1e-5)
 
 
+@pytest.mark.parametrize("nt,share", [(1, 1), (3, 2), (4, 4)])
+def test_stream_tiles_probe_reads_every_word_once(device, nt, share):
+    """The feed-rate probe bench.py times: each workgroup must have read exactly the rows of its (sequence, head) in
+    every tensor - its XOR over them is compared with numpy's."""
+    import numpy as np
+    from fla_amd import _backend as be
+    B, T, H = 2, 192, 3
+    gen = torch.Generator().manual_seed(5)
+    x = torch.randint(-2**31, 2**31 - 1, (nt, B, T, H, 64), dtype=torch.int32, generator=gen)
+    xd = x.to(device)
+    sink = torch.zeros(B * H * share, dtype=torch.int32, device=device)
+    print(f"stream tiles nt={nt} share={share}", flush=True)
+    be.check(be.lib().fla_selftest_stream_tiles(be.ptr(xd), B * T * H * 256, nt, be.ptr(sink), B, T, H, share,
+                                                be.stream_of(xd)), "stream_tiles")
+    torch.cuda.synchronize()
+    ref = np.bitwise_xor.reduce(x.numpy().view(np.uint32).transpose(1, 3, 0, 2, 4).reshape(B * H, -1), axis=1)
+    got = sink.cpu().numpy().view(np.uint32).reshape(B * H, share)
+    for s_ in range(share):
+        assert (got[:, s_] == ref).all()
+
+
 @pytest.mark.parametrize("shape", [(2, 300, 4, 64), (1, 150, 3, 100), (2, 1024, 2, 0), (3, 77, 5, 0), (1, 64, 2, 6)])
 @pytest.mark.parametrize("chunk", [32, 64])
 @pytest.mark.parametrize("reverse", [False, True])
