@@ -685,8 +685,9 @@ def bench_gla_stages(device, steps=20):
 
 
 def bench_simple_gla(device, steps=20):
-    """chunk_simple_gla forward (one log-gate per token and head) at config 1's shape: the per-head-gate
-    launch against the same operator through the per-key-gate kernel on a materialised gate tensor."""
+    """chunk_simple_gla forward (one log-gate per token and head) at config 1's shape: the operator's own launch
+    against the same operator through the per-key-gate kernel on a materialised gate tensor, and its two kernels
+    (the delta-rule scan without the delta rule, the GLA kernel's per-head-gate form) side by side."""
     import torch
     import torch.nn.functional as F
     from fla_amd.ops.gla import chunk_gla
@@ -697,11 +698,24 @@ def bench_simple_gla(device, steps=20):
     g = F.logsigmoid(torch.randn(B, T, H, device=device, generator=gen))
     h0 = torch.randn(B, H, D, D, device=device, generator=gen) * 0.1
     nbytes = 4 * q.numel() * 2 + g.numel() * 4 + 2 * h0.numel() * 4
+    import fla_amd.ops.simple_gla.chunk as sg_mod
+    routes = {}
     with torch.no_grad():
         us = event_avg_us(lambda: chunk_simple_gla(q, k, v, g, initial_state=h0, output_final_state=True,
                                                    head_first=False), steps)
         us_b = event_avg_us(lambda: chunk_gla(q, k, v, g[..., None].expand(B, T, H, D), initial_state=h0,
                                               output_final_state=True, head_first=False), steps)
+        # the two kernels that can serve a forward without gradients (the plain scan is the default), at B=8 and B=4
+        default = sg_mod.SCAN_FORWARD
+        try:
+            for name, flag in (("plain_scan_kernel", True), ("gla_kernel_per_head_gates", False)):
+                sg_mod.SCAN_FORWARD = flag
+                for Bx in (8, 4):
+                    fn = lambda: chunk_simple_gla(q[:Bx], k[:Bx], v[:Bx], g[:Bx], initial_state=h0[:Bx],
+                                                  output_final_state=True, head_first=False)
+                    routes[f"{name}_B{Bx}_us"] = round(event_avg_us(fn, steps), 1)
+        finally:
+            sg_mod.SCAN_FORWARD = default
     # forward + backward at config 4's batch (B=4): per-head-gate forward that keeps the states, per-head-gate backward
     Bb = 4
     leaves = [x[:Bb].clone().requires_grad_() for x in (q, k, v, g)]
@@ -720,7 +734,7 @@ def bench_simple_gla(device, steps=20):
     us_fb_b = event_avg_us(lambda: fb(chunk_gla, lambda x: x[..., None].expand(Bb, T, H, D)), steps)
     return {"us": round(us, 1), "tokens_per_s": round(B * T / us * 1e6, 1), "algorithmic_bytes": nbytes,
             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-            "through_per_key_gate_kernel_us": round(us_b, 1),
+            "through_per_key_gate_kernel_us": round(us_b, 1), **routes,
             "fwd_bwd_B4_us": round(us_fb, 1), "fwd_bwd_B4_through_per_key_gate_kernels_us": round(us_fb_b, 1)}
 
 

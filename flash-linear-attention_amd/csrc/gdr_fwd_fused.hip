@@ -105,10 +105,15 @@ FLA_DEVICE typename Elem<T>::v8 pair_rows(f32x4 a, f32x4 b) {
 // columns of the score blocks, rq on the scale of the inter-chunk output.  rk comes from the first launch; rq is formed
 // by the staging lanes from the q pieces they hold (a row sits in K / 8 adjacent lanes: four packed dot products and
 // four lane exchanges per piece).
-template <typename T, int K, bool KEEP, int NMW = 4, bool L2N = false>
+// DELTA = false: the same scan without the delta rule - v_new = v, no (k h) correction, no Tu tile - which is
+// chunk_simple_gla (fla/ops/simple_gla/chunk.py:16-131): h <- e^{g_last} h + (k e^{g_last - g})^T v,
+// o = s e^{g} (q h) + s tril(q k^T * Gamma) v.  p.gam then holds the RAW per-head log-gates and the staging wave that
+// owns the gate row forms the chunk-local prefix sum itself (64 lanes, DPP row scans).
+template <typename T, int K, bool KEEP, int NMW = 4, bool L2N = false, bool DELTA = true>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void gdr_fwd_scan_kernel(
     GdrScanParams p) {
   static_assert(!(KEEP && L2N), "a forward that keeps its intermediates takes normalised q and k");
+  static_assert(DELTA || (!KEEP && !L2N), "the plain scan: forward only, no l2 norm");
   typedef typename Elem<T>::v8 v8;
   typedef typename Elem<T>::v4 v4;
   constexpr int BV = 16 * NMW;
@@ -286,8 +291,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     auto load = [&](Regs& R) __attribute__((always_inline)) {
       const bool last = lcv >= nchunks - 1;
       const uint32_t limv = (last ? limv_last : limv_full) + colv;
-      R.a0 = *(const v8*)(la + offa0);   // a full tile whatever the chunk length
-      R.a1 = *(const v8*)(la + offa1);   // its last 64 pieces: every wave loads them, the first one writes them
+      if constexpr (DELTA) {
+        R.a0 = *(const v8*)(la + offa0);   // a full tile whatever the chunk length
+        R.a1 = *(const v8*)(la + offa1);   // its last 64 pieces: every wave loads them, the first one writes them
+      }
 #pragma unroll
       for (int i = 0; i < RV; ++i) R.v[i] = *(const v4*)(lv + (offv[i] < limv ? offv[i] : limv));
       if (lcv + 1 < nchunks) {
@@ -327,8 +334,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int i = 0; i < NPW; ++i) *(v8*)&sK[wq3][dq[i]] = R.k[i];
       if (wave == 4) {
         // lanes past the end of a short chunk carry the last row's gate
-        const float gam = __uint_as_float(R.gam & gmask);
-        const float glast = __uint_as_float(__builtin_amdgcn_readlane(R.gam & gmask, 63));
+        float gam = __uint_as_float(R.gam & gmask);
+        if constexpr (!DELTA) {
+          // raw gates: inclusive prefix sum over the 64 rows (rows past the end add zero)
+          const int Lw = wq == nchunks - 1 ? Llast : BT;
+          const float x = row_prefix16(lane < Lw ? gam : 0.f);
+          const float t0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 15));
+          const float t1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 31));
+          const float t2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 47));
+          const int rr = lane >> 4;
+          gam = x + (rr >= 1 ? t0 : 0.f) + (rr >= 2 ? t1 : 0.f) + (rr >= 3 ? t2 : 0.f);
+        }
+        const float glast = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gam), 63));
         sGam[wq3][lane] = gam;
         sEg[wq3][lane] = __expf(gam);
         if constexpr (L2N) {
@@ -352,8 +369,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < RV; ++i)
           if (urg * RV + i >= Llast) R.v[i] = v4{(T)0.f, (T)0.f, (T)0.f, (T)0.f};
       }
-      *(v8*)&sAT[b][st * 8] = R.a0;
-      if (wave == 4) *(v8*)&sAT[b][2048 + lane * 8] = R.a1;
+      if constexpr (DELTA) {
+        *(v8*)&sAT[b][st * 8] = R.a0;
+        if (wave == 4) *(v8*)&sAT[b][2048 + lane * 8] = R.a1;
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         rvv vc;
@@ -503,7 +522,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         auto load_kq = [&](int tt, v8* f) {
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            f[ks] = frag16<T>(Kr, LDR, 16 * tt, 32 * ks, lane);
+            if constexpr (DELTA) f[ks] = frag16<T>(Kr, LDR, 16 * tt, 32 * ks, lane);
             f[KS + ks] = frag16<T>(Q, LDR, 16 * tt, 32 * ks, lane);
           }
         };
@@ -542,7 +561,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           oq[tt] = zero4();
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            d[tt] = Elem<T>::mfma16(f[ks], hb[ks], d[tt]);
+            if constexpr (DELTA) d[tt] = Elem<T>::mfma16(f[ks], hb[ks], d[tt]);
             oq[tt] = Elem<T>::mfma16(f[KS + ks], hb[ks], oq[tt]);
           }
         };
@@ -567,12 +586,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           vv[tt] = *(const v4*)(vt + swz_t(vrow, 16 * tt + 4 * g));
         }
         const float dec = sDec[b3];
-        ft[0] = frag_tri<T>(Tu, 0, 0, lane);
-        ft[1] = frag_tri<T>(Tu, 1, 0, lane);
-        ft[2] = frag_tri<T>(Tu, 2, 0, lane);
-        ft[3] = frag_tri<T>(Tu, 2, 1, lane);
-        ft[4] = frag_tri<T>(Tu, 3, 0, lane);
-        ft[5] = frag_tri<T>(Tu, 3, 1, lane);
+        if constexpr (DELTA) {
+          ft[0] = frag_tri<T>(Tu, 0, 0, lane);
+          ft[1] = frag_tri<T>(Tu, 1, 0, lane);
+          ft[2] = frag_tri<T>(Tu, 2, 0, lane);
+          ft[3] = frag_tri<T>(Tu, 2, 1, lane);
+          ft[4] = frag_tri<T>(Tu, 3, 0, lane);
+          ft[5] = frag_tri<T>(Tu, 3, 1, lane);
+        }
         __builtin_amdgcn_sched_barrier(0);
         mm_kq(3, fb);
         __builtin_amdgcn_sched_barrier(0);
@@ -585,20 +606,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         fp[4] = frag_tri<T>(P, 3, 0, lane);
         fp[5] = frag_tri<T>(P, 3, 1, lane);
         __builtin_amdgcn_sched_barrier(0);
-        // r = v - e^{gamma} (k h), as the operand contracting over time
-        v8 rb[2];
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) rb[tt >> 1][(tt & 1) * 4 + r] = (T)((float)vv[tt][r] - d[tt][r] * eg[tt][r]);
-        // v_new = Tu r; Tu is lower triangular: row tiles 0 and 1 only meet the first 32 rows of r
         f32x4 vn[4];
-        vn[0] = Elem<T>::mfma16(ft[0], rb[0], zero4());
-        vn[1] = Elem<T>::mfma16(ft[1], rb[0], zero4());
-        vn[2] = Elem<T>::mfma16(ft[2], rb[0], zero4());
-        vn[3] = Elem<T>::mfma16(ft[4], rb[0], zero4());
-        vn[2] = Elem<T>::mfma16(ft[3], rb[1], vn[2]);
-        vn[3] = Elem<T>::mfma16(ft[5], rb[1], vn[3]);
+        if constexpr (DELTA) {
+          // r = v - e^{gamma} (k h), as the operand contracting over time
+          v8 rb[2];
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) rb[tt >> 1][(tt & 1) * 4 + r] = (T)((float)vv[tt][r] - d[tt][r] * eg[tt][r]);
+          // v_new = Tu r; Tu is lower triangular: row tiles 0 and 1 only meet the first 32 rows of r
+          vn[0] = Elem<T>::mfma16(ft[0], rb[0], zero4());
+          vn[1] = Elem<T>::mfma16(ft[1], rb[0], zero4());
+          vn[2] = Elem<T>::mfma16(ft[2], rb[0], zero4());
+          vn[3] = Elem<T>::mfma16(ft[4], rb[0], zero4());
+          vn[2] = Elem<T>::mfma16(ft[3], rb[1], vn[2]);
+          vn[3] = Elem<T>::mfma16(ft[5], rb[1], vn[3]);
+        } else {
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vn[tt][r] = (float)vv[tt][r];
+        }
         if constexpr (L2N) {
           // the (q h) term carries e^{gamma} / |q| instead
 #pragma unroll
@@ -684,6 +712,19 @@ int launch_scan(const GdrScanParams& p, int K, hipStream_t st) {
   if (narrow) nblk *= 2;
   dim3 grid((unsigned)nblk), block(512);
   const bool keep = p.v_new != nullptr;
+  if (!p.AT) {
+    // the plain scan (no delta rule, raw per-head gates)
+    if (keep || p.l2_eps >= 0.f) return FLA_E_UNSUPPORTED;
+#define FLA_SCAN_PLAIN(KK)                                                                                     \
+  if (narrow) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, false, 2, false, false>), grid, block, 0, st, p);  \
+  else hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, false, 4, false, false>), grid, block, 0, st, p);
+    if (K == 64) { FLA_SCAN_PLAIN(64) }
+    else if (K == 128) { FLA_SCAN_PLAIN(128) }
+    else return FLA_E_UNSUPPORTED;
+#undef FLA_SCAN_PLAIN
+    FLA_CHECK_LAUNCH();
+    return FLA_OK;
+  }
 #define FLA_SCAN(KK, KEEPV)                                                                              \
   if (narrow) hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 2>), grid, block, 0, st, p);          \
   else hipLaunchKernelGGL((gdr_fwd_scan_kernel<T, KK, KEEPV, 4>), grid, block, 0, st, p);
@@ -714,7 +755,7 @@ static int gdr_fwd_scan_impl(const void* q, const void* k, const void* v, const 
                              const int64_t* offsets, const int64_t* chunk_offsets, const int64_t* seq_order,
                              int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
                              float scale, float l2_eps, fla_stream_t stream, const float* k_rstd = nullptr) {
-  FLA_REQUIRE(q && k && v && AT && o, FLA_E_INVALID);
+  FLA_REQUIRE(q && k && v && o, FLA_E_INVALID);   // AT == NULL: the plain scan (fla_chunk_simple_gla_fwd_scan)
   FLA_REQUIRE((l2_eps >= 0.f) == (k_rstd != nullptr), FLA_E_INVALID);
   FLA_REQUIRE(B >= 0 && T >= 0 && H > 0 && K > 0 && V > 0 && N >= 0, FLA_E_INVALID);
   FLA_REQUIRE(offsets ? (B == 1 && chunk_offsets != nullptr) : N == B, FLA_E_INVALID);
@@ -736,6 +777,7 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan(const void* q, const void* k,
                                                    const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T,
                                                    int64_t H, int64_t K, int64_t V, int64_t N, float scale,
                                                    fla_stream_t stream) {
+  FLA_REQUIRE(AT, FLA_E_INVALID);
   return gdr_fwd_scan_impl(q, k, v, AT, g_cumsum, h0, o, ht, v_new, h_frag_t, Aqk_out, offsets, chunk_offsets,
                            seq_order, qkv_dtype, B, T, H, K, V, N, scale, -1.f, stream);
 }
@@ -750,4 +792,13 @@ extern "C" int fla_chunk_gated_delta_rule_fwd_scan_l2norm(const void* q, const v
   FLA_REQUIRE(eps >= 0.f && k_rstd, FLA_E_INVALID);
   return gdr_fwd_scan_impl(q, k, v, AT, g_cumsum, h0, o, ht, nullptr, nullptr, nullptr, offsets, chunk_offsets,
                            seq_order, qkv_dtype, B, T, H, K, V, N, scale, eps, stream, k_rstd);
+}
+
+extern "C" int fla_chunk_simple_gla_fwd_scan(const void* q, const void* k, const void* v, const float* g,
+                                             const float* h0, void* o, float* ht, const int64_t* offsets,
+                                             const int64_t* chunk_offsets, const int64_t* seq_order, int qkv_dtype,
+                                             int64_t B, int64_t T, int64_t H, int64_t K, int64_t V, int64_t N,
+                                             float scale, fla_stream_t stream) {
+  return gdr_fwd_scan_impl(q, k, v, nullptr, g, h0, o, ht, nullptr, nullptr, nullptr, offsets, chunk_offsets,
+                           seq_order, qkv_dtype, B, T, H, K, V, N, scale, -1.f, stream);
 }

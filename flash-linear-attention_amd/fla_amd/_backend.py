@@ -16,7 +16,7 @@ _lib = None
 
 FLA_F32, FLA_BF16, FLA_F16 = 0, 1, 2
 FLA_H_ROW_MAJOR, FLA_H_FRAGMENT, FLA_H_FRAGMENT_T = 0, 1, 2
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _DTYPES = {torch.float32: FLA_F32, torch.bfloat16: FLA_BF16, torch.float16: FLA_F16}
 
@@ -55,6 +55,7 @@ SIGNATURES = {
     "fla_chunk_gated_delta_rule_fwd_h_both": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, P]),
     "fla_gdr_fwd_prep": (c_int, [P, P, P, I, P, P, P, P, P, P, I64, I, I64, I64, I64, I64, P]),
     "fla_chunk_gated_delta_rule_fwd_scan": (c_int, [P] * 14 + [I, I64, I64, I64, I64, I64, I64, F, P]),
+    "fla_chunk_simple_gla_fwd_scan": (c_int, [P] * 10 + [I, I64, I64, I64, I64, I64, I64, F, P]),
     "fla_gdr_fwd_prep_l2norm": (c_int, [P, P, P, I, P, P, P, P, P, I64, I, I64, I64, I64, I64, F, P]),
     "fla_chunk_gated_delta_rule_fwd_scan_l2norm": (c_int, [P] * 12 + [I, I64, I64, I64, I64, I64, I64, F, F, P]),
     "fla_chunk_gated_delta_rule_fwd_onepass": (c_int, [P] * 11 + [I, I64, I64, I64, I64, I64, I64, F, I, F, P]),

@@ -10,10 +10,40 @@ from typing import Optional, Tuple
 
 import torch
 
+import os
+
 from ... import _backend as be
-from ...utils import check_varlen_args, contiguous, resolve_offsets
+from ...utils import VarlenPlan, check_varlen_args, contiguous, resolve_offsets
 from ..gla import chunk as gla_chunk
 from ..gla.chunk import chunk_gla, chunk_gla_bwd_device, chunk_gla_fwd_fused
+
+
+# A forward without gradients runs on the delta-rule scan kernel with the delta rule taken out
+# (``fla_chunk_simple_gla_fwd_scan``): raw q and k tiles, gates on the score blocks and on rows, no range guard.
+# ``FLA_AMD_SIMPLE_GLA_FUSED=1`` sends it through the GLA kernel's per-head-gate instantiation instead.
+SCAN_FORWARD = os.environ.get("FLA_AMD_SIMPLE_GLA_FUSED", "0") != "1"
+
+
+def chunk_simple_gla_fwd_scan(q, k, v, g, scale, initial_state, output_final_state, offsets=None):
+    """``fla_chunk_simple_gla_fwd_scan``: seq-first 16-bit ``q, k, v``, raw per-head log-gates ``g`` ``[B,T,H]`` (any
+    float dtype; ``None`` for no decay), K in {64, 128}, V a multiple of 64.  Returns ``(o, final_state)``."""
+    be.require_gpu(q, k, v)
+    B, T, H, K = k.shape
+    V = v.shape[-1]
+    N, co, order = B, None, None
+    if offsets is not None:
+        plan = VarlenPlan(offsets, 64)
+        N, offsets, co, order = plan.N, plan.offsets, plan.chunk_offsets, plan.seq_order
+    o = torch.empty_like(v)
+    ht = k.new_empty(N, H, K, V, dtype=torch.float32) if output_final_state else None
+    h0 = None
+    if initial_state is not None:
+        h0 = (initial_state if initial_state.dtype == torch.float32 else initial_state.float()).contiguous()
+    gf = None if g is None else (g if g.dtype == torch.float32 else g.float()).contiguous()
+    be.check(be.lib().fla_chunk_simple_gla_fwd_scan(
+        be.ptr(q), be.ptr(k), be.ptr(v), be.ptr(gf), be.ptr(h0), be.ptr(o), be.ptr(ht), be.ptr(offsets), be.ptr(co),
+        be.ptr(order), be.dt(k), B, T, H, K, V, N, float(scale), be.stream_of(k)), "fla_chunk_simple_gla_fwd_scan")
+    return o, ht
 
 
 class ChunkSimpleGLAFunction(torch.autograd.Function):
@@ -90,6 +120,9 @@ def chunk_simple_gla(
             and q.dtype in (torch.bfloat16, torch.float16) and k.dtype == q.dtype and v.dtype == q.dtype):
         if needs_grad:
             return ChunkSimpleGLAFunction.apply(q, k, v, g, scale, initial_state, output_final_state, offsets)
+        if SCAN_FORWARD:
+            return chunk_simple_gla_fwd_scan(q.contiguous(), k.contiguous(), v.contiguous(), g, scale, initial_state,
+                                             output_final_state, offsets=offsets)
         return chunk_gla_fwd_fused(q.contiguous(), k.contiguous(), v.contiguous(), g.float().contiguous(), scale,
                                    initial_state, output_final_state, offsets=offsets, head_gates=True)
     if g is None:

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 13
+#define FLA_ABI_VERSION 14
 
 enum fla_dtype { FLA_F32 = 0, FLA_BF16 = 1, FLA_F16 = 2 };
 
@@ -281,6 +281,17 @@ int fla_chunk_simple_gla_fwd_fused(const void* q, const void* k, const void* v, 
                                    const int64_t* chunk_offsets, const int64_t* seq_order, int64_t NT,
                                    int qkv_dtype, int64_t B, int64_t T, int64_t H, int64_t K, int64_t V,
                                    int64_t N, float scale, fla_stream_t stream);
+
+/* chunk_simple_gla forward without kept activations (fla/ops/simple_gla/chunk.py:16-131: chunk_fwd_h + chunk_fwd_o
+ * with one gate per (token, head)) on the delta-rule scan kernel with the delta rule taken out (v_new = v, no
+ * correction term, no WY tile): q and k reach LDS as they are, the gates ride on the 64x64 score blocks, on the rows
+ * of (q h) and on the rows of v, the chunk-local prefix sum of g is formed inside the launch, and the decay factors
+ * e^{G_i - G_j} (j <= i) never exceed one, so no range guard is needed.  g: raw log-gates fp32 [B,T,H] or NULL.
+ * K in {64, 128}, V a multiple of 64; packed batches as for fla_chunk_gated_delta_rule_fwd_scan. */
+int fla_chunk_simple_gla_fwd_scan(const void* q, const void* k, const void* v, const float* g, const float* h0,
+                                  void* o, float* ht, const int64_t* offsets, const int64_t* chunk_offsets,
+                                  const int64_t* seq_order, int qkv_dtype, int64_t B, int64_t T, int64_t H,
+                                  int64_t K, int64_t V, int64_t N, float scale, fla_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Chunked gated delta rule forward (chunk size 64).  g_cumsum is the fp32

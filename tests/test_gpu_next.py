@@ -246,9 +246,12 @@ def test_packed_batch_with_empty_sequence(device, op):
 @pytest.mark.parametrize("T,K,V", [(64, 128, 128), (300, 128, 64), (1000, 64, 128), (37, 64, 64)])
 @pytest.mark.parametrize("varlen", [False, True])
 @pytest.mark.parametrize("gate_scale", [1.0, 40.0])   # 40: chunk-cumulative gates far beyond the single-reference range
-def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, gate_scale):
+@pytest.mark.parametrize("route", ["scan", "fused"])   # the plain scan kernel (default) / the GLA kernel's per-head-gate form
+def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, gate_scale, route, monkeypatch):
+    import fla_amd.ops.simple_gla.chunk as sg_mod
     from fla_amd.ops.simple_gla import chunk_simple_gla
     from oracle.recurrent import naive_recurrent_gla
+    monkeypatch.setattr(sg_mod, "SCAN_FORWARD", route == "scan")
     N, H = 3, 3
     B = 1 if varlen else 2
     gen = torch.Generator().manual_seed(T + K + int(gate_scale))
@@ -259,7 +262,7 @@ def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, 
     g = F.logsigmoid(torch.randn(B, T, H, generator=gen)) * gate_scale
     h0 = torch.randn(N if varlen else B, H, K, V, generator=gen) * 0.1
     dev = _dev(device)
-    print(f"chunk_simple_gla no-grad T={T} K={K} V={V} varlen={varlen} gate x{gate_scale}", flush=True)
+    print(f"chunk_simple_gla no-grad T={T} K={K} V={V} varlen={varlen} gate x{gate_scale} route={route}", flush=True)
     with torch.no_grad():
         o, ht = chunk_simple_gla(dev(q), dev(k), dev(v), dev(g), initial_state=dev(h0), output_final_state=True,
                                  cu_seqlens=dev(offs), head_first=False)
@@ -272,7 +275,11 @@ def test_chunk_simple_gla_forward_per_head_gate_kernel(device, T, K, V, varlen, 
                                   output_final_state=True, offsets=None if offs is None else offs.tolist())
     assert_close("o", ro, o, TOL_O)
     assert_close("ht", rht, ht, TOL_HT)
-    assert torch.equal(o, o2) and torch.equal(ht, ht2)   # same arithmetic on both routes
+    if route == "fused":
+        assert torch.equal(o, o2) and torch.equal(ht, ht2)   # same arithmetic as the per-key-gate launch
+    else:
+        assert_close("o vs the per-key-gate launch", o2, o, TOL_O)
+        assert_close("ht vs the per-key-gate launch", ht2, ht, TOL_HT)
 
 
 def test_chunk_simple_gla_per_head_gate_kernel_fp16_and_gradients(device):
